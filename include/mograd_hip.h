@@ -1,0 +1,288 @@
+/*
+ * mograd_hip.h — C ABI of libmograd_hip.so: MI355X (gfx950) kernels for the backward hot
+ * path of mograd (LayerNorm, softmax cross-entropy, Linear gradients, flash attention),
+ * plus the stream and caching-pool plumbing those kernels need.
+ *
+ * Conventions
+ *   - Every function returns 0 on success and a non-zero mg_status on failure;
+ *     mg_last_error() then returns a thread-local message.  The reference raises Mojo
+ *     errors in the same situations; a binding re-raises from the message.
+ *   - All data pointers are DEVICE pointers unless a parameter is documented as host.
+ *   - The caller owns inputs and outputs.  Outputs need no initialisation.  Scratch is
+ *     taken from the library's pool and returned before the call returns; this is safe
+ *     because all work of one call is enqueued on the one stream passed in, and the pool
+ *     hands memory back out only to later calls (the reference's single in-order-stream
+ *     contract, mograd/memory.mojo:27-31).  Calls on different streams that overlap in
+ *     time must not share the pool's scratch: serialise them or use one stream.
+ *   - `stream` is a hipStream_t passed as void*; NULL is the default stream.  No function
+ *     synchronises the host unless its comment says so.
+ *   - The symbols are new names: the reference's own `mograd_*` exports use the Mojo ABI
+ *     with Mojo-only argument types (mograd/runtime/gpu/kernels/dispatch.mojo:83-554)
+ *     and cannot be honoured from C.  Each declaration cites the export it replaces.
+ */
+#ifndef MOGRAD_HIP_H
+#define MOGRAD_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element types.  The reference supports f16, f32 and i64 (mograd/buffer.mojo:136);
+ * bf16 and i32 are additions. */
+typedef enum mg_dtype {
+  MG_F32 = 0,
+  MG_F16 = 1,
+  MG_BF16 = 2,
+  MG_I32 = 3,
+  MG_I64 = 4
+} mg_dtype;
+
+typedef enum mg_status {
+  MG_OK = 0,
+  MG_ERR_INVALID = 1,     /* bad argument (shape, dtype, alignment, flag combination) */
+  MG_ERR_UNSUPPORTED = 2, /* valid request this build has no kernel for */
+  MG_ERR_HIP = 3,         /* a HIP runtime call failed; message carries hipGetErrorString */
+  MG_ERR_OOM = 4          /* device allocation failed after flushing the cache */
+} mg_status;
+
+typedef void* mg_stream;
+
+/* ------------------------------------------------------------------------------------ */
+/* Library, errors, streams                                                              */
+/* ------------------------------------------------------------------------------------ */
+
+/* Version string "mograd_hip x.y (gfx950)". */
+const char* mg_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* mg_last_error(void);
+
+/* Selects `device` for this thread and reads its properties (CU count).  Optional:
+ * every entry point initialises lazily on the current device.
+ * Replaces Device() construction, mograd/device_ctx.mojo:44-54. */
+int mg_init(int device);
+
+/* Number of compute units of the current device (the reference's MULTIPROCESSOR_COUNT,
+ * kernels/normalization.mojo:322). */
+int mg_device_cu_count(void);
+
+/* One in-order stream, default priority.  Replaces the DeviceContext's stream. */
+int mg_stream_create(mg_stream* out);
+int mg_stream_destroy(mg_stream stream);
+/* Blocks the host until `stream` drains (ctx.synchronize(), scheduler.mojo:80). */
+int mg_stream_sync(mg_stream stream);
+
+/* Events on a stream, for timing kernels where they run.  mg_event_elapsed_ms blocks the
+ * host until `stop` has completed.  (The reference times with perf_counter_ns around a
+ * synchronize, mograd/debug.mojo:98-114.) */
+typedef void* mg_event;
+int mg_event_create(mg_event* out);
+int mg_event_destroy(mg_event event);
+int mg_event_record(mg_event event, mg_stream stream);
+int mg_event_elapsed_ms(mg_event start, mg_event stop, float* ms);
+
+/* Host <-> device copies and fills for buffers the caller owns.  The copies are
+ * synchronous with respect to the host (they return when the bytes have arrived).
+ * Replace Buffer.from_data / to_list / full, mograd/buffer.mojo. */
+int mg_copy_to_device(void* dst, const void* host_src, int64_t nbytes, mg_stream stream);
+int mg_copy_to_host(void* host_dst, const void* src, int64_t nbytes, mg_stream stream);
+int mg_copy_device(void* dst, const void* src, int64_t nbytes, mg_stream stream);
+/* dst[i] = value for i < numel, converted to `dtype` (any mg_dtype).  Asynchronous. */
+int mg_fill(void* dst, double value, int64_t numel, int dtype, mg_stream stream);
+
+/* ------------------------------------------------------------------------------------ */
+/* Caching device-memory pool (mograd/memory.mojo)                                       */
+/* ------------------------------------------------------------------------------------ */
+
+typedef struct mg_pool_stats {
+  int64_t allocated_bytes; /* class bytes handed out and not yet returned */
+  int64_t reserved_bytes;  /* allocated + cached in free lists */
+  int64_t peak_allocated;
+  int64_t peak_reserved;
+  int64_t alloc_count; /* real hipMalloc calls */
+  int64_t hit_count;
+  int64_t miss_count;
+  int64_t free_count; /* returns to the free lists */
+} mg_pool_stats;
+
+/* Size class of a request: multiples of prev_pow2(n)/8, minimum 512 B.
+ * memory.mojo:59-72 (round_class). */
+int64_t mg_round_class(int64_t nbytes);
+
+/* 1 unless the environment has MOGRAD_POOL=0 (memory.mojo:132). */
+int mg_pool_enabled(void);
+
+/* Returns storage of at least nbytes, reusing a cached block of the same class.  On
+ * hipMalloc failure the cache is emptied, the device synchronised and the allocation
+ * retried once (memory.mojo:242-295, take_storage/_driver_alloc). */
+int mg_pool_alloc(void** out, int64_t nbytes);
+
+/* Returns a block to its class free list (Storage.__deinit__/_release,
+ * memory.mojo:227-311).  Memory goes back to the driver only in mg_pool_empty_cache. */
+int mg_pool_free(void* ptr);
+
+/* Frees every cached block to the driver; reserved == allocated afterwards
+ * (memory.mojo:353-362). */
+int mg_pool_empty_cache(void);
+
+/* memory_stats, memory.mojo:377-382. */
+int mg_pool_get_stats(mg_pool_stats* out);
+
+/* memory_summary, memory.mojo:385-412.  Writes at most cap-1 bytes plus NUL into the
+ * HOST buffer `buf`; returns the full length needed. */
+int64_t mg_pool_summary(char* buf, int64_t cap);
+
+/* ------------------------------------------------------------------------------------ */
+/* LayerNorm over the last axis.  rows = numel / cols, cols = last dim                   */
+/* (kernels/dispatch.mojo:295-313,336-357).  dtype in {F32, F16, BF16}; math in fp32.     */
+/* ------------------------------------------------------------------------------------ */
+
+/* y = (x - mean) * rstd * gamma + beta, biased variance.
+ * Replaces mograd_layer_norm_fwd, kernels/__init__.mojo:1309-1334. */
+int mg_layer_norm_fwd(const void* x, const void* gamma, const void* beta, void* y, int64_t rows,
+                      int64_t cols, float eps, int dtype, mg_stream stream);
+
+/* Same, and also writes the per-row statistics (fp32, `rows` each) for the backward to
+ * reuse.  No counterpart in the reference, whose forward has one output
+ * (mograd/runtime/__init__.mojo:425-426). */
+int mg_layer_norm_fwd_stats(const void* x, const void* gamma, const void* beta, void* y,
+                            float* mean, float* rstd, int64_t rows, int64_t cols, float eps,
+                            int dtype, mg_stream stream);
+
+/* dx (rows, cols), dgamma (cols), dbeta (cols) from dy, x, gamma.  dgamma/dbeta are
+ * fully overwritten (the reference's caller zero-fills them first; not needed here).
+ * Two launches: row kernel with per-group partial sums, then a column reduction; no
+ * atomics.  Replaces mograd_layer_norm_bwd, kernels/__init__.mojo:1337-1366
+ * (kernels/normalization.mojo:85-400). */
+int mg_layer_norm_bwd(const void* dy, const void* x, const void* gamma, void* dx, void* dgamma,
+                      void* dbeta, int64_t rows, int64_t cols, float eps, int dtype,
+                      mg_stream stream);
+
+/* Same with the forward's saved statistics instead of recomputing them from x. */
+int mg_layer_norm_bwd_stats(const void* dy, const void* x, const void* gamma, const float* mean,
+                            const float* rstd, void* dx, void* dgamma, void* dbeta, int64_t rows,
+                            int64_t cols, int dtype, mg_stream stream);
+
+/* ------------------------------------------------------------------------------------ */
+/* Softmax cross-entropy.  N = numel / C rows, C = last dim                              */
+/* (kernels/__init__.mojo:1386-1387).  dtype in {F32, F16, BF16}; math in fp32.           */
+/* ------------------------------------------------------------------------------------ */
+
+/* loss[0] = -(1/N) sum_rows sum_c labels * log_softmax(logits), DENSE labels of the
+ * logits' shape and dtype (one-hot or soft).  Unlike the reference this does not
+ * synchronise the host.  Replaces mograd_cross_entropy, kernels/__init__.mojo:1374-1408
+ * (kernels/cross_entropy.mojo:14-77,155-177). */
+int mg_cross_entropy(const void* logits, const void* labels, void* loss, int64_t N, int64_t C,
+                     int dtype, mg_stream stream);
+
+/* dlogits = (softmax(logits) - labels) * upstream[0] / N.  `upstream` is a 1-element
+ * device buffer of `dtype`.  Replaces mograd_cross_entropy_grad,
+ * kernels/__init__.mojo:1462-1489 (kernels/cross_entropy.mojo:185-241). */
+int mg_cross_entropy_grad(const void* logits, const void* labels, const void* upstream,
+                          void* dlogits, int64_t N, int64_t C, int dtype, mg_stream stream);
+
+/* Strided forms: logits and labels are `rank`-dimensional views sharing `shape` (HOST
+ * array) with independent element strides (HOST arrays); the last dim is C.  The output
+ * of the gradient is contiguous.  Replace mograd_cross_entropy_strided and
+ * mograd_cross_entropy_grad_strided, kernels/__init__.mojo:1411-1454,1492-1528. */
+int mg_cross_entropy_strided(const void* logits, const void* labels, void* loss, int rank,
+                             const int64_t* shape, const int64_t* logits_strides,
+                             const int64_t* labels_strides, int dtype, mg_stream stream);
+int mg_cross_entropy_grad_strided(const void* logits, const void* labels, const void* upstream,
+                                  void* dlogits, int rank, const int64_t* shape,
+                                  const int64_t* logits_strides, const int64_t* labels_strides,
+                                  int dtype, mg_stream stream);
+
+/* Integer class ids instead of dense labels: `ids` holds N values of `id_dtype`
+ * (MG_I32 or MG_I64), each in [0, C).  Results equal the dense forms with
+ * labels = one_hot(ids).  No counterpart in the reference (labels reach it as
+ * one_hot(...).cast(f32), examples/mnist/train.mojo:36).
+ *   _ids        loss only        (reads logits once)
+ *   _grad_ids   dlogits only     (reads logits once, writes dlogits once)
+ *   _fused_ids  loss and dlogits in one pass over the logits.
+ * `upstream` may be NULL, meaning 1. */
+int mg_cross_entropy_ids(const void* logits, const void* ids, void* loss, int64_t N, int64_t C,
+                         int dtype, int id_dtype, mg_stream stream);
+int mg_cross_entropy_grad_ids(const void* logits, const void* ids, const void* upstream,
+                              void* dlogits, int64_t N, int64_t C, int dtype, int id_dtype,
+                              mg_stream stream);
+int mg_cross_entropy_fused_ids(const void* logits, const void* ids, const void* upstream,
+                               void* loss, void* dlogits, int64_t N, int64_t C, int dtype,
+                               int id_dtype, mg_stream stream);
+/* Dense-label loss and dlogits in one pass. */
+int mg_cross_entropy_fused(const void* logits, const void* labels, const void* upstream,
+                           void* loss, void* dlogits, int64_t N, int64_t C, int dtype,
+                           mg_stream stream);
+
+/* ------------------------------------------------------------------------------------ */
+/* Matmul family.  dst is always contiguous (batch, M, N).                               */
+/* Operand strides are in elements.  dtype in {F32, F16, BF16}; fp32 accumulation.        */
+/* ------------------------------------------------------------------------------------ */
+
+/* dst[b] = A[b] (M,K; strides lda0, lda1) x B[b] (K,N; strides ldb0, ldb1).
+ * batch_stride_b == 0 broadcasts one B over the batch.
+ * Replaces mograd_matmul, kernels/__init__.mojo:616-684.  This is the entry dW^T = X^T dY
+ * reaches with A = X^T as a strided view (mograd/grad.mojo:183). */
+int mg_matmul(const void* a, const void* b, void* dst, int64_t batch, int64_t M, int64_t N,
+              int64_t K, int64_t lda0, int64_t lda1, int64_t ldb0, int64_t ldb1,
+              int64_t batch_stride_a, int64_t batch_stride_b, int dtype, mg_stream stream);
+
+/* dst[b] = A[b] (M,K) x B[b]^T with B given as (N,K; strides ldb0, ldb1).
+ * Replaces mograd_matmul_bt, kernels/__init__.mojo:687-755.  This is the entry
+ * dX = dY W reaches with B = W^T as a strided view. */
+int mg_matmul_bt(const void* a, const void* b, void* dst, int64_t batch, int64_t M, int64_t N,
+                 int64_t K, int64_t lda0, int64_t lda1, int64_t ldb0, int64_t ldb1,
+                 int64_t batch_stride_a, int64_t batch_stride_b, int dtype, mg_stream stream);
+
+/* dst = A x B^T + bias[n].  Replaces mograd_matmul_bias_bt, kernels/__init__.mojo:758-840. */
+int mg_matmul_bias_bt(const void* a, const void* b, const void* bias, void* dst, int64_t batch,
+                      int64_t M, int64_t N, int64_t K, int64_t lda0, int64_t lda1, int64_t ldb0,
+                      int64_t ldb1, int64_t batch_stride_a, int64_t batch_stride_b, int dtype,
+                      mg_stream stream);
+
+/* The three Linear gradients for Y(M,N) = X(M,K) W(N,K)^T + b, all contiguous:
+ *   dx(M,K) = dY W          (NULL to skip)
+ *   dw(N,K) = dY^T X        written directly in W's layout, no transposed view
+ *   db(N)   = column sums   (NULL to skip)
+ * Covers the graph mograd/grad.mojo:180-187,278-288 emits for a Linear layer. */
+int mg_linear_bwd(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db,
+                  int64_t M, int64_t N, int64_t K, int dtype, mg_stream stream);
+
+/* dst(outer, inner) = sum over the middle axis of a contiguous (outer, reduce, inner)
+ * array.  db = sum over rows is outer=1, reduce=M, inner=N.  Two-stage, no atomics.
+ * Replaces mograd_sum_axis for contiguous inputs, kernels/__init__.mojo:1163-1189
+ * (kernels/reduce.mojo:137-173). */
+int mg_sum_axis(const void* a, void* dst, int64_t outer, int64_t reduce, int64_t inner, int dtype,
+                mg_stream stream);
+
+/* dst = upstream where out > 0 else 0, contiguous, n elements.
+ * Replaces mograd_relu_grad for contiguous inputs (kernels/elementwise.mojo:66-67). */
+int mg_relu_grad(const void* out, const void* upstream, void* dst, int64_t n, int dtype,
+                 mg_stream stream);
+
+/* ------------------------------------------------------------------------------------ */
+/* Flash attention.  Q, K, V, dQ, dK, dV are BSHD; O and dO are BHSD; mask is            */
+/* (B,H,S,S) additive bias in natural-log units, of `dtype`; LSE is (B,H,S) fp32 natural  */
+/* log (kernels/attention/generic.mojo:29-35).  dtype in {F32, F16, BF16}.                */
+/* causal != 0 with has_bias != 0 is rejected (kernels/__init__.mojo:868-873); with       */
+/* has_bias == 0 `mask` is never read and may be any pointer.  1 <= D <= 512 else error   */
+/* (kernels/attention/dispatch.mojo:28-29,124-125).                                       */
+/* ------------------------------------------------------------------------------------ */
+
+/* Replaces mograd_flash_attn_fwd, kernels/__init__.mojo:848-921. */
+int mg_flash_attn_fwd(const void* q, const void* k, const void* v, const void* mask, void* o,
+                      float* lse, int64_t B, int64_t S, int64_t H, int64_t D, float scale,
+                      int causal, int has_bias, int dtype, mg_stream stream);
+
+/* Replaces mograd_flash_attn_bwd, kernels/__init__.mojo:924-1006. */
+int mg_flash_attn_bwd(const void* d_o, const void* o, const void* q, const void* k, const void* v,
+                      const void* mask, const float* lse, void* dq, void* dk, void* dv, int64_t B,
+                      int64_t S, int64_t H, int64_t D, float scale, int causal, int has_bias,
+                      int dtype, mg_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOGRAD_HIP_H */

@@ -1,0 +1,81 @@
+// C ABI for LayerNorm: argument checks and dtype dispatch.
+#include "mg_internal.h"
+
+namespace mg {
+#define MG_DECLARE_LAYER_NORM(SUFFIX)                                                                         \
+  int ln_fwd_##SUFFIX(const void*, const void*, const void*, void*, float*, float*, int64_t, int64_t, float,  \
+                      hipStream_t);                                                                           \
+  int ln_bwd_##SUFFIX(const void*, const void*, const void*, const float*, const float*, void*, void*, void*, \
+                      int64_t, int64_t, float, hipStream_t);
+MG_DECLARE_LAYER_NORM(f32)
+MG_DECLARE_LAYER_NORM(f16)
+MG_DECLARE_LAYER_NORM(bf16)
+#undef MG_DECLARE_LAYER_NORM
+
+static int check_ln(const char* who, int64_t rows, int64_t cols, int dtype) {
+  if (!is_float_dtype(dtype)) return fail(MG_ERR_INVALID, "%s: unsupported dtype %s", who, dtype_name(dtype));
+  if (rows < 0 || cols <= 0 || cols > 0x3fffffffLL || rows > 0x7fffffffLL)
+    return fail(MG_ERR_INVALID, "%s: bad shape rows=%lld cols=%lld", who, static_cast<long long>(rows),
+                static_cast<long long>(cols));
+  return MG_OK;
+}
+
+static int ln_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean, float* rstd, int64_t rows,
+                  int64_t cols, float eps, int dtype, mg_stream stream) {
+  MG_TRY(check_ln("layer_norm_fwd", rows, cols, dtype));
+  if (rows == 0) return MG_OK;
+  if (!x || !gamma || !beta || !y) return fail(MG_ERR_INVALID, "layer_norm_fwd: null pointer argument");
+  hipStream_t s = to_stream(stream);
+  switch (dtype) {
+    case MG_F32: return ln_fwd_f32(x, gamma, beta, y, mean, rstd, rows, cols, eps, s);
+    case MG_F16: return ln_fwd_f16(x, gamma, beta, y, mean, rstd, rows, cols, eps, s);
+    default: return ln_fwd_bf16(x, gamma, beta, y, mean, rstd, rows, cols, eps, s);
+  }
+}
+
+static int ln_bwd(const void* dy, const void* x, const void* gamma, const float* mean, const float* rstd, void* dx,
+                  void* dgamma, void* dbeta, int64_t rows, int64_t cols, float eps, int dtype, mg_stream stream) {
+  MG_TRY(check_ln("layer_norm_bwd", rows, cols, dtype));
+  if (!dgamma || !dbeta) return fail(MG_ERR_INVALID, "layer_norm_bwd: null pointer argument");
+  hipStream_t s = to_stream(stream);
+  if (rows == 0) {  // the column sums of an empty matrix are zero
+    MG_HIP(hipMemsetAsync(dgamma, 0, static_cast<size_t>(cols) * dtype_size(dtype), s));
+    MG_HIP(hipMemsetAsync(dbeta, 0, static_cast<size_t>(cols) * dtype_size(dtype), s));
+    return MG_OK;
+  }
+  if (!dy || !x || !gamma || !dx) return fail(MG_ERR_INVALID, "layer_norm_bwd: null pointer argument");
+  switch (dtype) {
+    case MG_F32: return ln_bwd_f32(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps, s);
+    case MG_F16: return ln_bwd_f16(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps, s);
+    default: return ln_bwd_bf16(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps, s);
+  }
+}
+
+}  // namespace mg
+
+extern "C" {
+
+int mg_layer_norm_fwd(const void* x, const void* gamma, const void* beta, void* y, int64_t rows, int64_t cols,
+                      float eps, int dtype, mg_stream stream) {
+  return mg::ln_fwd(x, gamma, beta, y, nullptr, nullptr, rows, cols, eps, dtype, stream);
+}
+
+int mg_layer_norm_fwd_stats(const void* x, const void* gamma, const void* beta, void* y, float* mean, float* rstd,
+                            int64_t rows, int64_t cols, float eps, int dtype, mg_stream stream) {
+  if (!mean || !rstd) return mg::fail(MG_ERR_INVALID, "layer_norm_fwd_stats: null statistics pointer");
+  return mg::ln_fwd(x, gamma, beta, y, mean, rstd, rows, cols, eps, dtype, stream);
+}
+
+int mg_layer_norm_bwd(const void* dy, const void* x, const void* gamma, void* dx, void* dgamma, void* dbeta,
+                      int64_t rows, int64_t cols, float eps, int dtype, mg_stream stream) {
+  return mg::ln_bwd(dy, x, gamma, nullptr, nullptr, dx, dgamma, dbeta, rows, cols, eps, dtype, stream);
+}
+
+int mg_layer_norm_bwd_stats(const void* dy, const void* x, const void* gamma, const float* mean, const float* rstd,
+                            void* dx, void* dgamma, void* dbeta, int64_t rows, int64_t cols, int dtype,
+                            mg_stream stream) {
+  if (!mean || !rstd) return mg::fail(MG_ERR_INVALID, "layer_norm_bwd_stats: null statistics pointer");
+  return mg::ln_bwd(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, 0.f, dtype, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,106 @@
+// Host-side internals shared by every translation unit of libmograd_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "mograd_hip.h"
+
+namespace mg {
+
+// Records `msg` as this thread's last error and returns `code`.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+struct DeviceInfo {
+  int device = -1;
+  int cu_count = 0;
+  int max_threads = 0;
+};
+// Properties of the current device, read once per device.
+const DeviceInfo& device_info();
+
+// Pool (runtime.hip).  Thread-safe; see mg_pool_alloc / mg_pool_free.
+int pool_take(void** out, int64_t nbytes);
+int pool_release(void* ptr);
+
+// A scratch buffer from the pool, returned when the object dies.  Work that uses it has
+// already been enqueued on the caller's stream by then; the block is only handed out to
+// later calls, which enqueue behind that work on the same stream.
+class Scratch {
+ public:
+  Scratch() = default;
+  ~Scratch() {
+    if (ptr_) pool_release(ptr_);
+  }
+  Scratch(const Scratch&) = delete;
+  Scratch& operator=(const Scratch&) = delete;
+  int take(int64_t nbytes) { return pool_take(&ptr_, nbytes); }
+  template <typename T>
+  T* as() const {
+    return static_cast<T*>(ptr_);
+  }
+
+ private:
+  void* ptr_ = nullptr;
+};
+
+// A view of up to kMaxRank dimensions: extents and element strides, passed to kernels by
+// value.
+constexpr int kMaxRank = 8;
+struct StridedView {
+  int rank;
+  int64_t shape[kMaxRank];
+  int64_t stride[kMaxRank];
+};
+
+inline hipStream_t to_stream(mg_stream s) { return static_cast<hipStream_t>(s); }
+
+inline bool is_float_dtype(int dtype) { return dtype == MG_F32 || dtype == MG_F16 || dtype == MG_BF16; }
+inline int dtype_size(int dtype) {
+  switch (dtype) {
+    case MG_F32: return 4;
+    case MG_F16: return 2;
+    case MG_BF16: return 2;
+    case MG_I32: return 4;
+    case MG_I64: return 8;
+    default: return 0;
+  }
+}
+inline const char* dtype_name(int dtype) {
+  switch (dtype) {
+    case MG_F32: return "float32";
+    case MG_F16: return "float16";
+    case MG_BF16: return "bfloat16";
+    case MG_I32: return "int32";
+    case MG_I64: return "int64";
+    default: return "?";
+  }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace mg
+
+#define MG_HIP(expr)                                                                        \
+  do {                                                                                      \
+    hipError_t mg_e_ = (expr);                                                              \
+    if (mg_e_ != hipSuccess)                                                                \
+      return ::mg::fail(MG_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(mg_e_), \
+                        __FILE__, __LINE__);                                                \
+  } while (0)
+
+#define MG_TRY(expr)            \
+  do {                          \
+    int mg_rc_ = (expr);        \
+    if (mg_rc_ != 0) return mg_rc_; \
+  } while (0)
+
+// After a kernel launch: surfaces launch-configuration errors without synchronising.
+#define MG_LAUNCH_CHECK() MG_HIP(hipGetLastError())

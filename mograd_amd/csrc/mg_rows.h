@@ -1,0 +1,110 @@
+// Building blocks shared by the row-oriented kernels (LayerNorm, cross-entropy, column
+// sums): a register-resident row tile, the reduction over the threads sharing a row, and
+// the second stage of the two-stage column reduction.
+#pragma once
+
+#include "mg_device.h"
+
+namespace mg {
+
+// ------------------------------------------------------------------------------------
+// Row tile: VPT chunks of VEC elements per thread.
+// ------------------------------------------------------------------------------------
+
+template <typename T, int VEC, int TPR, int VPT>
+struct RowTile {
+  float v[VPT][VEC];
+
+  // Column of element 0 of this thread's chunk i.  Rows are narrower than 2^31 elements
+  // (checked on the host), so 32-bit column arithmetic is enough.
+  static __device__ __forceinline__ int col(int i, int t) { return (i * TPR + t) * VEC; }
+
+  __device__ __forceinline__ void load(const T* row_ptr, int t, int cols) {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int c = col(i, t);
+      if (c < cols) {
+        VecIO<T, VEC>::load(row_ptr + c, v[i]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[i][e] = 0.f;
+      }
+    }
+  }
+  __device__ __forceinline__ void store(T* row_ptr, int t, int cols) const {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int c = col(i, t);
+      if (c < cols) VecIO<T, VEC>::store(row_ptr + c, v[i]);
+    }
+  }
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[i][e] = 0.f;
+  }
+};
+
+// Reduction over the TPR threads that share a row: wave-only when TPR == 64, otherwise
+// the whole workgroup (TPR == WG).
+// Position of a thread among the TPR threads of its row, and which of the WG/TPR row
+// slots of the workgroup it serves.  With one row per workgroup the slot is the constant
+// 0, which keeps row addresses wave-uniform (scalar registers).
+template <int TPR, int WG>
+__device__ __forceinline__ void row_thread(int& t, int& sub) {
+  if constexpr (TPR == WG) {
+    t = threadIdx.x;
+    sub = 0;
+  } else {
+    t = threadIdx.x % TPR;
+    sub = threadIdx.x / TPR;
+  }
+}
+
+template <int TPR, int WG, int K>
+__device__ __forceinline__ void row_allreduce_sum(float (&v)[K], float* slots, int& phase) {
+  if constexpr (TPR == kWave) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = wave_sum(v[k]);
+  } else {
+    static_assert(TPR == WG, "a row is shared by one wave or by the whole workgroup");
+    block_allreduce<SumOp, WG / kWave, K>(v, slots, phase);
+    phase ^= 1;
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// Second stage of a column reduction: out[c] = sum_g part[g][c], plain stores, fixed
+// order (used by LayerNorm's dgamma/dbeta and by the bias gradient).
+// Workgroup = 64 columns x 4 row slices; blockIdx.y selects which of up to two
+// (partials, output) pairs to reduce.
+// ------------------------------------------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ part0, T* __restrict__ out0,
+                                                              const float* __restrict__ part1, T* __restrict__ out1,
+                                                              int64_t groups, int64_t cols) {
+  __shared__ float tile[4][64];
+  const float* part = blockIdx.y == 0 ? part0 : part1;
+  T* out = blockIdx.y == 0 ? out0 : out1;
+  const int cx = threadIdx.x % 64;
+  const int sy = threadIdx.x / 64;
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * 64 + cx;
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+  if (c < cols) {
+    int64_t g = sy;
+    for (; g + 12 < groups; g += 16) {
+      a0 += part[g * cols + c];
+      a1 += part[(g + 4) * cols + c];
+      a2 += part[(g + 8) * cols + c];
+      a3 += part[(g + 12) * cols + c];
+    }
+    for (; g < groups; g += 4) a0 += part[g * cols + c];
+  }
+  tile[sy][cx] = (a0 + a1) + (a2 + a3);
+  __syncthreads();
+  if (sy == 0 && c < cols) out[c] = from_float<T>((tile[0][cx] + tile[1][cx]) + (tile[2][cx] + tile[3][cx]));
+}
+
+}  // namespace mg

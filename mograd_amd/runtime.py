@@ -1,0 +1,542 @@
+"""Host-side mirror of mograd's kernel-dispatch surface for the backward hot path.
+
+The reference's scheduler maps an op node to a `BoundExecFn(node, inputs, device) ->
+List[AnyBuffer]` (mograd/scheduler.mojo:13-15) whose body marshals layouts into a
+kernel call (mograd/runtime/gpu/kernels/dispatch.mojo).  This module restates that
+surface in Python over libmograd_hip.so, with the same names, argument derivations
+and error conditions, so that tests of the HIP kernels read like the reference's own
+tests.  It contains no arithmetic: every result comes from the C ABI.
+
+    Layout      shape + element strides + base offset      mograd/layout.mojo:15-28
+    Device      stream + pool handle                       mograd/device_ctx.mojo:25-113
+    AnyBuffer   typed device allocation from the pool      mograd/buffer.mojo:135-214
+    Node        (op_type, layout, dtype, srcs, attrs)      mograd/op.mojo:124-185
+    SCHEDULER_RULES   op type -> exec function             mograd/runtime/__init__.mojo:113-167
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import _lib
+from ._lib import BF16, F16, F32, I32, I64, MogradError
+
+__all__ = [
+    "Layout", "Device", "AnyBuffer", "Node", "SCHEDULER_RULES", "MogradError",
+    "float32", "float16", "bfloat16", "int32", "int64",
+]
+
+float32, float16, bfloat16, int32, int64 = F32, F16, BF16, I32, I64
+
+_NP_OF = {F32: np.float32, F16: np.float16, I32: np.int32, I64: np.int64}
+
+
+# --------------------------------------------------------------------------- #
+# bfloat16 <-> float32 on the host (numpy has no bfloat16)
+# --------------------------------------------------------------------------- #
+
+
+def f32_to_bf16_bits(a) -> np.ndarray:
+    """Round-to-nearest-even float32 -> bfloat16 bit patterns (uint16)."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+    r = np.where(nan, (u >> 16) | 0x40, r)
+    return r.astype(np.uint16)
+
+
+def bf16_bits_to_f32(bits) -> np.ndarray:
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def round_to_dtype(a, dtype: int) -> np.ndarray:
+    """`a` rounded once to `dtype`, returned as float32 (what the kernel will see)."""
+    a = np.asarray(a, dtype=np.float32)
+    if dtype == F32:
+        return a
+    if dtype == F16:
+        return a.astype(np.float16).astype(np.float32)
+    if dtype == BF16:
+        return bf16_bits_to_f32(f32_to_bf16_bits(a)).reshape(a.shape)
+    raise ValueError(f"not a float dtype: {dtype}")
+
+
+# --------------------------------------------------------------------------- #
+# Layout
+# --------------------------------------------------------------------------- #
+
+
+def _row_major(shape: Sequence[int]) -> Tuple[int, ...]:
+    strides = [1] * len(shape)
+    for i in range(len(shape) - 2, -1, -1):
+        strides[i] = strides[i + 1] * shape[i + 1]
+    return tuple(strides)
+
+
+@dataclass(frozen=True)
+class Layout:
+    """Shape, element strides and base offset (mograd/layout.mojo)."""
+
+    dims: Tuple[int, ...]
+    strides: Tuple[int, ...] = ()
+    base_offset: int = 0
+
+    def __init__(self, *shape, strides: Optional[Sequence[int]] = None, base_offset: int = 0):
+        if len(shape) == 1 and isinstance(shape[0], (tuple, list)):
+            shape = tuple(shape[0])
+        object.__setattr__(self, "dims", tuple(int(s) for s in shape))
+        st = _row_major(self.dims) if strides is None else tuple(int(s) for s in strides)
+        if len(st) != len(self.dims):
+            raise ValueError("strides rank differs from shape rank")
+        object.__setattr__(self, "strides", st)
+        object.__setattr__(self, "base_offset", int(base_offset))
+
+    def rank(self) -> int:
+        return len(self.dims)
+
+    def shape(self, idx: Optional[int] = None):
+        return self.dims if idx is None else self.dims[idx]
+
+    def stride(self, idx: Optional[int] = None):
+        return self.strides if idx is None else self.strides[idx]
+
+    def numel(self) -> int:
+        n = 1
+        for s in self.dims:
+            n *= s
+        return n
+
+    def is_contiguous(self) -> bool:  # layout.mojo:210-212
+        return self.strides == _row_major(self.dims)
+
+    def as_contiguous(self) -> "Layout":  # layout.mojo:238-240
+        return Layout(*self.dims)
+
+    def batch_dims_collapsible(self) -> bool:  # layout.mojo:214-236
+        for i in range(self.rank() - 4, -1, -1):
+            if self.strides[i] != self.dims[i + 1] * self.strides[i + 1]:
+                return False
+        return True
+
+    def reduce_dims(self, axis: int) -> Tuple[int, int, int]:  # layout.mojo:287-298
+        ax = axis + self.rank() if axis < 0 else axis
+        if not 0 <= ax < self.rank():
+            raise MogradError(1, f"axis {axis} out of range for rank {self.rank()}")
+        reduce_size = self.dims[ax]
+        inner = 1
+        for s in self.dims[ax + 1:]:
+            inner *= s
+        outer = self.numel() // (reduce_size * inner)
+        return outer, reduce_size, inner
+
+    def transpose(self, dim0: int = -2, dim1: int = -1) -> "Layout":  # layout.mojo:435-452
+        d0 = dim0 % self.rank()
+        d1 = dim1 % self.rank()
+        dims = list(self.dims)
+        st = list(self.strides)
+        dims[d0], dims[d1] = dims[d1], dims[d0]
+        st[d0], st[d1] = st[d1], st[d0]
+        return Layout(*dims, strides=st, base_offset=self.base_offset)
+
+    def slice_axis(self, axis: int, start: int, stop: int, step: int = 1) -> "Layout":  # layout.mojo:321-340
+        ax = axis % self.rank()
+        extent = max(0, (stop - start + step - 1) // step)
+        dims = list(self.dims)
+        st = list(self.strides)
+        dims[ax] = extent
+        st[ax] = self.strides[ax] * step
+        return Layout(*dims, strides=st, base_offset=self.base_offset + start * self.strides[ax])
+
+
+# --------------------------------------------------------------------------- #
+# Device and buffers
+# --------------------------------------------------------------------------- #
+
+
+class Device:
+    """One GPU, one in-order stream, and the process-wide caching pool
+    (mograd/device_ctx.mojo:25-113).  Raises if the HIP library is missing."""
+
+    def __init__(self, index: int = 0):
+        self.lib = _lib.load()
+        self.lib.mg_init(index)
+        self.index = index
+        s = C.c_void_p()
+        self.lib.mg_stream_create(C.byref(s))
+        self.stream = s
+
+    def synchronize(self) -> None:
+        self.lib.mg_stream_sync(self.stream)
+
+    def empty_cache(self) -> None:
+        self.lib.mg_pool_empty_cache()
+
+    def memory_stats(self) -> _lib.PoolStats:
+        st = _lib.PoolStats()
+        self.lib.mg_pool_get_stats(C.byref(st))
+        return st
+
+    def memory_summary(self) -> str:
+        n = self.lib.mg_pool_summary(None, 0)
+        buf = C.create_string_buffer(int(n) + 1)
+        self.lib.mg_pool_summary(buf, n + 1)
+        return buf.value.decode()
+
+    def pool_enabled(self) -> bool:
+        return bool(self.lib.mg_pool_enabled())
+
+    def cu_count(self) -> int:
+        return int(self.lib.mg_device_cu_count())
+
+    def close(self) -> None:
+        if self.stream is not None:
+            self.lib.mg_stream_sync(self.stream)
+            self.lib.mg_stream_destroy(self.stream)
+            self.stream = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class _Storage:
+    """One pooled allocation; returns to the free lists when the last view dies
+    (Storage, mograd/memory.mojo:199-239)."""
+
+    def __init__(self, device: Device, nbytes: int):
+        self.device = device
+        self.lib = device.lib
+        p = C.c_void_p()
+        self.lib.mg_pool_alloc(C.byref(p), nbytes)
+        self.ptr = p.value or 0
+        self.nbytes = nbytes
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                self.lib.mg_pool_free(C.c_void_p(self.ptr))
+                self.ptr = 0
+        except Exception:
+            pass
+
+
+class AnyBuffer:
+    """A typed device buffer (mograd/buffer.mojo:135-214).  `view` shares storage."""
+
+    def __init__(self, storage: _Storage, dtype: int, numel: int, offset_elems: int = 0):
+        self.storage = storage
+        self.dtype = dtype
+        self.numel = numel
+        self.offset_elems = offset_elems
+
+    @staticmethod
+    def supports(dtype: int) -> bool:
+        return dtype in _lib.DTYPE_SIZE
+
+    @staticmethod
+    def create(dtype: int, device: Device, numel: int, fill: Optional[float] = None) -> "AnyBuffer":
+        if dtype not in _lib.DTYPE_SIZE:
+            raise MogradError(1, f"Unsupported dtype: {dtype}")
+        buf = AnyBuffer(_Storage(device, numel * _lib.DTYPE_SIZE[dtype]), dtype, numel)
+        if fill is not None:
+            device.lib.mg_fill(buf.data_ptr(), float(fill), numel, dtype, device.stream)
+        return buf
+
+    @staticmethod
+    def from_numpy(device: Device, array, dtype: Optional[int] = None) -> "AnyBuffer":
+        """Uploads `array`.  Float arrays are rounded once to `dtype` (default float32)."""
+        a = np.asarray(array)
+        if dtype is None:
+            dtype = {np.dtype(np.int32): I32, np.dtype(np.int64): I64, np.dtype(np.float16): F16}.get(a.dtype, F32)
+        if dtype == BF16:
+            host = f32_to_bf16_bits(a.astype(np.float32)).reshape(-1)
+        else:
+            host = np.ascontiguousarray(a, dtype=_NP_OF[dtype]).reshape(-1)
+        buf = AnyBuffer.create(dtype, device, host.size)
+        device.lib.mg_copy_to_device(buf.data_ptr(), host.ctypes.data_as(C.c_void_p), host.nbytes, device.stream)
+        return buf
+
+    def data_ptr(self, with_offset: bool = True) -> C.c_void_p:
+        off = self.offset_elems * _lib.DTYPE_SIZE[self.dtype] if with_offset else 0
+        return C.c_void_p(self.storage.ptr + off)
+
+    def size_bytes(self) -> int:
+        return self.numel * _lib.DTYPE_SIZE[self.dtype]
+
+    def view(self, layout: Layout) -> "AnyBuffer":
+        return AnyBuffer(self.storage, self.dtype, layout.numel(), layout.base_offset)
+
+    def to_numpy(self, shape: Optional[Sequence[int]] = None) -> np.ndarray:
+        """Synchronous download.  bfloat16 comes back as float32."""
+        dev = self.storage.device
+        if self.dtype == BF16:
+            host = np.empty(self.numel, dtype=np.uint16)
+        else:
+            host = np.empty(self.numel, dtype=_NP_OF[self.dtype])
+        dev.lib.mg_copy_to_host(host.ctypes.data_as(C.c_void_p), self.data_ptr(), host.nbytes, dev.stream)
+        out = bf16_bits_to_f32(host) if self.dtype == BF16 else host
+        return out.reshape(tuple(shape)) if shape is not None else out
+
+    def item(self) -> float:
+        return self.to_numpy().reshape(-1)[0].item()
+
+
+# --------------------------------------------------------------------------- #
+# Op nodes
+# --------------------------------------------------------------------------- #
+
+
+@dataclass
+class Node:
+    """Just enough of an op node for the exec functions: its own layout and dtype, the
+    layouts of its sources, and its attributes (mograd/op.mojo:124-185)."""
+
+    op_type: str
+    node_layout: Layout
+    node_dtype: int
+    srcs: List["Node"] = field(default_factory=list)
+    node_attrs: Dict[str, object] = field(default_factory=dict)
+
+    def layout(self) -> Layout:
+        return self.node_layout
+
+    def dtype(self) -> int:
+        return self.node_dtype
+
+    def numel(self) -> int:
+        return self.node_layout.numel()
+
+    def src(self, i: int) -> "Node":
+        return self.srcs[i]
+
+    def attrs(self) -> Dict[str, object]:
+        return self.node_attrs
+
+    def shape(self, i: int) -> int:
+        return self.node_layout.shape(i)
+
+    @staticmethod
+    def leaf(layout: Layout, dtype: int = F32) -> "Node":
+        return Node("BUFFER", layout, dtype)
+
+
+def _require_float(dtype: int, who: str) -> None:
+    if dtype not in (F32, F16, BF16):  # dispatch_dtype[float_only=True], dispatch.mojo:564-576
+        raise MogradError(1, f"{who}: unsupported dtype")
+
+
+# --------------------------------------------------------------------------- #
+# Exec functions (BoundExecFn bodies)
+# --------------------------------------------------------------------------- #
+
+
+def layer_norm_fwd(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """LAYER_NORM[x, gamma, beta]{eps}.  dispatch.mojo:294-314."""
+    x_layout = node.src(0).layout()
+    cols = x_layout.shape(x_layout.rank() - 1)
+    rows = x_layout.numel() // cols
+    eps = float(node.attrs()["eps"])
+    _require_float(node.dtype(), "layer_norm_fwd")
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_layer_norm_fwd(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), out.data_ptr(),
+                                 rows, cols, eps, node.dtype(), device.stream)
+    return [out]
+
+
+def layer_norm_bwd(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """LAYER_NORM_GRAD[dy, x, gamma]{eps} -> [dx, dgamma, dbeta].  dispatch.mojo:332-358."""
+    x_layout = node.src(1).layout()
+    gamma_layout = node.src(2).layout()
+    cols = x_layout.shape(x_layout.rank() - 1)
+    rows = x_layout.numel() // cols
+    eps = float(node.attrs()["eps"])
+    _require_float(node.dtype(), "layer_norm_bwd")
+    dx = AnyBuffer.create(node.dtype(), device, x_layout.numel())
+    dgamma = AnyBuffer.create(node.dtype(), device, gamma_layout.numel())
+    dbeta = AnyBuffer.create(node.dtype(), device, gamma_layout.numel())
+    device.lib.mg_layer_norm_bwd(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), dx.data_ptr(),
+                                 dgamma.data_ptr(), dbeta.data_ptr(), rows, cols, eps, node.dtype(), device.stream)
+    return [dx, dgamma, dbeta]
+
+
+def flash_attn_fwd_sched(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """FLASH_ATTN[Q, K, V, mask]{scale, is_causal, has_bias} -> [O (BHSD), LSE (BHS f32)].
+    dispatch.mojo:380-415: B,S,H,D from the BSHD Q layout; has_bias defaults to True."""
+    q_layout = node.src(0).layout()
+    B, S, H, D = (q_layout.shape(i) for i in range(4))
+    scale = float(node.attrs()["scale"])
+    is_causal = bool(node.attrs()["is_causal"])
+    has_bias = bool(node.attrs().get("has_bias", True))
+    _require_float(node.dtype(), "flash_attn_fwd")
+    dst = AnyBuffer.create(node.dtype(), device, node.numel())
+    lse = AnyBuffer.create(F32, device, B * H * S)
+    device.lib.mg_flash_attn_fwd(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+                                 inputs[3].data_ptr(), dst.data_ptr(), lse.data_ptr(), B, S, H, D, scale,
+                                 int(is_causal), int(has_bias), node.dtype(), device.stream)
+    return [dst, lse]
+
+
+def flash_attn_bwd_sched(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """FLASH_ATTN_GRAD[dO, O, Q, K, V, mask, LSE] -> [dQ, dK, dV].
+    dispatch.mojo:441-481: has_bias defaults to `not is_causal`."""
+    q_layout = node.src(2).layout()
+    B, S, H, D = (q_layout.shape(i) for i in range(4))
+    scale = float(node.attrs()["scale"])
+    is_causal = bool(node.attrs()["is_causal"])
+    has_bias = bool(node.attrs().get("has_bias", not is_causal))
+    numel = q_layout.numel()
+    _require_float(node.dtype(), "flash_attn_bwd")
+    dq = AnyBuffer.create(node.dtype(), device, numel)
+    dk = AnyBuffer.create(node.dtype(), device, numel)
+    dv = AnyBuffer.create(node.dtype(), device, numel)
+    device.lib.mg_flash_attn_bwd(*(inputs[i].data_ptr() for i in range(7)), dq.data_ptr(), dk.data_ptr(),
+                                 dv.data_ptr(), B, S, H, D, scale, int(is_causal), int(has_bias), node.dtype(),
+                                 device.stream)
+    return [dq, dk, dv]
+
+
+def _i64_array(values: Sequence[int]):
+    return (C.c_int64 * len(values))(*values)
+
+
+def cross_entropy(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """CROSS_ENTROPY[logits, labels] -> (1,).  runtime/__init__.mojo:530-533:
+    contiguous operands take the flat kernel, anything else the strided one."""
+    la = node.src(0).layout()
+    lb = node.src(1).layout()
+    _require_float(node.dtype(), "cross_entropy")
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    C_ = la.shape(la.rank() - 1)
+    N = la.numel() // C_
+    if la.is_contiguous() and lb.is_contiguous():
+        device.lib.mg_cross_entropy(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), N, C_, node.dtype(),
+                                    device.stream)
+    else:
+        device.lib.mg_cross_entropy_strided(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), la.rank(),
+                                            _i64_array(la.shape()), _i64_array(la.stride()),
+                                            _i64_array(lb.stride()), node.dtype(), device.stream)
+    return [out]
+
+
+def cross_entropy_grad(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """CROSS_ENTROPY_GRAD[logits, labels, upstream].  runtime/__init__.mojo:563-580."""
+    la = node.src(0).layout()
+    lb = node.src(1).layout()
+    _require_float(node.dtype(), "cross_entropy_grad")
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    C_ = la.shape(la.rank() - 1)
+    N = la.numel() // C_
+    if la.is_contiguous() and lb.is_contiguous():
+        device.lib.mg_cross_entropy_grad(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+                                         out.data_ptr(), N, C_, node.dtype(), device.stream)
+    else:
+        device.lib.mg_cross_entropy_grad_strided(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+                                                 out.data_ptr(), la.rank(), _i64_array(la.shape()),
+                                                 _i64_array(la.stride()), _i64_array(lb.stride()), node.dtype(),
+                                                 device.stream)
+    return [out]
+
+
+def _matmul_dims(la: Layout, lb: Layout, N: int, b_is_nk: bool, who: str):
+    """kernels/__init__.mojo:629-644,700-715,774-786."""
+    rank = la.rank()
+    if not (la.batch_dims_collapsible() and lb.batch_dims_collapsible()):
+        raise MogradError(1, f"{who}: received non-collapsible batch dims, expected op.mojo to materialise these first")
+    M = la.shape(rank - 2)
+    K = la.shape(rank - 1)
+    lda0, lda1 = la.stride(rank - 2), la.stride(rank - 1)
+    ldb0, ldb1 = lb.stride(lb.rank() - 2), lb.stride(lb.rank() - 1)
+    batch = la.numel() // (M * K)
+    bsa = la.stride(rank - 3) if rank >= 3 else M * K
+    bsb = lb.stride(lb.rank() - 3) if lb.rank() >= 3 else (N * K if b_is_nk else K * N)
+    return batch, M, K, lda0, lda1, ldb0, ldb1, bsa, bsb
+
+
+def matmul(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """MATMUL[A (.., M, K), B (.., K, N)].  dispatch.mojo:227-244."""
+    la, lb = node.src(0).layout(), node.src(1).layout()
+    N = node.shape(node.layout().rank() - 1)
+    batch, M, K, lda0, lda1, ldb0, ldb1, bsa, bsb = _matmul_dims(la, lb, N, False, "matmul")
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_matmul(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), batch, M, N, K, lda0, lda1,
+                         ldb0, ldb1, bsa, bsb, node.dtype(), device.stream)
+    return [out]
+
+
+def matmul_t(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """MATMUL_BT[A (.., M, K), B (.., N, K)] = A B^T.  dispatch.mojo:227-244."""
+    la, lb = node.src(0).layout(), node.src(1).layout()
+    N = node.shape(node.layout().rank() - 1)
+    batch, M, K, lda0, lda1, ldb0, ldb1, bsa, bsb = _matmul_dims(la, lb, N, True, "matmul")
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_matmul_bt(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), batch, M, N, K, lda0, lda1,
+                            ldb0, ldb1, bsa, bsb, node.dtype(), device.stream)
+    return [out]
+
+
+def matmul_bias_bt(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """MATMUL_BIAS_BT[A, B (N, K), bias (N)] = A B^T + bias.  dispatch.mojo:260-278."""
+    la, lb = node.src(0).layout(), node.src(1).layout()
+    N = node.shape(node.layout().rank() - 1)
+    batch, M, K, lda0, lda1, ldb0, ldb1, bsa, bsb = _matmul_dims(la, lb, N, True, "matmul_bias")
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_matmul_bias_bt(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), out.data_ptr(),
+                                 batch, M, N, K, lda0, lda1, ldb0, ldb1, bsa, bsb, node.dtype(), device.stream)
+    return [out]
+
+
+def sum(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:  # noqa: A001 (reference name)
+    """SUM{axis}.  runtime/__init__.mojo:390-393, dispatch.mojo:196-212.  Only the axis
+    form over a contiguous source is on this path (db = dY.sum(0))."""
+    if "axis" not in node.attrs():
+        raise MogradError(2, "sum: the full reduction is outside the backward hot path")
+    layout = node.src(0).layout()
+    if not layout.is_contiguous():
+        raise MogradError(2, "sum: strided source is outside the backward hot path; materialise it first")
+    outer, reduce_size, inner = layout.reduce_dims(int(node.attrs()["axis"]))
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_sum_axis(inputs[0].data_ptr(), out.data_ptr(), outer, reduce_size, inner, node.dtype(),
+                           device.stream)
+    return [out]
+
+
+def relu_grad(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """RELU_GRAD[relu_out, upstream].  runtime/__init__.mojo:351-352."""
+    for i in (0, 1):
+        if not node.src(i).layout().is_contiguous():
+            raise MogradError(2, "relu_grad: strided operand is outside the backward hot path")
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_relu_grad(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), node.numel(), node.dtype(),
+                            device.stream)
+    return [out]
+
+
+# Op type -> exec function, the rows of the reference's rule table that belong to this
+# path (mograd/runtime/__init__.mojo:113-167).
+SCHEDULER_RULES = {
+    "RELU_GRAD": relu_grad,
+    "SUM": sum,
+    "MATMUL": matmul,
+    "MATMUL_BT": matmul_t,
+    "MATMUL_BIAS_BT": matmul_bias_bt,
+    "LAYER_NORM": layer_norm_fwd,
+    "LAYER_NORM_GRAD": layer_norm_bwd,
+    "FLASH_ATTN": flash_attn_fwd_sched,
+    "FLASH_ATTN_GRAD": flash_attn_bwd_sched,
+    "CROSS_ENTROPY": cross_entropy,
+    "CROSS_ENTROPY_GRAD": cross_entropy_grad,
+}
+
+
+def run(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """One scheduler step: first matching rule wins (pattern_matcher.mojo:74-80)."""
+    try:
+        fn = SCHEDULER_RULES[node.op_type]
+    except KeyError:
+        raise MogradError(2, f"no scheduler rule for op {node.op_type} on the backward hot path") from None
+    return fn(node, inputs, device)

@@ -1,0 +1,57 @@
+"""Shared test helpers: seeded inputs and tolerance checks.
+
+Inputs follow one rule everywhere: one numpy PCG64 generator per tensor, seeded with
+1000 * config + tensor index, and the same host bytes go to the oracle and to the GPU.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+# Tolerances of the parity contract.
+RTOL_F32, ATOL_F32 = 1e-4, 1e-5       # fp32 reductions
+RTOL_BF16_ATTN = 2e-2                 # bf16 attention gradients
+
+
+def rng_for(config: int, tensor: int) -> np.random.Generator:
+    return np.random.Generator(np.random.PCG64(1000 * config + tensor))
+
+
+def normal(config, tensor, shape, std=1.0, mean=0.0):
+    return (rng_for(config, tensor).standard_normal(shape) * std + mean).astype(np.float32)
+
+
+def uniform(config, tensor, shape, lo, hi):
+    return rng_for(config, tensor).uniform(lo, hi, shape).astype(np.float32)
+
+
+def integers(config, tensor, shape, lo, hi, dtype=np.int32):
+    return rng_for(config, tensor).integers(lo, hi, shape).astype(dtype)
+
+
+def worst_violation(got, want, rtol, atol):
+    """max over elements of |got - want| / (atol + rtol * |want|); <= 1 passes."""
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    if not np.all(np.isfinite(got)):
+        return float("inf")
+    return float(np.max(np.abs(got - want) / (atol + rtol * np.abs(want)))) if got.size else 0.0
+
+
+def assert_close(got, want, rtol, atol, what=""):
+    v = worst_violation(got, want, rtol, atol)
+    assert v <= 1.0, f"{what}: worst |err| / (atol + rtol*|want|) = {v:.3g} (rtol={rtol}, atol={atol})"
+
+
+def assert_sum_close(got, want, term_l1, rtol=RTOL_F32, atol=ATOL_F32, what=""):
+    """For an fp32 sum of many terms: rtol against the value, plus an absolute floor of
+    `atol` scaled by the mean magnitude of what was summed (term_l1 / 1 per output), i.e.
+    the floor is relative to the size of the summands rather than to a result that may
+    have cancelled to near zero."""
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    floor = atol * np.maximum(1.0, np.asarray(term_l1, dtype=np.float64))
+    err = np.abs(got - want)
+    bound = floor + rtol * np.abs(want)
+    worst = float(np.max(err / bound))
+    assert np.all(np.isfinite(got)) and worst <= 1.0, f"{what}: worst err/bound = {worst:.3g}"

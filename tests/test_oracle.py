@@ -1,0 +1,363 @@
+"""Pins the CPU oracle (oracle/oracle_np.py, oracle/oracle_c.c) before anything is
+checked against it: the reference's own golden vectors, closed forms, a library routine
+(torch on CPU, float64) and brute-force loops.  No GPU."""
+import ctypes as C
+import math
+import subprocess
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle_np as O
+
+ROOT = Path(__file__).resolve().parent.parent
+ORACLE_SO = ROOT / "oracle" / "liboracle_c.so"
+
+
+# --------------------------------------------------------------------------- #
+# LayerNorm — goldens from the reference's tests
+# --------------------------------------------------------------------------- #
+
+
+def test_ln_fwd_goldens():
+    # tests/test_nn.mojo:283-324
+    y = O.layer_norm_fwd([[1, 2, 3, 4]], [1, 2, 1, 2], [0.1, 0.2, 0.1, 0.2])
+    np.testing.assert_allclose(y, [[-1.241641, -0.694427, 0.547214, 2.883282]], atol=1e-4)
+    y = O.layer_norm_fwd([[1, 2, 3, 4], [-1, -2, -3, -4]], [1] * 4, [0] * 4)
+    want = [-1.341641, -0.447214, 0.447214, 1.341641]
+    np.testing.assert_allclose(y, [want, want[::-1]], atol=1e-4)
+    y = O.layer_norm_fwd([[3, 3, 3, 3]], [1] * 4, [0.5] * 4)
+    np.testing.assert_allclose(y, [[0.5] * 4], atol=1e-4)
+
+
+def test_ln_bwd_goldens():
+    # tests/test_grad.mojo:776-856
+    x = [[1.0, 2, 3, 4]]
+    dy = [[0.1, 0.2, 0.3, 0.4]]
+    dx, dg, db = O.layer_norm_bwd(dy, x, [1, 2, 1, 2])
+    np.testing.assert_allclose(dx, [[0.0, 0.089443, -0.178886, 0.089443]], atol=2e-4)
+    np.testing.assert_allclose(dg, [-0.134164, -0.089443, 0.134164, 0.536656], atol=2e-4)
+    np.testing.assert_allclose(db, [0.1, 0.2, 0.3, 0.4], atol=1e-5)
+    # two identical rows: dbeta doubles
+    _, _, db2 = O.layer_norm_bwd(dy * 2, x * 2, [1] * 4)
+    np.testing.assert_allclose(db2, [0.2, 0.4, 0.6, 0.8], atol=1e-5)
+    # uniform dy with gamma = 1 gives zero dx
+    dx0, _, _ = O.layer_norm_bwd([[1, 1, 1, 1]], x, [1] * 4)
+    np.testing.assert_allclose(dx0, np.zeros((1, 4)), atol=1e-5)
+
+
+def test_ln_bwd_matches_torch_autograd_and_invariants():
+    rng = np.random.default_rng(0)
+    x = rng.normal(size=(7, 33))
+    g = rng.uniform(0.5, 1.5, size=33)
+    b = rng.normal(size=33)
+    dy = rng.normal(size=(7, 33))
+    xt = torch.tensor(x, requires_grad=True)
+    gt = torch.tensor(g, requires_grad=True)
+    bt = torch.tensor(b, requires_grad=True)
+    y = torch.nn.functional.layer_norm(xt, (33,), gt, bt, eps=1e-5)
+    y.backward(torch.tensor(dy))
+    np.testing.assert_allclose(O.layer_norm_fwd(x, g, b), y.detach().numpy(), rtol=1e-10, atol=1e-12)
+    dx, dg, db = O.layer_norm_bwd(dy, x, g)
+    np.testing.assert_allclose(dx, xt.grad.numpy(), rtol=1e-9, atol=1e-11)
+    np.testing.assert_allclose(dg, gt.grad.numpy(), rtol=1e-9, atol=1e-11)
+    np.testing.assert_allclose(db, bt.grad.numpy(), rtol=1e-9, atol=1e-11)
+    # gamma = 1: dx is orthogonal to 1 in every row, and to xhat as eps -> 0
+    dx1, _, _ = O.layer_norm_bwd(dy, x, np.ones(33), eps=1e-14)
+    mu, rstd = O.layer_norm_stats(x, 1e-14)
+    np.testing.assert_allclose(dx1.sum(axis=1), 0, atol=1e-12)
+    np.testing.assert_allclose((dx1 * (x - mu) * rstd).sum(axis=1), 0, atol=1e-10)
+
+
+def test_ln_rank3_is_rows_of_last_dim():
+    # rows = numel / cols (dispatch.mojo:336-340)
+    rng = np.random.default_rng(1)
+    x = rng.normal(size=(2, 3, 8))
+    dy = rng.normal(size=(2, 3, 8))
+    g = rng.normal(size=8)
+    a = O.layer_norm_bwd(dy, x, g)
+    b = O.layer_norm_bwd(dy.reshape(6, 8), x.reshape(6, 8), g)
+    np.testing.assert_allclose(a[0].reshape(6, 8), b[0])
+    np.testing.assert_allclose(a[1], b[1])
+
+
+# --------------------------------------------------------------------------- #
+# Cross-entropy — goldens
+# --------------------------------------------------------------------------- #
+
+
+def test_ce_goldens():
+    # tests/test_ops.mojo:155-175
+    assert abs(O.cross_entropy(np.zeros((4, 10)), O.one_hot([0, 1, 2, 3], 10)) - 2.302585) < 1e-3
+    assert abs(O.cross_entropy(np.zeros((2, 4)), np.full((2, 4), 0.25)) - 1.386294) < 1e-3
+    assert abs(O.cross_entropy([[100, 0, 0], [0, 100, 0]], [[1, 0, 0], [0, 1, 0]])) < 1e-3
+    # tests/test_non_contiguous.mojo:275-299 (strided views; values after applying the view)
+    assert abs(O.cross_entropy([[0, 0], [0, 0]], [[0.5, 0.5], [0.5, 0.5]]) - 0.693147) < 1e-3
+    assert abs(O.cross_entropy(np.zeros((2, 2)), [[1, 0], [0, 1]]) - 0.693147) < 1e-3
+
+
+def test_ce_grad_goldens():
+    # tests/test_non_contiguous.mojo:302-310: logits = a^T with a = [[1,2],[3,4]], labels = I;
+    # the expected gradient is with respect to a, i.e. the transpose of dlogits.
+    a = np.array([[1.0, 2], [3, 4]])
+    d = O.cross_entropy_grad(a.T, np.eye(2))
+    np.testing.assert_allclose(d.T.reshape(-1), [-0.440398, 0.059601, 0.440398, -0.059601], atol=1e-3)
+    # tests/test_grad.mojo:432-446: rows of the gradient sum to zero
+    d = O.cross_entropy_grad(np.ones((4, 10)), O.one_hot([0, 1, 2, 3], 10))
+    np.testing.assert_allclose(d.sum(axis=1), 0, atol=1e-12)
+
+
+def test_ce_matches_torch_and_id_forms():
+    rng = np.random.default_rng(2)
+    x = rng.normal(scale=2, size=(9, 17))
+    ids = rng.integers(0, 17, size=9)
+    soft = rng.uniform(size=(9, 17))
+    soft /= soft.sum(axis=1, keepdims=True)
+    xt = torch.tensor(x, requires_grad=True)
+    loss = torch.nn.functional.cross_entropy(xt, torch.tensor(ids))
+    loss.backward()
+    assert abs(O.cross_entropy_ids(x, ids) - loss.item()) < 1e-12
+    assert abs(O.cross_entropy(x, O.one_hot(ids, 17)) - loss.item()) < 1e-12
+    np.testing.assert_allclose(O.cross_entropy_grad_ids(x, ids), xt.grad.numpy(), atol=1e-13)
+    np.testing.assert_allclose(O.cross_entropy_grad(x, O.one_hot(ids, 17), 1.0), xt.grad.numpy(), atol=1e-13)
+    xt2 = torch.tensor(x, requires_grad=True)
+    loss2 = torch.nn.functional.cross_entropy(xt2, torch.tensor(soft))
+    (loss2 * 0.7).backward()
+    assert abs(O.cross_entropy(x, soft) - loss2.item()) < 1e-12
+    np.testing.assert_allclose(O.cross_entropy_grad(x, soft, 0.7), xt2.grad.numpy(), atol=1e-13)
+
+
+def test_ce_rank3_matches_reshape():
+    # tests/test_ops.mojo:178-186, tests/test_grad.mojo:467-483
+    x = (np.arange(24) * 0.1).reshape(2, 3, 4)
+    y = O.one_hot([0, 2, 1, 3, 0, 1], 4).reshape(2, 3, 4)
+    assert abs(O.cross_entropy(x, y) - O.cross_entropy(x.reshape(6, 4), y.reshape(6, 4))) < 1e-14
+    np.testing.assert_allclose(O.cross_entropy_grad(x, y).reshape(6, 4),
+                               O.cross_entropy_grad(x.reshape(6, 4), y.reshape(6, 4)))
+
+
+# --------------------------------------------------------------------------- #
+# Attention — closed forms, brute force, library
+# --------------------------------------------------------------------------- #
+
+
+def test_sdpa_closed_forms():
+    rng = np.random.default_rng(3)
+    B, S, H, D = 1, 128, 1, 8
+    v = rng.normal(size=(B, S, H, D))
+    z = np.zeros((B, S, H, D))
+    # tests/test_grad.mojo:1001-1023: Q = K = 0 causal, loss = sum(O):
+    # dV[j] = sum_{i >= j} 1/(i+1)
+    _, _, dv = O.sdpa_bwd(z, z, v, np.ones((B, H, S, D)), causal=True)
+    tail = np.array([sum(1.0 / (i + 1) for i in range(j, S)) for j in range(S)])
+    np.testing.assert_allclose(dv[0, :, 0, :], np.repeat(tail[:, None], D, axis=1), rtol=1e-12)
+    # tests/test_ops.mojo:903-919: causal row 0 attends only to itself
+    q = rng.normal(size=(B, S, H, D))
+    k = rng.normal(size=(B, S, H, D))
+    o, lse = O.sdpa_fwd(q, k, v, causal=True)
+    np.testing.assert_allclose(o[0, 0, 0], v[0, 0, 0], rtol=1e-12)
+    # tests/test_ops.mojo:932-946: uniform scores average V
+    o, lse = O.sdpa_fwd(z, z, v)
+    np.testing.assert_allclose(o[0, 0], np.repeat(v[0, :, 0].mean(axis=0)[None], S, axis=0), rtol=1e-12)
+    np.testing.assert_allclose(lse, math.log(S))
+
+
+def test_sdpa_bias_shift_invariance():
+    # tests/kernels/attention/generic.mojo:322-366: a constant added to the bias changes
+    # LSE by that constant and nothing else
+    rng = np.random.default_rng(4)
+    B, S, H, D = 2, 9, 2, 4
+    q, k, v = (rng.normal(size=(B, S, H, D)) for _ in range(3))
+    m = rng.normal(size=(B, H, S, S))
+    o1, l1 = O.sdpa_fwd(q, k, v, mask=m)
+    o2, l2 = O.sdpa_fwd(q, k, v, mask=m + 3.0)
+    np.testing.assert_allclose(o1, o2, atol=1e-12)
+    np.testing.assert_allclose(l2 - l1, 3.0, atol=1e-12)
+
+
+@pytest.mark.parametrize("causal,has_mask", [(False, False), (True, False), (False, True)])
+def test_sdpa_vectorised_equals_loops(causal, has_mask):
+    rng = np.random.default_rng(5)
+    B, S, H, D = 2, 7, 3, 5
+    q, k, v = (rng.normal(size=(B, S, H, D)) for _ in range(3))
+    do = rng.normal(size=(B, H, S, D))
+    m = rng.normal(size=(B, H, S, S)) if has_mask else None
+    scale = 0.37
+    o, lse = O.sdpa_fwd(q, k, v, m, causal, scale)
+    dq, dk, dv = O.sdpa_bwd(q, k, v, do, m, causal, scale)
+    mflat = m.reshape(-1).tolist() if has_mask else []
+    ol, ll = O.sdpa_fwd_loops(q.reshape(-1).tolist(), k.reshape(-1).tolist(), v.reshape(-1).tolist(), mflat, has_mask,
+                              causal, B, S, H, D, scale)
+    dql, dkl, dvl = O.sdpa_bwd_loops(q.reshape(-1).tolist(), k.reshape(-1).tolist(), v.reshape(-1).tolist(),
+                                     do.reshape(-1).tolist(), mflat, has_mask, causal, B, S, H, D, scale)
+    np.testing.assert_allclose(o.reshape(-1), ol, atol=1e-13)
+    np.testing.assert_allclose(lse.reshape(-1), ll, atol=1e-13)
+    np.testing.assert_allclose(dq.reshape(-1), dql, atol=1e-13)
+    np.testing.assert_allclose(dk.reshape(-1), dkl, atol=1e-13)
+    np.testing.assert_allclose(dv.reshape(-1), dvl, atol=1e-13)
+
+
+@pytest.mark.parametrize("causal,has_mask", [(False, False), (True, False), (False, True)])
+def test_sdpa_matches_torch_autograd(causal, has_mask):
+    rng = np.random.default_rng(6)
+    B, S, H, D = 2, 10, 2, 8
+    q, k, v = (rng.normal(size=(B, S, H, D)) for _ in range(3))
+    do = rng.normal(size=(B, H, S, D))
+    m = rng.normal(size=(B, H, S, S)) if has_mask else None
+    qt, kt, vt = (torch.tensor(a, requires_grad=True) for a in (q, k, v))
+    out = torch.nn.functional.scaled_dot_product_attention(
+        qt.transpose(1, 2), kt.transpose(1, 2), vt.transpose(1, 2),
+        attn_mask=torch.tensor(m) if has_mask else None, is_causal=causal)
+    out.backward(torch.tensor(do))
+    o, _ = O.sdpa_fwd(q, k, v, m, causal)
+    dq, dk, dv = O.sdpa_bwd(q, k, v, do, m, causal)
+    np.testing.assert_allclose(o, out.detach().numpy(), atol=1e-12)
+    np.testing.assert_allclose(dq, qt.grad.numpy(), atol=1e-12)
+    np.testing.assert_allclose(dk, kt.grad.numpy(), atol=1e-12)
+    np.testing.assert_allclose(dv, vt.grad.numpy(), atol=1e-12)
+
+
+# --------------------------------------------------------------------------- #
+# Linear gradients, relu_grad, pool classes
+# --------------------------------------------------------------------------- #
+
+
+def test_linear_grads_match_autograd():
+    rng = np.random.default_rng(7)
+    M, N, K = 5, 4, 6
+    x, w, b = rng.normal(size=(M, K)), rng.normal(size=(N, K)), rng.normal(size=N)
+    dy = rng.normal(size=(M, N))
+    xt, wt, bt = (torch.tensor(a, requires_grad=True) for a in (x, w, b))
+    y = torch.nn.functional.linear(xt, wt, bt)
+    y.backward(torch.tensor(dy))
+    np.testing.assert_allclose(O.matmul_bias_bt(x, w, b), y.detach().numpy(), atol=1e-13)
+    np.testing.assert_allclose(O.linear_grad_x(dy, w), xt.grad.numpy(), atol=1e-13)
+    np.testing.assert_allclose(O.linear_grad_w(dy, x), wt.grad.numpy(), atol=1e-13)
+    np.testing.assert_allclose(O.linear_grad_b(dy), bt.grad.numpy(), atol=1e-13)
+    out = np.maximum(y.detach().numpy(), 0)
+    np.testing.assert_array_equal(O.relu_grad(out, dy), np.where(out > 0, dy, 0))
+
+
+def test_round_class():
+    # tests/test_memory.mojo:18-30 and mograd/memory.mojo:59-72
+    assert O.round_class(1000) == 1024 and O.round_class(1025) == 1152
+    assert O.round_class(1) == 512 and O.round_class(512) == 512 and O.round_class(513) == 576
+    assert O.round_class(4096) == 4096 and O.round_class(990) == 1024
+    for n in [600, 5000, 123457, 1 << 20, (1 << 20) + 1, 3 << 28]:
+        c = O.round_class(n)
+        assert c >= n and (c - n) * 8 <= c and c % 64 == 0
+
+
+# --------------------------------------------------------------------------- #
+# The C restatement (fp32, OpenMP) against the float64 numpy oracle
+# --------------------------------------------------------------------------- #
+
+
+@pytest.fixture(scope="module")
+def orc():
+    if not ORACLE_SO.exists():
+        subprocess.run(["make", "-C", str(ROOT / "oracle")], check=True, capture_output=True)
+    lib = C.CDLL(str(ORACLE_SO))
+    lib.orc_cross_entropy_f32.restype = C.c_float
+    lib.orc_cross_entropy_ids_f32.restype = C.c_float
+    lib.orc_round_class.restype = C.c_int64
+    lib.orc_round_class.argtypes = [C.c_int64]
+    return lib
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _l(v):
+    return C.c_int64(v)
+
+
+def test_c_oracle_layer_norm(orc):
+    rng = np.random.default_rng(8)
+    rows, cols = 37, 130
+    x = rng.normal(size=(rows, cols)).astype(np.float32)
+    dy = rng.normal(size=(rows, cols)).astype(np.float32)
+    g = rng.uniform(0.5, 1.5, size=cols).astype(np.float32)
+    b = rng.normal(size=cols).astype(np.float32)
+    y = np.empty_like(x)
+    orc.orc_layer_norm_fwd_f32(_p(x), _p(g), _p(b), _p(y), _l(rows), _l(cols), C.c_float(1e-5))
+    np.testing.assert_allclose(y, O.layer_norm_fwd(x, g, b), rtol=1e-4, atol=1e-5)
+    dx = np.empty_like(x)
+    dg = np.empty_like(g)
+    db = np.empty_like(g)
+    orc.orc_layer_norm_bwd_f32(_p(dy), _p(x), _p(g), _p(dx), _p(dg), _p(db), _l(rows), _l(cols), C.c_float(1e-5), _l(8))
+    rdx, rdg, rdb = O.layer_norm_bwd(dy, x, g)
+    np.testing.assert_allclose(dx, rdx, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(dg, rdg, rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(db, rdb, rtol=1e-4, atol=1e-4)
+
+
+def test_c_oracle_cross_entropy(orc):
+    rng = np.random.default_rng(9)
+    N, Cc = 19, 77
+    x = rng.normal(scale=2, size=(N, Cc)).astype(np.float32)
+    ids = rng.integers(0, Cc, size=N).astype(np.int32)
+    y = O.one_hot(ids, Cc).astype(np.float32)
+    up = np.array([0.5], dtype=np.float32)
+    assert abs(orc.orc_cross_entropy_f32(_p(x), _p(y), _l(N), _l(Cc)) - O.cross_entropy(x, y)) < 1e-5
+    assert abs(orc.orc_cross_entropy_ids_f32(_p(x), _p(ids), _l(N), _l(Cc)) - O.cross_entropy(x, y)) < 1e-5
+    d = np.empty_like(x)
+    orc.orc_cross_entropy_grad_f32(_p(x), _p(y), _p(up), _p(d), _l(N), _l(Cc))
+    np.testing.assert_allclose(d, O.cross_entropy_grad(x, y, 0.5), rtol=1e-4, atol=1e-7)
+    orc.orc_cross_entropy_grad_ids_f32(_p(x), _p(ids), _p(up), _p(d), _l(N), _l(Cc))
+    np.testing.assert_allclose(d, O.cross_entropy_grad(x, y, 0.5), rtol=1e-4, atol=1e-7)
+
+
+def test_c_oracle_linear(orc):
+    rng = np.random.default_rng(10)
+    M, N, K = 13, 11, 17
+    x = rng.normal(size=(M, K)).astype(np.float32)
+    w = rng.normal(size=(N, K)).astype(np.float32)
+    b = rng.normal(size=N).astype(np.float32)
+    dy = rng.normal(size=(M, N)).astype(np.float32)
+    y = np.empty((M, N), np.float32)
+    orc.orc_matmul_bias_bt_f32(_p(x), _p(w), _p(b), _p(y), _l(M), _l(N), _l(K))
+    np.testing.assert_allclose(y, O.matmul_bias_bt(x, w, b), rtol=1e-4, atol=1e-5)
+    dx = np.empty((M, K), np.float32)
+    dw = np.empty((N, K), np.float32)
+    db = np.empty(N, np.float32)
+    orc.orc_linear_grad_x_f32(_p(dy), _p(w), _p(dx), _l(M), _l(N), _l(K))
+    orc.orc_linear_grad_w_f32(_p(dy), _p(x), _p(dw), _l(M), _l(N), _l(K))
+    orc.orc_linear_grad_b_f32(_p(dy), _p(db), _l(M), _l(N))
+    np.testing.assert_allclose(dx, O.linear_grad_x(dy, w), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(dw, O.linear_grad_w(dy, x), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(db, O.linear_grad_b(dy), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("causal,has_mask", [(False, False), (True, False), (False, True)])
+def test_c_oracle_attention(orc, causal, has_mask):
+    rng = np.random.default_rng(11)
+    B, S, H, D = 2, 21, 2, 8
+    q, k, v = (rng.normal(size=(B, S, H, D)).astype(np.float32) for _ in range(3))
+    do = rng.normal(size=(B, H, S, D)).astype(np.float32)
+    m = rng.normal(size=(B, H, S, S)).astype(np.float32)
+    scale = 1 / math.sqrt(D)
+    o = np.empty((B, H, S, D), np.float32)
+    lse = np.empty((B, H, S), np.float32)
+    orc.orc_sdpa_fwd_f32(_p(q), _p(k), _p(v), _p(m), int(has_mask), int(causal), _p(o), _p(lse), _l(B), _l(S), _l(H),
+                         _l(D), C.c_float(scale), _l(B * H))
+    ro, rl = O.sdpa_fwd(q, k, v, m if has_mask else None, causal, scale)
+    np.testing.assert_allclose(o, ro, atol=5e-6)
+    np.testing.assert_allclose(lse, rl, atol=5e-6)
+    dq, dk, dv = (np.empty_like(q) for _ in range(3))
+    orc.orc_sdpa_bwd_f32(_p(q), _p(k), _p(v), _p(do), _p(m), int(has_mask), int(causal), _p(dq), _p(dk), _p(dv),
+                         _l(B), _l(S), _l(H), _l(D), C.c_float(scale), _l(B * H))
+    rdq, rdk, rdv = O.sdpa_bwd(q, k, v, do, m if has_mask else None, causal, scale)
+    # the reference's own budget for an fp32 backward at this size: 5e-6 abs
+    # (tests/kernels/attention/generic.mojo:440)
+    np.testing.assert_allclose(dq, rdq, atol=5e-6)
+    np.testing.assert_allclose(dk, rdk, atol=5e-6)
+    np.testing.assert_allclose(dv, rdv, atol=5e-6)
+
+
+def test_c_oracle_round_class(orc):
+    for n in [1, 512, 513, 990, 1000, 1024, 1025, 4096, 5000, 123457, (1 << 20) + 1]:
+        assert orc.orc_round_class(n) == O.round_class(n)
