@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the backward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = LayerNorm forward + backward on fp32 (2048, 4096) and fused softmax
+cross-entropy forward + backward on fp32 logits (8192, 50304) with int32 labels, all
+inputs resident in HBM before the timed region.  Prints ONE JSON line:
+  value/ms_per_step   wall time per step (K steps between two stream synchronisations)
+  roofline            the dominant kernel (cross-entropy rows kernel): algorithmic bytes
+                      per launch / mean launch duration from HIP events on the stream
+                      the kernel runs on, against the 8 TB/s HBM peak
+  kernels             the same for every kernel of the step
+  cpu_baseline        the C restatement of the reference's arithmetic (oracle/), timed on
+                      this host's cores on a bounded sample of the same workload
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0
+
+LN_ROWS, LN_COLS = 2048, 4096
+CE_ROWS, CE_COLS = 8192, 50304
+
+# Algorithmic bytes per launch: what any implementation must move.
+LN_FWD_BYTES = 2 * LN_ROWS * LN_COLS * 4 + 2 * LN_COLS * 4            # x, y, gamma, beta
+LN_BWD_BYTES = 3 * LN_ROWS * LN_COLS * 4 + 3 * LN_COLS * 4            # dy, x, dx, gamma, dgamma, dbeta
+CE_FUSED_BYTES = 2 * CE_ROWS * CE_COLS * 4 + CE_ROWS * 4 + 4          # logits, dlogits, labels, loss
+
+
+def _rng(config: int, tensor: int) -> np.random.Generator:
+    return np.random.Generator(np.random.PCG64(1000 * config + tensor))
+
+
+class EventTimer:
+    """Mean duration of a callable's device work, from HIP event pairs recorded on the
+    library's stream around each call."""
+
+    def __init__(self, device, n: int):
+        self.dev = device
+        self.lib = device.lib
+        self.starts = [C.c_void_p() for _ in range(n)]
+        self.stops = [C.c_void_p() for _ in range(n)]
+        for e in self.starts + self.stops:
+            self.lib.mg_event_create(C.byref(e))
+
+    def run(self, fn, iters: int):
+        assert iters <= len(self.starts)
+        for i in range(iters):
+            self.lib.mg_event_record(self.starts[i], self.dev.stream)
+            fn(i)
+            self.lib.mg_event_record(self.stops[i], self.dev.stream)
+        self.dev.synchronize()
+        ms = C.c_float()
+        out = []
+        for i in range(iters):
+            self.lib.mg_event_elapsed_ms(self.starts[i], self.stops[i], C.byref(ms))
+            out.append(ms.value)
+        return out
+
+    def close(self):
+        for e in self.starts + self.stops:
+            self.lib.mg_event_destroy(e)
+
+
+def cpu_baseline(sample_ce_rows: int = 256):
+    """Times the C restatement (oracle/oracle_c.c) on this host: LayerNorm at full size,
+    cross-entropy on `sample_ce_rows` rows scaled to 8192."""
+    import subprocess
+
+    so = ROOT / "oracle" / "liboracle_c.so"
+    if not so.exists():
+        subprocess.run(["make", "-C", str(ROOT / "oracle")], check=True, capture_output=True)
+    orc = C.CDLL(str(so))
+    orc.orc_num_threads.restype = C.c_int
+    orc.orc_cross_entropy_ids_f32.restype = C.c_float
+    cores = int(orc.orc_num_threads())
+    p = lambda a: a.ctypes.data_as(C.c_void_p)  # noqa: E731
+    L = C.c_int64
+
+    x = _rng(2, 0).standard_normal((LN_ROWS, LN_COLS), dtype=np.float32)
+    g = _rng(2, 1).uniform(0.5, 1.5, LN_COLS).astype(np.float32)
+    b = (_rng(2, 2).standard_normal(LN_COLS) * 0.1).astype(np.float32)
+    dy = _rng(2, 3).standard_normal((LN_ROWS, LN_COLS), dtype=np.float32)
+    y, dx = np.empty_like(x), np.empty_like(x)
+    dg, db = np.empty_like(g), np.empty_like(g)
+
+    def ln():
+        orc.orc_layer_norm_fwd_f32(p(x), p(g), p(b), p(y), L(LN_ROWS), L(LN_COLS), C.c_float(1e-5))
+        orc.orc_layer_norm_bwd_f32(p(dy), p(x), p(g), p(dx), p(dg), p(db), L(LN_ROWS), L(LN_COLS), C.c_float(1e-5),
+                                   L(256))
+
+    n = sample_ce_rows
+    logits = (_rng(2, 10).standard_normal((n, CE_COLS), dtype=np.float32) * 2.0)
+    ids = _rng(2, 11).integers(0, CE_COLS, n).astype(np.int32)
+    up = np.ones(1, np.float32)
+    dlogits = np.empty_like(logits)
+
+    def ce():
+        # the reference runs forward and gradient as separate kernels
+        orc.orc_cross_entropy_ids_f32(p(logits), p(ids), L(n), L(CE_COLS))
+        orc.orc_cross_entropy_grad_ids_f32(p(logits), p(ids), p(up), p(dlogits), L(n), L(CE_COLS))
+
+    def best(fn, reps):
+        fn()
+        t = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            t.append(time.perf_counter() - t0)
+        return min(t)
+
+    ln_ms = best(ln, 5) * 1e3
+    ce_ms = best(ce, 3) * 1e3 * (CE_ROWS / n)
+    return {
+        "value": round(ln_ms + ce_ms, 3),
+        "unit": "ms",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"LayerNorm fwd+bwd full (2048x4096) {ln_ms:.2f} ms; cross-entropy fwd+grad on {n} of 8192 rows "
+                  f"scaled x{CE_ROWS // n} = {ce_ms:.1f} ms; best of 3-5 runs, OpenMP on {cores} threads",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path runs on one GPU; --gpus N with N > 1 is not supported "
+              "(no collective is part of the backward hot path)", file=sys.stderr)
+        return 2
+
+    from mograd_amd import F32, I32, AnyBuffer, Device
+
+    dev = Device(0)
+    lib = dev.lib
+    st = dev.stream
+
+    # ---- inputs, resident in HBM -------------------------------------------------------
+    # LayerNorm: four rotating sets (4 x 100 MB) so that no set is still in the 256 MB
+    # memory-side cache when it is used again.
+    LN_SETS = 4
+    gamma = AnyBuffer.from_numpy(dev, _rng(2, 1).uniform(0.5, 1.5, LN_COLS).astype(np.float32))
+    beta = AnyBuffer.from_numpy(dev, (_rng(2, 2).standard_normal(LN_COLS) * 0.1).astype(np.float32))
+    ln_sets = []
+    for s in range(LN_SETS):
+        x = AnyBuffer.from_numpy(dev, _rng(2, 100 + s).standard_normal((LN_ROWS, LN_COLS), dtype=np.float32))
+        dy = AnyBuffer.from_numpy(dev, _rng(2, 200 + s).standard_normal((LN_ROWS, LN_COLS), dtype=np.float32))
+        y = AnyBuffer.create(F32, dev, LN_ROWS * LN_COLS)
+        dx = AnyBuffer.create(F32, dev, LN_ROWS * LN_COLS)
+        ln_sets.append((x, dy, y, dx))
+    dgamma = AnyBuffer.create(F32, dev, LN_COLS)
+    dbeta = AnyBuffer.create(F32, dev, LN_COLS)
+
+    # Cross-entropy: 1.65 GB of logits, uploaded in slabs.
+    logits = AnyBuffer.create(F32, dev, CE_ROWS * CE_COLS)
+    dlogits = AnyBuffer.create(F32, dev, CE_ROWS * CE_COLS)
+    rng = _rng(2, 10)
+    slab = 1024
+    for r0 in range(0, CE_ROWS, slab):
+        part = rng.standard_normal((slab, CE_COLS), dtype=np.float32) * 2.0
+        lib.mg_copy_to_device(C.c_void_p(logits.data_ptr().value + r0 * CE_COLS * 4), part.ctypes.data_as(C.c_void_p),
+                              part.nbytes, st)
+    ids = AnyBuffer.from_numpy(dev, _rng(2, 11).integers(0, CE_COLS, CE_ROWS).astype(np.int32), I32)
+    loss = AnyBuffer.create(F32, dev, 1)
+
+    def ln_fwd(i):
+        x, dy, y, dx = ln_sets[i % LN_SETS]
+        lib.mg_layer_norm_fwd(x.data_ptr(), gamma.data_ptr(), beta.data_ptr(), y.data_ptr(), LN_ROWS, LN_COLS, 1e-5,
+                              F32, st)
+
+    def ln_bwd(i):
+        x, dy, y, dx = ln_sets[i % LN_SETS]
+        lib.mg_layer_norm_bwd(dy.data_ptr(), x.data_ptr(), gamma.data_ptr(), dx.data_ptr(), dgamma.data_ptr(),
+                              dbeta.data_ptr(), LN_ROWS, LN_COLS, 1e-5, F32, st)
+
+    def ce_fused(i):
+        lib.mg_cross_entropy_fused_ids(logits.data_ptr(), ids.data_ptr(), None, loss.data_ptr(), dlogits.data_ptr(),
+                                       CE_ROWS, CE_COLS, F32, I32, st)
+
+    def step(i):
+        ln_fwd(i)
+        ln_bwd(i)
+        ce_fused(i)
+
+    # ---- whole step: W warm-up steps, then exactly K timed steps -------------------------
+    for i in range(args.warmup):
+        step(i)
+    dev.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(args.warmup + i)
+    dev.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # ---- per-kernel launch durations from HIP events on the library's stream ------------
+    iters = max(10, min(args.steps, 100))
+    timer = EventTimer(dev, iters)
+    kernels = []
+    for name, fn, nbytes in (("layer_norm_fwd", ln_fwd, LN_FWD_BYTES), ("layer_norm_bwd", ln_bwd, LN_BWD_BYTES),
+                             ("cross_entropy_fused_ids", ce_fused, CE_FUSED_BYTES)):
+        fn(0)
+        dev.synchronize()
+        ts = timer.run(fn, iters)
+        mean_ms = float(np.mean(ts))
+        gbs = nbytes / (mean_ms * 1e-3) / 1e9
+        kernels.append({"name": name, "mean_ms": round(mean_ms, 5), "median_ms": round(float(np.median(ts)), 5),
+                        "algorithmic_bytes": nbytes, "achieved_GBps": round(gbs, 1),
+                        "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)})
+    timer.close()
+    dominant = kernels[-1]
+
+    result = {
+        "metric": "fwd+bwd step ms; per-bwd-kernel HBM GB/s or MFMA % of MI355X peak",
+        "value": round(ms_per_step, 4),
+        "unit": "ms",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "LayerNorm fwd+bwd fp32 (2048,4096) + fused softmax-cross-entropy fwd+bwd fp32 logits "
+                        "(8192,50304), int32 labels",
+            "layer_norm": [LN_ROWS, LN_COLS],
+            "cross_entropy": [CE_ROWS, CE_COLS],
+            "labels": "int32 class ids",
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "ce_rows_kernel (mg_cross_entropy_fused_ids; the event pair also spans the one-workgroup "
+                      "loss reduction that follows it)",
+            "achieved": dominant["achieved_GBps"],
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(dominant["achieved_GBps"] / HBM_PEAK_GBS, 4),
+            "traffic": None,
+        },
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

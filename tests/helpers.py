@@ -35,7 +35,12 @@ def worst_violation(got, want, rtol, atol):
     assert got.shape == want.shape, (got.shape, want.shape)
     if not np.all(np.isfinite(got)):
         return float("inf")
-    return float(np.max(np.abs(got - want) / (atol + rtol * np.abs(want)))) if got.size else 0.0
+    if not got.size:
+        return 0.0
+    err = np.abs(got - want)
+    bound = atol + rtol * np.abs(want)
+    ratio = np.divide(err, bound, out=np.where(err > 0, np.inf, 0.0), where=bound > 0)
+    return float(np.max(ratio))
 
 
 def assert_close(got, want, rtol, atol, what=""):

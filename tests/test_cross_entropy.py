@@ -96,10 +96,10 @@ def test_dense_random_f32(device, N, Cc):
     soft = np.abs(normal(30, 1, (N, Cc))) + 0.01
     soft = (soft / soft.sum(axis=1, keepdims=True)).astype(np.float32)
     assert_close(_ce(device, x, soft), O.cross_entropy(x, soft), RTOL_F32, ATOL_F32, "loss")
-    # gradient entries are O(1/(N*C)); compare at the parity rtol with an absolute floor
-    # at the same relative level of the largest entry
+    # gradient entries are (p - y) * upstream / N: compare at the parity rtol with an
+    # absolute floor at the same relative level of that natural scale
     want = O.cross_entropy_grad(x, soft, 0.75)
-    assert_close(_ce_grad(device, x, soft, 0.75), want, RTOL_F32, RTOL_F32 * np.abs(want).max(), "dlogits")
+    assert_close(_ce_grad(device, x, soft, 0.75), want, RTOL_F32, RTOL_F32 * 0.75 / N, "dlogits")
 
 
 def _ids_calls(device, x, ids, upstream, id_dtype, dtype=F32):
@@ -130,12 +130,13 @@ def test_ids_random_f32(device, N, Cc, id_dtype):
     want = O.cross_entropy_grad_ids(x, ids, 1.25)
     assert_close(loss, want_loss, RTOL_F32, ATOL_F32, "loss")
     assert_close(loss2, want_loss, RTOL_F32, ATOL_F32, "fused loss")
-    floor = RTOL_F32 * np.abs(want).max()
+    floor = RTOL_F32 * 1.25 / N
     assert_close(grad, want, RTOL_F32, floor, "dlogits")
     np.testing.assert_array_equal(grad, grad2)  # the fused call runs the same gradient code
     # label gather is exact: the only negative entries of the gradient sit at the labels
-    neg_cols = [np.flatnonzero(grad[r] < 0) for r in range(N)]
-    assert all(list(c) == [ids[r]] for r, c in enumerate(neg_cols))
+    if Cc > 1:
+        neg_cols = [np.flatnonzero(grad[r] < 0) for r in range(N)]
+        assert all(list(c) == [ids[r]] for r, c in enumerate(neg_cols))
     # ids equal the dense one-hot form
     one_hot = O.one_hot(ids, Cc).astype(np.float32)
     assert_close(_ce(device, x, one_hot), want_loss, RTOL_F32, ATOL_F32, "dense loss")
@@ -154,7 +155,7 @@ def test_fused_dense(device):
                                       N, Cc, F32, device.stream)
     assert_close(loss.item(), O.cross_entropy(x, soft), RTOL_F32, ATOL_F32, "loss")
     want = O.cross_entropy_grad(x, soft, 0.5)
-    assert_close(grad.to_numpy((N, Cc)), want, RTOL_F32, RTOL_F32 * np.abs(want).max(), "dlogits")
+    assert_close(grad.to_numpy((N, Cc)), want, RTOL_F32, RTOL_F32 * 0.5 / N, "dlogits")
 
 
 def test_benchmark_shape_rows(device):
@@ -167,7 +168,7 @@ def test_benchmark_shape_rows(device):
     loss, grad, loss2, grad2 = _ids_calls(device, x, ids, 1.0, I32)
     assert_close(loss2, O.cross_entropy_ids(x, ids), RTOL_F32, ATOL_F32, "loss")
     want = O.cross_entropy_grad_ids(x, ids)
-    assert_close(grad2, want, RTOL_F32, RTOL_F32 * np.abs(want).max(), "dlogits")
+    assert_close(grad2, want, RTOL_F32, RTOL_F32 / N, "dlogits")
 
 
 def test_benchmark_shape_full_properties(device):
@@ -177,30 +178,29 @@ def test_benchmark_shape_full_properties(device):
     grad = AnyBuffer.create(F32, device, N * Cc)
     logits = AnyBuffer.create(F32, device, N * Cc)
     ids = integers(2, 13, (N,), 0, Cc)
-    # Upload in slabs to bound host memory.
+    # Upload in slabs to bound host memory; the oracle's loss is accumulated per slab.
     slab = 1024
+    want_loss = 0.0
     for r0 in range(0, N, slab):
         part = (rng.standard_normal((slab, Cc), dtype=np.float32) * 2.0)
+        want_loss += O.cross_entropy_ids(part, ids[r0:r0 + slab]) * slab / N
         lib.mg_copy_to_device(C.c_void_p(logits.data_ptr().value + r0 * Cc * 4), part.ctypes.data_as(C.c_void_p),
                               part.nbytes, device.stream)
     bi = AnyBuffer.from_numpy(device, ids, I32)
     loss = AnyBuffer.create(F32, device, 1)
     lib.mg_cross_entropy_fused_ids(logits.data_ptr(), bi.data_ptr(), None, loss.data_ptr(), grad.data_ptr(), N, Cc,
                                    F32, I32, device.stream)
+    assert_close(loss.item(), want_loss, RTOL_F32, ATOL_F32, "loss")
     g = grad.to_numpy((N, Cc))
     # every row of dlogits sums to zero; exactly one negative entry per row, at the label
     assert np.max(np.abs(g.astype(np.float64).sum(axis=1))) < 1e-8
     neg = g < 0
     assert np.all(neg.sum(axis=1) == 1)
     assert np.array_equal(np.argmax(neg, axis=1), ids)
-    # (softmax - onehot)/N: the positive part of each row sums to (1 - p_label)/N, and
-    # -log p_label averaged over the rows is the loss
-    p_label = 1.0 + g[np.arange(N), ids].astype(np.float64) * N
-    assert_close(loss.item(), float(np.mean(-np.log(p_label))), 1e-3, 1e-4, "loss from gradient")
-    # loss-only entry agrees with the fused one
+    # loss-only entry agrees with the oracle too
     loss_only = AnyBuffer.create(F32, device, 1)
     lib.mg_cross_entropy_ids(logits.data_ptr(), bi.data_ptr(), loss_only.data_ptr(), N, Cc, F32, I32, device.stream)
-    assert_close(loss_only.item(), loss.item(), RTOL_F32, ATOL_F32, "loss-only vs fused")
+    assert_close(loss_only.item(), want_loss, RTOL_F32, ATOL_F32, "loss-only")
 
 
 @pytest.mark.parametrize("dtype,rtol", [(F16, 2e-3), (BF16, 1.6e-2)])
@@ -213,7 +213,7 @@ def test_half_precision_storage(device, dtype, rtol, N, Cc):
     loss, grad, loss2, grad2 = _ids_calls(device, x, ids, up, I64, dtype)
     want_loss = O.cross_entropy_ids(x, ids)
     want = O.cross_entropy_grad_ids(x, ids, up)
-    floor = rtol * np.abs(want).max()
+    floor = rtol * up / N
     assert_close(loss, want_loss, rtol, rtol, "loss")
     assert_close(loss2, want_loss, rtol, rtol, "fused loss")
     assert_close(grad, want, rtol, floor, "dlogits")
