@@ -1,0 +1,142 @@
+// C ABI for the matmul family: operand classification, kernel choice, launches.
+#include "gemm_impl.h"
+
+namespace mg {
+
+// A x B with A element (m, k) at a[m * sam + k * sak] and B element (k, n) at
+// b[k * sbk + n * sbn]; C row-major (M, N).
+struct GemmArgs {
+  const void* a;
+  const void* b;
+  const void* bias;
+  void* c;
+  int64_t batch, M, N, K;
+  int64_t sam, sak, sbk, sbn;
+  int64_t bsa, bsb;
+  int dtype;
+};
+
+static bool mult4(int64_t v) { return (v & 3) == 0; }
+
+template <bool A_KC, bool B_KC>
+static int launch_f32_mfma(const GemmArgs& g, hipStream_t stream) {
+  const int tiles_m = static_cast<int>(ceil_div(g.M, kGemmBM));
+  const int tiles_n = static_cast<int>(ceil_div(g.N, kGemmBN));
+  const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.batch;
+  if (blocks > 0x7fffffffLL) return fail(MG_ERR_INVALID, "matmul: too many output tiles");
+  const int64_t lda = A_KC ? g.sam : g.sak;
+  const int64_t ldb = B_KC ? g.sbn : g.sbk;
+  const float* a = static_cast<const float*>(g.a);
+  const float* b = static_cast<const float*>(g.b);
+  const float* bias = static_cast<const float*>(g.bias);
+  float* c = static_cast<float*>(g.c);
+  if (bias)
+    hipLaunchKernelGGL((gemm_f32_mfma_kernel<A_KC, B_KC, true>), dim3(static_cast<unsigned>(blocks)), dim3(kGemmThreads),
+                       0, stream, a, b, bias, c, static_cast<int>(g.M), static_cast<int>(g.N), static_cast<int>(g.K), lda,
+                       ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n);
+  else
+    hipLaunchKernelGGL((gemm_f32_mfma_kernel<A_KC, B_KC, false>), dim3(static_cast<unsigned>(blocks)),
+                       dim3(kGemmThreads), 0, stream, a, b, bias, c, static_cast<int>(g.M), static_cast<int>(g.N),
+                       static_cast<int>(g.K), lda, ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n);
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+template <typename T>
+static int launch_generic(const GemmArgs& g, hipStream_t stream) {
+  const dim3 grid(static_cast<unsigned>(ceil_div(g.N, 64)), static_cast<unsigned>(ceil_div(g.M, 64)),
+                  static_cast<unsigned>(g.batch));
+  if (grid.y > 65535u || grid.z > 65535u) return fail(MG_ERR_INVALID, "matmul: shape exceeds the generic kernel's grid");
+  const T* a = static_cast<const T*>(g.a);
+  const T* b = static_cast<const T*>(g.b);
+  const T* bias = static_cast<const T*>(g.bias);
+  T* c = static_cast<T*>(g.c);
+  if (bias)
+    hipLaunchKernelGGL((gemm_generic_kernel<T, true>), grid, dim3(256), 0, stream, a, b, bias, c, static_cast<int>(g.M),
+                       static_cast<int>(g.N), static_cast<int>(g.K), g.sam, g.sak, g.sbk, g.sbn, g.N, g.bsa, g.bsb,
+                       g.M * g.N);
+  else
+    hipLaunchKernelGGL((gemm_generic_kernel<T, false>), grid, dim3(256), 0, stream, a, b, bias, c, static_cast<int>(g.M),
+                       static_cast<int>(g.N), static_cast<int>(g.K), g.sam, g.sak, g.sbk, g.sbn, g.N, g.bsa, g.bsb,
+                       g.M * g.N);
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+int gemm_dispatch(const char* who, const GemmArgs& g, hipStream_t stream) {
+  if (!is_float_dtype(g.dtype)) return fail(MG_ERR_INVALID, "%s: unsupported dtype %s", who, dtype_name(g.dtype));
+  if (g.batch < 0 || g.M < 0 || g.N < 0 || g.K < 0 || g.M > 0x7fffffffLL || g.N > 0x7fffffffLL || g.K > 0x7fffffffLL)
+    return fail(MG_ERR_INVALID, "%s: bad shape batch=%lld M=%lld N=%lld K=%lld", who, static_cast<long long>(g.batch),
+                static_cast<long long>(g.M), static_cast<long long>(g.N), static_cast<long long>(g.K));
+  if (g.batch == 0 || g.M == 0 || g.N == 0) return MG_OK;
+  if (!g.a || !g.b || !g.c) return fail(MG_ERR_INVALID, "%s: null pointer argument", who);
+
+  if (g.dtype == MG_F32 && g.K > 0) {
+    // Which dimension of each operand is contiguous, and can it be read 16 bytes at a time?
+    const bool a_kc = g.sak == 1 && mult4(g.sam) && mult4(g.K);
+    const bool a_mc = g.sam == 1 && mult4(g.sak) && mult4(g.M);
+    const bool b_kc = g.sbk == 1 && mult4(g.sbn) && mult4(g.K);
+    const bool b_nc = g.sbn == 1 && mult4(g.sbk) && mult4(g.N);
+    const bool aligned = aligned16(g.a) && aligned16(g.b) && mult4(g.bsa) && mult4(g.bsb);
+    // Tiny problems gain nothing from 128x128 tiles.
+    const bool worth_it = g.M * g.N >= 64 * 64 || g.K >= 512;
+    if (aligned && worth_it && (a_kc || a_mc) && (b_kc || b_nc)) {
+      if (a_kc && b_kc) return launch_f32_mfma<true, true>(g, stream);
+      if (a_kc) return launch_f32_mfma<true, false>(g, stream);
+      if (b_kc) return launch_f32_mfma<false, true>(g, stream);
+      return launch_f32_mfma<false, false>(g, stream);
+    }
+  }
+  switch (g.dtype) {
+    case MG_F32: return launch_generic<float>(g, stream);
+    case MG_F16: return launch_generic<f16_t>(g, stream);
+    default: return launch_generic<bf16_t>(g, stream);
+  }
+}
+
+int colsum_dispatch(const void* a, void* dst, int64_t outer, int64_t reduce, int64_t inner, int dtype,
+                    hipStream_t stream);  // reduce.hip
+
+}  // namespace mg
+
+extern "C" {
+
+int mg_matmul(const void* a, const void* b, void* dst, int64_t batch, int64_t M, int64_t N, int64_t K, int64_t lda0,
+              int64_t lda1, int64_t ldb0, int64_t ldb1, int64_t batch_stride_a, int64_t batch_stride_b, int dtype,
+              mg_stream stream) {
+  mg::GemmArgs g{a, b, nullptr, dst, batch, M, N, K, lda0, lda1, ldb0, ldb1, batch_stride_a, batch_stride_b, dtype};
+  return mg::gemm_dispatch("matmul", g, mg::to_stream(stream));
+}
+
+int mg_matmul_bt(const void* a, const void* b, void* dst, int64_t batch, int64_t M, int64_t N, int64_t K, int64_t lda0,
+                 int64_t lda1, int64_t ldb0, int64_t ldb1, int64_t batch_stride_a, int64_t batch_stride_b, int dtype,
+                 mg_stream stream) {
+  // B arrives as (N, K): element (k, n) of the product's right operand is b[n * ldb0 + k * ldb1].
+  mg::GemmArgs g{a, b, nullptr, dst, batch, M, N, K, lda0, lda1, ldb1, ldb0, batch_stride_a, batch_stride_b, dtype};
+  return mg::gemm_dispatch("matmul", g, mg::to_stream(stream));
+}
+
+int mg_matmul_bias_bt(const void* a, const void* b, const void* bias, void* dst, int64_t batch, int64_t M, int64_t N,
+                      int64_t K, int64_t lda0, int64_t lda1, int64_t ldb0, int64_t ldb1, int64_t batch_stride_a,
+                      int64_t batch_stride_b, int dtype, mg_stream stream) {
+  if (!bias) return mg::fail(MG_ERR_INVALID, "matmul_bias: null bias pointer");
+  mg::GemmArgs g{a, b, bias, dst, batch, M, N, K, lda0, lda1, ldb1, ldb0, batch_stride_a, batch_stride_b, dtype};
+  return mg::gemm_dispatch("matmul_bias", g, mg::to_stream(stream));
+}
+
+int mg_linear_bwd(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db, int64_t M, int64_t N,
+                  int64_t K, int dtype, mg_stream stream) {
+  hipStream_t s = mg::to_stream(stream);
+  if (dx) {  // dX (M,K) = dY (M,N) x W (N,K): reduction over N, W read as an n-contiguous right operand
+    mg::GemmArgs g{dy, w, nullptr, dx, 1, M, K, N, N, 1, K, 1, 0, 0, dtype};
+    MG_TRY(mg::gemm_dispatch("linear_bwd(dx)", g, s));
+  }
+  if (dw) {  // dW (N,K) = dY^T (N,M) x X (M,K): reduction over M, dY read as an m-contiguous left operand
+    mg::GemmArgs g{dy, x, nullptr, dw, 1, N, K, M, 1, N, K, 1, 0, 0, dtype};
+    MG_TRY(mg::gemm_dispatch("linear_bwd(dw)", g, s));
+  }
+  if (db) MG_TRY(mg::colsum_dispatch(dy, db, 1, M, N, dtype, s));
+  return MG_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,252 @@
+// Matrix products C = A x B (+ bias) for the Linear forward and its gradients.
+//
+// An operand is described by which of its two dimensions is contiguous in memory:
+//   A (M x K): "k-contiguous"  A[m * lda + k]   (a row-major (M,K) array), or
+//              "m-contiguous"  A[k * lda + m]   (the transposed view of a (K,M) array)
+//   B (K x N): "k-contiguous"  B[n * ldb + k]   (a row-major (N,K) array, i.e. B^T given), or
+//              "n-contiguous"  B[k * ldb + n]   (a row-major (K,N) array)
+// so Y = X W^T is (k,k), dX = dY W is (k,n) and dW = dY^T X is (m,n), all without
+// materialising a transpose.  C is row-major (M,N) with leading dimension ldc.
+//
+// fp32 kernel: 128x128 output tile per 256-thread workgroup, four waves in a 2x2 grid,
+// each wave a 64x64 tile as 2x2 v_mfma_f32_32x32x2_f32 accumulators (64 registers).
+// A K-chunk of 32 is staged through LDS: global -> registers (prefetch of the next
+// chunk overlaps the MFMAs of the current one) -> LDS -> MFMA operands.
+#pragma once
+
+#include "mg_device.h"
+#include "mg_internal.h"
+
+namespace mg {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kGemmBM = 128;
+constexpr int kGemmBN = 128;
+constexpr int kGemmBK = 32;
+constexpr int kGemmThreads = 256;
+constexpr int kKcStride = kGemmBK + 4;  // floats per LDS row of a k-contiguous operand tile
+
+// Workgroup -> output tile.  Consecutive workgroup ids go to different XCDs (id % 8), each
+// with its own L2; ids are regrouped so that one XCD works on a compact block of tiles
+// that share operand rows and columns.
+__device__ __forceinline__ void gemm_tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  constexpr int kXcd = 8;
+  int id = bid;
+  if (total % kXcd == 0) id = (bid % kXcd) * (total / kXcd) + bid / kXcd;
+  // Raster in bands of 4 tile-rows so that a band's A rows stay in L2.
+  constexpr int kBand = 4;
+  const int band_tiles = kBand * tiles_n;
+  const int band = id / band_tiles;
+  const int in_band = id % band_tiles;
+  const int rows_here = min(kBand, tiles_m - band * kBand);
+  tm = band * kBand + in_band % rows_here;
+  tn = in_band / rows_here;
+}
+
+// Registers holding one thread's share of a 128 x 32 (or 32 x 128) operand tile.
+struct GemmStage {
+  float4 v[4];
+};
+
+// Loads the tile of an operand whose "outer" index (m for A, n for B) starts at `o0` and
+// whose k index starts at `k0`.  KC: element (o, k) at base[o * ld + k]; else base[k * ld + o].
+template <bool KC>
+__device__ __forceinline__ void gemm_load_tile(const float* __restrict__ base, int64_t ld, int o0, int k0, int O, int K,
+                                               GemmStage& st) {
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = t + i * kGemmThreads;
+    if constexpr (KC) {
+      const int o = o0 + idx / 8;
+      const int k = k0 + (idx % 8) * 4;
+      const int oc = min(o, O - 1);  // rows past the edge are never stored
+      st.v[i] = k < K ? *reinterpret_cast<const float4*>(base + static_cast<int64_t>(oc) * ld + k)
+                      : make_float4(0.f, 0.f, 0.f, 0.f);
+    } else {
+      const int k = k0 + idx / 32;
+      const int o = o0 + (idx % 32) * 4;
+      st.v[i] = (k < K && o < O) ? *reinterpret_cast<const float4*>(base + static_cast<int64_t>(k) * ld + o)
+                                 : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  }
+}
+
+template <bool KC>
+__device__ __forceinline__ void gemm_store_tile(float* __restrict__ lds, const GemmStage& st) {
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = t + i * kGemmThreads;
+    if constexpr (KC) {
+      *reinterpret_cast<float4*>(lds + (idx / 8) * kKcStride + (idx % 8) * 4) = st.v[i];
+    } else {
+      *reinterpret_cast<float4*>(lds + (idx / 32) * kGemmBM + (idx % 32) * 4) = st.v[i];
+    }
+  }
+}
+
+// MFMA operand values of one 32-wide tile for one group of 8 k-values: lane (o = l % 32,
+// h = l / 32) takes k = g*8 + h*4 + j for j = 0..3, so MFMA j of the group multiplies
+// k in {g*8 + j, g*8 + 4 + j}: each k is used exactly once, in an order that lets a
+// k-contiguous operand be read with one 128-bit LDS load.
+template <bool KC>
+__device__ __forceinline__ void gemm_read_frag(const float* __restrict__ lds, int o_base, int g, float (&f)[4]) {
+  const int lane = threadIdx.x % kWave;
+  const int o = o_base + lane % 32;
+  const int k = g * 8 + (lane / 32) * 4;
+  if constexpr (KC) {
+    const float4 r = *reinterpret_cast<const float4*>(lds + o * kKcStride + k);
+    f[0] = r.x; f[1] = r.y; f[2] = r.z; f[3] = r.w;
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) f[j] = lds[(k + j) * kGemmBM + o];
+  }
+}
+
+template <bool A_KC, bool B_KC, bool HAS_BIAS>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_kernel(
+    const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias, float* __restrict__ C,
+    int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb, int64_t bsc, int tiles_m,
+    int tiles_n) {
+  __shared__ __attribute__((aligned(16))) float lds_a[kGemmBM * kKcStride];
+  __shared__ __attribute__((aligned(16))) float lds_b[kGemmBN * kKcStride];
+
+  const int tiles = tiles_m * tiles_n;
+  const int batch = blockIdx.x / tiles;
+  int tm, tn;
+  gemm_tile_of_block(blockIdx.x % tiles, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * kGemmBM;
+  const int n0 = tn * kGemmBN;
+  A += batch * bsa;
+  B += batch * bsb;
+  C += batch * bsc;
+
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int wm = (wave / 2) * 64;
+  const int wn = (wave % 2) * 64;
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  GemmStage sa, sb;
+  gemm_load_tile<A_KC>(A, lda, m0, 0, M, K, sa);
+  gemm_load_tile<B_KC>(B, ldb, n0, 0, N, K, sb);
+
+  for (int k0 = 0; k0 < K; k0 += kGemmBK) {
+    gemm_store_tile<A_KC>(lds_a, sa);
+    gemm_store_tile<B_KC>(lds_b, sb);
+    __syncthreads();
+    if (k0 + kGemmBK < K) {
+      gemm_load_tile<A_KC>(A, lda, m0, k0 + kGemmBK, M, K, sa);
+      gemm_load_tile<B_KC>(B, ldb, n0, k0 + kGemmBK, N, K, sb);
+    }
+#pragma unroll
+    for (int g = 0; g < kGemmBK / 8; ++g) {
+      float fa[2][4], fb[2][4];
+      gemm_read_frag<A_KC>(lds_a, wm, g, fa[0]);
+      gemm_read_frag<A_KC>(lds_a, wm + 32, g, fa[1]);
+      gemm_read_frag<B_KC>(lds_b, wn, g, fb[0]);
+      gemm_read_frag<B_KC>(lds_b, wn + 32, g, fb[1]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+          for (int tj = 0; tj < 2; ++tj)
+            acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[ti][j], fb[tj][j], acc[ti][tj], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // Accumulator element r of a lane is row (r/4)*8 + (lane/32)*4 + r%4, column lane%32.
+#pragma unroll
+  for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+      const int col = n0 + wn + tj * 32 + lane % 32;
+      if (col >= N) continue;
+      const float bv = HAS_BIAS ? bias[col] : 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + wm + ti * 32 + (r / 4) * 8 + (lane / 32) * 4 + (r % 4);
+        if (row < M) C[static_cast<int64_t>(row) * ldc + col] = acc[ti][tj][r] + bv;
+      }
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// Any strides, any of the three float types: 64x64 tile, 256 threads, 4x4 outputs per
+// thread, fp32 FMA.  The path for operands the MFMA kernels cannot take (unaligned
+// leading dimensions, both strides non-unit, skinny edge shapes).
+//   A element (m, k) at A[m * sam + k * sak];  B element (k, n) at B[k * sbk + n * sbn].
+// ------------------------------------------------------------------------------------
+
+template <typename T, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__ A, const T* __restrict__ B,
+                                                           const T* __restrict__ bias, T* __restrict__ C, int M, int N,
+                                                           int K, int64_t sam, int64_t sak, int64_t sbk, int64_t sbn,
+                                                           int64_t ldc, int64_t bsa, int64_t bsb, int64_t bsc) {
+  constexpr int TM = 64, TN = 64, TK = 16;
+  __shared__ float as[TK][TM + 1];
+  __shared__ float bs[TK][TN + 1];
+  const int batch = blockIdx.z;
+  A += batch * bsa;
+  B += batch * bsb;
+  C += batch * bsc;
+  const int m0 = blockIdx.y * TM;
+  const int n0 = blockIdx.x * TN;
+  const int tx = threadIdx.x % 16;
+  const int ty = threadIdx.x / 16;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += TK) {
+    for (int idx = threadIdx.x; idx < TM * TK; idx += 256) {
+      // Walk the contiguous dimension fastest for whichever stride is 1.
+      int m, k;
+      if (sak == 1) { k = idx % TK; m = idx / TK; } else { m = idx % TM; k = idx / TM; }
+      const int gm = m0 + m, gk = k0 + k;
+      as[k][m] = (gm < M && gk < K) ? to_float(A[gm * sam + gk * sak]) : 0.f;
+    }
+    for (int idx = threadIdx.x; idx < TN * TK; idx += 256) {
+      int n, k;
+      if (sbk == 1) { k = idx % TK; n = idx / TK; } else { n = idx % TN; k = idx / TN; }
+      const int gn = n0 + n, gk = k0 + k;
+      bs[k][n] = (gn < N && gk < K) ? to_float(B[gk * sbk + gn * sbn]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < TK; ++k) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = as[k][ty + i * 16];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = bs[k][tx + j * 16];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int gm = m0 + ty + i * 16, gn = n0 + tx + j * 16;
+      if (gm < M && gn < N) {
+        const float bv = HAS_BIAS ? to_float(bias[gn]) : 0.f;
+        C[static_cast<int64_t>(gm) * ldc + gn] = from_float<T>(acc[i][j] + bv);
+      }
+    }
+}
+
+}  // namespace mg

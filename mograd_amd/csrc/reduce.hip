@@ -1,0 +1,191 @@
+// Axis sums (the bias gradient db = sum over rows of dY) and relu_grad.
+#include "mg_device.h"
+#include "mg_internal.h"
+#include "mg_rows.h"
+
+namespace mg {
+
+// Stage 1 of dst(o, i) = sum_r a(o, r, i): each workgroup sums a slab of `rows_per_chunk`
+// rows for 256 * VEC columns with 16-byte loads.  DIRECT writes the final value (one
+// slab covers the whole axis); otherwise fp32 partials (outer, chunks, inner) go to
+// scratch and reduce_partials_kernel finishes in a fixed order.  No atomics.
+template <typename T, int VEC, bool DIRECT>
+__global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict__ a, float* __restrict__ part,
+                                                             T* __restrict__ dst, int64_t reduce, int64_t inner,
+                                                             int64_t rows_per_chunk) {
+  const int64_t col = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * VEC;
+  if (col >= inner) return;
+  const int64_t chunk = blockIdx.y;
+  const int64_t o = blockIdx.z;
+  const int64_t r0 = chunk * rows_per_chunk;
+  const int64_t r1 = min(r0 + rows_per_chunk, reduce);
+  const T* base = a + (o * reduce) * inner + col;
+  float acc[4][VEC];
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[u][e] = 0.f;
+  int64_t r = r0;
+  for (; r + 3 < r1; r += 4) {
+    float v[4][VEC];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) VecIO<T, VEC>::load(base + (r + u) * inner, v[u]);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[u][e] += v[u][e];
+  }
+  for (; r < r1; ++r) {
+    float v[VEC];
+    VecIO<T, VEC>::load(base + r * inner, v);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[0][e] += v[e];
+  }
+  float out[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) out[e] = (acc[0][e] + acc[1][e]) + (acc[2][e] + acc[3][e]);
+  if constexpr (DIRECT) {
+    VecIO<T, VEC>::store(dst + o * inner + col, out);
+  } else {
+    float* p = part + (o * gridDim.y + chunk) * inner + col;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) p[e] = out[e];
+  }
+}
+
+// Sum over the last axis (inner == 1): one wave per output element.
+template <typename T>
+__global__ __launch_bounds__(256) void rowsum_kernel(const T* __restrict__ a, T* __restrict__ dst, int64_t outer,
+                                                     int64_t reduce) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+  if (row >= outer) return;  // wave-uniform
+  const int lane = threadIdx.x % kWave;
+  float acc = 0.f;
+  for (int64_t c = lane; c < reduce; c += kWave) acc += to_float(a[row * reduce + c]);
+  acc = wave_sum(acc);
+  if (lane == 0) dst[row] = from_float<T>(acc);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void relu_grad_kernel(const T* __restrict__ out, const T* __restrict__ up,
+                                                        T* __restrict__ dst, int64_t n) {
+  constexpr int VEC = WideVec<T>::value;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256 * VEC;
+  for (int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * VEC; i < n; i += stride) {
+    if (i + VEC <= n) {
+      float o[VEC], u[VEC], r[VEC];
+      VecIO<T, VEC>::load(out + i, o);
+      VecIO<T, VEC>::load(up + i, u);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) r[e] = o[e] > 0.f ? u[e] : 0.f;
+      VecIO<T, VEC>::store(dst + i, r);
+    } else {
+      for (int64_t j = i; j < n; ++j) dst[j] = to_float(out[j]) > 0.f ? up[j] : from_float<T>(0.f);
+    }
+  }
+}
+
+template <typename T>
+static int colsum_typed(const T* a, T* dst, int64_t outer, int64_t reduce, int64_t inner, hipStream_t stream) {
+  if (reduce == 0) {
+    MG_HIP(hipMemsetAsync(dst, 0, static_cast<size_t>(outer * inner) * sizeof(T), stream));
+    return MG_OK;
+  }
+  if (inner == 1) {
+    hipLaunchKernelGGL((rowsum_kernel<T>), dim3(static_cast<unsigned>(ceil_div(outer, 4))), dim3(256), 0, stream, a, dst,
+                       outer, reduce);
+    MG_LAUNCH_CHECK();
+    return MG_OK;
+  }
+  constexpr int WIDE = WideVec<T>::value;
+  const bool wide = inner % WIDE == 0 && aligned16(a) && aligned16(dst);
+  const int vec = wide ? WIDE : 1;
+  const int64_t col_blocks = ceil_div(inner, 256 * vec);
+  if (outer > 65535) return fail(MG_ERR_UNSUPPORTED, "sum_axis: outer=%lld exceeds 65535", static_cast<long long>(outer));
+  // Enough slabs to fill the device, each at least 8 rows.
+  int64_t chunks = ceil_div(static_cast<int64_t>(device_info().cu_count) * 4, col_blocks * outer);
+  const int64_t max_chunks = ceil_div(reduce, 8);
+  if (chunks > max_chunks) chunks = max_chunks;
+  if (chunks < 1) chunks = 1;
+  if (chunks > 65535) chunks = 65535;
+  const int64_t rows_per_chunk = ceil_div(reduce, chunks);
+  chunks = ceil_div(reduce, rows_per_chunk);
+  const dim3 grid(static_cast<unsigned>(col_blocks), static_cast<unsigned>(chunks), static_cast<unsigned>(outer));
+  if (chunks == 1) {
+    if (wide)
+      hipLaunchKernelGGL((colsum_partial_kernel<T, WIDE, true>), grid, dim3(256), 0, stream, a, nullptr, dst, reduce,
+                         inner, rows_per_chunk);
+    else
+      hipLaunchKernelGGL((colsum_partial_kernel<T, 1, true>), grid, dim3(256), 0, stream, a, nullptr, dst, reduce, inner,
+                         rows_per_chunk);
+    MG_LAUNCH_CHECK();
+    return MG_OK;
+  }
+  Scratch part;
+  MG_TRY(part.take(outer * chunks * inner * static_cast<int64_t>(sizeof(float))));
+  if (wide)
+    hipLaunchKernelGGL((colsum_partial_kernel<T, WIDE, false>), grid, dim3(256), 0, stream, a, part.as<float>(), dst,
+                       reduce, inner, rows_per_chunk);
+  else
+    hipLaunchKernelGGL((colsum_partial_kernel<T, 1, false>), grid, dim3(256), 0, stream, a, part.as<float>(), dst,
+                       reduce, inner, rows_per_chunk);
+  MG_LAUNCH_CHECK();
+  for (int64_t o = 0; o < outer; ++o) {
+    hipLaunchKernelGGL((reduce_partials_kernel<T>), dim3(static_cast<unsigned>(ceil_div(inner, 64)), 1), dim3(256), 0,
+                       stream, part.as<float>() + o * chunks * inner, dst + o * inner, nullptr, nullptr, chunks, inner);
+    MG_LAUNCH_CHECK();
+  }
+  return MG_OK;
+}
+
+int colsum_dispatch(const void* a, void* dst, int64_t outer, int64_t reduce, int64_t inner, int dtype,
+                    hipStream_t stream) {
+  if (!is_float_dtype(dtype)) return fail(MG_ERR_INVALID, "sum_axis: unsupported dtype %s", dtype_name(dtype));
+  if (outer < 0 || reduce < 0 || inner < 0)
+    return fail(MG_ERR_INVALID, "sum_axis: bad shape (%lld, %lld, %lld)", static_cast<long long>(outer),
+                static_cast<long long>(reduce), static_cast<long long>(inner));
+  if (outer == 0 || inner == 0) return MG_OK;
+  if (!dst || (reduce > 0 && !a)) return fail(MG_ERR_INVALID, "sum_axis: null pointer argument");
+  switch (dtype) {
+    case MG_F32: return colsum_typed(static_cast<const float*>(a), static_cast<float*>(dst), outer, reduce, inner, stream);
+    case MG_F16: return colsum_typed(static_cast<const f16_t*>(a), static_cast<f16_t*>(dst), outer, reduce, inner, stream);
+    default: return colsum_typed(static_cast<const bf16_t*>(a), static_cast<bf16_t*>(dst), outer, reduce, inner, stream);
+  }
+}
+
+template <typename T>
+static int relu_grad_typed(const void* out, const void* up, void* dst, int64_t n, hipStream_t stream) {
+  constexpr int VEC = WideVec<T>::value;
+  if (!aligned16(out) || !aligned16(up) || !aligned16(dst))
+    return fail(MG_ERR_INVALID, "relu_grad: pointers must be 16-byte aligned");
+  int64_t blocks = ceil_div(n, 256 * VEC);
+  const int64_t cap = static_cast<int64_t>(device_info().cu_count) * 16;
+  if (blocks > cap) blocks = cap;
+  hipLaunchKernelGGL((relu_grad_kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
+                     static_cast<const T*>(out), static_cast<const T*>(up), static_cast<T*>(dst), n);
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+}  // namespace mg
+
+extern "C" {
+
+int mg_sum_axis(const void* a, void* dst, int64_t outer, int64_t reduce, int64_t inner, int dtype, mg_stream stream) {
+  return mg::colsum_dispatch(a, dst, outer, reduce, inner, dtype, mg::to_stream(stream));
+}
+
+int mg_relu_grad(const void* out, const void* upstream, void* dst, int64_t n, int dtype, mg_stream stream) {
+  if (!mg::is_float_dtype(dtype)) return mg::fail(MG_ERR_INVALID, "relu_grad: unsupported dtype %s", mg::dtype_name(dtype));
+  if (n < 0) return mg::fail(MG_ERR_INVALID, "relu_grad: negative size");
+  if (n == 0) return MG_OK;
+  if (!out || !upstream || !dst) return mg::fail(MG_ERR_INVALID, "relu_grad: null pointer argument");
+  hipStream_t s = mg::to_stream(stream);
+  switch (dtype) {
+    case MG_F32: return mg::relu_grad_typed<float>(out, upstream, dst, n, s);
+    case MG_F16: return mg::relu_grad_typed<mg::f16_t>(out, upstream, dst, n, s);
+    default: return mg::relu_grad_typed<mg::bf16_t>(out, upstream, dst, n, s);
+  }
+}
+
+}  // extern "C"

@@ -49,13 +49,18 @@ def assert_close(got, want, rtol, atol, what=""):
 
 
 def assert_sum_close(got, want, term_l1, rtol=RTOL_F32, atol=ATOL_F32, what=""):
-    """For an fp32 sum of many terms: rtol against the value, plus an absolute floor of
-    `atol` scaled by the mean magnitude of what was summed (term_l1 / 1 per output), i.e.
-    the floor is relative to the size of the summands rather than to a result that may
-    have cancelled to near zero."""
+    """For an fp32 sum of many terms (column sums, dot products of a matmul).
+
+    The parity tolerance rtol/atol applies to the value; on top of it the absolute floor
+    is never below 16 * 2^-24 * sum|terms|: an fp32 accumulator cannot resolve less than
+    about one unit roundoff of the mass it has summed, so a result that cancelled to near
+    zero is held to the rounding of its summands, not of itself.  `term_l1` is that mass
+    per output element.
+    """
     got = np.asarray(got, dtype=np.float64)
     want = np.asarray(want, dtype=np.float64)
-    floor = atol * np.maximum(1.0, np.asarray(term_l1, dtype=np.float64))
+    assert got.shape == want.shape, (got.shape, want.shape)
+    floor = np.maximum(atol, 16.0 * 2.0 ** -24 * np.asarray(term_l1, dtype=np.float64))
     err = np.abs(got - want)
     bound = floor + rtol * np.abs(want)
     worst = float(np.max(err / bound))

@@ -1,0 +1,174 @@
+"""Matmul family and Linear gradients on the GPU against the float64 oracle.
+
+The operand layouts are the ones mograd's graph produces for a Linear layer
+(mograd/grad.mojo:180-187, mograd/runtime/gpu/rewrites.mojo:163-174): forward
+X W^T + b, dX = MATMUL_BT(dY, TRANSPOSE(W)) with a strided right operand, and
+dW^T = MATMUL(TRANSPOSE(X), dY) with a strided left operand; db = SUM(axis=0).
+"""
+import numpy as np
+import pytest
+
+from helpers import ATOL_F32, RTOL_F32, assert_close, assert_sum_close, normal, uniform
+from oracle import oracle_np as O
+
+pytestmark = pytest.mark.gpu
+
+from mograd_amd import BF16, F16, F32, AnyBuffer, Layout, MogradError, Node  # noqa: E402
+from mograd_amd import runtime as R  # noqa: E402
+from mograd_amd.runtime import round_to_dtype  # noqa: E402
+
+
+def _run(device, op, out_layout, operands, dtype=F32, attrs=None):
+    """operands: list of (host array, layout view over it)."""
+    srcs = [Node.leaf(l, dtype) for _, l in operands]
+    node = Node(op, out_layout, dtype, srcs, attrs or {})
+    bufs = [AnyBuffer.from_numpy(device, a, dtype).view(l) for a, l in operands]
+    (out,) = R.run(node, bufs, device)
+    return out.to_numpy(out_layout.shape())
+
+
+def _linear_all(device, x, w, b, dy, dtype=F32):
+    """Forward and the three gradients, each through the scheduler entry the reference's
+    graph reaches."""
+    M, K = x.shape
+    N = w.shape[0]
+    y = _run(device, "MATMUL_BIAS_BT", Layout(M, N), [(x, Layout(M, K)), (w, Layout(N, K)), (b, Layout(N))], dtype)
+    # dX = MATMUL_BT(dY, W^T view): the right operand is the (K, N) transposed view of W
+    dx = _run(device, "MATMUL_BT", Layout(M, K), [(dy, Layout(M, N)), (w, Layout(N, K).transpose())], dtype)
+    # dW^T = MATMUL(X^T view, dY), shape (K, N)
+    dwt = _run(device, "MATMUL", Layout(K, N), [(x, Layout(M, K).transpose()), (dy, Layout(M, N))], dtype)
+    db = _run(device, "SUM", Layout(N), [(dy, Layout(M, N))], dtype, {"axis": 0})
+    return y, dx, dwt.T, db
+
+
+SHAPES = [(64, 10, 256), (64, 256, 784), (128, 128, 128), (256, 384, 512), (200, 136, 260), (130, 65, 384),
+          (1, 8, 16), (33, 7, 5), (512, 1024, 256), (300, 128, 1000)]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_linear_fwd_and_grads_f32(device, M, N, K):
+    x = normal(40, 0, (M, K))
+    bound = np.sqrt(6.0 / K)
+    w = uniform(40, 1, (N, K), -bound, bound)
+    b = uniform(40, 2, (N,), -bound, bound)
+    dy = normal(40, 3, (M, N))
+    y, dx, dw, db = _linear_all(device, x, w, b, dy)
+    # each output is a dot product of length K, N or M: tolerance at the parity rtol
+    # against the value, with the absolute floor scaled by the dot product's L1 mass
+    assert_sum_close(y, O.matmul_bias_bt(x, w, b), np.abs(x) @ np.abs(w).T, what="y")
+    assert_sum_close(dx, O.linear_grad_x(dy, w), np.abs(dy) @ np.abs(w), what="dx")
+    assert_sum_close(dw, O.linear_grad_w(dy, x), np.abs(dy).T @ np.abs(x), what="dw")
+    assert_sum_close(db, O.linear_grad_b(dy), np.abs(dy).sum(axis=0), what="db")
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 256, 512), (200, 136, 260), (64, 10, 256)])
+def test_linear_bwd_entry(device, M, N, K):
+    x, w, dy = normal(41, 0, (M, K)), normal(41, 1, (N, K)), normal(41, 2, (M, N))
+    bx, bw, bdy = (AnyBuffer.from_numpy(device, a) for a in (x, w, dy))
+    dx, dw, db = (AnyBuffer.create(F32, device, n) for n in (M * K, N * K, N))
+    device.lib.mg_linear_bwd(bdy.data_ptr(), bx.data_ptr(), bw.data_ptr(), dx.data_ptr(), dw.data_ptr(),
+                             db.data_ptr(), M, N, K, F32, device.stream)
+    assert_sum_close(dx.to_numpy((M, K)), O.linear_grad_x(dy, w), np.abs(dy) @ np.abs(w), what="dx")
+    assert_sum_close(dw.to_numpy((N, K)), O.linear_grad_w(dy, x), np.abs(dy).T @ np.abs(x), what="dw")
+    assert_sum_close(db.to_numpy(), O.linear_grad_b(dy), np.abs(dy).sum(axis=0), what="db")
+
+
+def test_batched_rank3_and_broadcast_weight(device):
+    # (B, T, K) activations against one (N, K) weight: the GPT's Linear layers
+    Bt, T, K, N = 3, 40, 64, 96
+    x = normal(42, 0, (Bt, T, K))
+    w = normal(42, 1, (N, K))
+    out = _run(device, "MATMUL_BT", Layout(Bt, T, N),
+               [(x, Layout(Bt, T, K)), (w, Layout(Bt, N, K, strides=(0, K, 1)))])
+    assert_sum_close(out, np.einsum("btk,nk->btn", x.astype(np.float64), w), 
+                     np.einsum("btk,nk->btn", np.abs(x), np.abs(w)), what="batched")
+
+
+def test_mlp_chain_matches_oracle(device):
+    # MNIST-shaped MLP 64x784 -> 256 (ReLU) -> 10, CE on labels: the whole gradient chain
+    # CE grad -> dW2, db2, dX -> ReLU grad -> dW1, db1
+    M, D0, D1, D2 = 64, 784, 256, 10
+    x = normal(1, 0, (M, D0))
+    w1 = uniform(1, 1, (D1, D0), -np.sqrt(6 / D0), np.sqrt(6 / D0))
+    b1 = uniform(1, 2, (D1,), -np.sqrt(6 / D0), np.sqrt(6 / D0))
+    w2 = uniform(1, 3, (D2, D1), -np.sqrt(6 / D1), np.sqrt(6 / D1))
+    b2 = uniform(1, 4, (D2,), -np.sqrt(6 / D1), np.sqrt(6 / D1))
+    ids = np.random.Generator(np.random.PCG64(1005)).integers(0, D2, M)
+    onehot = O.one_hot(ids, D2).astype(np.float32)
+    # oracle
+    h_pre = O.matmul_bias_bt(x, w1, b1)
+    h = np.maximum(h_pre, 0)
+    logits = O.matmul_bias_bt(h, w2, b2)
+    want_loss = O.cross_entropy(logits, onehot)
+    dlogits = O.cross_entropy_grad(logits, onehot)
+    want = {"dw2": O.linear_grad_w(dlogits, h), "db2": O.linear_grad_b(dlogits)}
+    dh = O.relu_grad(h, O.linear_grad_x(dlogits, w2))
+    want.update({"dw1": O.linear_grad_w(dh, x), "db1": O.linear_grad_b(dh)})
+    # GPU, buffers stay on the device between ops
+    lib, st = device.lib, device.stream
+    up = lambda a: AnyBuffer.from_numpy(device, a)  # noqa: E731
+    bx, bw1, bb1, bw2, bb2, by = up(x), up(w1), up(b1), up(w2), up(b2), up(onehot)
+    one = up(np.ones(1, np.float32))
+    new = lambda n: AnyBuffer.create(F32, device, n)  # noqa: E731
+    hpre, hb, lg, loss, dlg = new(M * D1), new(M * D1), new(M * D2), new(1), new(M * D2)
+    lib.mg_matmul_bias_bt(bx.data_ptr(), bw1.data_ptr(), bb1.data_ptr(), hpre.data_ptr(), 1, M, D1, D0, D0, 1, D0, 1,
+                          M * D0, D1 * D0, F32, st)
+    # relu forward is outside this path: relu(h_pre) == relu_grad(h_pre, h_pre)
+    lib.mg_relu_grad(hpre.data_ptr(), hpre.data_ptr(), hb.data_ptr(), M * D1, F32, st)
+    lib.mg_matmul_bias_bt(hb.data_ptr(), bw2.data_ptr(), bb2.data_ptr(), lg.data_ptr(), 1, M, D2, D1, D1, 1, D1, 1,
+                          M * D1, D2 * D1, F32, st)
+    lib.mg_cross_entropy(lg.data_ptr(), by.data_ptr(), loss.data_ptr(), M, D2, F32, st)
+    lib.mg_cross_entropy_grad(lg.data_ptr(), by.data_ptr(), one.data_ptr(), dlg.data_ptr(), M, D2, F32, st)
+    dw2, db2, dhb, dh2, dw1, db1 = new(D2 * D1), new(D2), new(M * D1), new(M * D1), new(D1 * D0), new(D1)
+    lib.mg_linear_bwd(dlg.data_ptr(), hb.data_ptr(), bw2.data_ptr(), dhb.data_ptr(), dw2.data_ptr(), db2.data_ptr(),
+                      M, D2, D1, F32, st)
+    lib.mg_relu_grad(hb.data_ptr(), dhb.data_ptr(), dh2.data_ptr(), M * D1, F32, st)
+    lib.mg_linear_bwd(dh2.data_ptr(), bx.data_ptr(), bw1.data_ptr(), None, dw1.data_ptr(), db1.data_ptr(), M, D1, D0,
+                      F32, st)
+    assert_close(loss.item(), want_loss, RTOL_F32, ATOL_F32, "loss")
+    got = {"dw2": dw2.to_numpy((D2, D1)), "db2": db2.to_numpy(), "dw1": dw1.to_numpy((D1, D0)), "db1": db1.to_numpy()}
+    for k in want:
+        assert_close(got[k], want[k], RTOL_F32, ATOL_F32, k)
+
+
+@pytest.mark.parametrize("dtype,rtol", [(F16, 2e-3), (BF16, 1.6e-2)])
+def test_half_precision_storage(device, dtype, rtol):
+    M, N, K = 96, 80, 136
+    x = round_to_dtype(normal(43, 0, (M, K)), dtype)
+    w = round_to_dtype(normal(43, 1, (N, K), std=0.1), dtype)
+    b = round_to_dtype(normal(43, 2, (N,), std=0.1), dtype)
+    dy = round_to_dtype(normal(43, 3, (M, N)), dtype)
+    y, dx, dw, db = _linear_all(device, x, w, b, dy, dtype)
+    for got, want, name in ((y, O.matmul_bias_bt(x, w, b), "y"), (dx, O.linear_grad_x(dy, w), "dx"),
+                            (dw, O.linear_grad_w(dy, x), "dw"), (db, O.linear_grad_b(dy), "db")):
+        assert_close(got, want, rtol, rtol * np.abs(want).max(), name)
+
+
+def test_sum_axis_shapes(device):
+    for shape, axis in [((2048, 4096), 0), ((7, 5), 0), ((3, 50, 8), 1), ((4, 6, 10), 2), ((1000, 3), 0), ((2, 3, 4), 0)]:
+        a = normal(44, len(shape) * 10 + axis, shape)
+        out_shape = tuple(s for i, s in enumerate(shape) if i != axis)
+        got = _run(device, "SUM", Layout(*out_shape), [(a, Layout(*shape))], F32, {"axis": axis})
+        assert_sum_close(got, a.astype(np.float64).sum(axis=axis), np.abs(a).sum(axis=axis), what=f"sum{shape}/{axis}")
+
+
+def test_relu_grad(device):
+    for n in (1, 7, 4096, 100003):
+        out = np.maximum(normal(45, n % 97, (n,)), 0)
+        up = normal(45, 1 + n % 97, (n,))
+        got = _run(device, "RELU_GRAD", Layout(n), [(out, Layout(n)), (up, Layout(n))])
+        np.testing.assert_array_equal(got, O.relu_grad(out, up).astype(np.float32))  # a select: bit-exact
+
+
+def test_errors(device):
+    a = normal(46, 0, (2, 3, 4, 5))
+    with pytest.raises(MogradError, match="non-collapsible batch dims"):
+        # transpose(1, 2) of a rank-4 tensor: batch dims no longer fold into one stride
+        _run(device, "MATMUL", Layout(2, 4, 3, 3),
+             [(a, Layout(2, 3, 4, 5).transpose(1, 2)), (a, Layout(2, 3, 4, 5).transpose(1, 2).transpose(2, 3))])
+    buf = AnyBuffer.create(F32, device, 16)
+    p = buf.data_ptr()
+    with pytest.raises(MogradError, match="unsupported dtype"):
+        device.lib.mg_matmul(p, p, p, 1, 2, 2, 2, 2, 1, 2, 1, 4, 4, R.int64, device.stream)
+    with pytest.raises(MogradError, match="null bias"):
+        device.lib.mg_matmul_bias_bt(p, p, None, p, 1, 2, 2, 2, 2, 1, 2, 1, 4, 4, F32, device.stream)
