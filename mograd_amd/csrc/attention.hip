@@ -1,0 +1,117 @@
+// C ABI for flash attention: argument checks, routing between the MFMA kernels (16-bit
+// storage, head dimension up to 128) and the general fp32-arithmetic kernels.
+#include "attention_generic.h"
+#include "mg_internal.h"
+
+namespace mg {
+
+// attention_mfma.hip.  Return MG_ERR_UNSUPPORTED (without setting an error) when the
+// shape is not one the MFMA kernels take.
+bool attn_mfma_supported(int dtype, int64_t D, const void* const* ptrs, int nptrs);
+int attn_fwd_mfma(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, AttnDims a,
+                  float scale, bool causal, bool has_bias, int dtype, hipStream_t stream);
+int attn_bwd_mfma(const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
+                  const float* lse, void* dq, void* dk, void* dv, AttnDims a, float scale, bool causal, bool has_bias,
+                  int dtype, hipStream_t stream);
+
+static int check_attn(const char* who, int64_t B, int64_t S, int64_t H, int64_t D, int causal, int has_bias, int dtype) {
+  if (!is_float_dtype(dtype)) return fail(MG_ERR_INVALID, "%s: unsupported dtype %s", who, dtype_name(dtype));
+  if (D <= 0 || D > 512) return fail(MG_ERR_INVALID, "%s: D=%lld out of range (1..512)", who, static_cast<long long>(D));
+  if (causal != 0 && has_bias != 0)
+    return fail(MG_ERR_INVALID, "%s: causal attention with additive bias is not supported", who);
+  if (B <= 0 || S <= 0 || H <= 0 || B * H * S > 0x7fffffffLL || S > (1 << 24))
+    return fail(MG_ERR_INVALID, "%s: bad shape B=%lld S=%lld H=%lld", who, static_cast<long long>(B),
+                static_cast<long long>(S), static_cast<long long>(H));
+  return MG_OK;
+}
+
+template <typename T>
+static int fwd_generic(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, AttnDims a,
+                       float scale, bool causal, bool has_bias, hipStream_t stream) {
+  const int64_t rows = static_cast<int64_t>(a.B) * a.H * a.S;
+  const dim3 grid(static_cast<unsigned>(ceil_div(rows, 4)));
+#define MG_FWD(C_, B_)                                                                                              \
+  hipLaunchKernelGGL((attn_fwd_generic_kernel<T, C_, B_>), grid, dim3(256), 0, stream, static_cast<const T*>(q),    \
+                     static_cast<const T*>(k), static_cast<const T*>(v), static_cast<const T*>(mask),               \
+                     static_cast<T*>(o), lse, a, scale)
+  if (causal) MG_FWD(true, false);
+  else if (has_bias) MG_FWD(false, true);
+  else MG_FWD(false, false);
+#undef MG_FWD
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+template <typename T>
+static int bwd_generic(const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
+                       const float* lse, void* dq, void* dk, void* dv, AttnDims a, float scale, bool causal,
+                       bool has_bias, hipStream_t stream) {
+  const int64_t rows = static_cast<int64_t>(a.B) * a.H * a.S;
+  Scratch delta;
+  MG_TRY(delta.take(rows * static_cast<int64_t>(sizeof(float))));
+  const dim3 grid(static_cast<unsigned>(ceil_div(rows, 4)));
+  hipLaunchKernelGGL((attn_delta_kernel<T>), grid, dim3(256), 0, stream, static_cast<const T*>(d_o),
+                     static_cast<const T*>(o), delta.as<float>(), rows, a.D);
+  MG_LAUNCH_CHECK();
+#define MG_BWD(C_, B_)                                                                                                \
+  do {                                                                                                                \
+    hipLaunchKernelGGL((attn_dq_generic_kernel<T, C_, B_>), grid, dim3(256), 0, stream, static_cast<const T*>(d_o),   \
+                       static_cast<const T*>(q), static_cast<const T*>(k), static_cast<const T*>(v),                  \
+                       static_cast<const T*>(mask), lse, delta.as<float>(), static_cast<T*>(dq), a, scale);           \
+    hipLaunchKernelGGL((attn_dkdv_generic_kernel<T, C_, B_>), grid, dim3(256), 0, stream, static_cast<const T*>(d_o), \
+                       static_cast<const T*>(q), static_cast<const T*>(k), static_cast<const T*>(v),                  \
+                       static_cast<const T*>(mask), lse, delta.as<float>(), static_cast<T*>(dk), static_cast<T*>(dv), \
+                       a, scale);                                                                                     \
+  } while (0)
+  if (causal) MG_BWD(true, false);
+  else if (has_bias) MG_BWD(false, true);
+  else MG_BWD(false, false);
+#undef MG_BWD
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+}  // namespace mg
+
+extern "C" {
+
+int mg_flash_attn_fwd(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, int64_t B,
+                      int64_t S, int64_t H, int64_t D, float scale, int causal, int has_bias, int dtype,
+                      mg_stream stream) {
+  MG_TRY(mg::check_attn("flash_attn_fwd", B, S, H, D, causal, has_bias, dtype));
+  if (!q || !k || !v || !o || !lse || (has_bias && !mask))
+    return mg::fail(MG_ERR_INVALID, "flash_attn_fwd: null pointer argument");
+  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D)};
+  hipStream_t s = mg::to_stream(stream);
+  const void* ptrs[] = {q, k, v, o, has_bias ? mask : nullptr};
+  if (mg::attn_mfma_supported(dtype, D, ptrs, 5))
+    return mg::attn_fwd_mfma(q, k, v, mask, o, lse, a, scale, causal != 0, has_bias != 0, dtype, s);
+  switch (dtype) {
+    case MG_F32: return mg::fwd_generic<float>(q, k, v, mask, o, lse, a, scale, causal != 0, has_bias != 0, s);
+    case MG_F16: return mg::fwd_generic<mg::f16_t>(q, k, v, mask, o, lse, a, scale, causal != 0, has_bias != 0, s);
+    default: return mg::fwd_generic<mg::bf16_t>(q, k, v, mask, o, lse, a, scale, causal != 0, has_bias != 0, s);
+  }
+}
+
+int mg_flash_attn_bwd(const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
+                      const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t S, int64_t H, int64_t D,
+                      float scale, int causal, int has_bias, int dtype, mg_stream stream) {
+  MG_TRY(mg::check_attn("flash_attn_bwd", B, S, H, D, causal, has_bias, dtype));
+  if (!d_o || !o || !q || !k || !v || !lse || !dq || !dk || !dv || (has_bias && !mask))
+    return mg::fail(MG_ERR_INVALID, "flash_attn_bwd: null pointer argument");
+  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D)};
+  hipStream_t s = mg::to_stream(stream);
+  const void* ptrs[] = {d_o, o, q, k, v, dq, dk, dv, has_bias ? mask : nullptr};
+  if (mg::attn_mfma_supported(dtype, D, ptrs, 9))
+    return mg::attn_bwd_mfma(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal != 0, has_bias != 0, dtype, s);
+  switch (dtype) {
+    case MG_F32:
+      return mg::bwd_generic<float>(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal != 0, has_bias != 0, s);
+    case MG_F16:
+      return mg::bwd_generic<mg::f16_t>(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal != 0, has_bias != 0, s);
+    default:
+      return mg::bwd_generic<mg::bf16_t>(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal != 0, has_bias != 0, s);
+  }
+}
+
+}  // extern "C"

@@ -1,0 +1,186 @@
+"""Flash attention forward/backward on the GPU against the float64 oracle.
+
+Follows the reference's attention tests: the f64 oracle and error budgets of
+tests/kernels/attention/{harness,generic,mma}.mojo, the closed forms of
+tests/test_ops.mojo:903-946 and tests/test_grad.mojo:1001-1023, through the same
+dispatch surface (FLASH_ATTN / FLASH_ATTN_GRAD nodes).
+"""
+import math
+
+import numpy as np
+import pytest
+
+from helpers import RTOL_BF16_ATTN, normal
+from oracle import oracle_np as O
+
+pytestmark = pytest.mark.gpu
+
+from mograd_amd import BF16, F16, F32, AnyBuffer, Layout, MogradError, Node  # noqa: E402
+from mograd_amd import runtime as R  # noqa: E402
+from mograd_amd.runtime import round_to_dtype  # noqa: E402
+
+
+def _fwd(device, q, k, v, mask, causal, scale, dtype):
+    B, S, H, D = q.shape
+    attrs = {"scale": scale, "is_causal": causal, "has_bias": mask is not None}
+    m = mask if mask is not None else np.zeros(8, np.float32)  # placeholder the kernels never read
+    srcs = [Node.leaf(Layout(B, S, H, D), dtype)] * 3 + [Node.leaf(Layout(*m.shape), dtype)]
+    node = Node("FLASH_ATTN", Layout(B, H, S, D), dtype, srcs, attrs)
+    bufs = [AnyBuffer.from_numpy(device, a, dtype) for a in (q, k, v, m)]
+    o, lse = R.run(node, bufs, device)
+    return o, lse, bufs
+
+
+def _fwd_bwd(device, q, k, v, do, mask=None, causal=False, scale=None, dtype=F32):
+    """Forward for O/LSE chained into the backward, as the reference's run_bwd does
+    (tests/kernels/attention/harness.mojo:266-344)."""
+    B, S, H, D = q.shape
+    scale = scale if scale is not None else 1.0 / math.sqrt(D)
+    o, lse, (bq, bk, bv, bm) = _fwd(device, q, k, v, mask, causal, scale, dtype)
+    attrs = {"scale": scale, "is_causal": causal, "has_bias": mask is not None}
+    leaf = Node.leaf(Layout(B, S, H, D), dtype)
+    srcs = [Node.leaf(Layout(B, H, S, D), dtype), Node.leaf(Layout(B, H, S, D), dtype), leaf, leaf, leaf,
+            Node.leaf(Layout(bm.numel), dtype), Node.leaf(Layout(B, H, S), F32)]
+    node = Node("FLASH_ATTN_GRAD", Layout(B, S, H, D), dtype, srcs, attrs)
+    bdo = AnyBuffer.from_numpy(device, do, dtype)
+    dq, dk, dv = R.run(node, [bdo, o, bq, bk, bv, bm, lse], device)
+    return (o.to_numpy((B, H, S, D)), lse.to_numpy((B, H, S)), dq.to_numpy((B, S, H, D)), dk.to_numpy((B, S, H, D)),
+            dv.to_numpy((B, S, H, D)))
+
+
+def _inputs(cfg, B, S, H, D, dtype, with_mask):
+    q, k, v = (round_to_dtype(normal(cfg, i, (B, S, H, D)), dtype) for i in range(3))
+    do = round_to_dtype(normal(cfg, 4, (B, H, S, D)), dtype)
+    m = round_to_dtype(normal(cfg, 3, (B, H, S, S)), dtype) if with_mask else None
+    return q, k, v, do, m
+
+
+def _max_err(got, want):
+    assert np.all(np.isfinite(got)), "non-finite output"
+    return float(np.max(np.abs(got.astype(np.float64) - want)))
+
+
+MODES = [("plain", False, False), ("causal", True, False), ("bias", False, True)]
+
+# fp32: the reference's budgets at (B2, H2, S96), abs error vs the f64 oracle
+# (tests/kernels/attention/generic.mojo:440,485,530,575,620,665)
+F32_CASES = [(64, 5e-6), (256, 2e-5), (512, 5e-5), (8, 5e-6), (40, 5e-6), (128, 1e-5)]
+
+
+@pytest.mark.parametrize("name,causal,with_mask", MODES)
+@pytest.mark.parametrize("D,budget", F32_CASES)
+def test_f32_error_budget(device, name, causal, with_mask, D, budget):
+    B, H, S = 2, 2, 96
+    q, k, v, do, m = _inputs(50, B, S, H, D, F32, with_mask)
+    o, lse, dq, dk, dv = _fwd_bwd(device, q, k, v, do, m, causal)
+    ro, rl = O.sdpa_fwd(q, k, v, m, causal)
+    rdq, rdk, rdv = O.sdpa_bwd(q, k, v, do, m, causal)
+    assert _max_err(o, ro) <= budget and _max_err(lse, rl) <= budget
+    assert _max_err(dq, rdq) <= budget and _max_err(dk, rdk) <= budget and _max_err(dv, rdv) <= budget
+
+
+HALF_SHAPES = [(2, 2, 96, 64), (1, 3, 200, 64), (2, 1, 128, 128), (1, 2, 257, 32), (1, 1, 4, 8), (1, 2, 96, 256),
+               (1, 2, 130, 72)]
+
+
+@pytest.mark.parametrize("dtype,budget_fwd,budget_bwd", [(F16, 2e-3, 8e-3), (BF16, 1.6e-2, 6.4e-2)])
+@pytest.mark.parametrize("name,causal,with_mask", MODES)
+@pytest.mark.parametrize("B,H,S,D", HALF_SHAPES)
+def test_half_error_budget(device, dtype, budget_fwd, budget_bwd, name, causal, with_mask, B, H, S, D):
+    # fp16: the reference's budget for its tensor-core backward is 8e-3 abs at S96
+    # (tests/kernels/attention/mma.mojo:424); bf16 has 3 fewer mantissa bits: x8.
+    q, k, v, do, m = _inputs(51, B, S, H, D, dtype, with_mask)
+    o, lse, dq, dk, dv = _fwd_bwd(device, q, k, v, do, m, causal, dtype=dtype)
+    ro, rl = O.sdpa_fwd(q, k, v, m, causal)
+    # The backward is checked against the oracle's gradients at the O the kernel saw (its
+    # own forward output, rounded to the storage type) entering only through delta.
+    rdq, rdk, rdv = O.sdpa_bwd(q, k, v, do, m, causal)
+    grow = math.sqrt(S / 96.0)
+    assert _max_err(o, ro) <= budget_fwd
+    assert _max_err(lse, rl) <= 1e-3 * max(1.0, float(np.abs(rl).max()))
+    for got, want, what in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv")):
+        err = _max_err(got, want)
+        assert err <= budget_bwd * grow, f"{what}: {err}"
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_bf16_gradients_rtol(device, causal):
+    # Parity bar for bf16 attention gradients: rtol 2e-2 (with an absolute floor at the
+    # same fraction of each tensor's largest entry, for entries that cancel to ~0).
+    B, H, S, D = 2, 3, 256, 64
+    q, k, v, do, _ = _inputs(4, B, S, H, D, BF16, False)
+    _, _, dq, dk, dv = _fwd_bwd(device, q, k, v, do, None, causal, dtype=BF16)
+    for got, want, what in zip((dq, dk, dv), O.sdpa_bwd(q, k, v, do, None, causal), ("dq", "dk", "dv")):
+        bound = RTOL_BF16_ATTN * (np.abs(want) + np.abs(want).max())
+        assert np.all(np.abs(got - want) <= bound), f"{what}: worst {np.max(np.abs(got - want) / bound):.3g}"
+
+
+def test_closed_forms(device):
+    B, S, H, D = 1, 128, 1, 8
+    z = np.zeros((B, S, H, D), np.float32)
+    v = normal(52, 0, (B, S, H, D))
+    # Q = K = 0 causal, loss = sum(O): dV[j] = sum_{i>=j} 1/(i+1)   (tests/test_grad.mojo:1001-1023)
+    for dtype, tol in ((F32, 1e-5), (F16, 2e-2), (BF16, 2e-2)):
+        _, _, _, _, dv = _fwd_bwd(device, z, z, v, np.ones((B, H, S, D), np.float32), None, True, dtype=dtype)
+        tail = np.array([sum(1.0 / (i + 1) for i in range(j, S)) for j in range(S)])
+        np.testing.assert_allclose(dv[0, :, 0, :], np.repeat(tail[:, None], D, axis=1), rtol=tol, atol=tol)
+    # causal row 0 is V[0]; uniform scores average V; T=2 known value  (tests/test_ops.mojo:903-946)
+    q, k = normal(52, 1, (B, S, H, D)), normal(52, 2, (B, S, H, D))
+    o, lse, *_ = _fwd_bwd(device, q, k, v, np.ones((B, H, S, D), np.float32), None, True)
+    np.testing.assert_allclose(o[0, 0, 0], v[0, 0, 0], rtol=1e-6)
+    o, lse, *_ = _fwd_bwd(device, z, z, v, np.ones((B, H, S, D), np.float32), None, False)
+    np.testing.assert_allclose(o[0, 0], np.repeat(v[0, :, 0].mean(axis=0)[None], S, axis=0), atol=1e-6)
+    np.testing.assert_allclose(lse, math.log(S), rtol=1e-6)
+
+
+def test_bias_shift_invariance(device):
+    # tests/kernels/attention/generic.mojo:322-366
+    q, k, v, do, m = _inputs(53, 2, 40, 2, 64, F32, True)
+    o1, l1, dq1, dk1, dv1 = _fwd_bwd(device, q, k, v, do, m)
+    o2, l2, dq2, dk2, dv2 = _fwd_bwd(device, q, k, v, do, m + np.float32(3.0))
+    assert _max_err(o1, o2.astype(np.float64)) < 1e-5 and _max_err(l2 - l1, np.full(l1.shape, 3.0)) < 1e-4
+    assert _max_err(dq1, dq2.astype(np.float64)) < 1e-5 and _max_err(dk1, dk2.astype(np.float64)) < 1e-5
+
+
+def test_large_logits_stay_finite(device):
+    # softmax is max-subtracted: std-8 Q, K give logits in the hundreds
+    B, S, H, D = 1, 64, 2, 64
+    q, k = normal(54, 0, (B, S, H, D), std=8.0), normal(54, 1, (B, S, H, D), std=8.0)
+    v, do = normal(54, 2, (B, S, H, D)), normal(54, 3, (B, H, S, D))
+    o, lse, dq, dk, dv = _fwd_bwd(device, q, k, v, do)
+    ro, rl = O.sdpa_fwd(q, k, v)
+    assert _max_err(o, ro) < 1e-3 and _max_err(lse, rl) < 1e-3 * np.abs(rl).max()
+
+
+def test_placeholder_mask_is_never_read(device):
+    # has_bias False: the mask operand is a 1-element placeholder  (rewrites.mojo:94-103)
+    q, k, v, do, _ = _inputs(55, 1, 33, 2, 64, F32, False)
+    o, lse, dq, dk, dv = _fwd_bwd(device, q, k, v, do, None, True)
+    rdq, rdk, rdv = O.sdpa_bwd(q, k, v, do, None, True)
+    assert _max_err(dq, rdq) < 5e-6 and _max_err(dk, rdk) < 5e-6 and _max_err(dv, rdv) < 5e-6
+
+
+def test_has_bias_defaults(device):
+    # forward dispatch: has_bias defaults to True; backward: to `not is_causal`
+    # (dispatch.mojo:393-395,453-455)
+    q, k, v, do, m = _inputs(56, 1, 16, 1, 8, F32, True)
+    node = Node("FLASH_ATTN", Layout(1, 1, 16, 8), F32,
+                [Node.leaf(Layout(1, 16, 1, 8))] * 3 + [Node.leaf(Layout(1, 1, 16, 16))], {"scale": 0.5, "is_causal": False})
+    bufs = [AnyBuffer.from_numpy(device, a) for a in (q, k, v, m)]
+    o, lse = R.run(node, bufs, device)
+    ro, _ = O.sdpa_fwd(q, k, v, m, False, 0.5)
+    assert _max_err(o.to_numpy((1, 1, 16, 8)), ro) < 5e-6
+
+
+def test_errors(device):
+    buf = AnyBuffer.create(F32, device, 64)
+    p = buf.data_ptr()
+    lib, st = device.lib, device.stream
+    with pytest.raises(MogradError, match=r"D=513 out of range \(1..512\)"):
+        lib.mg_flash_attn_fwd(p, p, p, p, p, p, 1, 1, 1, 513, 1.0, 0, 0, F32, st)
+    with pytest.raises(MogradError, match=r"D=0 out of range"):
+        lib.mg_flash_attn_bwd(p, p, p, p, p, p, p, p, p, p, 1, 1, 1, 0, 1.0, 0, 0, F32, st)
+    with pytest.raises(MogradError, match="causal attention with additive bias is not supported"):
+        lib.mg_flash_attn_fwd(p, p, p, p, p, p, 1, 2, 1, 8, 1.0, 1, 1, F32, st)
+    with pytest.raises(MogradError, match="unsupported dtype"):
+        lib.mg_flash_attn_fwd(p, p, p, p, p, p, 1, 2, 1, 8, 1.0, 0, 0, R.int64, st)
