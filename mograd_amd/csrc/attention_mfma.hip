@@ -1,19 +1,569 @@
-// Flash attention on the matrix cores (placeholder until the MFMA kernels land).
+// Flash attention on the matrix cores for 16-bit storage (bf16, fp16), head dim <= 128.
+//
+// All three kernels use v_mfma_f32_32x32x16 with fp32 accumulation and share one idea:
+// the tensor that a workgroup keeps for its whole life sits in registers as the MFMA's
+// B operand (column = lane), the tensor that streams past comes through LDS as the A
+// operand, and the 32x32 score tile comes out with "column = lane, rows in runs of four",
+// which is exactly the B-operand shape of the next product, so probabilities and score
+// gradients never leave registers.
+//
+//   forward   workgroup = 128 queries (4 waves x 32); streams 64-key blocks.
+//             S^T = K Q^T, online softmax per lane (lane = one query), O^T += V^T P^T.
+//   dQ        same shape; S^T and dP^T = V dO^T, dS^T = P (dP - delta), dQ^T += K^T dS^T.
+//   dK, dV    workgroup = 128 keys (4 waves x 32); streams 64-query blocks.
+//             S = Q K^T, dP = dO V^T, dV^T += dO^T P, dK^T += Q^T dS.
+// dQ has its own kernel that recomputes S and dP: seven products instead of five, but no
+// atomics, so every output is written once and results are reproducible.
+//
+// A product that contracts over the streamed index needs the streamed tile transposed
+// ([d][row]); tiles are staged in LDS in both orientations, the transposed one written as
+// packed pairs of rows so that the LDS stores are full dwords.
+//
+// Layouts: Q, K, V, dQ, dK, dV BSHD; O, dO BHSD; mask (B,H,S,S); LSE, delta (B,H,S) fp32.
+#include <cstdlib>
+
 #include "attention_generic.h"
 #include "mg_internal.h"
 
 namespace mg {
 
-bool attn_mfma_supported(int, int64_t, const void* const*, int) { return false; }
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 
-int attn_fwd_mfma(const void*, const void*, const void*, const void*, void*, float*, AttnDims, float, bool, bool, int,
-                  hipStream_t) {
-  return fail(MG_ERR_UNSUPPORTED, "flash_attn_fwd: MFMA path not built");
+template <typename T>
+struct Mma;
+template <>
+struct Mma<bf16_t> {
+  static __device__ __forceinline__ floatx16 run(uint4 a, uint4 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0,
+                                                   0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    return static_cast<uint32_t>(bf16_bits_rne(lo)) | (static_cast<uint32_t>(bf16_bits_rne(hi)) << 16);
+  }
+};
+template <>
+struct Mma<f16_t> {
+  static __device__ __forceinline__ floatx16 run(uint4 a, uint4 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0,
+                                                  0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    union { uint32_t u; f16_t h[2]; } cv;
+    cv.h[0] = static_cast<f16_t>(lo);
+    cv.h[1] = static_cast<f16_t>(hi);
+    return cv.u;
+  }
+};
+
+constexpr int kAttnThreads = 256;
+
+// ---- LDS tiles -------------------------------------------------------------------------
+// Row-major tile: R rows x DP columns of T, row stride DP + 8 elements (the 16-byte pad
+// spreads the 128-bit fragment reads of 8 consecutive rows over all banks).
+template <int DP>
+constexpr int row_stride() { return DP + 8; }
+// Transposed tile: DP rows (one per d) x R columns, stored as dwords holding two
+// consecutive columns; row stride R/2 + 2 dwords.
+template <int R>
+constexpr int tr_stride_dw() { return R / 2 + 2; }
+
+// Global rows [r0, r0 + R) of a matrix whose row `r` starts at base + r * ld (elements),
+// D valid columns, rows >= r_end read as zero.  Writes the row-major tile.
+template <typename T, int R, int DP>
+__device__ __forceinline__ void stage_rows(uint16_t* __restrict__ lds, const T* __restrict__ base, int64_t ld, int r0,
+                                           int r_end, int D) {
+  constexpr int CH = DP / 8;  // 16-byte chunks per row
+  for (int idx = threadIdx.x; idx < R * CH; idx += kAttnThreads) {
+    const int r = idx / CH, c = idx % CH;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (r0 + r < r_end && c * 8 < D) v = *reinterpret_cast<const uint4*>(base + (r0 + r) * ld + c * 8);
+    *reinterpret_cast<uint4*>(lds + r * row_stride<DP>() + c * 8) = v;
+  }
 }
 
-int attn_bwd_mfma(const void*, const void*, const void*, const void*, const void*, const void*, const float*, void*,
-                  void*, void*, AttnDims, float, bool, bool, int, hipStream_t) {
-  return fail(MG_ERR_UNSUPPORTED, "flash_attn_bwd: MFMA path not built");
+// Same rows, written transposed: dword (d, p) holds columns 2p and 2p+1 of row d.
+template <typename T, int R, int DP>
+__device__ __forceinline__ void stage_transposed(uint32_t* __restrict__ lds, const T* __restrict__ base, int64_t ld,
+                                                 int r0, int r_end, int D) {
+  constexpr int CH = DP / 8;
+  constexpr int PAIRS = R / 2;
+  for (int idx = threadIdx.x; idx < PAIRS * CH; idx += kAttnThreads) {
+    const int p = idx % PAIRS, c = idx / PAIRS;
+    uint4 lo = make_uint4(0, 0, 0, 0), hi = make_uint4(0, 0, 0, 0);
+    const int ra = r0 + 2 * p;
+    if (c * 8 < D) {
+      if (ra < r_end) lo = *reinterpret_cast<const uint4*>(base + ra * ld + c * 8);
+      if (ra + 1 < r_end) hi = *reinterpret_cast<const uint4*>(base + (ra + 1) * ld + c * 8);
+    }
+    const uint32_t a[4] = {lo.x, lo.y, lo.z, lo.w};
+    const uint32_t b[4] = {hi.x, hi.y, hi.z, hi.w};
+    uint32_t* dst = lds + (c * 8) * tr_stride_dw<R>() + p;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      dst[(2 * e) * tr_stride_dw<R>()] = (a[e] & 0xffffu) | (b[e] << 16);
+      dst[(2 * e + 1) * tr_stride_dw<R>()] = (a[e] >> 16) | (b[e] & 0xffff0000u);
+    }
+  }
+}
+
+// A operand from a row-major tile: rows rt*32 + lane%32, columns ks*16 + (lane/32)*8 .. +7.
+template <int DP>
+__device__ __forceinline__ uint4 frag_rows(const uint16_t* __restrict__ lds, int rt, int ks, int lane) {
+  return *reinterpret_cast<const uint4*>(lds + (rt * 32 + lane % 32) * row_stride<DP>() + ks * 16 + (lane / 32) * 8);
+}
+
+// A operand from a transposed tile for the product that contracts over the tile's
+// columns.  k-slot e of lane half h stands for column t*16 + (e/4)*8 + 4h + e%4: the
+// same assignment the score tile's registers have (see frag_from_acc).
+template <int R>
+__device__ __forceinline__ uint4 frag_transposed(const uint32_t* __restrict__ lds, int dt, int t, int lane) {
+  const uint32_t* p = lds + (dt * 32 + lane % 32) * tr_stride_dw<R>() + t * 8 + (lane / 32) * 2;
+  const uint2 lo = *reinterpret_cast<const uint2*>(p);
+  const uint2 hi = *reinterpret_cast<const uint2*>(p + 4);
+  return make_uint4(lo.x, lo.y, hi.x, hi.y);
+}
+
+// B operand from a 32x32 accumulator tile: registers 8*half .. 8*half+7, i.e. rows
+// half*16 + (e/4)*8 + 4*(lane/32) + e%4 of column lane%32.
+template <typename T>
+__device__ __forceinline__ uint4 frag_from_acc(const floatx16& acc, int half) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = Mma<T>::pack2(acc[half * 8 + 2 * i], acc[half * 8 + 2 * i + 1]);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// Row index inside a 32-row tile of accumulator register r.
+__device__ __forceinline__ int acc_row(int r, int lane) { return (r / 4) * 8 + (lane / 32) * 4 + (r % 4); }
+
+__device__ __forceinline__ floatx16 zero16() {
+  floatx16 z;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) z[r] = 0.f;
+  return z;
+}
+
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+
+// ---- forward -----------------------------------------------------------------------------
+
+template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
+__global__ __launch_bounds__(kAttnThreads) void attn_fwd_mfma_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                                     const T* __restrict__ v, const T* __restrict__ mask,
+                                                                     T* __restrict__ o, float* __restrict__ lse,
+                                                                     AttnDims a, float scale) {
+  constexpr int BM = 128, BN = 64, KS = DP / 16, DT = DP / 32;
+  __shared__ __attribute__((aligned(16))) uint16_t k_rows[BN * row_stride<DP>()];
+  __shared__ __attribute__((aligned(16))) uint32_t v_tr[DP * tr_stride_dw<BN>()];
+
+  const int nqb = (a.S + BM - 1) / BM;
+  const int qb = blockIdx.x % nqb;
+  const int h = (blockIdx.x / nqb) % a.H;
+  const int b = blockIdx.x / (nqb * a.H);
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const int half = lane / 32;
+  const int m_wave = qb * BM + wave * 32;
+  const int m = m_wave + lane % 32;
+  const int64_t ld = static_cast<int64_t>(a.H) * a.D;  // BSHD row stride
+  const T* kbase = k + bshd(a, b, 0, h);
+  const T* vbase = v + bshd(a, b, 0, h);
+
+  uint4 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d = ks * 16 + half * 8;
+    qf[ks] = (m < a.S && d < a.D) ? *reinterpret_cast<const uint4*>(q + bshd(a, b, m, h) + d) : make_uint4(0, 0, 0, 0);
+  }
+  floatx16 acc_o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) acc_o[dt] = zero16();
+  float m_run = -INFINITY, l_run = 0.f;
+  const float c = scale * kAttnLog2e;
+  const T* mrow = HAS_BIAS ? mask + ((static_cast<int64_t>(b) * a.H + h) * a.S + min(m, a.S - 1)) * a.S : nullptr;
+
+  const int n_end = CAUSAL ? min(a.S, qb * BM + BM) : a.S;
+  for (int n0 = 0; n0 < n_end; n0 += BN) {
+    __syncthreads();
+    stage_rows<T, BN, DP>(k_rows, kbase, ld, n0, a.S, a.D);
+    stage_transposed<T, BN, DP>(v_tr, vbase, ld, n0, a.S, a.D);
+    __syncthreads();
+    if (CAUSAL && n0 > m_wave + 31) continue;  // every key of the block is in this wave's future
+
+    floatx16 s[2];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      s[nt] = zero16();
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) s[nt] = Mma<T>::run(frag_rows<DP>(k_rows, nt, ks, lane), qf[ks], s[nt]);
+    }
+    // scale, bias, mask -> log2-domain scores; row maximum of this lane's query
+    float mx = -INFINITY;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int n = n0 + nt * 32 + acc_row(r, lane);
+        bool valid = n < a.S;
+        if (CAUSAL) valid = valid && n <= m;
+        float sv = s[nt][r] * c;
+        if (HAS_BIAS) sv = valid ? fmaf(to_float(mrow[n]), kAttnLog2e, sv) : sv;
+        sv = valid ? sv : -INFINITY;
+        s[nt][r] = sv;
+        mx = fmaxf(mx, sv);
+      }
+    mx = fmaxf(mx, xor32(mx));
+    const float m_new = fmaxf(m_run, mx);
+    // m_new is -inf only for rows past the end of the sequence (all their keys masked)
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = exp2f(m_run - m_use);
+    float lsum = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = exp2f(s[nt][r] - m_use);
+        s[nt][r] = p;
+        lsum += p;
+      }
+    lsum += xor32(lsum);
+    l_run = l_run * corr + lsum;
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc_o[dt][r] *= corr;
+#pragma unroll
+    for (int t = 0; t < BN / 16; ++t) {
+      const uint4 pf = frag_from_acc<T>(s[t / 2], t % 2);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) acc_o[dt] = Mma<T>::run(frag_transposed<BN>(v_tr, dt, t, lane), pf, acc_o[dt]);
+    }
+  }
+
+  if (m < a.S) {
+    const float inv = 1.0f / l_run;
+    T* orow = o + bhsd(a, b, h, m);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d = dt * 32 + g * 8 + half * 4;
+        if (d < a.D) {
+          uint2 w;
+          w.x = Mma<T>::pack2(acc_o[dt][g * 4] * inv, acc_o[dt][g * 4 + 1] * inv);
+          w.y = Mma<T>::pack2(acc_o[dt][g * 4 + 2] * inv, acc_o[dt][g * 4 + 3] * inv);
+          *reinterpret_cast<uint2*>(orow + d) = w;
+        }
+      }
+    if (half == 0) lse[(static_cast<int64_t>(b) * a.H + h) * a.S + m] = m_run * kAttnLn2 + logf(l_run);
+  }
+}
+
+// ---- dQ ----------------------------------------------------------------------------------
+
+template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
+__global__ __launch_bounds__(kAttnThreads) void attn_dq_mfma_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
+                                                                    const T* __restrict__ k, const T* __restrict__ v,
+                                                                    const T* __restrict__ mask, const float* __restrict__ lse,
+                                                                    const float* __restrict__ delta, T* __restrict__ dq,
+                                                                    AttnDims a, float scale) {
+  constexpr int BM = 128, BN = 64, KS = DP / 16, DT = DP / 32;
+  __shared__ __attribute__((aligned(16))) uint16_t k_rows[BN * row_stride<DP>()];
+  __shared__ __attribute__((aligned(16))) uint16_t v_rows[BN * row_stride<DP>()];
+  __shared__ __attribute__((aligned(16))) uint32_t k_tr[DP * tr_stride_dw<BN>()];
+
+  const int nqb = (a.S + BM - 1) / BM;
+  const int qb = blockIdx.x % nqb;
+  const int h = (blockIdx.x / nqb) % a.H;
+  const int b = blockIdx.x / (nqb * a.H);
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const int half = lane / 32;
+  const int m_wave = qb * BM + wave * 32;
+  const int m = m_wave + lane % 32;
+  const int64_t ld = static_cast<int64_t>(a.H) * a.D;
+  const T* kbase = k + bshd(a, b, 0, h);
+  const T* vbase = v + bshd(a, b, 0, h);
+  const int64_t bh = static_cast<int64_t>(b) * a.H + h;
+
+  uint4 qf[KS], dof[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d = ks * 16 + half * 8;
+    const bool ok = m < a.S && d < a.D;
+    qf[ks] = ok ? *reinterpret_cast<const uint4*>(q + bshd(a, b, m, h) + d) : make_uint4(0, 0, 0, 0);
+    dof[ks] = ok ? *reinterpret_cast<const uint4*>(d_o + bhsd(a, b, h, m) + d) : make_uint4(0, 0, 0, 0);
+  }
+  // Rows past the end get lse = +inf so that their probabilities vanish.
+  const float lse2 = m < a.S ? lse[bh * a.S + m] * kAttnLog2e : INFINITY;
+  const float dl = m < a.S ? delta[bh * a.S + m] : 0.f;
+  floatx16 acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
+  const float c = scale * kAttnLog2e;
+  const T* mrow = HAS_BIAS ? mask + (bh * a.S + min(m, a.S - 1)) * a.S : nullptr;
+
+  const int n_end = CAUSAL ? min(a.S, qb * BM + BM) : a.S;
+  for (int n0 = 0; n0 < n_end; n0 += BN) {
+    __syncthreads();
+    stage_rows<T, BN, DP>(k_rows, kbase, ld, n0, a.S, a.D);
+    stage_rows<T, BN, DP>(v_rows, vbase, ld, n0, a.S, a.D);
+    stage_transposed<T, BN, DP>(k_tr, kbase, ld, n0, a.S, a.D);
+    __syncthreads();
+    if (CAUSAL && n0 > m_wave + 31) continue;
+
+    floatx16 s[2], dp[2];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      s[nt] = zero16();
+      dp[nt] = zero16();
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        s[nt] = Mma<T>::run(frag_rows<DP>(k_rows, nt, ks, lane), qf[ks], s[nt]);
+        dp[nt] = Mma<T>::run(frag_rows<DP>(v_rows, nt, ks, lane), dof[ks], dp[nt]);
+      }
+    }
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int n = n0 + nt * 32 + acc_row(r, lane);
+        bool valid = n < a.S;
+        if (CAUSAL) valid = valid && n <= m;
+        float sv = s[nt][r] * c;
+        if (HAS_BIAS) sv = valid ? fmaf(to_float(mrow[n]), kAttnLog2e, sv) : sv;
+        const float p = valid ? exp2f(sv - lse2) : 0.f;
+        s[nt][r] = p * (dp[nt][r] - dl);  // dS^T
+      }
+#pragma unroll
+    for (int t = 0; t < BN / 16; ++t) {
+      const uint4 dsf = frag_from_acc<T>(s[t / 2], t % 2);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) acc[dt] = Mma<T>::run(frag_transposed<BN>(k_tr, dt, t, lane), dsf, acc[dt]);
+    }
+  }
+
+  if (m < a.S) {
+    T* out = dq + bshd(a, b, m, h);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d = dt * 32 + g * 8 + half * 4;
+        if (d < a.D) {
+          uint2 w;
+          w.x = Mma<T>::pack2(acc[dt][g * 4] * scale, acc[dt][g * 4 + 1] * scale);
+          w.y = Mma<T>::pack2(acc[dt][g * 4 + 2] * scale, acc[dt][g * 4 + 3] * scale);
+          *reinterpret_cast<uint2*>(out + d) = w;
+        }
+      }
+  }
+}
+
+// ---- dK, dV ------------------------------------------------------------------------------
+
+template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
+__global__ __launch_bounds__(kAttnThreads) void attn_dkdv_mfma_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
+                                                                      const T* __restrict__ k, const T* __restrict__ v,
+                                                                      const T* __restrict__ mask,
+                                                                      const float* __restrict__ lse,
+                                                                      const float* __restrict__ delta, T* __restrict__ dk,
+                                                                      T* __restrict__ dv, AttnDims a, float scale) {
+  constexpr int BNK = 128;                 // keys per workgroup
+  constexpr int BQ = DP <= 64 ? 64 : 32;   // queries per step (LDS budget)
+  constexpr int MT = BQ / 32, KS = DP / 16, DT = DP / 32;
+  __shared__ __attribute__((aligned(16))) uint16_t q_rows[BQ * row_stride<DP>()];
+  __shared__ __attribute__((aligned(16))) uint16_t do_rows[BQ * row_stride<DP>()];
+  __shared__ __attribute__((aligned(16))) uint32_t q_tr[DP * tr_stride_dw<BQ>()];
+  __shared__ __attribute__((aligned(16))) uint32_t do_tr[DP * tr_stride_dw<BQ>()];
+  __shared__ __attribute__((aligned(16))) float lse_s[BQ];
+  __shared__ __attribute__((aligned(16))) float delta_s[BQ];
+
+  const int nkb = (a.S + BNK - 1) / BNK;
+  const int kb = blockIdx.x % nkb;
+  const int h = (blockIdx.x / nkb) % a.H;
+  const int b = blockIdx.x / (nkb * a.H);
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const int half = lane / 32;
+  const int n_wave = kb * BNK + wave * 32;
+  const int n = n_wave + lane % 32;
+  const int64_t ld = static_cast<int64_t>(a.H) * a.D;
+  const T* qbase = q + bshd(a, b, 0, h);
+  const T* dobase = d_o + bhsd(a, b, h, 0);
+  const int64_t bh = static_cast<int64_t>(b) * a.H + h;
+
+  uint4 kf[KS], vf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d = ks * 16 + half * 8;
+    const bool ok = n < a.S && d < a.D;
+    kf[ks] = ok ? *reinterpret_cast<const uint4*>(k + bshd(a, b, n, h) + d) : make_uint4(0, 0, 0, 0);
+    vf[ks] = ok ? *reinterpret_cast<const uint4*>(v + bshd(a, b, n, h) + d) : make_uint4(0, 0, 0, 0);
+  }
+  floatx16 acc_k[DT], acc_v[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    acc_k[dt] = zero16();
+    acc_v[dt] = zero16();
+  }
+  const float c = scale * kAttnLog2e;
+
+  // Causal: queries before the workgroup's first key see none of its keys.
+  const int m_begin = CAUSAL ? (kb * BNK / BQ) * BQ : 0;
+  for (int m0 = m_begin; m0 < a.S; m0 += BQ) {
+    __syncthreads();
+    stage_rows<T, BQ, DP>(q_rows, qbase, ld, m0, a.S, a.D);
+    stage_rows<T, BQ, DP>(do_rows, dobase, a.D, m0, a.S, a.D);
+    stage_transposed<T, BQ, DP>(q_tr, qbase, ld, m0, a.S, a.D);
+    stage_transposed<T, BQ, DP>(do_tr, dobase, a.D, m0, a.S, a.D);
+    if (threadIdx.x < BQ) {
+      const int mm = m0 + threadIdx.x;
+      lse_s[threadIdx.x] = mm < a.S ? lse[bh * a.S + mm] * kAttnLog2e : INFINITY;
+      delta_s[threadIdx.x] = mm < a.S ? delta[bh * a.S + mm] : 0.f;
+    }
+    __syncthreads();
+    if (CAUSAL && m0 + BQ - 1 < n_wave) continue;  // all of this step's queries precede the wave's keys
+
+    floatx16 s[MT], dp[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      s[mt] = zero16();
+      dp[mt] = zero16();
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        s[mt] = Mma<T>::run(frag_rows<DP>(q_rows, mt, ks, lane), kf[ks], s[mt]);
+        dp[mt] = Mma<T>::run(frag_rows<DP>(do_rows, mt, ks, lane), vf[ks], dp[mt]);
+      }
+    }
+    // s -> P, dp -> dS (both: column = this lane's key, rows = queries)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int ml = mt * 32 + acc_row(r, lane);
+        const int mm = m0 + ml;
+        bool valid = n < a.S;  // rows past the end carry lse = +inf
+        if (CAUSAL) valid = valid && n <= mm;
+        float sv = s[mt][r] * c;
+        if (HAS_BIAS) sv = (valid && mm < a.S) ? fmaf(to_float(mask[(bh * a.S + mm) * a.S + n]), kAttnLog2e, sv) : sv;
+        const float p = valid ? exp2f(sv - lse_s[ml]) : 0.f;
+        s[mt][r] = p;
+        dp[mt][r] = p * (dp[mt][r] - delta_s[ml]);
+      }
+#pragma unroll
+    for (int t = 0; t < BQ / 16; ++t) {
+      const uint4 pf = frag_from_acc<T>(s[t / 2], t % 2);
+      const uint4 dsf = frag_from_acc<T>(dp[t / 2], t % 2);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        acc_v[dt] = Mma<T>::run(frag_transposed<BQ>(do_tr, dt, t, lane), pf, acc_v[dt]);
+        acc_k[dt] = Mma<T>::run(frag_transposed<BQ>(q_tr, dt, t, lane), dsf, acc_k[dt]);
+      }
+    }
+  }
+
+  if (n < a.S) {
+    T* outk = dk + bshd(a, b, n, h);
+    T* outv = dv + bshd(a, b, n, h);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d = dt * 32 + g * 8 + half * 4;
+        if (d < a.D) {
+          uint2 wk, wv;
+          wk.x = Mma<T>::pack2(acc_k[dt][g * 4] * scale, acc_k[dt][g * 4 + 1] * scale);
+          wk.y = Mma<T>::pack2(acc_k[dt][g * 4 + 2] * scale, acc_k[dt][g * 4 + 3] * scale);
+          wv.x = Mma<T>::pack2(acc_v[dt][g * 4], acc_v[dt][g * 4 + 1]);
+          wv.y = Mma<T>::pack2(acc_v[dt][g * 4 + 2], acc_v[dt][g * 4 + 3]);
+          *reinterpret_cast<uint2*>(outk + d) = wk;
+          *reinterpret_cast<uint2*>(outv + d) = wv;
+        }
+      }
+  }
+}
+
+// ---- host side ---------------------------------------------------------------------------
+
+bool attn_mfma_supported(int dtype, int64_t D, const void* const* ptrs, int nptrs) {
+  if (dtype != MG_F16 && dtype != MG_BF16) return false;
+  if (D % 8 != 0 || D > 128) return false;  // rows are read 16 bytes at a time
+  for (int i = 0; i < nptrs; ++i)
+    if (ptrs[i] != nullptr && !aligned16(ptrs[i])) return false;
+  const char* force = std::getenv("MOGRAD_HIP_ATTN_GENERIC");
+  if (force && force[0] == '1') return false;
+  return true;
+}
+
+template <typename T, int DP>
+static int fwd_typed(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, AttnDims a,
+                     float scale, bool causal, bool has_bias, hipStream_t stream) {
+  const int64_t blocks = static_cast<int64_t>(a.B) * a.H * ceil_div(a.S, 128);
+#define MG_LAUNCH(C_, B_)                                                                                             \
+  hipLaunchKernelGGL((attn_fwd_mfma_kernel<T, DP, C_, B_>), dim3(static_cast<unsigned>(blocks)), dim3(kAttnThreads), 0, \
+                     stream, static_cast<const T*>(q), static_cast<const T*>(k), static_cast<const T*>(v),            \
+                     static_cast<const T*>(mask), static_cast<T*>(o), lse, a, scale)
+  if (causal) MG_LAUNCH(true, false);
+  else if (has_bias) MG_LAUNCH(false, true);
+  else MG_LAUNCH(false, false);
+#undef MG_LAUNCH
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+template <typename T, int DP>
+static int bwd_typed(const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
+                     const float* lse, void* dq, void* dk, void* dv, AttnDims a, float scale, bool causal, bool has_bias,
+                     hipStream_t stream) {
+  const int64_t rows = static_cast<int64_t>(a.B) * a.H * a.S;
+  Scratch delta;
+  MG_TRY(delta.take(rows * static_cast<int64_t>(sizeof(float))));
+  hipLaunchKernelGGL((attn_delta_kernel<T>), dim3(static_cast<unsigned>(ceil_div(rows, 4))), dim3(256), 0, stream,
+                     static_cast<const T*>(d_o), static_cast<const T*>(o), delta.as<float>(), rows, a.D);
+  MG_LAUNCH_CHECK();
+  const int64_t blocks = static_cast<int64_t>(a.B) * a.H * ceil_div(a.S, 128);
+#define MG_LAUNCH(C_, B_)                                                                                              \
+  do {                                                                                                                 \
+    hipLaunchKernelGGL((attn_dkdv_mfma_kernel<T, DP, C_, B_>), dim3(static_cast<unsigned>(blocks)), dim3(kAttnThreads), \
+                       0, stream, static_cast<const T*>(d_o), static_cast<const T*>(q), static_cast<const T*>(k),      \
+                       static_cast<const T*>(v), static_cast<const T*>(mask), lse, delta.as<float>(),                  \
+                       static_cast<T*>(dk), static_cast<T*>(dv), a, scale);                                            \
+    hipLaunchKernelGGL((attn_dq_mfma_kernel<T, DP, C_, B_>), dim3(static_cast<unsigned>(blocks)), dim3(kAttnThreads), 0, \
+                       stream, static_cast<const T*>(d_o), static_cast<const T*>(q), static_cast<const T*>(k),         \
+                       static_cast<const T*>(v), static_cast<const T*>(mask), lse, delta.as<float>(),                  \
+                       static_cast<T*>(dq), a, scale);                                                                 \
+  } while (0)
+  if (causal) MG_LAUNCH(true, false);
+  else if (has_bias) MG_LAUNCH(false, true);
+  else MG_LAUNCH(false, false);
+#undef MG_LAUNCH
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+int attn_fwd_mfma(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, AttnDims a,
+                  float scale, bool causal, bool has_bias, int dtype, hipStream_t stream) {
+  const bool small = a.D <= 64;
+  if (dtype == MG_BF16)
+    return small ? fwd_typed<bf16_t, 64>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream)
+                 : fwd_typed<bf16_t, 128>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
+  return small ? fwd_typed<f16_t, 64>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream)
+               : fwd_typed<f16_t, 128>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
+}
+
+int attn_bwd_mfma(const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
+                  const float* lse, void* dq, void* dk, void* dv, AttnDims a, float scale, bool causal, bool has_bias,
+                  int dtype, hipStream_t stream) {
+  const bool small = a.D <= 64;
+  if (dtype == MG_BF16)
+    return small ? bwd_typed<bf16_t, 64>(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal, has_bias, stream)
+                 : bwd_typed<bf16_t, 128>(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal, has_bias, stream);
+  return small ? bwd_typed<f16_t, 64>(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal, has_bias, stream)
+               : bwd_typed<f16_t, 128>(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal, has_bias, stream);
 }
 
 }  // namespace mg
