@@ -47,9 +47,9 @@ __device__ __forceinline__ int64_t load_id(const void* ids, int64_t row, bool id
 // ------------------------------------------------------------------------------------
 
 template <typename T, int VEC, int TPR, int VPT, int WG, bool DENSE>
-__global__ __launch_bounds__(WG) void ce_rows_kernel(const T* __restrict__ logits, const void* __restrict__ labels,
-                                                     const T* __restrict__ upstream, float* __restrict__ rowloss,
-                                                     T* __restrict__ dlogits, int64_t N, int C, int id64) {
+__global__ __launch_bounds__(WG, (TPR == 256 && VPT > 32) ? 2 : 1) void ce_rows_kernel(
+    const T* __restrict__ logits, const void* __restrict__ labels, const T* __restrict__ upstream,
+    float* __restrict__ rowloss, T* __restrict__ dlogits, int64_t N, int C, int id64) {
   constexpr int RPW = WG / TPR;
   using Tile = RowTile<T, VEC, TPR, VPT>;
   __shared__ float slots[2 * (WG / kWave)];
@@ -59,57 +59,65 @@ __global__ __launch_bounds__(WG) void ce_rows_kernel(const T* __restrict__ logit
   const float inv_rows = 1.0f / static_cast<float>(N);
   const float scale = (upstream != nullptr ? to_float(upstream[0]) : 1.0f) * inv_rows;
 
-  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * RPW; row0 < N; row0 += static_cast<int64_t>(gridDim.x) * RPW) {
-    const int64_t row = row0 + sub;
-    if (row >= N) continue;  // uniform per wave (TPR == 64) or per workgroup (RPW == 1)
+  // One row per TPR threads and no row loop: a loop would let the compiler start the next
+  // row's loads before this row's stores and double the register footprint.
+  {
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * RPW + sub;
+    if (row >= N) return;  // uniform per wave (TPR == 64) or per workgroup (RPW == 1); no barrier follows for TPR == 64
     const T* xr = logits + row * C;
     Tile x;
     x.load(xr, t, C);
 
-    // Padding chunks hold zeros; they take part in the max only if the row has no
-    // larger value, so they are masked to -inf here and skipped in the sums below.
+    // Padding chunks hold zeros: mask them to -inf for the max and skip them in the sums.
+    const int nfull = Tile::full_chunks(C);
     float m[1] = {-INFINITY};
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-      const bool valid = Tile::col(i, t) < C;
+      if (i < nfull) {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) m[0] = fmaxf(m[0], valid ? x.v[i][e] : -INFINITY);
+        for (int e = 0; e < VEC; ++e) m[0] = fmaxf(m[0], x.v[i][e]);
+      } else if (i == nfull) {
+        const bool valid = Tile::col(i, t) < C;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) m[0] = fmaxf(m[0], valid ? x.v[i][e] : -INFINITY);
+      }
     }
     row_allreduce_max<TPR, WG, 1>(m, slots, phase);
     const float m2 = m[0] * kLog2e;
-
-    float s[1] = {0.f};
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-      const bool valid = Tile::col(i, t) < C;
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        const float ex = fast_exp2(fmaf(x.v[i][e], kLog2e, -m2));
-        s[0] += valid ? ex : 0.f;
-      }
-    }
-    row_allreduce_sum<TPR, WG, 1>(s, slots, phase);
-    // softmax = exp(x - lse), formed directly from the log-sum-exp so that the
-    // exponentials of the previous pass need not stay live in registers.
-    const float shift = m[0] + logf(s[0]);
-    const float shift2 = shift * kLog2e;
-
     T* out_row = dlogits + row * C;
+
     if constexpr (DENSE) {
-      const T* yr = static_cast<const T*>(labels) + row * C;
-      float acc[1] = {0.f};
+      float s[1] = {0.f};
 #pragma unroll
       for (int i = 0; i < VPT; ++i) {
-        const int c = Tile::col(i, t);
-        if (c < C) {
+        if (i < nfull) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) s[0] += fast_exp2(fmaf(x.v[i][e], kLog2e, -m2));
+        } else if (i == nfull) {
+          const bool valid = Tile::col(i, t) < C;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) s[0] += valid ? fast_exp2(fmaf(x.v[i][e], kLog2e, -m2)) : 0.f;
+        }
+      }
+      row_allreduce_sum<TPR, WG, 1>(s, slots, phase);
+      // softmax = exp(x - lse), formed directly from the log-sum-exp so that the
+      // exponentials of the previous pass need not stay live next to the logits.
+      const float shift = m[0] + logf(s[0]);
+      const float shift2 = shift * kLog2e;
+      const T* yr = static_cast<const T*>(labels) + row * C;
+      float acc[1] = {0.f};
+      const unsigned lane_off = static_cast<unsigned>(t) * VEC;
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        if (i < nfull || (i == nfull && Tile::col(i, t) < C)) {
           float y[VEC], out[VEC];
-          VecIO<T, VEC>::load(yr + c, y);
+          VecIO<T, VEC>::load(yr + i * (TPR * VEC) + lane_off, y);
 #pragma unroll
           for (int e = 0; e < VEC; ++e) {
             acc[0] += (x.v[i][e] - shift) * y[e];
             out[e] = (fast_exp2(fmaf(x.v[i][e], kLog2e, -shift2)) - y[e]) * scale;
           }
-          VecIO<T, VEC>::store(out_row + c, out);
+          VecIO<T, VEC>::store(out_row + i * (TPR * VEC) + lane_off, out);
         }
       }
       if (rowloss != nullptr) {
@@ -117,32 +125,49 @@ __global__ __launch_bounds__(WG) void ce_rows_kernel(const T* __restrict__ logit
         if (t == 0) rowloss[row] = -acc[0] * inv_rows;
       }
     } else {
-      const int64_t id = load_id(labels, row, id64 != 0);
-      const bool id_ok = id >= 0 && id < C;
-      // Column `id` relative to this thread's first element: chunk i, element e holds it
-      // iff rel == i * TPR * VEC + e.
-      const int rel = id_ok ? static_cast<int>(id) - t * VEC : -1;
-      float picked = 0.f;
+      // Integer labels: the exponentials replace the logits in registers, the gradient is
+      // one multiply per element, and the single "- 1" at the label column is patched by
+      // its owner thread with a scalar store issued after its vector stores (same thread,
+      // same address: program order holds).
+      float s[1] = {0.f};
 #pragma unroll
       for (int i = 0; i < VPT; ++i) {
-        const int c = Tile::col(i, t);
-        float out[VEC];
+        if (i < nfull) {
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          const bool hit = rel == i * TPR * VEC + e;
-          const float p = fast_exp2(fmaf(x.v[i][e], kLog2e, -shift2));
-          picked = hit ? x.v[i][e] : picked;
-          out[e] = (hit ? p - 1.0f : p) * scale;
+          for (int e = 0; e < VEC; ++e) {
+            x.v[i][e] = fast_exp2(fmaf(x.v[i][e], kLog2e, -m2));
+            s[0] += x.v[i][e];
+          }
+        } else if (i == nfull) {
+          const bool valid = Tile::col(i, t) < C;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            x.v[i][e] = fast_exp2(fmaf(x.v[i][e], kLog2e, -m2));
+            s[0] += valid ? x.v[i][e] : 0.f;
+          }
         }
-        if (c < C) VecIO<T, VEC>::store(out_row + c, out);
       }
-      if (rowloss != nullptr) {
-        // Exactly one thread owns column `id`.  An id outside [0, C) selects no column:
-        // the row's loss term is flagged NaN rather than left unwritten.
-        const bool owner = id_ok && (static_cast<int>(id) / VEC) % TPR == t;
-        if (owner) rowloss[row] = -(picked - shift) * inv_rows;
-        if (!id_ok && t == 0) rowloss[row] = NAN;
+      row_allreduce_sum<TPR, WG, 1>(s, slots, phase);
+      const float k = scale / s[0];
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        if (i <= nfull) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) x.v[i][e] *= k;
+        }
       }
+      x.store(out_row, t, C);
+      const int64_t id = load_id(labels, row, id64 != 0);
+      const bool id_ok = id >= 0 && id < C;
+      const bool owner = id_ok && (static_cast<int>(id) / VEC) % TPR == t;
+      if (owner) {
+        const float xl = to_float(xr[id]);
+        const float lp = xl - m[0] - logf(s[0]);  // log softmax at the label
+        out_row[id] = from_float<T>((fast_exp2(fmaf(xl, kLog2e, -m2)) / s[0] - 1.0f) * scale);
+        if (rowloss != nullptr) rowloss[row] = -lp * inv_rows;
+      }
+      // An id outside [0, C) selects no column: the row's loss term is flagged NaN.
+      if (rowloss != nullptr && !id_ok && t == 0) rowloss[row] = NAN;
     }
   }
 }
@@ -355,11 +380,6 @@ __global__ __launch_bounds__(1024) void sum_rows_kernel(const float* __restrict_
 // Host side
 // ------------------------------------------------------------------------------------
 
-inline int env_int(const char* name, int fallback) {
-  const char* v = std::getenv(name);
-  return (v && *v) ? std::atoi(v) : fallback;
-}
-
 template <typename T>
 struct CrossEntropyOps {
   static constexpr int WIDE = WideVec<T>::value;
@@ -376,12 +396,18 @@ struct CrossEntropyOps {
     else if (chunks <= 2048) *s = {512, 4};
     else if (chunks <= 4096) *s = {512, 8};
     else if (chunks <= 8192) *s = {512, 16};
-    else if (wide && chunks <= 12800) *s = {512, 25};
+    else if (wide && chunks <= 12800) *s = {256, 50};
     else if (wide && chunks <= 16384) *s = {1024, 16};
     else return false;
-    // MOGRAD_HIP_CE_WIDE_ROW=1024 selects the 1024-thread layout for rows of 8193..13312
-    // chunks (13 chunks per thread) instead of 512 threads x 25.
-    if (wide && chunks > 8192 && chunks <= 13312 && env_int("MOGRAD_HIP_CE_WIDE_ROW", 512) == 1024) *s = {1024, 13};
+    // Rows of 8193..12800 chunks (the 50304-column fp32 case): 256 threads x 50 chunks by
+    // default, which leaves room for two workgroups per CU so that one row's arithmetic
+    // overlaps the other's memory traffic.  MOGRAD_HIP_CE_WIDE_ROW=512|1024 selects the
+    // 512 x 25 or 1024 x 13 layout instead (tuning aid).
+    if (wide && chunks > 8192 && chunks <= 12800) {
+      const int pick = env_int("MOGRAD_HIP_CE_WIDE_ROW", 256);
+      if (pick == 512) *s = {512, 25};
+      if (pick == 1024) *s = {1024, 13};
+    }
     return true;
   }
 
@@ -420,6 +446,7 @@ struct CrossEntropyOps {
     MG_CE_CASE(512, 8);
     MG_CE_CASE(512, 16);
     if constexpr (VEC > 1) {
+      MG_CE_CASE(256, 50);
       MG_CE_CASE(512, 25);
       MG_CE_CASE(1024, 13);
       MG_CE_CASE(1024, 16);

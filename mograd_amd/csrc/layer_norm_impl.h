@@ -364,7 +364,7 @@ struct LayerNormOps {
     constexpr int WG = TPR == 64 ? 256 : TPR;
     constexpr int RPW = WG / TPR;
     const int64_t want = ceil_div(rows, RPW);
-    const int64_t cap = static_cast<int64_t>(device_info().cu_count) * 8;
+    const int64_t cap = static_cast<int64_t>(device_info().cu_count) * env_int("MOGRAD_HIP_LN_FWD_WG_PER_CU", 4);
     const unsigned grid = static_cast<unsigned>(want < cap ? want : cap);
     hipLaunchKernelGGL((ln_fwd_rows_kernel<T, VEC, TPR, VPT, WG>), dim3(grid), dim3(WG), 0, stream, x, gamma, beta, y,
                        mean, rstd, rows, static_cast<int>(cols), eps);
@@ -409,7 +409,8 @@ struct LayerNormOps {
   // enough that the (groups, cols) partial sums stay a small fraction of the traffic.
   static int64_t bwd_groups(int64_t rows, int rows_per_iter, int wg) {
     const int64_t cus = device_info().cu_count;
-    const int64_t per_cu = wg >= 512 ? 1 : (wg >= 256 ? 2 : 4);
+    int64_t per_cu = wg >= 512 ? 1 : (wg >= 256 ? 2 : 4);
+    per_cu = env_int("MOGRAD_HIP_LN_GROUPS_PER_CU", static_cast<int>(per_cu));
     int64_t groups = cus * per_cu;
     const int64_t max_groups = ceil_div(rows, rows_per_iter);
     if (groups > max_groups) groups = max_groups;

@@ -6,6 +6,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <string>
 
 #include "mograd_hip.h"
@@ -80,6 +81,13 @@ inline const char* dtype_name(int dtype) {
     case MG_I64: return "int64";
     default: return "?";
   }
+}
+
+// Integer tuning knob from the environment (read on every call; used by benchmarks to
+// compare kernel layouts without rebuilding).
+inline int env_int(const char* name, int fallback) {
+  const char* v = std::getenv(name);
+  return (v && *v) ? std::atoi(v) : fallback;
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

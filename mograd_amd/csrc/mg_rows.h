@@ -19,23 +19,40 @@ struct RowTile {
   // (checked on the host), so 32-bit column arithmetic is enough.
   static __device__ __forceinline__ int col(int i, int t) { return (i * TPR + t) * VEC; }
 
+  // Number of leading chunk indices i for which every one of the TPR threads has a valid
+  // chunk.  It is wave-uniform, so "i < full_chunks(cols)" is a scalar branch: only chunk
+  // index full_chunks(cols) needs per-lane predication, later ones are absent.
+  static __device__ __forceinline__ int full_chunks(int cols) { return (cols / VEC) / TPR; }
+
+  // Addresses are formed as (uniform row pointer + chunk offset) + (unsigned lane offset),
+  // the shape the compiler can turn into scalar-base + 32-bit-vector-offset memory
+  // instructions, so that no per-chunk 64-bit address registers are kept.
   __device__ __forceinline__ void load(const T* row_ptr, int t, int cols) {
+    const unsigned lane_off = static_cast<unsigned>(t) * VEC;
+    const int nfull = full_chunks(cols);
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-      const int c = col(i, t);
-      if (c < cols) {
-        VecIO<T, VEC>::load(row_ptr + c, v[i]);
+      const T* chunk_base = row_ptr + i * (TPR * VEC);
+      if (i < nfull) {
+        VecIO<T, VEC>::load(chunk_base + lane_off, v[i]);
       } else {
 #pragma unroll
         for (int e = 0; e < VEC; ++e) v[i][e] = 0.f;
+        if (i == nfull && col(i, t) < cols) VecIO<T, VEC>::load(chunk_base + lane_off, v[i]);
       }
     }
   }
   __device__ __forceinline__ void store(T* row_ptr, int t, int cols) const {
+    const unsigned lane_off = static_cast<unsigned>(t) * VEC;
+    const int nfull = full_chunks(cols);
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-      const int c = col(i, t);
-      if (c < cols) VecIO<T, VEC>::store(row_ptr + c, v[i]);
+      T* chunk_base = row_ptr + i * (TPR * VEC);
+      if (i < nfull) {
+        VecIO<T, VEC>::store(chunk_base + lane_off, v[i]);
+      } else if (i == nfull && col(i, t) < cols) {
+        VecIO<T, VEC>::store(chunk_base + lane_off, v[i]);
+      }
     }
   }
   __device__ __forceinline__ void zero() {
