@@ -28,8 +28,11 @@
 namespace mg {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 
 template <typename T>
 struct Mma;
@@ -39,8 +42,10 @@ struct Mma<bf16_t> {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0,
                                                    0, 0);
   }
+  // Two fp32 -> packed pair, round to nearest even (one v_cvt_pk_bf16_f32).
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    return static_cast<uint32_t>(bf16_bits_rne(lo)) | (static_cast<uint32_t>(bf16_bits_rne(hi)) << 16);
+    const float2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
   }
 };
 template <>
@@ -50,14 +55,14 @@ struct Mma<f16_t> {
                                                   0);
   }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    union { uint32_t u; f16_t h[2]; } cv;
-    cv.h[0] = static_cast<f16_t>(lo);
-    cv.h[1] = static_cast<f16_t>(hi);
-    return cv.u;
+    const float2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
   }
 };
 
 constexpr int kAttnThreads = 256;
+
+__device__ __forceinline__ float fexp2(float v) { return __builtin_amdgcn_exp2f(v); }
 
 // ---- LDS tiles -------------------------------------------------------------------------
 // Row-major tile: R rows x DP columns of T, row stride DP + 8 elements (the 16-byte pad
@@ -69,44 +74,64 @@ constexpr int row_stride() { return DP + 8; }
 template <int R>
 constexpr int tr_stride_dw() { return R / 2 + 2; }
 
-// Global rows [r0, r0 + R) of a matrix whose row `r` starts at base + r * ld (elements),
-// D valid columns, rows >= r_end read as zero.  Writes the row-major tile.
+// Global -> registers -> LDS staging of R rows x DP columns.  A thread owns "pair chunks":
+// 8 columns of two consecutive rows.  Fetching into registers and committing to LDS are
+// separate so that the next tile's loads can be in flight while the current tile is used.
+// From the same registers a tile can be committed row-major, transposed, or both.
 template <typename T, int R, int DP>
-__device__ __forceinline__ void stage_rows(uint16_t* __restrict__ lds, const T* __restrict__ base, int64_t ld, int r0,
-                                           int r_end, int D) {
-  constexpr int CH = DP / 8;  // 16-byte chunks per row
-  for (int idx = threadIdx.x; idx < R * CH; idx += kAttnThreads) {
-    const int r = idx / CH, c = idx % CH;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (r0 + r < r_end && c * 8 < D) v = *reinterpret_cast<const uint4*>(base + (r0 + r) * ld + c * 8);
-    *reinterpret_cast<uint4*>(lds + r * row_stride<DP>() + c * 8) = v;
-  }
-}
+struct TileStager {
+  static constexpr int CH = DP / 8;
+  static constexpr int PAIRS = R / 2;
+  static constexpr int TASKS = PAIRS * CH;
+  static constexpr int PER = (TASKS + kAttnThreads - 1) / kAttnThreads;
+  uint4 lo[PER], hi[PER];
 
-// Same rows, written transposed: dword (d, p) holds columns 2p and 2p+1 of row d.
-template <typename T, int R, int DP>
-__device__ __forceinline__ void stage_transposed(uint32_t* __restrict__ lds, const T* __restrict__ base, int64_t ld,
-                                                 int r0, int r_end, int D) {
-  constexpr int CH = DP / 8;
-  constexpr int PAIRS = R / 2;
-  for (int idx = threadIdx.x; idx < PAIRS * CH; idx += kAttnThreads) {
-    const int p = idx % PAIRS, c = idx / PAIRS;
-    uint4 lo = make_uint4(0, 0, 0, 0), hi = make_uint4(0, 0, 0, 0);
-    const int ra = r0 + 2 * p;
-    if (c * 8 < D) {
-      if (ra < r_end) lo = *reinterpret_cast<const uint4*>(base + ra * ld + c * 8);
-      if (ra + 1 < r_end) hi = *reinterpret_cast<const uint4*>(base + (ra + 1) * ld + c * 8);
-    }
-    const uint32_t a[4] = {lo.x, lo.y, lo.z, lo.w};
-    const uint32_t b[4] = {hi.x, hi.y, hi.z, hi.w};
-    uint32_t* dst = lds + (c * 8) * tr_stride_dw<R>() + p;
+  // Rows [r0, r0 + R) of a matrix whose row r starts at base + r * ld (elements); D valid
+  // columns; rows >= r_end and columns >= D read as zero.
+  __device__ __forceinline__ void fetch(const T* __restrict__ base, int64_t ld, int r0, int r_end, int D) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      dst[(2 * e) * tr_stride_dw<R>()] = (a[e] & 0xffffu) | (b[e] << 16);
-      dst[(2 * e + 1) * tr_stride_dw<R>()] = (a[e] >> 16) | (b[e] & 0xffff0000u);
+    for (int i = 0; i < PER; ++i) {
+      const int idx = threadIdx.x + i * kAttnThreads;
+      const int p = idx % PAIRS, c = idx / PAIRS;
+      const int ra = r0 + 2 * p;
+      lo[i] = make_uint4(0, 0, 0, 0);
+      hi[i] = make_uint4(0, 0, 0, 0);
+      if (idx < TASKS && c * 8 < D) {
+        if (ra < r_end) lo[i] = *reinterpret_cast<const uint4*>(base + ra * ld + c * 8);
+        if (ra + 1 < r_end) hi[i] = *reinterpret_cast<const uint4*>(base + (ra + 1) * ld + c * 8);
+      }
     }
   }
-}
+  __device__ __forceinline__ void commit_rows(uint16_t* __restrict__ lds) const {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = threadIdx.x + i * kAttnThreads;
+      const int p = idx % PAIRS, c = idx / PAIRS;
+      if (idx < TASKS) {
+        *reinterpret_cast<uint4*>(lds + (2 * p) * row_stride<DP>() + c * 8) = lo[i];
+        *reinterpret_cast<uint4*>(lds + (2 * p + 1) * row_stride<DP>() + c * 8) = hi[i];
+      }
+    }
+  }
+  // dword (d, p) of the transposed tile holds columns 2p and 2p+1 of row d.
+  __device__ __forceinline__ void commit_transposed(uint32_t* __restrict__ lds) const {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = threadIdx.x + i * kAttnThreads;
+      const int p = idx % PAIRS, c = idx / PAIRS;
+      if (idx < TASKS) {
+        const uint32_t a[4] = {lo[i].x, lo[i].y, lo[i].z, lo[i].w};
+        const uint32_t b[4] = {hi[i].x, hi[i].y, hi[i].z, hi[i].w};
+        uint32_t* dst = lds + (c * 8) * tr_stride_dw<R>() + p;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          dst[(2 * e) * tr_stride_dw<R>()] = __builtin_amdgcn_perm(b[e], a[e], 0x05040100);
+          dst[(2 * e + 1) * tr_stride_dw<R>()] = __builtin_amdgcn_perm(b[e], a[e], 0x07060302);
+        }
+      }
+    }
+  }
+};
 
 // A operand from a row-major tile: rows rt*32 + lane%32, columns ks*16 + (lane/32)*8 .. +7.
 template <int DP>
@@ -147,19 +172,29 @@ __device__ __forceinline__ floatx16 zero16() {
 
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
+// Packed store of four consecutive accumulator registers (four consecutive d) times `f`.
+template <typename T>
+__device__ __forceinline__ void store4(T* dst, const floatx16& acc, int g, float f) {
+  uint2 w;
+  w.x = Mma<T>::pack2(acc[g * 4] * f, acc[g * 4 + 1] * f);
+  w.y = Mma<T>::pack2(acc[g * 4 + 2] * f, acc[g * 4 + 3] * f);
+  *reinterpret_cast<uint2*>(dst) = w;
+}
+
 // ---- forward -----------------------------------------------------------------------------
 
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
-__global__ __launch_bounds__(kAttnThreads) void attn_fwd_mfma_kernel(const T* __restrict__ q, const T* __restrict__ k,
-                                                                     const T* __restrict__ v, const T* __restrict__ mask,
-                                                                     T* __restrict__ o, float* __restrict__ lse,
-                                                                     AttnDims a, float scale) {
+__global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                                        const T* __restrict__ v,
+                                                                        const T* __restrict__ mask, T* __restrict__ o,
+                                                                        float* __restrict__ lse, AttnDims a, float scale) {
   constexpr int BM = 128, BN = 64, KS = DP / 16, DT = DP / 32;
   __shared__ __attribute__((aligned(16))) uint16_t k_rows[BN * row_stride<DP>()];
   __shared__ __attribute__((aligned(16))) uint32_t v_tr[DP * tr_stride_dw<BN>()];
 
   const int nqb = (a.S + BM - 1) / BM;
-  const int qb = blockIdx.x % nqb;
+  // Causal: later query blocks have more keys to visit; launch them first.
+  const int qb = CAUSAL ? nqb - 1 - blockIdx.x % nqb : blockIdx.x % nqb;
   const int h = (blockIdx.x / nqb) % a.H;
   const int b = blockIdx.x / (nqb * a.H);
   const int lane = threadIdx.x % kWave;
@@ -185,11 +220,18 @@ __global__ __launch_bounds__(kAttnThreads) void attn_fwd_mfma_kernel(const T* __
   const T* mrow = HAS_BIAS ? mask + ((static_cast<int64_t>(b) * a.H + h) * a.S + min(m, a.S - 1)) * a.S : nullptr;
 
   const int n_end = CAUSAL ? min(a.S, qb * BM + BM) : a.S;
+  TileStager<T, BN, DP> ks_stage, vs_stage;
+  ks_stage.fetch(kbase, ld, 0, a.S, a.D);
+  vs_stage.fetch(vbase, ld, 0, a.S, a.D);
   for (int n0 = 0; n0 < n_end; n0 += BN) {
     __syncthreads();
-    stage_rows<T, BN, DP>(k_rows, kbase, ld, n0, a.S, a.D);
-    stage_transposed<T, BN, DP>(v_tr, vbase, ld, n0, a.S, a.D);
+    ks_stage.commit_rows(k_rows);
+    vs_stage.commit_transposed(v_tr);
     __syncthreads();
+    if (n0 + BN < n_end) {
+      ks_stage.fetch(kbase, ld, n0 + BN, a.S, a.D);
+      vs_stage.fetch(vbase, ld, n0 + BN, a.S, a.D);
+    }
     if (CAUSAL && n0 > m_wave + 31) continue;  // every key of the block is in this wave's future
 
     floatx16 s[2];
@@ -199,38 +241,64 @@ __global__ __launch_bounds__(kAttnThreads) void attn_fwd_mfma_kernel(const T* __
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) s[nt] = Mma<T>::run(frag_rows<DP>(k_rows, nt, ks, lane), qf[ks], s[nt]);
     }
-    // scale, bias, mask -> log2-domain scores; row maximum of this lane's query
-    float mx = -INFINITY;
+    // A block needs per-element masking only at the end of the sequence and, for causal
+    // attention, where it crosses the diagonal of this wave's queries.
+    const bool plain = !HAS_BIAS && c > 0.f && n0 + BN <= a.S && (!CAUSAL || n0 + BN - 1 <= m_wave);
+    float corr;
+    if (plain) {
+      float mx = s[0][0];
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+      for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int n = n0 + nt * 32 + acc_row(r, lane);
-        bool valid = n < a.S;
-        if (CAUSAL) valid = valid && n <= m;
-        float sv = s[nt][r] * c;
-        if (HAS_BIAS) sv = valid ? fmaf(to_float(mrow[n]), kAttnLog2e, sv) : sv;
-        sv = valid ? sv : -INFINITY;
-        s[nt][r] = sv;
-        mx = fmaxf(mx, sv);
-      }
-    mx = fmaxf(mx, xor32(mx));
-    const float m_new = fmaxf(m_run, mx);
-    // m_new is -inf only for rows past the end of the sequence (all their keys masked)
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float corr = exp2f(m_run - m_use);
-    float lsum = 0.f;
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[nt][r]);
+      mx = fmaxf(mx, xor32(mx)) * c;
+      const float m_new = fmaxf(m_run, mx);
+      corr = fexp2(m_run - m_new);
+      float lsum = 0.f;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+      for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float p = exp2f(s[nt][r] - m_use);
-        s[nt][r] = p;
-        lsum += p;
-      }
-    lsum += xor32(lsum);
-    l_run = l_run * corr + lsum;
-    m_run = m_new;
+        for (int r = 0; r < 16; ++r) {
+          const float p = fexp2(fmaf(s[nt][r], c, -m_new));
+          s[nt][r] = p;
+          lsum += p;
+        }
+      lsum += xor32(lsum);
+      l_run = l_run * corr + lsum;
+      m_run = m_new;
+    } else {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int n = n0 + nt * 32 + acc_row(r, lane);
+          bool valid = n < a.S;
+          if (CAUSAL) valid = valid && n <= m;
+          float sv = s[nt][r] * c;
+          if (HAS_BIAS) sv = valid ? fmaf(to_float(mrow[n]), kAttnLog2e, sv) : sv;
+          sv = valid ? sv : -INFINITY;
+          s[nt][r] = sv;
+          mx = fmaxf(mx, sv);
+        }
+      mx = fmaxf(mx, xor32(mx));
+      const float m_new = fmaxf(m_run, mx);
+      // m_new is -inf only for rows past the end of the sequence (all their keys masked)
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      corr = fexp2(m_run - m_use);
+      float lsum = 0.f;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float p = fexp2(s[nt][r] - m_use);
+          s[nt][r] = p;
+          lsum += p;
+        }
+      lsum += xor32(lsum);
+      l_run = l_run * corr + lsum;
+      m_run = m_new;
+    }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -251,12 +319,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_fwd_mfma_kernel(const T* __
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int d = dt * 32 + g * 8 + half * 4;
-        if (d < a.D) {
-          uint2 w;
-          w.x = Mma<T>::pack2(acc_o[dt][g * 4] * inv, acc_o[dt][g * 4 + 1] * inv);
-          w.y = Mma<T>::pack2(acc_o[dt][g * 4 + 2] * inv, acc_o[dt][g * 4 + 3] * inv);
-          *reinterpret_cast<uint2*>(orow + d) = w;
-        }
+        if (d < a.D) store4<T>(orow + d, acc_o[dt], g, inv);
       }
     if (half == 0) lse[(static_cast<int64_t>(b) * a.H + h) * a.S + m] = m_run * kAttnLn2 + logf(l_run);
   }
@@ -265,18 +328,19 @@ __global__ __launch_bounds__(kAttnThreads) void attn_fwd_mfma_kernel(const T* __
 // ---- dQ ----------------------------------------------------------------------------------
 
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
-__global__ __launch_bounds__(kAttnThreads) void attn_dq_mfma_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
-                                                                    const T* __restrict__ k, const T* __restrict__ v,
-                                                                    const T* __restrict__ mask, const float* __restrict__ lse,
-                                                                    const float* __restrict__ delta, T* __restrict__ dq,
-                                                                    AttnDims a, float scale) {
+__global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
+                                                                       const T* __restrict__ k, const T* __restrict__ v,
+                                                                       const T* __restrict__ mask,
+                                                                       const float* __restrict__ lse,
+                                                                       const float* __restrict__ delta,
+                                                                       T* __restrict__ dq, AttnDims a, float scale) {
   constexpr int BM = 128, BN = 64, KS = DP / 16, DT = DP / 32;
   __shared__ __attribute__((aligned(16))) uint16_t k_rows[BN * row_stride<DP>()];
   __shared__ __attribute__((aligned(16))) uint16_t v_rows[BN * row_stride<DP>()];
   __shared__ __attribute__((aligned(16))) uint32_t k_tr[DP * tr_stride_dw<BN>()];
 
   const int nqb = (a.S + BM - 1) / BM;
-  const int qb = blockIdx.x % nqb;
+  const int qb = CAUSAL ? nqb - 1 - blockIdx.x % nqb : blockIdx.x % nqb;
   const int h = (blockIdx.x / nqb) % a.H;
   const int b = blockIdx.x / (nqb * a.H);
   const int lane = threadIdx.x % kWave;
@@ -307,12 +371,19 @@ __global__ __launch_bounds__(kAttnThreads) void attn_dq_mfma_kernel(const T* __r
   const T* mrow = HAS_BIAS ? mask + (bh * a.S + min(m, a.S - 1)) * a.S : nullptr;
 
   const int n_end = CAUSAL ? min(a.S, qb * BM + BM) : a.S;
+  TileStager<T, BN, DP> ks_stage, vs_stage;
+  ks_stage.fetch(kbase, ld, 0, a.S, a.D);
+  vs_stage.fetch(vbase, ld, 0, a.S, a.D);
   for (int n0 = 0; n0 < n_end; n0 += BN) {
     __syncthreads();
-    stage_rows<T, BN, DP>(k_rows, kbase, ld, n0, a.S, a.D);
-    stage_rows<T, BN, DP>(v_rows, vbase, ld, n0, a.S, a.D);
-    stage_transposed<T, BN, DP>(k_tr, kbase, ld, n0, a.S, a.D);
+    ks_stage.commit_rows(k_rows);
+    ks_stage.commit_transposed(k_tr);
+    vs_stage.commit_rows(v_rows);
     __syncthreads();
+    if (n0 + BN < n_end) {
+      ks_stage.fetch(kbase, ld, n0 + BN, a.S, a.D);
+      vs_stage.fetch(vbase, ld, n0 + BN, a.S, a.D);
+    }
     if (CAUSAL && n0 > m_wave + 31) continue;
 
     floatx16 s[2], dp[2];
@@ -326,18 +397,26 @@ __global__ __launch_bounds__(kAttnThreads) void attn_dq_mfma_kernel(const T* __r
         dp[nt] = Mma<T>::run(frag_rows<DP>(v_rows, nt, ks, lane), dof[ks], dp[nt]);
       }
     }
+    const bool plain = !HAS_BIAS && n0 + BN <= a.S && (!CAUSAL || n0 + BN - 1 <= m_wave);
+    if (plain) {
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+      for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int n = n0 + nt * 32 + acc_row(r, lane);
-        bool valid = n < a.S;
-        if (CAUSAL) valid = valid && n <= m;
-        float sv = s[nt][r] * c;
-        if (HAS_BIAS) sv = valid ? fmaf(to_float(mrow[n]), kAttnLog2e, sv) : sv;
-        const float p = valid ? exp2f(sv - lse2) : 0.f;
-        s[nt][r] = p * (dp[nt][r] - dl);  // dS^T
-      }
+        for (int r = 0; r < 16; ++r) s[nt][r] = fexp2(fmaf(s[nt][r], c, -lse2)) * (dp[nt][r] - dl);
+    } else {
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int n = n0 + nt * 32 + acc_row(r, lane);
+          bool valid = n < a.S;
+          if (CAUSAL) valid = valid && n <= m;
+          float sv = s[nt][r] * c;
+          if (HAS_BIAS) sv = valid ? fmaf(to_float(mrow[n]), kAttnLog2e, sv) : sv;
+          const float p = valid ? fexp2(sv - lse2) : 0.f;
+          s[nt][r] = p * (dp[nt][r] - dl);  // dS^T
+        }
+    }
 #pragma unroll
     for (int t = 0; t < BN / 16; ++t) {
       const uint4 dsf = frag_from_acc<T>(s[t / 2], t % 2);
@@ -353,12 +432,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_dq_mfma_kernel(const T* __r
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int d = dt * 32 + g * 8 + half * 4;
-        if (d < a.D) {
-          uint2 w;
-          w.x = Mma<T>::pack2(acc[dt][g * 4] * scale, acc[dt][g * 4 + 1] * scale);
-          w.y = Mma<T>::pack2(acc[dt][g * 4 + 2] * scale, acc[dt][g * 4 + 3] * scale);
-          *reinterpret_cast<uint2*>(out + d) = w;
-        }
+        if (d < a.D) store4<T>(out + d, acc[dt], g, scale);
       }
   }
 }
@@ -366,12 +440,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_dq_mfma_kernel(const T* __r
 // ---- dK, dV ------------------------------------------------------------------------------
 
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
-__global__ __launch_bounds__(kAttnThreads) void attn_dkdv_mfma_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
-                                                                      const T* __restrict__ k, const T* __restrict__ v,
-                                                                      const T* __restrict__ mask,
-                                                                      const float* __restrict__ lse,
-                                                                      const float* __restrict__ delta, T* __restrict__ dk,
-                                                                      T* __restrict__ dv, AttnDims a, float scale) {
+__global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
+    const T* __restrict__ d_o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+    const T* __restrict__ mask, const float* __restrict__ lse, const float* __restrict__ delta, T* __restrict__ dk,
+    T* __restrict__ dv, AttnDims a, float scale) {
   constexpr int BNK = 128;                 // keys per workgroup
   constexpr int BQ = DP <= 64 ? 64 : 32;   // queries per step (LDS budget)
   constexpr int MT = BQ / 32, KS = DP / 16, DT = DP / 32;
@@ -383,6 +455,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_dkdv_mfma_kernel(const T* _
   __shared__ __attribute__((aligned(16))) float delta_s[BQ];
 
   const int nkb = (a.S + BNK - 1) / BNK;
+  // Causal: earlier key blocks are seen by more queries; they already come first.
   const int kb = blockIdx.x % nkb;
   const int h = (blockIdx.x / nkb) % a.H;
   const int b = blockIdx.x / (nkb * a.H);
@@ -414,18 +487,35 @@ __global__ __launch_bounds__(kAttnThreads) void attn_dkdv_mfma_kernel(const T* _
 
   // Causal: queries before the workgroup's first key see none of its keys.
   const int m_begin = CAUSAL ? (kb * BNK / BQ) * BQ : 0;
+  TileStager<T, BQ, DP> q_stage, do_stage;
+  q_stage.fetch(qbase, ld, m_begin, a.S, a.D);
+  do_stage.fetch(dobase, a.D, m_begin, a.S, a.D);
+  float lse_next = INFINITY, delta_next = 0.f;
+  if (threadIdx.x < BQ && m_begin + threadIdx.x < a.S) {
+    lse_next = lse[bh * a.S + m_begin + threadIdx.x] * kAttnLog2e;
+    delta_next = delta[bh * a.S + m_begin + threadIdx.x];
+  }
   for (int m0 = m_begin; m0 < a.S; m0 += BQ) {
     __syncthreads();
-    stage_rows<T, BQ, DP>(q_rows, qbase, ld, m0, a.S, a.D);
-    stage_rows<T, BQ, DP>(do_rows, dobase, a.D, m0, a.S, a.D);
-    stage_transposed<T, BQ, DP>(q_tr, qbase, ld, m0, a.S, a.D);
-    stage_transposed<T, BQ, DP>(do_tr, dobase, a.D, m0, a.S, a.D);
+    q_stage.commit_rows(q_rows);
+    q_stage.commit_transposed(q_tr);
+    do_stage.commit_rows(do_rows);
+    do_stage.commit_transposed(do_tr);
     if (threadIdx.x < BQ) {
-      const int mm = m0 + threadIdx.x;
-      lse_s[threadIdx.x] = mm < a.S ? lse[bh * a.S + mm] * kAttnLog2e : INFINITY;
-      delta_s[threadIdx.x] = mm < a.S ? delta[bh * a.S + mm] : 0.f;
+      lse_s[threadIdx.x] = lse_next;  // rows past the end carry lse = +inf, delta = 0
+      delta_s[threadIdx.x] = delta_next;
     }
     __syncthreads();
+    if (m0 + BQ < a.S) {
+      q_stage.fetch(qbase, ld, m0 + BQ, a.S, a.D);
+      do_stage.fetch(dobase, a.D, m0 + BQ, a.S, a.D);
+      lse_next = INFINITY;
+      delta_next = 0.f;
+      if (threadIdx.x < BQ && m0 + BQ + threadIdx.x < a.S) {
+        lse_next = lse[bh * a.S + m0 + BQ + threadIdx.x] * kAttnLog2e;
+        delta_next = delta[bh * a.S + m0 + BQ + threadIdx.x];
+      }
+    }
     if (CAUSAL && m0 + BQ - 1 < n_wave) continue;  // all of this step's queries precede the wave's keys
 
     floatx16 s[MT], dp[MT];
@@ -439,21 +529,43 @@ __global__ __launch_bounds__(kAttnThreads) void attn_dkdv_mfma_kernel(const T* _
         dp[mt] = Mma<T>::run(frag_rows<DP>(do_rows, mt, ks, lane), vf[ks], dp[mt]);
       }
     }
-    // s -> P, dp -> dS (both: column = this lane's key, rows = queries)
+    // s -> P, dp -> dS (both: column = this lane's key, rows = queries).  Per-element
+    // masking is needed only for key columns past the end and where the step crosses the
+    // diagonal of this wave's keys.
+    const bool plain = !HAS_BIAS && n_wave + 31 < a.S && (!CAUSAL || n_wave + 31 <= m0);
+    if (plain) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+      for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int ml = mt * 32 + acc_row(r, lane);
-        const int mm = m0 + ml;
-        bool valid = n < a.S;  // rows past the end carry lse = +inf
-        if (CAUSAL) valid = valid && n <= mm;
-        float sv = s[mt][r] * c;
-        if (HAS_BIAS) sv = (valid && mm < a.S) ? fmaf(to_float(mask[(bh * a.S + mm) * a.S + n]), kAttnLog2e, sv) : sv;
-        const float p = valid ? exp2f(sv - lse_s[ml]) : 0.f;
-        s[mt][r] = p;
-        dp[mt][r] = p * (dp[mt][r] - delta_s[ml]);
-      }
+        for (int g = 0; g < 4; ++g) {
+          const float4 l4 = *reinterpret_cast<const float4*>(&lse_s[mt * 32 + g * 8 + half * 4]);
+          const float4 d4 = *reinterpret_cast<const float4*>(&delta_s[mt * 32 + g * 8 + half * 4]);
+          const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
+          const float dv4[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int r = g * 4 + j;
+            const float p = fexp2(fmaf(s[mt][r], c, -lv[j]));
+            s[mt][r] = p;
+            dp[mt][r] = p * (dp[mt][r] - dv4[j]);
+          }
+        }
+    } else {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int ml = mt * 32 + acc_row(r, lane);
+          const int mm = m0 + ml;
+          bool valid = n < a.S;
+          if (CAUSAL) valid = valid && n <= mm;
+          float sv = s[mt][r] * c;
+          if (HAS_BIAS) sv = (valid && mm < a.S) ? fmaf(to_float(mask[(bh * a.S + mm) * a.S + n]), kAttnLog2e, sv) : sv;
+          const float p = valid ? fexp2(sv - lse_s[ml]) : 0.f;
+          s[mt][r] = p;
+          dp[mt][r] = p * (dp[mt][r] - delta_s[ml]);
+        }
+    }
 #pragma unroll
     for (int t = 0; t < BQ / 16; ++t) {
       const uint4 pf = frag_from_acc<T>(s[t / 2], t % 2);
@@ -475,13 +587,8 @@ __global__ __launch_bounds__(kAttnThreads) void attn_dkdv_mfma_kernel(const T* _
       for (int g = 0; g < 4; ++g) {
         const int d = dt * 32 + g * 8 + half * 4;
         if (d < a.D) {
-          uint2 wk, wv;
-          wk.x = Mma<T>::pack2(acc_k[dt][g * 4] * scale, acc_k[dt][g * 4 + 1] * scale);
-          wk.y = Mma<T>::pack2(acc_k[dt][g * 4 + 2] * scale, acc_k[dt][g * 4 + 3] * scale);
-          wv.x = Mma<T>::pack2(acc_v[dt][g * 4], acc_v[dt][g * 4 + 1]);
-          wv.y = Mma<T>::pack2(acc_v[dt][g * 4 + 2], acc_v[dt][g * 4 + 3]);
-          *reinterpret_cast<uint2*>(outk + d) = wk;
-          *reinterpret_cast<uint2*>(outv + d) = wv;
+          store4<T>(outk + d, acc_k[dt], g, scale);
+          store4<T>(outv + d, acc_v[dt], g, 1.0f);
         }
       }
   }
