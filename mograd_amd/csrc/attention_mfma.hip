@@ -518,24 +518,21 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
     }
     if (CAUSAL && m0 + BQ - 1 < n_wave) continue;  // all of this step's queries precede the wave's keys
 
-    floatx16 s[MT], dp[MT];
+    // Per-element masking is needed only for key columns past the end and where the step
+    // crosses the diagonal of this wave's keys.
+    const bool plain = !HAS_BIAS && n_wave + 31 < a.S && (!CAUSAL || n_wave + 31 <= m0);
+    // One 32-query tile at a time: S and dP (column = this lane's key, rows = queries),
+    // then P and dS in place, then their contributions to dV and dK.  Only one tile's
+    // scores are live, and the next tile's products can run under this tile's arithmetic.
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      s[mt] = zero16();
-      dp[mt] = zero16();
+      floatx16 s = zero16(), dp = zero16();
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        s[mt] = Mma<T>::run(frag_rows<DP>(q_rows, mt, ks, lane), kf[ks], s[mt]);
-        dp[mt] = Mma<T>::run(frag_rows<DP>(do_rows, mt, ks, lane), vf[ks], dp[mt]);
+        s = Mma<T>::run(frag_rows<DP>(q_rows, mt, ks, lane), kf[ks], s);
+        dp = Mma<T>::run(frag_rows<DP>(do_rows, mt, ks, lane), vf[ks], dp);
       }
-    }
-    // s -> P, dp -> dS (both: column = this lane's key, rows = queries).  Per-element
-    // masking is needed only for key columns past the end and where the step crosses the
-    // diagonal of this wave's keys.
-    const bool plain = !HAS_BIAS && n_wave + 31 < a.S && (!CAUSAL || n_wave + 31 <= m0);
-    if (plain) {
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+      if (plain) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const float4 l4 = *reinterpret_cast<const float4*>(&lse_s[mt * 32 + g * 8 + half * 4]);
@@ -545,35 +542,35 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const int r = g * 4 + j;
-            const float p = fexp2(fmaf(s[mt][r], c, -lv[j]));
-            s[mt][r] = p;
-            dp[mt][r] = p * (dp[mt][r] - dv4[j]);
+            const float p = fexp2(fmaf(s[r], c, -lv[j]));
+            s[r] = p;
+            dp[r] = p * (dp[r] - dv4[j]);
           }
         }
-    } else {
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+      } else {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int ml = mt * 32 + acc_row(r, lane);
           const int mm = m0 + ml;
           bool valid = n < a.S;
           if (CAUSAL) valid = valid && n <= mm;
-          float sv = s[mt][r] * c;
+          float sv = s[r] * c;
           if (HAS_BIAS) sv = (valid && mm < a.S) ? fmaf(to_float(mask[(bh * a.S + mm) * a.S + n]), kAttnLog2e, sv) : sv;
           const float p = valid ? fexp2(sv - lse_s[ml]) : 0.f;
-          s[mt][r] = p;
-          dp[mt][r] = p * (dp[mt][r] - delta_s[ml]);
+          s[r] = p;
+          dp[r] = p * (dp[r] - delta_s[ml]);
         }
-    }
+      }
 #pragma unroll
-    for (int t = 0; t < BQ / 16; ++t) {
-      const uint4 pf = frag_from_acc<T>(s[t / 2], t % 2);
-      const uint4 dsf = frag_from_acc<T>(dp[t / 2], t % 2);
+      for (int hf = 0; hf < 2; ++hf) {
+        const int t = mt * 2 + hf;
+        const uint4 pf = frag_from_acc<T>(s, hf);
+        const uint4 dsf = frag_from_acc<T>(dp, hf);
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        acc_v[dt] = Mma<T>::run(frag_transposed<BQ>(do_tr, dt, t, lane), pf, acc_v[dt]);
-        acc_k[dt] = Mma<T>::run(frag_transposed<BQ>(q_tr, dt, t, lane), dsf, acc_k[dt]);
+        for (int dt = 0; dt < DT; ++dt) {
+          acc_v[dt] = Mma<T>::run(frag_transposed<BQ>(do_tr, dt, t, lane), pf, acc_v[dt]);
+          acc_k[dt] = Mma<T>::run(frag_transposed<BQ>(q_tr, dt, t, lane), dsf, acc_k[dt]);
+        }
       }
     }
   }
