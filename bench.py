@@ -199,6 +199,12 @@ def main() -> int:
         ln_bwd(i)
         ce_fused(i)
 
+    # One plain device-to-device copy of known size (logits -> dlogits, 1.648 GB each way),
+    # outside every timed region: under `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` it is the
+    # calibration that the counters of the real kernels are scaled by.
+    lib.mg_copy_device(dlogits.data_ptr(), logits.data_ptr(), CE_ROWS * CE_COLS * 4, st)
+    dev.synchronize()
+
     # ---- whole step: W warm-up steps, then exactly K timed steps -------------------------
     for i in range(args.warmup):
         step(i)
