@@ -39,6 +39,12 @@ LN_FWD_BYTES = 2 * LN_ROWS * LN_COLS * 4 + 2 * LN_COLS * 4            # x, y, ga
 LN_BWD_BYTES = 3 * LN_ROWS * LN_COLS * 4 + 3 * LN_COLS * 4            # dy, x, dx, gamma, dgamma, dbeta
 CE_FUSED_BYTES = 2 * CE_ROWS * CE_COLS * 4 + CE_ROWS * 4 + 4          # logits, dlogits, labels, loss
 
+# HBM bytes per launch of the cross-entropy rows kernel, from two `rocprofv3 --pmc` runs
+# (FETCH_SIZE, then WRITE_SIZE) of this same script, each scaled by what the counter reads
+# for the calibration copy below: (805943.2 / 0.50005 + 1610376.8 / 1.0) KiB.  The counter
+# runs and the factors are in profiles/ce_rows_kernel_8192x50304_hbm_traffic.md.
+CE_MEASURED_TRAFFIC_BYTES = int((805943.2 / 0.50005 + 1610376.8) * 1024)
+
 
 def _rng(config: int, tensor: int) -> np.random.Generator:
     return np.random.Generator(np.random.PCG64(1000 * config + tensor))
@@ -260,7 +266,7 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(dominant["achieved_GBps"] / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": CE_MEASURED_TRAFFIC_BYTES,
         },
         "kernels": kernels,
     }
