@@ -326,15 +326,17 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
 }
 
 // ---- dQ ----------------------------------------------------------------------------------
+// A wave owns MQ tiles of 32 queries; every A fragment read from LDS (K rows, V rows,
+// K^T) feeds MQ MFMAs, which is what keeps LDS bandwidth below the MFMA rate.
 
-template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
+template <typename T, int DP, int MQ, bool CAUSAL, bool HAS_BIAS>
 __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
                                                                        const T* __restrict__ k, const T* __restrict__ v,
                                                                        const T* __restrict__ mask,
                                                                        const float* __restrict__ lse,
                                                                        const float* __restrict__ delta,
                                                                        T* __restrict__ dq, AttnDims a, float scale) {
-  constexpr int BM = 128, BN = 64, KS = DP / 16, DT = DP / 32;
+  constexpr int BM = 128 * MQ, BN = 64, KS = DP / 16, DT = DP / 32;
   __shared__ __attribute__((aligned(16))) uint16_t k_rows[BN * row_stride<DP>()];
   __shared__ __attribute__((aligned(16))) uint16_t v_rows[BN * row_stride<DP>()];
   __shared__ __attribute__((aligned(16))) uint32_t k_tr[DP * tr_stride_dw<BN>()];
@@ -346,29 +348,35 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int half = lane / 32;
-  const int m_wave = qb * BM + wave * 32;
-  const int m = m_wave + lane % 32;
+  const int m_wave = qb * BM + wave * (32 * MQ);
   const int64_t ld = static_cast<int64_t>(a.H) * a.D;
   const T* kbase = k + bshd(a, b, 0, h);
   const T* vbase = v + bshd(a, b, 0, h);
   const int64_t bh = static_cast<int64_t>(b) * a.H + h;
 
-  uint4 qf[KS], dof[KS];
+  int m[MQ];
+  uint4 qf[MQ][KS], dof[MQ][KS];
+  float lse2[MQ], dl[MQ];
+  const T* mrow[MQ];
+  floatx16 acc[MQ][DT];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    const int d = ks * 16 + half * 8;
-    const bool ok = m < a.S && d < a.D;
-    qf[ks] = ok ? *reinterpret_cast<const uint4*>(q + bshd(a, b, m, h) + d) : make_uint4(0, 0, 0, 0);
-    dof[ks] = ok ? *reinterpret_cast<const uint4*>(d_o + bhsd(a, b, h, m) + d) : make_uint4(0, 0, 0, 0);
+  for (int mq = 0; mq < MQ; ++mq) {
+    m[mq] = m_wave + mq * 32 + lane % 32;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 16 + half * 8;
+      const bool ok = m[mq] < a.S && d < a.D;
+      qf[mq][ks] = ok ? *reinterpret_cast<const uint4*>(q + bshd(a, b, m[mq], h) + d) : make_uint4(0, 0, 0, 0);
+      dof[mq][ks] = ok ? *reinterpret_cast<const uint4*>(d_o + bhsd(a, b, h, m[mq]) + d) : make_uint4(0, 0, 0, 0);
+    }
+    // Rows past the end get lse = +inf so that their probabilities vanish.
+    lse2[mq] = m[mq] < a.S ? lse[bh * a.S + m[mq]] * kAttnLog2e : INFINITY;
+    dl[mq] = m[mq] < a.S ? delta[bh * a.S + m[mq]] : 0.f;
+    mrow[mq] = HAS_BIAS ? mask + (bh * a.S + min(m[mq], a.S - 1)) * a.S : nullptr;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[mq][dt] = zero16();
   }
-  // Rows past the end get lse = +inf so that their probabilities vanish.
-  const float lse2 = m < a.S ? lse[bh * a.S + m] * kAttnLog2e : INFINITY;
-  const float dl = m < a.S ? delta[bh * a.S + m] : 0.f;
-  floatx16 acc[DT];
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
   const float c = scale * kAttnLog2e;
-  const T* mrow = HAS_BIAS ? mask + (bh * a.S + min(m, a.S - 1)) * a.S : nullptr;
 
   const int n_end = CAUSAL ? min(a.S, qb * BM + BM) : a.S;
   TileStager<T, BN, DP> ks_stage, vs_stage;
@@ -384,56 +392,76 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
       ks_stage.fetch(kbase, ld, n0 + BN, a.S, a.D);
       vs_stage.fetch(vbase, ld, n0 + BN, a.S, a.D);
     }
-    if (CAUSAL && n0 > m_wave + 31) continue;
+    if (CAUSAL && n0 > m_wave + 32 * MQ - 1) continue;  // every key of the block is in this wave's future
 
-    floatx16 s[2], dp[2];
+    // One 32-key tile at a time: S^T and dP^T for all MQ query tiles, dS^T in place, then
+    // its contribution to dQ^T.
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-      s[nt] = zero16();
-      dp[nt] = zero16();
+    for (int nt = 0; nt < BN / 32; ++nt) {
+      floatx16 s[MQ], dp[MQ];
+#pragma unroll
+      for (int mq = 0; mq < MQ; ++mq) {
+        s[mq] = zero16();
+        dp[mq] = zero16();
+      }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        s[nt] = Mma<T>::run(frag_rows<DP>(k_rows, nt, ks, lane), qf[ks], s[nt]);
-        dp[nt] = Mma<T>::run(frag_rows<DP>(v_rows, nt, ks, lane), dof[ks], dp[nt]);
-      }
-    }
-    const bool plain = !HAS_BIAS && n0 + BN <= a.S && (!CAUSAL || n0 + BN - 1 <= m_wave);
-    if (plain) {
+        const uint4 ka = frag_rows<DP>(k_rows, nt, ks, lane);
+        const uint4 va = frag_rows<DP>(v_rows, nt, ks, lane);
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[nt][r] = fexp2(fmaf(s[nt][r], c, -lse2)) * (dp[nt][r] - dl);
-    } else {
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int n = n0 + nt * 32 + acc_row(r, lane);
-          bool valid = n < a.S;
-          if (CAUSAL) valid = valid && n <= m;
-          float sv = s[nt][r] * c;
-          if (HAS_BIAS) sv = valid ? fmaf(to_float(mrow[n]), kAttnLog2e, sv) : sv;
-          const float p = valid ? fexp2(sv - lse2) : 0.f;
-          s[nt][r] = p * (dp[nt][r] - dl);  // dS^T
+        for (int mq = 0; mq < MQ; ++mq) {
+          s[mq] = Mma<T>::run(ka, qf[mq][ks], s[mq]);
+          dp[mq] = Mma<T>::run(va, dof[mq][ks], dp[mq]);
         }
-    }
+      }
+      const int nb = n0 + nt * 32;
 #pragma unroll
-    for (int t = 0; t < BN / 16; ++t) {
-      const uint4 dsf = frag_from_acc<T>(s[t / 2], t % 2);
+      for (int mq = 0; mq < MQ; ++mq) {
+        const bool plain = !HAS_BIAS && nb + 32 <= a.S && (!CAUSAL || nb + 31 <= m_wave + mq * 32);
+        if (plain) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) acc[dt] = Mma<T>::run(frag_transposed<BN>(k_tr, dt, t, lane), dsf, acc[dt]);
+          for (int r = 0; r < 16; ++r) s[mq][r] = fexp2(fmaf(s[mq][r], c, -lse2[mq])) * (dp[mq][r] - dl[mq]);
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int n = nb + acc_row(r, lane);
+            bool valid = n < a.S;
+            if (CAUSAL) valid = valid && n <= m[mq];
+            float sv = s[mq][r] * c;
+            if (HAS_BIAS) sv = valid ? fmaf(to_float(mrow[mq][n]), kAttnLog2e, sv) : sv;
+            const float p = valid ? fexp2(sv - lse2[mq]) : 0.f;
+            s[mq][r] = p * (dp[mq][r] - dl[mq]);  // dS^T
+          }
+        }
+      }
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        const int t = nt * 2 + hf;
+        uint4 dsf[MQ];
+#pragma unroll
+        for (int mq = 0; mq < MQ; ++mq) dsf[mq] = frag_from_acc<T>(s[mq], hf);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const uint4 kt = frag_transposed<BN>(k_tr, dt, t, lane);
+#pragma unroll
+          for (int mq = 0; mq < MQ; ++mq) acc[mq][dt] = Mma<T>::run(kt, dsf[mq], acc[mq][dt]);
+        }
+      }
     }
   }
 
-  if (m < a.S) {
-    T* out = dq + bshd(a, b, m, h);
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+  for (int mq = 0; mq < MQ; ++mq) {
+    if (m[mq] < a.S) {
+      T* out = dq + bshd(a, b, m[mq], h);
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int d = dt * 32 + g * 8 + half * 4;
-        if (d < a.D) store4<T>(out + d, acc[dt], g, scale);
-      }
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int d = dt * 32 + g * 8 + half * 4;
+          if (d < a.D) store4<T>(out + d, acc[mq][dt], g, scale);
+        }
+    }
   }
 }
 
@@ -630,16 +658,29 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
                      static_cast<const T*>(d_o), static_cast<const T*>(o), delta.as<float>(), rows, a.D);
   MG_LAUNCH_CHECK();
   const int64_t blocks = static_cast<int64_t>(a.B) * a.H * ceil_div(a.S, 128);
+  // dQ: two query tiles per wave when the head dimension leaves registers for it and
+  // there are still enough workgroups to fill the device.
+  const int64_t blocks_q2 = static_cast<int64_t>(a.B) * a.H * ceil_div(a.S, 256);
+  const int q2_knob = env_int("MOGRAD_HIP_ATTN_DQ_TILES", 0);  // 0 = choose, 1 or 2 = force
+  const bool q2 = DP <= 64 && q2_knob != 1 &&
+                  q2_knob == 2;  // measured slower than one tile per wave on MI355X; kept as a tuning aid
 #define MG_LAUNCH(C_, B_)                                                                                              \
   do {                                                                                                                 \
     hipLaunchKernelGGL((attn_dkdv_mfma_kernel<T, DP, C_, B_>), dim3(static_cast<unsigned>(blocks)), dim3(kAttnThreads), \
                        0, stream, static_cast<const T*>(d_o), static_cast<const T*>(q), static_cast<const T*>(k),      \
                        static_cast<const T*>(v), static_cast<const T*>(mask), lse, delta.as<float>(),                  \
                        static_cast<T*>(dk), static_cast<T*>(dv), a, scale);                                            \
-    hipLaunchKernelGGL((attn_dq_mfma_kernel<T, DP, C_, B_>), dim3(static_cast<unsigned>(blocks)), dim3(kAttnThreads), 0, \
-                       stream, static_cast<const T*>(d_o), static_cast<const T*>(q), static_cast<const T*>(k),         \
-                       static_cast<const T*>(v), static_cast<const T*>(mask), lse, delta.as<float>(),                  \
-                       static_cast<T*>(dq), a, scale);                                                                 \
+    if (q2)                                                                                                            \
+      hipLaunchKernelGGL((attn_dq_mfma_kernel<T, DP, (DP <= 64 ? 2 : 1), C_, B_>),                                     \
+                         dim3(static_cast<unsigned>(blocks_q2)), dim3(kAttnThreads), 0, stream,                        \
+                         static_cast<const T*>(d_o), static_cast<const T*>(q), static_cast<const T*>(k),               \
+                         static_cast<const T*>(v), static_cast<const T*>(mask), lse, delta.as<float>(),                \
+                         static_cast<T*>(dq), a, scale);                                                               \
+    else                                                                                                               \
+      hipLaunchKernelGGL((attn_dq_mfma_kernel<T, DP, 1, C_, B_>), dim3(static_cast<unsigned>(blocks)),                 \
+                         dim3(kAttnThreads), 0, stream, static_cast<const T*>(d_o), static_cast<const T*>(q),          \
+                         static_cast<const T*>(k), static_cast<const T*>(v), static_cast<const T*>(mask), lse,         \
+                         delta.as<float>(), static_cast<T*>(dq), a, scale);                                            \
   } while (0)
   if (causal) MG_LAUNCH(true, false);
   else if (has_bias) MG_LAUNCH(false, true);

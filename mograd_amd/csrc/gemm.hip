@@ -42,6 +42,83 @@ static int launch_f32_mfma(const GemmArgs& g, hipStream_t stream) {
   return MG_OK;
 }
 
+static bool mult8(int64_t v) { return (v & 7) == 0; }
+
+// 16-bit MFMA path, optionally split along K when the output has too few tiles to fill
+// the device (dW of a narrow layer: reduction over thousands of rows into a small matrix).
+template <typename T, bool A_KC, bool B_KC>
+static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
+  const int tiles_m = static_cast<int>(ceil_div(g.M, kGemmBM));
+  const int tiles_n = static_cast<int>(ceil_div(g.N, kGemmBN));
+  const int64_t tiles = static_cast<int64_t>(tiles_m) * tiles_n;
+  const int64_t blocks = tiles * g.batch;
+  if (blocks > 0x7fffffffLL) return fail(MG_ERR_INVALID, "matmul: too many output tiles");
+  const int64_t lda = A_KC ? g.sam : g.sak;
+  const int64_t ldb = B_KC ? g.sbn : g.sbk;
+  const T* a = static_cast<const T*>(g.a);
+  const T* b = static_cast<const T*>(g.b);
+  const T* bias = static_cast<const T*>(g.bias);
+  T* c = static_cast<T*>(g.c);
+  const int M = static_cast<int>(g.M), N = static_cast<int>(g.N), K = static_cast<int>(g.K);
+  const int64_t cus = device_info().cu_count;
+  int splits = 1;
+  if (g.batch == 1 && blocks < cus && g.K >= 1024) {
+    splits = static_cast<int>(ceil_div(2 * cus, blocks));
+    const int max_splits = static_cast<int>(g.K / 256);
+    if (splits > max_splits) splits = max_splits;
+    if (splits > 64) splits = 64;
+  }
+  if (splits <= 1) {
+    if (bias)
+      hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, true, false>), dim3(static_cast<unsigned>(blocks)),
+                         dim3(kGemmThreads), 0, stream, a, b, bias, c, nullptr, M, N, K, lda, ldb, g.N, g.bsa, g.bsb,
+                         g.M * g.N, tiles_m, tiles_n, K);
+    else
+      hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, false, false>), dim3(static_cast<unsigned>(blocks)),
+                         dim3(kGemmThreads), 0, stream, a, b, bias, c, nullptr, M, N, K, lda, ldb, g.N, g.bsa, g.bsb,
+                         g.M * g.N, tiles_m, tiles_n, K);
+    MG_LAUNCH_CHECK();
+    return MG_OK;
+  }
+  const int k_per_split = static_cast<int>(ceil_div(ceil_div(g.K, splits), kG16BK) * kG16BK);
+  splits = static_cast<int>(ceil_div(g.K, k_per_split));
+  Scratch partial;
+  const int64_t numel = g.M * g.N;
+  MG_TRY(partial.take(static_cast<int64_t>(splits) * numel * static_cast<int64_t>(sizeof(float))));
+  hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, false, true>),
+                     dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(splits)), dim3(kGemmThreads), 0, stream, a,
+                     b, bias, c, partial.as<float>(), M, N, K, lda, ldb, g.N, g.bsa, g.bsb, numel, tiles_m, tiles_n,
+                     k_per_split);
+  MG_LAUNCH_CHECK();
+  const unsigned rblocks = static_cast<unsigned>(ceil_div(numel, 1024));
+  if (bias)
+    hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, true>), dim3(rblocks), dim3(256), 0, stream, partial.as<float>(),
+                       bias, c, numel, splits, N);
+  else
+    hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, false>), dim3(rblocks), dim3(256), 0, stream, partial.as<float>(),
+                       bias, c, numel, splits, N);
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+template <typename T>
+static int dispatch_16bit(const GemmArgs& g, hipStream_t stream, bool* handled) {
+  *handled = false;
+  if (g.K <= 0) return MG_OK;
+  const bool a_kc = g.sak == 1 && mult8(g.sam) && mult8(g.K);
+  const bool a_mc = g.sam == 1 && mult8(g.sak) && mult8(g.M);
+  const bool b_kc = g.sbk == 1 && mult8(g.sbn) && mult8(g.K);
+  const bool b_nc = g.sbn == 1 && mult8(g.sbk) && mult8(g.N);
+  const bool aligned = aligned16(g.a) && aligned16(g.b) && mult8(g.bsa) && mult8(g.bsb);
+  const bool worth_it = g.M * g.N >= 64 * 64 || g.K >= 512;
+  if (!(aligned && worth_it && (a_kc || a_mc) && (b_kc || b_nc))) return MG_OK;
+  *handled = true;
+  if (a_kc && b_kc) return launch_16bit_mfma<T, true, true>(g, stream);
+  if (a_kc) return launch_16bit_mfma<T, true, false>(g, stream);
+  if (b_kc) return launch_16bit_mfma<T, false, true>(g, stream);
+  return launch_16bit_mfma<T, false, false>(g, stream);
+}
+
 template <typename T>
 static int launch_generic(const GemmArgs& g, hipStream_t stream) {
   const dim3 grid(static_cast<unsigned>(ceil_div(g.N, 64)), static_cast<unsigned>(ceil_div(g.M, 64)),
@@ -86,6 +163,12 @@ int gemm_dispatch(const char* who, const GemmArgs& g, hipStream_t stream) {
       if (b_kc) return launch_f32_mfma<false, true>(g, stream);
       return launch_f32_mfma<false, false>(g, stream);
     }
+  }
+  if (g.dtype != MG_F32) {
+    bool handled = false;
+    const int rc = g.dtype == MG_BF16 ? dispatch_16bit<bf16_t>(g, stream, &handled)
+                                      : dispatch_16bit<f16_t>(g, stream, &handled);
+    if (handled || rc != MG_OK) return rc;
   }
   switch (g.dtype) {
     case MG_F32: return launch_generic<float>(g, stream);

@@ -250,3 +250,213 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
 }
 
 }  // namespace mg
+
+// ------------------------------------------------------------------------------------
+// 16-bit storage (bf16, fp16) on v_mfma_f32_32x32x16: 128x128 output tile, K-chunks of 64,
+// four waves in a 2x2 grid, each a 64x64 tile (2x2 accumulators), fp32 accumulation.
+// Both operand tiles live in LDS as [row][k] with k contiguous, which is what the MFMA
+// wants (8 consecutive k per lane).  A k-contiguous operand is copied as is; an
+// m/n-contiguous operand is transposed on the way in: a thread loads 8 columns of two
+// consecutive k rows and stores 8 dwords, each packing (k, k+1) for one column.
+// SPLIT_K: blockIdx.y selects a K range and fp32 partial tiles go to scratch
+// (splits, M, N); reduce_partials_kernel sums them in a fixed order.
+// ------------------------------------------------------------------------------------
+
+namespace mg {
+
+typedef __bf16 gemm_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 gemm_f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 gemm_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 gemm_f16x2 __attribute__((ext_vector_type(2)));
+typedef float gemm_f32x2 __attribute__((ext_vector_type(2)));
+
+template <typename T>
+struct GemmMma16;
+template <>
+struct GemmMma16<bf16_t> {
+  static __device__ __forceinline__ floatx16 run(uint4 a, uint4 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(gemm_bf16x8, a), __builtin_bit_cast(gemm_bf16x8, b),
+                                                   c, 0, 0, 0);
+  }
+};
+template <>
+struct GemmMma16<f16_t> {
+  static __device__ __forceinline__ floatx16 run(uint4 a, uint4 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(gemm_f16x8, a), __builtin_bit_cast(gemm_f16x8, b), c,
+                                                  0, 0, 0);
+  }
+};
+
+constexpr int kG16BK = 64;
+constexpr int kG16Stride = kG16BK + 8;  // elements per LDS row: 144 bytes, 16-byte aligned, bank-spreading
+
+struct Gemm16Stage {
+  uint4 v[4];
+};
+
+// KC: element (o, k) at base[o * ld + k].  4 chunks of 8 k-values per thread.
+// else: element (o, k) at base[k * ld + o].  2 tasks per thread, each two k rows x 8 o.
+template <typename T, bool KC>
+__device__ __forceinline__ void gemm16_load(const T* __restrict__ base, int64_t ld, int o0, int k0, int O, int k_end,
+                                            Gemm16Stage& st) {
+  const int t = threadIdx.x;
+  if constexpr (KC) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = t + i * kGemmThreads;
+      const int o = min(o0 + idx / 8, O - 1);  // rows past the edge are never stored
+      const int k = k0 + (idx % 8) * 8;
+      st.v[i] = k < k_end ? *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(o) * ld + k)
+                          : make_uint4(0, 0, 0, 0);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int idx = t + i * kGemmThreads;
+      const int kp = idx % 32, oc = idx / 32;
+      const int k = k0 + 2 * kp;
+      const int o = o0 + oc * 8;
+      const bool o_ok = o < O;
+      st.v[2 * i] = (o_ok && k < k_end) ? *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(k) * ld + o)
+                                        : make_uint4(0, 0, 0, 0);
+      st.v[2 * i + 1] = (o_ok && k + 1 < k_end)
+                            ? *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(k + 1) * ld + o)
+                            : make_uint4(0, 0, 0, 0);
+    }
+  }
+}
+
+template <bool KC>
+__device__ __forceinline__ void gemm16_store(uint16_t* __restrict__ lds, const Gemm16Stage& st) {
+  const int t = threadIdx.x;
+  if constexpr (KC) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = t + i * kGemmThreads;
+      *reinterpret_cast<uint4*>(lds + (idx / 8) * kG16Stride + (idx % 8) * 8) = st.v[i];
+    }
+  } else {
+    uint32_t* lds32 = reinterpret_cast<uint32_t*>(lds);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int idx = t + i * kGemmThreads;
+      const int kp = idx % 32, oc = idx / 32;
+      const uint32_t a[4] = {st.v[2 * i].x, st.v[2 * i].y, st.v[2 * i].z, st.v[2 * i].w};
+      const uint32_t b[4] = {st.v[2 * i + 1].x, st.v[2 * i + 1].y, st.v[2 * i + 1].z, st.v[2 * i + 1].w};
+      uint32_t* dst = lds32 + (oc * 8) * (kG16Stride / 2) + kp;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        dst[(2 * e) * (kG16Stride / 2)] = __builtin_amdgcn_perm(b[e], a[e], 0x05040100);
+        dst[(2 * e + 1) * (kG16Stride / 2)] = __builtin_amdgcn_perm(b[e], a[e], 0x07060302);
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ uint4 gemm16_frag(const uint16_t* __restrict__ lds, int o_base, int ks, int lane) {
+  return *reinterpret_cast<const uint4*>(lds + (o_base + lane % 32) * kG16Stride + ks * 16 + (lane / 32) * 8);
+}
+
+template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
+    const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C,
+    float* __restrict__ partial, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb,
+    int64_t bsc, int tiles_m, int tiles_n, int k_per_split) {
+  __shared__ __attribute__((aligned(16))) uint16_t lds_a[kGemmBM * kG16Stride];
+  __shared__ __attribute__((aligned(16))) uint16_t lds_b[kGemmBN * kG16Stride];
+
+  const int tiles = tiles_m * tiles_n;
+  const int batch = SPLIT_K ? 0 : blockIdx.x / tiles;
+  int tm, tn;
+  gemm_tile_of_block(blockIdx.x % tiles, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * kGemmBM;
+  const int n0 = tn * kGemmBN;
+  A += batch * bsa;
+  B += batch * bsb;
+  const int k_begin = SPLIT_K ? blockIdx.y * k_per_split : 0;
+  const int k_end = SPLIT_K ? min(K, k_begin + k_per_split) : K;
+
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int wm = (wave / 2) * 64;
+  const int wn = (wave % 2) * 64;
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  Gemm16Stage sa, sb;
+  gemm16_load<T, A_KC>(A, lda, m0, k_begin, M, k_end, sa);
+  gemm16_load<T, B_KC>(B, ldb, n0, k_begin, N, k_end, sb);
+
+  for (int k0 = k_begin; k0 < k_end; k0 += kG16BK) {
+    gemm16_store<A_KC>(lds_a, sa);
+    gemm16_store<B_KC>(lds_b, sb);
+    __syncthreads();
+    if (k0 + kG16BK < k_end) {
+      gemm16_load<T, A_KC>(A, lda, m0, k0 + kG16BK, M, k_end, sa);
+      gemm16_load<T, B_KC>(B, ldb, n0, k0 + kG16BK, N, k_end, sb);
+    }
+#pragma unroll
+    for (int ks = 0; ks < kG16BK / 16; ++ks) {
+      const uint4 fa0 = gemm16_frag(lds_a, wm, ks, lane);
+      const uint4 fa1 = gemm16_frag(lds_a, wm + 32, ks, lane);
+      const uint4 fb0 = gemm16_frag(lds_b, wn, ks, lane);
+      const uint4 fb1 = gemm16_frag(lds_b, wn + 32, ks, lane);
+      acc[0][0] = GemmMma16<T>::run(fa0, fb0, acc[0][0]);
+      acc[0][1] = GemmMma16<T>::run(fa0, fb1, acc[0][1]);
+      acc[1][0] = GemmMma16<T>::run(fa1, fb0, acc[1][0]);
+      acc[1][1] = GemmMma16<T>::run(fa1, fb1, acc[1][1]);
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+      const int col = n0 + wn + tj * 32 + lane % 32;
+      if (col >= N) continue;
+      const float bv = (HAS_BIAS && !SPLIT_K) ? to_float(bias[col]) : 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + wm + ti * 32 + (r / 4) * 8 + (lane / 32) * 4 + (r % 4);
+        if (row < M) {
+          if constexpr (SPLIT_K)
+            partial[(static_cast<int64_t>(blockIdx.y) * M + row) * N + col] = acc[ti][tj][r];
+          else
+            C[batch * bsc + static_cast<int64_t>(row) * ldc + col] = from_float<T>(acc[ti][tj][r] + bv);
+        }
+      }
+    }
+}
+
+// out[i] = sum_s partial[s][i] (+ bias[i % N]), converted to T.
+template <typename T, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ partial,
+                                                                 const T* __restrict__ bias, T* __restrict__ out,
+                                                                 int64_t numel, int splits, int N) {
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  if (i >= numel) return;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool full = i + 3 < numel;
+  for (int s = 0; s < splits; ++s) {
+    const float* p = partial + static_cast<int64_t>(s) * numel + i;
+    if (full) {
+      const float4 v = *reinterpret_cast<const float4*>(p);
+      acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
+    } else {
+      for (int e = 0; e < 4 && i + e < numel; ++e) acc[e] += p[e];
+    }
+  }
+  for (int e = 0; e < 4 && i + e < numel; ++e) {
+    const float bv = HAS_BIAS ? to_float(bias[(i + e) % N]) : 0.f;
+    out[i + e] = from_float<T>(acc[e] + bv);
+  }
+}
+
+}  // namespace mg

@@ -172,3 +172,41 @@ def test_errors(device):
         device.lib.mg_matmul(p, p, p, 1, 2, 2, 2, 2, 1, 2, 1, 4, 4, R.int64, device.stream)
     with pytest.raises(MogradError, match="null bias"):
         device.lib.mg_matmul_bias_bt(p, p, None, p, 1, 2, 2, 2, 2, 1, 2, 1, 4, 4, F32, device.stream)
+
+
+# ---- 16-bit storage on the matrix cores (shapes that take the MFMA kernels) ------------
+
+HALF_MFMA_SHAPES = [(256, 384, 512), (384, 128, 1536), (200, 136, 264), (128, 64, 4096), (4096, 128, 128),
+                    (1024, 384, 384), (72, 1536, 384)]
+
+
+@pytest.mark.parametrize("dtype,rtol", [(F16, 2e-3), (BF16, 1.6e-2)])
+@pytest.mark.parametrize("M,N,K", HALF_MFMA_SHAPES)
+def test_half_precision_mfma_paths(device, dtype, rtol, M, N, K):
+    # forward (k,k), dX (k,n), dW (m,n) operand layouts; dW of the tall shapes is split
+    # along K.  Error bound: the storage type's rounding of the result, relative to the
+    # largest entry (inputs are rounded once; the oracle sees the rounded values).
+    x = round_to_dtype(normal(47, 0, (M, K)), dtype)
+    w = round_to_dtype(normal(47, 1, (N, K), std=0.05), dtype)
+    b = round_to_dtype(normal(47, 2, (N,), std=0.1), dtype)
+    dy = round_to_dtype(normal(47, 3, (M, N), std=0.5), dtype)
+    y, dx, dw, db = _linear_all(device, x, w, b, dy, dtype)
+    for got, want, name in ((y, O.matmul_bias_bt(x, w, b), "y"), (dx, O.linear_grad_x(dy, w), "dx"),
+                            (dw, O.linear_grad_w(dy, x), "dw"), (db, O.linear_grad_b(dy), "db")):
+        assert_close(got, want, rtol, rtol * np.abs(want).max(), name)
+
+
+def test_bf16_linear_bwd_entry_gpt_shapes(device):
+    # (tokens, d_model) x (d_ff, d_model): the GPT block's MLP up-projection, scaled down
+    M, N, K = 2048, 1536, 384
+    x = round_to_dtype(normal(48, 0, (M, K)), BF16)
+    w = round_to_dtype(normal(48, 1, (N, K), std=0.05), BF16)
+    dy = round_to_dtype(normal(48, 2, (M, N), std=0.5), BF16)
+    bx, bw, bdy = (AnyBuffer.from_numpy(device, a, BF16) for a in (x, w, dy))
+    dx, dw, db = (AnyBuffer.create(BF16, device, n) for n in (M * K, N * K, N))
+    device.lib.mg_linear_bwd(bdy.data_ptr(), bx.data_ptr(), bw.data_ptr(), dx.data_ptr(), dw.data_ptr(),
+                             db.data_ptr(), M, N, K, BF16, device.stream)
+    for got, want, name in ((dx.to_numpy((M, K)), O.linear_grad_x(dy, w), "dx"),
+                            (dw.to_numpy((N, K)), O.linear_grad_w(dy, x), "dw"),
+                            (db.to_numpy(), O.linear_grad_b(dy), "db")):
+        assert_close(got, want, 1.6e-2, 1.6e-2 * np.abs(want).max(), name)
