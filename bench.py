@@ -140,12 +140,245 @@ def cpu_baseline(sample_ce_rows: int = 256):
     }
 
 
+MFMA_F32_PEAK_TFLOPS = 157.3
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def _orc():
+    import subprocess
+
+    so = ROOT / "oracle" / "liboracle_c.so"
+    if not so.exists():
+        subprocess.run(["make", "-C", str(ROOT / "oracle")], check=True, capture_output=True)
+    orc = C.CDLL(str(so))
+    orc.orc_num_threads.restype = C.c_int
+    return orc
+
+
+def _time_steps(dev, step, warmup, steps):
+    for i in range(warmup):
+        step(i)
+    dev.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(warmup + i)
+    dev.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def _kernel_table(dev, entries, iters):
+    """entries: (name, fn, work, unit) with unit 'B' (bytes, HBM bound) or 'F' (flops, MFMA
+    bound, against `peak` TFLOP/s given as a 5th element)."""
+    timer = EventTimer(dev, iters)
+    out = []
+    for name, fn, work, unit, peak in entries:
+        fn(0)
+        dev.synchronize()
+        ts = timer.run(fn, iters)
+        mean_ms = float(np.mean(ts))
+        row = {"name": name, "mean_ms": round(mean_ms, 5), "median_ms": round(float(np.median(ts)), 5)}
+        if unit == "B":
+            gbs = work / (mean_ms * 1e-3) / 1e9
+            row.update({"algorithmic_bytes": work, "achieved_GBps": round(gbs, 1),
+                        "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)})
+        else:
+            tf = work / (mean_ms * 1e-3) / 1e12
+            row.update({"algorithmic_flops": work, "achieved_TFLOPs": round(tf, 1), "peak_TFLOPs": peak,
+                        "frac_of_mfma_peak": round(tf / peak, 4)})
+        out.append(row)
+    timer.close()
+    return out
+
+
+def bench_mlp(args, dev) -> int:
+    """README MLP, fp32: x (2048,4096) -> Linear 4096->4096 +ReLU -> LayerNorm(4096) -> Linear 4096->4096 +ReLU
+    -> Linear 4096->10, cross-entropy on labels in [0,10).  Forward and backward through the C ABI."""
+    from mograd_amd import F32, I32, AnyBuffer
+
+    lib, st = dev.lib, dev.stream
+    M, D, NC = 2048, 4096, 10
+    bound = float(np.sqrt(6.0 / D))
+    up = lambda a: AnyBuffer.from_numpy(dev, a)  # noqa: E731
+    new = lambda n: AnyBuffer.create(F32, dev, n)  # noqa: E731
+    x = up(_rng(3, 0).standard_normal((M, D), dtype=np.float32))
+    w1, w2 = (up(_rng(3, i).uniform(-bound, bound, (D, D)).astype(np.float32)) for i in (1, 3))
+    b1, b2 = (up(_rng(3, i).uniform(-bound, bound, D).astype(np.float32)) for i in (2, 4))
+    w3 = up(_rng(3, 5).uniform(-bound, bound, (NC, D)).astype(np.float32))
+    b3 = up(_rng(3, 6).uniform(-bound, bound, NC).astype(np.float32))
+    gamma, beta = up(np.ones(D, np.float32)), up(np.zeros(D, np.float32))
+    ids = AnyBuffer.from_numpy(dev, _rng(3, 7).integers(0, NC, M).astype(np.int32), I32)
+    h1p, h1, ln, h2p, h2, logits = new(M * D), new(M * D), new(M * D), new(M * D), new(M * D), new(M * NC)
+    loss, dlogits = new(1), new(M * NC)
+    dh2, dh2p, dln, dh1, dh1p = new(M * D), new(M * D), new(M * D), new(M * D), new(M * D)
+    dw1, dw2, dw3, db1, db2, db3, dg, dbt = new(D * D), new(D * D), new(NC * D), new(D), new(D), new(NC), new(D), new(D)
+    P = lambda b: b.data_ptr()  # noqa: E731
+
+    def linear(a, w, b, y, n_out, k):
+        lib.mg_matmul_bias_bt(P(a), P(w), P(b), P(y), 1, M, n_out, k, k, 1, k, 1, M * k, n_out * k, F32, st)
+
+    def fwd(i):
+        linear(x, w1, b1, h1p, D, D)
+        lib.mg_relu_grad(P(h1p), P(h1p), P(h1), M * D, F32, st)  # relu(v) == relu_grad(v, v)
+        lib.mg_layer_norm_fwd(P(h1), P(gamma), P(beta), P(ln), M, D, 1e-5, F32, st)
+        linear(ln, w2, b2, h2p, D, D)
+        lib.mg_relu_grad(P(h2p), P(h2p), P(h2), M * D, F32, st)
+        linear(h2, w3, b3, logits, NC, D)
+
+    def bwd(i):
+        lib.mg_cross_entropy_fused_ids(P(logits), P(ids), None, P(loss), P(dlogits), M, NC, F32, I32, st)
+        lib.mg_linear_bwd(P(dlogits), P(h2), P(w3), P(dh2), P(dw3), P(db3), M, NC, D, F32, st)
+        lib.mg_relu_grad(P(h2), P(dh2), P(dh2p), M * D, F32, st)
+        lib.mg_linear_bwd(P(dh2p), P(ln), P(w2), P(dln), P(dw2), P(db2), M, D, D, F32, st)
+        lib.mg_layer_norm_bwd(P(dln), P(h1), P(gamma), P(dh1), P(dg), P(dbt), M, D, 1e-5, F32, st)
+        lib.mg_relu_grad(P(h1), P(dh1), P(dh1p), M * D, F32, st)
+        lib.mg_linear_bwd(P(dh1p), P(x), P(w1), None, P(dw1), P(db1), M, D, D, F32, st)
+
+    def step(i):
+        fwd(i)
+        bwd(i)
+
+    ms = _time_steps(dev, step, args.warmup, args.steps)
+    fl = 2.0 * M * D * D
+    entries = [
+        ("dX = dY W (mg_linear_bwd dx only, 2048x4096x4096)",
+         lambda i: lib.mg_linear_bwd(P(dh2p), P(ln), P(w2), P(dln), None, None, M, D, D, F32, st), fl, "F", MFMA_F32_PEAK_TFLOPS),
+        ("dW = dY^T X (mg_linear_bwd dw only)",
+         lambda i: lib.mg_linear_bwd(P(dh2p), P(ln), P(w2), None, P(dw2), None, M, D, D, F32, st), fl, "F", MFMA_F32_PEAK_TFLOPS),
+        ("db = sum rows dY (mg_sum_axis)",
+         lambda i: lib.mg_sum_axis(P(dh2p), P(db2), 1, M, D, F32, st), M * D * 4 + D * 4, "B", None),
+        ("Y = X W^T + b (mg_matmul_bias_bt)", lambda i: linear(ln, w2, b2, h2p, D, D), fl, "F", MFMA_F32_PEAK_TFLOPS),
+    ]
+    kernels = _kernel_table(dev, entries, max(10, min(args.steps, 50)))
+    dom = min(kernels[:2], key=lambda r: r["frac_of_mfma_peak"])
+    result = {
+        "metric": "fwd+bwd step ms; per-bwd-kernel HBM GB/s or MFMA % of MI355X peak", "value": round(ms, 4),
+        "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "README MLP fwd+bwd fp32: x (2048,4096) -> Linear 4096 +ReLU -> LayerNorm -> Linear 4096 "
+                               "+ReLU -> Linear 10, cross-entropy, labels in [0,10)"},
+        "roofline": {"bound": "mfma", "kernel": "gemm_f32_mfma_kernel, " + dom["name"], "achieved": dom["achieved_TFLOPs"],
+                     "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac_of_mfma_peak"], "traffic": None},
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        # Linear gradients of one 4096x4096 layer on a slab of 128 of the 2048 rows (dX scales
+        # with rows; dW's reduction length scales with rows), scaled x16; three layers' worth
+        # is dominated by the two square ones.
+        orc = _orc()
+        cores = int(orc.orc_num_threads())
+        rows = 128
+        p = lambda a: a.ctypes.data_as(C.c_void_p)  # noqa: E731
+        L = C.c_int64
+        dy = _rng(3, 20).standard_normal((rows, D), dtype=np.float32)
+        xs = _rng(3, 21).standard_normal((rows, D), dtype=np.float32)
+        w = _rng(3, 22).uniform(-bound, bound, (D, D)).astype(np.float32)
+        dxh, dwh, dbh = np.empty((rows, D), np.float32), np.empty((D, D), np.float32), np.empty(D, np.float32)
+        t0 = time.perf_counter()
+        orc.orc_linear_grad_x_f32(p(dy), p(w), p(dxh), L(rows), L(D), L(D))
+        orc.orc_linear_grad_w_f32(p(dy), p(xs), p(dwh), L(rows), L(D), L(D))
+        orc.orc_linear_grad_b_f32(p(dy), p(dbh), L(rows), L(D))
+        slab_ms = (time.perf_counter() - t0) * 1e3
+        result["cpu_baseline"] = {
+            "value": round(slab_ms * (M / rows), 1), "unit": "ms", "cores": cores, "kind": "port",
+            "sample": f"dX + dW + db of one 4096x4096 Linear on {rows} of {M} rows ({slab_ms:.1f} ms) scaled x{M // rows}; "
+                      f"one layer, not the whole step; OpenMP on {cores} threads"}
+    print(json.dumps(result))
+    return 0
+
+
+def bench_attention(args, dev) -> int:
+    """Flash attention fwd+bwd, bf16 with fp32 accumulation: causal B8 H12 S1024 D64 (the step), and
+    non-causal B2 H12 S4096 D64 in the kernel table."""
+    from mograd_amd import BF16, F32, AnyBuffer
+
+    lib, st = dev.lib, dev.stream
+
+    def make(B, H, S, D, cfg):
+        n = B * S * H * D
+        q, k, v, do = (AnyBuffer.from_numpy(dev, _rng(4, cfg * 10 + i).standard_normal(n, dtype=np.float32), BF16)
+                       for i in range(4))
+        o, dq, dk, dv = (AnyBuffer.create(BF16, dev, n) for _ in range(4))
+        lse = AnyBuffer.create(F32, dev, B * H * S)
+        return q, k, v, do, o, dq, dk, dv, lse
+
+    def runner(B, H, S, D, causal, bufs):
+        q, k, v, do, o, dq, dk, dv, lse = bufs
+        sc = 1.0 / float(np.sqrt(D))
+        P = lambda b: b.data_ptr()  # noqa: E731
+        f = lambda i: lib.mg_flash_attn_fwd(P(q), P(k), P(v), None, P(o), P(lse), B, S, H, D, sc, causal, 0, BF16, st)  # noqa: E731
+        b = lambda i: lib.mg_flash_attn_bwd(P(do), P(o), P(q), P(k), P(v), None, P(lse), P(dq), P(dk), P(dv), B, S, H, D,  # noqa: E731
+                                            sc, causal, 0, BF16, st)
+        return f, b
+
+    c1 = (8, 12, 1024, 64)
+    c2 = (2, 12, 4096, 64)
+    f1, b1 = runner(*c1, 1, make(*c1, 1))
+    f2, b2 = runner(*c2, 0, make(*c2, 2))
+
+    def step(i):
+        f1(i)
+        b1(i)
+
+    ms = _time_steps(dev, step, args.warmup, args.steps)
+    B, H, S, D = c1
+    fl1 = B * H * S * S * D
+    B2, H2, S2, D2 = c2
+    fl2 = B2 * H2 * S2 * S2 * D2
+    entries = [
+        ("flash_attn_bwd bf16 causal B8 H12 S1024 D64 (5 B H S^2 D)", b1, 5.0 * fl1, "F", MFMA_BF16_PEAK_TFLOPS),
+        ("flash_attn_fwd bf16 causal B8 H12 S1024 D64 (2 B H S^2 D)", f1, 2.0 * fl1, "F", MFMA_BF16_PEAK_TFLOPS),
+        ("flash_attn_bwd bf16 B2 H12 S4096 D64 (10 B H S^2 D)", b2, 10.0 * fl2, "F", MFMA_BF16_PEAK_TFLOPS),
+        ("flash_attn_fwd bf16 B2 H12 S4096 D64 (4 B H S^2 D)", f2, 4.0 * fl2, "F", MFMA_BF16_PEAK_TFLOPS),
+    ]
+    kernels = _kernel_table(dev, entries, max(10, min(args.steps, 50)))
+    dom = kernels[0]
+    result = {
+        "metric": "fwd+bwd step ms; per-bwd-kernel HBM GB/s or MFMA % of MI355X peak", "value": round(ms, 4),
+        "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "causal flash-attention fwd+bwd bf16 (fp32 accumulate) B8 H12 S1024 D64, scale 1/8; "
+                               "kernel table also has non-causal B2 H12 S4096 D64"},
+        "roofline": {"bound": "mfma", "kernel": "attn_dkdv_mfma_kernel + attn_dq_mfma_kernel + attn_delta_kernel "
+                                                "(mg_flash_attn_bwd, causal S1024)",
+                     "achieved": dom["achieved_TFLOPs"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": dom["frac_of_mfma_peak"], "traffic": None},
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        # fp32 naive O(S^2) attention (the reference's oracle structure) on 4 of the 96 (b,h)
+        # pairs of the causal configuration, scaled x24.
+        orc = _orc()
+        cores = int(orc.orc_num_threads())
+        p = lambda a: a.ctypes.data_as(C.c_void_p)  # noqa: E731
+        L = C.c_int64
+        Bs, Hs = 1, 4
+        n = Bs * S * Hs * D
+        q, k, v, do = (_rng(4, 50 + i).standard_normal(n, dtype=np.float32) for i in range(4))
+        o, dq, dk, dv = (np.empty(n, np.float32) for _ in range(4))
+        lse = np.empty(Bs * Hs * S, np.float32)
+        t0 = time.perf_counter()
+        orc.orc_sdpa_fwd_f32(p(q), p(k), p(v), None, 0, 1, p(o), p(lse), L(Bs), L(S), L(Hs), L(D), C.c_float(0.125), L(Bs * Hs))
+        orc.orc_sdpa_bwd_f32(p(q), p(k), p(v), p(do), None, 0, 1, p(dq), p(dk), p(dv), L(Bs), L(S), L(Hs), L(D),
+                             C.c_float(0.125), L(Bs * Hs))
+        slab_ms = (time.perf_counter() - t0) * 1e3
+        scale_up = (B * H) // (Bs * Hs)
+        result["cpu_baseline"] = {
+            "value": round(slab_ms * scale_up, 1), "unit": "ms", "cores": cores, "kind": "port",
+            "sample": f"naive fp32 attention fwd+bwd on {Bs * Hs} of {B * H} (batch, head) pairs of the causal "
+                      f"configuration ({slab_ms:.1f} ms) scaled x{scale_up}; OpenMP on {cores} threads"}
+    print(json.dumps(result))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
+    ap.add_argument("--workload", choices=["ln_ce", "mlp", "attention"], default="ln_ce",
+                    help="ln_ce (default): the configuration the metric is quoted on; mlp: README MLP fwd+bwd fp32 "
+                         "(matmul_bias_bt, dX, dW, db); attention: bf16 flash attention fwd+bwd")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path runs on one GPU; --gpus N with N > 1 is not supported "
@@ -157,6 +390,10 @@ def main() -> int:
     dev = Device(0)
     lib = dev.lib
     st = dev.stream
+    if args.workload == "mlp":
+        return bench_mlp(args, dev)
+    if args.workload == "attention":
+        return bench_attention(args, dev)
 
     # ---- inputs, resident in HBM -------------------------------------------------------
     # LayerNorm: four rotating sets (4 x 100 MB) so that no set is still in the 256 MB
