@@ -102,9 +102,11 @@ static int colsum_typed(const T* a, T* dst, int64_t outer, int64_t reduce, int64
   const int vec = wide ? WIDE : 1;
   const int64_t col_blocks = ceil_div(inner, 256 * vec);
   if (outer > 65535) return fail(MG_ERR_UNSUPPORTED, "sum_axis: outer=%lld exceeds 65535", static_cast<long long>(outer));
-  // Enough slabs to fill the device, each at least 8 rows.
-  int64_t chunks = ceil_div(static_cast<int64_t>(device_info().cu_count) * 4, col_blocks * outer);
-  const int64_t max_chunks = ceil_div(reduce, 8);
+  // Enough slabs to fill the device, each at least 32 rows (fewer, longer slabs keep the
+  // fp32 partial sums a small fraction of the traffic).
+  int64_t chunks = ceil_div(static_cast<int64_t>(device_info().cu_count) * env_int("MOGRAD_HIP_COLSUM_WG_PER_CU", 4),
+                            col_blocks * outer);
+  const int64_t max_chunks = ceil_div(reduce, env_int("MOGRAD_HIP_COLSUM_MIN_ROWS", 32));
   if (chunks > max_chunks) chunks = max_chunks;
   if (chunks < 1) chunks = 1;
   if (chunks > 65535) chunks = 65535;
