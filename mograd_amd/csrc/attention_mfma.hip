@@ -550,8 +550,9 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
     // crosses the diagonal of this wave's keys.
     const bool plain = !HAS_BIAS && n_wave + 31 < a.S && (!CAUSAL || n_wave + 31 <= m0);
     // One 32-query tile at a time: S and dP (column = this lane's key, rows = queries),
-    // then P and dS in place, then their contributions to dV and dK.  Only one tile's
-    // scores are live, and the next tile's products can run under this tile's arithmetic.
+    // then P and dS in place, then their contributions to dV and dK.  LDS fragments are
+    // fetched a phase ahead (the transposed ones, and the next tile's row fragments, while
+    // the exponentials run) so that no MFMA waits on an LDS read it has just issued.
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       floatx16 s = zero16(), dp = zero16();
@@ -560,6 +561,17 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
         s = Mma<T>::run(frag_rows<DP>(q_rows, mt, ks, lane), kf[ks], s);
         dp = Mma<T>::run(frag_rows<DP>(do_rows, mt, ks, lane), vf[ks], dp);
       }
+      // The transposed fragments of the second phase are fetched now, so that their LDS
+      // latency runs under the exponentials instead of in front of each MFMA.
+      uint4 tq[2][DT], tdo[2][DT];
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          tdo[hf][dt] = frag_transposed<BQ>(do_tr, dt, mt * 2 + hf, lane);
+          tq[hf][dt] = frag_transposed<BQ>(q_tr, dt, mt * 2 + hf, lane);
+        }
+      __builtin_amdgcn_sched_barrier(0);
       if (plain) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
@@ -591,13 +603,12 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
       }
 #pragma unroll
       for (int hf = 0; hf < 2; ++hf) {
-        const int t = mt * 2 + hf;
         const uint4 pf = frag_from_acc<T>(s, hf);
         const uint4 dsf = frag_from_acc<T>(dp, hf);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-          acc_v[dt] = Mma<T>::run(frag_transposed<BQ>(do_tr, dt, t, lane), pf, acc_v[dt]);
-          acc_k[dt] = Mma<T>::run(frag_transposed<BQ>(q_tr, dt, t, lane), dsf, acc_k[dt]);
+          acc_v[dt] = Mma<T>::run(tdo[hf][dt], pf, acc_v[dt]);
+          acc_k[dt] = Mma<T>::run(tq[hf][dt], dsf, acc_k[dt]);
         }
       }
     }
