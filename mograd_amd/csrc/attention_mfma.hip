@@ -276,7 +276,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
           bool valid = n < a.S;
           if (CAUSAL) valid = valid && n <= m;
           float sv = s[nt][r] * c;
-          if (HAS_BIAS) sv = valid ? fmaf(to_float(mrow[n]), kAttnLog2e, sv) : sv;
+          if (HAS_BIAS) sv = fmaf(to_float(mrow[min(n, a.S - 1)]), kAttnLog2e, sv);
           sv = valid ? sv : -INFINITY;
           s[nt][r] = sv;
           mx = fmaxf(mx, sv);
@@ -428,8 +428,9 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
             bool valid = n < a.S;
             if (CAUSAL) valid = valid && n <= m[mq];
             float sv = s[mq][r] * c;
-            if (HAS_BIAS) sv = valid ? fmaf(to_float(mrow[mq][n]), kAttnLog2e, sv) : sv;
-            const float p = valid ? fexp2(sv - lse2[mq]) : 0.f;
+            if (HAS_BIAS) sv = fmaf(to_float(mrow[mq][min(n, a.S - 1)]), kAttnLog2e, sv);
+            float p = fexp2(sv - lse2[mq]);
+            p = valid ? p : 0.f;
             s[mq][r] = p * (dp[mq][r] - dl[mq]);  // dS^T
           }
         }
@@ -588,17 +589,31 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
           }
         }
       } else {
+        // Same arithmetic on every element, then a select: no per-element branches.
+        const bool col_ok = n < a.S;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int ml = mt * 32 + acc_row(r, lane);
-          const int mm = m0 + ml;
-          bool valid = n < a.S;
-          if (CAUSAL) valid = valid && n <= mm;
-          float sv = s[r] * c;
-          if (HAS_BIAS) sv = (valid && mm < a.S) ? fmaf(to_float(mask[(bh * a.S + mm) * a.S + n]), kAttnLog2e, sv) : sv;
-          const float p = valid ? fexp2(sv - lse_s[ml]) : 0.f;
-          s[r] = p;
-          dp[r] = p * (dp[r] - delta_s[ml]);
+        for (int g = 0; g < 4; ++g) {
+          const float4 l4 = *reinterpret_cast<const float4*>(&lse_s[mt * 32 + g * 8 + half * 4]);
+          const float4 d4 = *reinterpret_cast<const float4*>(&delta_s[mt * 32 + g * 8 + half * 4]);
+          const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
+          const float dv4[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int r = g * 4 + j;
+            const int mm = m0 + mt * 32 + g * 8 + half * 4 + j;
+            bool valid = col_ok;
+            if (CAUSAL) valid = valid && n <= mm;
+            float sv = s[r] * c;
+            if (HAS_BIAS) {
+              // clamped address: always in bounds, the value is discarded when invalid
+              const int64_t mi = (bh * a.S + min(mm, a.S - 1)) * a.S + min(n, a.S - 1);
+              sv = fmaf(to_float(mask[mi]), kAttnLog2e, sv);
+            }
+            float p = fexp2(sv - lv[j]);  // rows past the end carry lse = +inf: p = 0
+            p = valid ? p : 0.f;
+            s[r] = p;
+            dp[r] = p * (dp[r] - dv4[j]);
+          }
         }
       }
 #pragma unroll
