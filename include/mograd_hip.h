@@ -263,6 +263,49 @@ int mg_relu_grad(const void* out, const void* upstream, void* dst, int64_t n, in
                  mg_stream stream);
 
 /* ------------------------------------------------------------------------------------ */
+/* The other per-step ops of a transformer block: residual adds, relu, casts, making a   */
+/* transposed view contiguous, embedding lookup and its gradient.  Float dtypes only;    */
+/* contiguous operands unless strides are passed.                                        */
+/* ------------------------------------------------------------------------------------ */
+
+/* dst = a + b over n contiguous elements (dst may alias a or b).
+ * Replaces mograd_add, kernels/__init__.mojo:462-471. */
+int mg_add(const void* a, const void* b, void* dst, int64_t n, int dtype, mg_stream stream);
+
+/* dst = max(a, 0) over n contiguous elements (dst may alias a).
+ * Replaces mograd_relu for a contiguous layout, kernels/__init__.mojo:274-286. */
+int mg_relu(const void* a, void* dst, int64_t n, int dtype, mg_stream stream);
+
+/* dst[i] = (out_dtype) a[i], one rounding (nearest even), n contiguous elements.
+ * Replaces mograd_cast for a contiguous layout and float types,
+ * kernels/__init__.mojo:304-335 (kernels/elementwise.mojo:75-90). */
+int mg_cast(const void* a, void* dst, int64_t n, int in_dtype, int out_dtype, mg_stream stream);
+
+/* dst (row-major, contiguous) = the view of `a` with the given shape and element strides
+ * (host arrays of `rank` <= 8 entries, strides >= 0, base offset already applied to `a`).
+ * Any dtype of the enum.  Replaces mograd_contiguous, kernels/__init__.mojo:338-350. */
+int mg_contiguous(const void* a, void* dst, int rank, const int64_t* shape, const int64_t* strides,
+                  int dtype, mg_stream stream);
+
+/* dst(i, :) = src(indices[i], :), i < n_idx; src is (num_rows, row_size) with the given
+ * element strides, dst and indices contiguous, idx_dtype MG_I32 or MG_I64 (the reference
+ * takes int64 only).  An index outside [0, num_rows) yields a row of zeros (the reference
+ * reads out of bounds).  Replaces mograd_gather, kernels/__init__.mojo:132-163
+ * (kernels/gather_scatter.mojo:14-38). */
+int mg_gather(const void* src, const void* indices, void* dst, int64_t n_idx, int64_t num_rows,
+              int64_t row_size, int64_t src_row_stride, int64_t src_col_stride, int idx_dtype,
+              int dtype, mg_stream stream);
+
+/* dst(r, :) = sum over i with indices[i] == r of values(i, :); dst is (num_rows, row_size)
+ * and is fully written (rows nobody indexes become zero), values is (n_idx, row_size)
+ * contiguous.  Rows are added in index order with fp32 accumulation and no atomics, so
+ * the result is deterministic (the reference uses atomic adds into a zero-filled
+ * buffer).  Indices outside [0, num_rows) are ignored.  Replaces mograd_scatter_add,
+ * kernels/__init__.mojo:166-211 (kernels/gather_scatter.mojo:46-71). */
+int mg_scatter_add(const void* indices, const void* values, void* dst, int64_t n_idx,
+                   int64_t num_rows, int64_t row_size, int idx_dtype, int dtype, mg_stream stream);
+
+/* ------------------------------------------------------------------------------------ */
 /* Flash attention.  Q, K, V, dQ, dK, dV are BSHD; O and dO are BHSD; mask is            */
 /* (B,H,S,S) additive bias in natural-log units, of `dtype`; LSE is (B,H,S) fp32 natural  */
 /* log (kernels/attention/generic.mojo:29-35).  dtype in {F32, F16, BF16}.                */

@@ -93,6 +93,12 @@ PROTOTYPES = {
     "mg_linear_bwd": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _l, _i, _p], True),
     "mg_sum_axis": (_i, [_p, _p, _l, _l, _l, _i, _p], True),
     "mg_relu_grad": (_i, [_p, _p, _p, _l, _i, _p], True),
+    "mg_add": (_i, [_p, _p, _p, _l, _i, _p], True),
+    "mg_relu": (_i, [_p, _p, _l, _i, _p], True),
+    "mg_cast": (_i, [_p, _p, _l, _i, _i, _p], True),
+    "mg_contiguous": (_i, [_p, _p, _i, _pl, _pl, _i, _p], True),
+    "mg_gather": (_i, [_p, _p, _p, _l, _l, _l, _l, _l, _i, _i, _p], True),
+    "mg_scatter_add": (_i, [_p, _p, _p, _l, _l, _l, _i, _i, _p], True),
     "mg_flash_attn_fwd": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _l, _l, _f, _i, _i, _i, _p], True),
     "mg_flash_attn_bwd": (_i, [_p] * 10 + [_l, _l, _l, _l, _f, _i, _i, _i, _p], True),
 }

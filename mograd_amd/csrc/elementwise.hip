@@ -1,0 +1,282 @@
+// Elementwise maps of the training step around the backward kernels: residual and gradient
+// adds, relu, dtype casts, and the copy that makes a strided view contiguous.  All are
+// HBM-bound streaming kernels with 16-byte accesses.
+#include "mg_device.h"
+#include "mg_internal.h"
+
+namespace mg {
+
+template <typename T>
+__global__ __launch_bounds__(256) void add_kernel(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ dst,
+                                                  int64_t n) {
+  constexpr int VEC = WideVec<T>::value;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256 * VEC;
+  for (int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * VEC; i < n; i += stride) {
+    if (i + VEC <= n) {
+      float x[VEC], y[VEC];
+      VecIO<T, VEC>::load(a + i, x);
+      VecIO<T, VEC>::load(b + i, y);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) x[e] += y[e];
+      VecIO<T, VEC>::store(dst + i, x);
+    } else {
+      for (int64_t j = i; j < n; ++j) dst[j] = from_float<T>(to_float(a[j]) + to_float(b[j]));
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void relu_kernel(const T* __restrict__ a, T* __restrict__ dst, int64_t n) {
+  constexpr int VEC = WideVec<T>::value;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256 * VEC;
+  for (int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * VEC; i < n; i += stride) {
+    if (i + VEC <= n) {
+      float x[VEC];
+      VecIO<T, VEC>::load(a + i, x);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) x[e] = x[e] > 0.f ? x[e] : 0.f;
+      VecIO<T, VEC>::store(dst + i, x);
+    } else {
+      for (int64_t j = i; j < n; ++j) dst[j] = to_float(a[j]) > 0.f ? a[j] : from_float<T>(0.f);
+    }
+  }
+}
+
+// Eight elements per thread: two 16-byte accesses on the fp32 side, one on the 16-bit side.
+template <typename S, typename D>
+__global__ __launch_bounds__(256) void cast_kernel(const S* __restrict__ a, D* __restrict__ dst, int64_t n) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256 * 8;
+  for (int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 8; i < n; i += stride) {
+    if (i + 8 <= n) {
+      float v[8];
+      if constexpr (sizeof(S) == 4) {
+        float lo[4], hi[4];
+        VecIO<S, 4>::load(a + i, lo);
+        VecIO<S, 4>::load(a + i + 4, hi);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = lo[e];
+          v[4 + e] = hi[e];
+        }
+      } else {
+        VecIO<S, 8>::load(a + i, v);
+      }
+      if constexpr (sizeof(D) == 4) {
+        const float lo[4] = {v[0], v[1], v[2], v[3]};
+        const float hi[4] = {v[4], v[5], v[6], v[7]};
+        VecIO<D, 4>::store(dst + i, lo);
+        VecIO<D, 4>::store(dst + i + 4, hi);
+      } else {
+        VecIO<D, 8>::store(dst + i, v);
+      }
+    } else {
+      for (int64_t j = i; j < n; ++j) dst[j] = from_float<D>(to_float(a[j]));
+    }
+  }
+}
+
+// dst[flat] = src[offset(flat)] over chunks of sizeof(V) bytes.  The view's shape and
+// strides are in chunk units; flat runs over the row-major order of the shape.  Index is
+// uint32_t when every extent and offset fits, else int64_t.
+struct CopyView {
+  int rank;
+  int64_t shape[kMaxRank];
+  int64_t stride[kMaxRank];
+};
+
+template <typename V, typename Index>
+__global__ __launch_bounds__(256) void contiguous_kernel(const V* __restrict__ src, V* __restrict__ dst, CopyView v,
+                                                         int64_t n) {
+  const int64_t step = static_cast<int64_t>(gridDim.x) * 256;
+  for (int64_t flat = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; flat < n; flat += step) {
+    Index rem = static_cast<Index>(flat);
+    Index off = 0;
+    for (int d = v.rank - 1; d > 0; --d) {
+      const Index extent = static_cast<Index>(v.shape[d]);
+      const Index q = rem / extent;
+      off += (rem - q * extent) * static_cast<Index>(v.stride[d]);
+      rem = q;
+    }
+    off += rem * static_cast<Index>(v.stride[0]);
+    dst[flat] = src[off];
+  }
+}
+
+static unsigned stream_blocks(int64_t n, int per_thread) {
+  int64_t blocks = ceil_div(n, static_cast<int64_t>(256) * per_thread);
+  const int64_t cap = static_cast<int64_t>(device_info().cu_count) * 16;
+  if (blocks > cap) blocks = cap;
+  return static_cast<unsigned>(blocks < 1 ? 1 : blocks);
+}
+
+template <typename T>
+static int add_typed(const void* a, const void* b, void* dst, int64_t n, hipStream_t s) {
+  hipLaunchKernelGGL((add_kernel<T>), dim3(stream_blocks(n, WideVec<T>::value)), dim3(256), 0, s,
+                     static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(dst), n);
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+template <typename T>
+static int relu_typed(const void* a, void* dst, int64_t n, hipStream_t s) {
+  hipLaunchKernelGGL((relu_kernel<T>), dim3(stream_blocks(n, WideVec<T>::value)), dim3(256), 0, s,
+                     static_cast<const T*>(a), static_cast<T*>(dst), n);
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+template <typename S, typename D>
+static int cast_typed(const void* a, void* dst, int64_t n, hipStream_t s) {
+  hipLaunchKernelGGL((cast_kernel<S, D>), dim3(stream_blocks(n, 8)), dim3(256), 0, s, static_cast<const S*>(a),
+                     static_cast<D*>(dst), n);
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+template <typename S>
+static int cast_from(const void* a, void* dst, int64_t n, int out_dtype, hipStream_t s) {
+  switch (out_dtype) {
+    case MG_F32: return cast_typed<S, float>(a, dst, n, s);
+    case MG_F16: return cast_typed<S, f16_t>(a, dst, n, s);
+    default: return cast_typed<S, bf16_t>(a, dst, n, s);
+  }
+}
+
+template <typename V>
+static int contiguous_launch(const void* src, void* dst, const CopyView& v, int64_t n, bool narrow, hipStream_t s) {
+  const dim3 grid(stream_blocks(n, 1));
+  if (narrow)
+    hipLaunchKernelGGL((contiguous_kernel<V, uint32_t>), grid, dim3(256), 0, s, static_cast<const V*>(src),
+                       static_cast<V*>(dst), v, n);
+  else
+    hipLaunchKernelGGL((contiguous_kernel<V, int64_t>), grid, dim3(256), 0, s, static_cast<const V*>(src),
+                       static_cast<V*>(dst), v, n);
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+static int contiguous_dispatch(const void* src, void* dst, int rank, const int64_t* shape, const int64_t* strides,
+                               int dtype, hipStream_t s) {
+  const int esz = dtype_size(dtype);
+  if (esz == 0) return fail(MG_ERR_INVALID, "contiguous: unsupported dtype %d", dtype);
+  if (rank < 0 || rank > kMaxRank) return fail(MG_ERR_INVALID, "contiguous: rank %d outside 0..%d", rank, kMaxRank);
+  if (rank > 0 && (!shape || !strides)) return fail(MG_ERR_INVALID, "contiguous: null shape or strides");
+  int64_t n = 1;
+  for (int d = 0; d < rank; ++d) {
+    if (shape[d] < 0 || strides[d] < 0)
+      return fail(MG_ERR_INVALID, "contiguous: negative extent or stride at dim %d", d);
+    n *= shape[d];
+  }
+  if (n == 0) return MG_OK;
+  if (!src || !dst) return fail(MG_ERR_INVALID, "contiguous: null pointer argument");
+  // Drop unit dims and merge neighbours that are contiguous with each other.
+  int64_t sh[kMaxRank], st[kMaxRank];
+  int r = 0;
+  for (int d = 0; d < rank; ++d) {
+    if (shape[d] == 1) continue;
+    if (r > 0 && st[r - 1] == shape[d] * strides[d]) {
+      sh[r - 1] *= shape[d];
+      st[r - 1] = strides[d];
+    } else {
+      sh[r] = shape[d];
+      st[r] = strides[d];
+      ++r;
+    }
+  }
+  if (r == 0) {
+    sh[0] = 1;
+    st[0] = 1;
+    r = 1;
+  }
+  // Widest chunk (bytes) that divides the innermost run and every outer stride.
+  int chunk = esz;
+  if (st[r - 1] == 1) {
+    for (int c = 16; c > esz; c /= 2) {
+      const int64_t elems = c / esz;
+      bool ok = sh[r - 1] % elems == 0 && reinterpret_cast<uintptr_t>(src) % c == 0 &&
+                reinterpret_cast<uintptr_t>(dst) % c == 0;
+      for (int d = 0; d + 1 < r && ok; ++d) ok = st[d] % elems == 0;
+      if (ok) {
+        chunk = c;
+        break;
+      }
+    }
+  }
+  const int64_t elems = chunk / esz;
+  CopyView v;
+  v.rank = r;
+  int64_t max_off = 0;
+  for (int d = 0; d < r; ++d) {
+    v.shape[d] = d == r - 1 ? sh[d] / elems : sh[d];
+    v.stride[d] = d == r - 1 ? st[d] : st[d] / elems;  // innermost stride is 1 chunk when elems > 1
+    max_off += (v.shape[d] - 1) * v.stride[d];
+  }
+  const int64_t chunks = n / elems;
+  const bool narrow = chunks < (int64_t{1} << 31) && max_off < (int64_t{1} << 31);
+  switch (chunk) {
+    case 16: return contiguous_launch<uint4>(src, dst, v, chunks, narrow, s);
+    case 8: return contiguous_launch<uint2>(src, dst, v, chunks, narrow, s);
+    case 4: return contiguous_launch<uint32_t>(src, dst, v, chunks, narrow, s);
+    default: return contiguous_launch<uint16_t>(src, dst, v, chunks, narrow, s);
+  }
+}
+
+}  // namespace mg
+
+extern "C" {
+
+int mg_add(const void* a, const void* b, void* dst, int64_t n, int dtype, mg_stream stream) {
+  if (!mg::is_float_dtype(dtype)) return mg::fail(MG_ERR_INVALID, "add: unsupported dtype %s", mg::dtype_name(dtype));
+  if (n < 0) return mg::fail(MG_ERR_INVALID, "add: negative size");
+  if (n == 0) return MG_OK;
+  if (!a || !b || !dst) return mg::fail(MG_ERR_INVALID, "add: null pointer argument");
+  if (!mg::aligned16(a) || !mg::aligned16(b) || !mg::aligned16(dst))
+    return mg::fail(MG_ERR_INVALID, "add: pointers must be 16-byte aligned");
+  hipStream_t s = mg::to_stream(stream);
+  switch (dtype) {
+    case MG_F32: return mg::add_typed<float>(a, b, dst, n, s);
+    case MG_F16: return mg::add_typed<mg::f16_t>(a, b, dst, n, s);
+    default: return mg::add_typed<mg::bf16_t>(a, b, dst, n, s);
+  }
+}
+
+int mg_relu(const void* a, void* dst, int64_t n, int dtype, mg_stream stream) {
+  if (!mg::is_float_dtype(dtype)) return mg::fail(MG_ERR_INVALID, "relu: unsupported dtype %s", mg::dtype_name(dtype));
+  if (n < 0) return mg::fail(MG_ERR_INVALID, "relu: negative size");
+  if (n == 0) return MG_OK;
+  if (!a || !dst) return mg::fail(MG_ERR_INVALID, "relu: null pointer argument");
+  if (!mg::aligned16(a) || !mg::aligned16(dst)) return mg::fail(MG_ERR_INVALID, "relu: pointers must be 16-byte aligned");
+  hipStream_t s = mg::to_stream(stream);
+  switch (dtype) {
+    case MG_F32: return mg::relu_typed<float>(a, dst, n, s);
+    case MG_F16: return mg::relu_typed<mg::f16_t>(a, dst, n, s);
+    default: return mg::relu_typed<mg::bf16_t>(a, dst, n, s);
+  }
+}
+
+int mg_cast(const void* a, void* dst, int64_t n, int in_dtype, int out_dtype, mg_stream stream) {
+  if (!mg::is_float_dtype(in_dtype) || !mg::is_float_dtype(out_dtype))
+    return mg::fail(MG_ERR_INVALID, "cast: unsupported dtype combination %s -> %s", mg::dtype_name(in_dtype),
+                    mg::dtype_name(out_dtype));
+  if (n < 0) return mg::fail(MG_ERR_INVALID, "cast: negative size");
+  if (n == 0) return MG_OK;
+  if (!a || !dst) return mg::fail(MG_ERR_INVALID, "cast: null pointer argument");
+  if (!mg::aligned16(a) || !mg::aligned16(dst)) return mg::fail(MG_ERR_INVALID, "cast: pointers must be 16-byte aligned");
+  hipStream_t s = mg::to_stream(stream);
+  if (in_dtype == out_dtype) {
+    MG_HIP(hipMemcpyAsync(dst, a, static_cast<size_t>(n) * mg::dtype_size(in_dtype), hipMemcpyDeviceToDevice, s));
+    return MG_OK;
+  }
+  switch (in_dtype) {
+    case MG_F32: return mg::cast_from<float>(a, dst, n, out_dtype, s);
+    case MG_F16: return mg::cast_from<mg::f16_t>(a, dst, n, out_dtype, s);
+    default: return mg::cast_from<mg::bf16_t>(a, dst, n, out_dtype, s);
+  }
+}
+
+int mg_contiguous(const void* a, void* dst, int rank, const int64_t* shape, const int64_t* strides, int dtype,
+                  mg_stream stream) {
+  return mg::contiguous_dispatch(a, dst, rank, shape, strides, dtype, mg::to_stream(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,211 @@
+// Row gather (embedding lookup) and its gradient, the row scatter-add.
+//
+// The scatter-add uses no atomics: each wave owns one destination row (and one slab of
+// the index list), scans the indices 64 at a time, and adds the matching value rows in
+// index order with fp32 accumulation, so the result does not depend on scheduling.
+#include "mg_device.h"
+#include "mg_internal.h"
+#include "mg_rows.h"
+
+namespace mg {
+
+// dst(i, :) = src(indices[i], :) over chunks of VEC elements; rows whose index is outside
+// [0, num_rows) are filled with zeros.
+template <typename T, typename I, int VEC>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const T* __restrict__ src, const I* __restrict__ indices,
+                                                          T* __restrict__ dst, int64_t n_idx, int64_t num_rows,
+                                                          int64_t row_size, int64_t row_stride, int64_t col_stride) {
+  const int64_t chunks_per_row = row_size / VEC;
+  const int64_t total = n_idx * chunks_per_row;
+  const int64_t step = static_cast<int64_t>(gridDim.x) * 256;
+  for (int64_t flat = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; flat < total; flat += step) {
+    const int64_t i = flat / chunks_per_row;
+    const int64_t c = (flat - i * chunks_per_row) * VEC;
+    const int64_t r = static_cast<int64_t>(indices[i]);
+    float v[VEC];
+    if (r >= 0 && r < num_rows) {
+      if constexpr (VEC == 1) {
+        v[0] = to_float(src[r * row_stride + c * col_stride]);
+      } else {
+        VecIO<T, VEC>::load(src + r * row_stride + c, v);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[e] = 0.f;
+    }
+    VecIO<T, VEC>::store(dst + i * row_size + c, v);
+  }
+}
+
+// One wave per (destination row, column block, slab).  DIRECT writes the row itself (one
+// slab); otherwise fp32 partials (slab, row, col) go to scratch for reduce_partials_kernel.
+template <typename T, typename I, int VEC, bool DIRECT>
+__global__ __launch_bounds__(64) void scatter_rows_kernel(const I* __restrict__ indices, const T* __restrict__ values,
+                                                          float* __restrict__ part, T* __restrict__ dst, int64_t n_idx,
+                                                          int64_t num_rows, int64_t row_size, int64_t slab_len) {
+  const int lane = threadIdx.x;
+  const int64_t col = (static_cast<int64_t>(blockIdx.y) * 64 + lane) * VEC;
+  const int64_t row = blockIdx.x;
+  const int64_t slab = blockIdx.z;
+  const int64_t i0 = slab * slab_len;
+  const int64_t i1 = min(i0 + slab_len, n_idx);
+  const bool active = col < row_size;
+  float acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+  for (int64_t base = i0; base < i1; base += 64) {
+    const int64_t mine = base + lane;
+    const bool hit = mine < i1 && static_cast<int64_t>(indices[mine]) == row;
+    uint64_t hits = __ballot(hit);
+    while (hits) {  // wave-uniform: ascending index order
+      const int bit = __ffsll(static_cast<long long>(hits)) - 1;
+      hits &= hits - 1;
+      if (active) {
+        float v[VEC];
+        VecIO<T, VEC>::load(values + (base + bit) * row_size + col, v);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] += v[e];
+      }
+    }
+  }
+  if (!active) return;
+  if constexpr (DIRECT) {
+    VecIO<T, VEC>::store(dst + row * row_size + col, acc);
+  } else {
+    float* p = part + (slab * num_rows + row) * row_size + col;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) p[e] = acc[e];
+  }
+}
+
+template <typename T, typename I>
+static int gather_typed(const void* src, const void* indices, void* dst, int64_t n_idx, int64_t num_rows,
+                        int64_t row_size, int64_t row_stride, int64_t col_stride, hipStream_t s) {
+  constexpr int WIDE = WideVec<T>::value;
+  const bool wide = col_stride == 1 && row_size % WIDE == 0 && row_stride % WIDE == 0 && aligned16(src) && aligned16(dst);
+  const int64_t chunks = n_idx * (wide ? row_size / WIDE : row_size);
+  int64_t blocks = ceil_div(chunks, 256);
+  const int64_t cap = static_cast<int64_t>(device_info().cu_count) * 16;
+  if (blocks > cap) blocks = cap;
+  const dim3 grid(static_cast<unsigned>(blocks));
+  if (wide)
+    hipLaunchKernelGGL((gather_rows_kernel<T, I, WIDE>), grid, dim3(256), 0, s, static_cast<const T*>(src),
+                       static_cast<const I*>(indices), static_cast<T*>(dst), n_idx, num_rows, row_size, row_stride,
+                       col_stride);
+  else
+    hipLaunchKernelGGL((gather_rows_kernel<T, I, 1>), grid, dim3(256), 0, s, static_cast<const T*>(src),
+                       static_cast<const I*>(indices), static_cast<T*>(dst), n_idx, num_rows, row_size, row_stride,
+                       col_stride);
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+template <typename T, typename I, int VEC>
+static int scatter_launch(const I* indices, const T* values, T* dst, int64_t n_idx, int64_t num_rows, int64_t row_size,
+                          hipStream_t s) {
+  const int64_t col_blocks = ceil_div(row_size, 64 * VEC);
+  // Slabs of the index list: enough waves to fill the device, at least 256 indices each,
+  // partial sums capped at 64 MiB.
+  int64_t slabs = ceil_div(static_cast<int64_t>(device_info().cu_count) * 16, num_rows * col_blocks);
+  const int64_t by_len = ceil_div(n_idx, 256);
+  if (slabs > by_len) slabs = by_len;
+  const int64_t by_bytes = (int64_t{64} << 20) / (num_rows * row_size * static_cast<int64_t>(sizeof(float)));
+  if (slabs > by_bytes) slabs = by_bytes;
+  if (slabs > 65535) slabs = 65535;
+  if (slabs < 1) slabs = 1;
+  const int64_t slab_len = ceil_div(ceil_div(n_idx, slabs), 64) * 64;
+  slabs = n_idx > 0 ? ceil_div(n_idx, slab_len) : 1;
+  const dim3 grid(static_cast<unsigned>(num_rows), static_cast<unsigned>(col_blocks), static_cast<unsigned>(slabs));
+  if (slabs == 1) {
+    hipLaunchKernelGGL((scatter_rows_kernel<T, I, VEC, true>), grid, dim3(64), 0, s, indices, values, nullptr, dst,
+                       n_idx, num_rows, row_size, slab_len);
+    MG_LAUNCH_CHECK();
+    return MG_OK;
+  }
+  Scratch part;
+  MG_TRY(part.take(slabs * num_rows * row_size * static_cast<int64_t>(sizeof(float))));
+  hipLaunchKernelGGL((scatter_rows_kernel<T, I, VEC, false>), grid, dim3(64), 0, s, indices, values, part.as<float>(),
+                     dst, n_idx, num_rows, row_size, slab_len);
+  MG_LAUNCH_CHECK();
+  const int64_t cols = num_rows * row_size;
+  hipLaunchKernelGGL((reduce_partials_kernel<T>), dim3(static_cast<unsigned>(ceil_div(cols, 64)), 1), dim3(256), 0, s,
+                     part.as<float>(), dst, nullptr, nullptr, slabs, cols);
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+template <typename T, typename I>
+static int scatter_typed(const void* indices, const void* values, void* dst, int64_t n_idx, int64_t num_rows,
+                         int64_t row_size, hipStream_t s) {
+  constexpr int WIDE = WideVec<T>::value;
+  const bool wide = row_size % WIDE == 0 && aligned16(values) && aligned16(dst);
+  if (wide)
+    return scatter_launch<T, I, WIDE>(static_cast<const I*>(indices), static_cast<const T*>(values),
+                                      static_cast<T*>(dst), n_idx, num_rows, row_size, s);
+  return scatter_launch<T, I, 1>(static_cast<const I*>(indices), static_cast<const T*>(values), static_cast<T*>(dst),
+                                 n_idx, num_rows, row_size, s);
+}
+
+template <typename T>
+static int gather_by_index(const void* src, const void* indices, void* dst, int64_t n_idx, int64_t num_rows,
+                           int64_t row_size, int64_t row_stride, int64_t col_stride, int idx_dtype, hipStream_t s) {
+  if (idx_dtype == MG_I32)
+    return gather_typed<T, int32_t>(src, indices, dst, n_idx, num_rows, row_size, row_stride, col_stride, s);
+  return gather_typed<T, int64_t>(src, indices, dst, n_idx, num_rows, row_size, row_stride, col_stride, s);
+}
+
+template <typename T>
+static int scatter_by_index(const void* indices, const void* values, void* dst, int64_t n_idx, int64_t num_rows,
+                            int64_t row_size, int idx_dtype, hipStream_t s) {
+  if (idx_dtype == MG_I32) return scatter_typed<T, int32_t>(indices, values, dst, n_idx, num_rows, row_size, s);
+  return scatter_typed<T, int64_t>(indices, values, dst, n_idx, num_rows, row_size, s);
+}
+
+}  // namespace mg
+
+extern "C" {
+
+int mg_gather(const void* src, const void* indices, void* dst, int64_t n_idx, int64_t num_rows, int64_t row_size,
+              int64_t src_row_stride, int64_t src_col_stride, int idx_dtype, int dtype, mg_stream stream) {
+  if (!mg::is_float_dtype(dtype)) return mg::fail(MG_ERR_INVALID, "gather: unsupported dtype %s", mg::dtype_name(dtype));
+  if (idx_dtype != MG_I32 && idx_dtype != MG_I64)
+    return mg::fail(MG_ERR_INVALID, "gather: indices must be int32 or int64, got %s", mg::dtype_name(idx_dtype));
+  if (n_idx < 0 || num_rows < 0 || row_size < 0 || src_row_stride < 0 || src_col_stride < 0)
+    return mg::fail(MG_ERR_INVALID, "gather: negative size or stride");
+  if (n_idx == 0 || row_size == 0) return MG_OK;
+  if (!indices || !dst || (num_rows > 0 && !src)) return mg::fail(MG_ERR_INVALID, "gather: null pointer argument");
+  hipStream_t s = mg::to_stream(stream);
+  switch (dtype) {
+    case MG_F32:
+      return mg::gather_by_index<float>(src, indices, dst, n_idx, num_rows, row_size, src_row_stride, src_col_stride,
+                                        idx_dtype, s);
+    case MG_F16:
+      return mg::gather_by_index<mg::f16_t>(src, indices, dst, n_idx, num_rows, row_size, src_row_stride,
+                                            src_col_stride, idx_dtype, s);
+    default:
+      return mg::gather_by_index<mg::bf16_t>(src, indices, dst, n_idx, num_rows, row_size, src_row_stride,
+                                             src_col_stride, idx_dtype, s);
+  }
+}
+
+int mg_scatter_add(const void* indices, const void* values, void* dst, int64_t n_idx, int64_t num_rows,
+                   int64_t row_size, int idx_dtype, int dtype, mg_stream stream) {
+  if (!mg::is_float_dtype(dtype))
+    return mg::fail(MG_ERR_INVALID, "scatter_add: unsupported dtype %s", mg::dtype_name(dtype));
+  if (idx_dtype != MG_I32 && idx_dtype != MG_I64)
+    return mg::fail(MG_ERR_INVALID, "scatter_add: indices must be int32 or int64, got %s", mg::dtype_name(idx_dtype));
+  if (n_idx < 0 || num_rows < 0 || row_size < 0) return mg::fail(MG_ERR_INVALID, "scatter_add: negative size");
+  if (num_rows == 0 || row_size == 0) return MG_OK;
+  if (num_rows > INT32_MAX || row_size > int64_t{65535} * 64)
+    return mg::fail(MG_ERR_UNSUPPORTED, "scatter_add: destination (%lld, %lld) exceeds the launch grid",
+                    static_cast<long long>(num_rows), static_cast<long long>(row_size));
+  if (!dst || (n_idx > 0 && (!indices || !values))) return mg::fail(MG_ERR_INVALID, "scatter_add: null pointer argument");
+  hipStream_t s = mg::to_stream(stream);
+  switch (dtype) {
+    case MG_F32: return mg::scatter_by_index<float>(indices, values, dst, n_idx, num_rows, row_size, idx_dtype, s);
+    case MG_F16: return mg::scatter_by_index<mg::f16_t>(indices, values, dst, n_idx, num_rows, row_size, idx_dtype, s);
+    default: return mg::scatter_by_index<mg::bf16_t>(indices, values, dst, n_idx, num_rows, row_size, idx_dtype, s);
+  }
+}
+
+}  // extern "C"

@@ -46,7 +46,7 @@ static bool mult8(int64_t v) { return (v & 7) == 0; }
 
 // 16-bit MFMA path, optionally split along K when the output has too few tiles to fill
 // the device (dW of a narrow layer: reduction over thousands of rows into a small matrix).
-template <typename T, bool A_KC, bool B_KC>
+template <typename T, bool A_KC, bool B_KC, bool RAGGED>
 static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
   const int tiles_m = static_cast<int>(ceil_div(g.M, kGemmBM));
   const int tiles_n = static_cast<int>(ceil_div(g.N, kGemmBN));
@@ -70,11 +70,11 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
   }
   if (splits <= 1) {
     if (bias)
-      hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, true, false>), dim3(static_cast<unsigned>(blocks)),
+      hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, true, false, RAGGED>), dim3(static_cast<unsigned>(blocks)),
                          dim3(kGemmThreads), 0, stream, a, b, bias, c, nullptr, M, N, K, lda, ldb, g.N, g.bsa, g.bsb,
                          g.M * g.N, tiles_m, tiles_n, K);
     else
-      hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, false, false>), dim3(static_cast<unsigned>(blocks)),
+      hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, false, false, RAGGED>), dim3(static_cast<unsigned>(blocks)),
                          dim3(kGemmThreads), 0, stream, a, b, bias, c, nullptr, M, N, K, lda, ldb, g.N, g.bsa, g.bsb,
                          g.M * g.N, tiles_m, tiles_n, K);
     MG_LAUNCH_CHECK();
@@ -85,7 +85,7 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
   Scratch partial;
   const int64_t numel = g.M * g.N;
   MG_TRY(partial.take(static_cast<int64_t>(splits) * numel * static_cast<int64_t>(sizeof(float))));
-  hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, false, true>),
+  hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, false, true, RAGGED>),
                      dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(splits)), dim3(kGemmThreads), 0, stream, a,
                      b, bias, c, partial.as<float>(), M, N, K, lda, ldb, g.N, g.bsa, g.bsb, numel, tiles_m, tiles_n,
                      k_per_split);
@@ -105,18 +105,29 @@ template <typename T>
 static int dispatch_16bit(const GemmArgs& g, hipStream_t stream, bool* handled) {
   *handled = false;
   if (g.K <= 0) return MG_OK;
-  const bool a_kc = g.sak == 1 && mult8(g.sam) && mult8(g.K);
-  const bool a_mc = g.sam == 1 && mult8(g.sak) && mult8(g.M);
-  const bool b_kc = g.sbk == 1 && mult8(g.sbn) && mult8(g.K);
-  const bool b_nc = g.sbn == 1 && mult8(g.sbk) && mult8(g.N);
-  const bool aligned = aligned16(g.a) && aligned16(g.b) && mult8(g.bsa) && mult8(g.bsb);
+  // Each operand must be contiguous along k or along its other axis.  When leading
+  // dimensions, extents and addresses are all multiples of 8 elements the tiles are staged
+  // with 16-byte loads; otherwise with element loads (the ragged variant).
+  const bool a_kc = g.sak == 1;
+  const bool a_mc = g.sam == 1;
+  const bool b_kc = g.sbk == 1;
+  const bool b_nc = g.sbn == 1;
   const bool worth_it = g.M * g.N >= 64 * 64 || g.K >= 512;
-  if (!(aligned && worth_it && (a_kc || a_mc) && (b_kc || b_nc))) return MG_OK;
+  if (!(worth_it && (a_kc || a_mc) && (b_kc || b_nc))) return MG_OK;
+  const bool a_wide = a_kc ? mult8(g.sam) && mult8(g.K) : mult8(g.sak) && mult8(g.M);
+  const bool b_wide = b_kc ? mult8(g.sbn) && mult8(g.K) : mult8(g.sbk) && mult8(g.N);
+  const bool wide = a_wide && b_wide && aligned16(g.a) && aligned16(g.b) && mult8(g.bsa) && mult8(g.bsb);
   *handled = true;
-  if (a_kc && b_kc) return launch_16bit_mfma<T, true, true>(g, stream);
-  if (a_kc) return launch_16bit_mfma<T, true, false>(g, stream);
-  if (b_kc) return launch_16bit_mfma<T, false, true>(g, stream);
-  return launch_16bit_mfma<T, false, false>(g, stream);
+  if (wide) {
+    if (a_kc && b_kc) return launch_16bit_mfma<T, true, true, false>(g, stream);
+    if (a_kc) return launch_16bit_mfma<T, true, false, false>(g, stream);
+    if (b_kc) return launch_16bit_mfma<T, false, true, false>(g, stream);
+    return launch_16bit_mfma<T, false, false, false>(g, stream);
+  }
+  if (a_kc && b_kc) return launch_16bit_mfma<T, true, true, true>(g, stream);
+  if (a_kc) return launch_16bit_mfma<T, true, false, true>(g, stream);
+  if (b_kc) return launch_16bit_mfma<T, false, true, true>(g, stream);
+  return launch_16bit_mfma<T, false, false, true>(g, stream);
 }
 
 template <typename T>

@@ -296,11 +296,44 @@ struct Gemm16Stage {
 
 // KC: element (o, k) at base[o * ld + k].  4 chunks of 8 k-values per thread.
 // else: element (o, k) at base[k * ld + o].  2 tasks per thread, each two k rows x 8 o.
-template <typename T, bool KC>
+// RAGGED: leading dimension, extents or base address are not multiples of 8 elements, so
+// each chunk is assembled from eight 2-byte loads with per-element bounds.
+template <typename T>
+__device__ __forceinline__ uint4 gemm16_gather8(const T* __restrict__ p, int valid) {
+  const uint16_t* q = reinterpret_cast<const uint16_t*>(p);
+  uint32_t w[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const uint32_t lo = 2 * e < valid ? q[2 * e] : 0u;
+    const uint32_t hi = 2 * e + 1 < valid ? q[2 * e + 1] : 0u;
+    w[e] = lo | (hi << 16);
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+template <typename T, bool KC, bool RAGGED>
 __device__ __forceinline__ void gemm16_load(const T* __restrict__ base, int64_t ld, int o0, int k0, int O, int k_end,
                                             Gemm16Stage& st) {
   const int t = threadIdx.x;
-  if constexpr (KC) {
+  if constexpr (RAGGED && KC) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = t + i * kGemmThreads;
+      const int o = min(o0 + idx / 8, O - 1);
+      const int k = k0 + (idx % 8) * 8;
+      st.v[i] = gemm16_gather8(base + static_cast<int64_t>(o) * ld + k, k_end - k);
+    }
+  } else if constexpr (RAGGED) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int idx = t + i * kGemmThreads;
+      const int kp = idx % 32, oc = idx / 32;
+      const int k = k0 + 2 * kp;
+      const int o = o0 + oc * 8;
+      st.v[2 * i] = gemm16_gather8(base + static_cast<int64_t>(k) * ld + o, k < k_end ? O - o : 0);
+      st.v[2 * i + 1] = gemm16_gather8(base + static_cast<int64_t>(k + 1) * ld + o, k + 1 < k_end ? O - o : 0);
+    }
+  } else if constexpr (KC) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int idx = t + i * kGemmThreads;
@@ -357,7 +390,7 @@ __device__ __forceinline__ uint4 gemm16_frag(const uint16_t* __restrict__ lds, i
   return *reinterpret_cast<const uint4*>(lds + (o_base + lane % 32) * kG16Stride + ks * 16 + (lane / 32) * 8);
 }
 
-template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K>
+template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, bool RAGGED>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
     const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C,
     float* __restrict__ partial, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb,
@@ -390,16 +423,16 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   Gemm16Stage sa, sb;
-  gemm16_load<T, A_KC>(A, lda, m0, k_begin, M, k_end, sa);
-  gemm16_load<T, B_KC>(B, ldb, n0, k_begin, N, k_end, sb);
+  gemm16_load<T, A_KC, RAGGED>(A, lda, m0, k_begin, M, k_end, sa);
+  gemm16_load<T, B_KC, RAGGED>(B, ldb, n0, k_begin, N, k_end, sb);
 
   for (int k0 = k_begin; k0 < k_end; k0 += kG16BK) {
     gemm16_store<A_KC>(lds_a, sa);
     gemm16_store<B_KC>(lds_b, sb);
     __syncthreads();
     if (k0 + kG16BK < k_end) {
-      gemm16_load<T, A_KC>(A, lda, m0, k0 + kG16BK, M, k_end, sa);
-      gemm16_load<T, B_KC>(B, ldb, n0, k0 + kG16BK, N, k_end, sb);
+      gemm16_load<T, A_KC, RAGGED>(A, lda, m0, k0 + kG16BK, M, k_end, sa);
+      gemm16_load<T, B_KC, RAGGED>(B, ldb, n0, k0 + kG16BK, N, k_end, sb);
     }
 #pragma unroll
     for (int ks = 0; ks < kG16BK / 16; ++ks) {

@@ -516,9 +516,86 @@ def relu_grad(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBu
     return [out]
 
 
+def _require_contiguous(node: Node, count: int, who: str) -> None:
+    for i in range(count):
+        if not node.src(i).layout().is_contiguous():
+            raise MogradError(2, f"{who}: strided operand is outside this path; materialise it with contiguous first")
+
+
+def add(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """ADD[a, b] (residual connections, gradient accumulation).  runtime/__init__.mojo:319-333."""
+    _require_contiguous(node, 2, "add")
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_add(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), node.numel(), node.dtype(),
+                      device.stream)
+    return [out]
+
+
+def relu(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """RELU[a].  runtime/__init__.mojo:296-297."""
+    _require_contiguous(node, 1, "relu")
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_relu(inputs[0].data_ptr(), out.data_ptr(), node.numel(), node.dtype(), device.stream)
+    return [out]
+
+
+def cast(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """CAST[a] to node.dtype().  runtime/__init__.mojo:300-311."""
+    _require_contiguous(node, 1, "cast")
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_cast(inputs[0].data_ptr(), out.data_ptr(), node.numel(), node.src(0).dtype(), node.dtype(),
+                       device.stream)
+    return [out]
+
+
+def contiguous(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """CONTIGUOUS[a]: row-major copy of a strided view.  runtime/__init__.mojo:456-461."""
+    layout = node.src(0).layout()
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_contiguous(inputs[0].data_ptr(), out.data_ptr(), layout.rank(), _i64_array(layout.shape()),
+                             _i64_array(layout.stride()), node.dtype(), device.stream)
+    return [out]
+
+
+def gather(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """GATHER[src (rows, row_size), indices] -> (*indices.shape, row_size).
+    runtime/__init__.mojo:239-240, kernels/__init__.mojo:132-163."""
+    la = node.src(0).layout()
+    lb = node.src(1).layout()
+    if la.rank() != 2:  # op.mojo:367-368
+        raise MogradError(1, "gather expects a 2D source tensor [num_rows, row_size]")
+    if not lb.is_contiguous():
+        raise MogradError(2, "gather: strided indices are outside this path")
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_gather(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), lb.numel(), la.shape(0),
+                         la.shape(1), la.stride(0), la.stride(1), node.src(1).dtype(), node.dtype(), device.stream)
+    return [out]
+
+
+def scatter_add(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """SCATTER_ADD[indices, values (*indices.shape, row_size)] -> (num_rows, row_size).
+    runtime/__init__.mojo:243-256; the output needs no zero fill here."""
+    la = node.src(0).layout()
+    lb = node.src(1).layout()
+    if lb.rank() != la.rank() + 1:  # op.mojo:375-376
+        raise MogradError(1, "scatter_add expects values shaped [*indices.shape, row_size]")
+    _require_contiguous(node, 2, "scatter_add")
+    row_size = lb.shape(lb.rank() - 1)
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_scatter_add(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), la.numel(),
+                              node.shape(0), row_size, node.src(0).dtype(), node.dtype(), device.stream)
+    return [out]
+
+
 # Op type -> exec function, the rows of the reference's rule table that belong to this
 # path (mograd/runtime/__init__.mojo:113-167).
 SCHEDULER_RULES = {
+    "ADD": add,
+    "RELU": relu,
+    "CAST": cast,
+    "CONTIGUOUS": contiguous,
+    "GATHER": gather,
+    "SCATTER_ADD": scatter_add,
     "RELU_GRAD": relu_grad,
     "SUM": sum,
     "MATMUL": matmul,

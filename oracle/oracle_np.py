@@ -21,6 +21,9 @@ Pinning (what makes each function trustworthy without running the reference):
                         tests/test_grad.mojo:1001-1023, brute-force loop twin
                         (sdpa_*_loops), torch SDPA autograd (f64)
   matmul* / sum_axis    numpy BLAS identities, finite differences
+  gather / scatter_add  index arithmetic by definition; adjoint identity
+                        <gather(W, i), Y> = <W, scatter_add(i, Y)>; torch index_add_
+  tiny_transformer_step torch autograd (f64) on the same model, finite differences
   round_class           tests/test_memory.mojo:18-30 (1000 -> 1024, 1025 -> 1152)
 All of the above are exercised in tests/test_oracle.py.
 """
@@ -344,6 +347,112 @@ def relu_grad(out, upstream):
     """upstream where relu output > 0, else 0.  kernels/elementwise.mojo:66-67."""
     out = np.asarray(out, dtype=F64)
     return np.where(out > 0, np.asarray(upstream, dtype=F64), 0.0)
+
+
+def relu(a):
+    """max(a, 0).  kernels/elementwise.mojo (relu_op)."""
+    a = np.asarray(a, dtype=F64)
+    return np.where(a > 0, a, 0.0)
+
+
+# --------------------------------------------------------------------------- #
+# Embedding lookup and its gradient
+# --------------------------------------------------------------------------- #
+
+
+def gather(src, indices):
+    """out[..., :] = src[indices[...], :].  kernels/gather_scatter.mojo:14-38."""
+    src = np.asarray(src, dtype=F64)
+    idx = np.asarray(indices, dtype=np.int64)
+    return src[idx]
+
+
+def scatter_add(indices, values, num_rows):
+    """dst[r, :] = sum of values[i, :] over i with indices[i] == r, dst zero elsewhere.
+    kernels/gather_scatter.mojo:46-71 (atomic adds into a zero-filled buffer)."""
+    idx = np.asarray(indices, dtype=np.int64).reshape(-1)
+    vals = np.asarray(values, dtype=F64)
+    vals = vals.reshape(idx.size, -1)
+    dst = np.zeros((num_rows, vals.shape[1]), dtype=F64)
+    for i in range(idx.size):  # plain loop: this is the definition
+        dst[idx[i]] += vals[i]
+    return dst
+
+
+# --------------------------------------------------------------------------- #
+# The char-level transformer of examples/tinyshakespear/model.mojo: forward, loss and
+# every parameter gradient, composed from the functions above the way mograd/grad.mojo
+# composes the gradient graph.
+#   h = embed[ids]
+#   per block: h = h + W_O(attn(W_Q(LN1 h), W_K(LN1 h), W_V(LN1 h), causal))
+#              h = h + W2(relu(W1(LN2 h) + b1))
+#   logits = lm_head(h) ; loss = mean cross-entropy
+# --------------------------------------------------------------------------- #
+
+
+def tiny_transformer_step(params, ids, labels, n_heads, eps=1e-5):
+    """Returns (loss, grads) with grads shaped like params.
+
+    params = {"embed": (V, d), "lm_head": (V, d), "blocks": [ {"ln1_g","ln1_b","wq","wk",
+    "wv","wo" (d, d), "ln2_g","ln2_b","w1" (ff, d),"b1" (ff),"w2" (d, ff)} ... ]};
+    ids, labels: (B, T) integers.  model.mojo:22-26,62-64,88-101,120-121.
+    """
+    ids = np.asarray(ids, dtype=np.int64)
+    labels = np.asarray(labels, dtype=np.int64)
+    B, T = ids.shape
+    embed = np.asarray(params["embed"], dtype=F64)
+    V, d = embed.shape
+    dh = d // n_heads
+    n = B * T
+    h = gather(embed, ids.reshape(-1))  # (n, d)
+    saved = []
+    for blk in params["blocks"]:
+        c = {"h_in": h}
+        c["x1"] = layer_norm_fwd(h, blk["ln1_g"], blk["ln1_b"], eps)
+        q = matmul_bias_bt(c["x1"], blk["wq"]).reshape(B, T, n_heads, dh)
+        k = matmul_bias_bt(c["x1"], blk["wk"]).reshape(B, T, n_heads, dh)
+        v = matmul_bias_bt(c["x1"], blk["wv"]).reshape(B, T, n_heads, dh)
+        o, _ = sdpa_fwd(q, k, v, causal=True)  # BHSD
+        c["q"], c["k"], c["v"] = q, k, v
+        c["ctx"] = o.transpose(0, 2, 1, 3).reshape(n, d)
+        h = h + matmul_bias_bt(c["ctx"], blk["wo"])
+        c["h_mid"] = h
+        c["x2"] = layer_norm_fwd(h, blk["ln2_g"], blk["ln2_b"], eps)
+        c["a"] = relu(matmul_bias_bt(c["x2"], blk["w1"], blk["b1"]))
+        h = h + matmul_bias_bt(c["a"], blk["w2"])
+        saved.append(c)
+    logits = matmul_bias_bt(h, params["lm_head"])
+    flat_labels = labels.reshape(-1)
+    loss = cross_entropy_ids(logits, flat_labels)
+    dlogits = cross_entropy_grad_ids(logits, flat_labels, 1.0)
+
+    grads = {"lm_head": linear_grad_w(dlogits, h), "blocks": []}
+    dh_ = linear_grad_x(dlogits, params["lm_head"])
+    for blk, c in zip(reversed(params["blocks"]), reversed(saved)):
+        g = {}
+        # h = h_mid + W2 a
+        g["w2"] = linear_grad_w(dh_, c["a"])
+        da = relu_grad(c["a"], linear_grad_x(dh_, blk["w2"]))
+        g["w1"] = linear_grad_w(da, c["x2"])
+        g["b1"] = linear_grad_b(da)
+        dx2 = linear_grad_x(da, blk["w1"])
+        dmid, g["ln2_g"], g["ln2_b"] = layer_norm_bwd(dx2, c["h_mid"], blk["ln2_g"], eps)
+        dh_ = dh_ + dmid
+        # h_mid = h_in + W_O ctx
+        g["wo"] = linear_grad_w(dh_, c["ctx"])
+        dctx = linear_grad_x(dh_, blk["wo"])
+        do = dctx.reshape(B, T, n_heads, dh).transpose(0, 2, 1, 3)  # BHSD
+        dq, dk, dv = sdpa_bwd(c["q"], c["k"], c["v"], do, causal=True)
+        dq, dk, dv = (t.reshape(n, d) for t in (dq, dk, dv))
+        g["wq"] = linear_grad_w(dq, c["x1"])
+        g["wk"] = linear_grad_w(dk, c["x1"])
+        g["wv"] = linear_grad_w(dv, c["x1"])
+        dx1 = linear_grad_x(dq, blk["wq"]) + linear_grad_x(dk, blk["wk"]) + linear_grad_x(dv, blk["wv"])
+        din, g["ln1_g"], g["ln1_b"] = layer_norm_bwd(dx1, c["h_in"], blk["ln1_g"], eps)
+        dh_ = dh_ + din
+        grads["blocks"].insert(0, g)
+    grads["embed"] = scatter_add(ids.reshape(-1), dh_, V)
+    return float(loss), grads
 
 
 # --------------------------------------------------------------------------- #

@@ -177,7 +177,9 @@ def test_errors(device):
 # ---- 16-bit storage on the matrix cores (shapes that take the MFMA kernels) ------------
 
 HALF_MFMA_SHAPES = [(256, 384, 512), (384, 128, 1536), (200, 136, 264), (128, 64, 4096), (4096, 128, 128),
-                    (1024, 384, 384), (72, 1536, 384)]
+                    (1024, 384, 384), (72, 1536, 384),
+                    # extents that are not multiples of 8 (a 65-symbol vocabulary): element-wise staging
+                    (2048, 65, 384), (333, 65, 129), (130, 77, 1031), (4099, 65, 384)]
 
 
 @pytest.mark.parametrize("dtype,rtol", [(F16, 2e-3), (BF16, 1.6e-2)])

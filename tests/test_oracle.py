@@ -358,6 +358,108 @@ def test_c_oracle_attention(orc, causal, has_mask):
     np.testing.assert_allclose(dv, rdv, atol=5e-6)
 
 
+# --------------------------------------------------------------------------- #
+# Embedding lookup / scatter-add and the whole transformer step
+# --------------------------------------------------------------------------- #
+
+
+def test_gather_scatter_add_pins():
+    rng = np.random.default_rng(21)
+    V, d, n = 7, 5, 40
+    w = rng.normal(size=(V, d))
+    y = rng.normal(size=(n, d))
+    idx = rng.integers(0, V, size=n)
+    idx[:3] = 2  # repeats are the point
+    g = O.gather(w, idx)
+    for i in range(n):
+        np.testing.assert_array_equal(g[i], w[idx[i]])
+    sa = O.scatter_add(idx, y, V)
+    # adjoint identity: <gather(W, i), Y> = <W, scatter_add(i, Y)>
+    assert abs((g * y).sum() - (w * sa).sum()) < 1e-10
+    # library routine
+    ref = torch.zeros(V, d, dtype=torch.float64).index_add_(0, torch.from_numpy(idx), torch.from_numpy(y)).numpy()
+    np.testing.assert_allclose(sa, ref, atol=1e-12)
+    # a row nobody indexes stays zero
+    idx2 = np.where(idx == 4, 3, idx)
+    assert not O.scatter_add(idx2, y, V)[4].any()
+    # (B, T) index arrays flatten row-major
+    np.testing.assert_array_equal(O.gather(w, idx.reshape(4, 10)).reshape(n, d), g)
+
+
+def tiny_params(rng, V, d, ff, layers):
+    def lin(o, i):
+        b = math.sqrt(6.0 / i)
+        return rng.uniform(-b, b, size=(o, i))
+
+    blocks = []
+    for _ in range(layers):
+        blocks.append({
+            "ln1_g": rng.uniform(0.5, 1.5, d), "ln1_b": rng.normal(0, 0.1, d),
+            "wq": lin(d, d), "wk": lin(d, d), "wv": lin(d, d), "wo": lin(d, d),
+            "ln2_g": rng.uniform(0.5, 1.5, d), "ln2_b": rng.normal(0, 0.1, d),
+            "w1": lin(ff, d), "b1": rng.uniform(-0.1, 0.1, ff), "w2": lin(d, ff),
+        })
+    return {"embed": rng.normal(size=(V, d)), "lm_head": lin(V, d), "blocks": blocks}
+
+
+def torch_tiny_transformer(params, ids, labels, n_heads, eps=1e-5):
+    """The same model written with torch modules' functional forms and autograd (f64)."""
+    F = torch.nn.functional
+    leaf = lambda a: torch.tensor(np.asarray(a), dtype=torch.float64, requires_grad=True)
+    tp = {"embed": leaf(params["embed"]), "lm_head": leaf(params["lm_head"]),
+          "blocks": [{k: leaf(v) for k, v in b.items()} for b in params["blocks"]]}
+    B, T = ids.shape
+    d = tp["embed"].shape[1]
+    h = F.embedding(torch.from_numpy(ids), tp["embed"])
+    for b in tp["blocks"]:
+        x1 = F.layer_norm(h, (d,), b["ln1_g"], b["ln1_b"], eps)
+        q, k, v = (F.linear(x1, b[w]).reshape(B, T, n_heads, d // n_heads).transpose(1, 2) for w in ("wq", "wk", "wv"))
+        ctx = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(B, T, d)
+        h = h + F.linear(ctx, b["wo"])
+        x2 = F.layer_norm(h, (d,), b["ln2_g"], b["ln2_b"], eps)
+        h = h + F.linear(F.relu(F.linear(x2, b["w1"], b["b1"])), b["w2"])
+    logits = F.linear(h, tp["lm_head"])
+    loss = F.cross_entropy(logits.reshape(B * T, -1), torch.from_numpy(labels).reshape(-1))
+    loss.backward()
+    grads = {"embed": tp["embed"].grad.numpy(), "lm_head": tp["lm_head"].grad.numpy(),
+             "blocks": [{k: v.grad.numpy() for k, v in b.items()} for b in tp["blocks"]]}
+    return loss.item(), grads
+
+
+def test_tiny_transformer_step_vs_torch_autograd():
+    rng = np.random.default_rng(33)
+    V, d, ff, layers, heads, B, T = 11, 16, 40, 2, 2, 3, 9
+    params = tiny_params(rng, V, d, ff, layers)
+    ids = rng.integers(0, V, size=(B, T))
+    labels = rng.integers(0, V, size=(B, T))
+    loss, grads = O.tiny_transformer_step(params, ids, labels, heads)
+    tl, tg = torch_tiny_transformer(params, ids, labels, heads)
+    assert abs(loss - tl) < 1e-12
+    np.testing.assert_allclose(grads["embed"], tg["embed"], atol=1e-12)
+    np.testing.assert_allclose(grads["lm_head"], tg["lm_head"], atol=1e-12)
+    for g, t in zip(grads["blocks"], tg["blocks"]):
+        assert set(g) == set(t)
+        for name in g:
+            np.testing.assert_allclose(g[name], t[name], atol=1e-12, err_msg=name)
+
+
+def test_tiny_transformer_step_finite_difference():
+    rng = np.random.default_rng(34)
+    V, d, ff, layers, heads, B, T = 5, 8, 12, 1, 2, 2, 4
+    params = tiny_params(rng, V, d, ff, layers)
+    ids = rng.integers(0, V, size=(B, T))
+    labels = rng.integers(0, V, size=(B, T))
+    _, grads = O.tiny_transformer_step(params, ids, labels, heads)
+    h = 1e-6
+    for name, pos in [("wq", (1, 2)), ("w2", (3, 5)), ("b1", (4,)), ("ln1_g", (2,)), ("ln2_b", (6,))]:
+        base = params["blocks"][0][name]
+        up = base.copy(); up[pos] += h
+        dn = base.copy(); dn[pos] -= h
+        lu, _ = O.tiny_transformer_step({**params, "blocks": [{**params["blocks"][0], name: up}]}, ids, labels, heads)
+        ld, _ = O.tiny_transformer_step({**params, "blocks": [{**params["blocks"][0], name: dn}]}, ids, labels, heads)
+        assert abs((lu - ld) / (2 * h) - grads["blocks"][0][name][pos]) < 1e-7, name
+
+
 def test_c_oracle_round_class(orc):
     for n in [1, 512, 513, 990, 1000, 1024, 1025, 4096, 5000, 123457, (1 << 20) + 1]:
         assert orc.orc_round_class(n) == O.round_class(n)

@@ -1,0 +1,172 @@
+"""The remaining per-step ops of a transformer block on the GPU: add, relu, cast,
+contiguous, gather and scatter_add, through the scheduler entries the reference's graph
+reaches (mograd/runtime/__init__.mojo:239-256,296-333,456-461).
+
+add / relu / contiguous / gather move or combine values with at most one rounding, so
+they are checked bit for bit against numpy on the same (already rounded) inputs.
+scatter_add is a sum: it is checked against the float64 oracle at the fp32-reduction
+tolerance, for run-to-run bit equality (it uses no atomics), and through the adjoint
+identity with gather at full size.
+"""
+import numpy as np
+import pytest
+
+from helpers import ATOL_F32, RTOL_F32, assert_close, assert_sum_close, integers, normal
+from oracle import oracle_np as O
+
+pytestmark = pytest.mark.gpu
+
+from mograd_amd import BF16, F16, F32, I32, I64, AnyBuffer, Layout, MogradError, Node  # noqa: E402
+from mograd_amd import runtime as R  # noqa: E402
+from mograd_amd.runtime import round_to_dtype  # noqa: E402
+
+FLOATS = [F32, F16, BF16]
+
+
+def _run(device, op, out_layout, operands, dtype=F32, attrs=None):
+    """operands: list of (host array, layout view, dtype)."""
+    srcs = [Node.leaf(l, d) for _, l, d in operands]
+    node = Node(op, out_layout, dtype, srcs, attrs or {})
+    bufs = [AnyBuffer.from_numpy(device, a, d).view(l) for a, l, d in operands]
+    (out,) = R.run(node, bufs, device)
+    return out.to_numpy(out_layout.shape())
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("n", [1, 7, 8, 1000, 4096, 1 << 20, (1 << 20) + 3])
+def test_add_relu_exact(device, dtype, n):
+    a = round_to_dtype(normal(60, 0, (n,)), dtype)
+    b = round_to_dtype(normal(60, 1, (n,)), dtype)
+    got = _run(device, "ADD", Layout(n), [(a, Layout(n), dtype), (b, Layout(n), dtype)], dtype)
+    # one fp32 add, one rounding to the storage type
+    np.testing.assert_array_equal(got, round_to_dtype(a + b, dtype))
+    got = _run(device, "RELU", Layout(n), [(a, Layout(n), dtype)], dtype)
+    np.testing.assert_array_equal(got, np.maximum(a, 0))
+
+
+@pytest.mark.parametrize("src,dst", [(F32, BF16), (F32, F16), (BF16, F32), (F16, F32), (F16, BF16), (BF16, F16),
+                                     (F32, F32)])
+@pytest.mark.parametrize("n", [5, 8, 4099, 1 << 18])
+def test_cast_single_rounding(device, src, dst, n):
+    a = round_to_dtype(normal(61, 0, (n,), std=3.0), src)
+    a[:3] = [0.0, 1.0 + 2.0 ** -8, -60000.0][: min(3, n)]  # 1 + 2^-8 is a rounding tie for bf16
+    a = round_to_dtype(a, src)
+    got = _run(device, "CAST", Layout(n), [(a, Layout(n), src)], dst)
+    np.testing.assert_array_equal(got, round_to_dtype(a, dst))
+
+
+CONTIG_CASES = [
+    # shape of the view, strides of the view (elements), size of the backing array
+    ((4, 6), (1, 4), 24),                        # transpose of (6, 4)
+    ((2, 5, 3, 8), (120, 8, 40, 1), 240),        # BHSD buffer read as BSHD: (B,S,H,D) view
+    ((2, 3, 5, 8), (120, 8, 24, 1), 240),        # BSHD buffer read as BHSD
+    ((3, 4, 16), (0, 16, 1), 64),                # broadcast leading dim
+    ((5, 7), (14, 2), 70),                       # every other column
+    ((2, 3, 4), (12, 4, 1), 24),                 # already contiguous
+    ((6,), (3,), 18),
+    ((1, 1), (1, 1), 1),
+]
+
+
+@pytest.mark.parametrize("shape,strides,backing", CONTIG_CASES)
+@pytest.mark.parametrize("dtype", [F32, BF16, I64, I32])
+def test_contiguous_matches_numpy_view(device, shape, strides, backing, dtype):
+    if dtype in (I64, I32):
+        base = integers(62, 0, (backing,), -1000, 1000, np.int64 if dtype == I64 else np.int32)
+    else:
+        base = round_to_dtype(normal(62, 0, (backing,)), dtype)
+    item = base.itemsize
+    want = np.lib.stride_tricks.as_strided(base, shape, tuple(s * item for s in strides))
+    view = Layout(*shape, strides=strides)
+    got = _run(device, "CONTIGUOUS", Layout(*shape), [(base, view, dtype)], dtype)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_contiguous_attention_layout_full_size(device):
+    # O (B, H, S, D) -> (B, S, H, D) at the GPT step's size, bf16
+    B, H, S, D = 64, 6, 256, 64
+    o = round_to_dtype(normal(63, 0, (B, H, S, D)), BF16)
+    view = Layout(B, H, S, D).transpose(1, 2)
+    got = _run(device, "CONTIGUOUS", Layout(B, S, H, D), [(o, view, BF16)], BF16)
+    np.testing.assert_array_equal(got, o.transpose(0, 2, 1, 3))
+
+
+def test_contiguous_rejects_bad_rank(device):
+    buf = AnyBuffer.create(F32, device, 4)
+    with pytest.raises(MogradError):
+        device.lib.mg_contiguous(buf.data_ptr(), buf.data_ptr(), 9, R._i64_array([1] * 9), R._i64_array([1] * 9), F32,
+                                 device.stream)
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("idx_dtype", [I32, I64])
+@pytest.mark.parametrize("V,d,idx_shape", [(65, 384, (4, 33)), (7, 5, (11,)), (1000, 64, (2, 3, 5)), (3, 8, (1,))])
+def test_gather_rows_exact(device, dtype, idx_dtype, V, d, idx_shape):
+    w = round_to_dtype(normal(64, 0, (V, d)), dtype)
+    idx = integers(64, 1, idx_shape, 0, V, np.int32 if idx_dtype == I32 else np.int64)
+    got = _run(device, "GATHER", Layout(*idx_shape, d), [(w, Layout(V, d), dtype), (idx, Layout(*idx_shape), idx_dtype)],
+               dtype)
+    np.testing.assert_array_equal(got, w[idx])
+
+
+def test_gather_strided_source_and_bad_index(device):
+    V, d = 9, 12
+    wt = normal(65, 0, (d, V))  # the source is the transposed view of this array
+    idx = np.array([0, 8, 3, 3, -1, 9], dtype=np.int64)
+    got = _run(device, "GATHER", Layout(6, d), [(wt, Layout(d, V).transpose(), F32), (idx, Layout(6), I64)], F32)
+    np.testing.assert_array_equal(got[:4], wt.T[idx[:4]])
+    assert not got[4:].any()  # out-of-range rows come back as zeros
+    with pytest.raises(MogradError):  # op.mojo:367-368
+        _run(device, "GATHER", Layout(6, d), [(wt, Layout(d * V), F32), (idx, Layout(6), I64)], F32)
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("idx_dtype", [I32, I64])
+@pytest.mark.parametrize("V,d,n", [(65, 384, 4096), (7, 5, 40), (1000, 64, 300), (3, 8, 1), (50, 136, 5000)])
+def test_scatter_add_vs_oracle(device, dtype, idx_dtype, V, d, n):
+    y = round_to_dtype(normal(66, 0, (n, d)), dtype)
+    idx = integers(66, 1, (n,), 0, V, np.int32 if idx_dtype == I32 else np.int64)
+    operands = [(idx, Layout(n), idx_dtype), (y, Layout(n, d), dtype)]
+    got = _run(device, "SCATTER_ADD", Layout(V, d), operands, dtype)
+    want = O.scatter_add(idx, y, V)
+    mass = O.scatter_add(idx, np.abs(y), V)
+    if dtype == F32:
+        assert_sum_close(got, want, mass, what="scatter_add")
+    else:
+        # fp32 accumulation, then one rounding to the 16-bit output
+        eps = 2.0 ** -8 if dtype == BF16 else 2.0 ** -11
+        assert np.all(np.abs(got - want) <= eps * np.abs(want) + 16 * 2.0 ** -24 * mass + 1e-30)
+    again = _run(device, "SCATTER_ADD", Layout(V, d), operands, dtype)
+    np.testing.assert_array_equal(got, again)  # no atomics: bit-identical on every run
+    untouched = np.setdiff1d(np.arange(V), idx)
+    assert not got[untouched].any()
+
+
+def test_scatter_add_ignores_bad_indices_and_checks_rank(device):
+    V, d, n = 5, 8, 6
+    y = normal(67, 0, (n, d))
+    idx = np.array([0, 4, -1, 5, 4, 100], dtype=np.int64)
+    got = _run(device, "SCATTER_ADD", Layout(V, d), [(idx, Layout(n), I64), (y, Layout(n, d), F32)], F32)
+    keep = (idx >= 0) & (idx < V)
+    assert_close(got, O.scatter_add(idx[keep], y[keep], V), RTOL_F32, ATOL_F32, "scatter_add")
+    with pytest.raises(MogradError):  # op.mojo:375-376
+        _run(device, "SCATTER_ADD", Layout(V, d), [(idx, Layout(n), I64), (y, Layout(n * d), F32)], F32)
+
+
+def test_embedding_grad_adjoint_full_size(device):
+    # GPT step size: 16384 tokens, vocab 65, d 384.  <gather(W, i), Y> = <W, scatter_add(i, Y)>
+    # ties the two kernels to each other without a CPU loop over tokens.
+    V, d, n = 65, 384, 16384
+    w = normal(68, 0, (V, d))
+    y = normal(68, 1, (n, d))
+    idx = integers(68, 2, (n,), 0, V, np.int32)
+    g = _run(device, "GATHER", Layout(n, d), [(w, Layout(V, d), F32), (idx, Layout(n), I32)], F32)
+    sa = _run(device, "SCATTER_ADD", Layout(V, d), [(idx, Layout(n), I32), (y, Layout(n, d), F32)], F32)
+    lhs = np.sum(g.astype(np.float64) * y)
+    rhs = np.sum(w.astype(np.float64) * sa)
+    mass = np.sum(np.abs(g.astype(np.float64) * y))
+    assert abs(lhs - rhs) <= RTOL_F32 * abs(lhs) + 16 * 2.0 ** -24 * mass
+    # and the counts: scattering ones gives the histogram of the indices, exactly
+    ones = np.ones((n, 8), np.float32)
+    hist = _run(device, "SCATTER_ADD", Layout(V, 8), [(idx, Layout(n), I32), (ones, Layout(n, 8), F32)], F32)
+    np.testing.assert_array_equal(hist[:, 0], np.bincount(idx, minlength=V).astype(np.float32))
