@@ -1,0 +1,263 @@
+"""One training step (forward, loss, every parameter gradient) of the character-level
+transformer in the reference's examples/tinyshakespear/model.mojo, issued as a fixed
+sequence of libmograd_hip calls on one stream.
+
+    h = embed[ids]                                             model.mojo:22-26
+    per block:  h = h + W_O(attn(W_Q x, W_K x, W_V x, causal)),  x = LN1(h)   :62-64,88-101
+                h = h + W2(relu(W1 x + b1)),                     x = LN2(h)   :120-121
+    logits = lm_head(h);  loss = mean softmax cross-entropy over all tokens
+
+The backward pass is the graph mograd/grad.mojo builds for that forward, with the fused
+entries in place of their unfused chains: mg_linear_bwd for every Linear,
+mg_layer_norm_bwd_stats, mg_flash_attn_bwd, mg_cross_entropy_fused_ids, mg_relu_grad,
+mg_scatter_add for the embedding.
+
+Mixed precision: the parameters live in one fp32 arena (master weights); each step casts
+the whole arena once to the compute dtype (bf16 by default), runs every kernel in that
+dtype with fp32 accumulation, writes the weight gradients into a compute-dtype arena of
+the same layout and casts that once to an fp32 gradient arena.  All activations and
+temporaries are allocated once per (batch, context) shape, so a step performs no
+allocation.  This module contains no arithmetic; there is no CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from typing import Dict, List, Tuple
+
+import numpy as np
+
+from ._lib import BF16, F32, I32, I64, DTYPE_SIZE
+from .runtime import AnyBuffer, Device, MogradError
+
+BLOCK_PARAMS = ("ln1_g", "ln1_b", "wq", "wk", "wv", "wo", "ln2_g", "ln2_b", "w1", "b1", "w2")
+_ALIGN = 64  # elements: every parameter starts on a 128-byte boundary in either arena
+
+
+class _Slice:
+    """A parameter's place in the arenas."""
+
+    __slots__ = ("name", "shape", "offset", "numel")
+
+    def __init__(self, name: str, shape: Tuple[int, ...], offset: int):
+        self.name, self.shape, self.offset = name, shape, offset
+        self.numel = int(np.prod(shape))
+
+
+class TinyTransformer:
+    def __init__(self, device: Device, vocab_size: int, d_model: int, d_ff: int, n_layers: int, n_heads: int,
+                 compute_dtype: int = BF16, eps: float = 1e-5):
+        if d_model % n_heads:
+            raise MogradError(1, "d_model must be a multiple of n_heads")
+        self.device, self.lib, self.stream = device, device.lib, device.stream
+        self.V, self.d, self.ff, self.L, self.H = vocab_size, d_model, d_ff, n_layers, n_heads
+        self.dh = d_model // n_heads
+        self.cd = compute_dtype
+        self.eps = eps
+        self.slices: Dict[str, _Slice] = {}
+        off = 0
+
+        def place(name, shape):
+            nonlocal off
+            self.slices[name] = _Slice(name, shape, off)
+            off += -(-int(np.prod(shape)) // _ALIGN) * _ALIGN
+
+        d, ff, V = d_model, d_ff, vocab_size
+        place("embed", (V, d))
+        block_shapes = {"ln1_g": (d,), "ln1_b": (d,), "wq": (d, d), "wk": (d, d), "wv": (d, d), "wo": (d, d),
+                        "ln2_g": (d,), "ln2_b": (d,), "w1": (ff, d), "b1": (ff,), "w2": (d, ff)}
+        for layer in range(n_layers):
+            for name in BLOCK_PARAMS:
+                place(f"blocks.{layer}.{name}", block_shapes[name])
+        place("lm_head", (V, d))
+        self.total = off
+        self.master = AnyBuffer.create(F32, device, self.total, fill=0.0)  # fp32 master weights
+        self.grads = AnyBuffer.create(F32, device, self.total, fill=0.0)   # fp32 gradients, same layout
+        self.work = AnyBuffer.create(self.cd, device, self.total)          # weights in the compute dtype
+        self.wgrad = AnyBuffer.create(self.cd, device, self.total, fill=0.0)
+        self._plan_key = None
+
+    # ------------------------------------------------------------------ parameters
+
+    def load_params(self, params: dict) -> None:
+        """params: {"embed", "lm_head", "blocks": [{name: array} ...]} (float arrays)."""
+        host = np.zeros(self.total, dtype=np.float32)
+        for name, sl in self.slices.items():
+            host[sl.offset:sl.offset + sl.numel] = np.asarray(self._lookup(params, name), dtype=np.float32).reshape(-1)
+        self.lib.mg_copy_to_device(self.master.data_ptr(), host.ctypes.data_as(C.c_void_p), host.nbytes, self.stream)
+
+    @staticmethod
+    def _lookup(tree: dict, name: str):
+        parts = name.split(".")
+        if parts[0] == "blocks":
+            return tree["blocks"][int(parts[1])][parts[2]]
+        return tree[name]
+
+    def gradients(self) -> dict:
+        """Downloads the fp32 gradient arena as a tree shaped like load_params' argument."""
+        flat = self.grads.to_numpy()
+        out = {"blocks": [dict() for _ in range(self.L)]}
+        for name, sl in self.slices.items():
+            g = flat[sl.offset:sl.offset + sl.numel].reshape(sl.shape).copy()
+            parts = name.split(".")
+            if parts[0] == "blocks":
+                out["blocks"][int(parts[1])][parts[2]] = g
+            else:
+                out[name] = g
+        return out
+
+    def _w(self, name: str) -> C.c_void_p:
+        return C.c_void_p(self.work.storage.ptr + self.slices[name].offset * DTYPE_SIZE[self.cd])
+
+    def _g(self, name: str) -> C.c_void_p:
+        return C.c_void_p(self.wgrad.storage.ptr + self.slices[name].offset * DTYPE_SIZE[self.cd])
+
+    # ------------------------------------------------------------------ workspace
+
+    def _plan(self, B: int, T: int) -> None:
+        if self._plan_key == (B, T):
+            return
+        n, d, ff, V = B * T, self.d, self.ff, self.V
+        dev, cd = self.device, self.cd
+        new = lambda numel, dtype=cd: AnyBuffer.create(dtype, dev, numel)
+        self.h = [new(n * d) for _ in range(self.L + 1)]  # residual stream entering each block, and the last
+        self.saved: List[dict] = []
+        for _ in range(self.L):
+            self.saved.append({
+                "x1": new(n * d), "q": new(n * d), "k": new(n * d), "v": new(n * d), "o": new(n * d),
+                "lse": new(B * self.H * T, F32), "ctx": new(n * d),
+                "h_mid": new(n * d), "x2": new(n * d), "a": new(n * ff),
+                "mean1": new(n, F32), "rstd1": new(n, F32), "mean2": new(n, F32), "rstd2": new(n, F32),
+            })
+        self.tmp = {name: new(n * d) for name in ("proj", "dh", "dres", "dctx", "do", "dq", "dk", "dv", "dx_a", "dx_b",
+                                                  "dx_c")}
+        self.tmp["da"] = new(n * ff)
+        self.tmp["logits"] = new(n * V)
+        self.tmp["dlogits"] = new(n * V)
+        self.loss = new(1)
+        self._plan_key = (B, T)
+
+    # ------------------------------------------------------------------ one step
+
+    def step(self, ids: AnyBuffer, labels: AnyBuffer, B: int, T: int, marks=None) -> AnyBuffer:
+        """Runs forward, loss and backward for `ids`/`labels` ((B, T) int32 or int64 device
+        buffers).  Returns the loss buffer (one element, compute dtype); the fp32 gradients
+        are in `self.grads`.  Nothing is synchronised.  `marks`, if given, is called with
+        "forward" and "backward" at the boundaries (for event timing)."""
+        if ids.dtype not in (I32, I64) or labels.dtype not in (I32, I64):
+            raise MogradError(1, "ids and labels must be int32 or int64")
+        if ids.numel != B * T or labels.numel != B * T:
+            raise MogradError(1, "ids/labels do not match (B, T)")
+        self._plan(B, T)
+        lib, s, cd = self.lib, self.stream, self.cd
+        n, d, ff, V, H, dh = B * T, self.d, self.ff, self.V, self.H, self.dh
+        scale = 1.0 / math.sqrt(dh)
+        i64 = lambda *v: (C.c_int64 * len(v))(*v)
+
+        def linear(x, w, out, N, K, bias=None):  # out(n, N) = x(n, K) w(N, K)^T (+ bias)
+            if bias is None:
+                lib.mg_matmul_bt(x, w, out, 1, n, N, K, K, 1, K, 1, n * K, N * K, cd, s)
+            else:
+                lib.mg_matmul_bias_bt(x, w, bias, out, 1, n, N, K, K, 1, K, 1, n * K, N * K, cd, s)
+
+        P = lambda buf: buf.data_ptr()
+
+        lib.mg_cast(P(self.master), P(self.work), self.total, F32, cd, s)
+
+        # ---- forward
+        lib.mg_gather(self._w("embed"), P(ids), P(self.h[0]), n, V, d, d, 1, ids.dtype, cd, s)
+        for l in range(self.L):
+            c, w = self.saved[l], (lambda name, l=l: self._w(f"blocks.{l}.{name}"))
+            h_in, h_out = P(self.h[l]), P(self.h[l + 1])
+            lib.mg_layer_norm_fwd_stats(h_in, w("ln1_g"), w("ln1_b"), P(c["x1"]), P(c["mean1"]), P(c["rstd1"]), n, d,
+                                        self.eps, cd, s)
+            linear(P(c["x1"]), w("wq"), P(c["q"]), d, d)
+            linear(P(c["x1"]), w("wk"), P(c["k"]), d, d)
+            linear(P(c["x1"]), w("wv"), P(c["v"]), d, d)
+            # (n, d) row-major is (B, T, H, dh): the layout the attention kernels take for Q, K, V
+            lib.mg_flash_attn_fwd(P(c["q"]), P(c["k"]), P(c["v"]), None, P(c["o"]), P(c["lse"]), B, T, H, dh, scale, 1,
+                                  0, cd, s)
+            # O comes back (B, H, T, dh); the projection wants (B, T, H*dh)
+            lib.mg_contiguous(P(c["o"]), P(c["ctx"]), 4, i64(B, T, H, dh), i64(H * T * dh, dh, T * dh, 1), cd, s)
+            linear(P(c["ctx"]), w("wo"), P(self.tmp["proj"]), d, d)
+            lib.mg_add(h_in, P(self.tmp["proj"]), P(c["h_mid"]), n * d, cd, s)
+            lib.mg_layer_norm_fwd_stats(P(c["h_mid"]), w("ln2_g"), w("ln2_b"), P(c["x2"]), P(c["mean2"]),
+                                        P(c["rstd2"]), n, d, self.eps, cd, s)
+            linear(P(c["x2"]), w("w1"), P(c["a"]), ff, d, bias=w("b1"))
+            lib.mg_relu(P(c["a"]), P(c["a"]), n * ff, cd, s)
+            linear(P(c["a"]), w("w2"), P(self.tmp["proj"]), d, ff)
+            lib.mg_add(P(c["h_mid"]), P(self.tmp["proj"]), h_out, n * d, cd, s)
+        linear(P(self.h[self.L]), self._w("lm_head"), P(self.tmp["logits"]), V, d)
+        lib.mg_cross_entropy_fused_ids(P(self.tmp["logits"]), P(labels), None, P(self.loss), P(self.tmp["dlogits"]), n,
+                                       V, cd, labels.dtype, s)
+        if marks:
+            marks("forward")
+
+        # ---- backward
+        t = {k: P(v) for k, v in self.tmp.items()}
+        lib.mg_linear_bwd(t["dlogits"], P(self.h[self.L]), self._w("lm_head"), t["dh"], self._g("lm_head"), None, n, V,
+                          d, cd, s)
+        for l in reversed(range(self.L)):
+            c = self.saved[l]
+            w = lambda name, l=l: self._w(f"blocks.{l}.{name}")
+            g = lambda name, l=l: self._g(f"blocks.{l}.{name}")
+            # h_out = h_mid + W2 a
+            lib.mg_linear_bwd(t["dh"], P(c["a"]), w("w2"), t["da"], g("w2"), None, n, d, ff, cd, s)
+            lib.mg_relu_grad(P(c["a"]), t["da"], t["da"], n * ff, cd, s)
+            lib.mg_linear_bwd(t["da"], P(c["x2"]), w("w1"), t["dx_a"], g("w1"), g("b1"), n, ff, d, cd, s)
+            lib.mg_layer_norm_bwd_stats(t["dx_a"], P(c["h_mid"]), w("ln2_g"), P(c["mean2"]), P(c["rstd2"]), t["dres"],
+                                        g("ln2_g"), g("ln2_b"), n, d, cd, s)
+            lib.mg_add(t["dh"], t["dres"], t["dh"], n * d, cd, s)
+            # h_mid = h_in + W_O ctx
+            lib.mg_linear_bwd(t["dh"], P(c["ctx"]), w("wo"), t["dctx"], g("wo"), None, n, d, d, cd, s)
+            # dctx is (B, T, H, dh); the attention backward takes dO as (B, H, T, dh)
+            lib.mg_contiguous(t["dctx"], t["do"], 4, i64(B, H, T, dh), i64(T * H * dh, dh, H * dh, 1), cd, s)
+            lib.mg_flash_attn_bwd(t["do"], P(c["o"]), P(c["q"]), P(c["k"]), P(c["v"]), None, P(c["lse"]), t["dq"],
+                                  t["dk"], t["dv"], B, T, H, dh, scale, 1, 0, cd, s)
+            lib.mg_linear_bwd(t["dq"], P(c["x1"]), w("wq"), t["dx_a"], g("wq"), None, n, d, d, cd, s)
+            lib.mg_linear_bwd(t["dk"], P(c["x1"]), w("wk"), t["dx_b"], g("wk"), None, n, d, d, cd, s)
+            lib.mg_linear_bwd(t["dv"], P(c["x1"]), w("wv"), t["dx_c"], g("wv"), None, n, d, d, cd, s)
+            lib.mg_add(t["dx_a"], t["dx_b"], t["dx_a"], n * d, cd, s)
+            lib.mg_add(t["dx_a"], t["dx_c"], t["dx_a"], n * d, cd, s)
+            lib.mg_layer_norm_bwd_stats(t["dx_a"], P(self.h[l]), w("ln1_g"), P(c["mean1"]), P(c["rstd1"]), t["dres"],
+                                        g("ln1_g"), g("ln1_b"), n, d, cd, s)
+            lib.mg_add(t["dh"], t["dres"], t["dh"], n * d, cd, s)
+        lib.mg_scatter_add(P(ids), t["dh"], self._g("embed"), n, V, d, ids.dtype, cd, s)
+        lib.mg_cast(P(self.wgrad), P(self.grads), self.total, cd, F32, s)
+        if marks:
+            marks("backward")
+        return self.loss
+
+    # ------------------------------------------------------------------ bookkeeping
+
+    def flops_per_step(self, B: int, T: int) -> float:
+        """Matmul and attention FLOPs of one forward+backward, counted the usual way:
+        2mnk per product, 3 products per Linear (forward, dX, dW), and for causal
+        attention half of 4*B*H*T^2*dh forward plus 2.5 times that backward."""
+        n, d, ff, V = B * T, self.d, self.ff, self.V
+        per_block = 4 * d * d + 2 * d * ff
+        linear = 3 * 2 * n * (self.L * per_block + V * d)
+        attn_fwd = 0.5 * 4 * B * self.H * T * T * self.dh
+        return linear + self.L * 3.5 * attn_fwd
+
+
+def init_params(rng: np.random.Generator, vocab_size: int, d_model: int, d_ff: int, n_layers: int) -> dict:
+    """Random parameters with the reference's initialisers: Embedding ~ N(0, 1)
+    (nn/modules/embedding.mojo:23-29), Linear weight and bias ~ U(+-sqrt(6 / fan_in))
+    (nn/modules/linear.mojo:29-47), LayerNorm gamma 1, beta 0."""
+    def lin(o, i):
+        b = math.sqrt(6.0 / i)
+        return rng.uniform(-b, b, size=(o, i)).astype(np.float32)
+
+    d, ff = d_model, d_ff
+    blocks = []
+    for _ in range(n_layers):
+        blocks.append({
+            "ln1_g": np.ones(d, np.float32), "ln1_b": np.zeros(d, np.float32),
+            "wq": lin(d, d), "wk": lin(d, d), "wv": lin(d, d), "wo": lin(d, d),
+            "ln2_g": np.ones(d, np.float32), "ln2_b": np.zeros(d, np.float32),
+            "w1": lin(ff, d), "b1": rng.uniform(-math.sqrt(6.0 / d), math.sqrt(6.0 / d), ff).astype(np.float32),
+            "w2": lin(d, ff),
+        })
+    return {"embed": rng.standard_normal((vocab_size, d)).astype(np.float32), "lm_head": lin(vocab_size, d),
+            "blocks": blocks}

@@ -390,13 +390,18 @@ def scatter_add(indices, values, num_rows):
 # --------------------------------------------------------------------------- #
 
 
-def tiny_transformer_step(params, ids, labels, n_heads, eps=1e-5):
+def tiny_transformer_step(params, ids, labels, n_heads, eps=1e-5, store=None):
     """Returns (loss, grads) with grads shaped like params.
 
     params = {"embed": (V, d), "lm_head": (V, d), "blocks": [ {"ln1_g","ln1_b","wq","wk",
     "wv","wo" (d, d), "ln2_g","ln2_b","w1" (ff, d),"b1" (ff),"w2" (d, ff)} ... ]};
     ids, labels: (B, T) integers.  model.mojo:22-26,62-64,88-101,120-121.
+
+    `store`, if given, is applied to every tensor an op of the graph writes to memory
+    (each activation, each gradient); passing the rounding of a 16-bit storage type
+    reproduces where a reduced-precision run rounds, the arithmetic staying float64.
     """
+    r = (lambda a: a) if store is None else (lambda a: np.asarray(store(a), dtype=F64))
     ids = np.asarray(ids, dtype=np.int64)
     labels = np.asarray(labels, dtype=np.int64)
     B, T = ids.shape
@@ -408,50 +413,53 @@ def tiny_transformer_step(params, ids, labels, n_heads, eps=1e-5):
     saved = []
     for blk in params["blocks"]:
         c = {"h_in": h}
-        c["x1"] = layer_norm_fwd(h, blk["ln1_g"], blk["ln1_b"], eps)
-        q = matmul_bias_bt(c["x1"], blk["wq"]).reshape(B, T, n_heads, dh)
-        k = matmul_bias_bt(c["x1"], blk["wk"]).reshape(B, T, n_heads, dh)
-        v = matmul_bias_bt(c["x1"], blk["wv"]).reshape(B, T, n_heads, dh)
+        c["x1"] = r(layer_norm_fwd(h, blk["ln1_g"], blk["ln1_b"], eps))
+        q = r(matmul_bias_bt(c["x1"], blk["wq"])).reshape(B, T, n_heads, dh)
+        k = r(matmul_bias_bt(c["x1"], blk["wk"])).reshape(B, T, n_heads, dh)
+        v = r(matmul_bias_bt(c["x1"], blk["wv"])).reshape(B, T, n_heads, dh)
         o, _ = sdpa_fwd(q, k, v, causal=True)  # BHSD
+        o = r(o)
         c["q"], c["k"], c["v"] = q, k, v
         c["ctx"] = o.transpose(0, 2, 1, 3).reshape(n, d)
-        h = h + matmul_bias_bt(c["ctx"], blk["wo"])
+        h = r(h + r(matmul_bias_bt(c["ctx"], blk["wo"])))
         c["h_mid"] = h
-        c["x2"] = layer_norm_fwd(h, blk["ln2_g"], blk["ln2_b"], eps)
-        c["a"] = relu(matmul_bias_bt(c["x2"], blk["w1"], blk["b1"]))
-        h = h + matmul_bias_bt(c["a"], blk["w2"])
+        c["x2"] = r(layer_norm_fwd(h, blk["ln2_g"], blk["ln2_b"], eps))
+        c["a"] = relu(r(matmul_bias_bt(c["x2"], blk["w1"], blk["b1"])))
+        h = r(h + r(matmul_bias_bt(c["a"], blk["w2"])))
         saved.append(c)
-    logits = matmul_bias_bt(h, params["lm_head"])
+    logits = r(matmul_bias_bt(h, params["lm_head"]))
     flat_labels = labels.reshape(-1)
     loss = cross_entropy_ids(logits, flat_labels)
-    dlogits = cross_entropy_grad_ids(logits, flat_labels, 1.0)
+    dlogits = r(cross_entropy_grad_ids(logits, flat_labels, 1.0))
 
-    grads = {"lm_head": linear_grad_w(dlogits, h), "blocks": []}
-    dh_ = linear_grad_x(dlogits, params["lm_head"])
+    grads = {"lm_head": r(linear_grad_w(dlogits, h)), "blocks": []}
+    dh_ = r(linear_grad_x(dlogits, params["lm_head"]))
     for blk, c in zip(reversed(params["blocks"]), reversed(saved)):
         g = {}
         # h = h_mid + W2 a
-        g["w2"] = linear_grad_w(dh_, c["a"])
-        da = relu_grad(c["a"], linear_grad_x(dh_, blk["w2"]))
-        g["w1"] = linear_grad_w(da, c["x2"])
-        g["b1"] = linear_grad_b(da)
-        dx2 = linear_grad_x(da, blk["w1"])
-        dmid, g["ln2_g"], g["ln2_b"] = layer_norm_bwd(dx2, c["h_mid"], blk["ln2_g"], eps)
-        dh_ = dh_ + dmid
+        g["w2"] = r(linear_grad_w(dh_, c["a"]))
+        da = relu_grad(c["a"], r(linear_grad_x(dh_, blk["w2"])))
+        g["w1"] = r(linear_grad_w(da, c["x2"]))
+        g["b1"] = r(linear_grad_b(da))
+        dx2 = r(linear_grad_x(da, blk["w1"]))
+        dmid, dg, db = layer_norm_bwd(dx2, c["h_mid"], blk["ln2_g"], eps)
+        g["ln2_g"], g["ln2_b"] = r(dg), r(db)
+        dh_ = r(dh_ + r(dmid))
         # h_mid = h_in + W_O ctx
-        g["wo"] = linear_grad_w(dh_, c["ctx"])
-        dctx = linear_grad_x(dh_, blk["wo"])
+        g["wo"] = r(linear_grad_w(dh_, c["ctx"]))
+        dctx = r(linear_grad_x(dh_, blk["wo"]))
         do = dctx.reshape(B, T, n_heads, dh).transpose(0, 2, 1, 3)  # BHSD
         dq, dk, dv = sdpa_bwd(c["q"], c["k"], c["v"], do, causal=True)
-        dq, dk, dv = (t.reshape(n, d) for t in (dq, dk, dv))
-        g["wq"] = linear_grad_w(dq, c["x1"])
-        g["wk"] = linear_grad_w(dk, c["x1"])
-        g["wv"] = linear_grad_w(dv, c["x1"])
-        dx1 = linear_grad_x(dq, blk["wq"]) + linear_grad_x(dk, blk["wk"]) + linear_grad_x(dv, blk["wv"])
-        din, g["ln1_g"], g["ln1_b"] = layer_norm_bwd(dx1, c["h_in"], blk["ln1_g"], eps)
-        dh_ = dh_ + din
+        dq, dk, dv = (r(t).reshape(n, d) for t in (dq, dk, dv))
+        g["wq"] = r(linear_grad_w(dq, c["x1"]))
+        g["wk"] = r(linear_grad_w(dk, c["x1"]))
+        g["wv"] = r(linear_grad_w(dv, c["x1"]))
+        dx1 = r(r(r(linear_grad_x(dq, blk["wq"])) + r(linear_grad_x(dk, blk["wk"]))) + r(linear_grad_x(dv, blk["wv"])))
+        din, dg, db = layer_norm_bwd(dx1, c["h_in"], blk["ln1_g"], eps)
+        g["ln1_g"], g["ln1_b"] = r(dg), r(db)
+        dh_ = r(dh_ + r(din))
         grads["blocks"].insert(0, g)
-    grads["embed"] = scatter_add(ids.reshape(-1), dh_, V)
+    grads["embed"] = r(scatter_add(ids.reshape(-1), dh_, V))
     return float(loss), grads
 
 
