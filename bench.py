@@ -370,13 +370,205 @@ def bench_attention(args, dev) -> int:
     return 0
 
 
+def bench_gpt(args, dev) -> int:
+    """Character-level GPT training step (examples/tinyshakespear/model.mojo shape): vocab 65, context 256,
+    batch 64, 6 layers, d_model 384, 6 heads, MLP 4x, pre-LayerNorm, bf16 activations with fp32 master weights,
+    token ids uniform in [0, 65); forward, loss and every parameter gradient."""
+    from mograd_amd import BF16, F32, I32, AnyBuffer
+    from mograd_amd.tiny_transformer import TinyTransformer, init_params
+
+    lib, st = dev.lib, dev.stream
+    V, d, ff, L, H, B, T = 65, 384, 1536, 6, 6, 64, 256
+    n, dh = B * T, d // H
+    model = TinyTransformer(dev, V, d, ff, L, H, compute_dtype=BF16)
+    model.load_params(init_params(_rng(5, 0), V, d, ff, L))
+    ids = AnyBuffer.from_numpy(dev, _rng(5, 1).integers(0, V, (B, T)).astype(np.int32))
+    labels = AnyBuffer.from_numpy(dev, _rng(5, 2).integers(0, V, (B, T)).astype(np.int32))
+
+    ms = _time_steps(dev, lambda i: model.step(ids, labels, B, T), args.warmup, args.steps)
+    loss = model.loss.item()
+
+    # forward / backward split, from events recorded on the library's stream inside the step
+    iters = max(5, min(args.steps, 20))
+    ev = [[C.c_void_p() for _ in range(3)] for _ in range(iters)]
+    for row in ev:
+        for e in row:
+            lib.mg_event_create(C.byref(e))
+    for row in ev:
+        lib.mg_event_record(row[0], st)
+        model.step(ids, labels, B, T, marks=lambda which, row=row: lib.mg_event_record(row[1 if which == "forward" else 2], st))
+    dev.synchronize()
+    fwd_ms, bwd_ms = [], []
+    for row in ev:
+        a, b = C.c_float(), C.c_float()
+        lib.mg_event_elapsed_ms(row[0], row[1], C.byref(a))
+        lib.mg_event_elapsed_ms(row[1], row[2], C.byref(b))
+        fwd_ms.append(a.value)
+        bwd_ms.append(b.value)
+        for e in row:
+            lib.mg_event_destroy(e)
+
+    # per-kernel table at the step's shapes
+    P = lambda b: b.data_ptr()  # noqa: E731
+    new = lambda numel, dt=BF16: AnyBuffer.create(dt, dev, numel)  # noqa: E731
+    rnd = lambda numel, k: AnyBuffer.from_numpy(dev, _rng(5, 10 + k).standard_normal(numel, dtype=np.float32), BF16)  # noqa: E731
+    x_d, x_ff, dy_d, dy_ff = rnd(n * d, 0), rnd(n * ff, 1), rnd(n * d, 2), rnd(n * ff, 3)
+    w_dd, w_fd, w_df, w_vd = rnd(d * d, 4), rnd(ff * d, 5), rnd(d * ff, 6), rnd(V * d, 7)
+    bias_f, gam, bet = rnd(ff, 8), rnd(d, 9), rnd(d, 10)
+    out_d, out_ff, out_v, dlog = new(n * d), new(n * ff), new(n * V), new(n * V)
+    dw_big, db_big, dgam, dbet = new(ff * d), new(ff), new(d), new(d)
+    mean, rstd, lse, loss1 = new(n, F32), new(n, F32), new(B * H * T, F32), new(1)
+    q, k, v, o, do, dq, dk, dv = rnd(n * d, 11), rnd(n * d, 12), rnd(n * d, 13), new(n * d), rnd(n * d, 14), new(n * d), new(n * d), new(n * d)
+    i64 = lambda *a: (C.c_int64 * len(a))(*a)  # noqa: E731
+    sc = 1.0 / float(np.sqrt(dh))
+    lib.mg_layer_norm_fwd_stats(P(x_d), P(gam), P(bet), P(out_d), P(mean), P(rstd), n, d, 1e-5, BF16, st)
+    lib.mg_flash_attn_fwd(P(q), P(k), P(v), None, P(o), P(lse), B, T, H, dh, sc, 1, 0, BF16, st)
+    lib.mg_matmul_bt(P(x_d), P(w_vd), P(out_v), 1, n, V, d, d, 1, d, 1, n * d, V * d, BF16, st)
+
+    def mm(x, w, out, N, K, bias=None):
+        if bias is None:
+            return lambda i: lib.mg_matmul_bt(P(x), P(w), P(out), 1, n, N, K, K, 1, K, 1, n * K, N * K, BF16, st)
+        return lambda i: lib.mg_matmul_bias_bt(P(x), P(w), P(bias), P(out), 1, n, N, K, K, 1, K, 1, n * K, N * K, BF16, st)
+
+    def lbwd(dy, x, w, dx, N, K, db=None):
+        return lambda i: lib.mg_linear_bwd(P(dy), P(x), P(w), P(dx), P(dw_big), P(db) if db else None, n, N, K, BF16, st)
+
+    PF = MFMA_BF16_PEAK_TFLOPS
+    e2 = 2  # bytes per bf16
+    attn_fl = B * H * T * T * dh
+    entries = [
+        ("linear_bwd dX+dW bf16 (16384, 384<-384)", lbwd(dy_d, x_d, w_dd, out_d, d, d), 4.0 * n * d * d, "F", PF),
+        ("linear_bwd dX+dW+db bf16 (16384, 1536<-384)", lbwd(dy_ff, x_d, w_fd, out_d, ff, d, db_big), 4.0 * n * d * ff, "F", PF),
+        ("linear_bwd dX+dW bf16 (16384, 384<-1536)", lbwd(dy_d, x_ff, w_df, out_ff, d, ff), 4.0 * n * d * ff, "F", PF),
+        ("linear_bwd dX+dW bf16 lm_head (16384, 65<-384)", lbwd(dlog, x_d, w_vd, out_d, V, d), 4.0 * n * d * V, "F", PF),
+        ("matmul_bt bf16 (16384, 384<-384)", mm(x_d, w_dd, out_d, d, d), 2.0 * n * d * d, "F", PF),
+        ("matmul_bias_bt bf16 (16384, 1536<-384)", mm(x_d, w_fd, out_ff, ff, d, bias_f), 2.0 * n * d * ff, "F", PF),
+        ("matmul_bt bf16 (16384, 384<-1536)", mm(x_ff, w_df, out_d, d, ff), 2.0 * n * d * ff, "F", PF),
+        ("matmul_bt bf16 lm_head (16384, 65<-384)", mm(x_d, w_vd, out_v, V, d), 2.0 * n * d * V, "F", PF),
+        ("flash_attn_bwd bf16 causal B64 H6 S256 D64 (5 B H S^2 D)",
+         lambda i: lib.mg_flash_attn_bwd(P(do), P(o), P(q), P(k), P(v), None, P(lse), P(dq), P(dk), P(dv), B, T, H, dh, sc, 1, 0, BF16, st),
+         5.0 * attn_fl, "F", PF),
+        ("flash_attn_fwd bf16 causal B64 H6 S256 D64 (2 B H S^2 D)",
+         lambda i: lib.mg_flash_attn_fwd(P(q), P(k), P(v), None, P(o), P(lse), B, T, H, dh, sc, 1, 0, BF16, st), 2.0 * attn_fl, "F", PF),
+        ("layer_norm_bwd_stats bf16 (16384, 384)",
+         lambda i: lib.mg_layer_norm_bwd_stats(P(dy_d), P(x_d), P(gam), P(mean), P(rstd), P(out_d), P(dgam), P(dbet), n, d, BF16, st),
+         3 * n * d * e2 + 2 * n * 4 + 3 * d * e2, "B", None),
+        ("layer_norm_fwd_stats bf16 (16384, 384)",
+         lambda i: lib.mg_layer_norm_fwd_stats(P(x_d), P(gam), P(bet), P(out_d), P(mean), P(rstd), n, d, 1e-5, BF16, st),
+         2 * n * d * e2 + 2 * n * 4 + 2 * d * e2, "B", None),
+        ("cross_entropy_fused_ids bf16 (16384, 65)",
+         lambda i: lib.mg_cross_entropy_fused_ids(P(out_v), P(labels), None, P(loss1), P(dlog), n, V, BF16, I32, st),
+         2 * n * V * e2 + n * 4 + e2, "B", None),
+        ("add bf16 (16384 x 384)", lambda i: lib.mg_add(P(x_d), P(dy_d), P(out_d), n * d, BF16, st), 3 * n * d * e2, "B", None),
+        ("relu bf16 (16384 x 1536)", lambda i: lib.mg_relu(P(x_ff), P(out_ff), n * ff, BF16, st), 2 * n * ff * e2, "B", None),
+        ("relu_grad bf16 (16384 x 1536)", lambda i: lib.mg_relu_grad(P(x_ff), P(dy_ff), P(out_ff), n * ff, BF16, st), 3 * n * ff * e2, "B", None),
+        ("contiguous bf16 (B,H,T,dh) -> (B,T,H,dh)",
+         lambda i: lib.mg_contiguous(P(o), P(out_d), 4, i64(B, T, H, dh), i64(H * T * dh, dh, T * dh, 1), BF16, st), 2 * n * d * e2, "B", None),
+        ("gather bf16 16384 rows of (65, 384)", lambda i: lib.mg_gather(P(w_vd), P(ids), P(out_d), n, V, d, d, 1, I32, BF16, st),
+         n * d * e2 + n * 4, "B", None),
+        ("scatter_add bf16 16384 rows into (65, 384)", lambda i: lib.mg_scatter_add(P(ids), P(dy_d), P(dw_big), n, V, d, I32, BF16, st),
+         n * d * e2 + n * 4 + V * d * e2, "B", None),
+        ("cast fp32 -> bf16 parameter arena", lambda i: lib.mg_cast(P(model.master), P(model.work), model.total, F32, BF16, st),
+         model.total * 6, "B", None),
+    ]
+    kernels = _kernel_table(dev, entries, max(10, min(args.steps, 30)))
+    flops = model.flops_per_step(B, T)
+    tf = flops / (ms * 1e-3) / 1e12
+    result = {
+        "metric": "fwd+bwd step ms; per-bwd-kernel HBM GB/s or MFMA % of MI355X peak", "value": round(ms, 4),
+        "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "char-level GPT training step: vocab 65, ctx 256, batch 64, 6 layers, d_model 384, 6 heads, "
+                               "MLP 4x, pre-LayerNorm, bf16 activations / fp32 master weights, ids uniform in [0,65); "
+                               "forward + loss + all parameter gradients",
+                   "tokens_per_step": n, "loss": round(loss, 4)},
+        "phases_ms": {"forward": round(float(np.mean(fwd_ms)), 4), "backward": round(float(np.mean(bwd_ms)), 4)},
+        "roofline": {"bound": "mfma", "kernel": "whole step (matmul and attention FLOPs of forward + backward)",
+                     "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "algorithmic_flops": flops},
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = _gpt_cpu_baseline(V, d, ff, L, H, B, T)
+    print(json.dumps(result))
+    return 0
+
+
+def _gpt_cpu_baseline(V, d, ff, L, H, B, T):
+    """fp32 C restatement of one transformer block (forward + backward) on 4 of the 64 sequences, scaled by
+    16 x 6 layers; embedding, lm_head and the loss (under 2% of the work) are left out."""
+    orc = _orc()
+    cores = int(orc.orc_num_threads())
+    p = lambda a: a.ctypes.data_as(C.c_void_p)  # noqa: E731
+    Li, F = C.c_int64, C.c_float
+    Bs = 4
+    n, dh = Bs * T, d // H
+    r = lambda k, *shape: _rng(5, 100 + k).standard_normal(shape, dtype=np.float32)  # noqa: E731
+    x, dy = r(0, n, d), r(1, n, d)
+    g, be = np.ones(d, np.float32), np.zeros(d, np.float32)
+    w = {name: r(2 + i, *shape) * 0.05 for i, (name, shape) in enumerate(
+        [("wq", (d, d)), ("wk", (d, d)), ("wv", (d, d)), ("wo", (d, d)), ("w1", (ff, d)), ("w2", (d, ff))])}
+    b1 = np.zeros(ff, np.float32)
+    e = lambda *shape: np.empty(shape, np.float32)  # noqa: E731
+    x1, q, k, v, o, ctx, proj, hmid, x2, a, f = e(n, d), e(n, d), e(n, d), e(n, d), e(n, d), e(n, d), e(n, d), e(n, d), e(n, d), e(n, ff), e(n, d)
+    lse = e(Bs * H * T)
+    da, dxa, dxb, dxc, dres, dq, dk, dv, dctx = e(n, ff), e(n, d), e(n, d), e(n, d), e(n, d), e(n, d), e(n, d), e(n, d), e(n, d)
+    dw_dd, dw_fd, dw_df, db1, dg, db = e(d, d), e(ff, d), e(d, ff), e(ff), e(d), e(d)
+
+    def lin(xi, wi, bi, yi, N, K):
+        orc.orc_matmul_bias_bt_f32(p(xi), p(wi), p(bi) if bi is not None else None, p(yi), Li(n), Li(N), Li(K))
+
+    def lin_bwd(dyi, xi, wi, dxi, dwi, N, K, dbi=None):
+        orc.orc_linear_grad_x_f32(p(dyi), p(wi), p(dxi), Li(n), Li(N), Li(K))
+        orc.orc_linear_grad_w_f32(p(dyi), p(xi), p(dwi), Li(n), Li(N), Li(K))
+        if dbi is not None:
+            orc.orc_linear_grad_b_f32(p(dyi), p(dbi), Li(n), Li(N))
+
+    def block():
+        orc.orc_layer_norm_fwd_f32(p(x), p(g), p(be), p(x1), Li(n), Li(d), F(1e-5))
+        lin(x1, w["wq"], None, q, d, d)
+        lin(x1, w["wk"], None, k, d, d)
+        lin(x1, w["wv"], None, v, d, d)
+        orc.orc_sdpa_fwd_f32(p(q), p(k), p(v), None, 0, 1, p(o), p(lse), Li(Bs), Li(T), Li(H), Li(dh), F(0.125), Li(Bs * H))
+        ctx[:] = o.reshape(Bs, H, T, dh).transpose(0, 2, 1, 3).reshape(n, d)
+        lin(ctx, w["wo"], None, proj, d, d)
+        np.add(x, proj, out=hmid)
+        orc.orc_layer_norm_fwd_f32(p(hmid), p(g), p(be), p(x2), Li(n), Li(d), F(1e-5))
+        lin(x2, w["w1"], b1, a, ff, d)
+        np.maximum(a, 0, out=a)
+        lin(a, w["w2"], None, f, d, ff)
+        # backward
+        lin_bwd(dy, a, w["w2"], da, dw_df, d, ff)
+        orc.orc_relu_grad_f32(p(a), p(da), p(da), Li(n * ff))
+        lin_bwd(da, x2, w["w1"], dxa, dw_fd, ff, d, db1)
+        orc.orc_layer_norm_bwd_f32(p(dxa), p(hmid), p(g), p(dres), p(dg), p(db), Li(n), Li(d), F(1e-5), Li(256))
+        lin_bwd(dres, ctx, w["wo"], dctx, dw_dd, d, d)
+        do = np.ascontiguousarray(dctx.reshape(Bs, T, H, dh).transpose(0, 2, 1, 3))
+        orc.orc_sdpa_bwd_f32(p(q), p(k), p(v), p(do), None, 0, 1, p(dq), p(dk), p(dv), Li(Bs), Li(T), Li(H), Li(dh), F(0.125), Li(Bs * H))
+        lin_bwd(dq, x1, w["wq"], dxa, dw_dd, d, d)
+        lin_bwd(dk, x1, w["wk"], dxb, dw_dd, d, d)
+        lin_bwd(dv, x1, w["wv"], dxc, dw_dd, d, d)
+        np.add(dxa, dxb, out=dxa)
+        np.add(dxa, dxc, out=dxa)
+        orc.orc_layer_norm_bwd_f32(p(dxa), p(x), p(g), p(dres), p(dg), p(db), Li(n), Li(d), F(1e-5), Li(256))
+
+    block()
+    t0 = time.perf_counter()
+    block()
+    one = (time.perf_counter() - t0) * 1e3
+    scale_up = (B // Bs) * L
+    return {"value": round(one * scale_up, 1), "unit": "ms", "cores": cores, "kind": "port",
+            "sample": f"one transformer block fwd+bwd in fp32 on {Bs} of {B} sequences ({one:.1f} ms) scaled x{scale_up} "
+                      f"(16 batch slices x {L} layers); embedding, lm_head and loss left out; OpenMP on {cores} threads"}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
-    ap.add_argument("--workload", choices=["ln_ce", "mlp", "attention"], default="ln_ce",
+    ap.add_argument("--workload", choices=["ln_ce", "mlp", "attention", "gpt"], default="ln_ce",
                     help="ln_ce (default): the configuration the metric is quoted on; mlp: README MLP fwd+bwd fp32 "
                          "(matmul_bias_bt, dX, dW, db); attention: bf16 flash attention fwd+bwd")
     args = ap.parse_args()
@@ -392,6 +584,8 @@ def main() -> int:
     st = dev.stream
     if args.workload == "mlp":
         return bench_mlp(args, dev)
+    if args.workload == "gpt":
+        return bench_gpt(args, dev)
     if args.workload == "attention":
         return bench_attention(args, dev)
 
