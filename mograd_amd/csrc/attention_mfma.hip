@@ -193,10 +193,14 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
   __shared__ __attribute__((aligned(16))) uint32_t v_tr[DP * tr_stride_dw<BN>()];
 
   const int nqb = (a.S + BM - 1) / BM;
-  // Causal: later query blocks have more keys to visit; launch them first.
-  const int qb = CAUSAL ? nqb - 1 - blockIdx.x % nqb : blockIdx.x % nqb;
-  const int h = (blockIdx.x / nqb) % a.H;
-  const int b = blockIdx.x / (nqb * a.H);
+  // Consecutive workgroups go to different XCDs, so the (batch, head) index varies fastest:
+  // every XCD then gets the same mix of query blocks, and the blocks of one (batch, head)
+  // share one XCD's L2 when B*H is a multiple of the XCD count.  Causal: later query
+  // blocks visit more keys; all of them launch first.
+  const int n_bh = a.B * a.H;
+  const int qb = CAUSAL ? nqb - 1 - blockIdx.x / n_bh : blockIdx.x / n_bh;
+  const int h = (blockIdx.x % n_bh) % a.H;
+  const int b = (blockIdx.x % n_bh) / a.H;
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int half = lane / 32;
@@ -342,9 +346,11 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
   __shared__ __attribute__((aligned(16))) uint32_t k_tr[DP * tr_stride_dw<BN>()];
 
   const int nqb = (a.S + BM - 1) / BM;
-  const int qb = CAUSAL ? nqb - 1 - blockIdx.x % nqb : blockIdx.x % nqb;
-  const int h = (blockIdx.x / nqb) % a.H;
-  const int b = blockIdx.x / (nqb * a.H);
+  // (batch, head) varies fastest across consecutive workgroups, heaviest query blocks first.
+  const int n_bh = a.B * a.H;
+  const int qb = CAUSAL ? nqb - 1 - blockIdx.x / n_bh : blockIdx.x / n_bh;
+  const int h = (blockIdx.x % n_bh) % a.H;
+  const int b = (blockIdx.x % n_bh) / a.H;
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int half = lane / 32;
@@ -484,10 +490,12 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
   __shared__ __attribute__((aligned(16))) float delta_s[BQ];
 
   const int nkb = (a.S + BNK - 1) / BNK;
-  // Causal: earlier key blocks are seen by more queries; they already come first.
-  const int kb = blockIdx.x % nkb;
-  const int h = (blockIdx.x / nkb) % a.H;
-  const int b = blockIdx.x / (nkb * a.H);
+  // (batch, head) varies fastest across consecutive workgroups.  Causal: earlier key blocks
+  // are seen by more queries; all of them launch first.
+  const int n_bh = a.B * a.H;
+  const int kb = blockIdx.x / n_bh;
+  const int h = (blockIdx.x % n_bh) % a.H;
+  const int b = (blockIdx.x % n_bh) / a.H;
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int half = lane / 32;

@@ -63,8 +63,8 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
   const int64_t cus = device_info().cu_count;
   int splits = 1;
   if (g.batch == 1 && blocks < cus && g.K >= 1024) {
-    splits = static_cast<int>(ceil_div(2 * cus, blocks));
-    const int max_splits = static_cast<int>(g.K / 256);
+    splits = static_cast<int>(ceil_div(env_int("MOGRAD_HIP_GEMM_SPLITK_WG_PER_CU", 2) * cus, blocks));
+    const int max_splits = static_cast<int>(g.K / env_int("MOGRAD_HIP_GEMM_SPLITK_MIN_K", 256));
     if (splits > max_splits) splits = max_splits;
     if (splits > 64) splits = 64;
   }
