@@ -681,6 +681,48 @@ static int fwd_typed(const void* q, const void* k, const void* v, const void* ma
   return MG_OK;
 }
 
+// delta[row] = sum_d dO[row, d] * O[row, d] for contiguous rows of D = 8 * CPR elements, CPR a
+// power of two: one 16-byte chunk of each tensor per thread, then a sum over the CPR
+// neighbouring lanes that share a row.
+template <typename T, int CPR>
+__global__ __launch_bounds__(256) void attn_delta_rows_kernel(const T* __restrict__ d_o, const T* __restrict__ o,
+                                                              float* __restrict__ delta, int64_t rows) {
+  const int64_t chunk = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  const int64_t row = chunk / CPR;
+  float acc = 0.f;
+  if (row < rows) {
+    float x[8], y[8];
+    VecIO<T, 8>::load(d_o + chunk * 8, x);
+    VecIO<T, 8>::load(o + chunk * 8, y);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc = fmaf(x[e], y[e], acc);
+  }
+#pragma unroll
+  for (int w = 1; w < CPR; w *= 2) acc += __shfl_xor(acc, w);
+  if (row < rows && threadIdx.x % CPR == 0) delta[row] = acc;
+}
+
+template <typename T>
+static int launch_delta(const T* d_o, const T* o, float* delta, int64_t rows, int D, hipStream_t stream) {
+  const int cpr = D / 8;
+  const bool vec = D % 8 == 0 && (cpr & (cpr - 1)) == 0 && cpr <= 16;
+  if (vec) {
+    const dim3 grid(static_cast<unsigned>(ceil_div(rows * cpr, 256)));
+    switch (cpr) {
+      case 1: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 1>), grid, dim3(256), 0, stream, d_o, o, delta, rows); break;
+      case 2: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 2>), grid, dim3(256), 0, stream, d_o, o, delta, rows); break;
+      case 4: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 4>), grid, dim3(256), 0, stream, d_o, o, delta, rows); break;
+      case 8: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 8>), grid, dim3(256), 0, stream, d_o, o, delta, rows); break;
+      default: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 16>), grid, dim3(256), 0, stream, d_o, o, delta, rows); break;
+    }
+  } else {
+    hipLaunchKernelGGL((attn_delta_kernel<T>), dim3(static_cast<unsigned>(ceil_div(rows, 4))), dim3(256), 0, stream, d_o,
+                       o, delta, rows, D);
+  }
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
 template <typename T, int DP>
 static int bwd_typed(const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
                      const float* lse, void* dq, void* dk, void* dv, AttnDims a, float scale, bool causal, bool has_bias,
@@ -688,9 +730,7 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
   const int64_t rows = static_cast<int64_t>(a.B) * a.H * a.S;
   Scratch delta;
   MG_TRY(delta.take(rows * static_cast<int64_t>(sizeof(float))));
-  hipLaunchKernelGGL((attn_delta_kernel<T>), dim3(static_cast<unsigned>(ceil_div(rows, 4))), dim3(256), 0, stream,
-                     static_cast<const T*>(d_o), static_cast<const T*>(o), delta.as<float>(), rows, a.D);
-  MG_LAUNCH_CHECK();
+  MG_TRY(launch_delta(static_cast<const T*>(d_o), static_cast<const T*>(o), delta.as<float>(), rows, a.D, stream));
   const int64_t blocks = static_cast<int64_t>(a.B) * a.H * ceil_div(a.S, 128);
   // dQ: two query tiles per wave when the head dimension leaves registers for it and
   // there are still enough workgroups to fill the device.
