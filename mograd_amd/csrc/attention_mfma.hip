@@ -47,6 +47,9 @@ struct Mma<bf16_t> {
     const float2_t v = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
   }
+  static __device__ __forceinline__ float2_t unpack2(uint32_t w) {
+    return __builtin_convertvector(__builtin_bit_cast(bf16x2_t, w), float2_t);
+  }
 };
 template <>
 struct Mma<f16_t> {
@@ -58,7 +61,32 @@ struct Mma<f16_t> {
     const float2_t v = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
   }
+  static __device__ __forceinline__ float2_t unpack2(uint32_t w) {
+    return __builtin_convertvector(__builtin_bit_cast(f16x2_t, w), float2_t);
+  }
 };
+
+// Eight packed elements times `f`, rounded back to T.  Used once per workgroup to fold the
+// softmax scale (times log2 e) into the resident operand of the score product, so that the
+// product comes out of the matrix core already in the exponent's units.
+template <typename T>
+__device__ __forceinline__ uint4 scale_frag(uint4 v, float f) {
+  const uint32_t in[4] = {v.x, v.y, v.z, v.w};
+  uint32_t out[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float2_t x = Mma<T>::unpack2(in[i]);
+    out[i] = Mma<T>::pack2(x[0] * f, x[1] * f);
+  }
+  return make_uint4(out[0], out[1], out[2], out[3]);
+}
+
+__device__ __forceinline__ floatx16 splat16(float v) {
+  floatx16 z;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) z[r] = v;
+  return z;
+}
 
 constexpr int kAttnThreads = 256;
 
@@ -360,9 +388,14 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
   const T* vbase = v + bshd(a, b, 0, h);
   const int64_t bh = static_cast<int64_t>(b) * a.H + h;
 
+  // Q is held pre-multiplied by scale * log2(e), and the score and dP products start from
+  // accumulators holding -lse (log2 units) and -delta, this lane's query being the same
+  // for every tile: the matrix core then delivers S*c - lse and dP - delta directly.
+  const float c = scale * kAttnLog2e;
   int m[MQ];
   uint4 qf[MQ][KS], dof[MQ][KS];
   float lse2[MQ], dl[MQ];
+  floatx16 s_init[MQ], dp_init[MQ];
   const T* mrow[MQ];
   floatx16 acc[MQ][DT];
 #pragma unroll
@@ -373,16 +406,18 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
       const int d = ks * 16 + half * 8;
       const bool ok = m[mq] < a.S && d < a.D;
       qf[mq][ks] = ok ? *reinterpret_cast<const uint4*>(q + bshd(a, b, m[mq], h) + d) : make_uint4(0, 0, 0, 0);
+      qf[mq][ks] = scale_frag<T>(qf[mq][ks], c);
       dof[mq][ks] = ok ? *reinterpret_cast<const uint4*>(d_o + bhsd(a, b, h, m[mq]) + d) : make_uint4(0, 0, 0, 0);
     }
     // Rows past the end get lse = +inf so that their probabilities vanish.
     lse2[mq] = m[mq] < a.S ? lse[bh * a.S + m[mq]] * kAttnLog2e : INFINITY;
     dl[mq] = m[mq] < a.S ? delta[bh * a.S + m[mq]] : 0.f;
     mrow[mq] = HAS_BIAS ? mask + (bh * a.S + min(m[mq], a.S - 1)) * a.S : nullptr;
+    s_init[mq] = splat16(-lse2[mq]);
+    dp_init[mq] = splat16(-dl[mq]);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[mq][dt] = zero16();
   }
-  const float c = scale * kAttnLog2e;
 
   const int n_end = CAUSAL ? min(a.S, qb * BM + BM) : a.S;
   TileStager<T, BN, DP> ks_stage, vs_stage;
@@ -407,8 +442,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
       floatx16 s[MQ], dp[MQ];
 #pragma unroll
       for (int mq = 0; mq < MQ; ++mq) {
-        s[mq] = zero16();
-        dp[mq] = zero16();
+        s[mq] = s_init[mq];
+        dp[mq] = dp_init[mq];
       }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
@@ -426,18 +461,18 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
         const bool plain = !HAS_BIAS && nb + 32 <= a.S && (!CAUSAL || nb + 31 <= m_wave + mq * 32);
         if (plain) {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) s[mq][r] = fexp2(fmaf(s[mq][r], c, -lse2[mq])) * (dp[mq][r] - dl[mq]);
+          for (int r = 0; r < 16; ++r) s[mq][r] = fexp2(s[mq][r]) * dp[mq][r];
         } else {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int n = nb + acc_row(r, lane);
             bool valid = n < a.S;
             if (CAUSAL) valid = valid && n <= m[mq];
-            float sv = s[mq][r] * c;
+            float sv = s[mq][r];
             if (HAS_BIAS) sv = fmaf(to_float(mrow[mq][min(n, a.S - 1)]), kAttnLog2e, sv);
-            float p = fexp2(sv - lse2[mq]);
+            float p = fexp2(sv);
             p = valid ? p : 0.f;
-            s[mq][r] = p * (dp[mq][r] - dl[mq]);  // dS^T
+            s[mq][r] = p * dp[mq][r];  // dS^T
           }
         }
       }
@@ -512,6 +547,9 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
     const int d = ks * 16 + half * 8;
     const bool ok = n < a.S && d < a.D;
     kf[ks] = ok ? *reinterpret_cast<const uint4*>(k + bshd(a, b, n, h) + d) : make_uint4(0, 0, 0, 0);
+    // K is held pre-multiplied by scale * log2(e): the score product then comes out in the
+    // exponent's units.  (dK is formed from the unscaled Q tile, so nothing else changes.)
+    kf[ks] = scale_frag<T>(kf[ks], scale * kAttnLog2e);
     vf[ks] = ok ? *reinterpret_cast<const uint4*>(v + bshd(a, b, n, h) + d) : make_uint4(0, 0, 0, 0);
   }
   floatx16 acc_k[DT], acc_v[DT];
@@ -520,7 +558,6 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
     acc_k[dt] = zero16();
     acc_v[dt] = zero16();
   }
-  const float c = scale * kAttnLog2e;
 
   // Causal: queries before the workgroup's first key see none of its keys.
   const int m_begin = CAUSAL ? (kb * BNK / BQ) * BQ : 0;
@@ -539,8 +576,10 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
     do_stage.commit_rows(do_rows);
     do_stage.commit_transposed(do_tr);
     if (threadIdx.x < BQ) {
-      lse_s[threadIdx.x] = lse_next;  // rows past the end carry lse = +inf, delta = 0
-      delta_s[threadIdx.x] = delta_next;
+      // Stored negated: they initialise the accumulators of the S and dP products.  Rows
+      // past the end carry -lse = -inf (their probabilities vanish) and delta = 0.
+      lse_s[threadIdx.x] = -lse_next;
+      delta_s[threadIdx.x] = -delta_next;
     }
     __syncthreads();
     if (m0 + BQ < a.S) {
@@ -564,7 +603,16 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
     // the exponentials run) so that no MFMA waits on an LDS read it has just issued.
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      floatx16 s = zero16(), dp = zero16();
+      // Accumulators start at -lse and -delta of their rows (register r <-> query row
+      // (r/4)*8 + half*4 + r%4): the products deliver S*c - lse and dP - delta.
+      floatx16 s, dp;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const float4 l4 = *reinterpret_cast<const float4*>(&lse_s[mt * 32 + g * 8 + half * 4]);
+        const float4 d4 = *reinterpret_cast<const float4*>(&delta_s[mt * 32 + g * 8 + half * 4]);
+        s[g * 4 + 0] = l4.x; s[g * 4 + 1] = l4.y; s[g * 4 + 2] = l4.z; s[g * 4 + 3] = l4.w;
+        dp[g * 4 + 0] = d4.x; dp[g * 4 + 1] = d4.y; dp[g * 4 + 2] = d4.z; dp[g * 4 + 3] = d4.w;
+      }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         s = Mma<T>::run(frag_rows<DP>(q_rows, mt, ks, lane), kf[ks], s);
@@ -583,45 +631,29 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
       __builtin_amdgcn_sched_barrier(0);
       if (plain) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const float4 l4 = *reinterpret_cast<const float4*>(&lse_s[mt * 32 + g * 8 + half * 4]);
-          const float4 d4 = *reinterpret_cast<const float4*>(&delta_s[mt * 32 + g * 8 + half * 4]);
-          const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
-          const float dv4[4] = {d4.x, d4.y, d4.z, d4.w};
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const int r = g * 4 + j;
-            const float p = fexp2(fmaf(s[r], c, -lv[j]));
-            s[r] = p;
-            dp[r] = p * (dp[r] - dv4[j]);
-          }
+        for (int r = 0; r < 16; ++r) {
+          const float p = fexp2(s[r]);
+          s[r] = p;
+          dp[r] = p * dp[r];
         }
       } else {
         // Same arithmetic on every element, then a select: no per-element branches.
         const bool col_ok = n < a.S;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const float4 l4 = *reinterpret_cast<const float4*>(&lse_s[mt * 32 + g * 8 + half * 4]);
-          const float4 d4 = *reinterpret_cast<const float4*>(&delta_s[mt * 32 + g * 8 + half * 4]);
-          const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
-          const float dv4[4] = {d4.x, d4.y, d4.z, d4.w};
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const int r = g * 4 + j;
-            const int mm = m0 + mt * 32 + g * 8 + half * 4 + j;
-            bool valid = col_ok;
-            if (CAUSAL) valid = valid && n <= mm;
-            float sv = s[r] * c;
-            if (HAS_BIAS) {
-              // clamped address: always in bounds, the value is discarded when invalid
-              const int64_t mi = (bh * a.S + min(mm, a.S - 1)) * a.S + min(n, a.S - 1);
-              sv = fmaf(to_float(mask[mi]), kAttnLog2e, sv);
-            }
-            float p = fexp2(sv - lv[j]);  // rows past the end carry lse = +inf: p = 0
-            p = valid ? p : 0.f;
-            s[r] = p;
-            dp[r] = p * (dp[r] - dv4[j]);
+        for (int r = 0; r < 16; ++r) {
+          const int mm = m0 + mt * 32 + acc_row(r, lane);
+          bool valid = col_ok;
+          if (CAUSAL) valid = valid && n <= mm;
+          float sv = s[r];
+          if (HAS_BIAS) {
+            // clamped address: always in bounds, the value is discarded when invalid
+            const int64_t mi = (bh * a.S + min(mm, a.S - 1)) * a.S + min(n, a.S - 1);
+            sv = fmaf(to_float(mask[mi]), kAttnLog2e, sv);
           }
+          float p = fexp2(sv);  // rows past the end started from -inf: p = 0
+          p = valid ? p : 0.f;
+          s[r] = p;
+          dp[r] = p * dp[r];
         }
       }
 #pragma unroll
