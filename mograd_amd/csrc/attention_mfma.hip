@@ -517,12 +517,14 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
   constexpr int BNK = 128;                 // keys per workgroup
   constexpr int BQ = DP <= 64 ? 64 : 32;   // queries per step (LDS budget)
   constexpr int MT = BQ / 32, KS = DP / 16, DT = DP / 32;
-  __shared__ __attribute__((aligned(16))) uint16_t q_rows[BQ * row_stride<DP>()];
-  __shared__ __attribute__((aligned(16))) uint16_t do_rows[BQ * row_stride<DP>()];
-  __shared__ __attribute__((aligned(16))) uint32_t q_tr[DP * tr_stride_dw<BQ>()];
-  __shared__ __attribute__((aligned(16))) uint32_t do_tr[DP * tr_stride_dw<BQ>()];
-  __shared__ __attribute__((aligned(16))) float lse_s[BQ];
-  __shared__ __attribute__((aligned(16))) float delta_s[BQ];
+  // Two copies of every staged tile: step i computes from copy i % 2 while the tile of step
+  // i + 1 is written into the other, so one barrier per step suffices.
+  __shared__ __attribute__((aligned(16))) uint16_t q_rows_s[2][BQ * row_stride<DP>()];
+  __shared__ __attribute__((aligned(16))) uint16_t do_rows_s[2][BQ * row_stride<DP>()];
+  __shared__ __attribute__((aligned(16))) uint32_t q_tr_s[2][DP * tr_stride_dw<BQ>()];
+  __shared__ __attribute__((aligned(16))) uint32_t do_tr_s[2][DP * tr_stride_dw<BQ>()];
+  __shared__ __attribute__((aligned(16))) float lse_ss[2][BQ];
+  __shared__ __attribute__((aligned(16))) float delta_ss[2][BQ];
 
   const int nkb = (a.S + BNK - 1) / BNK;
   // (batch, head) varies fastest across consecutive workgroups.  Causal: earlier key blocks
@@ -562,36 +564,48 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
   // Causal: queries before the workgroup's first key see none of its keys.
   const int m_begin = CAUSAL ? (kb * BNK / BQ) * BQ : 0;
   TileStager<T, BQ, DP> q_stage, do_stage;
-  q_stage.fetch(qbase, ld, m_begin, a.S, a.D);
-  do_stage.fetch(dobase, a.D, m_begin, a.S, a.D);
-  float lse_next = INFINITY, delta_next = 0.f;
-  if (threadIdx.x < BQ && m_begin + threadIdx.x < a.S) {
-    lse_next = lse[bh * a.S + m_begin + threadIdx.x] * kAttnLog2e;
-    delta_next = delta[bh * a.S + m_begin + threadIdx.x];
-  }
-  for (int m0 = m_begin; m0 < a.S; m0 += BQ) {
-    __syncthreads();
-    q_stage.commit_rows(q_rows);
-    q_stage.commit_transposed(q_tr);
-    do_stage.commit_rows(do_rows);
-    do_stage.commit_transposed(do_tr);
+  float lse_next, delta_next;
+  // Global -> registers for the step starting at query m.
+  auto fetch_step = [&](int m) {
+    q_stage.fetch(qbase, ld, m, a.S, a.D);
+    do_stage.fetch(dobase, a.D, m, a.S, a.D);
+    lse_next = INFINITY;
+    delta_next = 0.f;
+    if (threadIdx.x < BQ && m + threadIdx.x < a.S) {
+      lse_next = lse[bh * a.S + m + threadIdx.x] * kAttnLog2e;
+      delta_next = delta[bh * a.S + m + threadIdx.x];
+    }
+  };
+  // Registers -> LDS copy `buf`.
+  auto commit_step = [&](int buf) {
+    q_stage.commit_rows(q_rows_s[buf]);
+    q_stage.commit_transposed(q_tr_s[buf]);
+    do_stage.commit_rows(do_rows_s[buf]);
+    do_stage.commit_transposed(do_tr_s[buf]);
     if (threadIdx.x < BQ) {
       // Stored negated: they initialise the accumulators of the S and dP products.  Rows
       // past the end carry -lse = -inf (their probabilities vanish) and delta = 0.
-      lse_s[threadIdx.x] = -lse_next;
-      delta_s[threadIdx.x] = -delta_next;
+      lse_ss[buf][threadIdx.x] = -lse_next;
+      delta_ss[buf][threadIdx.x] = -delta_next;
     }
+  };
+  fetch_step(m_begin);
+  commit_step(0);
+  if (m_begin + BQ < a.S) fetch_step(m_begin + BQ);
+  int cur = 0;
+  for (int m0 = m_begin; m0 < a.S; m0 += BQ, cur ^= 1) {
+    // Copy `cur` is complete and every wave has finished reading the other copy.
     __syncthreads();
     if (m0 + BQ < a.S) {
-      q_stage.fetch(qbase, ld, m0 + BQ, a.S, a.D);
-      do_stage.fetch(dobase, a.D, m0 + BQ, a.S, a.D);
-      lse_next = INFINITY;
-      delta_next = 0.f;
-      if (threadIdx.x < BQ && m0 + BQ + threadIdx.x < a.S) {
-        lse_next = lse[bh * a.S + m0 + BQ + threadIdx.x] * kAttnLog2e;
-        delta_next = delta[bh * a.S + m0 + BQ + threadIdx.x];
-      }
+      commit_step(cur ^ 1);
+      if (m0 + 2 * BQ < a.S) fetch_step(m0 + 2 * BQ);
     }
+    const uint16_t* q_rows = q_rows_s[cur];
+    const uint16_t* do_rows = do_rows_s[cur];
+    const uint32_t* q_tr = q_tr_s[cur];
+    const uint32_t* do_tr = do_tr_s[cur];
+    const float* lse_s = lse_ss[cur];
+    const float* delta_s = delta_ss[cur];
     if (CAUSAL && m0 + BQ - 1 < n_wave) continue;  // all of this step's queries precede the wave's keys
 
     // Per-element masking is needed only for key columns past the end and where the step
