@@ -81,6 +81,13 @@ __device__ __forceinline__ uint4 scale_frag(uint4 v, float f) {
   return make_uint4(out[0], out[1], out[2], out[3]);
 }
 
+// Makes a fragment loaded from global memory before a loop count as "arrived" at this
+// point.  Without it the compiler's wait-count bookkeeping treats the load as possibly
+// still in flight at the loop header and waits for *all* outstanding global loads at the
+// fragment's first use inside the loop, which also drains the tile prefetch issued a few
+// instructions earlier.
+__device__ __forceinline__ void settle(uint4& v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
+
 __device__ __forceinline__ floatx16 splat16(float v) {
   floatx16 z;
 #pragma unroll
@@ -243,6 +250,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
   for (int ks = 0; ks < KS; ++ks) {
     const int d = ks * 16 + half * 8;
     qf[ks] = (m < a.S && d < a.D) ? *reinterpret_cast<const uint4*>(q + bshd(a, b, m, h) + d) : make_uint4(0, 0, 0, 0);
+    settle(qf[ks]);
   }
   floatx16 acc_o[DT];
 #pragma unroll
@@ -408,6 +416,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
       qf[mq][ks] = ok ? *reinterpret_cast<const uint4*>(q + bshd(a, b, m[mq], h) + d) : make_uint4(0, 0, 0, 0);
       qf[mq][ks] = scale_frag<T>(qf[mq][ks], c);
       dof[mq][ks] = ok ? *reinterpret_cast<const uint4*>(d_o + bhsd(a, b, h, m[mq]) + d) : make_uint4(0, 0, 0, 0);
+      settle(dof[mq][ks]);
     }
     // Rows past the end get lse = +inf so that their probabilities vanish.
     lse2[mq] = m[mq] < a.S ? lse[bh * a.S + m[mq]] * kAttnLog2e : INFINITY;
@@ -553,6 +562,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
     // exponent's units.  (dK is formed from the unscaled Q tile, so nothing else changes.)
     kf[ks] = scale_frag<T>(kf[ks], scale * kAttnLog2e);
     vf[ks] = ok ? *reinterpret_cast<const uint4*>(v + bshd(a, b, n, h) + d) : make_uint4(0, 0, 0, 0);
+    settle(vf[ks]);
   }
   floatx16 acc_k[DT], acc_v[DT];
 #pragma unroll
@@ -572,7 +582,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
     lse_next = INFINITY;
     delta_next = 0.f;
     if (threadIdx.x < BQ && m + threadIdx.x < a.S) {
-      lse_next = lse[bh * a.S + m + threadIdx.x] * kAttnLog2e;
+      lse_next = lse[bh * a.S + m + threadIdx.x];  // scaled to log2 units when it is committed
       delta_next = delta[bh * a.S + m + threadIdx.x];
     }
   };
@@ -585,7 +595,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
     if (threadIdx.x < BQ) {
       // Stored negated: they initialise the accumulators of the S and dP products.  Rows
       // past the end carry -lse = -inf (their probabilities vanish) and delta = 0.
-      lse_ss[buf][threadIdx.x] = -lse_next;
+      lse_ss[buf][threadIdx.x] = -lse_next * kAttnLog2e;
       delta_ss[buf][threadIdx.x] = -delta_next;
     }
   };
