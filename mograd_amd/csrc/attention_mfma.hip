@@ -224,8 +224,10 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
                                                                         const T* __restrict__ mask, T* __restrict__ o,
                                                                         float* __restrict__ lse, AttnDims a, float scale) {
   constexpr int BM = 128, BN = 64, KS = DP / 16, DT = DP / 32;
-  __shared__ __attribute__((aligned(16))) uint16_t k_rows[BN * row_stride<DP>()];
-  __shared__ __attribute__((aligned(16))) uint32_t v_tr[DP * tr_stride_dw<BN>()];
+  // Two copies of each staged tile: step i computes from copy i % 2 while the tile of step
+  // i + 1 is written into the other, so one barrier per step suffices.
+  __shared__ __attribute__((aligned(16))) uint16_t k_rows_s[2][BN * row_stride<DP>()];
+  __shared__ __attribute__((aligned(16))) uint32_t v_tr_s[2][DP * tr_stride_dw<BN>()];
 
   const int nqb = (a.S + BM - 1) / BM;
   // Consecutive workgroups go to different XCDs, so the (batch, head) index varies fastest:
@@ -263,15 +265,26 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
   TileStager<T, BN, DP> ks_stage, vs_stage;
   ks_stage.fetch(kbase, ld, 0, a.S, a.D);
   vs_stage.fetch(vbase, ld, 0, a.S, a.D);
-  for (int n0 = 0; n0 < n_end; n0 += BN) {
-    __syncthreads();
-    ks_stage.commit_rows(k_rows);
-    vs_stage.commit_transposed(v_tr);
+  ks_stage.commit_rows(k_rows_s[0]);
+  vs_stage.commit_transposed(v_tr_s[0]);
+  if (BN < n_end) {
+    ks_stage.fetch(kbase, ld, BN, a.S, a.D);
+    vs_stage.fetch(vbase, ld, BN, a.S, a.D);
+  }
+  int cur = 0;
+  for (int n0 = 0; n0 < n_end; n0 += BN, cur ^= 1) {
+    // Copy `cur` is complete and every wave has finished reading the other copy.
     __syncthreads();
     if (n0 + BN < n_end) {
-      ks_stage.fetch(kbase, ld, n0 + BN, a.S, a.D);
-      vs_stage.fetch(vbase, ld, n0 + BN, a.S, a.D);
+      ks_stage.commit_rows(k_rows_s[cur ^ 1]);
+      vs_stage.commit_transposed(v_tr_s[cur ^ 1]);
+      if (n0 + 2 * BN < n_end) {
+        ks_stage.fetch(kbase, ld, n0 + 2 * BN, a.S, a.D);
+        vs_stage.fetch(vbase, ld, n0 + 2 * BN, a.S, a.D);
+      }
     }
+    const uint16_t* k_rows = k_rows_s[cur];
+    const uint32_t* v_tr = v_tr_s[cur];
     if (CAUSAL && n0 > m_wave + 31) continue;  // every key of the block is in this wave's future
 
     floatx16 s[2];
@@ -377,9 +390,10 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
                                                                        const float* __restrict__ delta,
                                                                        T* __restrict__ dq, AttnDims a, float scale) {
   constexpr int BM = 128 * MQ, BN = 64, KS = DP / 16, DT = DP / 32;
-  __shared__ __attribute__((aligned(16))) uint16_t k_rows[BN * row_stride<DP>()];
-  __shared__ __attribute__((aligned(16))) uint16_t v_rows[BN * row_stride<DP>()];
-  __shared__ __attribute__((aligned(16))) uint32_t k_tr[DP * tr_stride_dw<BN>()];
+  // Two copies of each staged tile: one barrier per step.
+  __shared__ __attribute__((aligned(16))) uint16_t k_rows_s[2][BN * row_stride<DP>()];
+  __shared__ __attribute__((aligned(16))) uint16_t v_rows_s[2][BN * row_stride<DP>()];
+  __shared__ __attribute__((aligned(16))) uint32_t k_tr_s[2][DP * tr_stride_dw<BN>()];
 
   const int nqb = (a.S + BM - 1) / BM;
   // (batch, head) varies fastest across consecutive workgroups, heaviest query blocks first.
@@ -432,16 +446,29 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
   TileStager<T, BN, DP> ks_stage, vs_stage;
   ks_stage.fetch(kbase, ld, 0, a.S, a.D);
   vs_stage.fetch(vbase, ld, 0, a.S, a.D);
-  for (int n0 = 0; n0 < n_end; n0 += BN) {
-    __syncthreads();
-    ks_stage.commit_rows(k_rows);
-    ks_stage.commit_transposed(k_tr);
-    vs_stage.commit_rows(v_rows);
+  ks_stage.commit_rows(k_rows_s[0]);
+  ks_stage.commit_transposed(k_tr_s[0]);
+  vs_stage.commit_rows(v_rows_s[0]);
+  if (BN < n_end) {
+    ks_stage.fetch(kbase, ld, BN, a.S, a.D);
+    vs_stage.fetch(vbase, ld, BN, a.S, a.D);
+  }
+  int cur = 0;
+  for (int n0 = 0; n0 < n_end; n0 += BN, cur ^= 1) {
+    // Copy `cur` is complete and every wave has finished reading the other copy.
     __syncthreads();
     if (n0 + BN < n_end) {
-      ks_stage.fetch(kbase, ld, n0 + BN, a.S, a.D);
-      vs_stage.fetch(vbase, ld, n0 + BN, a.S, a.D);
+      ks_stage.commit_rows(k_rows_s[cur ^ 1]);
+      ks_stage.commit_transposed(k_tr_s[cur ^ 1]);
+      vs_stage.commit_rows(v_rows_s[cur ^ 1]);
+      if (n0 + 2 * BN < n_end) {
+        ks_stage.fetch(kbase, ld, n0 + 2 * BN, a.S, a.D);
+        vs_stage.fetch(vbase, ld, n0 + 2 * BN, a.S, a.D);
+      }
     }
+    const uint16_t* k_rows = k_rows_s[cur];
+    const uint16_t* v_rows = v_rows_s[cur];
+    const uint32_t* k_tr = k_tr_s[cur];
     if (CAUSAL && n0 > m_wave + 32 * MQ - 1) continue;  // every key of the block is in this wave's future
 
     // One 32-key tile at a time: S^T and dP^T for all MQ query tiles, dS^T in place, then
