@@ -448,6 +448,44 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
     __syncthreads();
   }
 
+  // Output.  The accumulators have lanes along n and registers along m, so a direct store
+  // writes 2-byte elements.  When rows of C can be written 16 bytes at a time, each wave
+  // instead transposes its 64x64 tile through its own quarter of the (now idle) staging
+  // memory and stores eight elements per lane.
+  if constexpr (!SPLIT_K) {
+    const bool wide_out = (N % 8 == 0) && (ldc % 8 == 0) && (bsc % 8 == 0) && (reinterpret_cast<uintptr_t>(C) % 16 == 0);
+    if (wide_out) {
+      uint16_t* mine = (wave < 2 ? lds_a : lds_b) + (wave % 2) * 64 * kG16Stride;
+#pragma unroll
+      for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+        for (int tj = 0; tj < 2; ++tj) {
+          const int cl = tj * 32 + lane % 32;
+          const int col = n0 + wn + cl;
+          const float bv = (HAS_BIAS && col < N) ? to_float(bias[col]) : 0.f;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int rl = ti * 32 + (r / 4) * 8 + (lane / 32) * 4 + (r % 4);
+            const T v = from_float<T>(acc[ti][tj][r] + bv);
+            mine[rl * kG16Stride + cl] = __builtin_bit_cast(uint16_t, v);
+          }
+        }
+      __syncthreads();
+      T* cbase = C + batch * bsc;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int chunk = lane + i * kWave;
+        const int rl = chunk / 8, ch = chunk % 8;
+        const int row = m0 + wm + rl;
+        const int col = n0 + wn + ch * 8;
+        if (row < M && col < N) {
+          const uint4 v = *reinterpret_cast<const uint4*>(mine + rl * kG16Stride + ch * 8);
+          *reinterpret_cast<uint4*>(cbase + static_cast<int64_t>(row) * ldc + col) = v;
+        }
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
