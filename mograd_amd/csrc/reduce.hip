@@ -5,39 +5,47 @@
 
 namespace mg {
 
-// Stage 1 of dst(o, i) = sum_r a(o, r, i): each workgroup sums a slab of `rows_per_chunk`
-// rows for 256 * VEC columns with 16-byte loads.  DIRECT writes the final value (one
-// slab covers the whole axis); otherwise fp32 partials (outer, chunks, inner) go to
-// scratch and reduce_partials_kernel finishes in a fixed order.  No atomics.
+// Stage 1 of dst(o, i) = sum_r a(o, r, i): a workgroup is TX column threads by 256 / TX row
+// lanes; a thread sums every (256 / TX)-th row of its slab for VEC columns with 16-byte
+// loads (narrow matrices get more row lanes instead of idle column threads).  DIRECT writes
+// the final value (one slab, one row lane); otherwise fp32 partials
+// (outer, slab * row_lanes + lane, inner) go to scratch and reduce_partials_kernel finishes
+// in a fixed order.  No atomics.
 template <typename T, int VEC, bool DIRECT>
 __global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict__ a, float* __restrict__ part,
                                                              T* __restrict__ dst, int64_t reduce, int64_t inner,
-                                                             int64_t rows_per_chunk) {
-  const int64_t col = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * VEC;
+                                                             int64_t rows_per_chunk, int tx_log2) {
+  const int tx = 1 << tx_log2;
+  const int ry = 256 >> tx_log2;
+  const int cx = threadIdx.x & (tx - 1);
+  const int ly = threadIdx.x >> tx_log2;
+  const int64_t col = (static_cast<int64_t>(blockIdx.x) * tx + cx) * VEC;
   if (col >= inner) return;
   const int64_t chunk = blockIdx.y;
   const int64_t o = blockIdx.z;
-  const int64_t r0 = chunk * rows_per_chunk;
-  const int64_t r1 = min(r0 + rows_per_chunk, reduce);
+  const int64_t r0 = chunk * rows_per_chunk + ly;
+  const int64_t r1 = min(chunk * rows_per_chunk + rows_per_chunk, reduce);
   const T* base = a + (o * reduce) * inner + col;
+  const int64_t step = static_cast<int64_t>(ry) * inner;  // elements between this thread's rows
   float acc[4][VEC];
 #pragma unroll
   for (int u = 0; u < 4; ++u)
 #pragma unroll
     for (int e = 0; e < VEC; ++e) acc[u][e] = 0.f;
   int64_t r = r0;
-  for (; r + 3 < r1; r += 4) {
+  const T* p = base + r0 * inner;
+  for (; r + 3 * ry < r1; r += 4 * ry, p += 4 * step) {
     float v[4][VEC];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) VecIO<T, VEC>::load(base + (r + u) * inner, v[u]);
+    for (int u = 0; u < 4; ++u) VecIO<T, VEC>::load(p + u * step, v[u]);
 #pragma unroll
     for (int u = 0; u < 4; ++u)
 #pragma unroll
       for (int e = 0; e < VEC; ++e) acc[u][e] += v[u][e];
   }
-  for (; r < r1; ++r) {
+  for (; r < r1; r += ry, p += step) {
     float v[VEC];
-    VecIO<T, VEC>::load(base + r * inner, v);
+    VecIO<T, VEC>::load(p, v);
 #pragma unroll
     for (int e = 0; e < VEC; ++e) acc[0][e] += v[e];
   }
@@ -47,9 +55,9 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict
   if constexpr (DIRECT) {
     VecIO<T, VEC>::store(dst + o * inner + col, out);
   } else {
-    float* p = part + (o * gridDim.y + chunk) * inner + col;
+    float* q = part + ((o * gridDim.y + chunk) * ry + ly) * inner + col;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) p[e] = out[e];
+    for (int e = 0; e < VEC; ++e) q[e] = out[e];
   }
 }
 
@@ -100,41 +108,46 @@ static int colsum_typed(const T* a, T* dst, int64_t outer, int64_t reduce, int64
   constexpr int WIDE = WideVec<T>::value;
   const bool wide = inner % WIDE == 0 && aligned16(a) && aligned16(dst);
   const int vec = wide ? WIDE : 1;
-  const int64_t col_blocks = ceil_div(inner, 256 * vec);
+  // Column threads per workgroup: the smallest power of two covering the columns, at most 256.
+  int tx_log2 = 3;
+  while (tx_log2 < 8 && (int64_t{1} << tx_log2) * vec < inner) ++tx_log2;
+  const int tx = 1 << tx_log2, ry = 256 >> tx_log2;
+  const int64_t col_blocks = ceil_div(inner, static_cast<int64_t>(tx) * vec);
   if (outer > 65535) return fail(MG_ERR_UNSUPPORTED, "sum_axis: outer=%lld exceeds 65535", static_cast<long long>(outer));
-  // Enough slabs to fill the device, each at least 32 rows (fewer, longer slabs keep the
-  // fp32 partial sums a small fraction of the traffic).
+  // Enough slabs to fill the device, each at least 32 rows per row lane (fewer, longer
+  // slabs keep the fp32 partial sums a small fraction of the traffic).
   int64_t chunks = ceil_div(static_cast<int64_t>(device_info().cu_count) * env_int("MOGRAD_HIP_COLSUM_WG_PER_CU", 4),
                             col_blocks * outer);
-  const int64_t max_chunks = ceil_div(reduce, env_int("MOGRAD_HIP_COLSUM_MIN_ROWS", 32));
+  const int64_t max_chunks = ceil_div(reduce, static_cast<int64_t>(env_int("MOGRAD_HIP_COLSUM_MIN_ROWS", 32)) * ry);
   if (chunks > max_chunks) chunks = max_chunks;
   if (chunks < 1) chunks = 1;
   if (chunks > 65535) chunks = 65535;
   const int64_t rows_per_chunk = ceil_div(reduce, chunks);
   chunks = ceil_div(reduce, rows_per_chunk);
   const dim3 grid(static_cast<unsigned>(col_blocks), static_cast<unsigned>(chunks), static_cast<unsigned>(outer));
-  if (chunks == 1) {
+  if (chunks == 1 && ry == 1) {
     if (wide)
       hipLaunchKernelGGL((colsum_partial_kernel<T, WIDE, true>), grid, dim3(256), 0, stream, a, nullptr, dst, reduce,
-                         inner, rows_per_chunk);
+                         inner, rows_per_chunk, tx_log2);
     else
       hipLaunchKernelGGL((colsum_partial_kernel<T, 1, true>), grid, dim3(256), 0, stream, a, nullptr, dst, reduce, inner,
-                         rows_per_chunk);
+                         rows_per_chunk, tx_log2);
     MG_LAUNCH_CHECK();
     return MG_OK;
   }
+  const int64_t groups = chunks * ry;
   Scratch part;
-  MG_TRY(part.take(outer * chunks * inner * static_cast<int64_t>(sizeof(float))));
+  MG_TRY(part.take(outer * groups * inner * static_cast<int64_t>(sizeof(float))));
   if (wide)
     hipLaunchKernelGGL((colsum_partial_kernel<T, WIDE, false>), grid, dim3(256), 0, stream, a, part.as<float>(), dst,
-                       reduce, inner, rows_per_chunk);
+                       reduce, inner, rows_per_chunk, tx_log2);
   else
     hipLaunchKernelGGL((colsum_partial_kernel<T, 1, false>), grid, dim3(256), 0, stream, a, part.as<float>(), dst,
-                       reduce, inner, rows_per_chunk);
+                       reduce, inner, rows_per_chunk, tx_log2);
   MG_LAUNCH_CHECK();
   for (int64_t o = 0; o < outer; ++o) {
     hipLaunchKernelGGL((reduce_partials_kernel<T>), dim3(static_cast<unsigned>(ceil_div(inner, 64)), 1), dim3(256), 0,
-                       stream, part.as<float>() + o * chunks * inner, dst + o * inner, nullptr, nullptr, chunks, inner);
+                       stream, part.as<float>() + o * groups * inner, dst + o * inner, nullptr, nullptr, groups, inner);
     MG_LAUNCH_CHECK();
   }
   return MG_OK;
