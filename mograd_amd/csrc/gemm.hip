@@ -90,7 +90,7 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
                      b, bias, c, partial.as<float>(), M, N, K, lda, ldb, g.N, g.bsa, g.bsb, numel, tiles_m, tiles_n,
                      k_per_split);
   MG_LAUNCH_CHECK();
-  const unsigned rblocks = static_cast<unsigned>(ceil_div(numel, 1024));
+  const unsigned rblocks = static_cast<unsigned>(ceil_div(numel, 256));
   if (bias)
     hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, true>), dim3(rblocks), dim3(256), 0, stream, partial.as<float>(),
                        bias, c, numel, splits, N);

@@ -506,27 +506,51 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
     }
 }
 
-// out[i] = sum_s partial[s][i] (+ bias[i % N]), converted to T.
+// out[i] = sum_s partial[s][i] (+ bias[i % N]), converted to T.  A workgroup covers 64
+// groups of four consecutive outputs; its four waves each sum every fourth split (eight
+// independent 16-byte loads in flight per thread) and the four sums meet in LDS.  The
+// order of the additions is fixed, so the result is deterministic.
 template <typename T, bool HAS_BIAS>
 __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ partial,
                                                                  const T* __restrict__ bias, T* __restrict__ out,
                                                                  int64_t numel, int splits, int N) {
-  const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
-  if (i >= numel) return;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  const bool full = i + 3 < numel;
-  for (int s = 0; s < splits; ++s) {
-    const float* p = partial + static_cast<int64_t>(s) * numel + i;
+  __shared__ float4 tile[4][64];
+  const int cx = threadIdx.x % 64;
+  const int sl = threadIdx.x / 64;
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * 64 + cx) * 4;
+  float4 acc0 = make_float4(0.f, 0.f, 0.f, 0.f), acc1 = acc0;
+  if (i < numel) {
+    const bool full = i + 3 < numel;
+    int s = sl;
     if (full) {
-      const float4 v = *reinterpret_cast<const float4*>(p);
-      acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
+      for (; s + 4 < splits; s += 8) {
+        const float4 u = *reinterpret_cast<const float4*>(partial + static_cast<int64_t>(s) * numel + i);
+        const float4 w = *reinterpret_cast<const float4*>(partial + static_cast<int64_t>(s + 4) * numel + i);
+        acc0.x += u.x; acc0.y += u.y; acc0.z += u.z; acc0.w += u.w;
+        acc1.x += w.x; acc1.y += w.y; acc1.z += w.z; acc1.w += w.w;
+      }
+      for (; s < splits; s += 4) {
+        const float4 u = *reinterpret_cast<const float4*>(partial + static_cast<int64_t>(s) * numel + i);
+        acc0.x += u.x; acc0.y += u.y; acc0.z += u.z; acc0.w += u.w;
+      }
     } else {
-      for (int e = 0; e < 4 && i + e < numel; ++e) acc[e] += p[e];
+      for (; s < splits; s += 4) {
+        const float* p = partial + static_cast<int64_t>(s) * numel + i;
+        acc0.x += p[0];
+        if (i + 1 < numel) acc0.y += p[1];
+        if (i + 2 < numel) acc0.z += p[2];
+      }
     }
   }
+  tile[sl][cx] = make_float4(acc0.x + acc1.x, acc0.y + acc1.y, acc0.z + acc1.z, acc0.w + acc1.w);
+  __syncthreads();
+  if (sl != 0 || i >= numel) return;
+  const float4 t0 = tile[0][cx], t1 = tile[1][cx], t2 = tile[2][cx], t3 = tile[3][cx];
+  const float r[4] = {(t0.x + t1.x) + (t2.x + t3.x), (t0.y + t1.y) + (t2.y + t3.y), (t0.z + t1.z) + (t2.z + t3.z),
+                      (t0.w + t1.w) + (t2.w + t3.w)};
   for (int e = 0; e < 4 && i + e < numel; ++e) {
     const float bv = HAS_BIAS ? to_float(bias[(i + e) % N]) : 0.f;
-    out[i + e] = from_float<T>(acc[e] + bv);
+    out[i + e] = from_float<T>(r[e] + bv);
   }
 }
 
