@@ -327,7 +327,7 @@ __device__ __forceinline__ void gemm16_load(const T* __restrict__ base, int64_t 
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int idx = t + i * kGemmThreads;
-      const int kp = idx % 32, oc = idx / 32;
+      const int oc = idx % 16, kp = idx / 16;
       const int k = k0 + 2 * kp;
       const int o = o0 + oc * 8;
       st.v[2 * i] = gemm16_gather8(base + static_cast<int64_t>(k) * ld + o, k < k_end ? O - o : 0);
@@ -343,10 +343,11 @@ __device__ __forceinline__ void gemm16_load(const T* __restrict__ base, int64_t 
                           : make_uint4(0, 0, 0, 0);
     }
   } else {
+    // 16 consecutive lanes read the 256 contiguous bytes of one k row: whole cache lines.
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int idx = t + i * kGemmThreads;
-      const int kp = idx % 32, oc = idx / 32;
+      const int oc = idx % 16, kp = idx / 16;
       const int k = k0 + 2 * kp;
       const int o = o0 + oc * 8;
       const bool o_ok = o < O;
@@ -373,10 +374,13 @@ __device__ __forceinline__ void gemm16_store(uint16_t* __restrict__ lds, const G
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int idx = t + i * kGemmThreads;
-      const int kp = idx % 32, oc = idx / 32;
+      const int oc = idx % 16, kp = idx / 16;
       const uint32_t a[4] = {st.v[2 * i].x, st.v[2 * i].y, st.v[2 * i].z, st.v[2 * i].w};
       const uint32_t b[4] = {st.v[2 * i + 1].x, st.v[2 * i + 1].y, st.v[2 * i + 1].z, st.v[2 * i + 1].w};
-      uint32_t* dst = lds32 + (oc * 8) * (kG16Stride / 2) + kp;
+      // The 16-byte k group of a row is stored at group index (g ^ (row / 8) % 8): the 16
+      // lanes that hold different 8-row blocks of the same k pair then hit different banks
+      // (row stride 36 dwords is 4 mod 32, so 8-row blocks alone would all collide).
+      uint32_t* dst = lds32 + (oc * 8) * (kG16Stride / 2) + (((kp / 4) ^ (oc & 7)) * 4 + kp % 4);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         dst[(2 * e) * (kG16Stride / 2)] = __builtin_amdgcn_perm(b[e], a[e], 0x05040100);
@@ -386,8 +390,12 @@ __device__ __forceinline__ void gemm16_store(uint16_t* __restrict__ lds, const G
   }
 }
 
+template <bool SWIZZLED>
 __device__ __forceinline__ uint4 gemm16_frag(const uint16_t* __restrict__ lds, int o_base, int ks, int lane) {
-  return *reinterpret_cast<const uint4*>(lds + (o_base + lane % 32) * kG16Stride + ks * 16 + (lane / 32) * 8);
+  const int row = o_base + lane % 32;
+  int g = ks * 2 + lane / 32;  // 16-byte k group
+  if constexpr (SWIZZLED) g ^= (row >> 3) & 7;
+  return *reinterpret_cast<const uint4*>(lds + row * kG16Stride + g * 8);
 }
 
 template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, bool RAGGED>
@@ -436,10 +444,10 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
     }
 #pragma unroll
     for (int ks = 0; ks < kG16BK / 16; ++ks) {
-      const uint4 fa0 = gemm16_frag(lds_a, wm, ks, lane);
-      const uint4 fa1 = gemm16_frag(lds_a, wm + 32, ks, lane);
-      const uint4 fb0 = gemm16_frag(lds_b, wn, ks, lane);
-      const uint4 fb1 = gemm16_frag(lds_b, wn + 32, ks, lane);
+      const uint4 fa0 = gemm16_frag<!A_KC>(lds_a, wm, ks, lane);
+      const uint4 fa1 = gemm16_frag<!A_KC>(lds_a, wm + 32, ks, lane);
+      const uint4 fb0 = gemm16_frag<!B_KC>(lds_b, wn, ks, lane);
+      const uint4 fb1 = gemm16_frag<!B_KC>(lds_b, wn + 32, ks, lane);
       acc[0][0] = GemmMma16<T>::run(fa0, fb0, acc[0][0]);
       acc[0][1] = GemmMma16<T>::run(fa0, fb1, acc[0][1]);
       acc[1][0] = GemmMma16<T>::run(fa1, fb0, acc[1][0]);
