@@ -250,6 +250,31 @@ int mg_matmul_bias_bt(const void* a, const void* b, const void* bias, void* dst,
 int mg_linear_bwd(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db,
                   int64_t M, int64_t N, int64_t K, int dtype, mg_stream stream);
 
+/* Fused forms used by a transformer block.  None has a counterpart in the reference, whose
+ * graph runs the matmul and the elementwise op as separate kernels
+ * (examples/tinyshakespear/model.mojo:62-64,120-121; mograd/grad.mojo:130-131,180-187).
+ * Each gives bit for bit what the separate calls give: for 16-bit types the product is
+ * rounded to the storage type before a residual is added.
+ *   mg_matmul_bt_add        dst = A x B^T + residual; residual is laid out like dst
+ *                           (batch, M, N) and may be dst itself.      MATMUL_BT + ADD
+ *   mg_matmul_bias_relu_bt  dst = max(A x B^T + bias, 0).             MATMUL_BIAS_BT + RELU
+ *   mg_linear_bwd_fused     mg_linear_bwd with, for dx only:
+ *                           x_is_relu_output != 0: dx = (dY W) where x > 0, else 0
+ *                                                  (the RELU_GRAD of the layer below);
+ *                           dx_accumulate != 0:    dx += that (sum of the input
+ *                                                  gradients of layers sharing x). */
+int mg_matmul_bt_add(const void* a, const void* b, const void* residual, void* dst, int64_t batch,
+                     int64_t M, int64_t N, int64_t K, int64_t lda0, int64_t lda1, int64_t ldb0,
+                     int64_t ldb1, int64_t batch_stride_a, int64_t batch_stride_b, int dtype,
+                     mg_stream stream);
+int mg_matmul_bias_relu_bt(const void* a, const void* b, const void* bias, void* dst, int64_t batch,
+                           int64_t M, int64_t N, int64_t K, int64_t lda0, int64_t lda1,
+                           int64_t ldb0, int64_t ldb1, int64_t batch_stride_a,
+                           int64_t batch_stride_b, int dtype, mg_stream stream);
+int mg_linear_bwd_fused(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db,
+                        int64_t M, int64_t N, int64_t K, int dx_accumulate, int x_is_relu_output,
+                        int dtype, mg_stream stream);
+
 /* dst(outer, inner) = sum over the middle axis of a contiguous (outer, reduce, inner)
  * array.  db = sum over rows is outer=1, reduce=M, inner=N.  Two-stage, no atomics.
  * Replaces mograd_sum_axis for contiguous inputs, kernels/__init__.mojo:1163-1189

@@ -91,6 +91,9 @@ PROTOTYPES = {
     "mg_matmul_bt": (_i, [_p, _p, _p] + [_l] * 10 + [_i, _p], True),
     "mg_matmul_bias_bt": (_i, [_p, _p, _p, _p] + [_l] * 10 + [_i, _p], True),
     "mg_linear_bwd": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _l, _i, _p], True),
+    "mg_matmul_bt_add": (_i, [_p, _p, _p, _p, _l, _l, _l, _l, _l, _l, _l, _l, _l, _l, _i, _p], True),
+    "mg_matmul_bias_relu_bt": (_i, [_p, _p, _p, _p, _l, _l, _l, _l, _l, _l, _l, _l, _l, _l, _i, _p], True),
+    "mg_linear_bwd_fused": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _l, _i, _i, _i, _p], True),
     "mg_sum_axis": (_i, [_p, _p, _l, _l, _l, _i, _p], True),
     "mg_relu_grad": (_i, [_p, _p, _p, _l, _i, _p], True),
     "mg_add": (_i, [_p, _p, _p, _l, _i, _p], True),

@@ -14,7 +14,16 @@ struct GemmArgs {
   int64_t sam, sak, sbk, sbn;
   int64_t bsa, bsb;
   int dtype;
+  // Epilogue (see GemmEpilogue): all optional.
+  const void* residual = nullptr;
+  const void* relu_mask = nullptr;
+  int relu = 0;
 };
+
+template <typename T>
+static GemmEpilogue<T> epilogue_of(const GemmArgs& g) {
+  return GemmEpilogue<T>{static_cast<const T*>(g.residual), static_cast<const T*>(g.relu_mask), g.relu};
+}
 
 static bool mult4(int64_t v) { return (v & 3) == 0; }
 
@@ -33,11 +42,11 @@ static int launch_f32_mfma(const GemmArgs& g, hipStream_t stream) {
   if (bias)
     hipLaunchKernelGGL((gemm_f32_mfma_kernel<A_KC, B_KC, true>), dim3(static_cast<unsigned>(blocks)), dim3(kGemmThreads),
                        0, stream, a, b, bias, c, static_cast<int>(g.M), static_cast<int>(g.N), static_cast<int>(g.K), lda,
-                       ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n);
+                       ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n, epilogue_of<float>(g));
   else
     hipLaunchKernelGGL((gemm_f32_mfma_kernel<A_KC, B_KC, false>), dim3(static_cast<unsigned>(blocks)),
                        dim3(kGemmThreads), 0, stream, a, b, bias, c, static_cast<int>(g.M), static_cast<int>(g.N),
-                       static_cast<int>(g.K), lda, ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n);
+                       static_cast<int>(g.K), lda, ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n, epilogue_of<float>(g));
   MG_LAUNCH_CHECK();
   return MG_OK;
 }
@@ -72,11 +81,11 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
     if (bias)
       hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, true, false, RAGGED>), dim3(static_cast<unsigned>(blocks)),
                          dim3(kGemmThreads), 0, stream, a, b, bias, c, nullptr, M, N, K, lda, ldb, g.N, g.bsa, g.bsb,
-                         g.M * g.N, tiles_m, tiles_n, K);
+                         g.M * g.N, tiles_m, tiles_n, K, epilogue_of<T>(g));
     else
       hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, false, false, RAGGED>), dim3(static_cast<unsigned>(blocks)),
                          dim3(kGemmThreads), 0, stream, a, b, bias, c, nullptr, M, N, K, lda, ldb, g.N, g.bsa, g.bsb,
-                         g.M * g.N, tiles_m, tiles_n, K);
+                         g.M * g.N, tiles_m, tiles_n, K, epilogue_of<T>(g));
     MG_LAUNCH_CHECK();
     return MG_OK;
   }
@@ -88,15 +97,15 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
   hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, false, true, RAGGED>),
                      dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(splits)), dim3(kGemmThreads), 0, stream, a,
                      b, bias, c, partial.as<float>(), M, N, K, lda, ldb, g.N, g.bsa, g.bsb, numel, tiles_m, tiles_n,
-                     k_per_split);
+                     k_per_split, GemmEpilogue<T>{nullptr, nullptr, 0});
   MG_LAUNCH_CHECK();
   const unsigned rblocks = static_cast<unsigned>(ceil_div(numel, 256));
   if (bias)
     hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, true>), dim3(rblocks), dim3(256), 0, stream, partial.as<float>(),
-                       bias, c, numel, splits, N);
+                       bias, c, numel, splits, N, epilogue_of<T>(g));
   else
     hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, false>), dim3(rblocks), dim3(256), 0, stream, partial.as<float>(),
-                       bias, c, numel, splits, N);
+                       bias, c, numel, splits, N, epilogue_of<T>(g));
   MG_LAUNCH_CHECK();
   return MG_OK;
 }
@@ -142,11 +151,11 @@ static int launch_generic(const GemmArgs& g, hipStream_t stream) {
   if (bias)
     hipLaunchKernelGGL((gemm_generic_kernel<T, true>), grid, dim3(256), 0, stream, a, b, bias, c, static_cast<int>(g.M),
                        static_cast<int>(g.N), static_cast<int>(g.K), g.sam, g.sak, g.sbk, g.sbn, g.N, g.bsa, g.bsb,
-                       g.M * g.N);
+                       g.M * g.N, epilogue_of<T>(g));
   else
     hipLaunchKernelGGL((gemm_generic_kernel<T, false>), grid, dim3(256), 0, stream, a, b, bias, c, static_cast<int>(g.M),
                        static_cast<int>(g.N), static_cast<int>(g.K), g.sam, g.sak, g.sbk, g.sbn, g.N, g.bsa, g.bsb,
-                       g.M * g.N);
+                       g.M * g.N, epilogue_of<T>(g));
   MG_LAUNCH_CHECK();
   return MG_OK;
 }
@@ -218,11 +227,34 @@ int mg_matmul_bias_bt(const void* a, const void* b, const void* bias, void* dst,
   return mg::gemm_dispatch("matmul_bias", g, mg::to_stream(stream));
 }
 
-int mg_linear_bwd(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db, int64_t M, int64_t N,
-                  int64_t K, int dtype, mg_stream stream) {
+int mg_matmul_bt_add(const void* a, const void* b, const void* residual, void* dst, int64_t batch, int64_t M, int64_t N,
+                     int64_t K, int64_t lda0, int64_t lda1, int64_t ldb0, int64_t ldb1, int64_t batch_stride_a,
+                     int64_t batch_stride_b, int dtype, mg_stream stream) {
+  if (!residual) return mg::fail(MG_ERR_INVALID, "matmul_add: null residual pointer");
+  mg::GemmArgs g{a, b, nullptr, dst, batch, M, N, K, lda0, lda1, ldb1, ldb0, batch_stride_a, batch_stride_b, dtype};
+  g.residual = residual;
+  return mg::gemm_dispatch("matmul_add", g, mg::to_stream(stream));
+}
+
+int mg_matmul_bias_relu_bt(const void* a, const void* b, const void* bias, void* dst, int64_t batch, int64_t M, int64_t N,
+                           int64_t K, int64_t lda0, int64_t lda1, int64_t ldb0, int64_t ldb1, int64_t batch_stride_a,
+                           int64_t batch_stride_b, int dtype, mg_stream stream) {
+  if (!bias) return mg::fail(MG_ERR_INVALID, "matmul_bias_relu: null bias pointer");
+  mg::GemmArgs g{a, b, bias, dst, batch, M, N, K, lda0, lda1, ldb1, ldb0, batch_stride_a, batch_stride_b, dtype};
+  g.relu = 1;
+  return mg::gemm_dispatch("matmul_bias_relu", g, mg::to_stream(stream));
+}
+
+static int linear_bwd_impl(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db, int64_t M,
+                           int64_t N, int64_t K, bool dx_accumulate, bool x_is_relu_output, int dtype, mg_stream stream) {
   hipStream_t s = mg::to_stream(stream);
   if (dx) {  // dX (M,K) = dY (M,N) x W (N,K): reduction over N, W read as an n-contiguous right operand
     mg::GemmArgs g{dy, w, nullptr, dx, 1, M, K, N, N, 1, K, 1, 0, 0, dtype};
+    if (x_is_relu_output) {
+      if (!x) return mg::fail(MG_ERR_INVALID, "linear_bwd: x is needed as the relu mask");
+      g.relu_mask = x;  // (M, K), laid out like dX
+    }
+    if (dx_accumulate) g.residual = dx;
     MG_TRY(mg::gemm_dispatch("linear_bwd(dx)", g, s));
   }
   if (dw) {  // dW (N,K) = dY^T (N,M) x X (M,K): reduction over M, dY read as an m-contiguous left operand
@@ -231,6 +263,16 @@ int mg_linear_bwd(const void* dy, const void* x, const void* w, void* dx, void* 
   }
   if (db) MG_TRY(mg::colsum_dispatch(dy, db, 1, M, N, dtype, s));
   return MG_OK;
+}
+
+int mg_linear_bwd(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db, int64_t M, int64_t N,
+                  int64_t K, int dtype, mg_stream stream) {
+  return linear_bwd_impl(dy, x, w, dx, dw, db, M, N, K, false, false, dtype, stream);
+}
+
+int mg_linear_bwd_fused(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db, int64_t M, int64_t N,
+                        int64_t K, int dx_accumulate, int x_is_relu_output, int dtype, mg_stream stream) {
+  return linear_bwd_impl(dy, x, w, dx, dw, db, M, N, K, dx_accumulate != 0, x_is_relu_output != 0, dtype, stream);
 }
 
 }  // extern "C"

@@ -46,6 +46,26 @@ __device__ __forceinline__ void gemm_tile_of_block(int bid, int tiles_m, int til
   tn = in_band / rows_here;
 }
 
+// What happens to a product element after the bias: v = acc + bias; relu: v = max(v, 0);
+// relu_mask (laid out like C): v = 0 where mask <= 0; v is rounded to T; residual (laid out
+// like C, may be C itself): v = round(v + residual).  For 16-bit types the residual is added
+// to the rounded product, which is bit for bit what a separate add kernel computes.
+template <typename T>
+struct GemmEpilogue {
+  const T* residual;
+  const T* relu_mask;
+  int relu;
+};
+
+template <typename T>
+__device__ __forceinline__ T gemm_finish(float v, const GemmEpilogue<T>& ep, int64_t index) {
+  if (ep.relu) v = v > 0.f ? v : 0.f;
+  if (ep.relu_mask) v = to_float(ep.relu_mask[index]) > 0.f ? v : 0.f;
+  T out = from_float<T>(v);
+  if (ep.residual) out = from_float<T>(to_float(out) + to_float(ep.residual[index]));
+  return out;
+}
+
 // Registers holding one thread's share of a 128 x 32 (or 32 x 128) operand tile.
 struct GemmStage {
   float4 v[4];
@@ -111,7 +131,7 @@ template <bool A_KC, bool B_KC, bool HAS_BIAS>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_kernel(
     const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias, float* __restrict__ C,
     int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb, int64_t bsc, int tiles_m,
-    int tiles_n) {
+    int tiles_n, GemmEpilogue<float> ep) {
   __shared__ __attribute__((aligned(16))) float lds_a[kGemmBM * kKcStride];
   __shared__ __attribute__((aligned(16))) float lds_b[kGemmBN * kKcStride];
 
@@ -124,6 +144,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_kernel(
   A += batch * bsa;
   B += batch * bsb;
   C += batch * bsc;
+  if (ep.residual) ep.residual += batch * bsc;
+  if (ep.relu_mask) ep.relu_mask += batch * bsc;
 
   const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
@@ -179,7 +201,10 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm + ti * 32 + (r / 4) * 8 + (lane / 32) * 4 + (r % 4);
-        if (row < M) C[static_cast<int64_t>(row) * ldc + col] = acc[ti][tj][r] + bv;
+        if (row < M) {
+          const int64_t at = static_cast<int64_t>(row) * ldc + col;
+          C[at] = gemm_finish<float>(acc[ti][tj][r] + bv, ep, at);
+        }
       }
     }
 }
@@ -195,7 +220,8 @@ template <typename T, bool HAS_BIAS>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__ A, const T* __restrict__ B,
                                                            const T* __restrict__ bias, T* __restrict__ C, int M, int N,
                                                            int K, int64_t sam, int64_t sak, int64_t sbk, int64_t sbn,
-                                                           int64_t ldc, int64_t bsa, int64_t bsb, int64_t bsc) {
+                                                           int64_t ldc, int64_t bsa, int64_t bsb, int64_t bsc,
+                                                           GemmEpilogue<T> ep) {
   constexpr int TM = 64, TN = 64, TK = 16;
   __shared__ float as[TK][TM + 1];
   __shared__ float bs[TK][TN + 1];
@@ -203,6 +229,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
   A += batch * bsa;
   B += batch * bsb;
   C += batch * bsc;
+  if (ep.residual) ep.residual += batch * bsc;
+  if (ep.relu_mask) ep.relu_mask += batch * bsc;
   const int m0 = blockIdx.y * TM;
   const int n0 = blockIdx.x * TN;
   const int tx = threadIdx.x % 16;
@@ -244,7 +272,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
       const int gm = m0 + ty + i * 16, gn = n0 + tx + j * 16;
       if (gm < M && gn < N) {
         const float bv = HAS_BIAS ? to_float(bias[gn]) : 0.f;
-        C[static_cast<int64_t>(gm) * ldc + gn] = from_float<T>(acc[i][j] + bv);
+        const int64_t at = static_cast<int64_t>(gm) * ldc + gn;
+        C[at] = gemm_finish<T>(acc[i][j] + bv, ep, at);
       }
     }
 }
@@ -402,7 +431,7 @@ template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, bool RA
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
     const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C,
     float* __restrict__ partial, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb,
-    int64_t bsc, int tiles_m, int tiles_n, int k_per_split) {
+    int64_t bsc, int tiles_m, int tiles_n, int k_per_split, GemmEpilogue<T> ep) {
   __shared__ __attribute__((aligned(16))) uint16_t lds_a[kGemmBM * kG16Stride];
   __shared__ __attribute__((aligned(16))) uint16_t lds_b[kGemmBN * kG16Stride];
 
@@ -474,12 +503,16 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int rl = ti * 32 + (r / 4) * 8 + (lane / 32) * 4 + (r % 4);
-            const T v = from_float<T>(acc[ti][tj][r] + bv);
+            float f = acc[ti][tj][r] + bv;
+            if (ep.relu) f = f > 0.f ? f : 0.f;
+            const T v = from_float<T>(f);
             mine[rl * kG16Stride + cl] = __builtin_bit_cast(uint16_t, v);
           }
         }
       __syncthreads();
       T* cbase = C + batch * bsc;
+      const T* rbase = ep.residual ? ep.residual + batch * bsc : nullptr;
+      const T* mbase = ep.relu_mask ? ep.relu_mask + batch * bsc : nullptr;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const int chunk = lane + i * kWave;
@@ -487,8 +520,26 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
         const int row = m0 + wm + rl;
         const int col = n0 + wn + ch * 8;
         if (row < M && col < N) {
-          const uint4 v = *reinterpret_cast<const uint4*>(mine + rl * kG16Stride + ch * 8);
-          *reinterpret_cast<uint4*>(cbase + static_cast<int64_t>(row) * ldc + col) = v;
+          const int64_t at = static_cast<int64_t>(row) * ldc + col;
+          if (rbase || mbase) {
+            float v[8];
+            VecIO<T, 8>::load(reinterpret_cast<const T*>(mine + rl * kG16Stride + ch * 8), v);
+            if (mbase) {
+              float mk[8];
+              VecIO<T, 8>::load(mbase + at, mk);
+#pragma unroll
+              for (int e = 0; e < 8; ++e) v[e] = mk[e] > 0.f ? v[e] : 0.f;
+            }
+            if (rbase) {
+              float rs[8];
+              VecIO<T, 8>::load(rbase + at, rs);
+#pragma unroll
+              for (int e = 0; e < 8; ++e) v[e] += rs[e];
+            }
+            VecIO<T, 8>::store(cbase + at, v);
+          } else {
+            *reinterpret_cast<uint4*>(cbase + at) = *reinterpret_cast<const uint4*>(mine + rl * kG16Stride + ch * 8);
+          }
         }
       }
       return;
@@ -507,8 +558,10 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
         if (row < M) {
           if constexpr (SPLIT_K)
             partial[(static_cast<int64_t>(blockIdx.y) * M + row) * N + col] = acc[ti][tj][r];
-          else
-            C[batch * bsc + static_cast<int64_t>(row) * ldc + col] = from_float<T>(acc[ti][tj][r] + bv);
+          else {
+            const int64_t at = batch * bsc + static_cast<int64_t>(row) * ldc + col;
+            C[at] = gemm_finish<T>(acc[ti][tj][r] + bv, ep, at);
+          }
         }
       }
     }
@@ -521,7 +574,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
 template <typename T, bool HAS_BIAS>
 __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ partial,
                                                                  const T* __restrict__ bias, T* __restrict__ out,
-                                                                 int64_t numel, int splits, int N) {
+                                                                 int64_t numel, int splits, int N, GemmEpilogue<T> ep) {
   __shared__ float4 tile[4][64];
   const int cx = threadIdx.x % 64;
   const int sl = threadIdx.x / 64;
@@ -558,7 +611,7 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
                       (t0.w + t1.w) + (t2.w + t3.w)};
   for (int e = 0; e < 4 && i + e < numel; ++e) {
     const float bv = HAS_BIAS ? to_float(bias[(i + e) % N]) : 0.f;
-    out[i + e] = from_float<T>(r[e] + bv);
+    out[i + e] = gemm_finish<T>(r[e] + bv, ep, i + e);
   }
 }
 

@@ -8,9 +8,11 @@ sequence of libmograd_hip calls on one stream.
     logits = lm_head(h);  loss = mean softmax cross-entropy over all tokens
 
 The backward pass is the graph mograd/grad.mojo builds for that forward, with the fused
-entries in place of their unfused chains: mg_linear_bwd for every Linear,
-mg_layer_norm_bwd_stats, mg_flash_attn_bwd, mg_cross_entropy_fused_ids, mg_relu_grad,
-mg_scatter_add for the embedding.
+entries in place of their unfused chains: mg_linear_bwd(_fused) for every Linear (with the
+ReLU gradient and the sum of the Q/K/V input gradients folded into the dX products),
+mg_layer_norm_bwd_stats, mg_flash_attn_bwd, mg_cross_entropy_fused_ids, mg_scatter_add for
+the embedding; in the forward the residual additions and the ReLU ride on the products
+that feed them (mg_matmul_bt_add, mg_matmul_bias_relu_bt).
 
 Mixed precision: the parameters live in one fp32 arena (master weights); each step casts
 the whole arena once to the compute dtype (bf16 by default), runs every kernel in that
@@ -129,8 +131,7 @@ class TinyTransformer:
                 "h_mid": new(n * d), "x2": new(n * d), "a": new(n * ff),
                 "mean1": new(n, F32), "rstd1": new(n, F32), "mean2": new(n, F32), "rstd2": new(n, F32),
             })
-        self.tmp = {name: new(n * d) for name in ("proj", "dh", "dres", "dctx", "do", "dq", "dk", "dv", "dx_a", "dx_b",
-                                                  "dx_c")}
+        self.tmp = {name: new(n * d) for name in ("dh", "dres", "dctx", "do", "dq", "dk", "dv", "dx_a")}
         self.tmp["da"] = new(n * ff)
         self.tmp["logits"] = new(n * V)
         self.tmp["dlogits"] = new(n * V)
@@ -179,14 +180,13 @@ class TinyTransformer:
                                   0, cd, s)
             # O comes back (B, H, T, dh); the projection wants (B, T, H*dh)
             lib.mg_contiguous(P(c["o"]), P(c["ctx"]), 4, i64(B, T, H, dh), i64(H * T * dh, dh, T * dh, 1), cd, s)
-            linear(P(c["ctx"]), w("wo"), P(self.tmp["proj"]), d, d)
-            lib.mg_add(h_in, P(self.tmp["proj"]), P(c["h_mid"]), n * d, cd, s)
+            lib.mg_matmul_bt_add(P(c["ctx"]), w("wo"), h_in, P(c["h_mid"]), 1, n, d, d, d, 1, d, 1, n * d, d * d, cd, s)
             lib.mg_layer_norm_fwd_stats(P(c["h_mid"]), w("ln2_g"), w("ln2_b"), P(c["x2"]), P(c["mean2"]),
                                         P(c["rstd2"]), n, d, self.eps, cd, s)
-            linear(P(c["x2"]), w("w1"), P(c["a"]), ff, d, bias=w("b1"))
-            lib.mg_relu(P(c["a"]), P(c["a"]), n * ff, cd, s)
-            linear(P(c["a"]), w("w2"), P(self.tmp["proj"]), d, ff)
-            lib.mg_add(P(c["h_mid"]), P(self.tmp["proj"]), h_out, n * d, cd, s)
+            lib.mg_matmul_bias_relu_bt(P(c["x2"]), w("w1"), w("b1"), P(c["a"]), 1, n, ff, d, d, 1, d, 1, n * d, ff * d, cd,
+                                       s)
+            lib.mg_matmul_bt_add(P(c["a"]), w("w2"), P(c["h_mid"]), h_out, 1, n, d, ff, ff, 1, ff, 1, n * ff, d * ff, cd,
+                                 s)
         linear(P(self.h[self.L]), self._w("lm_head"), P(self.tmp["logits"]), V, d)
         lib.mg_cross_entropy_fused_ids(P(self.tmp["logits"]), P(labels), None, P(self.loss), P(self.tmp["dlogits"]), n,
                                        V, cd, labels.dtype, s)
@@ -202,8 +202,7 @@ class TinyTransformer:
             w = lambda name, l=l: self._w(f"blocks.{l}.{name}")
             g = lambda name, l=l: self._g(f"blocks.{l}.{name}")
             # h_out = h_mid + W2 a
-            lib.mg_linear_bwd(t["dh"], P(c["a"]), w("w2"), t["da"], g("w2"), None, n, d, ff, cd, s)
-            lib.mg_relu_grad(P(c["a"]), t["da"], t["da"], n * ff, cd, s)
+            lib.mg_linear_bwd_fused(t["dh"], P(c["a"]), w("w2"), t["da"], g("w2"), None, n, d, ff, 0, 1, cd, s)
             lib.mg_linear_bwd(t["da"], P(c["x2"]), w("w1"), t["dx_a"], g("w1"), g("b1"), n, ff, d, cd, s)
             lib.mg_layer_norm_bwd_stats(t["dx_a"], P(c["h_mid"]), w("ln2_g"), P(c["mean2"]), P(c["rstd2"]), t["dres"],
                                         g("ln2_g"), g("ln2_b"), n, d, cd, s)
@@ -215,10 +214,8 @@ class TinyTransformer:
             lib.mg_flash_attn_bwd(t["do"], P(c["o"]), P(c["q"]), P(c["k"]), P(c["v"]), None, P(c["lse"]), t["dq"],
                                   t["dk"], t["dv"], B, T, H, dh, scale, 1, 0, cd, s)
             lib.mg_linear_bwd(t["dq"], P(c["x1"]), w("wq"), t["dx_a"], g("wq"), None, n, d, d, cd, s)
-            lib.mg_linear_bwd(t["dk"], P(c["x1"]), w("wk"), t["dx_b"], g("wk"), None, n, d, d, cd, s)
-            lib.mg_linear_bwd(t["dv"], P(c["x1"]), w("wv"), t["dx_c"], g("wv"), None, n, d, d, cd, s)
-            lib.mg_add(t["dx_a"], t["dx_b"], t["dx_a"], n * d, cd, s)
-            lib.mg_add(t["dx_a"], t["dx_c"], t["dx_a"], n * d, cd, s)
+            lib.mg_linear_bwd_fused(t["dk"], P(c["x1"]), w("wk"), t["dx_a"], g("wk"), None, n, d, d, 1, 0, cd, s)
+            lib.mg_linear_bwd_fused(t["dv"], P(c["x1"]), w("wv"), t["dx_a"], g("wv"), None, n, d, d, 1, 0, cd, s)
             lib.mg_layer_norm_bwd_stats(t["dx_a"], P(self.h[l]), w("ln1_g"), P(c["mean1"]), P(c["rstd1"]), t["dres"],
                                         g("ln1_g"), g("ln1_b"), n, d, cd, s)
             lib.mg_add(t["dh"], t["dres"], t["dh"], n * d, cd, s)

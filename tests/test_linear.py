@@ -212,3 +212,79 @@ def test_bf16_linear_bwd_entry_gpt_shapes(device):
                             (dw.to_numpy((N, K)), O.linear_grad_w(dy, x), "dw"),
                             (db.to_numpy(), O.linear_grad_b(dy), "db")):
         assert_close(got, want, 1.6e-2, 1.6e-2 * np.abs(want).max(), name)
+
+
+# ---- fused epilogues: each must give exactly what the separate calls give -----------------
+
+FUSED_SHAPES = [(256, 384, 512), (200, 136, 264), (130, 65, 384), (64, 10, 256), (33, 7, 5), (4096, 128, 128),
+                (128, 64, 4096)]
+
+
+def _ptr(b):
+    return b.data_ptr()
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
+@pytest.mark.parametrize("M,N,K", FUSED_SHAPES)
+def test_fused_epilogues_equal_separate_calls(device, dtype, M, N, K):
+    lib, st = device.lib, device.stream
+    x = round_to_dtype(normal(49, 0, (M, K)), dtype)
+    w = round_to_dtype(normal(49, 1, (N, K), std=0.1), dtype)
+    b = round_to_dtype(normal(49, 2, (N,), std=0.5), dtype)
+    res = round_to_dtype(normal(49, 3, (M, N)), dtype)
+    dy = round_to_dtype(normal(49, 4, (M, N), std=0.5), dtype)
+    bx, bw, bb, bres, bdy = (AnyBuffer.from_numpy(device, a, dtype) for a in (x, w, b, res, dy))
+    new = lambda n: AnyBuffer.create(dtype, device, n)  # noqa: E731
+    mm = (1, M, N, K, K, 1, K, 1, M * K, N * K, dtype, st)
+
+    # A B^T + residual  ==  matmul_bt, then add
+    y, y_ref, got = new(M * N), new(M * N), new(M * N)
+    lib.mg_matmul_bt(_ptr(bx), _ptr(bw), _ptr(y), *mm)
+    lib.mg_add(_ptr(y), _ptr(bres), _ptr(y_ref), M * N, dtype, st)
+    lib.mg_matmul_bt_add(_ptr(bx), _ptr(bw), _ptr(bres), _ptr(got), *mm)
+    np.testing.assert_array_equal(got.to_numpy(), y_ref.to_numpy())
+    # in place: the residual buffer is also the destination
+    inplace = AnyBuffer.from_numpy(device, res, dtype)
+    lib.mg_matmul_bt_add(_ptr(bx), _ptr(bw), _ptr(inplace), _ptr(inplace), *mm)
+    np.testing.assert_array_equal(inplace.to_numpy(), y_ref.to_numpy())
+    # and against the oracle
+    want = O.matmul_bias_bt(x, w) + res
+    rt = {F32: 1e-4, F16: 2e-3, BF16: 1.6e-2}[dtype]
+    assert_close(got.to_numpy((M, N)), want, rt, rt * np.abs(want).max(), "matmul_bt_add")
+
+    # max(A B^T + bias, 0)  ==  matmul_bias_bt, then relu
+    lib.mg_matmul_bias_bt(_ptr(bx), _ptr(bw), _ptr(bb), _ptr(y), *mm)
+    lib.mg_relu(_ptr(y), _ptr(y_ref), M * N, dtype, st)
+    lib.mg_matmul_bias_relu_bt(_ptr(bx), _ptr(bw), _ptr(bb), _ptr(got), *mm)
+    np.testing.assert_array_equal(got.to_numpy(), y_ref.to_numpy())
+
+    # linear_bwd_fused: relu mask from x, accumulation into dx
+    xr = np.maximum(x, 0)  # x as the output of a relu: about half zeros
+    bxr = AnyBuffer.from_numpy(device, xr, dtype)
+    dx, dx_ref, dw, dw_ref, db, db_ref = new(M * K), new(M * K), new(N * K), new(N * K), new(N), new(N)
+    lib.mg_linear_bwd(_ptr(bdy), _ptr(bxr), _ptr(bw), _ptr(dx), _ptr(dw_ref), _ptr(db_ref), M, N, K, dtype, st)
+    lib.mg_relu_grad(_ptr(bxr), _ptr(dx), _ptr(dx_ref), M * K, dtype, st)
+    lib.mg_linear_bwd_fused(_ptr(bdy), _ptr(bxr), _ptr(bw), _ptr(dx), _ptr(dw), _ptr(db), M, N, K, 0, 1, dtype, st)
+    np.testing.assert_array_equal(dx.to_numpy(), dx_ref.to_numpy())
+    np.testing.assert_array_equal(dw.to_numpy(), dw_ref.to_numpy())
+    np.testing.assert_array_equal(db.to_numpy(), db_ref.to_numpy())
+    assert not dx.to_numpy((M, K))[xr <= 0].any()
+    # accumulate: dx starts as `prior`, ends as prior + dY W
+    prior = round_to_dtype(normal(49, 5, (M, K)), dtype)
+    acc = AnyBuffer.from_numpy(device, prior, dtype)
+    bprior = AnyBuffer.from_numpy(device, prior, dtype)
+    lib.mg_linear_bwd(_ptr(bdy), _ptr(bx), _ptr(bw), _ptr(dx), None, None, M, N, K, dtype, st)
+    lib.mg_add(_ptr(dx), _ptr(bprior), _ptr(dx_ref), M * K, dtype, st)
+    lib.mg_linear_bwd_fused(_ptr(bdy), _ptr(bx), _ptr(bw), _ptr(acc), None, None, M, N, K, 1, 0, dtype, st)
+    np.testing.assert_array_equal(acc.to_numpy(), dx_ref.to_numpy())
+
+
+def test_fused_entry_errors(device):
+    buf = AnyBuffer.create(F32, device, 16)
+    p = buf.data_ptr()
+    with pytest.raises(MogradError, match="null residual"):
+        device.lib.mg_matmul_bt_add(p, p, None, p, 1, 2, 2, 2, 2, 1, 2, 1, 4, 4, F32, device.stream)
+    with pytest.raises(MogradError, match="null bias"):
+        device.lib.mg_matmul_bias_relu_bt(p, p, None, p, 1, 2, 2, 2, 2, 1, 2, 1, 4, 4, F32, device.stream)
+    with pytest.raises(MogradError, match="relu mask"):
+        device.lib.mg_linear_bwd_fused(p, None, p, p, None, None, 2, 2, 2, 0, 1, F32, device.stream)
