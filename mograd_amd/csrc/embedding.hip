@@ -38,7 +38,7 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const T* __restrict__ 
 }
 
 // One wave per (destination row, column block, slab).  DIRECT writes the row itself (one
-// slab); otherwise fp32 partials (slab, row, col) go to scratch for reduce_partials_kernel.
+// slab); otherwise fp32 partials (slab, row, col) go to scratch for the partials reduction.
 template <typename T, typename I, int VEC, bool DIRECT>
 __global__ __launch_bounds__(64) void scatter_rows_kernel(const I* __restrict__ indices, const T* __restrict__ values,
                                                           float* __restrict__ part, T* __restrict__ dst, int64_t n_idx,
@@ -128,8 +128,7 @@ static int scatter_launch(const I* indices, const T* values, T* dst, int64_t n_i
                      dst, n_idx, num_rows, row_size, slab_len);
   MG_LAUNCH_CHECK();
   const int64_t cols = num_rows * row_size;
-  hipLaunchKernelGGL((reduce_partials_kernel<T>), dim3(static_cast<unsigned>(ceil_div(cols, 64)), 1), dim3(256), 0, s,
-                     part.as<float>(), dst, nullptr, nullptr, slabs, cols);
+  launch_reduce_partials<T>(part.as<float>(), dst, nullptr, nullptr, slabs, cols, device_info().cu_count, s);
   MG_LAUNCH_CHECK();
   return MG_OK;
 }

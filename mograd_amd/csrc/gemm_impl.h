@@ -288,7 +288,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
 // m/n-contiguous operand is transposed on the way in: a thread loads 8 columns of two
 // consecutive k rows and stores 8 dwords, each packing (k, k+1) for one column.
 // SPLIT_K: blockIdx.y selects a K range and fp32 partial tiles go to scratch
-// (splits, M, N); reduce_partials_kernel sums them in a fixed order.
+// (splits, M, N); gemm_splitk_reduce_kernel sums them in a fixed order.
 // ------------------------------------------------------------------------------------
 
 namespace mg {

@@ -433,8 +433,8 @@ struct LayerNormOps {
                        dim3(WG), 0, stream, dy, x, gamma, mean, rstd, dx, part_g.as<float>(), part_b.as<float>(), rows,
                        static_cast<int>(cols), eps, rows_per_group);
     MG_LAUNCH_CHECK();
-    hipLaunchKernelGGL((reduce_partials_kernel<T>), dim3(static_cast<unsigned>(ceil_div(cols, 64)), 2), dim3(256), 0,
-                       stream, part_g.as<float>(), dgamma, part_b.as<float>(), dbeta, groups, cols);
+    launch_reduce_partials<T>(part_g.as<float>(), dgamma, part_b.as<float>(), dbeta, groups, cols,
+                              device_info().cu_count, stream);
     MG_LAUNCH_CHECK();
     return MG_OK;
   }
@@ -478,8 +478,8 @@ struct LayerNormOps {
                        dim3(256), 0, stream, dy, x, stat_mean.as<float>(), stat_rstd.as<float>(), part_g.as<float>(),
                        part_b.as<float>(), rows, cols, rows_per_group);
     MG_LAUNCH_CHECK();
-    hipLaunchKernelGGL((reduce_partials_kernel<T>), dim3(static_cast<unsigned>(ceil_div(cols, 64)), 2), dim3(256), 0,
-                       stream, part_g.as<float>(), dgamma, part_b.as<float>(), dbeta, groups, cols);
+    launch_reduce_partials<T>(part_g.as<float>(), dgamma, part_b.as<float>(), dbeta, groups, cols,
+                              device_info().cu_count, stream);
     MG_LAUNCH_CHECK();
     return MG_OK;
   }

@@ -94,34 +94,57 @@ __device__ __forceinline__ void row_allreduce_sum(float (&v)[K], float* slots, i
 // ------------------------------------------------------------------------------------
 // Second stage of a column reduction: out[c] = sum_g part[g][c], plain stores, fixed
 // order (used by LayerNorm's dgamma/dbeta and by the bias gradient).
-// Workgroup = 64 columns x 4 row slices; blockIdx.y selects which of up to two
+// Workgroup = CW columns x 256/CW row slices; blockIdx.y selects which of up to two
 // (partials, output) pairs to reduce.
 // ------------------------------------------------------------------------------------
 
-template <typename T>
-__global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ part0, T* __restrict__ out0,
-                                                              const float* __restrict__ part1, T* __restrict__ out1,
-                                                              int64_t groups, int64_t cols) {
-  __shared__ float tile[4][64];
+template <typename T, int CW>
+__global__ __launch_bounds__(256) void reduce_partials_cw_kernel(const float* __restrict__ part0, T* __restrict__ out0,
+                                                                 const float* __restrict__ part1, T* __restrict__ out1,
+                                                                 int64_t groups, int64_t cols) {
+  constexpr int SL = 256 / CW;  // row slices per workgroup
+  __shared__ float tile[SL][CW];
   const float* part = blockIdx.y == 0 ? part0 : part1;
   T* out = blockIdx.y == 0 ? out0 : out1;
-  const int cx = threadIdx.x % 64;
-  const int sy = threadIdx.x / 64;
-  const int64_t c = static_cast<int64_t>(blockIdx.x) * 64 + cx;
+  const int cx = threadIdx.x % CW;
+  const int sy = threadIdx.x / CW;
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * CW + cx;
   float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
   if (c < cols) {
     int64_t g = sy;
-    for (; g + 12 < groups; g += 16) {
+    for (; g + 3 * SL < groups; g += 4 * SL) {
       a0 += part[g * cols + c];
-      a1 += part[(g + 4) * cols + c];
-      a2 += part[(g + 8) * cols + c];
-      a3 += part[(g + 12) * cols + c];
+      a1 += part[(g + SL) * cols + c];
+      a2 += part[(g + 2 * SL) * cols + c];
+      a3 += part[(g + 3 * SL) * cols + c];
     }
-    for (; g < groups; g += 4) a0 += part[g * cols + c];
+    for (; g < groups; g += SL) a0 += part[g * cols + c];
   }
   tile[sy][cx] = (a0 + a1) + (a2 + a3);
   __syncthreads();
-  if (sy == 0 && c < cols) out[c] = from_float<T>((tile[0][cx] + tile[1][cx]) + (tile[2][cx] + tile[3][cx]));
+  // fixed-order tree over the slices
+#pragma unroll
+  for (int w = SL / 2; w > 0; w /= 2) {
+    if (sy < w) tile[sy][cx] += tile[sy + w][cx];
+    __syncthreads();
+  }
+  if (sy == 0 && c < cols) out[c] = from_float<T>(tile[0][cx]);
+}
+
+// Launches the reduction of one or two (groups, cols) partial arrays.  Wide outputs use 64
+// columns x 4 slices per workgroup; narrow ones 16 columns x 16 slices, so that a few
+// hundred columns still spread over enough workgroups to hide the load latency.
+template <typename T>
+inline void launch_reduce_partials(const float* part0, T* out0, const float* part1, T* out1, int64_t groups, int64_t cols,
+                                   int cu_count, hipStream_t stream) {
+  const unsigned pairs = part1 ? 2u : 1u;
+  if (ceil_div(cols, 64) * pairs >= static_cast<int64_t>(cu_count)) {
+    hipLaunchKernelGGL((reduce_partials_cw_kernel<T, 64>), dim3(static_cast<unsigned>(ceil_div(cols, 64)), pairs),
+                       dim3(256), 0, stream, part0, out0, part1, out1, groups, cols);
+  } else {
+    hipLaunchKernelGGL((reduce_partials_cw_kernel<T, 16>), dim3(static_cast<unsigned>(ceil_div(cols, 16)), pairs),
+                       dim3(256), 0, stream, part0, out0, part1, out1, groups, cols);
+  }
 }
 
 }  // namespace mg

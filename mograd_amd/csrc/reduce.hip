@@ -9,7 +9,7 @@ namespace mg {
 // lanes; a thread sums every (256 / TX)-th row of its slab for VEC columns with 16-byte
 // loads (narrow matrices get more row lanes instead of idle column threads).  DIRECT writes
 // the final value (one slab, one row lane); otherwise fp32 partials
-// (outer, slab * row_lanes + lane, inner) go to scratch and reduce_partials_kernel finishes
+// (outer, slab * row_lanes + lane, inner) go to scratch and reduce_partials_cw_kernel finishes
 // in a fixed order.  No atomics.
 template <typename T, int VEC, bool DIRECT>
 __global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict__ a, float* __restrict__ part,
@@ -146,8 +146,8 @@ static int colsum_typed(const T* a, T* dst, int64_t outer, int64_t reduce, int64
                        reduce, inner, rows_per_chunk, tx_log2);
   MG_LAUNCH_CHECK();
   for (int64_t o = 0; o < outer; ++o) {
-    hipLaunchKernelGGL((reduce_partials_kernel<T>), dim3(static_cast<unsigned>(ceil_div(inner, 64)), 1), dim3(256), 0,
-                       stream, part.as<float>() + o * groups * inner, dst + o * inner, nullptr, nullptr, groups, inner);
+    launch_reduce_partials<T>(part.as<float>() + o * groups * inner, dst + o * inner, nullptr, nullptr, groups, inner,
+                              device_info().cu_count, stream);
     MG_LAUNCH_CHECK();
   }
   return MG_OK;
