@@ -331,6 +331,24 @@ int mg_scatter_add(const void* indices, const void* values, void* dst, int64_t n
                    int64_t num_rows, int64_t row_size, int idx_dtype, int dtype, mg_stream stream);
 
 /* ------------------------------------------------------------------------------------ */
+/* Optimizer updates on flat fp32 arrays (parameters, gradients and moments are fp32 in   */
+/* the reference).  One streaming kernel each; in place.                                  */
+/* ------------------------------------------------------------------------------------ */
+
+/* One Adam (decoupled_weight_decay == 0: weight decay added to the gradient) or AdamW
+ * (!= 0: w scaled by 1 - lr*wd first) update of n parameters, t = step count from 1:
+ *   m = m*b1 + g*(1-b1);  v = v*b2 + g*g*(1-b2)
+ *   w = w - lr * (m / (1 - b1^t)) / (sqrt(v / (1 - b2^t)) + eps)
+ * with the reference's order of operations.  Replaces the elementwise graph that
+ * mograd/nn/optim/adam.mojo:6-78 (_adam_step) evaluates per parameter. */
+int mg_adam_step(void* w, const void* g, void* m, void* v, int64_t n, float lr, float beta1,
+                 float beta2, float eps, float weight_decay, int64_t t,
+                 int decoupled_weight_decay, mg_stream stream);
+
+/* w = w - g * lr.  Replaces mograd/nn/optim/sgd.mojo:24-45. */
+int mg_sgd_step(void* w, const void* g, int64_t n, float lr, mg_stream stream);
+
+/* ------------------------------------------------------------------------------------ */
 /* Flash attention.  Q, K, V, dQ, dK, dV are BSHD; O and dO are BHSD; mask is            */
 /* (B,H,S,S) additive bias in natural-log units, of `dtype`; LSE is (B,H,S) fp32 natural  */
 /* log (kernels/attention/generic.mojo:29-35).  dtype in {F32, F16, BF16}.                */

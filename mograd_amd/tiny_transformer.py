@@ -225,6 +225,34 @@ class TinyTransformer:
             marks("backward")
         return self.loss
 
+    # ------------------------------------------------------------------ optimizer
+
+    def adam_step(self, lr: float = 1e-3, beta1: float = 0.9, beta2: float = 0.999, eps: float = 1e-8,
+                  weight_decay: float = 0.0, decoupled: bool = False) -> None:
+        """One Adam / AdamW update of every parameter from the gradients of the last
+        `step` (mograd/nn/optim/adam.mojo): a single kernel over the fp32 arenas."""
+        if not hasattr(self, "adam_m"):
+            self.adam_m = AnyBuffer.create(F32, self.device, self.total, fill=0.0)
+            self.adam_v = AnyBuffer.create(F32, self.device, self.total, fill=0.0)
+            self.adam_t = 0
+        self.adam_t += 1
+        self.lib.mg_adam_step(self.master.data_ptr(), self.grads.data_ptr(), self.adam_m.data_ptr(),
+                              self.adam_v.data_ptr(), self.total, lr, beta1, beta2, eps, weight_decay, self.adam_t,
+                              int(decoupled), self.stream)
+
+    def parameters(self) -> dict:
+        """Downloads the fp32 master weights as a tree shaped like load_params' argument."""
+        flat = self.master.to_numpy()
+        out = {"blocks": [dict() for _ in range(self.L)]}
+        for name, sl in self.slices.items():
+            a = flat[sl.offset:sl.offset + sl.numel].reshape(sl.shape).copy()
+            parts = name.split(".")
+            if parts[0] == "blocks":
+                out["blocks"][int(parts[1])][parts[2]] = a
+            else:
+                out[name] = a
+        return out
+
     # ------------------------------------------------------------------ bookkeeping
 
     def flops_per_step(self, B: int, T: int) -> float:

@@ -24,6 +24,7 @@ Pinning (what makes each function trustworthy without running the reference):
   gather / scatter_add  index arithmetic by definition; adjoint identity
                         <gather(W, i), Y> = <W, scatter_add(i, Y)>; torch index_add_
   tiny_transformer_step torch autograd (f64) on the same model, finite differences
+  adam_step / sgd_step  torch.optim.Adam / AdamW / SGD over several steps (f64)
   round_class           tests/test_memory.mojo:18-30 (1000 -> 1024, 1025 -> 1152)
 All of the above are exercised in tests/test_oracle.py.
 """
@@ -461,6 +462,32 @@ def tiny_transformer_step(params, ids, labels, n_heads, eps=1e-5, store=None):
         grads["blocks"].insert(0, g)
     grads["embed"] = r(scatter_add(ids.reshape(-1), dh_, V))
     return float(loss), grads
+
+
+# --------------------------------------------------------------------------- #
+# Optimizer updates
+# --------------------------------------------------------------------------- #
+
+
+def adam_step(w, g, m, v, lr, beta1, beta2, eps, weight_decay, t, decoupled):
+    """One Adam (decoupled=False) or AdamW (True) update; returns (w, m, v).
+    mograd/nn/optim/adam.mojo:20-53."""
+    w, g, m, v = (np.asarray(a, dtype=F64) for a in (w, g, m, v))
+    bc1 = 1.0 - beta1 ** t
+    bc2 = 1.0 - beta2 ** t
+    if not decoupled and weight_decay > 0.0:
+        g = g + w * weight_decay
+    m = m * beta1 + g * (1.0 - beta1)
+    v = v * beta2 + (g * g) * (1.0 - beta2)
+    update = (m / bc1) / (np.sqrt(v / bc2) + eps) * lr
+    if decoupled and weight_decay > 0.0:
+        w = w * (1.0 - lr * weight_decay)
+    return w - update, m, v
+
+
+def sgd_step(w, g, lr):
+    """w - g * lr.  mograd/nn/optim/sgd.mojo:33-36."""
+    return np.asarray(w, dtype=F64) - np.asarray(g, dtype=F64) * lr
 
 
 # --------------------------------------------------------------------------- #

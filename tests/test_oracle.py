@@ -460,6 +460,27 @@ def test_tiny_transformer_step_finite_difference():
         assert abs((lu - ld) / (2 * h) - grads["blocks"][0][name][pos]) < 1e-7, name
 
 
+@pytest.mark.parametrize("decoupled,wd", [(False, 0.0), (False, 0.1), (True, 0.1), (True, 0.0)])
+def test_adam_and_sgd_vs_torch_optim(decoupled, wd):
+    rng = np.random.default_rng(50)
+    w0 = rng.normal(size=37)
+    grads = [rng.normal(size=37) * s for s in (1.0, 0.1, 3.0, 1e-3)]
+    lr, b1, b2, eps = 3e-3, 0.9, 0.999, 1e-8
+    p = torch.tensor(w0, dtype=torch.float64, requires_grad=True)
+    opt = (torch.optim.AdamW if decoupled else torch.optim.Adam)([p], lr=lr, betas=(b1, b2), eps=eps, weight_decay=wd)
+    w, m, v = w0.copy(), np.zeros(37), np.zeros(37)
+    for t, g in enumerate(grads, start=1):
+        p.grad = torch.tensor(g, dtype=torch.float64)
+        opt.step()
+        w, m, v = O.adam_step(w, g, m, v, lr, b1, b2, eps, wd, t, decoupled)
+        np.testing.assert_allclose(w, p.detach().numpy(), rtol=1e-12, atol=1e-14)
+    p = torch.tensor(w0, dtype=torch.float64, requires_grad=True)
+    opt = torch.optim.SGD([p], lr=0.05)
+    p.grad = torch.tensor(grads[0], dtype=torch.float64)
+    opt.step()
+    np.testing.assert_allclose(O.sgd_step(w0, grads[0], 0.05), p.detach().numpy(), rtol=1e-15)
+
+
 def test_c_oracle_round_class(orc):
     for n in [1, 512, 513, 990, 1000, 1024, 1025, 4096, 5000, 123457, (1 << 20) + 1]:
         assert orc.orc_round_class(n) == O.round_class(n)

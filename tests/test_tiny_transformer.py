@@ -107,3 +107,28 @@ def test_step_full_size_properties(device):
     assert np.abs(lm.sum(axis=0)).max() <= 2e-2 * np.abs(lm).sum(axis=0).max()
     # untouched embedding rows would be zero; with 16384 uniform tokens over 65 symbols all rows are hit
     assert (np.abs(g1["embed"]).sum(axis=1) > 0).all()
+
+
+def test_training_reduces_the_loss(device):
+    # forward + backward + AdamW in a loop on one fixed batch: the loss must fall well below
+    # chance, and the first update must equal the oracle's AdamW applied to the step's gradients
+    V, d, ff, L, H, B, T = 17, 64, 128, 2, 2, 4, 32
+    rng = np.random.Generator(np.random.PCG64(72_000))
+    params = init_params(rng, V, d, ff, L)
+    model = TinyTransformer(device, V, d, ff, L, H, compute_dtype=F32)
+    model.load_params(params)
+    ids = AnyBuffer.from_numpy(device, integers(72, 1, (B, T), 0, V, np.int32))
+    labels = AnyBuffer.from_numpy(device, integers(72, 2, (B, T), 0, V, np.int32))
+    first = model.step(ids, labels, B, T).item()
+    g0 = _flatten(model.gradients())
+    model.adam_step(lr=3e-3, weight_decay=0.01, decoupled=True)
+    after = _flatten(model.parameters())
+    for name, w0 in _flatten(params).items():
+        f = lambda h: float(np.float32(h))  # the hyper-parameters as the library receives them
+        want, _, _ = O.adam_step(w0, g0[name], 0.0, 0.0, f(3e-3), f(0.9), f(0.999), f(1e-8), f(0.01), 1, True)
+        np.testing.assert_allclose(after[name], want, rtol=1e-5, atol=1e-7, err_msg=name)
+    for _ in range(60):
+        loss = model.step(ids, labels, B, T)
+        model.adam_step(lr=3e-3, weight_decay=0.01, decoupled=True)
+    last = loss.item()
+    assert first > math.log(V) - 0.5 and last < 0.5 * first, (first, last)
