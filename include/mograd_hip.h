@@ -331,6 +331,27 @@ int mg_scatter_add(const void* indices, const void* values, void* dst, int64_t n
                    int64_t num_rows, int64_t row_size, int idx_dtype, int dtype, mg_stream stream);
 
 /* ------------------------------------------------------------------------------------ */
+/* Row softmax, its gradient, argmax.  Contiguous operands, float dtypes, fp32 arithmetic. */
+/* ------------------------------------------------------------------------------------ */
+
+/* y = softmax over the last axis of (rows, cols).  Replaces mograd_softmax for a
+ * contiguous source, kernels/__init__.mojo:1015-1030 (kernels/softmax.mojo:19-38). */
+int mg_softmax(const void* x, void* y, int64_t rows, int64_t cols, int dtype, mg_stream stream);
+
+/* dst = y * (upstream - sum over the row of y * upstream).  Replaces mograd_softmax_grad,
+ * kernels/__init__.mojo:1062-1090 (kernels/softmax.mojo:76-98). */
+int mg_softmax_grad(const void* y, const void* upstream, void* dst, int64_t rows, int64_t cols,
+                    int dtype, mg_stream stream);
+
+/* dst(outer, inner) = index along the middle axis of a contiguous (outer, reduce, inner)
+ * array of its largest value, stored as a value of `dtype` like the reference does.  A
+ * value wins only if strictly greater: ties go to the lowest index, NaN never wins, an
+ * all-NaN or empty lane gives 0.  Replaces mograd_argmax_axis for contiguous sources,
+ * kernels/__init__.mojo:1269-1301 (kernels/reduce.mojo:208-239). */
+int mg_argmax_axis(const void* a, void* dst, int64_t outer, int64_t reduce, int64_t inner, int dtype,
+                   mg_stream stream);
+
+/* ------------------------------------------------------------------------------------ */
 /* Optimizer updates on flat fp32 arrays (parameters, gradients and moments are fp32 in   */
 /* the reference).  One streaming kernel each; in place.                                  */
 /* ------------------------------------------------------------------------------------ */

@@ -96,6 +96,9 @@ PROTOTYPES = {
     "mg_linear_bwd_fused": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _l, _i, _i, _i, _p], True),
     "mg_sum_axis": (_i, [_p, _p, _l, _l, _l, _i, _p], True),
     "mg_relu_grad": (_i, [_p, _p, _p, _l, _i, _p], True),
+    "mg_softmax": (_i, [_p, _p, _l, _l, _i, _p], True),
+    "mg_softmax_grad": (_i, [_p, _p, _p, _l, _l, _i, _p], True),
+    "mg_argmax_axis": (_i, [_p, _p, _l, _l, _l, _i, _p], True),
     "mg_adam_step": (_i, [_p, _p, _p, _p, _l, _f, _f, _f, _f, _f, _l, _i, _p], True),
     "mg_sgd_step": (_i, [_p, _p, _l, _f, _p], True),
     "mg_add": (_i, [_p, _p, _p, _l, _i, _p], True),

@@ -587,6 +587,47 @@ def scatter_add(node: Node, inputs: List[AnyBuffer], device: Device) -> List[Any
     return [out]
 
 
+def softmax(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """SOFTMAX[a] over the last axis.  runtime/__init__.mojo (softmax), kernels/__init__.mojo:1015-1030."""
+    layout = node.src(0).layout()
+    _require_contiguous(node, 1, "softmax")
+    _require_float(node.dtype(), "softmax")
+    cols = layout.shape(layout.rank() - 1)
+    rows = layout.numel() // cols
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_softmax(inputs[0].data_ptr(), out.data_ptr(), rows, cols, node.dtype(), device.stream)
+    return [out]
+
+
+def softmax_grad(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """SOFTMAX_GRAD[y, upstream] (mograd/grad.mojo:232-234).  kernels/__init__.mojo:1062-1090."""
+    la = node.src(0).layout()
+    _require_contiguous(node, 2, "softmax_grad")
+    _require_float(node.dtype(), "softmax_grad")
+    size = la.shape(la.rank() - 1)
+    N = la.numel() // size
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_softmax_grad(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), N, size, node.dtype(),
+                               device.stream)
+    return [out]
+
+
+def argmax(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """ARGMAX{axis}: index of the first largest value, stored in the tensor's float dtype.
+    runtime/__init__.mojo:402-405; without `axis` the whole tensor is one lane."""
+    layout = node.src(0).layout()
+    _require_contiguous(node, 1, "argmax")
+    _require_float(node.dtype(), "argmax")
+    if "axis" in node.attrs():
+        outer, reduce_size, inner = layout.reduce_dims(int(node.attrs()["axis"]))
+    else:
+        outer, reduce_size, inner = 1, layout.numel(), 1
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_argmax_axis(inputs[0].data_ptr(), out.data_ptr(), outer, reduce_size, inner, node.dtype(),
+                              device.stream)
+    return [out]
+
+
 # Op type -> exec function, the rows of the reference's rule table that belong to this
 # path (mograd/runtime/__init__.mojo:113-167).
 SCHEDULER_RULES = {
@@ -597,6 +638,9 @@ SCHEDULER_RULES = {
     "GATHER": gather,
     "SCATTER_ADD": scatter_add,
     "RELU_GRAD": relu_grad,
+    "SOFTMAX": softmax,
+    "SOFTMAX_GRAD": softmax_grad,
+    "ARGMAX": argmax,
     "SUM": sum,
     "MATMUL": matmul,
     "MATMUL_BT": matmul_t,

@@ -25,6 +25,8 @@ Pinning (what makes each function trustworthy without running the reference):
                         <gather(W, i), Y> = <W, scatter_add(i, Y)>; torch index_add_
   tiny_transformer_step torch autograd (f64) on the same model, finite differences
   adam_step / sgd_step  torch.optim.Adam / AdamW / SGD over several steps (f64)
+  softmax / softmax_grad torch.softmax and its autograd (f64), rows sum to 1 / to 0
+  argmax_axis           numpy.argmax on NaN-free input (first occurrence), hand cases
   round_class           tests/test_memory.mojo:18-30 (1000 -> 1024, 1025 -> 1152)
 All of the above are exercised in tests/test_oracle.py.
 """
@@ -462,6 +464,41 @@ def tiny_transformer_step(params, ids, labels, n_heads, eps=1e-5, store=None):
         grads["blocks"].insert(0, g)
     grads["embed"] = r(scatter_add(ids.reshape(-1), dh_, V))
     return float(loss), grads
+
+
+# --------------------------------------------------------------------------- #
+# Softmax, its gradient, argmax
+# --------------------------------------------------------------------------- #
+
+
+def softmax(x):
+    """Row softmax over the last axis.  kernels/softmax.mojo:19-38 (wraps MAX nn.softmax)."""
+    x = np.asarray(x, dtype=F64)
+    e = np.exp(x - x.max(axis=-1, keepdims=True))
+    return e / e.sum(axis=-1, keepdims=True)
+
+
+def softmax_grad(y, upstream):
+    """y * (upstream - sum_c y * upstream).  kernels/softmax.mojo:76-98."""
+    y = np.asarray(y, dtype=F64)
+    up = np.asarray(upstream, dtype=F64)
+    return y * (up - (y * up).sum(axis=-1, keepdims=True))
+
+
+def argmax_axis(a, axis):
+    """Index of the first strictly-largest value along `axis`, by the reference's loop:
+    start from -inf at index 0, replace only on `v > best` (kernels/reduce.mojo:225-236).
+    Ties go to the lowest index; NaN never wins."""
+    a = np.moveaxis(np.asarray(a, dtype=F64), axis, -1)
+    flat = a.reshape(-1, a.shape[-1])
+    out = np.zeros(flat.shape[0], dtype=np.int64)
+    for r in range(flat.shape[0]):
+        best, idx = -np.inf, 0
+        for i, v in enumerate(flat[r]):
+            if v > best:
+                best, idx = v, i
+        out[r] = idx
+    return out.reshape(a.shape[:-1])
 
 
 # --------------------------------------------------------------------------- #

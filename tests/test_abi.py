@@ -84,5 +84,5 @@ def test_scheduler_rules_cover_the_path():
     from mograd_amd import SCHEDULER_RULES
 
     assert set(SCHEDULER_RULES) == {
-        "ADD", "RELU", "CAST", "CONTIGUOUS", "GATHER", "SCATTER_ADD", "RELU_GRAD", "SUM", "MATMUL", "MATMUL_BT", "MATMUL_BIAS_BT", "LAYER_NORM", "LAYER_NORM_GRAD", "FLASH_ATTN",
+        "ADD", "RELU", "CAST", "CONTIGUOUS", "GATHER", "SCATTER_ADD", "RELU_GRAD", "SOFTMAX", "SOFTMAX_GRAD", "ARGMAX", "SUM", "MATMUL", "MATMUL_BT", "MATMUL_BIAS_BT", "LAYER_NORM", "LAYER_NORM_GRAD", "FLASH_ATTN",
         "FLASH_ATTN_GRAD", "CROSS_ENTROPY", "CROSS_ENTROPY_GRAD"}

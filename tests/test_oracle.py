@@ -481,6 +481,30 @@ def test_adam_and_sgd_vs_torch_optim(decoupled, wd):
     np.testing.assert_allclose(O.sgd_step(w0, grads[0], 0.05), p.detach().numpy(), rtol=1e-15)
 
 
+def test_softmax_and_argmax_pins():
+    rng = np.random.default_rng(60)
+    x = rng.normal(size=(5, 3, 17)) * 4
+    up = rng.normal(size=(5, 3, 17))
+    tx = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    ty = torch.softmax(tx, dim=-1)
+    ty.backward(torch.tensor(up))
+    y = O.softmax(x)
+    np.testing.assert_allclose(y, ty.detach().numpy(), atol=1e-15)
+    np.testing.assert_allclose(y.sum(-1), 1.0, atol=1e-14)
+    g = O.softmax_grad(y, up)
+    np.testing.assert_allclose(g, tx.grad.numpy(), atol=1e-14)
+    np.testing.assert_allclose(g.sum(-1), 0.0, atol=1e-14)  # the softmax Jacobian annihilates constants
+    # argmax: first occurrence, like numpy on NaN-free data, along any axis
+    a = rng.integers(0, 4, size=(6, 7, 5)).astype(np.float64)  # many ties
+    for axis in (0, 1, 2, -1):
+        np.testing.assert_array_equal(O.argmax_axis(a, axis), np.argmax(a, axis=axis))
+    # hand cases for the reference's loop: NaN never wins, all -inf or all NaN gives 0
+    assert O.argmax_axis([[np.nan, 1.0, 3.0, 3.0]], -1)[0] == 2
+    assert O.argmax_axis([[np.nan, np.nan]], -1)[0] == 0
+    assert O.argmax_axis([[-np.inf, -np.inf]], -1)[0] == 0
+    assert O.argmax_axis([[2.0, np.nan, 5.0, np.nan]], -1)[0] == 2
+
+
 def test_c_oracle_round_class(orc):
     for n in [1, 512, 513, 990, 1000, 1024, 1025, 4096, 5000, 123457, (1 << 20) + 1]:
         assert orc.orc_round_class(n) == O.round_class(n)
