@@ -546,12 +546,12 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
 // ---- dK, dV ------------------------------------------------------------------------------
 
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
-__global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_mfma_kernel(
+__global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma_kernel(
     const T* __restrict__ d_o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
     const T* __restrict__ mask, const float* __restrict__ lse, const float* __restrict__ delta, T* __restrict__ dk,
     T* __restrict__ dv, AttnDims a, float scale) {
   constexpr int BNK = 128;                 // keys per workgroup
-  constexpr int BQ = DP <= 64 ? 64 : 32;   // queries per step (LDS budget)
+  constexpr int BQ = 64;                   // queries per step
   constexpr int MT = BQ / 32, KS = DP / 16, DT = DP / 32;
   // Two copies of every staged tile: step i computes from copy i % 2 while the tile of step
   // i + 1 is written into the other, so one barrier per step suffices.
