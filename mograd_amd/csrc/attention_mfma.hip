@@ -390,10 +390,12 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
                                                                        const float* __restrict__ delta,
                                                                        T* __restrict__ dq, AttnDims a, float scale) {
   constexpr int BM = 128 * MQ, BN = 64, KS = DP / 16, DT = DP / 32;
-  // Two copies of each staged tile: one barrier per step.
-  __shared__ __attribute__((aligned(16))) uint16_t k_rows_s[2][BN * row_stride<DP>()];
-  __shared__ __attribute__((aligned(16))) uint16_t v_rows_s[2][BN * row_stride<DP>()];
-  __shared__ __attribute__((aligned(16))) uint32_t k_tr_s[2][DP * tr_stride_dw<BN>()];
+  // Two copies of each staged tile (one barrier per step) while two workgroups still fit in
+  // a CU's LDS; for head dims above 64 one copy and two barriers per step.
+  constexpr int NBUF = DP <= 64 ? 2 : 1;
+  __shared__ __attribute__((aligned(16))) uint16_t k_rows_s[NBUF][BN * row_stride<DP>()];
+  __shared__ __attribute__((aligned(16))) uint16_t v_rows_s[NBUF][BN * row_stride<DP>()];
+  __shared__ __attribute__((aligned(16))) uint32_t k_tr_s[NBUF][DP * tr_stride_dw<BN>()];
 
   const int nqb = (a.S + BM - 1) / BM;
   // (batch, head) varies fastest across consecutive workgroups, heaviest query blocks first.
@@ -446,24 +448,38 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
   TileStager<T, BN, DP> ks_stage, vs_stage;
   ks_stage.fetch(kbase, ld, 0, a.S, a.D);
   vs_stage.fetch(vbase, ld, 0, a.S, a.D);
-  ks_stage.commit_rows(k_rows_s[0]);
-  ks_stage.commit_transposed(k_tr_s[0]);
-  vs_stage.commit_rows(v_rows_s[0]);
-  if (BN < n_end) {
-    ks_stage.fetch(kbase, ld, BN, a.S, a.D);
-    vs_stage.fetch(vbase, ld, BN, a.S, a.D);
+  if constexpr (NBUF == 2) {
+    ks_stage.commit_rows(k_rows_s[0]);
+    ks_stage.commit_transposed(k_tr_s[0]);
+    vs_stage.commit_rows(v_rows_s[0]);
+    if (BN < n_end) {
+      ks_stage.fetch(kbase, ld, BN, a.S, a.D);
+      vs_stage.fetch(vbase, ld, BN, a.S, a.D);
+    }
   }
   int cur = 0;
-  for (int n0 = 0; n0 < n_end; n0 += BN, cur ^= 1) {
-    // Copy `cur` is complete and every wave has finished reading the other copy.
-    __syncthreads();
-    if (n0 + BN < n_end) {
-      ks_stage.commit_rows(k_rows_s[cur ^ 1]);
-      ks_stage.commit_transposed(k_tr_s[cur ^ 1]);
-      vs_stage.commit_rows(v_rows_s[cur ^ 1]);
-      if (n0 + 2 * BN < n_end) {
-        ks_stage.fetch(kbase, ld, n0 + 2 * BN, a.S, a.D);
-        vs_stage.fetch(vbase, ld, n0 + 2 * BN, a.S, a.D);
+  for (int n0 = 0; n0 < n_end; n0 += BN, cur ^= (NBUF - 1)) {
+    if constexpr (NBUF == 2) {
+      // Copy `cur` is complete and every wave has finished reading the other copy.
+      __syncthreads();
+      if (n0 + BN < n_end) {
+        ks_stage.commit_rows(k_rows_s[cur ^ 1]);
+        ks_stage.commit_transposed(k_tr_s[cur ^ 1]);
+        vs_stage.commit_rows(v_rows_s[cur ^ 1]);
+        if (n0 + 2 * BN < n_end) {
+          ks_stage.fetch(kbase, ld, n0 + 2 * BN, a.S, a.D);
+          vs_stage.fetch(vbase, ld, n0 + 2 * BN, a.S, a.D);
+        }
+      }
+    } else {
+      __syncthreads();  // every wave has finished reading the previous tile
+      ks_stage.commit_rows(k_rows_s[0]);
+      ks_stage.commit_transposed(k_tr_s[0]);
+      vs_stage.commit_rows(v_rows_s[0]);
+      __syncthreads();
+      if (n0 + BN < n_end) {
+        ks_stage.fetch(kbase, ld, n0 + BN, a.S, a.D);
+        vs_stage.fetch(vbase, ld, n0 + BN, a.S, a.D);
       }
     }
     const uint16_t* k_rows = k_rows_s[cur];
