@@ -181,14 +181,36 @@ template <typename T, int VEC, int WG>
 __device__ __forceinline__ void stream_max_sum(const T* __restrict__ xr, int64_t C, float* slots, int& phase, float& m_out,
                                                float& s_out) {
   float m = -INFINITY, s = 0.f;
-  for (int64_t c = static_cast<int64_t>(threadIdx.x) * VEC; c < C; c += static_cast<int64_t>(WG) * VEC) {
+  constexpr int U = 4;  // chunks in flight per thread: the loop is bound by memory-level parallelism
+  const int64_t step = static_cast<int64_t>(WG) * VEC;
+  int64_t c = static_cast<int64_t>(threadIdx.x) * VEC;
+  for (; c + (U - 1) * step < C; c += U * step) {
+    float v[U][VEC];
+#pragma unroll
+    for (int u = 0; u < U; ++u) VecIO<T, VEC>::load(xr + c + u * step, v[u]);
+    float cm = v[0][0];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) cm = fmaxf(cm, v[u][e]);
+    if (cm > m) {
+      s *= fast_exp2((m - cm) * kLog2e);  // exp2(-inf) == 0 on the first chunk
+      m = cm;
+    }
+    const float m2 = m * kLog2e;
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) s += fast_exp2(fmaf(v[u][e], kLog2e, -m2));
+  }
+  for (; c < C; c += step) {
     float v[VEC];
     VecIO<T, VEC>::load(xr + c, v);
     float cm = v[0];
 #pragma unroll
     for (int e = 1; e < VEC; ++e) cm = fmaxf(cm, v[e]);
     if (cm > m) {
-      s *= fast_exp2((m - cm) * kLog2e);  // exp2(-inf) == 0 on the first chunk
+      s *= fast_exp2((m - cm) * kLog2e);
       m = cm;
     }
     const float m2 = m * kLog2e;
@@ -280,7 +302,32 @@ __global__ __launch_bounds__(WG) void ce_grad_stream_kernel(const T* __restrict_
   const float shift = m + logf(s);
   const int64_t id = DENSE ? 0 : load_id(labels, row, id64 != 0);
   float acc[1] = {0.f};
-  for (int64_t c = static_cast<int64_t>(threadIdx.x) * VEC; c < C; c += static_cast<int64_t>(WG) * VEC) {
+  constexpr int U = DENSE ? 1 : 4;  // integer labels: four chunks in flight per thread
+  const int64_t step = static_cast<int64_t>(WG) * VEC;
+  int64_t c0 = static_cast<int64_t>(threadIdx.x) * VEC;
+  if constexpr (!DENSE) {
+    for (; c0 + (U - 1) * step < C; c0 += U * step) {
+      float v[U][VEC];
+#pragma unroll
+      for (int u = 0; u < U; ++u) VecIO<T, VEC>::load(xr + c0 + u * step, v[u]);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t c = c0 + u * step;
+        float out[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          float p = fast_exp2(fmaf(v[u][e], kLog2e, -m2)) * inv_sum;
+          if (c + e == id) {
+            p -= 1.0f;
+            acc[0] += v[u][e] - shift;
+          }
+          out[e] = p * scale;
+        }
+        VecIO<T, VEC>::store(out_row + c, out);
+      }
+    }
+  }
+  for (int64_t c = c0; c < C; c += step) {
     float v[VEC], out[VEC];
     VecIO<T, VEC>::load(xr + c, v);
     if constexpr (DENSE) {
