@@ -47,7 +47,7 @@ __device__ __forceinline__ int64_t load_id(const void* ids, int64_t row, bool id
 // ------------------------------------------------------------------------------------
 
 template <typename T, int VEC, int TPR, int VPT, int WG, bool DENSE>
-__global__ __launch_bounds__(WG, (TPR == 256 && VPT > 32) ? 2 : 1) void ce_rows_kernel(
+__global__ __launch_bounds__(WG, (TPR == 256 && VPT * VEC > 128) ? 2 : 1) void ce_rows_kernel(
     const T* __restrict__ logits, const void* __restrict__ labels, const T* __restrict__ upstream,
     float* __restrict__ rowloss, T* __restrict__ dlogits, int64_t N, int C, int id64) {
   constexpr int RPW = WG / TPR;
@@ -442,15 +442,17 @@ struct CrossEntropyOps {
     else if (chunks <= 1024) *s = {256, 4};
     else if (chunks <= 2048) *s = {512, 4};
     else if (chunks <= 4096) *s = {512, 8};
+    else if (WIDE == 8 && wide && chunks <= 6400) *s = {256, 25};  // 16-bit rows up to 51200 columns: see below
     else if (chunks <= 8192) *s = {512, 16};
-    else if (wide && chunks <= 12800) *s = {256, 50};
+    else if (WIDE == 4 && wide && chunks <= 12800) *s = {256, 50};
     else if (wide && chunks <= 16384) *s = {1024, 16};
     else return false;
-    // Rows of 8193..12800 chunks (the 50304-column fp32 case): 256 threads x 50 chunks by
+    // Rows of about 50k columns (8193..12800 fp32 chunks, 4097..6400 16-bit chunks: 200
+    // values per thread either way): 256 threads x 50 (fp32) or x 25 (16-bit) chunks by
     // default, which leaves room for two workgroups per CU so that one row's arithmetic
     // overlaps the other's memory traffic.  MOGRAD_HIP_CE_WIDE_ROW=512|1024 selects the
     // 512 x 25 or 1024 x 13 layout instead (tuning aid).
-    if (wide && chunks > 8192 && chunks <= 12800) {
+    if (WIDE == 4 && wide && chunks > 8192 && chunks <= 12800) {
       const int pick = env_int("MOGRAD_HIP_CE_WIDE_ROW", 256);
       if (pick == 512) *s = {512, 25};
       if (pick == 1024) *s = {1024, 13};
@@ -492,6 +494,9 @@ struct CrossEntropyOps {
     MG_CE_CASE(512, 4);
     MG_CE_CASE(512, 8);
     MG_CE_CASE(512, 16);
+    if constexpr (VEC == 8) {
+      MG_CE_CASE(256, 25);
+    }
     if constexpr (VEC > 1) {
       MG_CE_CASE(256, 50);
       MG_CE_CASE(512, 25);
