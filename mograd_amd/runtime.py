@@ -496,8 +496,7 @@ def sum(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     if "axis" not in node.attrs():
         raise MogradError(2, "sum: the full reduction is outside the backward hot path")
     layout = node.src(0).layout()
-    if not layout.is_contiguous():
-        raise MogradError(2, "sum: strided source is outside the backward hot path; materialise it first")
+    inputs = _materialise(node, inputs, device, 1)
     outer, reduce_size, inner = layout.reduce_dims(int(node.attrs()["axis"]))
     out = AnyBuffer.create(node.dtype(), device, node.numel())
     device.lib.mg_sum_axis(inputs[0].data_ptr(), out.data_ptr(), outer, reduce_size, inner, node.dtype(),
@@ -507,24 +506,34 @@ def sum(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
 
 def relu_grad(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     """RELU_GRAD[relu_out, upstream].  runtime/__init__.mojo:351-352."""
-    for i in (0, 1):
-        if not node.src(i).layout().is_contiguous():
-            raise MogradError(2, "relu_grad: strided operand is outside the backward hot path")
+    inputs = _materialise(node, inputs, device, 2)
     out = AnyBuffer.create(node.dtype(), device, node.numel())
     device.lib.mg_relu_grad(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), node.numel(), node.dtype(),
                             device.stream)
     return [out]
 
 
-def _require_contiguous(node: Node, count: int, who: str) -> None:
+def _materialise(node: Node, inputs: List[AnyBuffer], device: Device, count: int) -> List[AnyBuffer]:
+    """The first `count` operands as contiguous buffers.  The reference reads strided views
+    element by element inside each kernel (`*_strided` exports, kernels/strided.mojo); here a
+    strided operand is first copied row-major with mg_contiguous and the contiguous kernel
+    runs on the copy: same values, one extra pass for the rare strided case."""
+    out = list(inputs)
     for i in range(count):
-        if not node.src(i).layout().is_contiguous():
-            raise MogradError(2, f"{who}: strided operand is outside this path; materialise it with contiguous first")
+        layout = node.src(i).layout()
+        if layout.is_contiguous():
+            continue
+        dtype = node.src(i).dtype()
+        tmp = AnyBuffer.create(dtype, device, layout.numel())
+        device.lib.mg_contiguous(inputs[i].data_ptr(), tmp.data_ptr(), layout.rank(), _i64_array(layout.shape()),
+                                 _i64_array(layout.stride()), dtype, device.stream)
+        out[i] = tmp
+    return out
 
 
 def add(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     """ADD[a, b] (residual connections, gradient accumulation).  runtime/__init__.mojo:319-333."""
-    _require_contiguous(node, 2, "add")
+    inputs = _materialise(node, inputs, device, 2)
     out = AnyBuffer.create(node.dtype(), device, node.numel())
     device.lib.mg_add(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), node.numel(), node.dtype(),
                       device.stream)
@@ -533,7 +542,7 @@ def add(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
 
 def relu(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     """RELU[a].  runtime/__init__.mojo:296-297."""
-    _require_contiguous(node, 1, "relu")
+    inputs = _materialise(node, inputs, device, 1)
     out = AnyBuffer.create(node.dtype(), device, node.numel())
     device.lib.mg_relu(inputs[0].data_ptr(), out.data_ptr(), node.numel(), node.dtype(), device.stream)
     return [out]
@@ -541,7 +550,7 @@ def relu(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]
 
 def cast(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     """CAST[a] to node.dtype().  runtime/__init__.mojo:300-311."""
-    _require_contiguous(node, 1, "cast")
+    inputs = _materialise(node, inputs, device, 1)
     out = AnyBuffer.create(node.dtype(), device, node.numel())
     device.lib.mg_cast(inputs[0].data_ptr(), out.data_ptr(), node.numel(), node.src(0).dtype(), node.dtype(),
                        device.stream)
@@ -564,8 +573,11 @@ def gather(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffe
     lb = node.src(1).layout()
     if la.rank() != 2:  # op.mojo:367-368
         raise MogradError(1, "gather expects a 2D source tensor [num_rows, row_size]")
-    if not lb.is_contiguous():
-        raise MogradError(2, "gather: strided indices are outside this path")
+    if not lb.is_contiguous():  # strided indices: copy them row-major first
+        idx = AnyBuffer.create(node.src(1).dtype(), device, lb.numel())
+        device.lib.mg_contiguous(inputs[1].data_ptr(), idx.data_ptr(), lb.rank(), _i64_array(lb.shape()),
+                                 _i64_array(lb.stride()), node.src(1).dtype(), device.stream)
+        inputs = [inputs[0], idx]
     out = AnyBuffer.create(node.dtype(), device, node.numel())
     device.lib.mg_gather(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), lb.numel(), la.shape(0),
                          la.shape(1), la.stride(0), la.stride(1), node.src(1).dtype(), node.dtype(), device.stream)
@@ -579,7 +591,7 @@ def scatter_add(node: Node, inputs: List[AnyBuffer], device: Device) -> List[Any
     lb = node.src(1).layout()
     if lb.rank() != la.rank() + 1:  # op.mojo:375-376
         raise MogradError(1, "scatter_add expects values shaped [*indices.shape, row_size]")
-    _require_contiguous(node, 2, "scatter_add")
+    inputs = _materialise(node, inputs, device, 2)
     row_size = lb.shape(lb.rank() - 1)
     out = AnyBuffer.create(node.dtype(), device, node.numel())
     device.lib.mg_scatter_add(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), la.numel(),
@@ -590,7 +602,7 @@ def scatter_add(node: Node, inputs: List[AnyBuffer], device: Device) -> List[Any
 def softmax(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     """SOFTMAX[a] over the last axis.  runtime/__init__.mojo (softmax), kernels/__init__.mojo:1015-1030."""
     layout = node.src(0).layout()
-    _require_contiguous(node, 1, "softmax")
+    inputs = _materialise(node, inputs, device, 1)
     _require_float(node.dtype(), "softmax")
     cols = layout.shape(layout.rank() - 1)
     rows = layout.numel() // cols
@@ -602,7 +614,7 @@ def softmax(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuff
 def softmax_grad(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     """SOFTMAX_GRAD[y, upstream] (mograd/grad.mojo:232-234).  kernels/__init__.mojo:1062-1090."""
     la = node.src(0).layout()
-    _require_contiguous(node, 2, "softmax_grad")
+    inputs = _materialise(node, inputs, device, 2)
     _require_float(node.dtype(), "softmax_grad")
     size = la.shape(la.rank() - 1)
     N = la.numel() // size
@@ -616,7 +628,7 @@ def argmax(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffe
     """ARGMAX{axis}: index of the first largest value, stored in the tensor's float dtype.
     runtime/__init__.mojo:402-405; without `axis` the whole tensor is one lane."""
     layout = node.src(0).layout()
-    _require_contiguous(node, 1, "argmax")
+    inputs = _materialise(node, inputs, device, 1)
     _require_float(node.dtype(), "argmax")
     if "axis" in node.attrs():
         outer, reduce_size, inner = layout.reduce_dims(int(node.attrs()["axis"]))

@@ -170,3 +170,32 @@ def test_embedding_grad_adjoint_full_size(device):
     ones = np.ones((n, 8), np.float32)
     hist = _run(device, "SCATTER_ADD", Layout(V, 8), [(idx, Layout(n), I32), (ones, Layout(n, 8), F32)], F32)
     np.testing.assert_array_equal(hist[:, 0], np.bincount(idx, minlength=V).astype(np.float32))
+
+
+def test_strided_operands_are_materialised(device):
+    # The reference's *_strided kernels read views element by element; here the scheduler entry
+    # copies a strided operand row-major first.  Same values either way.
+    a = normal(69, 0, (6, 8))
+    b = normal(69, 1, (8, 6))
+    at = Layout(6, 8).transpose()            # (8, 6) view of a
+    got = _run(device, "ADD", Layout(8, 6), [(a, at, F32), (b, Layout(8, 6), F32)], F32)
+    np.testing.assert_array_equal(got, a.T + b)
+    every_other = Layout(6, 8).slice_axis(1, 0, 8, 2)   # (6, 4), stride (8, 2)
+    got = _run(device, "RELU", Layout(6, 4), [(a, every_other, F32)], F32)
+    np.testing.assert_array_equal(got, np.maximum(a[:, ::2], 0))
+    got = _run(device, "CAST", Layout(8, 6), [(a, at, F32)], BF16)
+    np.testing.assert_array_equal(got, round_to_dtype(a.T, BF16))
+    up = normal(69, 2, (8, 6))
+    got = _run(device, "RELU_GRAD", Layout(8, 6), [(a, at, F32), (up, Layout(8, 6), F32)], F32)
+    np.testing.assert_array_equal(got, np.where(a.T > 0, up, 0).astype(np.float32))
+    got = _run(device, "SUM", Layout(6), [(a, at, F32)], F32, {"axis": 0})
+    np.testing.assert_allclose(got, a.T.sum(axis=0), rtol=1e-5, atol=1e-6)
+    got = _run(device, "SOFTMAX", Layout(8, 6), [(a, at, F32)], F32)
+    np.testing.assert_allclose(got, O.softmax(a.T), rtol=1e-4, atol=1e-6)
+    got = _run(device, "ARGMAX", Layout(8), [(a, at, F32)], F32, {"axis": 1})
+    np.testing.assert_array_equal(got, np.argmax(a.T, axis=1).astype(np.float32))
+    w = normal(69, 3, (10, 4))
+    idx = integers(69, 4, (3, 5), 0, 10, np.int64)
+    idx_t = Layout(3, 5).transpose()         # (5, 3) view of the index array
+    got = _run(device, "GATHER", Layout(5, 3, 4), [(w, Layout(10, 4), F32), (idx, idx_t, I64)], F32)
+    np.testing.assert_array_equal(got, w[idx.T])
