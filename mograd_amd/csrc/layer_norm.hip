@@ -39,8 +39,9 @@ static int ln_bwd(const void* dy, const void* x, const void* gamma, const float*
   if (!dgamma || !dbeta) return fail(MG_ERR_INVALID, "layer_norm_bwd: null pointer argument");
   hipStream_t s = to_stream(stream);
   if (rows == 0) {  // the column sums of an empty matrix are zero
-    MG_HIP(hipMemsetAsync(dgamma, 0, static_cast<size_t>(cols) * dtype_size(dtype), s));
-    MG_HIP(hipMemsetAsync(dbeta, 0, static_cast<size_t>(cols) * dtype_size(dtype), s));
+    // zero fill by kernel, not hipMemsetAsync: safe to record into a HIP graph
+    MG_TRY(mg_fill(dgamma, 0.0, cols, dtype, s));
+    MG_TRY(mg_fill(dbeta, 0.0, cols, dtype, s));
     return MG_OK;
   }
   if (!dy || !x || !gamma || !dx) return fail(MG_ERR_INVALID, "layer_norm_bwd: null pointer argument");

@@ -96,8 +96,9 @@ __global__ __launch_bounds__(256) void relu_grad_kernel(const T* __restrict__ ou
 template <typename T>
 static int colsum_typed(const T* a, T* dst, int64_t outer, int64_t reduce, int64_t inner, hipStream_t stream) {
   if (reduce == 0) {
-    MG_HIP(hipMemsetAsync(dst, 0, static_cast<size_t>(outer * inner) * sizeof(T), stream));
-    return MG_OK;
+    // zero fill by kernel, not hipMemsetAsync: safe to record into a HIP graph
+    const int dtype = sizeof(T) == 4 ? MG_F32 : MG_F16;  // all-zero bits are zero in every float type
+    return mg_fill(dst, 0.0, outer * inner, dtype, stream);
   }
   if (inner == 1) {
     hipLaunchKernelGGL((rowsum_kernel<T>), dim3(static_cast<unsigned>(ceil_div(outer, 4))), dim3(256), 0, stream, a, dst,
