@@ -409,7 +409,7 @@ struct LayerNormOps {
   // enough that the (groups, cols) partial sums stay a small fraction of the traffic.
   static int64_t bwd_groups(int64_t rows, int rows_per_iter, int wg) {
     const int64_t cus = device_info().cu_count;
-    int64_t per_cu = wg >= 512 ? 1 : (wg >= 256 ? 2 : 4);
+    int64_t per_cu = wg >= 1024 ? 1 : (wg >= 256 ? 2 : 4);
     per_cu = env_int("MOGRAD_HIP_LN_GROUPS_PER_CU", static_cast<int>(per_cu));
     int64_t groups = cus * per_cu;
     const int64_t max_groups = ceil_div(rows, rows_per_iter);
