@@ -1,0 +1,102 @@
+"""Seeded sweeps over odd shapes: every case is small enough for the float64 oracle, and
+the point is the dispatch (aligned / ragged / split-K / generic GEMM paths, attention tile
+edges, row-kernel shape ladders), not the size."""
+import math
+
+import numpy as np
+import pytest
+
+from helpers import ATOL_F32, RTOL_F32, assert_close
+from oracle import oracle_np as O
+
+pytestmark = pytest.mark.gpu
+
+from mograd_amd import BF16, F16, F32, I32, AnyBuffer  # noqa: E402
+from mograd_amd.runtime import round_to_dtype  # noqa: E402
+
+RT = {F32: 2e-4, F16: 2e-3, BF16: 1.6e-2}
+
+
+def test_random_linear_shapes(device):
+    rng = np.random.Generator(np.random.PCG64(95_000))
+    lib, st = device.lib, device.stream
+    for case in range(60):
+        dtype = (F32, F16, BF16)[case % 3]
+        M, N, K = (int(v) for v in rng.integers(1, 300, 3))
+        if case % 5 == 0:
+            K = int(rng.integers(1024, 3000))  # long reductions: split-K for the small outputs
+        x = round_to_dtype(rng.standard_normal((M, K)).astype(np.float32), dtype)
+        w = round_to_dtype((rng.standard_normal((N, K)) * 0.1).astype(np.float32), dtype)
+        b = round_to_dtype(rng.standard_normal(N).astype(np.float32), dtype)
+        dy = round_to_dtype(rng.standard_normal((M, N)).astype(np.float32), dtype)
+        bx, bw, bb, bdy = (AnyBuffer.from_numpy(device, a, dtype) for a in (x, w, b, dy))
+        y, dx, dw, db = (AnyBuffer.create(dtype, device, n) for n in (M * N, M * K, N * K, N))
+        lib.mg_matmul_bias_bt(bx.data_ptr(), bw.data_ptr(), bb.data_ptr(), y.data_ptr(), 1, M, N, K, K, 1, K, 1, M * K,
+                              N * K, dtype, st)
+        lib.mg_linear_bwd(bdy.data_ptr(), bx.data_ptr(), bw.data_ptr(), dx.data_ptr(), dw.data_ptr(), db.data_ptr(), M, N,
+                          K, dtype, st)
+        rt = RT[dtype]
+        for got, want, name in ((y.to_numpy((M, N)), O.matmul_bias_bt(x, w, b), "y"),
+                                (dx.to_numpy((M, K)), O.linear_grad_x(dy, w), "dx"),
+                                (dw.to_numpy((N, K)), O.linear_grad_w(dy, x), "dw"),
+                                (db.to_numpy(), O.linear_grad_b(dy), "db")):
+            assert_close(got, want, rt, rt * max(np.abs(want).max(), 1e-3), f"case {case} {(M, N, K)} dtype {dtype} {name}")
+
+
+def test_random_attention_shapes(device):
+    rng = np.random.Generator(np.random.PCG64(96_000))
+    lib, st = device.lib, device.stream
+    for case in range(24):
+        dtype = (BF16, F16)[case % 2]
+        B, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
+        S = int(rng.integers(1, 300))
+        D = int(rng.integers(1, 17)) * 8
+        causal = case % 3 == 0
+        scale = 1.0 / math.sqrt(D)
+        q, k, v = (round_to_dtype(rng.standard_normal((B, S, H, D)).astype(np.float32), dtype) for _ in range(3))
+        do = round_to_dtype(rng.standard_normal((B, H, S, D)).astype(np.float32), dtype)
+        bq, bk, bv, bdo = (AnyBuffer.from_numpy(device, a, dtype) for a in (q, k, v, do))
+        n = B * S * H * D
+        o, dq, dk, dv = (AnyBuffer.create(dtype, device, n) for _ in range(4))
+        lse = AnyBuffer.create(F32, device, B * H * S)
+        lib.mg_flash_attn_fwd(bq.data_ptr(), bk.data_ptr(), bv.data_ptr(), None, o.data_ptr(), lse.data_ptr(), B, S, H, D,
+                              scale, int(causal), 0, dtype, st)
+        lib.mg_flash_attn_bwd(bdo.data_ptr(), o.data_ptr(), bq.data_ptr(), bk.data_ptr(), bv.data_ptr(), None,
+                              lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, S, H, D, scale, int(causal),
+                              0, dtype, st)
+        wo, wl = O.sdpa_fwd(q, k, v, None, causal, scale)
+        wdq, wdk, wdv = O.sdpa_bwd(q, k, v, do, None, causal, scale)
+        tol = 2e-2 if dtype == BF16 else 4e-3
+        what = f"case {case} B{B} S{S} H{H} D{D} causal={causal} dtype {dtype}"
+        assert_close(lse.to_numpy((B, H, S)), wl, 1e-3, 2e-2 if dtype == BF16 else 4e-3, what + " lse")
+        for got, want, name in ((o.to_numpy((B, H, S, D)), wo, "o"), (dq.to_numpy((B, S, H, D)), wdq, "dq"),
+                                (dk.to_numpy((B, S, H, D)), wdk, "dk"), (dv.to_numpy((B, S, H, D)), wdv, "dv")):
+            assert_close(got, want, tol, tol * max(np.abs(want).max(), 1e-3), what + " " + name)
+
+
+def test_random_row_kernel_shapes(device):
+    rng = np.random.Generator(np.random.PCG64(97_000))
+    lib, st = device.lib, device.stream
+    for case in range(40):
+        rows = int(rng.integers(1, 70))
+        cols = int(rng.choice([1, 3, 8, 17, 64, 100, 256, 257, 1000, 1024, 2052, 4100, 9000]))
+        x = rng.standard_normal((rows, cols)).astype(np.float32) * 2 + 0.5
+        dy = rng.standard_normal((rows, cols)).astype(np.float32)
+        g = rng.uniform(0.5, 1.5, cols).astype(np.float32)
+        bx, bdy, bg = (AnyBuffer.from_numpy(device, a) for a in (x, dy, g))
+        dx, dg, db = (AnyBuffer.create(F32, device, n) for n in (rows * cols, cols, cols))
+        lib.mg_layer_norm_bwd(bdy.data_ptr(), bx.data_ptr(), bg.data_ptr(), dx.data_ptr(), dg.data_ptr(), db.data_ptr(),
+                              rows, cols, 1e-5, F32, st)
+        wdx, wdg, wdb = O.layer_norm_bwd(dy, x, g, 1e-5)
+        what = f"case {case} ({rows},{cols})"
+        # narrow rows have a large 1/sqrt(var + eps): hold dx to the gradient's own scale
+        assert_close(dx.to_numpy((rows, cols)), wdx, RTOL_F32, max(ATOL_F32, 1e-4 * np.abs(wdx).max()), what + " dx")
+        assert_close(dg.to_numpy(), wdg, RTOL_F32, max(ATOL_F32, 1e-5 * np.abs(dy).sum(0).max() * np.abs(wdg).max() / max(np.abs(wdg).max(), 1)), what + " dgamma")
+        assert_close(db.to_numpy(), wdb, RTOL_F32, max(ATOL_F32, 2e-6 * np.abs(dy).sum(0).max()), what + " dbeta")
+        ids = rng.integers(0, cols, rows).astype(np.int32)
+        bids = AnyBuffer.from_numpy(device, ids)
+        loss, dl = AnyBuffer.create(F32, device, 1), AnyBuffer.create(F32, device, rows * cols)
+        lib.mg_cross_entropy_fused_ids(bx.data_ptr(), bids.data_ptr(), None, loss.data_ptr(), dl.data_ptr(), rows, cols,
+                                       F32, I32, st)
+        assert_close(loss.item(), O.cross_entropy_ids(x, ids), RTOL_F32, ATOL_F32, what + " loss")
+        assert_close(dl.to_numpy((rows, cols)), O.cross_entropy_grad_ids(x, ids), RTOL_F32, RTOL_F32 / rows, what + " dlogits")
