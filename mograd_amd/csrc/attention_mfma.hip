@@ -205,7 +205,26 @@ __device__ __forceinline__ floatx16 zero16() {
   return z;
 }
 
-__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+// The two lanes that share a query (lane and lane ^ 32) exchange a value with one
+// v_permlane32_swap instead of a round trip through LDS (ds_bpermute): afterwards `lo` holds
+// lanes 0..31 of v in both halves of the wave and `hi` lanes 32..63.  The no-ops cover the
+// wait states between a VALU write of the operands, the swap, and a VALU read of the
+// results, which the compiler cannot see inside the asm.
+__device__ __forceinline__ void split_halves(float v, float& lo, float& hi) {
+  lo = v;
+  hi = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+}
+__device__ __forceinline__ float max_halves(float v) {
+  float lo, hi;
+  split_halves(v, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float sum_halves(float v) {
+  float lo, hi;
+  split_halves(v, lo, hi);
+  return lo + hi;
+}
 
 // Packed store of four consecutive accumulator registers (four consecutive d) times `f`.
 template <typename T>
@@ -304,7 +323,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[nt][r]);
-      mx = fmaxf(mx, xor32(mx)) * c;
+      mx = max_halves(mx) * c;
       const float m_new = fmaxf(m_run, mx);
       corr = fexp2(m_run - m_new);
       float lsum = 0.f;
@@ -316,7 +335,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
           s[nt][r] = p;
           lsum += p;
         }
-      lsum += xor32(lsum);
+      lsum = sum_halves(lsum);
       l_run = l_run * corr + lsum;
       m_run = m_new;
     } else {
@@ -334,7 +353,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
           s[nt][r] = sv;
           mx = fmaxf(mx, sv);
         }
-      mx = fmaxf(mx, xor32(mx));
+      mx = max_halves(mx);
       const float m_new = fmaxf(m_run, mx);
       // m_new is -inf only for rows past the end of the sequence (all their keys masked)
       const float m_use = m_new == -INFINITY ? 0.f : m_new;
@@ -348,7 +367,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
           s[nt][r] = p;
           lsum += p;
         }
-      lsum += xor32(lsum);
+      lsum = sum_halves(lsum);
       l_run = l_run * corr + lsum;
       m_run = m_new;
     }
