@@ -120,6 +120,46 @@ struct TileStager {
   static constexpr int TASKS = PAIRS * CH;
   static constexpr int PER = (TASKS + kAttnThreads - 1) / kAttnThreads;
   uint4 lo[PER], hi[PER];
+  // Walk over consecutive R-row tiles: where this thread reads in the next tile.
+  static_assert(kAttnThreads % PAIRS == 0, "chunk i of a thread must be its chunk 0 shifted by whole columns");
+  static constexpr int CHUNK_STEP = kAttnThreads / PAIRS * 8;  // columns between a thread's consecutive chunks
+  const T* base_;
+  const T* src_;
+  int64_t ld_;
+  int next_;
+
+  // Starts a walk at row r0 of the matrix whose row r begins at base + r * ld (elements).
+  __device__ __forceinline__ void begin(const T* __restrict__ base, int64_t ld, int r0) {
+    base_ = base;
+    ld_ = ld;
+    next_ = r0;
+    src_ = base + (r0 + 2 * (threadIdx.x % PAIRS)) * ld + (threadIdx.x / PAIRS) * 8;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      lo[i] = make_uint4(0, 0, 0, 0);
+      hi[i] = make_uint4(0, 0, 0, 0);
+    }
+  }
+  // Fetches the next tile of the walk.  A tile that lies inside the matrix takes the short
+  // path: two unconditional loads per chunk from pointers that advance by a constant (chunks
+  // of padding columns never load and keep their zeros); only the ragged last tile pays for
+  // per-row bounds checks.
+  __device__ __forceinline__ void fetch_next(int r_end, int D) {
+    if (next_ + R <= r_end) {
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int idx = threadIdx.x + i * kAttnThreads;
+        if (idx < TASKS && (idx / PAIRS) * 8 < D) {
+          lo[i] = *reinterpret_cast<const uint4*>(src_ + i * CHUNK_STEP);
+          hi[i] = *reinterpret_cast<const uint4*>(src_ + ld_ + i * CHUNK_STEP);
+        }
+      }
+    } else {
+      fetch(base_, ld_, next_, r_end, D);
+    }
+    src_ += R * ld_;
+    next_ += R;
+  }
 
   // Rows [r0, r0 + R) of a matrix whose row r starts at base + r * ld (elements); D valid
   // columns; rows >= r_end and columns >= D read as zero.
@@ -282,13 +322,15 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
 
   const int n_end = CAUSAL ? min(a.S, qb * BM + BM) : a.S;
   TileStager<T, BN, DP> ks_stage, vs_stage;
-  ks_stage.fetch(kbase, ld, 0, a.S, a.D);
-  vs_stage.fetch(vbase, ld, 0, a.S, a.D);
+  ks_stage.begin(kbase, ld, 0);
+  vs_stage.begin(vbase, ld, 0);
+  ks_stage.fetch_next(a.S, a.D);
+  vs_stage.fetch_next(a.S, a.D);
   ks_stage.commit_rows(k_rows_s[0]);
   vs_stage.commit_transposed(v_tr_s[0]);
   if (BN < n_end) {
-    ks_stage.fetch(kbase, ld, BN, a.S, a.D);
-    vs_stage.fetch(vbase, ld, BN, a.S, a.D);
+    ks_stage.fetch_next(a.S, a.D);
+    vs_stage.fetch_next(a.S, a.D);
   }
   int cur = 0;
   for (int n0 = 0; n0 < n_end; n0 += BN, cur ^= 1) {
@@ -298,8 +340,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
       ks_stage.commit_rows(k_rows_s[cur ^ 1]);
       vs_stage.commit_transposed(v_tr_s[cur ^ 1]);
       if (n0 + 2 * BN < n_end) {
-        ks_stage.fetch(kbase, ld, n0 + 2 * BN, a.S, a.D);
-        vs_stage.fetch(vbase, ld, n0 + 2 * BN, a.S, a.D);
+        ks_stage.fetch_next(a.S, a.D);
+        vs_stage.fetch_next(a.S, a.D);
       }
     }
     const uint16_t* k_rows = k_rows_s[cur];
@@ -465,15 +507,17 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
 
   const int n_end = CAUSAL ? min(a.S, qb * BM + BM) : a.S;
   TileStager<T, BN, DP> ks_stage, vs_stage;
-  ks_stage.fetch(kbase, ld, 0, a.S, a.D);
-  vs_stage.fetch(vbase, ld, 0, a.S, a.D);
+  ks_stage.begin(kbase, ld, 0);
+  vs_stage.begin(vbase, ld, 0);
+  ks_stage.fetch_next(a.S, a.D);
+  vs_stage.fetch_next(a.S, a.D);
   if constexpr (NBUF == 2) {
     ks_stage.commit_rows(k_rows_s[0]);
     ks_stage.commit_transposed(k_tr_s[0]);
     vs_stage.commit_rows(v_rows_s[0]);
     if (BN < n_end) {
-      ks_stage.fetch(kbase, ld, BN, a.S, a.D);
-      vs_stage.fetch(vbase, ld, BN, a.S, a.D);
+      ks_stage.fetch_next(a.S, a.D);
+      vs_stage.fetch_next(a.S, a.D);
     }
   }
   int cur = 0;
@@ -486,8 +530,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
         ks_stage.commit_transposed(k_tr_s[cur ^ 1]);
         vs_stage.commit_rows(v_rows_s[cur ^ 1]);
         if (n0 + 2 * BN < n_end) {
-          ks_stage.fetch(kbase, ld, n0 + 2 * BN, a.S, a.D);
-          vs_stage.fetch(vbase, ld, n0 + 2 * BN, a.S, a.D);
+          ks_stage.fetch_next(a.S, a.D);
+          vs_stage.fetch_next(a.S, a.D);
         }
       }
     } else {
@@ -497,8 +541,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
       vs_stage.commit_rows(v_rows_s[0]);
       __syncthreads();
       if (n0 + BN < n_end) {
-        ks_stage.fetch(kbase, ld, n0 + BN, a.S, a.D);
-        vs_stage.fetch(vbase, ld, n0 + BN, a.S, a.D);
+        ks_stage.fetch_next(a.S, a.D);
+        vs_stage.fetch_next(a.S, a.D);
       }
     }
     const uint16_t* k_rows = k_rows_s[cur];
@@ -637,16 +681,20 @@ __global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma
   const int m_begin = CAUSAL ? (kb * BNK / BQ) * BQ : 0;
   TileStager<T, BQ, DP> q_stage, do_stage;
   float lse_next, delta_next;
-  // Global -> registers for the step starting at query m.
+  q_stage.begin(qbase, ld, m_begin);
+  do_stage.begin(dobase, a.D, m_begin);
+  // Global -> registers for the next step of the walk, which starts at query m.
+  // The row statistics go first: the compiler guards the reuse of their registers with a
+  // wait for every load issued before it, which must not include this step's tile loads.
   auto fetch_step = [&](int m) {
-    q_stage.fetch(qbase, ld, m, a.S, a.D);
-    do_stage.fetch(dobase, a.D, m, a.S, a.D);
     lse_next = INFINITY;
     delta_next = 0.f;
     if (threadIdx.x < BQ && m + threadIdx.x < a.S) {
       lse_next = lse[bh * a.S + m + threadIdx.x];  // scaled to log2 units when it is committed
       delta_next = delta[bh * a.S + m + threadIdx.x];
     }
+    q_stage.fetch_next(a.S, a.D);
+    do_stage.fetch_next(a.S, a.D);
   };
   // Registers -> LDS copy `buf`.
   auto commit_step = [&](int buf) {
