@@ -71,7 +71,7 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
   const int M = static_cast<int>(g.M), N = static_cast<int>(g.N), K = static_cast<int>(g.K);
   const int64_t cus = device_info().cu_count;
   int splits = 1;
-  if (g.batch == 1 && blocks < cus && g.K >= 1024) {
+  if (g.batch <= 65535 && blocks < cus && g.K >= 1024) {
     splits = static_cast<int>(ceil_div(env_int("MOGRAD_HIP_GEMM_SPLITK_WG_PER_CU", 2) * cus, blocks));
     const int max_splits = static_cast<int>(g.K / env_int("MOGRAD_HIP_GEMM_SPLITK_MIN_K", 256));
     if (splits > max_splits) splits = max_splits;
@@ -91,13 +91,15 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
   }
   const int k_per_split = static_cast<int>(ceil_div(ceil_div(g.K, splits), kG16BK) * kG16BK);
   splits = static_cast<int>(ceil_div(g.K, k_per_split));
+  // The batches of C are contiguous ((batch, M, N) row-major), so partials and the reduction
+  // treat them as one array of batch * M * N elements.
   Scratch partial;
-  const int64_t numel = g.M * g.N;
+  const int64_t numel = g.batch * g.M * g.N;
   MG_TRY(partial.take(static_cast<int64_t>(splits) * numel * static_cast<int64_t>(sizeof(float))));
   hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, false, true, RAGGED>),
-                     dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(splits)), dim3(kGemmThreads), 0, stream, a,
-                     b, bias, c, partial.as<float>(), M, N, K, lda, ldb, g.N, g.bsa, g.bsb, numel, tiles_m, tiles_n,
-                     k_per_split, GemmEpilogue<T>{nullptr, nullptr, 0});
+                     dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(splits), static_cast<unsigned>(g.batch)),
+                     dim3(kGemmThreads), 0, stream, a, b, bias, c, partial.as<float>(), M, N, K, lda, ldb, g.N, g.bsa,
+                     g.bsb, g.M * g.N, tiles_m, tiles_n, k_per_split, GemmEpilogue<T>{nullptr, nullptr, 0});
   MG_LAUNCH_CHECK();
   const unsigned rblocks = static_cast<unsigned>(ceil_div(numel, 256));
   if (bias)

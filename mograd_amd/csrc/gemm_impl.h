@@ -436,7 +436,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
   __shared__ __attribute__((aligned(16))) uint16_t lds_b[kGemmBN * kG16Stride];
 
   const int tiles = tiles_m * tiles_n;
-  const int batch = SPLIT_K ? 0 : blockIdx.x / tiles;
+  // Split along K: grid (tiles, splits, batch).  Otherwise the batch index is folded into x.
+  const int batch = SPLIT_K ? blockIdx.z : blockIdx.x / tiles;
   int tm, tn;
   gemm_tile_of_block(blockIdx.x % tiles, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * kGemmBM;
@@ -557,7 +558,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
         const int row = m0 + wm + ti * 32 + (r / 4) * 8 + (lane / 32) * 4 + (r % 4);
         if (row < M) {
           if constexpr (SPLIT_K)
-            partial[(static_cast<int64_t>(blockIdx.y) * M + row) * N + col] = acc[ti][tj][r];
+            partial[((static_cast<int64_t>(blockIdx.y) * gridDim.z + batch) * M + row) * N + col] = acc[ti][tj][r];
           else {
             const int64_t at = batch * bsc + static_cast<int64_t>(row) * ldc + col;
             C[at] = gemm_finish<T>(acc[ti][tj][r] + bv, ep, at);

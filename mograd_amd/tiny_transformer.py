@@ -73,6 +73,11 @@ class TinyTransformer:
                 place(f"blocks.{layer}.{name}", block_shapes[name])
         place("lm_head", (V, d))
         self.total = off
+        # wq, wk, wv of a layer are consecutive equal slices: the batch stride of the batched
+        # projection.  Their gradients can come from one batched product only when the slices
+        # are not padded apart (the library writes batches of a result back to back).
+        self.qkv_stride = self.slices["blocks.0.wk"].offset - self.slices["blocks.0.wq"].offset if n_layers else 0
+        self.qkv_packed = self.qkv_stride == d * d
         self.master = AnyBuffer.create(F32, device, self.total, fill=0.0)  # fp32 master weights
         self.grads = AnyBuffer.create(F32, device, self.total, fill=0.0)   # fp32 gradients, same layout
         self.work = AnyBuffer.create(self.cd, device, self.total)          # weights in the compute dtype
@@ -126,12 +131,14 @@ class TinyTransformer:
         self.saved: List[dict] = []
         for _ in range(self.L):
             self.saved.append({
-                "x1": new(n * d), "q": new(n * d), "k": new(n * d), "v": new(n * d), "o": new(n * d),
+                # Q, K and V of a layer sit back to back: one batched product writes all three
+                "x1": new(n * d), "qkv": new(3 * n * d), "o": new(n * d),
                 "lse": new(B * self.H * T, F32), "ctx": new(n * d),
                 "h_mid": new(n * d), "x2": new(n * d), "a": new(n * ff),
                 "mean1": new(n, F32), "rstd1": new(n, F32), "mean2": new(n, F32), "rstd2": new(n, F32),
             })
-        self.tmp = {name: new(n * d) for name in ("dh", "dres", "dctx", "do", "dq", "dk", "dv", "dx_a")}
+        self.tmp = {name: new(n * d) for name in ("dh", "dres", "dctx", "do", "dx_a")}
+        self.tmp["dqkv"] = new(3 * n * d)  # dQ, dK, dV back to back, as the batched dW product reads them
         self.tmp["da"] = new(n * ff)
         self.tmp["logits"] = new(n * V)
         self.tmp["dlogits"] = new(n * V)
@@ -162,6 +169,8 @@ class TinyTransformer:
                 lib.mg_matmul_bias_bt(x, w, bias, out, 1, n, N, K, K, 1, K, 1, n * K, N * K, cd, s)
 
         P = lambda buf: buf.data_ptr()
+        # i-th (n, d) third of a buffer that holds three activations back to back
+        part = lambda buf, i: C.c_void_p(buf.storage.ptr + i * n * d * DTYPE_SIZE[cd])
 
         lib.mg_cast(P(self.master), P(self.work), self.total, F32, cd, s)
 
@@ -172,12 +181,12 @@ class TinyTransformer:
             h_in, h_out = P(self.h[l]), P(self.h[l + 1])
             lib.mg_layer_norm_fwd_stats(h_in, w("ln1_g"), w("ln1_b"), P(c["x1"]), P(c["mean1"]), P(c["rstd1"]), n, d,
                                         self.eps, cd, s)
-            linear(P(c["x1"]), w("wq"), P(c["q"]), d, d)
-            linear(P(c["x1"]), w("wk"), P(c["k"]), d, d)
-            linear(P(c["x1"]), w("wv"), P(c["v"]), d, d)
+            # The three projections share x1: one batched product over (wq, wk, wv), which are
+            # consecutive equal slices of the weight arena (batch stride 0 on x1).
+            q, k, v = (part(c["qkv"], i) for i in range(3))
+            lib.mg_matmul_bt(P(c["x1"]), w("wq"), q, 3, n, d, d, d, 1, d, 1, 0, self.qkv_stride, cd, s)
             # (n, d) row-major is (B, T, H, dh): the layout the attention kernels take for Q, K, V
-            lib.mg_flash_attn_fwd(P(c["q"]), P(c["k"]), P(c["v"]), None, P(c["o"]), P(c["lse"]), B, T, H, dh, scale, 1,
-                                  0, cd, s)
+            lib.mg_flash_attn_fwd(q, k, v, None, P(c["o"]), P(c["lse"]), B, T, H, dh, scale, 1, 0, cd, s)
             # O comes back (B, H, T, dh); the projection wants (B, T, H*dh)
             lib.mg_contiguous(P(c["o"]), P(c["ctx"]), 4, i64(B, T, H, dh), i64(H * T * dh, dh, T * dh, 1), cd, s)
             lib.mg_matmul_bt_add(P(c["ctx"]), w("wo"), h_in, P(c["h_mid"]), 1, n, d, d, d, 1, d, 1, n * d, d * d, cd, s)
@@ -211,11 +220,19 @@ class TinyTransformer:
             lib.mg_linear_bwd(t["dh"], P(c["ctx"]), w("wo"), t["dctx"], g("wo"), None, n, d, d, cd, s)
             # dctx is (B, T, H, dh); the attention backward takes dO as (B, H, T, dh)
             lib.mg_contiguous(t["dctx"], t["do"], 4, i64(B, H, T, dh), i64(T * H * dh, dh, H * dh, 1), cd, s)
-            lib.mg_flash_attn_bwd(t["do"], P(c["o"]), P(c["q"]), P(c["k"]), P(c["v"]), None, P(c["lse"]), t["dq"],
-                                  t["dk"], t["dv"], B, T, H, dh, scale, 1, 0, cd, s)
-            lib.mg_linear_bwd(t["dq"], P(c["x1"]), w("wq"), t["dx_a"], g("wq"), None, n, d, d, cd, s)
-            lib.mg_linear_bwd_fused(t["dk"], P(c["x1"]), w("wk"), t["dx_a"], g("wk"), None, n, d, d, 1, 0, cd, s)
-            lib.mg_linear_bwd_fused(t["dv"], P(c["x1"]), w("wv"), t["dx_a"], g("wv"), None, n, d, d, 1, 0, cd, s)
+            q, k, v = (part(c["qkv"], i) for i in range(3))
+            dq, dk, dv = (part(self.tmp["dqkv"], i) for i in range(3))
+            lib.mg_flash_attn_bwd(t["do"], P(c["o"]), q, k, v, None, P(c["lse"]), dq, dk, dv, B, T, H, dh, scale, 1, 0,
+                                  cd, s)
+            # dx1 = dQ Wq + dK Wk + dV Wv: three products, the second and third accumulating
+            gq, gk, gv = (None, None, None) if self.qkv_packed else (g("wq"), g("wk"), g("wv"))
+            lib.mg_linear_bwd(dq, P(c["x1"]), w("wq"), t["dx_a"], gq, None, n, d, d, cd, s)
+            lib.mg_linear_bwd_fused(dk, P(c["x1"]), w("wk"), t["dx_a"], gk, None, n, d, d, 1, 0, cd, s)
+            lib.mg_linear_bwd_fused(dv, P(c["x1"]), w("wv"), t["dx_a"], gv, None, n, d, d, 1, 0, cd, s)
+            if self.qkv_packed:
+                # dW_b = dY_b^T x1 for the three projections as one batched product (split along
+                # the token axis inside the library): A = dY_b^T is element (o, t) at dy_b[t*d + o].
+                lib.mg_matmul(dq, P(c["x1"]), g("wq"), 3, d, d, n, 1, d, d, 1, n * d, 0, cd, s)
             lib.mg_layer_norm_bwd_stats(t["dx_a"], P(self.h[l]), w("ln1_g"), P(c["mean1"]), P(c["rstd1"]), t["dres"],
                                         g("ln1_g"), g("ln1_b"), n, d, cd, s)
             lib.mg_add(t["dh"], t["dres"], t["dh"], n * d, cd, s)

@@ -214,6 +214,27 @@ def test_bf16_linear_bwd_entry_gpt_shapes(device):
         assert_close(got, want, 1.6e-2, 1.6e-2 * np.abs(want).max(), name)
 
 
+@pytest.mark.parametrize("dtype,rtol", [(F16, 2e-3), (BF16, 1.6e-2)])
+@pytest.mark.parametrize("M,d", [(2048, 96), (1500, 72), (300, 65)])
+def test_batched_projections_share_an_operand(device, dtype, rtol, M, d):
+    # Three projections of one activation (the Q, K and V of an attention block) as one
+    # batched call with batch stride 0 on the shared operand, and their three weight
+    # gradients dW_b = dY_b^T X as one batched product that is split along K (= tokens).
+    lib, st = device.lib, device.stream
+    x = round_to_dtype(normal(53, 0, (M, d)), dtype)
+    w = round_to_dtype(normal(53, 1, (3, d, d), std=0.1), dtype)
+    dy = round_to_dtype(normal(53, 2, (3, M, d), std=0.5), dtype)
+    bx, bw, bdy = (AnyBuffer.from_numpy(device, a, dtype) for a in (x, w, dy))
+    y, dw = AnyBuffer.create(dtype, device, 3 * M * d), AnyBuffer.create(dtype, device, 3 * d * d)
+    lib.mg_matmul_bt(bx.data_ptr(), bw.data_ptr(), y.data_ptr(), 3, M, d, d, d, 1, d, 1, 0, d * d, dtype, st)
+    # A = dY_b^T: element (o, t) at dy_b[t * d + o]; B = X: element (t, i) at x[t * d + i]
+    lib.mg_matmul(bdy.data_ptr(), bx.data_ptr(), dw.data_ptr(), 3, d, d, M, 1, d, d, 1, M * d, 0, dtype, st)
+    want_y = np.einsum("tk,bnk->btn", x.astype(np.float64), w.astype(np.float64))
+    want_dw = np.einsum("bto,ti->boi", dy.astype(np.float64), x.astype(np.float64))
+    assert_close(y.to_numpy((3, M, d)), want_y, rtol, rtol * np.abs(want_y).max(), "y")
+    assert_close(dw.to_numpy((3, d, d)), want_dw, rtol, rtol * np.abs(want_dw).max(), "dw")
+
+
 # ---- fused epilogues: each must give exactly what the separate calls give -----------------
 
 FUSED_SHAPES = [(256, 384, 512), (200, 136, 264), (130, 65, 384), (64, 10, 256), (33, 7, 5), (4096, 128, 128),
