@@ -5,6 +5,9 @@ Inputs follow one rule everywhere: one numpy PCG64 generator per tensor, seeded 
 """
 from __future__ import annotations
 
+import json
+from pathlib import Path
+
 import numpy as np
 
 # Tolerances of the parity contract.
@@ -65,3 +68,10 @@ def assert_sum_close(got, want, term_l1, rtol=RTOL_F32, atol=ATOL_F32, what=""):
     bound = floor + rtol * np.abs(want)
     worst = float(np.max(err / bound))
     assert np.all(np.isfinite(got)) and worst <= 1.0, f"{what}: worst err/bound = {worst:.3g}"
+
+
+def golden(section: str) -> list:
+    """Entries of one section of tests/golden/reference_vectors.json: the golden vectors the
+    reference's own tests hold for this path (inputs, expected outputs, tolerance, citation)."""
+    with open(Path(__file__).resolve().parent / "golden" / "reference_vectors.json") as f:
+        return json.load(f)[section]

@@ -10,7 +10,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from helpers import ATOL_F32, RTOL_F32, assert_close, integers, normal
+from helpers import ATOL_F32, RTOL_F32, assert_close, golden, integers, normal
 from oracle import oracle_np as O
 
 pytestmark = pytest.mark.gpu
@@ -47,10 +47,9 @@ def _ce_grad(device, logits, labels, upstream=1.0, la=None, lb=None, dtype=F32):
 # ---- the reference's golden values -----------------------------------------------
 
 
-def test_goldens_contiguous(device):
-    assert abs(_ce(device, np.zeros((4, 10)), O.one_hot([0, 1, 2, 3], 10)) - 2.302585) < 1e-3
-    assert abs(_ce(device, np.zeros((2, 4)), np.full((2, 4), 0.25)) - 1.386294) < 1e-3
-    assert abs(_ce(device, [[100, 0, 0], [0, 100, 0]], [[1, 0, 0], [0, 1, 0]])) < 1e-3
+@pytest.mark.parametrize("g", golden("cross_entropy"), ids=lambda g: g["cite"])
+def test_goldens_contiguous(device, g):
+    assert abs(_ce(device, g["logits"], g["labels"]) - g["loss"]) < g["atol"]
 
 
 def test_goldens_strided(device):
@@ -66,12 +65,13 @@ def test_goldens_strided(device):
     assert abs(_ce(device, np.zeros((2, 2)), np.eye(2), lb=t) - 0.693147) < 1e-3
 
 
-def test_grad_golden_transposed_logits(device):
-    # tests/test_non_contiguous.mojo:302-310.  The gradient arrives in the layout of the
-    # transposed view; the expected numbers are for the underlying array a.
-    a = np.array([[1, 2], [3, 4]], np.float32)
-    d = _ce_grad(device, a, np.eye(2), la=Layout(2, 2).transpose())
-    np.testing.assert_allclose(d.T.reshape(-1), [-0.440398, 0.059601, 0.440398, -0.059601], atol=1e-3)
+@pytest.mark.parametrize("g", golden("cross_entropy_grad"), ids=lambda g: g["cite"])
+def test_grad_golden_transposed_logits(device, g):
+    # The logits operand is the transposed view of `a`; the gradient arrives in the layout of
+    # that view, and the expected numbers are for the underlying array a.
+    a = np.array(g["a"], np.float32)
+    d = _ce_grad(device, a, g["labels"], g["upstream"], la=Layout(*a.shape).transpose())
+    np.testing.assert_allclose(d.T.reshape(-1), g["grad_a_flat"], atol=g["atol"])
 
 
 def test_grad_rows_sum_to_zero_and_rank3(device):

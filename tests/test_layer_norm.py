@@ -7,7 +7,7 @@ reach every kernel layout, the benchmark shape, and the edge cases.
 import numpy as np
 import pytest
 
-from helpers import ATOL_F32, RTOL_F32, assert_close, assert_sum_close, normal, uniform
+from helpers import ATOL_F32, RTOL_F32, assert_close, assert_sum_close, golden, normal, uniform
 from oracle import oracle_np as O
 
 pytestmark = pytest.mark.gpu
@@ -41,26 +41,19 @@ def _ln_bwd(device, dy, x, gamma, eps=1e-5, dtype=F32):
 # ---- the reference's golden vectors, through the dispatch surface -------------------
 
 
-def test_fwd_goldens(device):
-    y = _ln_fwd(device, [[1, 2, 3, 4]], [1, 2, 1, 2], [0.1, 0.2, 0.1, 0.2])
-    np.testing.assert_allclose(y, [[-1.241641, -0.694427, 0.547214, 2.883282]], atol=1e-4)
-    y = _ln_fwd(device, [[1, 2, 3, 4], [-1, -2, -3, -4]], [1] * 4, [0] * 4)
-    want = [-1.341641, -0.447214, 0.447214, 1.341641]
-    np.testing.assert_allclose(y, [want, want[::-1]], atol=1e-4)
-    y = _ln_fwd(device, [[3, 3, 3, 3]], [1] * 4, [0.5] * 4)
-    np.testing.assert_allclose(y, [[0.5] * 4], atol=1e-4)
+@pytest.mark.parametrize("g", golden("layer_norm_fwd"), ids=lambda g: g["cite"])
+def test_fwd_goldens(device, g):
+    y = _ln_fwd(device, g["x"], g["gamma"], g["beta"], g["eps"])
+    np.testing.assert_allclose(y, g["y"], atol=g["atol"])
 
 
-def test_bwd_goldens(device):
-    x, dy = [[1.0, 2, 3, 4]], [[0.1, 0.2, 0.3, 0.4]]
-    dx, dg, db = _ln_bwd(device, dy, x, [1, 2, 1, 2])
-    np.testing.assert_allclose(dx, [[0.0, 0.089443, -0.178886, 0.089443]], atol=2e-4)
-    np.testing.assert_allclose(dg, [-0.134164, -0.089443, 0.134164, 0.536656], atol=2e-4)
-    np.testing.assert_allclose(db, [0.1, 0.2, 0.3, 0.4], atol=1e-5)
-    _, _, db2 = _ln_bwd(device, dy * 2, x * 2, [1] * 4)
-    np.testing.assert_allclose(db2, [0.2, 0.4, 0.6, 0.8], atol=1e-5)
-    dx0, _, _ = _ln_bwd(device, [[1, 1, 1, 1]], x, [1] * 4)
-    np.testing.assert_allclose(dx0, np.zeros((1, 4)), atol=1e-5)
+@pytest.mark.parametrize("g", golden("layer_norm_bwd"), ids=lambda g: g["cite"])
+def test_bwd_goldens(device, g):
+    got = dict(zip(("dx", "dgamma", "dbeta"), _ln_bwd(device, g["dy"], g["x"], g["gamma"], g["eps"])))
+    checked = [k for k in got if k in g]
+    assert checked
+    for k in checked:
+        np.testing.assert_allclose(got[k], g[k], atol=g["atol"], err_msg=k)
 
 
 # ---- random shapes: every register layout, the scalar path, the streaming fallback ---

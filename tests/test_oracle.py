@@ -10,6 +10,7 @@ import numpy as np
 import pytest
 import torch
 
+from helpers import golden
 from oracle import oracle_np as O
 
 ROOT = Path(__file__).resolve().parent.parent
@@ -21,31 +22,19 @@ ORACLE_SO = ROOT / "oracle" / "liboracle_c.so"
 # --------------------------------------------------------------------------- #
 
 
-def test_ln_fwd_goldens():
-    # tests/test_nn.mojo:283-324
-    y = O.layer_norm_fwd([[1, 2, 3, 4]], [1, 2, 1, 2], [0.1, 0.2, 0.1, 0.2])
-    np.testing.assert_allclose(y, [[-1.241641, -0.694427, 0.547214, 2.883282]], atol=1e-4)
-    y = O.layer_norm_fwd([[1, 2, 3, 4], [-1, -2, -3, -4]], [1] * 4, [0] * 4)
-    want = [-1.341641, -0.447214, 0.447214, 1.341641]
-    np.testing.assert_allclose(y, [want, want[::-1]], atol=1e-4)
-    y = O.layer_norm_fwd([[3, 3, 3, 3]], [1] * 4, [0.5] * 4)
-    np.testing.assert_allclose(y, [[0.5] * 4], atol=1e-4)
+@pytest.mark.parametrize("g", golden("layer_norm_fwd"), ids=lambda g: g["cite"])
+def test_ln_fwd_goldens(g):
+    y = O.layer_norm_fwd(g["x"], g["gamma"], g["beta"], g["eps"])
+    np.testing.assert_allclose(y, g["y"], atol=g["atol"])
 
 
-def test_ln_bwd_goldens():
-    # tests/test_grad.mojo:776-856
-    x = [[1.0, 2, 3, 4]]
-    dy = [[0.1, 0.2, 0.3, 0.4]]
-    dx, dg, db = O.layer_norm_bwd(dy, x, [1, 2, 1, 2])
-    np.testing.assert_allclose(dx, [[0.0, 0.089443, -0.178886, 0.089443]], atol=2e-4)
-    np.testing.assert_allclose(dg, [-0.134164, -0.089443, 0.134164, 0.536656], atol=2e-4)
-    np.testing.assert_allclose(db, [0.1, 0.2, 0.3, 0.4], atol=1e-5)
-    # two identical rows: dbeta doubles
-    _, _, db2 = O.layer_norm_bwd(dy * 2, x * 2, [1] * 4)
-    np.testing.assert_allclose(db2, [0.2, 0.4, 0.6, 0.8], atol=1e-5)
-    # uniform dy with gamma = 1 gives zero dx
-    dx0, _, _ = O.layer_norm_bwd([[1, 1, 1, 1]], x, [1] * 4)
-    np.testing.assert_allclose(dx0, np.zeros((1, 4)), atol=1e-5)
+@pytest.mark.parametrize("g", golden("layer_norm_bwd"), ids=lambda g: g["cite"])
+def test_ln_bwd_goldens(g):
+    got = dict(zip(("dx", "dgamma", "dbeta"), O.layer_norm_bwd(g["dy"], g["x"], g["gamma"], g["eps"])))
+    checked = [k for k in got if k in g]
+    assert checked
+    for k in checked:
+        np.testing.assert_allclose(got[k], g[k], atol=g["atol"], err_msg=k)
 
 
 def test_ln_bwd_matches_torch_autograd_and_invariants():
@@ -88,23 +77,19 @@ def test_ln_rank3_is_rows_of_last_dim():
 # --------------------------------------------------------------------------- #
 
 
-def test_ce_goldens():
-    # tests/test_ops.mojo:155-175
-    assert abs(O.cross_entropy(np.zeros((4, 10)), O.one_hot([0, 1, 2, 3], 10)) - 2.302585) < 1e-3
-    assert abs(O.cross_entropy(np.zeros((2, 4)), np.full((2, 4), 0.25)) - 1.386294) < 1e-3
-    assert abs(O.cross_entropy([[100, 0, 0], [0, 100, 0]], [[1, 0, 0], [0, 1, 0]])) < 1e-3
-    # tests/test_non_contiguous.mojo:275-299 (strided views; values after applying the view)
-    assert abs(O.cross_entropy([[0, 0], [0, 0]], [[0.5, 0.5], [0.5, 0.5]]) - 0.693147) < 1e-3
-    assert abs(O.cross_entropy(np.zeros((2, 2)), [[1, 0], [0, 1]]) - 0.693147) < 1e-3
+@pytest.mark.parametrize("g", golden("cross_entropy"), ids=lambda g: g["cite"])
+def test_ce_goldens(g):
+    assert abs(O.cross_entropy(g["logits"], g["labels"]) - g["loss"]) < g["atol"]
 
 
-def test_ce_grad_goldens():
-    # tests/test_non_contiguous.mojo:302-310: logits = a^T with a = [[1,2],[3,4]], labels = I;
-    # the expected gradient is with respect to a, i.e. the transpose of dlogits.
-    a = np.array([[1.0, 2], [3, 4]])
-    d = O.cross_entropy_grad(a.T, np.eye(2))
-    np.testing.assert_allclose(d.T.reshape(-1), [-0.440398, 0.059601, 0.440398, -0.059601], atol=1e-3)
-    # tests/test_grad.mojo:432-446: rows of the gradient sum to zero
+@pytest.mark.parametrize("g", golden("cross_entropy_grad"), ids=lambda g: g["cite"])
+def test_ce_grad_goldens(g):
+    d = O.cross_entropy_grad(np.array(g["a"], dtype=np.float64).T, g["labels"], g["upstream"])
+    np.testing.assert_allclose(d.T.reshape(-1), g["grad_a_flat"], atol=g["atol"])
+
+
+def test_ce_grad_rows_sum_to_zero():
+    # tests/test_grad.mojo:432-446
     d = O.cross_entropy_grad(np.ones((4, 10)), O.one_hot([0, 1, 2, 3], 10))
     np.testing.assert_allclose(d.sum(axis=1), 0, atol=1e-12)
 
@@ -242,8 +227,9 @@ def test_linear_grads_match_autograd():
 
 def test_round_class():
     # tests/test_memory.mojo:18-30 and mograd/memory.mojo:59-72
-    assert O.round_class(1000) == 1024 and O.round_class(1025) == 1152
-    assert O.round_class(1) == 512 and O.round_class(512) == 512 and O.round_class(513) == 576
+    for g in golden("pool_round_class"):
+        assert O.round_class(g["nbytes"]) == g["class_bytes"], g
+    assert O.round_class(512) == 512 and O.round_class(513) == 576
     assert O.round_class(4096) == 4096 and O.round_class(990) == 1024
     for n in [600, 5000, 123457, 1 << 20, (1 << 20) + 1, 3 << 28]:
         c = O.round_class(n)
