@@ -332,6 +332,7 @@ int main(int argc, char** argv) {
   // Pool behaviour seen through AnyBuffer (tests/test_memory.mojo:18-60): a freed block of the
   // 1024-byte class serves the next request that rounds to the same class.
   run_case("pool reuses a size class", [&]() -> std::string {
+    if (!dev.fn<decltype(&::mg_pool_enabled)>("mg_pool_enabled")()) return "";  // MOGRAD_POOL=0: nothing is cached
     void* first;
     {
       AnyBuffer a = AnyBuffer::create(float32, dev, 250);  // 1000 bytes -> class 1024
