@@ -39,14 +39,19 @@ static int launch_f32_mfma(const GemmArgs& g, hipStream_t stream) {
   const float* b = static_cast<const float*>(g.b);
   const float* bias = static_cast<const float*>(g.bias);
   float* c = static_cast<float*>(g.c);
+  // Two workgroups are resident per CU; a larger problem is walked by that many workgroups.
+  int64_t grid = 2 * static_cast<int64_t>(device_info().cu_count) * env_int("MOGRAD_HIP_GEMM_F32_ROUNDS", 1);
+  if (grid > blocks || env_int("MOGRAD_HIP_GEMM_F32_ROUNDS", 1) == 0) grid = blocks;
   if (bias)
-    hipLaunchKernelGGL((gemm_f32_mfma_kernel<A_KC, B_KC, true>), dim3(static_cast<unsigned>(blocks)), dim3(kGemmThreads),
+    hipLaunchKernelGGL((gemm_f32_mfma_kernel<A_KC, B_KC, true>), dim3(static_cast<unsigned>(grid)), dim3(kGemmThreads),
                        0, stream, a, b, bias, c, static_cast<int>(g.M), static_cast<int>(g.N), static_cast<int>(g.K), lda,
-                       ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n, epilogue_of<float>(g));
+                       ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n, static_cast<int>(blocks),
+                       epilogue_of<float>(g));
   else
-    hipLaunchKernelGGL((gemm_f32_mfma_kernel<A_KC, B_KC, false>), dim3(static_cast<unsigned>(blocks)),
+    hipLaunchKernelGGL((gemm_f32_mfma_kernel<A_KC, B_KC, false>), dim3(static_cast<unsigned>(grid)),
                        dim3(kGemmThreads), 0, stream, a, b, bias, c, static_cast<int>(g.M), static_cast<int>(g.N),
-                       static_cast<int>(g.K), lda, ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n, epilogue_of<float>(g));
+                       static_cast<int>(g.K), lda, ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n,
+                       static_cast<int>(blocks), epilogue_of<float>(g));
   MG_LAUNCH_CHECK();
   return MG_OK;
 }

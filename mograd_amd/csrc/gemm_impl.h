@@ -131,19 +131,27 @@ template <bool A_KC, bool B_KC, bool HAS_BIAS>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_kernel(
     const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias, float* __restrict__ C,
     int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb, int64_t bsc, int tiles_m,
-    int tiles_n, GemmEpilogue<float> ep) {
+    int tiles_n, int total_work, GemmEpilogue<float> ep_in) {
   __shared__ __attribute__((aligned(16))) float lds_a[kGemmBM * kKcStride];
   __shared__ __attribute__((aligned(16))) float lds_b[kGemmBN * kKcStride];
 
   const int tiles = tiles_m * tiles_n;
-  const int batch = blockIdx.x / tiles;
+  const float* const A_in = A;
+  const float* const B_in = B;
+  float* const C_in = C;
+  // The grid holds at most the workgroups that are resident at once; each takes output tiles
+  // work, work + gridDim.x, ...  Workgroups that share operand slabs then start every tile
+  // together, which keeps their fetches of the shared rows close in time.
+  for (int work = blockIdx.x; work < total_work; work += gridDim.x) {
+  const int batch = work / tiles;
   int tm, tn;
-  gemm_tile_of_block(blockIdx.x % tiles, tiles_m, tiles_n, tm, tn);
+  gemm_tile_of_block(work % tiles, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * kGemmBM;
   const int n0 = tn * kGemmBN;
-  A += batch * bsa;
-  B += batch * bsb;
-  C += batch * bsc;
+  A = A_in + batch * bsa;
+  B = B_in + batch * bsb;
+  C = C_in + batch * bsc;
+  GemmEpilogue<float> ep = ep_in;
   if (ep.residual) ep.residual += batch * bsc;
   if (ep.relu_mask) ep.relu_mask += batch * bsc;
 
@@ -207,6 +215,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_mfma_kernel(
         }
       }
     }
+  }  // tiles of this workgroup
 }
 
 // ------------------------------------------------------------------------------------
