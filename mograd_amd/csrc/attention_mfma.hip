@@ -120,6 +120,14 @@ struct TileStager {
   static constexpr int TASKS = PAIRS * CH;
   static constexpr int PER = (TASKS + kAttnThreads - 1) / kAttnThreads;
   uint4 lo[PER], hi[PER];
+  // Pair chunk `idx` -> (row pair, 8-column chunk).  Two neighbouring lanes take the two
+  // chunks of one row pair and the next two lanes the next pair, so that the eight lanes of
+  // one 128-bit LDS write cycle cover four row pairs x two chunks: with the tile's row stride
+  // those are eight different groups of four banks (lanes on consecutive row pairs alone
+  // would hit each group twice).
+  static_assert(CH % 2 == 0, "chunks are handed out two at a time");
+  static __device__ __forceinline__ int pair_of(int idx) { return (idx / 2) % PAIRS; }
+  static __device__ __forceinline__ int chunk_of(int idx) { return idx % 2 + 2 * (idx / (2 * PAIRS)); }
   // Walk over consecutive R-row tiles: where this thread reads in the next tile.
   static_assert(kAttnThreads % PAIRS == 0, "chunk i of a thread must be its chunk 0 shifted by whole columns");
   static constexpr int CHUNK_STEP = kAttnThreads / PAIRS * 8;  // columns between a thread's consecutive chunks
@@ -133,7 +141,7 @@ struct TileStager {
     base_ = base;
     ld_ = ld;
     next_ = r0;
-    src_ = base + (r0 + 2 * (threadIdx.x % PAIRS)) * ld + (threadIdx.x / PAIRS) * 8;
+    src_ = base + (r0 + 2 * pair_of(threadIdx.x)) * ld + chunk_of(threadIdx.x) * 8;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       lo[i] = make_uint4(0, 0, 0, 0);
@@ -149,7 +157,7 @@ struct TileStager {
 #pragma unroll
       for (int i = 0; i < PER; ++i) {
         const int idx = threadIdx.x + i * kAttnThreads;
-        if (idx < TASKS && (idx / PAIRS) * 8 < D) {
+        if (idx < TASKS && chunk_of(idx) * 8 < D) {
           lo[i] = *reinterpret_cast<const uint4*>(src_ + i * CHUNK_STEP);
           hi[i] = *reinterpret_cast<const uint4*>(src_ + ld_ + i * CHUNK_STEP);
         }
@@ -167,7 +175,7 @@ struct TileStager {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int idx = threadIdx.x + i * kAttnThreads;
-      const int p = idx % PAIRS, c = idx / PAIRS;
+      const int p = pair_of(idx), c = chunk_of(idx);
       const int ra = r0 + 2 * p;
       lo[i] = make_uint4(0, 0, 0, 0);
       hi[i] = make_uint4(0, 0, 0, 0);
@@ -181,7 +189,7 @@ struct TileStager {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int idx = threadIdx.x + i * kAttnThreads;
-      const int p = idx % PAIRS, c = idx / PAIRS;
+      const int p = pair_of(idx), c = chunk_of(idx);
       if (idx < TASKS) {
         *reinterpret_cast<uint4*>(lds + (2 * p) * row_stride<DP>() + c * 8) = lo[i];
         *reinterpret_cast<uint4*>(lds + (2 * p + 1) * row_stride<DP>() + c * 8) = hi[i];
@@ -193,7 +201,7 @@ struct TileStager {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int idx = threadIdx.x + i * kAttnThreads;
-      const int p = idx % PAIRS, c = idx / PAIRS;
+      const int p = pair_of(idx), c = chunk_of(idx);
       if (idx < TASKS) {
         const uint32_t a[4] = {lo[i].x, lo[i].y, lo[i].z, lo[i].w};
         const uint32_t b[4] = {hi[i].x, hi[i].y, hi[i].z, hi[i].w};
