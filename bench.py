@@ -422,7 +422,7 @@ def bench_gpt(args, dev) -> int:
     i64 = lambda *a: (C.c_int64 * len(a))(*a)  # noqa: E731
     sc = 1.0 / float(np.sqrt(dh))
     lib.mg_layer_norm_fwd_stats(P(x_d), P(gam), P(bet), P(out_d), P(mean), P(rstd), n, d, 1e-5, BF16, st)
-    lib.mg_flash_attn_fwd(P(q), P(k), P(v), None, P(o), P(lse), B, T, H, dh, sc, 1, 0, BF16, st)
+    lib.mg_flash_attn_fwd_bshd(P(q), P(k), P(v), None, P(o), P(lse), B, T, H, dh, sc, 1, 0, BF16, st)
     lib.mg_matmul_bt(P(x_d), P(w_vd), P(out_v), 1, n, V, d, d, 1, d, 1, n * d, V * d, BF16, st)
 
     def mm(x, w, out, N, K, bias=None):
@@ -445,11 +445,11 @@ def bench_gpt(args, dev) -> int:
         ("matmul_bias_bt bf16 (16384, 1536<-384)", mm(x_d, w_fd, out_ff, ff, d, bias_f), 2.0 * n * d * ff, "F", PF),
         ("matmul_bt bf16 (16384, 384<-1536)", mm(x_ff, w_df, out_d, d, ff), 2.0 * n * d * ff, "F", PF),
         ("matmul_bt bf16 lm_head (16384, 65<-384)", mm(x_d, w_vd, out_v, V, d), 2.0 * n * d * V, "F", PF),
-        ("flash_attn_bwd bf16 causal B64 H6 S256 D64 (5 B H S^2 D)",
-         lambda i: lib.mg_flash_attn_bwd(P(do), P(o), P(q), P(k), P(v), None, P(lse), P(dq), P(dk), P(dv), B, T, H, dh, sc, 1, 0, BF16, st),
+        ("flash_attn_bwd_bshd bf16 causal B64 H6 S256 D64 (5 B H S^2 D)",
+         lambda i: lib.mg_flash_attn_bwd_bshd(P(do), P(o), P(q), P(k), P(v), None, P(lse), P(dq), P(dk), P(dv), B, T, H, dh, sc, 1, 0, BF16, st),
          5.0 * attn_fl, "F", PF),
-        ("flash_attn_fwd bf16 causal B64 H6 S256 D64 (2 B H S^2 D)",
-         lambda i: lib.mg_flash_attn_fwd(P(q), P(k), P(v), None, P(o), P(lse), B, T, H, dh, sc, 1, 0, BF16, st), 2.0 * attn_fl, "F", PF),
+        ("flash_attn_fwd_bshd bf16 causal B64 H6 S256 D64 (2 B H S^2 D)",
+         lambda i: lib.mg_flash_attn_fwd_bshd(P(q), P(k), P(v), None, P(o), P(lse), B, T, H, dh, sc, 1, 0, BF16, st), 2.0 * attn_fl, "F", PF),
         ("layer_norm_bwd_stats bf16 (16384, 384)",
          lambda i: lib.mg_layer_norm_bwd_stats(P(dy_d), P(x_d), P(gam), P(mean), P(rstd), P(out_d), P(dgam), P(dbet), n, d, BF16, st),
          3 * n * d * e2 + 2 * n * 4 + 3 * d * e2, "B", None),
@@ -462,7 +462,7 @@ def bench_gpt(args, dev) -> int:
         ("add bf16 (16384 x 384)", lambda i: lib.mg_add(P(x_d), P(dy_d), P(out_d), n * d, BF16, st), 3 * n * d * e2, "B", None),
         ("relu bf16 (16384 x 1536)", lambda i: lib.mg_relu(P(x_ff), P(out_ff), n * ff, BF16, st), 2 * n * ff * e2, "B", None),
         ("relu_grad bf16 (16384 x 1536)", lambda i: lib.mg_relu_grad(P(x_ff), P(dy_ff), P(out_ff), n * ff, BF16, st), 3 * n * ff * e2, "B", None),
-        ("contiguous bf16 (B,H,T,dh) -> (B,T,H,dh)",
+        ("contiguous bf16 (B,H,T,dh) -> (B,T,H,dh) (not in the step since attention writes (B,T,H,dh))",
          lambda i: lib.mg_contiguous(P(o), P(out_d), 4, i64(B, T, H, dh), i64(H * T * dh, dh, T * dh, 1), BF16, st), 2 * n * d * e2, "B", None),
         ("gather bf16 16384 rows of (65, 384)", lambda i: lib.mg_gather(P(w_vd), P(ids), P(out_d), n, V, d, d, 1, I32, BF16, st),
          n * d * e2 + n * 4, "B", None),

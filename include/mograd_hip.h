@@ -389,6 +389,20 @@ int mg_flash_attn_bwd(const void* d_o, const void* o, const void* q, const void*
                       int64_t S, int64_t H, int64_t D, float scale, int causal, int has_bias,
                       int dtype, mg_stream stream);
 
+/* The same two operations with O and dO laid out (B,S,H,D) like Q, K and V, so that the
+ * projection after attention reads O, and the one before it writes dO, without a
+ * (B,H,S,D) <-> (B,S,H,D) copy.  LSE stays (B,H,S).  The reference has no such form: its
+ * model makes the copy with a CONTIGUOUS node after `transpose(1, 2)`
+ * (examples/tinyshakespear/model.mojo:104); results are bit-identical to the standard
+ * entry points followed (or preceded) by mg_contiguous. */
+int mg_flash_attn_fwd_bshd(const void* q, const void* k, const void* v, const void* mask, void* o,
+                           float* lse, int64_t B, int64_t S, int64_t H, int64_t D, float scale,
+                           int causal, int has_bias, int dtype, mg_stream stream);
+int mg_flash_attn_bwd_bshd(const void* d_o, const void* o, const void* q, const void* k,
+                           const void* v, const void* mask, const float* lse, void* dq, void* dk,
+                           void* dv, int64_t B, int64_t S, int64_t H, int64_t D, float scale,
+                           int causal, int has_bias, int dtype, mg_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

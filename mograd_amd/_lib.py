@@ -109,6 +109,8 @@ PROTOTYPES = {
     "mg_scatter_add": (_i, [_p, _p, _p, _l, _l, _l, _i, _i, _p], True),
     "mg_flash_attn_fwd": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _l, _l, _f, _i, _i, _i, _p], True),
     "mg_flash_attn_bwd": (_i, [_p] * 10 + [_l, _l, _l, _l, _f, _i, _i, _i, _p], True),
+    "mg_flash_attn_fwd_bshd": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _l, _l, _f, _i, _i, _i, _p], True),
+    "mg_flash_attn_bwd_bshd": (_i, [_p] * 10 + [_l, _l, _l, _l, _f, _i, _i, _i, _p], True),
 }
 
 

@@ -51,7 +51,7 @@ static int bwd_generic(const void* d_o, const void* o, const void* q, const void
   MG_TRY(delta.take(rows * static_cast<int64_t>(sizeof(float))));
   const dim3 grid(static_cast<unsigned>(ceil_div(rows, 4)));
   hipLaunchKernelGGL((attn_delta_kernel<T>), grid, dim3(256), 0, stream, static_cast<const T*>(d_o),
-                     static_cast<const T*>(o), delta.as<float>(), rows, a.D);
+                     static_cast<const T*>(o), delta.as<float>(), rows, a.D, a.S, a.H, a.o_bshd);
   MG_LAUNCH_CHECK();
 #define MG_BWD(C_, B_)                                                                                                \
   do {                                                                                                                \
@@ -73,15 +73,13 @@ static int bwd_generic(const void* d_o, const void* o, const void* q, const void
 
 }  // namespace mg
 
-extern "C" {
-
-int mg_flash_attn_fwd(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, int64_t B,
+static int flash_attn_fwd_impl(int o_bshd, const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, int64_t B,
                       int64_t S, int64_t H, int64_t D, float scale, int causal, int has_bias, int dtype,
                       mg_stream stream) {
   MG_TRY(mg::check_attn("flash_attn_fwd", B, S, H, D, causal, has_bias, dtype));
   if (!q || !k || !v || !o || !lse || (has_bias && !mask))
     return mg::fail(MG_ERR_INVALID, "flash_attn_fwd: null pointer argument");
-  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D)};
+  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D), o_bshd};
   hipStream_t s = mg::to_stream(stream);
   const void* ptrs[] = {q, k, v, o, has_bias ? mask : nullptr};
   if (mg::attn_mfma_supported(dtype, D, ptrs, 5))
@@ -93,13 +91,13 @@ int mg_flash_attn_fwd(const void* q, const void* k, const void* v, const void* m
   }
 }
 
-int mg_flash_attn_bwd(const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
+static int flash_attn_bwd_impl(int o_bshd, const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
                       const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t S, int64_t H, int64_t D,
                       float scale, int causal, int has_bias, int dtype, mg_stream stream) {
   MG_TRY(mg::check_attn("flash_attn_bwd", B, S, H, D, causal, has_bias, dtype));
   if (!d_o || !o || !q || !k || !v || !lse || !dq || !dk || !dv || (has_bias && !mask))
     return mg::fail(MG_ERR_INVALID, "flash_attn_bwd: null pointer argument");
-  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D)};
+  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D), o_bshd};
   hipStream_t s = mg::to_stream(stream);
   const void* ptrs[] = {d_o, o, q, k, v, dq, dk, dv, has_bias ? mask : nullptr};
   if (mg::attn_mfma_supported(dtype, D, ptrs, 9))
@@ -113,5 +111,32 @@ int mg_flash_attn_bwd(const void* d_o, const void* o, const void* q, const void*
       return mg::bwd_generic<mg::bf16_t>(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal != 0, has_bias != 0, s);
   }
 }
+
+extern "C" {
+
+int mg_flash_attn_fwd(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, int64_t B,
+                      int64_t S, int64_t H, int64_t D, float scale, int causal, int has_bias, int dtype,
+                      mg_stream stream) {
+  return flash_attn_fwd_impl(0, q, k, v, mask, o, lse, B, S, H, D, scale, causal, has_bias, dtype, stream);
+}
+
+int mg_flash_attn_fwd_bshd(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, int64_t B,
+                           int64_t S, int64_t H, int64_t D, float scale, int causal, int has_bias, int dtype,
+                           mg_stream stream) {
+  return flash_attn_fwd_impl(1, q, k, v, mask, o, lse, B, S, H, D, scale, causal, has_bias, dtype, stream);
+}
+
+int mg_flash_attn_bwd(const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
+                      const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t S, int64_t H, int64_t D,
+                      float scale, int causal, int has_bias, int dtype, mg_stream stream) {
+  return flash_attn_bwd_impl(0, d_o, o, q, k, v, mask, lse, dq, dk, dv, B, S, H, D, scale, causal, has_bias, dtype, stream);
+}
+
+int mg_flash_attn_bwd_bshd(const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
+                           const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t S, int64_t H, int64_t D,
+                           float scale, int causal, int has_bias, int dtype, mg_stream stream) {
+  return flash_attn_bwd_impl(1, d_o, o, q, k, v, mask, lse, dq, dk, dv, B, S, H, D, scale, causal, has_bias, dtype, stream);
+}
+
 
 }  // extern "C"

@@ -18,6 +18,9 @@ constexpr int kAttnMaxDPerLane = 8;  // 512 / 64
 
 struct AttnDims {
   int B, S, H, D;
+  // O and dO are (B,H,S,D) in the reference's contract; with o_bshd they are (B,S,H,D) like
+  // Q, K and V, which is what a projection that follows (or precedes) attention reads.
+  int o_bshd = 0;
 };
 
 __device__ __forceinline__ int64_t bshd(const AttnDims& a, int b, int s, int h) {
@@ -25,6 +28,17 @@ __device__ __forceinline__ int64_t bshd(const AttnDims& a, int b, int s, int h) 
 }
 __device__ __forceinline__ int64_t bhsd(const AttnDims& a, int b, int h, int s) {
   return ((static_cast<int64_t>(b) * a.H + h) * a.S + s) * a.D;
+}
+// Offset of row (b, h, s) of O / dO, and the distance between consecutive s of one (b, h).
+__device__ __forceinline__ int64_t o_at(const AttnDims& a, int b, int h, int s) {
+  return a.o_bshd ? bshd(a, b, s, h) : bhsd(a, b, h, s);
+}
+__device__ __forceinline__ int64_t o_ld(const AttnDims& a) { return a.o_bshd ? static_cast<int64_t>(a.H) * a.D : a.D; }
+// delta and LSE are always (B,H,S): index of the statistics of row `row` of O in O's own row order.
+__device__ __forceinline__ int64_t o_row_to_bhs(int64_t row, int S, int H, int o_bshd) {
+  if (!o_bshd) return row;
+  const int64_t h = row % H, bs = row / H;
+  return ((bs / S) * H + h) * S + bs % S;
 }
 
 // A row of D elements spread over the 64 lanes: lane l holds d = l, l + 64, ...
@@ -48,14 +62,15 @@ __device__ __forceinline__ float dot_rows(const float (&a)[kAttnMaxDPerLane], co
 // delta[b,h,i] = sum_d dO[b,h,i,d] * O[b,h,i,d]
 template <typename T>
 __global__ __launch_bounds__(256) void attn_delta_kernel(const T* __restrict__ d_o, const T* __restrict__ o,
-                                                         float* __restrict__ delta, int64_t rows, int D) {
+                                                         float* __restrict__ delta, int64_t rows, int D, int S, int H,
+                                                         int o_bshd) {
   const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
   if (row >= rows) return;
   const int lane = threadIdx.x % kWave;
   float acc = 0.f;
   for (int d = lane; d < D; d += kWave) acc = fmaf(to_float(d_o[row * D + d]), to_float(o[row * D + d]), acc);
   acc = wave_sum(acc);
-  if (lane == 0) delta[row] = acc;
+  if (lane == 0) delta[o_row_to_bhs(row, S, H, o_bshd)] = acc;
 }
 
 // Forward: wave = one query row; online softmax in the exp2 domain.
@@ -94,7 +109,7 @@ __global__ __launch_bounds__(256) void attn_fwd_generic_kernel(const T* __restri
     m = m_new;
   }
   const float inv = 1.0f / l;
-  T* orow = o + bhsd(a, b, h, i);
+  T* orow = o + o_at(a, b, h, i);
 #pragma unroll
   for (int t = 0; t < kAttnMaxDPerLane; ++t) {
     const int d = lane + t * kWave;
@@ -119,7 +134,7 @@ __global__ __launch_bounds__(256) void attn_dq_generic_kernel(const T* __restric
   const int nd = (a.D + kWave - 1) / kWave;
   float qr[kAttnMaxDPerLane], dor[kAttnMaxDPerLane], acc[kAttnMaxDPerLane];
   load_row(q + bshd(a, b, i, h), a.D, lane, qr);
-  load_row(d_o + bhsd(a, b, h, i), a.D, lane, dor);
+  load_row(d_o + o_at(a, b, h, i), a.D, lane, dor);
 #pragma unroll
   for (int t = 0; t < kAttnMaxDPerLane; ++t) acc[t] = 0.f;
   const float c = scale * kAttnLog2e;
@@ -172,7 +187,7 @@ __global__ __launch_bounds__(256) void attn_dkdv_generic_kernel(const T* __restr
   for (int i = i_begin; i < a.S; ++i) {
     float qr[kAttnMaxDPerLane], dor[kAttnMaxDPerLane];
     load_row(q + bshd(a, b, i, h), a.D, lane, qr);
-    load_row(d_o + bhsd(a, b, h, i), a.D, lane, dor);
+    load_row(d_o + o_at(a, b, h, i), a.D, lane, dor);
     float s = dot_rows(qr, kr, nd) * c;
     if (HAS_BIAS) s = fmaf(to_float(mask[(bh * a.S + i) * a.S + j]), kAttnLog2e, s);
     const float p = exp2f(s - lse[bh * a.S + i] * kAttnLog2e);

@@ -435,7 +435,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
 
   if (m < a.S) {
     const float inv = 1.0f / l_run;
-    T* orow = o + bhsd(a, b, h, m);
+    T* orow = o + o_at(a, b, h, m);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -500,7 +500,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
       const bool ok = m[mq] < a.S && d < a.D;
       qf[mq][ks] = ok ? *reinterpret_cast<const uint4*>(q + bshd(a, b, m[mq], h) + d) : make_uint4(0, 0, 0, 0);
       qf[mq][ks] = scale_frag<T>(qf[mq][ks], c);
-      dof[mq][ks] = ok ? *reinterpret_cast<const uint4*>(d_o + bhsd(a, b, h, m[mq]) + d) : make_uint4(0, 0, 0, 0);
+      dof[mq][ks] = ok ? *reinterpret_cast<const uint4*>(d_o + o_at(a, b, h, m[mq]) + d) : make_uint4(0, 0, 0, 0);
       settle(dof[mq][ks]);
     }
     // Rows past the end get lse = +inf so that their probabilities vanish.
@@ -649,7 +649,6 @@ __global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma
   __shared__ __attribute__((aligned(16))) float lse_ss[2][BQ];
   __shared__ __attribute__((aligned(16))) float delta_ss[2][BQ];
 
-  const int nkb = (a.S + BNK - 1) / BNK;
   // (batch, head) varies fastest across consecutive workgroups.  Causal: earlier key blocks
   // are seen by more queries; all of them launch first.
   const int n_bh = a.B * a.H;
@@ -663,7 +662,7 @@ __global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma
   const int n = n_wave + lane % 32;
   const int64_t ld = static_cast<int64_t>(a.H) * a.D;
   const T* qbase = q + bshd(a, b, 0, h);
-  const T* dobase = d_o + bhsd(a, b, h, 0);
+  const T* dobase = d_o + o_at(a, b, h, 0);
   const int64_t bh = static_cast<int64_t>(b) * a.H + h;
 
   uint4 kf[KS], vf[KS];
@@ -690,7 +689,7 @@ __global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma
   TileStager<T, BQ, DP> q_stage, do_stage;
   float lse_next, delta_next;
   q_stage.begin(qbase, ld, m_begin);
-  do_stage.begin(dobase, a.D, m_begin);
+  do_stage.begin(dobase, o_ld(a), m_begin);
   // Global -> registers for the next step of the walk, which starts at query m.
   // The row statistics go first: the compiler guards the reuse of their registers with a
   // wait for every load issued before it, which must not include this step's tile loads.
@@ -860,7 +859,8 @@ static int fwd_typed(const void* q, const void* k, const void* v, const void* ma
 // neighbouring lanes that share a row.
 template <typename T, int CPR>
 __global__ __launch_bounds__(256) void attn_delta_rows_kernel(const T* __restrict__ d_o, const T* __restrict__ o,
-                                                              float* __restrict__ delta, int64_t rows) {
+                                                              float* __restrict__ delta, int64_t rows, int S, int H,
+                                                              int o_bshd) {
   const int64_t chunk = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   const int64_t row = chunk / CPR;
   float acc = 0.f;
@@ -873,25 +873,26 @@ __global__ __launch_bounds__(256) void attn_delta_rows_kernel(const T* __restric
   }
 #pragma unroll
   for (int w = 1; w < CPR; w *= 2) acc += __shfl_xor(acc, w);
-  if (row < rows && threadIdx.x % CPR == 0) delta[row] = acc;
+  if (row < rows && threadIdx.x % CPR == 0) delta[o_row_to_bhs(row, S, H, o_bshd)] = acc;
 }
 
 template <typename T>
-static int launch_delta(const T* d_o, const T* o, float* delta, int64_t rows, int D, hipStream_t stream) {
+static int launch_delta(const T* d_o, const T* o, float* delta, int64_t rows, const AttnDims& a, hipStream_t stream) {
+  const int D = a.D;
   const int cpr = D / 8;
   const bool vec = D % 8 == 0 && (cpr & (cpr - 1)) == 0 && cpr <= 16;
   if (vec) {
     const dim3 grid(static_cast<unsigned>(ceil_div(rows * cpr, 256)));
     switch (cpr) {
-      case 1: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 1>), grid, dim3(256), 0, stream, d_o, o, delta, rows); break;
-      case 2: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 2>), grid, dim3(256), 0, stream, d_o, o, delta, rows); break;
-      case 4: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 4>), grid, dim3(256), 0, stream, d_o, o, delta, rows); break;
-      case 8: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 8>), grid, dim3(256), 0, stream, d_o, o, delta, rows); break;
-      default: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 16>), grid, dim3(256), 0, stream, d_o, o, delta, rows); break;
+      case 1: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 1>), grid, dim3(256), 0, stream, d_o, o, delta, rows, a.S, a.H, a.o_bshd); break;
+      case 2: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 2>), grid, dim3(256), 0, stream, d_o, o, delta, rows, a.S, a.H, a.o_bshd); break;
+      case 4: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 4>), grid, dim3(256), 0, stream, d_o, o, delta, rows, a.S, a.H, a.o_bshd); break;
+      case 8: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 8>), grid, dim3(256), 0, stream, d_o, o, delta, rows, a.S, a.H, a.o_bshd); break;
+      default: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 16>), grid, dim3(256), 0, stream, d_o, o, delta, rows, a.S, a.H, a.o_bshd); break;
     }
   } else {
     hipLaunchKernelGGL((attn_delta_kernel<T>), dim3(static_cast<unsigned>(ceil_div(rows, 4))), dim3(256), 0, stream, d_o,
-                       o, delta, rows, D);
+                       o, delta, rows, D, a.S, a.H, a.o_bshd);
   }
   MG_LAUNCH_CHECK();
   return MG_OK;
@@ -904,7 +905,7 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
   const int64_t rows = static_cast<int64_t>(a.B) * a.H * a.S;
   Scratch delta;
   MG_TRY(delta.take(rows * static_cast<int64_t>(sizeof(float))));
-  MG_TRY(launch_delta(static_cast<const T*>(d_o), static_cast<const T*>(o), delta.as<float>(), rows, a.D, stream));
+  MG_TRY(launch_delta(static_cast<const T*>(d_o), static_cast<const T*>(o), delta.as<float>(), rows, a, stream));
   const int64_t blocks = static_cast<int64_t>(a.B) * a.H * ceil_div(a.S, 128);
   // dQ: two query tiles per wave when the head dimension leaves registers for it and
   // there are still enough workgroups to fill the device.

@@ -10,8 +10,9 @@ sequence of libmograd_hip calls on one stream.
 The backward pass is the graph mograd/grad.mojo builds for that forward, with the fused
 entries in place of their unfused chains: mg_linear_bwd(_fused) for every Linear (with the
 ReLU gradient and the sum of the Q/K/V input gradients folded into the dX products),
-mg_layer_norm_bwd_stats, mg_flash_attn_bwd, mg_cross_entropy_fused_ids, mg_scatter_add for
-the embedding; in the forward the residual additions and the ReLU ride on the products
+mg_layer_norm_bwd_stats, mg_flash_attn_bwd_bshd (O and dO in the projections' (B,T,H,dh)
+layout, so no transposing copies), mg_cross_entropy_fused_ids, mg_scatter_add for the
+embedding; in the forward the residual additions and the ReLU ride on the products
 that feed them (mg_matmul_bt_add, mg_matmul_bias_relu_bt).
 
 Mixed precision: the parameters live in one fp32 arena (master weights); each step casts
@@ -132,12 +133,12 @@ class TinyTransformer:
         for _ in range(self.L):
             self.saved.append({
                 # Q, K and V of a layer sit back to back: one batched product writes all three
-                "x1": new(n * d), "qkv": new(3 * n * d), "o": new(n * d),
+                "x1": new(n * d), "qkv": new(3 * n * d),
                 "lse": new(B * self.H * T, F32), "ctx": new(n * d),
                 "h_mid": new(n * d), "x2": new(n * d), "a": new(n * ff),
                 "mean1": new(n, F32), "rstd1": new(n, F32), "mean2": new(n, F32), "rstd2": new(n, F32),
             })
-        self.tmp = {name: new(n * d) for name in ("dh", "dres", "dctx", "do", "dx_a")}
+        self.tmp = {name: new(n * d) for name in ("dh", "dres", "dctx", "dx_a")}
         self.tmp["dqkv"] = new(3 * n * d)  # dQ, dK, dV back to back, as the batched dW product reads them
         self.tmp["da"] = new(n * ff)
         self.tmp["logits"] = new(n * V)
@@ -186,9 +187,8 @@ class TinyTransformer:
             q, k, v = (part(c["qkv"], i) for i in range(3))
             lib.mg_matmul_bt(P(c["x1"]), w("wq"), q, 3, n, d, d, d, 1, d, 1, 0, self.qkv_stride, cd, s)
             # (n, d) row-major is (B, T, H, dh): the layout the attention kernels take for Q, K, V
-            lib.mg_flash_attn_fwd(q, k, v, None, P(c["o"]), P(c["lse"]), B, T, H, dh, scale, 1, 0, cd, s)
-            # O comes back (B, H, T, dh); the projection wants (B, T, H*dh)
-            lib.mg_contiguous(P(c["o"]), P(c["ctx"]), 4, i64(B, T, H, dh), i64(H * T * dh, dh, T * dh, 1), cd, s)
+            # O is written (B, T, H, dh) = (n, d), the layout the output projection reads
+            lib.mg_flash_attn_fwd_bshd(q, k, v, None, P(c["ctx"]), P(c["lse"]), B, T, H, dh, scale, 1, 0, cd, s)
             lib.mg_matmul_bt_add(P(c["ctx"]), w("wo"), h_in, P(c["h_mid"]), 1, n, d, d, d, 1, d, 1, n * d, d * d, cd, s)
             lib.mg_layer_norm_fwd_stats(P(c["h_mid"]), w("ln2_g"), w("ln2_b"), P(c["x2"]), P(c["mean2"]),
                                         P(c["rstd2"]), n, d, self.eps, cd, s)
@@ -218,12 +218,11 @@ class TinyTransformer:
             lib.mg_add(t["dh"], t["dres"], t["dh"], n * d, cd, s)
             # h_mid = h_in + W_O ctx
             lib.mg_linear_bwd(t["dh"], P(c["ctx"]), w("wo"), t["dctx"], g("wo"), None, n, d, d, cd, s)
-            # dctx is (B, T, H, dh); the attention backward takes dO as (B, H, T, dh)
-            lib.mg_contiguous(t["dctx"], t["do"], 4, i64(B, H, T, dh), i64(T * H * dh, dh, H * dh, 1), cd, s)
             q, k, v = (part(c["qkv"], i) for i in range(3))
             dq, dk, dv = (part(self.tmp["dqkv"], i) for i in range(3))
-            lib.mg_flash_attn_bwd(t["do"], P(c["o"]), q, k, v, None, P(c["lse"]), dq, dk, dv, B, T, H, dh, scale, 1, 0,
-                                  cd, s)
+            # dctx and ctx are (B, T, H, dh): the backward reads dO and O in that layout
+            lib.mg_flash_attn_bwd_bshd(t["dctx"], P(c["ctx"]), q, k, v, None, P(c["lse"]), dq, dk, dv, B, T, H, dh, scale,
+                                       1, 0, cd, s)
             # dx1 = dQ Wq + dK Wk + dV Wv: three products, the second and third accumulating
             gq, gk, gv = (None, None, None) if self.qkv_packed else (g("wq"), g("wk"), g("wv"))
             lib.mg_linear_bwd(dq, P(c["x1"]), w("wq"), t["dx_a"], gq, None, n, d, d, cd, s)

@@ -184,3 +184,33 @@ def test_errors(device):
         lib.mg_flash_attn_fwd(p, p, p, p, p, p, 1, 2, 1, 8, 1.0, 1, 1, F32, st)
     with pytest.raises(MogradError, match="unsupported dtype"):
         lib.mg_flash_attn_fwd(p, p, p, p, p, p, 1, 2, 1, 8, 1.0, 0, 0, R.int64, st)
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
+@pytest.mark.parametrize("name,causal,with_mask", MODES)
+@pytest.mark.parametrize("B,H,S,D", [(2, 3, 200, 64), (1, 2, 130, 72), (2, 2, 96, 128), (1, 1, 4, 8), (1, 2, 77, 40)])
+def test_bshd_output_forms_equal_the_standard_forms(device, dtype, name, causal, with_mask, B, H, S, D):
+    # O written and dO/O read as (B,S,H,D): bit for bit the standard entry points with the
+    # (B,H,S,D) <-> (B,S,H,D) copies done on the host.  LSE stays (B,H,S).
+    lib, st = device.lib, device.stream
+    q, k, v, do, m = _inputs(54, B, S, H, D, dtype, with_mask)
+    bq, bk, bv, bdo = (AnyBuffer.from_numpy(device, a, dtype) for a in (q, k, v, do))
+    bdo_bshd = AnyBuffer.from_numpy(device, np.ascontiguousarray(do.transpose(0, 2, 1, 3)), dtype)
+    bm = AnyBuffer.from_numpy(device, m if with_mask else np.zeros(8, np.float32), dtype)
+    n = B * S * H * D
+    scale = 1.0 / math.sqrt(D)
+    new = lambda count=n, dt=dtype: AnyBuffer.create(dt, device, count)
+    o1, o2, lse1, lse2 = new(), new(), new(B * H * S, F32), new(B * H * S, F32)
+    P = lambda b: b.data_ptr()
+    lib.mg_flash_attn_fwd(P(bq), P(bk), P(bv), P(bm), P(o1), P(lse1), B, S, H, D, scale, int(causal), int(with_mask), dtype, st)
+    lib.mg_flash_attn_fwd_bshd(P(bq), P(bk), P(bv), P(bm), P(o2), P(lse2), B, S, H, D, scale, int(causal), int(with_mask),
+                               dtype, st)
+    np.testing.assert_array_equal(o2.to_numpy((B, S, H, D)), o1.to_numpy((B, H, S, D)).transpose(0, 2, 1, 3))
+    np.testing.assert_array_equal(lse2.to_numpy(), lse1.to_numpy())
+    g1, g2 = [new() for _ in range(3)], [new() for _ in range(3)]
+    lib.mg_flash_attn_bwd(P(bdo), P(o1), P(bq), P(bk), P(bv), P(bm), P(lse1), *(P(g) for g in g1), B, S, H, D, scale,
+                          int(causal), int(with_mask), dtype, st)
+    lib.mg_flash_attn_bwd_bshd(P(bdo_bshd), P(o2), P(bq), P(bk), P(bv), P(bm), P(lse2), *(P(g) for g in g2), B, S, H, D,
+                               scale, int(causal), int(with_mask), dtype, st)
+    for a, b, what in zip(g1, g2, ("dq", "dk", "dv")):
+        np.testing.assert_array_equal(b.to_numpy(), a.to_numpy(), err_msg=what)
