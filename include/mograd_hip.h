@@ -165,6 +165,15 @@ int mg_layer_norm_bwd_stats(const void* dy, const void* x, const void* gamma, co
                             const float* rstd, void* dx, void* dgamma, void* dbeta, int64_t rows,
                             int64_t cols, int dtype, mg_stream stream);
 
+/* mg_layer_norm_bwd_stats with the result added to `residual` (same shape and dtype as dx;
+ * may be dx itself: in-place accumulation into a gradient that already holds the skip
+ * connection's share).  dx = round(gradient) + residual, bit for bit what
+ * mg_layer_norm_bwd_stats followed by mg_add gives.  The reference has no such form: its
+ * graph accumulates gradients with a separate ADD node (Grad.accum, mograd/grad.mojo:93-95). */
+int mg_layer_norm_bwd_stats_add(const void* dy, const void* x, const void* gamma, const float* mean,
+                                const float* rstd, const void* residual, void* dx, void* dgamma,
+                                void* dbeta, int64_t rows, int64_t cols, int dtype, mg_stream stream);
+
 /* ------------------------------------------------------------------------------------ */
 /* Softmax cross-entropy.  N = numel / C rows, C = last dim                              */
 /* (kernels/__init__.mojo:1386-1387).  dtype in {F32, F16, BF16}; math in fp32.           */

@@ -79,6 +79,7 @@ PROTOTYPES = {
     "mg_layer_norm_fwd_stats": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _f, _i, _p], True),
     "mg_layer_norm_bwd": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _f, _i, _p], True),
     "mg_layer_norm_bwd_stats": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _l, _l, _i, _p], True),
+    "mg_layer_norm_bwd_stats_add": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _l, _l, _i, _p], True),
     "mg_cross_entropy": (_i, [_p, _p, _p, _l, _l, _i, _p], True),
     "mg_cross_entropy_grad": (_i, [_p, _p, _p, _p, _l, _l, _i, _p], True),
     "mg_cross_entropy_strided": (_i, [_p, _p, _p, _i, _pl, _pl, _pl, _i, _p], True),

@@ -5,8 +5,8 @@ namespace mg {
 #define MG_DECLARE_LAYER_NORM(SUFFIX)                                                                         \
   int ln_fwd_##SUFFIX(const void*, const void*, const void*, void*, float*, float*, int64_t, int64_t, float,  \
                       hipStream_t);                                                                           \
-  int ln_bwd_##SUFFIX(const void*, const void*, const void*, const float*, const float*, void*, void*, void*, \
-                      int64_t, int64_t, float, hipStream_t);
+  int ln_bwd_##SUFFIX(const void*, const void*, const void*, const float*, const float*, const void*, void*,  \
+                      void*, void*, int64_t, int64_t, float, int, hipStream_t);
 MG_DECLARE_LAYER_NORM(f32)
 MG_DECLARE_LAYER_NORM(f16)
 MG_DECLARE_LAYER_NORM(bf16)
@@ -33,8 +33,9 @@ static int ln_fwd(const void* x, const void* gamma, const void* beta, void* y, f
   }
 }
 
-static int ln_bwd(const void* dy, const void* x, const void* gamma, const float* mean, const float* rstd, void* dx,
-                  void* dgamma, void* dbeta, int64_t rows, int64_t cols, float eps, int dtype, mg_stream stream) {
+static int ln_bwd(const void* dy, const void* x, const void* gamma, const float* mean, const float* rstd,
+                  const void* residual, void* dx, void* dgamma, void* dbeta, int64_t rows, int64_t cols, float eps,
+                  int dtype, mg_stream stream) {
   MG_TRY(check_ln("layer_norm_bwd", rows, cols, dtype));
   if (!dgamma || !dbeta) return fail(MG_ERR_INVALID, "layer_norm_bwd: null pointer argument");
   hipStream_t s = to_stream(stream);
@@ -46,9 +47,9 @@ static int ln_bwd(const void* dy, const void* x, const void* gamma, const float*
   }
   if (!dy || !x || !gamma || !dx) return fail(MG_ERR_INVALID, "layer_norm_bwd: null pointer argument");
   switch (dtype) {
-    case MG_F32: return ln_bwd_f32(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps, s);
-    case MG_F16: return ln_bwd_f16(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps, s);
-    default: return ln_bwd_bf16(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps, s);
+    case MG_F32: return ln_bwd_f32(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows, cols, eps, dtype, s);
+    case MG_F16: return ln_bwd_f16(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows, cols, eps, dtype, s);
+    default: return ln_bwd_bf16(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows, cols, eps, dtype, s);
   }
 }
 
@@ -69,14 +70,22 @@ int mg_layer_norm_fwd_stats(const void* x, const void* gamma, const void* beta, 
 
 int mg_layer_norm_bwd(const void* dy, const void* x, const void* gamma, void* dx, void* dgamma, void* dbeta,
                       int64_t rows, int64_t cols, float eps, int dtype, mg_stream stream) {
-  return mg::ln_bwd(dy, x, gamma, nullptr, nullptr, dx, dgamma, dbeta, rows, cols, eps, dtype, stream);
+  return mg::ln_bwd(dy, x, gamma, nullptr, nullptr, nullptr, dx, dgamma, dbeta, rows, cols, eps, dtype, stream);
 }
 
 int mg_layer_norm_bwd_stats(const void* dy, const void* x, const void* gamma, const float* mean, const float* rstd,
                             void* dx, void* dgamma, void* dbeta, int64_t rows, int64_t cols, int dtype,
                             mg_stream stream) {
   if (!mean || !rstd) return mg::fail(MG_ERR_INVALID, "layer_norm_bwd_stats: null statistics pointer");
-  return mg::ln_bwd(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, 0.f, dtype, stream);
+  return mg::ln_bwd(dy, x, gamma, mean, rstd, nullptr, dx, dgamma, dbeta, rows, cols, 0.f, dtype, stream);
+}
+
+int mg_layer_norm_bwd_stats_add(const void* dy, const void* x, const void* gamma, const float* mean, const float* rstd,
+                                const void* residual, void* dx, void* dgamma, void* dbeta, int64_t rows, int64_t cols,
+                                int dtype, mg_stream stream) {
+  if (!mean || !rstd) return mg::fail(MG_ERR_INVALID, "layer_norm_bwd_stats_add: null statistics pointer");
+  if (!residual && rows > 0) return mg::fail(MG_ERR_INVALID, "layer_norm_bwd_stats_add: null residual pointer");
+  return mg::ln_bwd(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows, cols, 0.f, dtype, stream);
 }
 
 }  // extern "C"

@@ -120,9 +120,9 @@ __global__ __launch_bounds__(WG) void ln_fwd_stream_kernel(const T* __restrict__
 template <typename T, int VEC, int TPR, int VPT, int WG, bool HAS_STATS>
 __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ dy, const T* __restrict__ x,
                                                          const T* __restrict__ gamma, const float* __restrict__ mean_in,
-                                                         const float* __restrict__ rstd_in, T* __restrict__ dx,
-                                                         float* __restrict__ part_g, float* __restrict__ part_b,
-                                                         int64_t rows, int cols, float eps,
+                                                         const float* __restrict__ rstd_in, const T* residual,
+                                                         T* dx, float* __restrict__ part_g,
+                                                         float* __restrict__ part_b, int64_t rows, int cols, float eps,
                                                          int64_t rows_per_group) {
   constexpr int RPW = WG / TPR;
   constexpr int NW = WG / kWave;
@@ -200,7 +200,18 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
         acc_g.v[i][e] += d * xhat;
         acc_b.v[i][e] += d;
       }
-      if (c < cols) VecIO<T, VEC>::store(dx + row * cols + c, out);
+      if (c < cols) {
+        if (residual != nullptr) {
+          // dx = round(gradient) + residual: bit for bit what a separate add of the stored
+          // gradient gives.  `residual` may be `dx` itself (each element is read, then written,
+          // by the same thread).
+          float rs[VEC];
+          VecIO<T, VEC>::load(residual + row * cols + c, rs);
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) out[e] = to_float(from_float<T>(out[e])) + rs[e];
+        }
+        VecIO<T, VEC>::store(dx + row * cols + c, out);
+      }
     }
     if constexpr (PREFETCH) {
       if (next < r_end) {
@@ -419,8 +430,9 @@ struct LayerNormOps {
   }
 
   template <int VEC, int TPR, int VPT, bool HAS_STATS>
-  static int launch_bwd(const T* dy, const T* x, const T* gamma, const float* mean, const float* rstd, T* dx,
-                        T* dgamma, T* dbeta, int64_t rows, int64_t cols, float eps, hipStream_t stream) {
+  static int launch_bwd(const T* dy, const T* x, const T* gamma, const float* mean, const float* rstd,
+                        const T* residual, T* dx, T* dgamma, T* dbeta, int64_t rows, int64_t cols, float eps,
+                        hipStream_t stream) {
     constexpr int WG = TPR == 64 ? 256 : TPR;
     constexpr int RPW = WG / TPR;
     int64_t groups = bwd_groups(rows, RPW, WG);
@@ -430,7 +442,8 @@ struct LayerNormOps {
     MG_TRY(part_g.take(groups * cols * static_cast<int64_t>(sizeof(float))));
     MG_TRY(part_b.take(groups * cols * static_cast<int64_t>(sizeof(float))));
     hipLaunchKernelGGL((ln_bwd_rows_kernel<T, VEC, TPR, VPT, WG, HAS_STATS>), dim3(static_cast<unsigned>(groups)),
-                       dim3(WG), 0, stream, dy, x, gamma, mean, rstd, dx, part_g.as<float>(), part_b.as<float>(), rows,
+                       dim3(WG), 0, stream, dy, x, gamma, mean, rstd, residual, dx, part_g.as<float>(),
+                       part_b.as<float>(), rows,
                        static_cast<int>(cols), eps, rows_per_group);
     MG_LAUNCH_CHECK();
     launch_reduce_partials<T>(part_g.as<float>(), dgamma, part_b.as<float>(), dbeta, groups, cols,
@@ -441,10 +454,12 @@ struct LayerNormOps {
 
   template <int VEC, bool HAS_STATS>
   static int dispatch_bwd(Shape s, const T* dy, const T* x, const T* gamma, const float* mean, const float* rstd,
-                          T* dx, T* dgamma, T* dbeta, int64_t rows, int64_t cols, float eps, hipStream_t stream) {
+                          const T* residual, T* dx, T* dgamma, T* dbeta, int64_t rows, int64_t cols, float eps,
+                          hipStream_t stream) {
 #define MG_LN_BWD_CASE(TPR_, VPT_)       \
   if (s.tpr == TPR_ && s.vpt == VPT_)    \
-  return launch_bwd<VEC, TPR_, VPT_, HAS_STATS>(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps, stream)
+  return launch_bwd<VEC, TPR_, VPT_, HAS_STATS>(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows, cols, eps, \
+                                                stream)
     MG_LN_BWD_CASE(64, 1);
     MG_LN_BWD_CASE(64, 2);
     MG_LN_BWD_CASE(64, 4);
@@ -484,9 +499,12 @@ struct LayerNormOps {
     return MG_OK;
   }
 
+  // `residual` (optional, may alias dx): dx = round(gradient) + residual.
   template <bool HAS_STATS>
-  static int bwd(const void* dy_, const void* x_, const void* gamma_, const float* mean, const float* rstd, void* dx_,
-                 void* dgamma_, void* dbeta_, int64_t rows, int64_t cols, float eps, hipStream_t stream) {
+  static int bwd(const void* dy_, const void* x_, const void* gamma_, const float* mean, const float* rstd,
+                 const void* residual_, void* dx_, void* dgamma_, void* dbeta_, int64_t rows, int64_t cols, float eps,
+                 int dtype, hipStream_t stream) {
+    const T* residual = static_cast<const T*>(residual_);
     const T* dy = static_cast<const T*>(dy_);
     const T* x = static_cast<const T*>(x_);
     const T* gamma = static_cast<const T*>(gamma_);
@@ -497,11 +515,18 @@ struct LayerNormOps {
     // The backward keeps five row tiles per thread: at most 16 elements per tile with
     // 1024 threads (128 registers each), 32 with fewer threads.  Wider rows stream.
     auto fits = [](const Shape& sh, int vec) { return sh.vpt * vec <= (sh.tpr == 1024 ? 16 : 32); };
-    if (can_vectorise(cols, {dy, x, gamma, dx}) && pick_shape(cols / WIDE, &s) && fits(s, WIDE))
-      return dispatch_bwd<WIDE, HAS_STATS>(s, dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps, stream);
+    if (can_vectorise(cols, {dy, x, gamma, dx, residual}) && pick_shape(cols / WIDE, &s) && fits(s, WIDE))
+      return dispatch_bwd<WIDE, HAS_STATS>(s, dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows, cols, eps,
+                                           stream);
     if (pick_shape(cols, &s) && fits(s, 1))
-      return dispatch_bwd<1, HAS_STATS>(s, dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps, stream);
-    return bwd_stream<HAS_STATS>(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps, stream);
+      return dispatch_bwd<1, HAS_STATS>(s, dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows, cols, eps, stream);
+    if (residual == nullptr)
+      return bwd_stream<HAS_STATS>(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps, stream);
+    // Streaming fallback: the gradient goes to scratch first (the residual may be dx itself), then one add.
+    Scratch tmp;
+    MG_TRY(tmp.take(rows * cols * static_cast<int64_t>(sizeof(T))));
+    MG_TRY(bwd_stream<HAS_STATS>(dy, x, gamma, mean, rstd, tmp.as<T>(), dgamma, dbeta, rows, cols, eps, stream));
+    return mg_add(tmp.as<T>(), residual, dx, rows * cols, dtype, stream);
   }
 };
 
@@ -515,12 +540,12 @@ struct LayerNormOps {
     return LayerNormOps<T>::fwd(x, gamma, beta, y, mean, rstd, rows, cols, eps, stream);                         \
   }                                                                                                              \
   int ln_bwd_##SUFFIX(const void* dy, const void* x, const void* gamma, const float* mean, const float* rstd,    \
-                      void* dx, void* dgamma, void* dbeta, int64_t rows, int64_t cols, float eps,                \
-                      hipStream_t stream) {                                                                      \
+                      const void* residual, void* dx, void* dgamma, void* dbeta, int64_t rows, int64_t cols,     \
+                      float eps, int dtype, hipStream_t stream) {                                                \
     if (mean != nullptr)                                                                                         \
-      return LayerNormOps<T>::template bwd<true>(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps,   \
-                                                 stream);                                                        \
-    return LayerNormOps<T>::template bwd<false>(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps,    \
-                                                stream);                                                         \
+      return LayerNormOps<T>::template bwd<true>(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows,    \
+                                                 cols, eps, dtype, stream);                                      \
+    return LayerNormOps<T>::template bwd<false>(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows,     \
+                                                cols, eps, dtype, stream);                                       \
   }                                                                                                              \
   }

@@ -10,7 +10,8 @@ sequence of libmograd_hip calls on one stream.
 The backward pass is the graph mograd/grad.mojo builds for that forward, with the fused
 entries in place of their unfused chains: mg_linear_bwd(_fused) for every Linear (with the
 ReLU gradient and the sum of the Q/K/V input gradients folded into the dX products),
-mg_layer_norm_bwd_stats, mg_flash_attn_bwd_bshd (O and dO in the projections' (B,T,H,dh)
+mg_layer_norm_bwd_stats_add (the gradient added to the skip connection's in place),
+mg_flash_attn_bwd_bshd (O and dO in the projections' (B,T,H,dh)
 layout, so no transposing copies), mg_cross_entropy_fused_ids, mg_scatter_add for the
 embedding; in the forward the residual additions and the ReLU ride on the products
 that feed them (mg_matmul_bt_add, mg_matmul_bias_relu_bt).
@@ -138,7 +139,7 @@ class TinyTransformer:
                 "h_mid": new(n * d), "x2": new(n * d), "a": new(n * ff),
                 "mean1": new(n, F32), "rstd1": new(n, F32), "mean2": new(n, F32), "rstd2": new(n, F32),
             })
-        self.tmp = {name: new(n * d) for name in ("dh", "dres", "dctx", "dx_a")}
+        self.tmp = {name: new(n * d) for name in ("dh", "dctx", "dx_a")}
         self.tmp["dqkv"] = new(3 * n * d)  # dQ, dK, dV back to back, as the batched dW product reads them
         self.tmp["da"] = new(n * ff)
         self.tmp["logits"] = new(n * V)
@@ -213,9 +214,9 @@ class TinyTransformer:
             # h_out = h_mid + W2 a
             lib.mg_linear_bwd_fused(t["dh"], P(c["a"]), w("w2"), t["da"], g("w2"), None, n, d, ff, 0, 1, cd, s)
             lib.mg_linear_bwd(t["da"], P(c["x2"]), w("w1"), t["dx_a"], g("w1"), g("b1"), n, ff, d, cd, s)
-            lib.mg_layer_norm_bwd_stats(t["dx_a"], P(c["h_mid"]), w("ln2_g"), P(c["mean2"]), P(c["rstd2"]), t["dres"],
-                                        g("ln2_g"), g("ln2_b"), n, d, cd, s)
-            lib.mg_add(t["dh"], t["dres"], t["dh"], n * d, cd, s)
+            # dh += LayerNorm backward: the skip connection's share is already in dh
+            lib.mg_layer_norm_bwd_stats_add(t["dx_a"], P(c["h_mid"]), w("ln2_g"), P(c["mean2"]), P(c["rstd2"]), t["dh"],
+                                            t["dh"], g("ln2_g"), g("ln2_b"), n, d, cd, s)
             # h_mid = h_in + W_O ctx
             lib.mg_linear_bwd(t["dh"], P(c["ctx"]), w("wo"), t["dctx"], g("wo"), None, n, d, d, cd, s)
             q, k, v = (part(c["qkv"], i) for i in range(3))
@@ -232,9 +233,8 @@ class TinyTransformer:
                 # dW_b = dY_b^T x1 for the three projections as one batched product (split along
                 # the token axis inside the library): A = dY_b^T is element (o, t) at dy_b[t*d + o].
                 lib.mg_matmul(dq, P(c["x1"]), g("wq"), 3, d, d, n, 1, d, d, 1, n * d, 0, cd, s)
-            lib.mg_layer_norm_bwd_stats(t["dx_a"], P(self.h[l]), w("ln1_g"), P(c["mean1"]), P(c["rstd1"]), t["dres"],
-                                        g("ln1_g"), g("ln1_b"), n, d, cd, s)
-            lib.mg_add(t["dh"], t["dres"], t["dh"], n * d, cd, s)
+            lib.mg_layer_norm_bwd_stats_add(t["dx_a"], P(self.h[l]), w("ln1_g"), P(c["mean1"]), P(c["rstd1"]), t["dh"],
+                                            t["dh"], g("ln1_g"), g("ln1_b"), n, d, cd, s)
         lib.mg_scatter_add(P(ids), t["dh"], self._g("embed"), n, V, d, ids.dtype, cd, s)
         lib.mg_cast(P(self.wgrad), P(self.grads), self.total, cd, F32, s)
         if marks:

@@ -148,6 +148,38 @@ def test_saved_statistics_path(device):
     assert_sum_close(db.to_numpy(), rdb, np.abs(dy).sum(axis=0), what="dbeta")
 
 
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
+@pytest.mark.parametrize("rows,cols", [(64, 384), (9, 1000), (33, 4096), (5, 16384), (3, 40000), (7, 129)])
+def test_backward_added_to_a_residual_equals_separate_calls(device, dtype, rows, cols):
+    # mg_layer_norm_bwd_stats_add: bit for bit mg_layer_norm_bwd_stats followed by mg_add, with
+    # the residual in its own buffer and with the residual being dx itself (accumulation in
+    # place); every row layout incl. the streaming fallback for very wide rows.
+    lib, st = device.lib, device.stream
+    P = lambda b: b.data_ptr()
+    x = round_to_dtype(normal(24, 0, (rows, cols)), dtype)
+    g = round_to_dtype(uniform(24, 1, (cols,), 0.5, 1.5), dtype)
+    b = round_to_dtype(normal(24, 2, (cols,)), dtype)
+    dy = round_to_dtype(normal(24, 3, (rows, cols)), dtype)
+    res = round_to_dtype(normal(24, 4, (rows, cols)), dtype)
+    bx, bg, bb, bdy, bres = (AnyBuffer.from_numpy(device, a, dtype) for a in (x, g, b, dy, res))
+    n = rows * cols
+    y, mean, rstd = AnyBuffer.create(dtype, device, n), AnyBuffer.create(F32, device, rows), AnyBuffer.create(F32, device, rows)
+    lib.mg_layer_norm_fwd_stats(P(bx), P(bg), P(bb), P(y), P(mean), P(rstd), rows, cols, 1e-5, dtype, st)
+    dx, dg, db, want = (AnyBuffer.create(dtype, device, m) for m in (n, cols, cols, n))
+    lib.mg_layer_norm_bwd_stats(P(bdy), P(bx), P(bg), P(mean), P(rstd), P(dx), P(dg), P(db), rows, cols, dtype, st)
+    lib.mg_add(P(dx), P(bres), P(want), n, dtype, st)
+    got, dg2, db2 = (AnyBuffer.create(dtype, device, m) for m in (n, cols, cols))
+    lib.mg_layer_norm_bwd_stats_add(P(bdy), P(bx), P(bg), P(mean), P(rstd), P(bres), P(got), P(dg2), P(db2), rows, cols,
+                                    dtype, st)
+    np.testing.assert_array_equal(got.to_numpy(), want.to_numpy())
+    np.testing.assert_array_equal(dg2.to_numpy(), dg.to_numpy())
+    np.testing.assert_array_equal(db2.to_numpy(), db.to_numpy())
+    inplace = AnyBuffer.from_numpy(device, res, dtype)
+    lib.mg_layer_norm_bwd_stats_add(P(bdy), P(bx), P(bg), P(mean), P(rstd), P(inplace), P(inplace), P(dg2), P(db2), rows,
+                                    cols, dtype, st)
+    np.testing.assert_array_equal(inplace.to_numpy(), want.to_numpy())
+
+
 @pytest.mark.parametrize("dtype,rtol,atol", [(F16, 2e-3, 2e-3), (BF16, 1.6e-2, 1.6e-2)])
 @pytest.mark.parametrize("rows,cols", [(64, 384), (8, 1000), (33, 4096), (5, 16384), (3, 40000)])
 def test_half_precision_storage(device, dtype, rtol, atol, rows, cols):
