@@ -450,16 +450,17 @@ def bench_gpt(args, dev) -> int:
          5.0 * attn_fl, "F", PF),
         ("flash_attn_fwd_bshd bf16 causal B64 H6 S256 D64 (2 B H S^2 D)",
          lambda i: lib.mg_flash_attn_fwd_bshd(P(q), P(k), P(v), None, P(o), P(lse), B, T, H, dh, sc, 1, 0, BF16, st), 2.0 * attn_fl, "F", PF),
-        ("layer_norm_bwd_stats bf16 (16384, 384)",
-         lambda i: lib.mg_layer_norm_bwd_stats(P(dy_d), P(x_d), P(gam), P(mean), P(rstd), P(out_d), P(dgam), P(dbet), n, d, BF16, st),
-         3 * n * d * e2 + 2 * n * 4 + 3 * d * e2, "B", None),
+        ("layer_norm_bwd_stats_add bf16 (16384, 384), dx accumulated in place",
+         lambda i: lib.mg_layer_norm_bwd_stats_add(P(dy_d), P(x_d), P(gam), P(mean), P(rstd), P(out_d), P(out_d), P(dgam), P(dbet),
+                                                   n, d, BF16, st),
+         4 * n * d * e2 + 2 * n * 4 + 3 * d * e2, "B", None),
         ("layer_norm_fwd_stats bf16 (16384, 384)",
          lambda i: lib.mg_layer_norm_fwd_stats(P(x_d), P(gam), P(bet), P(out_d), P(mean), P(rstd), n, d, 1e-5, BF16, st),
          2 * n * d * e2 + 2 * n * 4 + 2 * d * e2, "B", None),
         ("cross_entropy_fused_ids bf16 (16384, 65)",
          lambda i: lib.mg_cross_entropy_fused_ids(P(out_v), P(labels), None, P(loss1), P(dlog), n, V, BF16, I32, st),
          2 * n * V * e2 + n * 4 + e2, "B", None),
-        ("add bf16 (16384 x 384)", lambda i: lib.mg_add(P(x_d), P(dy_d), P(out_d), n * d, BF16, st), 3 * n * d * e2, "B", None),
+        ("add bf16 (16384 x 384) (not in the step since LayerNorm backward accumulates)", lambda i: lib.mg_add(P(x_d), P(dy_d), P(out_d), n * d, BF16, st), 3 * n * d * e2, "B", None),
         ("relu bf16 (16384 x 1536)", lambda i: lib.mg_relu(P(x_ff), P(out_ff), n * ff, BF16, st), 2 * n * ff * e2, "B", None),
         ("relu_grad bf16 (16384 x 1536)", lambda i: lib.mg_relu_grad(P(x_ff), P(dy_ff), P(out_ff), n * ff, BF16, st), 3 * n * ff * e2, "B", None),
         ("contiguous bf16 (B,H,T,dh) -> (B,T,H,dh) (not in the step since attention writes (B,T,H,dh))",
