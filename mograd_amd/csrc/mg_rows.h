@@ -132,14 +132,20 @@ __global__ __launch_bounds__(256) void reduce_partials_cw_kernel(const float* __
 }
 
 // Launches the reduction of one or two (groups, cols) partial arrays.  Wide outputs use 64
-// columns x 4 slices per workgroup; narrow ones 16 columns x 16 slices, so that a few
-// hundred columns still spread over enough workgroups to hide the load latency.
+// columns x 4 slices per workgroup; narrower ones 32 x 8 (a workgroup still reads whole
+// 128-byte lines of the fp32 partials: with 64-byte pieces the two workgroups that share a
+// line sit on different XCDs and each L2 fetches the line, which doubled the kernel's
+// fetched bytes at 4096 columns); a few hundred columns use 16 x 16 so that they still
+// spread over enough workgroups to hide the load latency.
 template <typename T>
 inline void launch_reduce_partials(const float* part0, T* out0, const float* part1, T* out1, int64_t groups, int64_t cols,
                                    int cu_count, hipStream_t stream) {
   const unsigned pairs = part1 ? 2u : 1u;
   if (ceil_div(cols, 64) * pairs >= static_cast<int64_t>(cu_count)) {
     hipLaunchKernelGGL((reduce_partials_cw_kernel<T, 64>), dim3(static_cast<unsigned>(ceil_div(cols, 64)), pairs),
+                       dim3(256), 0, stream, part0, out0, part1, out1, groups, cols);
+  } else if (ceil_div(cols, 32) * pairs * 2 >= static_cast<int64_t>(cu_count)) {
+    hipLaunchKernelGGL((reduce_partials_cw_kernel<T, 32>), dim3(static_cast<unsigned>(ceil_div(cols, 32)), pairs),
                        dim3(256), 0, stream, part0, out0, part1, out1, groups, cols);
   } else {
     hipLaunchKernelGGL((reduce_partials_cw_kernel<T, 16>), dim3(static_cast<unsigned>(ceil_div(cols, 16)), pairs),
