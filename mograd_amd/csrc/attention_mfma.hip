@@ -907,29 +907,16 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
   MG_TRY(delta.take(rows * static_cast<int64_t>(sizeof(float))));
   MG_TRY(launch_delta(static_cast<const T*>(d_o), static_cast<const T*>(o), delta.as<float>(), rows, a, stream));
   const int64_t blocks = static_cast<int64_t>(a.B) * a.H * ceil_div(a.S, 128);
-  // dQ: two query tiles per wave when the head dimension leaves registers for it and
-  // there are still enough workgroups to fill the device.
-  const int64_t blocks_q2 = static_cast<int64_t>(a.B) * a.H * ceil_div(a.S, 256);
-  const int q2_knob = env_int("MOGRAD_HIP_ATTN_DQ_TILES", 0);  // 0 = choose, 1 or 2 = force
-  const bool q2 = DP <= 64 && q2_knob != 1 &&
-                  q2_knob == 2;  // measured slower than one tile per wave on MI355X; kept as a tuning aid
 #define MG_LAUNCH(C_, B_)                                                                                              \
   do {                                                                                                                 \
     hipLaunchKernelGGL((attn_dkdv_mfma_kernel<T, DP, C_, B_>), dim3(static_cast<unsigned>(blocks)), dim3(kAttnThreads), \
                        0, stream, static_cast<const T*>(d_o), static_cast<const T*>(q), static_cast<const T*>(k),      \
                        static_cast<const T*>(v), static_cast<const T*>(mask), lse, delta.as<float>(),                  \
                        static_cast<T*>(dk), static_cast<T*>(dv), a, scale);                                            \
-    if (q2)                                                                                                            \
-      hipLaunchKernelGGL((attn_dq_mfma_kernel<T, DP, (DP <= 64 ? 2 : 1), C_, B_>),                                     \
-                         dim3(static_cast<unsigned>(blocks_q2)), dim3(kAttnThreads), 0, stream,                        \
-                         static_cast<const T*>(d_o), static_cast<const T*>(q), static_cast<const T*>(k),               \
-                         static_cast<const T*>(v), static_cast<const T*>(mask), lse, delta.as<float>(),                \
-                         static_cast<T*>(dq), a, scale);                                                               \
-    else                                                                                                               \
-      hipLaunchKernelGGL((attn_dq_mfma_kernel<T, DP, 1, C_, B_>), dim3(static_cast<unsigned>(blocks)),                 \
-                         dim3(kAttnThreads), 0, stream, static_cast<const T*>(d_o), static_cast<const T*>(q),          \
-                         static_cast<const T*>(k), static_cast<const T*>(v), static_cast<const T*>(mask), lse,         \
-                         delta.as<float>(), static_cast<T*>(dq), a, scale);                                            \
+    hipLaunchKernelGGL((attn_dq_mfma_kernel<T, DP, 1, C_, B_>), dim3(static_cast<unsigned>(blocks)),                   \
+                       dim3(kAttnThreads), 0, stream, static_cast<const T*>(d_o), static_cast<const T*>(q),            \
+                       static_cast<const T*>(k), static_cast<const T*>(v), static_cast<const T*>(mask), lse,           \
+                       delta.as<float>(), static_cast<T*>(dq), a, scale);                                              \
   } while (0)
   if (causal) MG_LAUNCH(true, false);
   else if (has_bias) MG_LAUNCH(false, true);
