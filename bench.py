@@ -418,11 +418,12 @@ def bench_gpt(args, dev) -> int:
     out_d, out_ff, out_v, dlog = new(n * d), new(n * ff), new(n * V), new(n * V)
     dw_big, db_big, dgam, dbet = new(ff * d), new(ff), new(d), new(d)
     mean, rstd, lse, loss1 = new(n, F32), new(n, F32), new(B * H * T, F32), new(1)
-    q, k, v, o, do, dq, dk, dv = rnd(n * d, 11), rnd(n * d, 12), rnd(n * d, 13), new(n * d), rnd(n * d, 14), new(n * d), new(n * d), new(n * d)
+    qkv, o, do, dqkv = rnd(3 * n * d, 11), new(n * d), rnd(n * d, 14), rnd(3 * n * d, 15)  # Q | K | V per token
+    w_qkv = rnd(3 * d * d, 12)  # the stacked (3d, d) projection weight
     i64 = lambda *a: (C.c_int64 * len(a))(*a)  # noqa: E731
     sc = 1.0 / float(np.sqrt(dh))
     lib.mg_layer_norm_fwd_stats(P(x_d), P(gam), P(bet), P(out_d), P(mean), P(rstd), n, d, 1e-5, BF16, st)
-    lib.mg_flash_attn_fwd_bshd(P(q), P(k), P(v), None, P(o), P(lse), B, T, H, dh, sc, 1, 0, BF16, st)
+    lib.mg_flash_attn_fwd_packed(P(qkv), None, P(o), P(lse), B, T, H, dh, sc, 1, 0, BF16, st)
     lib.mg_matmul_bt(P(x_d), P(w_vd), P(out_v), 1, n, V, d, d, 1, d, 1, n * d, V * d, BF16, st)
 
     def mm(x, w, out, N, K, bias=None):
@@ -437,19 +438,22 @@ def bench_gpt(args, dev) -> int:
     e2 = 2  # bytes per bf16
     attn_fl = B * H * T * T * dh
     entries = [
+        ("linear_bwd dX+dW bf16, stacked Q|K|V projection (16384, 1152<-384)", lbwd(dqkv, x_d, w_qkv, out_d, 3 * d, d),
+         12.0 * n * d * d, "F", PF),
         ("linear_bwd dX+dW bf16 (16384, 384<-384)", lbwd(dy_d, x_d, w_dd, out_d, d, d), 4.0 * n * d * d, "F", PF),
         ("linear_bwd dX+dW+db bf16 (16384, 1536<-384)", lbwd(dy_ff, x_d, w_fd, out_d, ff, d, db_big), 4.0 * n * d * ff, "F", PF),
         ("linear_bwd dX+dW bf16 (16384, 384<-1536)", lbwd(dy_d, x_ff, w_df, out_ff, d, ff), 4.0 * n * d * ff, "F", PF),
         ("linear_bwd dX+dW bf16 lm_head (16384, 65<-384)", lbwd(dlog, x_d, w_vd, out_d, V, d), 4.0 * n * d * V, "F", PF),
+        ("matmul_bt bf16, stacked Q|K|V projection (16384, 1152<-384)", mm(x_d, w_qkv, dqkv, 3 * d, d), 6.0 * n * d * d, "F", PF),
         ("matmul_bt bf16 (16384, 384<-384)", mm(x_d, w_dd, out_d, d, d), 2.0 * n * d * d, "F", PF),
         ("matmul_bias_bt bf16 (16384, 1536<-384)", mm(x_d, w_fd, out_ff, ff, d, bias_f), 2.0 * n * d * ff, "F", PF),
         ("matmul_bt bf16 (16384, 384<-1536)", mm(x_ff, w_df, out_d, d, ff), 2.0 * n * d * ff, "F", PF),
         ("matmul_bt bf16 lm_head (16384, 65<-384)", mm(x_d, w_vd, out_v, V, d), 2.0 * n * d * V, "F", PF),
-        ("flash_attn_bwd_bshd bf16 causal B64 H6 S256 D64 (5 B H S^2 D)",
-         lambda i: lib.mg_flash_attn_bwd_bshd(P(do), P(o), P(q), P(k), P(v), None, P(lse), P(dq), P(dk), P(dv), B, T, H, dh, sc, 1, 0, BF16, st),
+        ("flash_attn_bwd_packed bf16 causal B64 H6 S256 D64 (5 B H S^2 D)",
+         lambda i: lib.mg_flash_attn_bwd_packed(P(do), P(o), P(qkv), None, P(lse), P(dqkv), B, T, H, dh, sc, 1, 0, BF16, st),
          5.0 * attn_fl, "F", PF),
-        ("flash_attn_fwd_bshd bf16 causal B64 H6 S256 D64 (2 B H S^2 D)",
-         lambda i: lib.mg_flash_attn_fwd_bshd(P(q), P(k), P(v), None, P(o), P(lse), B, T, H, dh, sc, 1, 0, BF16, st), 2.0 * attn_fl, "F", PF),
+        ("flash_attn_fwd_packed bf16 causal B64 H6 S256 D64 (2 B H S^2 D)",
+         lambda i: lib.mg_flash_attn_fwd_packed(P(qkv), None, P(o), P(lse), B, T, H, dh, sc, 1, 0, BF16, st), 2.0 * attn_fl, "F", PF),
         ("layer_norm_bwd_stats_add bf16 (16384, 384), dx accumulated in place",
          lambda i: lib.mg_layer_norm_bwd_stats_add(P(dy_d), P(x_d), P(gam), P(mean), P(rstd), P(out_d), P(out_d), P(dgam), P(dbet),
                                                    n, d, BF16, st),

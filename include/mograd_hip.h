@@ -412,6 +412,20 @@ int mg_flash_attn_bwd_bshd(const void* d_o, const void* o, const void* q, const 
                            void* dv, int64_t B, int64_t S, int64_t H, int64_t D, float scale,
                            int causal, int has_bias, int dtype, mg_stream stream);
 
+/* Q, K and V as the three slices of one (B,S,3,H,D) tensor (what a single projection of
+ * width 3*H*D writes), dQ, dK, dV likewise in one `dqkv`, O and dO (B,S,H,D), LSE (B,H,S).
+ * The gradient with respect to the projection's input and weight is then one product each
+ * instead of three.  Same arithmetic and results as the separate-tensor forms; no
+ * counterpart in the reference, whose model projects Q, K and V with three Linear layers
+ * (examples/tinyshakespear/model.mojo:80-101). */
+int mg_flash_attn_fwd_packed(const void* qkv, const void* mask, void* o, float* lse, int64_t B,
+                             int64_t S, int64_t H, int64_t D, float scale, int causal, int has_bias,
+                             int dtype, mg_stream stream);
+int mg_flash_attn_bwd_packed(const void* d_o, const void* o, const void* qkv, const void* mask,
+                             const float* lse, void* dqkv, int64_t B, int64_t S, int64_t H,
+                             int64_t D, float scale, int causal, int has_bias, int dtype,
+                             mg_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

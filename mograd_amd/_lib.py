@@ -112,6 +112,8 @@ PROTOTYPES = {
     "mg_flash_attn_bwd": (_i, [_p] * 10 + [_l, _l, _l, _l, _f, _i, _i, _i, _p], True),
     "mg_flash_attn_fwd_bshd": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _l, _l, _f, _i, _i, _i, _p], True),
     "mg_flash_attn_bwd_bshd": (_i, [_p] * 10 + [_l, _l, _l, _l, _f, _i, _i, _i, _p], True),
+    "mg_flash_attn_fwd_packed": (_i, [_p, _p, _p, _p, _l, _l, _l, _l, _f, _i, _i, _i, _p], True),
+    "mg_flash_attn_bwd_packed": (_i, [_p] * 6 + [_l, _l, _l, _l, _f, _i, _i, _i, _p], True),
 }
 
 

@@ -73,13 +73,13 @@ static int bwd_generic(const void* d_o, const void* o, const void* q, const void
 
 }  // namespace mg
 
-static int flash_attn_fwd_impl(int o_bshd, const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, int64_t B,
+static int flash_attn_fwd_impl(int o_bshd, int64_t ld, const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, int64_t B,
                       int64_t S, int64_t H, int64_t D, float scale, int causal, int has_bias, int dtype,
                       mg_stream stream) {
   MG_TRY(mg::check_attn("flash_attn_fwd", B, S, H, D, causal, has_bias, dtype));
   if (!q || !k || !v || !o || !lse || (has_bias && !mask))
     return mg::fail(MG_ERR_INVALID, "flash_attn_fwd: null pointer argument");
-  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D), o_bshd};
+  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D), o_bshd, ld ? ld : H * D};
   hipStream_t s = mg::to_stream(stream);
   const void* ptrs[] = {q, k, v, o, has_bias ? mask : nullptr};
   if (mg::attn_mfma_supported(dtype, D, ptrs, 5))
@@ -91,13 +91,13 @@ static int flash_attn_fwd_impl(int o_bshd, const void* q, const void* k, const v
   }
 }
 
-static int flash_attn_bwd_impl(int o_bshd, const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
+static int flash_attn_bwd_impl(int o_bshd, int64_t ld, const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
                       const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t S, int64_t H, int64_t D,
                       float scale, int causal, int has_bias, int dtype, mg_stream stream) {
   MG_TRY(mg::check_attn("flash_attn_bwd", B, S, H, D, causal, has_bias, dtype));
   if (!d_o || !o || !q || !k || !v || !lse || !dq || !dk || !dv || (has_bias && !mask))
     return mg::fail(MG_ERR_INVALID, "flash_attn_bwd: null pointer argument");
-  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D), o_bshd};
+  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D), o_bshd, ld ? ld : H * D};
   hipStream_t s = mg::to_stream(stream);
   const void* ptrs[] = {d_o, o, q, k, v, dq, dk, dv, has_bias ? mask : nullptr};
   if (mg::attn_mfma_supported(dtype, D, ptrs, 9))
@@ -117,26 +117,45 @@ extern "C" {
 int mg_flash_attn_fwd(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, int64_t B,
                       int64_t S, int64_t H, int64_t D, float scale, int causal, int has_bias, int dtype,
                       mg_stream stream) {
-  return flash_attn_fwd_impl(0, q, k, v, mask, o, lse, B, S, H, D, scale, causal, has_bias, dtype, stream);
+  return flash_attn_fwd_impl(0, 0, q, k, v, mask, o, lse, B, S, H, D, scale, causal, has_bias, dtype, stream);
 }
 
 int mg_flash_attn_fwd_bshd(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, int64_t B,
                            int64_t S, int64_t H, int64_t D, float scale, int causal, int has_bias, int dtype,
                            mg_stream stream) {
-  return flash_attn_fwd_impl(1, q, k, v, mask, o, lse, B, S, H, D, scale, causal, has_bias, dtype, stream);
+  return flash_attn_fwd_impl(1, 0, q, k, v, mask, o, lse, B, S, H, D, scale, causal, has_bias, dtype, stream);
 }
 
 int mg_flash_attn_bwd(const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
                       const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t S, int64_t H, int64_t D,
                       float scale, int causal, int has_bias, int dtype, mg_stream stream) {
-  return flash_attn_bwd_impl(0, d_o, o, q, k, v, mask, lse, dq, dk, dv, B, S, H, D, scale, causal, has_bias, dtype, stream);
+  return flash_attn_bwd_impl(0, 0, d_o, o, q, k, v, mask, lse, dq, dk, dv, B, S, H, D, scale, causal, has_bias, dtype, stream);
 }
 
 int mg_flash_attn_bwd_bshd(const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
                            const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t S, int64_t H, int64_t D,
                            float scale, int causal, int has_bias, int dtype, mg_stream stream) {
-  return flash_attn_bwd_impl(1, d_o, o, q, k, v, mask, lse, dq, dk, dv, B, S, H, D, scale, causal, has_bias, dtype, stream);
+  return flash_attn_bwd_impl(1, 0, d_o, o, q, k, v, mask, lse, dq, dk, dv, B, S, H, D, scale, causal, has_bias, dtype, stream);
 }
 
+int mg_flash_attn_fwd_packed(const void* qkv, const void* mask, void* o, float* lse, int64_t B, int64_t S, int64_t H,
+                             int64_t D, float scale, int causal, int has_bias, int dtype, mg_stream stream) {
+  if (!qkv) return mg::fail(MG_ERR_INVALID, "flash_attn_fwd_packed: null pointer argument");
+  const int64_t slice = H * D * mg::dtype_size(dtype);  // bytes from the Q slice of a token to its K slice
+  const char* base = static_cast<const char*>(qkv);
+  return flash_attn_fwd_impl(1, 3 * H * D, base, base + slice, base + 2 * slice, mask, o, lse, B, S, H, D, scale, causal,
+                             has_bias, dtype, stream);
+}
+
+int mg_flash_attn_bwd_packed(const void* d_o, const void* o, const void* qkv, const void* mask, const float* lse,
+                             void* dqkv, int64_t B, int64_t S, int64_t H, int64_t D, float scale, int causal,
+                             int has_bias, int dtype, mg_stream stream) {
+  if (!qkv || !dqkv) return mg::fail(MG_ERR_INVALID, "flash_attn_bwd_packed: null pointer argument");
+  const int64_t slice = H * D * mg::dtype_size(dtype);
+  const char* base = static_cast<const char*>(qkv);
+  char* out = static_cast<char*>(dqkv);
+  return flash_attn_bwd_impl(1, 3 * H * D, d_o, o, base, base + slice, base + 2 * slice, mask, lse, out, out + slice,
+                             out + 2 * slice, B, S, H, D, scale, causal, has_bias, dtype, stream);
+}
 
 }  // extern "C"

@@ -21,6 +21,9 @@ struct AttnDims {
   // O and dO are (B,H,S,D) in the reference's contract; with o_bshd they are (B,S,H,D) like
   // Q, K and V, which is what a projection that follows (or precedes) attention reads.
   int o_bshd = 0;
+  // Elements between consecutive tokens of Q, K, V (and dQ, dK, dV): H*D when each is its
+  // own (B,S,H,D) tensor, 3*H*D when they are the three slices of one (B,S,3,H,D) tensor.
+  int64_t ld = 0;
 };
 
 __device__ __forceinline__ int64_t bshd(const AttnDims& a, int b, int s, int h) {
@@ -28,6 +31,10 @@ __device__ __forceinline__ int64_t bshd(const AttnDims& a, int b, int s, int h) 
 }
 __device__ __forceinline__ int64_t bhsd(const AttnDims& a, int b, int h, int s) {
   return ((static_cast<int64_t>(b) * a.H + h) * a.S + s) * a.D;
+}
+// Offset of row (b, s, h) of Q, K, V, dQ, dK or dV.
+__device__ __forceinline__ int64_t qkv_at(const AttnDims& a, int b, int s, int h) {
+  return (static_cast<int64_t>(b) * a.S + s) * a.ld + static_cast<int64_t>(h) * a.D;
 }
 // Offset of row (b, h, s) of O / dO, and the distance between consecutive s of one (b, h).
 __device__ __forceinline__ int64_t o_at(const AttnDims& a, int b, int h, int s) {
@@ -87,7 +94,7 @@ __global__ __launch_bounds__(256) void attn_fwd_generic_kernel(const T* __restri
   const int b = static_cast<int>(row / (static_cast<int64_t>(a.S) * a.H));
   const int nd = (a.D + kWave - 1) / kWave;
   float qr[kAttnMaxDPerLane], acc[kAttnMaxDPerLane];
-  load_row(q + bshd(a, b, i, h), a.D, lane, qr);
+  load_row(q + qkv_at(a, b, i, h), a.D, lane, qr);
 #pragma unroll
   for (int t = 0; t < kAttnMaxDPerLane; ++t) acc[t] = 0.f;
   const float c = scale * kAttnLog2e;
@@ -96,8 +103,8 @@ __global__ __launch_bounds__(256) void attn_fwd_generic_kernel(const T* __restri
   const T* mrow = HAS_BIAS ? mask + ((static_cast<int64_t>(b) * a.H + h) * a.S + i) * a.S : nullptr;
   for (int j = 0; j < j_end; ++j) {
     float kr[kAttnMaxDPerLane], vr[kAttnMaxDPerLane];
-    load_row(k + bshd(a, b, j, h), a.D, lane, kr);
-    load_row(v + bshd(a, b, j, h), a.D, lane, vr);
+    load_row(k + qkv_at(a, b, j, h), a.D, lane, kr);
+    load_row(v + qkv_at(a, b, j, h), a.D, lane, vr);
     float s = dot_rows(qr, kr, nd) * c;
     if (HAS_BIAS) s = fmaf(to_float(mrow[j]), kAttnLog2e, s);
     const float m_new = fmaxf(m, s);
@@ -133,7 +140,7 @@ __global__ __launch_bounds__(256) void attn_dq_generic_kernel(const T* __restric
   const int b = static_cast<int>(row / (static_cast<int64_t>(a.S) * a.H));
   const int nd = (a.D + kWave - 1) / kWave;
   float qr[kAttnMaxDPerLane], dor[kAttnMaxDPerLane], acc[kAttnMaxDPerLane];
-  load_row(q + bshd(a, b, i, h), a.D, lane, qr);
+  load_row(q + qkv_at(a, b, i, h), a.D, lane, qr);
   load_row(d_o + o_at(a, b, h, i), a.D, lane, dor);
 #pragma unroll
   for (int t = 0; t < kAttnMaxDPerLane; ++t) acc[t] = 0.f;
@@ -144,8 +151,8 @@ __global__ __launch_bounds__(256) void attn_dq_generic_kernel(const T* __restric
   const T* mrow = HAS_BIAS ? mask + ((static_cast<int64_t>(b) * a.H + h) * a.S + i) * a.S : nullptr;
   for (int j = 0; j < j_end; ++j) {
     float kr[kAttnMaxDPerLane], vr[kAttnMaxDPerLane];
-    load_row(k + bshd(a, b, j, h), a.D, lane, kr);
-    load_row(v + bshd(a, b, j, h), a.D, lane, vr);
+    load_row(k + qkv_at(a, b, j, h), a.D, lane, kr);
+    load_row(v + qkv_at(a, b, j, h), a.D, lane, vr);
     float s = dot_rows(qr, kr, nd) * c;
     if (HAS_BIAS) s = fmaf(to_float(mrow[j]), kAttnLog2e, s);
     const float p = exp2f(s - lse2);
@@ -154,7 +161,7 @@ __global__ __launch_bounds__(256) void attn_dq_generic_kernel(const T* __restric
 #pragma unroll
     for (int t = 0; t < kAttnMaxDPerLane; ++t) acc[t] = fmaf(ds, kr[t], acc[t]);
   }
-  T* out = dq + bshd(a, b, i, h);
+  T* out = dq + qkv_at(a, b, i, h);
 #pragma unroll
   for (int t = 0; t < kAttnMaxDPerLane; ++t) {
     const int d = lane + t * kWave;
@@ -177,8 +184,8 @@ __global__ __launch_bounds__(256) void attn_dkdv_generic_kernel(const T* __restr
   const int b = static_cast<int>(row / (static_cast<int64_t>(a.S) * a.H));
   const int nd = (a.D + kWave - 1) / kWave;
   float kr[kAttnMaxDPerLane], vr[kAttnMaxDPerLane], acck[kAttnMaxDPerLane], accv[kAttnMaxDPerLane];
-  load_row(k + bshd(a, b, j, h), a.D, lane, kr);
-  load_row(v + bshd(a, b, j, h), a.D, lane, vr);
+  load_row(k + qkv_at(a, b, j, h), a.D, lane, kr);
+  load_row(v + qkv_at(a, b, j, h), a.D, lane, vr);
 #pragma unroll
   for (int t = 0; t < kAttnMaxDPerLane; ++t) acck[t] = accv[t] = 0.f;
   const float c = scale * kAttnLog2e;
@@ -186,7 +193,7 @@ __global__ __launch_bounds__(256) void attn_dkdv_generic_kernel(const T* __restr
   const int i_begin = CAUSAL ? j : 0;
   for (int i = i_begin; i < a.S; ++i) {
     float qr[kAttnMaxDPerLane], dor[kAttnMaxDPerLane];
-    load_row(q + bshd(a, b, i, h), a.D, lane, qr);
+    load_row(q + qkv_at(a, b, i, h), a.D, lane, qr);
     load_row(d_o + o_at(a, b, h, i), a.D, lane, dor);
     float s = dot_rows(qr, kr, nd) * c;
     if (HAS_BIAS) s = fmaf(to_float(mask[(bh * a.S + i) * a.S + j]), kAttnLog2e, s);
@@ -199,8 +206,8 @@ __global__ __launch_bounds__(256) void attn_dkdv_generic_kernel(const T* __restr
       acck[t] = fmaf(ds, qr[t], acck[t]);
     }
   }
-  T* outk = dk + bshd(a, b, j, h);
-  T* outv = dv + bshd(a, b, j, h);
+  T* outk = dk + qkv_at(a, b, j, h);
+  T* outv = dv + qkv_at(a, b, j, h);
 #pragma unroll
   for (int t = 0; t < kAttnMaxDPerLane; ++t) {
     const int d = lane + t * kWave;

@@ -310,15 +310,15 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
   const int half = lane / 32;
   const int m_wave = qb * BM + wave * 32;
   const int m = m_wave + lane % 32;
-  const int64_t ld = static_cast<int64_t>(a.H) * a.D;  // BSHD row stride
-  const T* kbase = k + bshd(a, b, 0, h);
-  const T* vbase = v + bshd(a, b, 0, h);
+  const int64_t ld = a.ld;  // token stride of Q, K, V
+  const T* kbase = k + qkv_at(a, b, 0, h);
+  const T* vbase = v + qkv_at(a, b, 0, h);
 
   uint4 qf[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     const int d = ks * 16 + half * 8;
-    qf[ks] = (m < a.S && d < a.D) ? *reinterpret_cast<const uint4*>(q + bshd(a, b, m, h) + d) : make_uint4(0, 0, 0, 0);
+    qf[ks] = (m < a.S && d < a.D) ? *reinterpret_cast<const uint4*>(q + qkv_at(a, b, m, h) + d) : make_uint4(0, 0, 0, 0);
     settle(qf[ks]);
   }
   floatx16 acc_o[DT];
@@ -476,9 +476,9 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
   const int wave = threadIdx.x / kWave;
   const int half = lane / 32;
   const int m_wave = qb * BM + wave * (32 * MQ);
-  const int64_t ld = static_cast<int64_t>(a.H) * a.D;
-  const T* kbase = k + bshd(a, b, 0, h);
-  const T* vbase = v + bshd(a, b, 0, h);
+  const int64_t ld = a.ld;
+  const T* kbase = k + qkv_at(a, b, 0, h);
+  const T* vbase = v + qkv_at(a, b, 0, h);
   const int64_t bh = static_cast<int64_t>(b) * a.H + h;
 
   // Q is held pre-multiplied by scale * log2(e), and the score and dP products start from
@@ -498,7 +498,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
     for (int ks = 0; ks < KS; ++ks) {
       const int d = ks * 16 + half * 8;
       const bool ok = m[mq] < a.S && d < a.D;
-      qf[mq][ks] = ok ? *reinterpret_cast<const uint4*>(q + bshd(a, b, m[mq], h) + d) : make_uint4(0, 0, 0, 0);
+      qf[mq][ks] = ok ? *reinterpret_cast<const uint4*>(q + qkv_at(a, b, m[mq], h) + d) : make_uint4(0, 0, 0, 0);
       qf[mq][ks] = scale_frag<T>(qf[mq][ks], c);
       dof[mq][ks] = ok ? *reinterpret_cast<const uint4*>(d_o + o_at(a, b, h, m[mq]) + d) : make_uint4(0, 0, 0, 0);
       settle(dof[mq][ks]);
@@ -618,7 +618,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
 #pragma unroll
   for (int mq = 0; mq < MQ; ++mq) {
     if (m[mq] < a.S) {
-      T* out = dq + bshd(a, b, m[mq], h);
+      T* out = dq + qkv_at(a, b, m[mq], h);
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -660,8 +660,8 @@ __global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma
   const int half = lane / 32;
   const int n_wave = kb * BNK + wave * 32;
   const int n = n_wave + lane % 32;
-  const int64_t ld = static_cast<int64_t>(a.H) * a.D;
-  const T* qbase = q + bshd(a, b, 0, h);
+  const int64_t ld = a.ld;
+  const T* qbase = q + qkv_at(a, b, 0, h);
   const T* dobase = d_o + o_at(a, b, h, 0);
   const int64_t bh = static_cast<int64_t>(b) * a.H + h;
 
@@ -670,11 +670,11 @@ __global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma
   for (int ks = 0; ks < KS; ++ks) {
     const int d = ks * 16 + half * 8;
     const bool ok = n < a.S && d < a.D;
-    kf[ks] = ok ? *reinterpret_cast<const uint4*>(k + bshd(a, b, n, h) + d) : make_uint4(0, 0, 0, 0);
+    kf[ks] = ok ? *reinterpret_cast<const uint4*>(k + qkv_at(a, b, n, h) + d) : make_uint4(0, 0, 0, 0);
     // K is held pre-multiplied by scale * log2(e): the score product then comes out in the
     // exponent's units.  (dK is formed from the unscaled Q tile, so nothing else changes.)
     kf[ks] = scale_frag<T>(kf[ks], scale * kAttnLog2e);
-    vf[ks] = ok ? *reinterpret_cast<const uint4*>(v + bshd(a, b, n, h) + d) : make_uint4(0, 0, 0, 0);
+    vf[ks] = ok ? *reinterpret_cast<const uint4*>(v + qkv_at(a, b, n, h) + d) : make_uint4(0, 0, 0, 0);
     settle(vf[ks]);
   }
   floatx16 acc_k[DT], acc_v[DT];
@@ -811,8 +811,8 @@ __global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma
   }
 
   if (n < a.S) {
-    T* outk = dk + bshd(a, b, n, h);
-    T* outv = dv + bshd(a, b, n, h);
+    T* outk = dk + qkv_at(a, b, n, h);
+    T* outv = dv + qkv_at(a, b, n, h);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll

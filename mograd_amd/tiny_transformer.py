@@ -9,11 +9,12 @@ sequence of libmograd_hip calls on one stream.
 
 The backward pass is the graph mograd/grad.mojo builds for that forward, with the fused
 entries in place of their unfused chains: mg_linear_bwd(_fused) for every Linear (with the
-ReLU gradient and the sum of the Q/K/V input gradients folded into the dX products),
+ReLU gradient folded into the dX product; the Q, K and V projections are one Linear with
+the stacked (3d, d) weight, so their input and weight gradients are one product each),
 mg_layer_norm_bwd_stats_add (the gradient added to the skip connection's in place),
-mg_flash_attn_bwd_bshd (O and dO in the projections' (B,T,H,dh)
-layout, so no transposing copies), mg_cross_entropy_fused_ids, mg_scatter_add for the
-embedding; in the forward the residual additions and the ReLU ride on the products
+mg_flash_attn_bwd_packed (Q | K | V and dQ | dK | dV as one (B,T,3,H,dh) tensor each, O and
+dO in the projections' (B,T,H,dh) layout, so no transposing copies),
+mg_cross_entropy_fused_ids, mg_scatter_add for the embedding; in the forward the residual additions and the ReLU ride on the products
 that feed them (mg_matmul_bt_add, mg_matmul_bias_relu_bt).
 
 Mixed precision: the parameters live in one fp32 arena (master weights); each step casts
@@ -72,14 +73,16 @@ class TinyTransformer:
                         "ln2_g": (d,), "ln2_b": (d,), "w1": (ff, d), "b1": (ff,), "w2": (d, ff)}
         for layer in range(n_layers):
             for name in BLOCK_PARAMS:
-                place(f"blocks.{layer}.{name}", block_shapes[name])
+                if name == "wq":
+                    # wq, wk, wv back to back with no padding between them: together they are
+                    # the (3d, d) weight of one projection whose output is Q | K | V per token.
+                    for i, part in enumerate(("wq", "wk", "wv")):
+                        self.slices[f"blocks.{layer}.{part}"] = _Slice(f"blocks.{layer}.{part}", (d, d), off + i * d * d)
+                    off += -(-3 * d * d // _ALIGN) * _ALIGN
+                elif name not in ("wk", "wv"):
+                    place(f"blocks.{layer}.{name}", block_shapes[name])
         place("lm_head", (V, d))
         self.total = off
-        # wq, wk, wv of a layer are consecutive equal slices: the batch stride of the batched
-        # projection.  Their gradients can come from one batched product only when the slices
-        # are not padded apart (the library writes batches of a result back to back).
-        self.qkv_stride = self.slices["blocks.0.wk"].offset - self.slices["blocks.0.wq"].offset if n_layers else 0
-        self.qkv_packed = self.qkv_stride == d * d
         self.master = AnyBuffer.create(F32, device, self.total, fill=0.0)  # fp32 master weights
         self.grads = AnyBuffer.create(F32, device, self.total, fill=0.0)   # fp32 gradients, same layout
         self.work = AnyBuffer.create(self.cd, device, self.total)          # weights in the compute dtype
@@ -133,14 +136,14 @@ class TinyTransformer:
         self.saved: List[dict] = []
         for _ in range(self.L):
             self.saved.append({
-                # Q, K and V of a layer sit back to back: one batched product writes all three
+                # Q | K | V per token: the (n, 3d) output of the stacked projection
                 "x1": new(n * d), "qkv": new(3 * n * d),
                 "lse": new(B * self.H * T, F32), "ctx": new(n * d),
                 "h_mid": new(n * d), "x2": new(n * d), "a": new(n * ff),
                 "mean1": new(n, F32), "rstd1": new(n, F32), "mean2": new(n, F32), "rstd2": new(n, F32),
             })
         self.tmp = {name: new(n * d) for name in ("dh", "dctx", "dx_a")}
-        self.tmp["dqkv"] = new(3 * n * d)  # dQ, dK, dV back to back, as the batched dW product reads them
+        self.tmp["dqkv"] = new(3 * n * d)  # dQ | dK | dV per token
         self.tmp["da"] = new(n * ff)
         self.tmp["logits"] = new(n * V)
         self.tmp["dlogits"] = new(n * V)
@@ -171,8 +174,6 @@ class TinyTransformer:
                 lib.mg_matmul_bias_bt(x, w, bias, out, 1, n, N, K, K, 1, K, 1, n * K, N * K, cd, s)
 
         P = lambda buf: buf.data_ptr()
-        # i-th (n, d) third of a buffer that holds three activations back to back
-        part = lambda buf, i: C.c_void_p(buf.storage.ptr + i * n * d * DTYPE_SIZE[cd])
 
         lib.mg_cast(P(self.master), P(self.work), self.total, F32, cd, s)
 
@@ -183,13 +184,11 @@ class TinyTransformer:
             h_in, h_out = P(self.h[l]), P(self.h[l + 1])
             lib.mg_layer_norm_fwd_stats(h_in, w("ln1_g"), w("ln1_b"), P(c["x1"]), P(c["mean1"]), P(c["rstd1"]), n, d,
                                         self.eps, cd, s)
-            # The three projections share x1: one batched product over (wq, wk, wv), which are
-            # consecutive equal slices of the weight arena (batch stride 0 on x1).
-            q, k, v = (part(c["qkv"], i) for i in range(3))
-            lib.mg_matmul_bt(P(c["x1"]), w("wq"), q, 3, n, d, d, d, 1, d, 1, 0, self.qkv_stride, cd, s)
-            # (n, d) row-major is (B, T, H, dh): the layout the attention kernels take for Q, K, V
+            # One projection with the stacked (3d, d) weight: row t of the (n, 3d) result is
+            # Q | K | V of token t, i.e. (B, T, 3, H, dh), which the attention kernels read in place.
+            linear(P(c["x1"]), w("wq"), P(c["qkv"]), 3 * d, d)
             # O is written (B, T, H, dh) = (n, d), the layout the output projection reads
-            lib.mg_flash_attn_fwd_bshd(q, k, v, None, P(c["ctx"]), P(c["lse"]), B, T, H, dh, scale, 1, 0, cd, s)
+            lib.mg_flash_attn_fwd_packed(P(c["qkv"]), None, P(c["ctx"]), P(c["lse"]), B, T, H, dh, scale, 1, 0, cd, s)
             lib.mg_matmul_bt_add(P(c["ctx"]), w("wo"), h_in, P(c["h_mid"]), 1, n, d, d, d, 1, d, 1, n * d, d * d, cd, s)
             lib.mg_layer_norm_fwd_stats(P(c["h_mid"]), w("ln2_g"), w("ln2_b"), P(c["x2"]), P(c["mean2"]),
                                         P(c["rstd2"]), n, d, self.eps, cd, s)
@@ -219,20 +218,11 @@ class TinyTransformer:
                                             t["dh"], g("ln2_g"), g("ln2_b"), n, d, cd, s)
             # h_mid = h_in + W_O ctx
             lib.mg_linear_bwd(t["dh"], P(c["ctx"]), w("wo"), t["dctx"], g("wo"), None, n, d, d, cd, s)
-            q, k, v = (part(c["qkv"], i) for i in range(3))
-            dq, dk, dv = (part(self.tmp["dqkv"], i) for i in range(3))
-            # dctx and ctx are (B, T, H, dh): the backward reads dO and O in that layout
-            lib.mg_flash_attn_bwd_bshd(t["dctx"], P(c["ctx"]), q, k, v, None, P(c["lse"]), dq, dk, dv, B, T, H, dh, scale,
-                                       1, 0, cd, s)
-            # dx1 = dQ Wq + dK Wk + dV Wv: three products, the second and third accumulating
-            gq, gk, gv = (None, None, None) if self.qkv_packed else (g("wq"), g("wk"), g("wv"))
-            lib.mg_linear_bwd(dq, P(c["x1"]), w("wq"), t["dx_a"], gq, None, n, d, d, cd, s)
-            lib.mg_linear_bwd_fused(dk, P(c["x1"]), w("wk"), t["dx_a"], gk, None, n, d, d, 1, 0, cd, s)
-            lib.mg_linear_bwd_fused(dv, P(c["x1"]), w("wv"), t["dx_a"], gv, None, n, d, d, 1, 0, cd, s)
-            if self.qkv_packed:
-                # dW_b = dY_b^T x1 for the three projections as one batched product (split along
-                # the token axis inside the library): A = dY_b^T is element (o, t) at dy_b[t*d + o].
-                lib.mg_matmul(dq, P(c["x1"]), g("wq"), 3, d, d, n, 1, d, d, 1, n * d, 0, cd, s)
+            # dctx and ctx are (B, T, H, dh); dQ | dK | dV come back as one (n, 3d) tensor
+            lib.mg_flash_attn_bwd_packed(t["dctx"], P(c["ctx"]), P(c["qkv"]), None, P(c["lse"]), t["dqkv"], B, T, H, dh,
+                                         scale, 1, 0, cd, s)
+            # gradient of the stacked projection: dx1 (n, d) and dW (3d, d) = dwq | dwk | dwv
+            lib.mg_linear_bwd(t["dqkv"], P(c["x1"]), w("wq"), t["dx_a"], g("wq"), None, n, 3 * d, d, cd, s)
             lib.mg_layer_norm_bwd_stats_add(t["dx_a"], P(self.h[l]), w("ln1_g"), P(c["mean1"]), P(c["rstd1"]), t["dh"],
                                             t["dh"], g("ln1_g"), g("ln1_b"), n, d, cd, s)
         lib.mg_scatter_add(P(ids), t["dh"], self._g("embed"), n, V, d, ids.dtype, cd, s)

@@ -214,3 +214,34 @@ def test_bshd_output_forms_equal_the_standard_forms(device, dtype, name, causal,
                                scale, int(causal), int(with_mask), dtype, st)
     for a, b, what in zip(g1, g2, ("dq", "dk", "dv")):
         np.testing.assert_array_equal(b.to_numpy(), a.to_numpy(), err_msg=what)
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
+@pytest.mark.parametrize("name,causal,with_mask", MODES)
+@pytest.mark.parametrize("B,H,S,D", [(2, 3, 200, 64), (1, 2, 130, 72), (2, 2, 96, 128), (1, 1, 4, 8), (1, 2, 77, 40)])
+def test_packed_qkv_forms_equal_the_separate_forms(device, dtype, name, causal, with_mask, B, H, S, D):
+    # Q, K, V as slices of one (B,S,3,H,D) tensor and dQ, dK, dV written into one: bit for bit
+    # the separate-tensor entry points (with O and dO in (B,S,H,D)).
+    lib, st = device.lib, device.stream
+    q, k, v, do, m = _inputs(55, B, S, H, D, dtype, with_mask)
+    do_bshd = np.ascontiguousarray(do.transpose(0, 2, 1, 3))
+    qkv = np.ascontiguousarray(np.stack([q, k, v], axis=2))  # (B, S, 3, H, D)
+    bq, bk, bv, bdo, bqkv = (AnyBuffer.from_numpy(device, a, dtype) for a in (q, k, v, do_bshd, qkv))
+    bm = AnyBuffer.from_numpy(device, m if with_mask else np.zeros(8, np.float32), dtype)
+    n = B * S * H * D
+    scale = 1.0 / math.sqrt(D)
+    new = lambda count=n, dt=dtype: AnyBuffer.create(dt, device, count)
+    P = lambda b: b.data_ptr()
+    flags = (B, S, H, D, scale, int(causal), int(with_mask), dtype, st)
+    o1, o2, lse1, lse2 = new(), new(), new(B * H * S, F32), new(B * H * S, F32)
+    lib.mg_flash_attn_fwd_bshd(P(bq), P(bk), P(bv), P(bm), P(o1), P(lse1), *flags)
+    lib.mg_flash_attn_fwd_packed(P(bqkv), P(bm), P(o2), P(lse2), *flags)
+    np.testing.assert_array_equal(o2.to_numpy(), o1.to_numpy())
+    np.testing.assert_array_equal(lse2.to_numpy(), lse1.to_numpy())
+    g = [new() for _ in range(3)]
+    dqkv = AnyBuffer.create(dtype, device, 3 * n, fill=7.0)
+    lib.mg_flash_attn_bwd_bshd(P(bdo), P(o1), P(bq), P(bk), P(bv), P(bm), P(lse1), *(P(x) for x in g), *flags)
+    lib.mg_flash_attn_bwd_packed(P(bdo), P(o2), P(bqkv), P(bm), P(lse2), P(dqkv), *flags)
+    got = dqkv.to_numpy((B, S, 3, H, D))
+    for i, what in enumerate(("dq", "dk", "dv")):
+        np.testing.assert_array_equal(got[:, :, i], g[i].to_numpy((B, S, H, D)), err_msg=what)
