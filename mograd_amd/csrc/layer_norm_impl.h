@@ -429,11 +429,21 @@ struct LayerNormOps {
     return groups;
   }
 
-  template <int VEC, int TPR, int VPT, bool HAS_STATS>
+  // WG: threads per workgroup; TPR of them share a row, so WG / TPR rows are in flight per
+  // workgroup.  One-wave rows (TPR = 64) of tall matrices use 1024 threads: sixteen rows in
+  // flight per workgroup cover the load latency that four do not, and the number of partial
+  // sums (one set per workgroup) stays the same.
+  template <int VEC, int TPR, int VPT, bool HAS_STATS, int WG_ = 0>
   static int launch_bwd(const T* dy, const T* x, const T* gamma, const float* mean, const float* rstd,
                         const T* residual, T* dx, T* dgamma, T* dbeta, int64_t rows, int64_t cols, float eps,
                         hipStream_t stream) {
-    constexpr int WG = TPR == 64 ? 256 : TPR;
+    if constexpr (TPR == 64 && WG_ == 0) {
+      const int64_t tall = static_cast<int64_t>(device_info().cu_count) * env_int("MOGRAD_HIP_LN_TALL_ROWS_PER_CU", 16);
+      if (rows >= tall)
+        return launch_bwd<VEC, TPR, VPT, HAS_STATS, 1024>(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows,
+                                                          cols, eps, stream);
+    }
+    constexpr int WG = WG_ != 0 ? WG_ : (TPR == 64 ? 256 : TPR);
     constexpr int RPW = WG / TPR;
     int64_t groups = bwd_groups(rows, RPW, WG);
     int64_t rows_per_group = ceil_div(ceil_div(rows, groups), RPW) * RPW;
