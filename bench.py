@@ -338,7 +338,7 @@ def bench_attention(args, dev) -> int:
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "causal flash-attention fwd+bwd bf16 (fp32 accumulate) B8 H12 S1024 D64, scale 1/8; "
                                "kernel table also has non-causal B2 H12 S4096 D64"},
-        "roofline": {"bound": "mfma", "kernel": "attn_dkdv_mfma_kernel + attn_dq_mfma_kernel + attn_delta_kernel "
+        "roofline": {"bound": "mfma", "kernel": "attn_bwd_mfma_kernel (dK/dV and dQ walks) + attn_delta_rows_kernel "
                                                 "(mg_flash_attn_bwd, causal S1024)",
                      "achieved": dom["achieved_TFLOPs"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": dom["frac_of_mfma_peak"], "traffic": None},

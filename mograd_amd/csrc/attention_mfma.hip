@@ -451,27 +451,35 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
 // A wave owns MQ tiles of 32 queries; every A fragment read from LDS (K rows, V rows,
 // K^T) feeds MQ MFMAs, which is what keeps LDS bandwidth below the MFMA rate.
 
+// Bytes of LDS the dQ walk stages its tiles in.
+template <int DP>
+constexpr int dq_lds_bytes() {
+  return (DP <= 64 ? 2 : 1) * (2 * 64 * row_stride<DP>() * 2 + DP * tr_stride_dw<64>() * 4);
+}
+
+// The work of workgroup `block` of a dQ launch; `smem` holds dq_lds_bytes<DP>() bytes.
 template <typename T, int DP, int MQ, bool CAUSAL, bool HAS_BIAS>
-__global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
-                                                                       const T* __restrict__ k, const T* __restrict__ v,
-                                                                       const T* __restrict__ mask,
-                                                                       const float* __restrict__ lse,
-                                                                       const float* __restrict__ delta,
-                                                                       T* __restrict__ dq, AttnDims a, float scale) {
+__device__ __forceinline__ void attn_dq_block(const int block, char* smem, const T* __restrict__ d_o,
+                                              const T* __restrict__ q, const T* __restrict__ k,
+                                              const T* __restrict__ v, const T* __restrict__ mask,
+                                              const float* __restrict__ lse, const float* __restrict__ delta,
+                                              T* __restrict__ dq, const AttnDims& a, float scale) {
   constexpr int BM = 128 * MQ, BN = 64, KS = DP / 16, DT = DP / 32;
   // Two copies of each staged tile (one barrier per step) while two workgroups still fit in
   // a CU's LDS; for head dims above 64 one copy and two barriers per step.
   constexpr int NBUF = DP <= 64 ? 2 : 1;
-  __shared__ __attribute__((aligned(16))) uint16_t k_rows_s[NBUF][BN * row_stride<DP>()];
-  __shared__ __attribute__((aligned(16))) uint16_t v_rows_s[NBUF][BN * row_stride<DP>()];
-  __shared__ __attribute__((aligned(16))) uint32_t k_tr_s[NBUF][DP * tr_stride_dw<BN>()];
+  constexpr int ROWS = BN * row_stride<DP>(), TR = DP * tr_stride_dw<BN>();
+  auto k_rows_s = reinterpret_cast<uint16_t(*)[ROWS]>(smem);
+  auto v_rows_s = reinterpret_cast<uint16_t(*)[ROWS]>(smem + NBUF * ROWS * 2);
+  auto k_tr_s = reinterpret_cast<uint32_t(*)[TR]>(smem + 2 * NBUF * ROWS * 2);
+  static_assert(dq_lds_bytes<DP>() == 2 * NBUF * ROWS * 2 + NBUF * TR * 4, "LDS size");
 
   const int nqb = (a.S + BM - 1) / BM;
   // (batch, head) varies fastest across consecutive workgroups, heaviest query blocks first.
   const int n_bh = a.B * a.H;
-  const int qb = CAUSAL ? nqb - 1 - blockIdx.x / n_bh : blockIdx.x / n_bh;
-  const int h = (blockIdx.x % n_bh) % a.H;
-  const int b = (blockIdx.x % n_bh) / a.H;
+  const int qb = CAUSAL ? nqb - 1 - block / n_bh : block / n_bh;
+  const int h = (block % n_bh) % a.H;
+  const int b = (block % n_bh) / a.H;
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int half = lane / 32;
@@ -632,29 +640,40 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
 
 // ---- dK, dV ------------------------------------------------------------------------------
 
+// Bytes of LDS the dK/dV walk stages its tiles and row statistics in.
+template <int DP>
+constexpr int dkdv_lds_bytes() {
+  return 2 * (2 * 64 * row_stride<DP>() * 2 + 2 * DP * tr_stride_dw<64>() * 4 + 2 * 64 * 4);
+}
+
+// The work of workgroup `block` of a dK/dV launch; `smem` holds dkdv_lds_bytes<DP>() bytes.
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
-__global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma_kernel(
-    const T* __restrict__ d_o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
-    const T* __restrict__ mask, const float* __restrict__ lse, const float* __restrict__ delta, T* __restrict__ dk,
-    T* __restrict__ dv, AttnDims a, float scale) {
+__device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, const T* __restrict__ d_o,
+                                                const T* __restrict__ q, const T* __restrict__ k,
+                                                const T* __restrict__ v, const T* __restrict__ mask,
+                                                const float* __restrict__ lse, const float* __restrict__ delta,
+                                                T* __restrict__ dk, T* __restrict__ dv, const AttnDims& a,
+                                                float scale) {
   constexpr int BNK = 128;                 // keys per workgroup
   constexpr int BQ = 64;                   // queries per step
   constexpr int MT = BQ / 32, KS = DP / 16, DT = DP / 32;
   // Two copies of every staged tile: step i computes from copy i % 2 while the tile of step
   // i + 1 is written into the other, so one barrier per step suffices.
-  __shared__ __attribute__((aligned(16))) uint16_t q_rows_s[2][BQ * row_stride<DP>()];
-  __shared__ __attribute__((aligned(16))) uint16_t do_rows_s[2][BQ * row_stride<DP>()];
-  __shared__ __attribute__((aligned(16))) uint32_t q_tr_s[2][DP * tr_stride_dw<BQ>()];
-  __shared__ __attribute__((aligned(16))) uint32_t do_tr_s[2][DP * tr_stride_dw<BQ>()];
-  __shared__ __attribute__((aligned(16))) float lse_ss[2][BQ];
-  __shared__ __attribute__((aligned(16))) float delta_ss[2][BQ];
+  constexpr int ROWS = BQ * row_stride<DP>(), TR = DP * tr_stride_dw<BQ>();
+  auto q_rows_s = reinterpret_cast<uint16_t(*)[ROWS]>(smem);
+  auto do_rows_s = reinterpret_cast<uint16_t(*)[ROWS]>(smem + 2 * ROWS * 2);
+  auto q_tr_s = reinterpret_cast<uint32_t(*)[TR]>(smem + 4 * ROWS * 2);
+  auto do_tr_s = reinterpret_cast<uint32_t(*)[TR]>(smem + 4 * ROWS * 2 + 2 * TR * 4);
+  auto lse_ss = reinterpret_cast<float(*)[BQ]>(smem + 4 * ROWS * 2 + 4 * TR * 4);
+  auto delta_ss = reinterpret_cast<float(*)[BQ]>(smem + 4 * ROWS * 2 + 4 * TR * 4 + 2 * BQ * 4);
+  static_assert(dkdv_lds_bytes<DP>() == 4 * ROWS * 2 + 4 * TR * 4 + 4 * BQ * 4, "LDS size");
 
   // (batch, head) varies fastest across consecutive workgroups.  Causal: earlier key blocks
   // are seen by more queries; all of them launch first.
   const int n_bh = a.B * a.H;
-  const int kb = blockIdx.x / n_bh;
-  const int h = (blockIdx.x % n_bh) % a.H;
-  const int b = (blockIdx.x % n_bh) / a.H;
+  const int kb = block / n_bh;
+  const int h = (block % n_bh) % a.H;
+  const int b = (block % n_bh) / a.H;
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int half = lane / 32;
@@ -826,6 +845,47 @@ __global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma
   }
 }
 
+// ---- backward launches --------------------------------------------------------------------
+
+template <typename T, int DP, int MQ, bool CAUSAL, bool HAS_BIAS>
+__global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
+                                                                       const T* __restrict__ k, const T* __restrict__ v,
+                                                                       const T* __restrict__ mask,
+                                                                       const float* __restrict__ lse,
+                                                                       const float* __restrict__ delta,
+                                                                       T* __restrict__ dq, AttnDims a, float scale) {
+  __shared__ __attribute__((aligned(16))) char smem[dq_lds_bytes<DP>()];
+  attn_dq_block<T, DP, MQ, CAUSAL, HAS_BIAS>(blockIdx.x, smem, d_o, q, k, v, mask, lse, delta, dq, a, scale);
+}
+
+template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
+__global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma_kernel(
+    const T* __restrict__ d_o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+    const T* __restrict__ mask, const float* __restrict__ lse, const float* __restrict__ delta, T* __restrict__ dk,
+    T* __restrict__ dv, AttnDims a, float scale) {
+  __shared__ __attribute__((aligned(16))) char smem[dkdv_lds_bytes<DP>()];
+  attn_dkdv_block<T, DP, CAUSAL, HAS_BIAS>(blockIdx.x, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
+}
+
+// Both walks in one launch (head dims up to 64, where the two have the same occupancy):
+// groups of eight consecutive workgroups alternate between dK/dV and dQ blocks, so every
+// XCD runs both kinds, and short sequences pay for one launch instead of two.  `blocks` is the block count of each walk; the grid is
+// 2 * round_up(blocks, 8) workgroups.
+template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
+__global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_mfma_kernel(
+    const T* __restrict__ d_o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+    const T* __restrict__ mask, const float* __restrict__ lse, const float* __restrict__ delta, T* __restrict__ dq,
+    T* __restrict__ dk, T* __restrict__ dv, AttnDims a, float scale, int blocks) {
+  constexpr int LDS = dkdv_lds_bytes<DP>() > dq_lds_bytes<DP>() ? dkdv_lds_bytes<DP>() : dq_lds_bytes<DP>();
+  __shared__ __attribute__((aligned(16))) char smem[LDS];
+  const int block = (blockIdx.x / 16) * 8 + blockIdx.x % 8;
+  if (block >= blocks) return;
+  if ((blockIdx.x / 8) % 2 == 0)
+    attn_dkdv_block<T, DP, CAUSAL, HAS_BIAS>(block, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
+  else
+    attn_dq_block<T, DP, 1, CAUSAL, HAS_BIAS>(block, smem, d_o, q, k, v, mask, lse, delta, dq, a, scale);
+}
+
 // ---- host side ---------------------------------------------------------------------------
 
 bool attn_mfma_supported(int dtype, int64_t D, const void* const* ptrs, int nptrs) {
@@ -907,16 +967,38 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
   MG_TRY(delta.take(rows * static_cast<int64_t>(sizeof(float))));
   MG_TRY(launch_delta(static_cast<const T*>(d_o), static_cast<const T*>(o), delta.as<float>(), rows, a, stream));
   const int64_t blocks = static_cast<int64_t>(a.B) * a.H * ceil_div(a.S, 128);
-#define MG_LAUNCH(C_, B_)                                                                                              \
-  do {                                                                                                                 \
-    hipLaunchKernelGGL((attn_dkdv_mfma_kernel<T, DP, C_, B_>), dim3(static_cast<unsigned>(blocks)), dim3(kAttnThreads), \
-                       0, stream, static_cast<const T*>(d_o), static_cast<const T*>(q), static_cast<const T*>(k),      \
-                       static_cast<const T*>(v), static_cast<const T*>(mask), lse, delta.as<float>(),                  \
-                       static_cast<T*>(dk), static_cast<T*>(dv), a, scale);                                            \
-    hipLaunchKernelGGL((attn_dq_mfma_kernel<T, DP, 1, C_, B_>), dim3(static_cast<unsigned>(blocks)),                   \
-                       dim3(kAttnThreads), 0, stream, static_cast<const T*>(d_o), static_cast<const T*>(q),            \
-                       static_cast<const T*>(k), static_cast<const T*>(v), static_cast<const T*>(mask), lse,           \
-                       delta.as<float>(), static_cast<T*>(dq), a, scale);                                              \
+  // One launch for both walks up to this sequence length (measured: 3-5% faster up to 512,
+  // even at 1024, 2-3% slower from 2048 on, where the two walks compete for the same CU
+  // instead of filling each other's gaps).  MOGRAD_HIP_ATTN_FUSED_BWD_MAX_S overrides it; 0
+  // always launches dK/dV and dQ separately.
+  static const int fused_max_s = [] {
+    const char* e = std::getenv("MOGRAD_HIP_ATTN_FUSED_BWD_MAX_S");
+    return e && e[0] ? std::atoi(e) : 1024;
+  }();
+  const bool fused = DP <= 64 && a.S <= fused_max_s && 2 * (blocks + 7) < 0x7fffffffLL;
+  const T* d_o_ = static_cast<const T*>(d_o);
+  const T* q_ = static_cast<const T*>(q);
+  const T* k_ = static_cast<const T*>(k);
+  const T* v_ = static_cast<const T*>(v);
+  const T* mask_ = static_cast<const T*>(mask);
+  T* dq_ = static_cast<T*>(dq);
+  T* dk_ = static_cast<T*>(dk);
+  T* dv_ = static_cast<T*>(dv);
+  const dim3 grid(static_cast<unsigned>(blocks)), grid_fused(static_cast<unsigned>(2 * ((blocks + 7) / 8 * 8)));
+#define MG_LAUNCH(C_, B_)                                                                                            \
+  do {                                                                                                               \
+    if constexpr (DP <= 64) {                                                                                        \
+      if (fused) {                                                                                                   \
+        hipLaunchKernelGGL((attn_bwd_mfma_kernel<T, DP, C_, B_>), grid_fused, dim3(kAttnThreads), 0, stream, d_o_,   \
+                           q_, k_, v_, mask_, lse, delta.as<float>(), dq_, dk_, dv_, a, scale,                       \
+                           static_cast<int>(blocks));                                                                \
+        break;                                                                                                       \
+      }                                                                                                              \
+    }                                                                                                                \
+    hipLaunchKernelGGL((attn_dkdv_mfma_kernel<T, DP, C_, B_>), grid, dim3(kAttnThreads), 0, stream, d_o_, q_, k_,    \
+                       v_, mask_, lse, delta.as<float>(), dk_, dv_, a, scale);                                       \
+    hipLaunchKernelGGL((attn_dq_mfma_kernel<T, DP, 1, C_, B_>), grid, dim3(kAttnThreads), 0, stream, d_o_, q_, k_,   \
+                       v_, mask_, lse, delta.as<float>(), dq_, a, scale);                                            \
   } while (0)
   if (causal) MG_LAUNCH(true, false);
   else if (has_bias) MG_LAUNCH(false, true);

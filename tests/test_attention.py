@@ -104,6 +104,20 @@ def test_half_error_budget(device, dtype, budget_fwd, budget_bwd, name, causal, 
 
 
 @pytest.mark.parametrize("causal", [True, False])
+def test_long_ragged_sequence(device, causal):
+    # Past 1024 tokens the head-dim-64 backward launches its dK/dV and dQ walks separately
+    # (one launch below that); 1100 is not a multiple of any tile.
+    B, H, S, D = 1, 2, 1100, 64
+    q, k, v, do, _ = _inputs(56, B, S, H, D, BF16, False)
+    o, lse, dq, dk, dv = _fwd_bwd(device, q, k, v, do, None, causal, dtype=BF16)
+    ro, rl = O.sdpa_fwd(q, k, v, None, causal)
+    assert _max_err(o, ro) <= 1.6e-2 and _max_err(lse, rl) <= 1e-3 * max(1.0, float(np.abs(rl).max()))
+    for got, want, what in zip((dq, dk, dv), O.sdpa_bwd(q, k, v, do, None, causal), ("dq", "dk", "dv")):
+        bound = RTOL_BF16_ATTN * (np.abs(want) + np.abs(want).max())
+        assert np.all(np.abs(got - want) <= bound), f"{what}: worst {np.max(np.abs(got - want) / bound):.3g}"
+
+
+@pytest.mark.parametrize("causal", [True, False])
 def test_bf16_gradients_rtol(device, causal):
     # Parity bar for bf16 attention gradients: rtol 2e-2 (with an absolute floor at the
     # same fraction of each tensor's largest entry, for entries that cancel to ~0).
