@@ -82,15 +82,40 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
     if (splits > max_splits) splits = max_splits;
     if (splits > 64) splits = 64;
   }
+  // Tiles copied straight into LDS (gemm_16bit_pipe_kernel) where that measured faster: an
+  // operand that is not k-contiguous is transposed by the LDS read instead of in registers
+  // (dX 15-25 %, dW 5-20 % faster at Linear-layer shapes, 20-30 % at 4096^3 and up), and long
+  // K loops gain from the single barrier per step (forward 8-10 % from K = 1024).  Short-K
+  // products of two k-contiguous operands stay with the register-staged kernel (4-8 %
+  // faster there), as does every shape the copy cannot take.  The pair is k per step and
+  // copies of the tiles: (32, 2) runs four workgroups per CU, (64, 2) two.
+  // MOGRAD_HIP_GEMM16_PIPE = 0 | 322 | 642 overrides the choice.
+  int pipe = 0;
+  if constexpr (!RAGGED) {
+    if (g.K % kG16BK == 0 && mult8(g.M) && mult8(g.N)) {
+      const int64_t k_wg = ceil_div(g.K, splits);  // the K range one workgroup walks
+      if (A_KC && B_KC) pipe = k_wg >= 1024 ? 642 : 0;
+      else pipe = k_wg >= 4096 ? 642 : 322;
+      pipe = static_cast<int>(env_int("MOGRAD_HIP_GEMM16_PIPE", pipe));
+    }
+  }
+#define MG_GEMM16_LAUNCH(BIAS_, SPLIT_, GRID_, PARTIAL_, KPS_, EP_)                                                     \
+  do {                                                                                                                 \
+    auto launch = [&](auto kernel) {                                                                                   \
+      hipLaunchKernelGGL(kernel, GRID_, dim3(kGemmThreads), 0, stream, a, b, bias, c, PARTIAL_, M, N, K, lda, ldb, g.N,  \
+                         g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n, KPS_, EP_);                                        \
+    };                                                                                                                 \
+    if constexpr (!RAGGED) {                                                                                           \
+      if (pipe == 322) { launch(gemm_16bit_pipe_kernel<T, A_KC, B_KC, BIAS_, SPLIT_, 32, 2>); break; }                 \
+      if (pipe == 642) { launch(gemm_16bit_pipe_kernel<T, A_KC, B_KC, BIAS_, SPLIT_, 64, 2>); break; }                 \
+    }                                                                                                                  \
+    launch(gemm_16bit_mfma_kernel<T, A_KC, B_KC, BIAS_, SPLIT_, RAGGED>);                                              \
+  } while (0)
   if (splits <= 1) {
-    if (bias)
-      hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, true, false, RAGGED>), dim3(static_cast<unsigned>(blocks)),
-                         dim3(kGemmThreads), 0, stream, a, b, bias, c, nullptr, M, N, K, lda, ldb, g.N, g.bsa, g.bsb,
-                         g.M * g.N, tiles_m, tiles_n, K, epilogue_of<T>(g));
-    else
-      hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, false, false, RAGGED>), dim3(static_cast<unsigned>(blocks)),
-                         dim3(kGemmThreads), 0, stream, a, b, bias, c, nullptr, M, N, K, lda, ldb, g.N, g.bsa, g.bsb,
-                         g.M * g.N, tiles_m, tiles_n, K, epilogue_of<T>(g));
+    const dim3 grid(static_cast<unsigned>(blocks));
+    float* no_partial = nullptr;
+    if (bias) MG_GEMM16_LAUNCH(true, false, grid, no_partial, K, epilogue_of<T>(g));
+    else MG_GEMM16_LAUNCH(false, false, grid, no_partial, K, epilogue_of<T>(g));
     MG_LAUNCH_CHECK();
     return MG_OK;
   }
@@ -101,10 +126,9 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
   Scratch partial;
   const int64_t numel = g.batch * g.M * g.N;
   MG_TRY(partial.take(static_cast<int64_t>(splits) * numel * static_cast<int64_t>(sizeof(float))));
-  hipLaunchKernelGGL((gemm_16bit_mfma_kernel<T, A_KC, B_KC, false, true, RAGGED>),
-                     dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(splits), static_cast<unsigned>(g.batch)),
-                     dim3(kGemmThreads), 0, stream, a, b, bias, c, partial.as<float>(), M, N, K, lda, ldb, g.N, g.bsa,
-                     g.bsb, g.M * g.N, tiles_m, tiles_n, k_per_split, GemmEpilogue<T>{nullptr, nullptr, 0});
+  const dim3 grid(static_cast<unsigned>(tiles), static_cast<unsigned>(splits), static_cast<unsigned>(g.batch));
+  MG_GEMM16_LAUNCH(false, true, grid, partial.as<float>(), k_per_split, (GemmEpilogue<T>{nullptr, nullptr, 0}));
+#undef MG_GEMM16_LAUNCH
   MG_LAUNCH_CHECK();
   const unsigned rblocks = static_cast<unsigned>(ceil_div(numel, 256));
   if (bias)

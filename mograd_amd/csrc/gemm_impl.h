@@ -436,73 +436,21 @@ __device__ __forceinline__ uint4 gemm16_frag(const uint16_t* __restrict__ lds, i
   return *reinterpret_cast<const uint4*>(lds + row * kG16Stride + g * 8);
 }
 
-template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, bool RAGGED>
-__global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
-    const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C,
-    float* __restrict__ partial, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb,
-    int64_t bsc, int tiles_m, int tiles_n, int k_per_split, GemmEpilogue<T> ep) {
-  __shared__ __attribute__((aligned(16))) uint16_t lds_a[kGemmBM * kG16Stride];
-  __shared__ __attribute__((aligned(16))) uint16_t lds_b[kGemmBN * kG16Stride];
-
-  const int tiles = tiles_m * tiles_n;
-  // Split along K: grid (tiles, splits, batch).  Otherwise the batch index is folded into x.
-  const int batch = SPLIT_K ? blockIdx.z : blockIdx.x / tiles;
-  int tm, tn;
-  gemm_tile_of_block(blockIdx.x % tiles, tiles_m, tiles_n, tm, tn);
-  const int m0 = tm * kGemmBM;
-  const int n0 = tn * kGemmBN;
-  A += batch * bsa;
-  B += batch * bsb;
-  const int k_begin = SPLIT_K ? blockIdx.y * k_per_split : 0;
-  const int k_end = SPLIT_K ? min(K, k_begin + k_per_split) : K;
-
-  const int wave = threadIdx.x / kWave;
-  const int lane = threadIdx.x % kWave;
-  const int wm = (wave / 2) * 64;
-  const int wn = (wave % 2) * 64;
-
-  floatx16 acc[2][2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-  Gemm16Stage sa, sb;
-  gemm16_load<T, A_KC, RAGGED>(A, lda, m0, k_begin, M, k_end, sa);
-  gemm16_load<T, B_KC, RAGGED>(B, ldb, n0, k_begin, N, k_end, sb);
-
-  for (int k0 = k_begin; k0 < k_end; k0 += kG16BK) {
-    gemm16_store<A_KC>(lds_a, sa);
-    gemm16_store<B_KC>(lds_b, sb);
-    __syncthreads();
-    if (k0 + kG16BK < k_end) {
-      gemm16_load<T, A_KC, RAGGED>(A, lda, m0, k0 + kG16BK, M, k_end, sa);
-      gemm16_load<T, B_KC, RAGGED>(B, ldb, n0, k0 + kG16BK, N, k_end, sb);
-    }
-#pragma unroll
-    for (int ks = 0; ks < kG16BK / 16; ++ks) {
-      const uint4 fa0 = gemm16_frag<!A_KC>(lds_a, wm, ks, lane);
-      const uint4 fa1 = gemm16_frag<!A_KC>(lds_a, wm + 32, ks, lane);
-      const uint4 fb0 = gemm16_frag<!B_KC>(lds_b, wn, ks, lane);
-      const uint4 fb1 = gemm16_frag<!B_KC>(lds_b, wn + 32, ks, lane);
-      acc[0][0] = GemmMma16<T>::run(fa0, fb0, acc[0][0]);
-      acc[0][1] = GemmMma16<T>::run(fa0, fb1, acc[0][1]);
-      acc[1][0] = GemmMma16<T>::run(fa1, fb0, acc[1][0]);
-      acc[1][1] = GemmMma16<T>::run(fa1, fb1, acc[1][1]);
-    }
-    __syncthreads();
-  }
-
-  // Output.  The accumulators have lanes along n and registers along m, so a direct store
-  // writes 2-byte elements.  When rows of C can be written 16 bytes at a time, each wave
-  // instead transposes its 64x64 tile through its own quarter of the (now idle) staging
-  // memory and stores eight elements per lane.
+// Output of one 128x128 tile from the four waves' accumulators (wave tile 64x64 at (wm, wn)).
+// The accumulators have lanes along n and registers along m, so a direct store writes
+// 2-byte elements.  When rows of C can be written 16 bytes at a time, each wave instead
+// transposes its tile through `mine`, 64 rows of kG16Stride elements of LDS that no wave
+// reads any more, and stores eight elements per lane.  SPLIT_K: fp32 partial tiles go to
+// partial[(split * batches + batch), M, N].
+template <typename T, bool HAS_BIAS, bool SPLIT_K>
+__device__ __forceinline__ void gemm16_write_tile(const floatx16 (&acc)[2][2], uint16_t* __restrict__ mine,
+                                                  const T* __restrict__ bias, T* __restrict__ C,
+                                                  float* __restrict__ partial, int M, int N, int64_t ldc, int64_t bsc,
+                                                  int batch, int split, int batches, int m0, int n0, int wm, int wn,
+                                                  int lane, const GemmEpilogue<T>& ep) {
   if constexpr (!SPLIT_K) {
     const bool wide_out = (N % 8 == 0) && (ldc % 8 == 0) && (bsc % 8 == 0) && (reinterpret_cast<uintptr_t>(C) % 16 == 0);
     if (wide_out) {
-      uint16_t* mine = (wave < 2 ? lds_a : lds_b) + (wave % 2) * 64 * kG16Stride;
 #pragma unroll
       for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
@@ -567,7 +515,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
         const int row = m0 + wm + ti * 32 + (r / 4) * 8 + (lane / 32) * 4 + (r % 4);
         if (row < M) {
           if constexpr (SPLIT_K)
-            partial[((static_cast<int64_t>(blockIdx.y) * gridDim.z + batch) * M + row) * N + col] = acc[ti][tj][r];
+            partial[((static_cast<int64_t>(split) * batches + batch) * M + row) * N + col] = acc[ti][tj][r];
           else {
             const int64_t at = batch * bsc + static_cast<int64_t>(row) * ldc + col;
             C[at] = gemm_finish<T>(acc[ti][tj][r] + bv, ep, at);
@@ -575,6 +523,268 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
         }
       }
     }
+}
+
+template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, bool RAGGED>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
+    const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C,
+    float* __restrict__ partial, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb,
+    int64_t bsc, int tiles_m, int tiles_n, int k_per_split, GemmEpilogue<T> ep) {
+  __shared__ __attribute__((aligned(16))) uint16_t lds_a[kGemmBM * kG16Stride];
+  __shared__ __attribute__((aligned(16))) uint16_t lds_b[kGemmBN * kG16Stride];
+
+  const int tiles = tiles_m * tiles_n;
+  // Split along K: grid (tiles, splits, batch).  Otherwise the batch index is folded into x.
+  const int batch = SPLIT_K ? blockIdx.z : blockIdx.x / tiles;
+  int tm, tn;
+  gemm_tile_of_block(blockIdx.x % tiles, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * kGemmBM;
+  const int n0 = tn * kGemmBN;
+  A += batch * bsa;
+  B += batch * bsb;
+  const int k_begin = SPLIT_K ? blockIdx.y * k_per_split : 0;
+  const int k_end = SPLIT_K ? min(K, k_begin + k_per_split) : K;
+
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int wm = (wave / 2) * 64;
+  const int wn = (wave % 2) * 64;
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  Gemm16Stage sa, sb;
+  gemm16_load<T, A_KC, RAGGED>(A, lda, m0, k_begin, M, k_end, sa);
+  gemm16_load<T, B_KC, RAGGED>(B, ldb, n0, k_begin, N, k_end, sb);
+
+  for (int k0 = k_begin; k0 < k_end; k0 += kG16BK) {
+    gemm16_store<A_KC>(lds_a, sa);
+    gemm16_store<B_KC>(lds_b, sb);
+    __syncthreads();
+    if (k0 + kG16BK < k_end) {
+      gemm16_load<T, A_KC, RAGGED>(A, lda, m0, k0 + kG16BK, M, k_end, sa);
+      gemm16_load<T, B_KC, RAGGED>(B, ldb, n0, k0 + kG16BK, N, k_end, sb);
+    }
+#pragma unroll
+    for (int ks = 0; ks < kG16BK / 16; ++ks) {
+      const uint4 fa0 = gemm16_frag<!A_KC>(lds_a, wm, ks, lane);
+      const uint4 fa1 = gemm16_frag<!A_KC>(lds_a, wm + 32, ks, lane);
+      const uint4 fb0 = gemm16_frag<!B_KC>(lds_b, wn, ks, lane);
+      const uint4 fb1 = gemm16_frag<!B_KC>(lds_b, wn + 32, ks, lane);
+      acc[0][0] = GemmMma16<T>::run(fa0, fb0, acc[0][0]);
+      acc[0][1] = GemmMma16<T>::run(fa0, fb1, acc[0][1]);
+      acc[1][0] = GemmMma16<T>::run(fa1, fb0, acc[1][0]);
+      acc[1][1] = GemmMma16<T>::run(fa1, fb1, acc[1][1]);
+    }
+    __syncthreads();
+  }
+
+  uint16_t* mine = (wave < 2 ? lds_a : lds_b) + (wave % 2) * 64 * kG16Stride;  // staging memory, idle now
+  gemm16_write_tile<T, HAS_BIAS, SPLIT_K>(acc, mine, bias, C, partial, M, N, ldc, bsc, batch,
+                                          SPLIT_K ? static_cast<int>(blockIdx.y) : 0, SPLIT_K ? static_cast<int>(gridDim.z) : 1,
+                                          m0, n0, wm, wn, lane, ep);
+}
+
+// ------------------------------------------------------------------------------------
+// The same product with the tiles copied global memory -> LDS by the memory pipeline itself
+// (`global_load_lds_dwordx4`: every lane names a 16-byte source, the wave's 64 chunks land
+// back to back at an LDS address common to the wave), NSTAGE k-steps deep.  No registers
+// hold data in flight, so several steps' loads are outstanding while one step is multiplied:
+// what short-K products at a few hundred FLOP per byte need, being bound by memory latency
+// and not by the matrix cores.  Operands as above, all extents and strides multiples of 8
+// elements, K (and every K split) a multiple of 64.
+//
+// LDS image of one operand's step (16 KB), chosen per 16-byte chunk by which source chunk
+// each lane names:
+//   k-contiguous: [128 rows][8 chunks], chunk c of row r at position c ^ (r % 8): the 32
+//     rows a fragment read touches spread over all banks;
+//   otherwise: [64 k][16 chunks of 8 rows], chunk c of k-row kk at position
+//     c ^ (2 * (kk % 4)), read with `ds_read_b64_tr_b16` (within 16 lanes, lane i supplies
+//     the four elements 4*i .. 4*i+3 of a 4 x 16 block and receives column i), which turns
+//     four k-rows of 16 consecutive rows into each lane's four consecutive k.
+// ------------------------------------------------------------------------------------
+
+// (Shown for 64 k per step; with 32 a k-contiguous row is 4 chunks and chunk c of row r
+// sits at c ^ ((r / 2) % 4), the other image simply has 32 k-rows.)
+
+typedef short gemm_i16x4 __attribute__((ext_vector_type(4)));
+
+// The four 16-byte source chunks this thread names for every k-step of one operand, as
+// element offsets from the operand's (batch, k_begin) origin; they advance by BK
+// (k-contiguous) or BK * ld per step.
+template <bool KC, int BK>
+__device__ __forceinline__ void gemm16_pipe_sources(int64_t ld, int o0, int O, int64_t (&src)[BK / 16]) {
+  constexpr int CPR = BK / 8;  // chunks per k-contiguous row
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+#pragma unroll
+  for (int i = 0; i < BK / 16; ++i) {
+    const int slot = (i * 4 + wave) * kWave + lane;  // 16-byte position in the LDS image
+    if constexpr (KC) {
+      const int r = slot / CPR, c = (slot % CPR) ^ ((r / (8 / CPR)) % CPR);
+      src[i] = static_cast<int64_t>(min(o0 + r, O - 1)) * ld + c * 8;  // rows past the edge are never stored
+    } else {
+      const int kk = slot / 16, c = (slot % 16) ^ (2 * (kk % 4));
+      const int o = o0 + c * 8;
+      src[i] = static_cast<int64_t>(kk) * ld + (o < O ? o : o0);
+    }
+  }
+}
+
+// Written as assembly on purpose.  Through the compiler's builtin for this instruction every
+// later LDS read of a kind whose aliasing it cannot judge (the transposing reads here) gets a
+// wait for *all* outstanding copies, the younger steps' included, which would undo the
+// pipeline; the waits are placed by hand in the kernel instead (MG_WAIT_VMCNT).  m0 (the
+// wave's LDS destination) is written here and used by nothing else in these kernels.
+template <int BK>
+__device__ __forceinline__ void gemm16_pipe_issue(const uint16_t* base, const int64_t* src, char* lds_step) {
+  using lds_ptr = __attribute__((address_space(3))) char*;
+  const int wave = threadIdx.x / kWave;
+  const unsigned dst = static_cast<unsigned>(reinterpret_cast<uintptr_t>((lds_ptr)lds_step)) + wave * 1024;
+#pragma unroll
+  for (int i = 0; i < BK / 16; ++i) {
+    const unsigned dst_i = __builtin_amdgcn_readfirstlane(dst + i * 4096);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst_i), "v"(base + src[i]) : "memory");
+  }
+}
+
+// MFMA operand fragment: row o_base + lane % 32, k = ks * 16 + (lane / 32) * 8 .. + 7.
+template <bool KC, int BK>
+__device__ __forceinline__ uint4 gemm16_pipe_frag(const char* __restrict__ lds_step, int o_base, int ks, int lane) {
+  if constexpr (KC) {
+    constexpr int CPR = BK / 8;
+    const int r = o_base + lane % 32;
+    const int g = ks * 2 + lane / 32;
+    return *reinterpret_cast<const uint4*>(lds_step + r * (BK * 2) + ((g ^ ((r / (8 / CPR)) % CPR)) * 16));
+  } else {
+    const int o = o_base + ((lane / 16) % 2) * 16 + 4 * (lane % 4);  // first of the 4 rows this lane supplies
+    const int kq = (lane % 16) / 4;                                 // its k-row within a group of 4
+    const int kk = ks * 16 + (lane / 32) * 8 + kq;
+    const char* at = lds_step + kk * 256 + (((o / 16) ^ kq) * 32) + (o % 16) * 2;
+    using lds_i16x4 = __attribute__((address_space(3))) gemm_i16x4;
+    const gemm_i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        reinterpret_cast<lds_i16x4*>(reinterpret_cast<uintptr_t>(at)));
+    const gemm_i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        reinterpret_cast<lds_i16x4*>(reinterpret_cast<uintptr_t>(at + 4 * 256)));
+    uint2 l = __builtin_bit_cast(uint2, lo), h = __builtin_bit_cast(uint2, hi);
+    return make_uint4(l.x, l.y, h.x, h.y);
+  }
+}
+
+// s_waitcnt with only the vector-memory counter set (gfx9 encoding: vmcnt in bits 3:0 and
+// 15:14, expcnt 6:4 and lgkmcnt 11:8 left at "no wait").
+#define MG_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0f70)
+
+// Workgroups of the pipelined kernel that fit a CU: by LDS (160 KB) and, at four waves per
+// workgroup, by the register file (at most four).
+constexpr int gemm16_pipe_lds_bytes(int bk, int nstage) {
+  const int stages = nstage * 2 * 128 * bk * 2, out = 4 * 64 * kG16Stride * 2;  // the output tile is transposed here
+  return stages > out ? stages : out;
+}
+constexpr int gemm16_pipe_occupancy(int bk, int nstage) {
+  const int by_lds = 160 * 1024 / gemm16_pipe_lds_bytes(bk, nstage);
+  return by_lds < 1 ? 1 : (by_lds > 4 ? 4 : by_lds);
+}
+
+template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, int BK, int NSTAGE>
+__global__ __launch_bounds__(kGemmThreads, gemm16_pipe_occupancy(BK, NSTAGE)) void gemm_16bit_pipe_kernel(
+    const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C,
+    float* __restrict__ partial, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb,
+    int64_t bsc, int tiles_m, int tiles_n, int k_per_split, GemmEpilogue<T> ep) {
+  static_assert(NSTAGE >= 2 && NSTAGE <= 4 && (BK == 32 || BK == 64), "stages");
+  constexpr int NI = BK / 16;  // copy requests per thread, operand and step
+  constexpr int OP = 128 * BK * 2;  // bytes of one operand's step
+  __shared__ __attribute__((aligned(1024))) char lds[gemm16_pipe_lds_bytes(BK, NSTAGE)];
+
+  const int tiles = tiles_m * tiles_n;
+  const int batch = SPLIT_K ? blockIdx.z : blockIdx.x / tiles;
+  int tm, tn;
+  gemm_tile_of_block(blockIdx.x % tiles, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * kGemmBM;
+  const int n0 = tn * kGemmBN;
+  const int k_begin = SPLIT_K ? blockIdx.y * k_per_split : 0;
+  const int k_end = SPLIT_K ? min(K, k_begin + k_per_split) : K;
+  const int steps = (k_end - k_begin) / BK;
+  A += batch * bsa + (A_KC ? static_cast<int64_t>(k_begin) : k_begin * lda);
+  B += batch * bsb + (B_KC ? static_cast<int64_t>(k_begin) : k_begin * ldb);
+  const int64_t a_step = A_KC ? BK : BK * lda;
+  const int64_t b_step = B_KC ? BK : BK * ldb;
+
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int wm = (wave / 2) * 64;
+  const int wn = (wave % 2) * 64;
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const uint16_t* a16 = reinterpret_cast<const uint16_t*>(A);
+  const uint16_t* b16 = reinterpret_cast<const uint16_t*>(B);
+  int64_t src_a[NI], src_b[NI];
+  gemm16_pipe_sources<A_KC, BK>(lda, m0, M, src_a);
+  gemm16_pipe_sources<B_KC, BK>(ldb, n0, N, src_b);
+
+  // Steps 0 .. NSTAGE-2 are requested up front; iteration `it` then waits for step `it`
+  // (its own 2 * NI requests; the barrier covers the other waves'), requests step
+  // it + NSTAGE - 1 into the copy that step it - 1 was just multiplied from, and multiplies.
+#pragma unroll
+  for (int s = 0; s < NSTAGE - 1; ++s)
+    if (s < steps) {
+      gemm16_pipe_issue<BK>(a16 + s * a_step, src_a, lds + (2 * s) * OP);
+      gemm16_pipe_issue<BK>(b16 + s * b_step, src_b, lds + (2 * s + 1) * OP);
+    }
+  int cur = 0, nxt = NSTAGE - 1;
+  for (int it = 0; it < steps; ++it) {
+    if (it + NSTAGE - 2 < steps) MG_WAIT_VMCNT(2 * NI * (NSTAGE - 2));  // all but the NSTAGE-2 younger steps
+    else MG_WAIT_VMCNT(0);
+    // A plain barrier: __syncthreads() carries a fence that waits for every outstanding
+    // copy into LDS, the younger steps' included.
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (it + NSTAGE - 1 < steps) {
+      gemm16_pipe_issue<BK>(a16 + (it + NSTAGE - 1) * a_step, src_a, lds + (2 * nxt) * OP);
+      gemm16_pipe_issue<BK>(b16 + (it + NSTAGE - 1) * b_step, src_b, lds + (2 * nxt + 1) * OP);
+    }
+    const char* la = lds + (2 * cur) * OP;
+    const char* lb = la + OP;
+    // The fragments of k-slice ks + 1 are requested before the products of slice ks, so
+    // their LDS latency runs under four MFMAs.
+    uint4 fa[2][2], fb[2][2];
+    fa[0][0] = gemm16_pipe_frag<A_KC, BK>(la, wm, 0, lane);
+    fa[0][1] = gemm16_pipe_frag<A_KC, BK>(la, wm + 32, 0, lane);
+    fb[0][0] = gemm16_pipe_frag<B_KC, BK>(lb, wn, 0, lane);
+    fb[0][1] = gemm16_pipe_frag<B_KC, BK>(lb, wn + 32, 0, lane);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      const int c = ks % 2, n = c ^ 1;
+      if (ks + 1 < BK / 16) {
+        fa[n][0] = gemm16_pipe_frag<A_KC, BK>(la, wm, ks + 1, lane);
+        fa[n][1] = gemm16_pipe_frag<A_KC, BK>(la, wm + 32, ks + 1, lane);
+        fb[n][0] = gemm16_pipe_frag<B_KC, BK>(lb, wn, ks + 1, lane);
+        fb[n][1] = gemm16_pipe_frag<B_KC, BK>(lb, wn + 32, ks + 1, lane);
+      }
+      acc[0][0] = GemmMma16<T>::run(fa[c][0], fb[c][0], acc[0][0]);
+      acc[0][1] = GemmMma16<T>::run(fa[c][0], fb[c][1], acc[0][1]);
+      acc[1][0] = GemmMma16<T>::run(fa[c][1], fb[c][0], acc[1][0]);
+      acc[1][1] = GemmMma16<T>::run(fa[c][1], fb[c][1], acc[1][1]);
+    }
+    cur = cur + 1 == NSTAGE ? 0 : cur + 1;
+    nxt = nxt + 1 == NSTAGE ? 0 : nxt + 1;
+  }
+  __syncthreads();  // every wave is done with the staged tiles: their memory serves the output
+
+  uint16_t* mine = reinterpret_cast<uint16_t*>(lds) + wave * 64 * kG16Stride;
+  gemm16_write_tile<T, HAS_BIAS, SPLIT_K>(acc, mine, bias, C, partial, M, N, ldc, bsc, batch,
+                                          SPLIT_K ? static_cast<int>(blockIdx.y) : 0, SPLIT_K ? static_cast<int>(gridDim.z) : 1,
+                                          m0, n0, wm, wn, lane, ep);
 }
 
 // out[i] = sum_s partial[s][i] (+ bias[i % N]), converted to T.  A workgroup covers 64

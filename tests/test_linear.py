@@ -198,6 +198,34 @@ def test_half_precision_mfma_paths(device, dtype, rtol, M, N, K):
         assert_close(got, want, rtol, rtol * np.abs(want).max(), name)
 
 
+@pytest.mark.parametrize("dtype,rtol", [(F16, 2e-3), (BF16, 1.6e-2)])
+@pytest.mark.parametrize("M,N,K", [(256, 384, 512), (384, 128, 1536), (200, 136, 256), (128, 64, 4096), (1024, 384, 1024),
+                                   (72, 1536, 64)])
+def test_tile_staging_variants_agree(device, monkeypatch, dtype, rtol, M, N, K):
+    # The 16-bit products have a register-staged kernel (0) and one whose tiles are copied
+    # straight into LDS, 32 or 64 k per step (322, 642); the library picks by operand layout
+    # and K.  All accumulate each output element over k in the same order on the same MFMA,
+    # so forcing either must not change a bit, for every operand layout (forward k/k, dX
+    # k/n, dW m/n, the last split along K for the tall shapes) and at ragged tile edges.
+    x = round_to_dtype(normal(49, 0, (M, K)), dtype)
+    w = round_to_dtype(normal(49, 1, (N, K), std=0.05), dtype)
+    b = round_to_dtype(normal(49, 2, (N,), std=0.1), dtype)
+    dy = round_to_dtype(normal(49, 3, (M, N), std=0.5), dtype)
+    results = {}
+    for variant in ("0", "322", "642"):
+        monkeypatch.setenv("MOGRAD_HIP_GEMM16_PIPE", variant)
+        results[variant] = _linear_all(device, x, w, b, dy, dtype)
+    monkeypatch.delenv("MOGRAD_HIP_GEMM16_PIPE")
+    results["auto"] = _linear_all(device, x, w, b, dy, dtype)
+    for variant in ("322", "642", "auto"):
+        for got, base, name in zip(results[variant], results["0"], ("y", "dx", "dw", "db")):
+            np.testing.assert_array_equal(got, base, err_msg=f"{name}, variant {variant}")
+    y, dx, dw, _ = results["auto"]
+    for got, want, name in ((y, O.matmul_bias_bt(x, w, b), "y"), (dx, O.linear_grad_x(dy, w), "dx"),
+                            (dw, O.linear_grad_w(dy, x), "dw")):
+        assert_close(got, want, rtol, rtol * np.abs(want).max(), name)
+
+
 def test_bf16_linear_bwd_entry_gpt_shapes(device):
     # (tokens, d_model) x (d_ff, d_model): the GPT block's MLP up-projection, scaled down
     M, N, K = 2048, 1536, 384
