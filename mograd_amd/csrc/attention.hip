@@ -73,13 +73,17 @@ static int bwd_generic(const void* d_o, const void* o, const void* q, const void
 
 }  // namespace mg
 
-static int flash_attn_fwd_impl(int o_bshd, int64_t ld, const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, int64_t B,
-                      int64_t S, int64_t H, int64_t D, float scale, int causal, int has_bias, int dtype,
-                      mg_stream stream) {
+// o_bshd: O and dO are laid out (B, S, H, D) like Q, K, V instead of (B, H, S, D).
+// ld: elements from one token's head-0 slice to the next token's in Q, K, V and their
+// gradients; 0 means H * D (each tensor contiguous).
+static int flash_attn_fwd_impl(int o_bshd, int64_t ld, const void* q, const void* k, const void* v, const void* mask,
+                               void* o, float* lse, int64_t B, int64_t S, int64_t H, int64_t D, float scale, int causal,
+                               int has_bias, int dtype, mg_stream stream) {
   MG_TRY(mg::check_attn("flash_attn_fwd", B, S, H, D, causal, has_bias, dtype));
   if (!q || !k || !v || !o || !lse || (has_bias && !mask))
     return mg::fail(MG_ERR_INVALID, "flash_attn_fwd: null pointer argument");
-  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D), o_bshd, ld ? ld : H * D};
+  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D),
+                       o_bshd,              ld ? ld : H * D};
   hipStream_t s = mg::to_stream(stream);
   const void* ptrs[] = {q, k, v, o, has_bias ? mask : nullptr};
   if (mg::attn_mfma_supported(dtype, D, ptrs, 5))
@@ -91,13 +95,15 @@ static int flash_attn_fwd_impl(int o_bshd, int64_t ld, const void* q, const void
   }
 }
 
-static int flash_attn_bwd_impl(int o_bshd, int64_t ld, const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
-                      const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t S, int64_t H, int64_t D,
-                      float scale, int causal, int has_bias, int dtype, mg_stream stream) {
+static int flash_attn_bwd_impl(int o_bshd, int64_t ld, const void* d_o, const void* o, const void* q, const void* k,
+                               const void* v, const void* mask, const float* lse, void* dq, void* dk, void* dv,
+                               int64_t B, int64_t S, int64_t H, int64_t D, float scale, int causal, int has_bias,
+                               int dtype, mg_stream stream) {
   MG_TRY(mg::check_attn("flash_attn_bwd", B, S, H, D, causal, has_bias, dtype));
   if (!d_o || !o || !q || !k || !v || !lse || !dq || !dk || !dv || (has_bias && !mask))
     return mg::fail(MG_ERR_INVALID, "flash_attn_bwd: null pointer argument");
-  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D), o_bshd, ld ? ld : H * D};
+  const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D),
+                       o_bshd,              ld ? ld : H * D};
   hipStream_t s = mg::to_stream(stream);
   const void* ptrs[] = {d_o, o, q, k, v, dq, dk, dv, has_bias ? mask : nullptr};
   if (mg::attn_mfma_supported(dtype, D, ptrs, 9))
@@ -129,13 +135,15 @@ int mg_flash_attn_fwd_bshd(const void* q, const void* k, const void* v, const vo
 int mg_flash_attn_bwd(const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
                       const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t S, int64_t H, int64_t D,
                       float scale, int causal, int has_bias, int dtype, mg_stream stream) {
-  return flash_attn_bwd_impl(0, 0, d_o, o, q, k, v, mask, lse, dq, dk, dv, B, S, H, D, scale, causal, has_bias, dtype, stream);
+  return flash_attn_bwd_impl(0, 0, d_o, o, q, k, v, mask, lse, dq, dk, dv, B, S, H, D, scale, causal, has_bias, dtype,
+                             stream);
 }
 
 int mg_flash_attn_bwd_bshd(const void* d_o, const void* o, const void* q, const void* k, const void* v, const void* mask,
                            const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t S, int64_t H, int64_t D,
                            float scale, int causal, int has_bias, int dtype, mg_stream stream) {
-  return flash_attn_bwd_impl(1, 0, d_o, o, q, k, v, mask, lse, dq, dk, dv, B, S, H, D, scale, causal, has_bias, dtype, stream);
+  return flash_attn_bwd_impl(1, 0, d_o, o, q, k, v, mask, lse, dq, dk, dv, B, S, H, D, scale, causal, has_bias, dtype,
+                             stream);
 }
 
 int mg_flash_attn_fwd_packed(const void* qkv, const void* mask, void* o, float* lse, int64_t B, int64_t S, int64_t H,

@@ -869,8 +869,8 @@ __global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma
 
 // Both walks in one launch (head dims up to 64, where the two have the same occupancy):
 // groups of eight consecutive workgroups alternate between dK/dV and dQ blocks, so every
-// XCD runs both kinds, and short sequences pay for one launch instead of two.  `blocks` is the block count of each walk; the grid is
-// 2 * round_up(blocks, 8) workgroups.
+// XCD runs both kinds, and short sequences pay for one launch instead of two.  `blocks` is
+// the block count of each walk; the grid is 2 * round_up(blocks, 8) workgroups.
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
 __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_mfma_kernel(
     const T* __restrict__ d_o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
@@ -943,13 +943,17 @@ static int launch_delta(const T* d_o, const T* o, float* delta, int64_t rows, co
   const bool vec = D % 8 == 0 && (cpr & (cpr - 1)) == 0 && cpr <= 16;
   if (vec) {
     const dim3 grid(static_cast<unsigned>(ceil_div(rows * cpr, 256)));
+#define MG_DELTA(CPR_)                                                                                              \
+  hipLaunchKernelGGL((attn_delta_rows_kernel<T, CPR_>), grid, dim3(256), 0, stream, d_o, o, delta, rows, a.S, a.H, \
+                     a.o_bshd)
     switch (cpr) {
-      case 1: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 1>), grid, dim3(256), 0, stream, d_o, o, delta, rows, a.S, a.H, a.o_bshd); break;
-      case 2: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 2>), grid, dim3(256), 0, stream, d_o, o, delta, rows, a.S, a.H, a.o_bshd); break;
-      case 4: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 4>), grid, dim3(256), 0, stream, d_o, o, delta, rows, a.S, a.H, a.o_bshd); break;
-      case 8: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 8>), grid, dim3(256), 0, stream, d_o, o, delta, rows, a.S, a.H, a.o_bshd); break;
-      default: hipLaunchKernelGGL((attn_delta_rows_kernel<T, 16>), grid, dim3(256), 0, stream, d_o, o, delta, rows, a.S, a.H, a.o_bshd); break;
+      case 1: MG_DELTA(1); break;
+      case 2: MG_DELTA(2); break;
+      case 4: MG_DELTA(4); break;
+      case 8: MG_DELTA(8); break;
+      default: MG_DELTA(16); break;
     }
+#undef MG_DELTA
   } else {
     hipLaunchKernelGGL((attn_delta_kernel<T>), dim3(static_cast<unsigned>(ceil_div(rows, 4))), dim3(256), 0, stream, d_o,
                        o, delta, rows, D, a.S, a.H, a.o_bshd);

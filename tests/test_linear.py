@@ -263,6 +263,25 @@ def test_batched_projections_share_an_operand(device, dtype, rtol, M, d):
     assert_close(dw.to_numpy((3, d, d)), want_dw, rtol, rtol * np.abs(want_dw).max(), "dw")
 
 
+@pytest.mark.parametrize("variant", ["0", "322", "642"])
+def test_batched_projections_tile_staging_variants(device, monkeypatch, variant):
+    # The same two batched products (batch stride 0 on the shared operand; the second split
+    # along K with the batch in the grid's z) through each 16-bit tile-staging variant.
+    monkeypatch.setenv("MOGRAD_HIP_GEMM16_PIPE", variant)
+    lib, st, dtype, M, d = device.lib, device.stream, BF16, 2048, 128
+    x = round_to_dtype(normal(57, 0, (M, d)), dtype)
+    w = round_to_dtype(normal(57, 1, (3, d, d), std=0.1), dtype)
+    dy = round_to_dtype(normal(57, 2, (3, M, d), std=0.5), dtype)
+    bx, bw, bdy = (AnyBuffer.from_numpy(device, a, dtype) for a in (x, w, dy))
+    y, dw = AnyBuffer.create(dtype, device, 3 * M * d), AnyBuffer.create(dtype, device, 3 * d * d)
+    lib.mg_matmul_bt(bx.data_ptr(), bw.data_ptr(), y.data_ptr(), 3, M, d, d, d, 1, d, 1, 0, d * d, dtype, st)
+    lib.mg_matmul(bdy.data_ptr(), bx.data_ptr(), dw.data_ptr(), 3, d, d, M, 1, d, d, 1, M * d, 0, dtype, st)
+    want_y = np.einsum("tk,bnk->btn", x.astype(np.float64), w.astype(np.float64))
+    want_dw = np.einsum("bto,ti->boi", dy.astype(np.float64), x.astype(np.float64))
+    assert_close(y.to_numpy((3, M, d)), want_y, 1.6e-2, 1.6e-2 * np.abs(want_y).max(), "y")
+    assert_close(dw.to_numpy((3, d, d)), want_dw, 1.6e-2, 1.6e-2 * np.abs(want_dw).max(), "dw")
+
+
 # ---- fused epilogues: each must give exactly what the separate calls give -----------------
 
 FUSED_SHAPES = [(256, 384, 512), (200, 136, 264), (130, 65, 384), (64, 10, 256), (33, 7, 5), (4096, 128, 128),
