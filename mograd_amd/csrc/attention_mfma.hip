@@ -96,141 +96,117 @@ __device__ __forceinline__ floatx16 splat16(float v) {
 }
 
 constexpr int kAttnThreads = 256;
+typedef short short4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float fexp2(float v) { return __builtin_amdgcn_exp2f(v); }
 
 // ---- LDS tiles -------------------------------------------------------------------------
-// Row-major tile: R rows x DP columns of T, row stride DP + 8 elements (the 16-byte pad
-// spreads the 128-bit fragment reads of 8 consecutive rows over all banks).
+// A staged tile is R rows x DP columns of T, row-major, rows of DP * 2 bytes without padding.
+// The 16-byte chunk c of row r is stored at chunk position c ^ swz(r) (low three bits), with
+// swz(r) = 2 * (r % 4) + (r / 4) % 2.  Both kinds of fragment read are then free of bank
+// conflicts: eight consecutive rows have eight different swz values (the 128-bit row reads of
+// eight lanes cover all banks), and four consecutive rows starting at a multiple of four move
+// a 32-byte unit to four different units (the transposing 64-bit reads of 16 lanes, four rows
+// x 32 bytes, cover all banks too).  One image serves the products that contract over the
+// tile's columns and those that contract over its rows.
 template <int DP>
-constexpr int row_stride() { return DP + 8; }
-// Transposed tile: DP rows (one per d) x R columns, stored as dwords holding two
-// consecutive columns; row stride R/2 + 2 dwords.
-template <int R>
-constexpr int tr_stride_dw() { return R / 2 + 2; }
+constexpr int tile_row_bytes() { return DP * 2; }
+__device__ __forceinline__ int tile_swz(int r) { return 2 * (r % 4) + (r / 4) % 2; }
+template <int DP>
+__device__ __forceinline__ int tile_chunk_at(int r, int c) { return r * tile_row_bytes<DP>() + ((c ^ tile_swz(r)) * 16); }
 
-// Global -> registers -> LDS staging of R rows x DP columns.  A thread owns "pair chunks":
-// 8 columns of two consecutive rows.  Fetching into registers and committing to LDS are
-// separate so that the next tile's loads can be in flight while the current tile is used.
-// From the same registers a tile can be committed row-major, transposed, or both.
+// Global -> registers -> LDS staging of R rows x DP columns.  A thread owns 16-byte chunks
+// (8 columns of one row); consecutive lanes take consecutive chunks of a row, so a 128-bit
+// LDS write cycle of eight lanes covers eight different chunk positions.  Fetching into
+// registers and committing to LDS are separate so that the next tile's loads can be in
+// flight while the current tile is used.
 template <typename T, int R, int DP>
 struct TileStager {
-  static constexpr int CH = DP / 8;
-  static constexpr int PAIRS = R / 2;
-  static constexpr int TASKS = PAIRS * CH;
-  static constexpr int PER = (TASKS + kAttnThreads - 1) / kAttnThreads;
-  uint4 lo[PER], hi[PER];
-  // Pair chunk `idx` -> (row pair, 8-column chunk).  Two neighbouring lanes take the two
-  // chunks of one row pair and the next two lanes the next pair, so that the eight lanes of
-  // one 128-bit LDS write cycle cover four row pairs x two chunks: with the tile's row stride
-  // those are eight different groups of four banks (lanes on consecutive row pairs alone
-  // would hit each group twice).
-  static_assert(CH % 2 == 0, "chunks are handed out two at a time");
-  static __device__ __forceinline__ int pair_of(int idx) { return (idx / 2) % PAIRS; }
-  static __device__ __forceinline__ int chunk_of(int idx) { return idx % 2 + 2 * (idx / (2 * PAIRS)); }
-  // Walk over consecutive R-row tiles: where this thread reads in the next tile.
-  static_assert(kAttnThreads % PAIRS == 0, "chunk i of a thread must be its chunk 0 shifted by whole columns");
-  static constexpr int CHUNK_STEP = kAttnThreads / PAIRS * 8;  // columns between a thread's consecutive chunks
-  const T* base_;
+  static constexpr int CH = DP / 8;                     // chunks per row
+  static constexpr int TASKS = R * CH;
+  static constexpr int PER = TASKS / kAttnThreads;      // chunks per thread
+  static constexpr int ROW_STEP = kAttnThreads / CH;    // rows between a thread's consecutive chunks
+  static_assert(TASKS % kAttnThreads == 0 && kAttnThreads % CH == 0, "whole chunks per thread, one column per thread");
+  uint4 v[PER];
   const T* src_;
   int64_t ld_;
   int next_;
+  static __device__ __forceinline__ int row_of(int i) { return threadIdx.x / CH + i * ROW_STEP; }
+  static __device__ __forceinline__ int chunk() { return threadIdx.x % CH; }
 
   // Starts a walk at row r0 of the matrix whose row r begins at base + r * ld (elements).
   __device__ __forceinline__ void begin(const T* __restrict__ base, int64_t ld, int r0) {
-    base_ = base;
     ld_ = ld;
     next_ = r0;
-    src_ = base + (r0 + 2 * pair_of(threadIdx.x)) * ld + chunk_of(threadIdx.x) * 8;
+    src_ = base + (r0 + row_of(0)) * ld + chunk() * 8;
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      lo[i] = make_uint4(0, 0, 0, 0);
-      hi[i] = make_uint4(0, 0, 0, 0);
-    }
+    for (int i = 0; i < PER; ++i) v[i] = make_uint4(0, 0, 0, 0);
   }
-  // Fetches the next tile of the walk.  A tile that lies inside the matrix takes the short
-  // path: two unconditional loads per chunk from pointers that advance by a constant (chunks
-  // of padding columns never load and keep their zeros); only the ragged last tile pays for
-  // per-row bounds checks.
+  // Fetches the next tile of the walk: rows >= r_end and columns >= D read as zero.  A tile
+  // that lies inside the matrix takes the short path, unconditional loads from a pointer that
+  // advances by a constant (chunks of padding columns never load and keep their zeros); only
+  // the ragged last tile pays for per-row bounds checks.
   __device__ __forceinline__ void fetch_next(int r_end, int D) {
-    if (next_ + R <= r_end) {
+    if (chunk() * 8 < D) {
+      if (next_ + R <= r_end) {
 #pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int idx = threadIdx.x + i * kAttnThreads;
-        if (idx < TASKS && chunk_of(idx) * 8 < D) {
-          lo[i] = *reinterpret_cast<const uint4*>(src_ + i * CHUNK_STEP);
-          hi[i] = *reinterpret_cast<const uint4*>(src_ + ld_ + i * CHUNK_STEP);
-        }
+        for (int i = 0; i < PER; ++i) v[i] = *reinterpret_cast<const uint4*>(src_ + i * ROW_STEP * ld_);
+      } else {
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+          v[i] = next_ + row_of(i) < r_end ? *reinterpret_cast<const uint4*>(src_ + i * ROW_STEP * ld_)
+                                           : make_uint4(0, 0, 0, 0);
       }
-    } else {
-      fetch(base_, ld_, next_, r_end, D);
     }
     src_ += R * ld_;
     next_ += R;
   }
-
-  // Rows [r0, r0 + R) of a matrix whose row r starts at base + r * ld (elements); D valid
-  // columns; rows >= r_end and columns >= D read as zero.
-  __device__ __forceinline__ void fetch(const T* __restrict__ base, int64_t ld, int r0, int r_end, int D) {
+  __device__ __forceinline__ void commit(char* __restrict__ lds) const {
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int idx = threadIdx.x + i * kAttnThreads;
-      const int p = pair_of(idx), c = chunk_of(idx);
-      const int ra = r0 + 2 * p;
-      lo[i] = make_uint4(0, 0, 0, 0);
-      hi[i] = make_uint4(0, 0, 0, 0);
-      if (idx < TASKS && c * 8 < D) {
-        if (ra < r_end) lo[i] = *reinterpret_cast<const uint4*>(base + ra * ld + c * 8);
-        if (ra + 1 < r_end) hi[i] = *reinterpret_cast<const uint4*>(base + (ra + 1) * ld + c * 8);
-      }
-    }
-  }
-  __device__ __forceinline__ void commit_rows(uint16_t* __restrict__ lds) const {
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int idx = threadIdx.x + i * kAttnThreads;
-      const int p = pair_of(idx), c = chunk_of(idx);
-      if (idx < TASKS) {
-        *reinterpret_cast<uint4*>(lds + (2 * p) * row_stride<DP>() + c * 8) = lo[i];
-        *reinterpret_cast<uint4*>(lds + (2 * p + 1) * row_stride<DP>() + c * 8) = hi[i];
-      }
-    }
-  }
-  // dword (d, p) of the transposed tile holds columns 2p and 2p+1 of row d.
-  __device__ __forceinline__ void commit_transposed(uint32_t* __restrict__ lds) const {
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int idx = threadIdx.x + i * kAttnThreads;
-      const int p = pair_of(idx), c = chunk_of(idx);
-      if (idx < TASKS) {
-        const uint32_t a[4] = {lo[i].x, lo[i].y, lo[i].z, lo[i].w};
-        const uint32_t b[4] = {hi[i].x, hi[i].y, hi[i].z, hi[i].w};
-        uint32_t* dst = lds + (c * 8) * tr_stride_dw<R>() + p;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          dst[(2 * e) * tr_stride_dw<R>()] = __builtin_amdgcn_perm(b[e], a[e], 0x05040100);
-          dst[(2 * e + 1) * tr_stride_dw<R>()] = __builtin_amdgcn_perm(b[e], a[e], 0x07060302);
-        }
-      }
-    }
+    for (int i = 0; i < PER; ++i) *reinterpret_cast<uint4*>(lds + tile_chunk_at<DP>(row_of(i), chunk())) = v[i];
   }
 };
 
-// A operand from a row-major tile: rows rt*32 + lane%32, columns ks*16 + (lane/32)*8 .. +7.
+// Where a lane reads its fragments inside a staged tile, as byte offsets that depend on the
+// lane only; everything else (which 32-row block, which 16 rows, which tile copy) is a
+// compile-time or wave-uniform addend, so the fragment reads of a whole step share these few
+// address registers.  That works because a row's swizzle depends only on r % 8, and the rows
+// a lane reads differ from its first one by multiples of 8.
 template <int DP>
-__device__ __forceinline__ uint4 frag_rows(const uint16_t* __restrict__ lds, int rt, int ks, int lane) {
-  return *reinterpret_cast<const uint4*>(lds + (rt * 32 + lane % 32) * row_stride<DP>() + ks * 16 + (lane / 32) * 8);
+struct TileLane {
+  int rows[DP / 16];  // per 16-column slice ks: row lane%32, columns ks*16 + (lane/32)*8 .. +7
+  int tr[DP / 32];    // per 32-column block dt: row 4*(lane/32) + (lane%16)/4, columns dt*32 + ((lane/16)%2)*16 + 4*(lane%4) .. +3
+  __device__ __forceinline__ explicit TileLane(int lane) {
+#pragma unroll
+    for (int ks = 0; ks < DP / 16; ++ks) rows[ks] = tile_chunk_at<DP>(lane % 32, ks * 2 + lane / 32);
+    const int col = ((lane / 16) % 2) * 16 + 4 * (lane % 4);
+#pragma unroll
+    for (int dt = 0; dt < DP / 32; ++dt)
+      tr[dt] = tile_chunk_at<DP>(4 * (lane / 32) + (lane % 16) / 4, (dt * 32 + col) / 8) + (col % 8) * 2;
+  }
+};
+
+// A operand for a product that contracts over the tile's columns: rows rt*32 + lane%32,
+// columns ks*16 + (lane/32)*8 .. +7.
+template <int DP>
+__device__ __forceinline__ uint4 frag_rows(const char* __restrict__ lds, const TileLane<DP>& at, int rt, int ks) {
+  return *reinterpret_cast<const uint4*>(lds + at.rows[ks] + rt * 32 * tile_row_bytes<DP>());
 }
 
-// A operand from a transposed tile for the product that contracts over the tile's
-// columns.  k-slot e of lane half h stands for column t*16 + (e/4)*8 + 4h + e%4: the
-// same assignment the score tile's registers have (see frag_from_acc).
-template <int R>
-__device__ __forceinline__ uint4 frag_transposed(const uint32_t* __restrict__ lds, int dt, int t, int lane) {
-  const uint32_t* p = lds + (dt * 32 + lane % 32) * tr_stride_dw<R>() + t * 8 + (lane / 32) * 2;
-  const uint2 lo = *reinterpret_cast<const uint2*>(p);
-  const uint2 hi = *reinterpret_cast<const uint2*>(p + 4);
-  return make_uint4(lo.x, lo.y, hi.x, hi.y);
+// A operand for a product that contracts over the tile's rows: MFMA row = tile column
+// dt*32 + lane%32; k-slot e of lane half h stands for tile row t*16 + (e/4)*8 + 4h + e%4, the
+// same assignment the score tile's registers have (see frag_from_acc).  Read with
+// ds_read_b64_tr_b16: within 16 lanes, lane i supplies the address of four consecutive
+// columns 4*(i%4).. of row i/4 of a 4 x 16 block and receives the four rows of column i.
+template <int DP>
+__device__ __forceinline__ uint4 frag_transposed(const char* __restrict__ lds, const TileLane<DP>& at, int dt, int t) {
+  using lds_i16x4 = __attribute__((address_space(3))) short4_t;
+  const char* p = lds + at.tr[dt] + t * 16 * tile_row_bytes<DP>();
+  const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_i16x4*>(reinterpret_cast<uintptr_t>(p)));
+  const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      reinterpret_cast<lds_i16x4*>(reinterpret_cast<uintptr_t>(p + 8 * tile_row_bytes<DP>())));
+  const uint2 l = __builtin_bit_cast(uint2, lo), h = __builtin_bit_cast(uint2, hi);
+  return make_uint4(l.x, l.y, h.x, h.y);
 }
 
 // B operand from a 32x32 accumulator tile: registers 8*half .. 8*half+7, i.e. rows
@@ -293,8 +269,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
   constexpr int BM = 128, BN = 64, KS = DP / 16, DT = DP / 32;
   // Two copies of each staged tile: step i computes from copy i % 2 while the tile of step
   // i + 1 is written into the other, so one barrier per step suffices.
-  __shared__ __attribute__((aligned(16))) uint16_t k_rows_s[2][BN * row_stride<DP>()];
-  __shared__ __attribute__((aligned(16))) uint32_t v_tr_s[2][DP * tr_stride_dw<BN>()];
+  __shared__ __attribute__((aligned(16))) char k_rows_s[2][BN * tile_row_bytes<DP>()];
+  __shared__ __attribute__((aligned(16))) char v_rows_s[2][BN * tile_row_bytes<DP>()];
 
   const int nqb = (a.S + BM - 1) / BM;
   // Consecutive workgroups go to different XCDs, so the (batch, head) index varies fastest:
@@ -308,6 +284,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int half = lane / 32;
+  const TileLane<DP> at(lane);
   const int m_wave = qb * BM + wave * 32;
   const int m = m_wave + lane % 32;
   const int64_t ld = a.ld;  // token stride of Q, K, V
@@ -334,8 +311,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
   vs_stage.begin(vbase, ld, 0);
   ks_stage.fetch_next(a.S, a.D);
   vs_stage.fetch_next(a.S, a.D);
-  ks_stage.commit_rows(k_rows_s[0]);
-  vs_stage.commit_transposed(v_tr_s[0]);
+  ks_stage.commit(k_rows_s[0]);
+  vs_stage.commit(v_rows_s[0]);
   if (BN < n_end) {
     ks_stage.fetch_next(a.S, a.D);
     vs_stage.fetch_next(a.S, a.D);
@@ -345,15 +322,15 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
     // Copy `cur` is complete and every wave has finished reading the other copy.
     __syncthreads();
     if (n0 + BN < n_end) {
-      ks_stage.commit_rows(k_rows_s[cur ^ 1]);
-      vs_stage.commit_transposed(v_tr_s[cur ^ 1]);
+      ks_stage.commit(k_rows_s[cur ^ 1]);
+      vs_stage.commit(v_rows_s[cur ^ 1]);
       if (n0 + 2 * BN < n_end) {
         ks_stage.fetch_next(a.S, a.D);
         vs_stage.fetch_next(a.S, a.D);
       }
     }
-    const uint16_t* k_rows = k_rows_s[cur];
-    const uint32_t* v_tr = v_tr_s[cur];
+    const char* k_rows = k_rows_s[cur];
+    const char* v_rows = v_rows_s[cur];
     if (CAUSAL && n0 > m_wave + 31) continue;  // every key of the block is in this wave's future
 
     floatx16 s[2];
@@ -361,7 +338,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
     for (int nt = 0; nt < 2; ++nt) {
       s[nt] = zero16();
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) s[nt] = Mma<T>::run(frag_rows<DP>(k_rows, nt, ks, lane), qf[ks], s[nt]);
+      for (int ks = 0; ks < KS; ++ks) s[nt] = Mma<T>::run(frag_rows<DP>(k_rows, at, nt, ks), qf[ks], s[nt]);
     }
     // A block needs per-element masking only at the end of the sequence and, for causal
     // attention, where it crosses the diagonal of this wave's queries.
@@ -429,7 +406,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
     for (int t = 0; t < BN / 16; ++t) {
       const uint4 pf = frag_from_acc<T>(s[t / 2], t % 2);
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) acc_o[dt] = Mma<T>::run(frag_transposed<BN>(v_tr, dt, t, lane), pf, acc_o[dt]);
+      for (int dt = 0; dt < DT; ++dt) acc_o[dt] = Mma<T>::run(frag_transposed<DP>(v_rows, at, dt, t), pf, acc_o[dt]);
     }
   }
 
@@ -454,7 +431,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
 // Bytes of LDS the dQ walk stages its tiles in.
 template <int DP>
 constexpr int dq_lds_bytes() {
-  return (DP <= 64 ? 2 : 1) * (2 * 64 * row_stride<DP>() * 2 + DP * tr_stride_dw<64>() * 4);
+  return (DP <= 64 ? 2 : 1) * 2 * 64 * tile_row_bytes<DP>();  // copies of a K tile and a V tile
 }
 
 // The work of workgroup `block` of a dQ launch; `smem` holds dq_lds_bytes<DP>() bytes.
@@ -465,14 +442,15 @@ __device__ __forceinline__ void attn_dq_block(const int block, char* smem, const
                                               const float* __restrict__ lse, const float* __restrict__ delta,
                                               T* __restrict__ dq, const AttnDims& a, float scale) {
   constexpr int BM = 128 * MQ, BN = 64, KS = DP / 16, DT = DP / 32;
-  // Two copies of each staged tile (one barrier per step) while two workgroups still fit in
-  // a CU's LDS; for head dims above 64 one copy and two barriers per step.
+  // Two copies of each staged tile (step i computes from copy i % 2 while the tile of step
+  // i + 1 is written into the other: one barrier per step) for head dims up to 64.  Above,
+  // one copy and two barriers per step: the two-copy schedule spills more there (68-108 bytes
+  // per lane against 44-80) and measured 20-30 % slower.
   constexpr int NBUF = DP <= 64 ? 2 : 1;
-  constexpr int ROWS = BN * row_stride<DP>(), TR = DP * tr_stride_dw<BN>();
-  auto k_rows_s = reinterpret_cast<uint16_t(*)[ROWS]>(smem);
-  auto v_rows_s = reinterpret_cast<uint16_t(*)[ROWS]>(smem + NBUF * ROWS * 2);
-  auto k_tr_s = reinterpret_cast<uint32_t(*)[TR]>(smem + 2 * NBUF * ROWS * 2);
-  static_assert(dq_lds_bytes<DP>() == 2 * NBUF * ROWS * 2 + NBUF * TR * 4, "LDS size");
+  constexpr int ROWS = BN * tile_row_bytes<DP>();
+  auto k_rows_s = reinterpret_cast<char(*)[ROWS]>(smem);
+  auto v_rows_s = reinterpret_cast<char(*)[ROWS]>(smem + NBUF * ROWS);
+  static_assert(dq_lds_bytes<DP>() == 2 * NBUF * ROWS, "LDS size");
 
   const int nqb = (a.S + BM - 1) / BM;
   // (batch, head) varies fastest across consecutive workgroups, heaviest query blocks first.
@@ -483,6 +461,7 @@ __device__ __forceinline__ void attn_dq_block(const int block, char* smem, const
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int half = lane / 32;
+  const TileLane<DP> at(lane);
   const int m_wave = qb * BM + wave * (32 * MQ);
   const int64_t ld = a.ld;
   const T* kbase = k + qkv_at(a, b, 0, h);
@@ -528,9 +507,8 @@ __device__ __forceinline__ void attn_dq_block(const int block, char* smem, const
   ks_stage.fetch_next(a.S, a.D);
   vs_stage.fetch_next(a.S, a.D);
   if constexpr (NBUF == 2) {
-    ks_stage.commit_rows(k_rows_s[0]);
-    ks_stage.commit_transposed(k_tr_s[0]);
-    vs_stage.commit_rows(v_rows_s[0]);
+    ks_stage.commit(k_rows_s[0]);
+    vs_stage.commit(v_rows_s[0]);
     if (BN < n_end) {
       ks_stage.fetch_next(a.S, a.D);
       vs_stage.fetch_next(a.S, a.D);
@@ -542,9 +520,8 @@ __device__ __forceinline__ void attn_dq_block(const int block, char* smem, const
       // Copy `cur` is complete and every wave has finished reading the other copy.
       __syncthreads();
       if (n0 + BN < n_end) {
-        ks_stage.commit_rows(k_rows_s[cur ^ 1]);
-        ks_stage.commit_transposed(k_tr_s[cur ^ 1]);
-        vs_stage.commit_rows(v_rows_s[cur ^ 1]);
+        ks_stage.commit(k_rows_s[cur ^ 1]);
+        vs_stage.commit(v_rows_s[cur ^ 1]);
         if (n0 + 2 * BN < n_end) {
           ks_stage.fetch_next(a.S, a.D);
           vs_stage.fetch_next(a.S, a.D);
@@ -552,18 +529,16 @@ __device__ __forceinline__ void attn_dq_block(const int block, char* smem, const
       }
     } else {
       __syncthreads();  // every wave has finished reading the previous tile
-      ks_stage.commit_rows(k_rows_s[0]);
-      ks_stage.commit_transposed(k_tr_s[0]);
-      vs_stage.commit_rows(v_rows_s[0]);
+      ks_stage.commit(k_rows_s[0]);
+      vs_stage.commit(v_rows_s[0]);
       __syncthreads();
       if (n0 + BN < n_end) {
         ks_stage.fetch_next(a.S, a.D);
         vs_stage.fetch_next(a.S, a.D);
       }
     }
-    const uint16_t* k_rows = k_rows_s[cur];
-    const uint16_t* v_rows = v_rows_s[cur];
-    const uint32_t* k_tr = k_tr_s[cur];
+    const char* k_rows = k_rows_s[cur];
+    const char* v_rows = v_rows_s[cur];
     if (CAUSAL && n0 > m_wave + 32 * MQ - 1) continue;  // every key of the block is in this wave's future
 
     // One 32-key tile at a time: S^T and dP^T for all MQ query tiles, dS^T in place, then
@@ -578,8 +553,8 @@ __device__ __forceinline__ void attn_dq_block(const int block, char* smem, const
       }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const uint4 ka = frag_rows<DP>(k_rows, nt, ks, lane);
-        const uint4 va = frag_rows<DP>(v_rows, nt, ks, lane);
+        const uint4 ka = frag_rows<DP>(k_rows, at, nt, ks);
+        const uint4 va = frag_rows<DP>(v_rows, at, nt, ks);
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq) {
           s[mq] = Mma<T>::run(ka, qf[mq][ks], s[mq]);
@@ -615,7 +590,7 @@ __device__ __forceinline__ void attn_dq_block(const int block, char* smem, const
         for (int mq = 0; mq < MQ; ++mq) dsf[mq] = frag_from_acc<T>(s[mq], hf);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-          const uint4 kt = frag_transposed<BN>(k_tr, dt, t, lane);
+          const uint4 kt = frag_transposed<DP>(k_rows, at, dt, t);
 #pragma unroll
           for (int mq = 0; mq < MQ; ++mq) acc[mq][dt] = Mma<T>::run(kt, dsf[mq], acc[mq][dt]);
         }
@@ -643,7 +618,7 @@ __device__ __forceinline__ void attn_dq_block(const int block, char* smem, const
 // Bytes of LDS the dK/dV walk stages its tiles and row statistics in.
 template <int DP>
 constexpr int dkdv_lds_bytes() {
-  return 2 * (2 * 64 * row_stride<DP>() * 2 + 2 * DP * tr_stride_dw<64>() * 4 + 2 * 64 * 4);
+  return 2 * (2 * 64 * tile_row_bytes<DP>() + 2 * 64 * 4);  // two copies of a Q tile, a dO tile, lse and delta
 }
 
 // The work of workgroup `block` of a dK/dV launch; `smem` holds dkdv_lds_bytes<DP>() bytes.
@@ -659,14 +634,12 @@ __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, con
   constexpr int MT = BQ / 32, KS = DP / 16, DT = DP / 32;
   // Two copies of every staged tile: step i computes from copy i % 2 while the tile of step
   // i + 1 is written into the other, so one barrier per step suffices.
-  constexpr int ROWS = BQ * row_stride<DP>(), TR = DP * tr_stride_dw<BQ>();
-  auto q_rows_s = reinterpret_cast<uint16_t(*)[ROWS]>(smem);
-  auto do_rows_s = reinterpret_cast<uint16_t(*)[ROWS]>(smem + 2 * ROWS * 2);
-  auto q_tr_s = reinterpret_cast<uint32_t(*)[TR]>(smem + 4 * ROWS * 2);
-  auto do_tr_s = reinterpret_cast<uint32_t(*)[TR]>(smem + 4 * ROWS * 2 + 2 * TR * 4);
-  auto lse_ss = reinterpret_cast<float(*)[BQ]>(smem + 4 * ROWS * 2 + 4 * TR * 4);
-  auto delta_ss = reinterpret_cast<float(*)[BQ]>(smem + 4 * ROWS * 2 + 4 * TR * 4 + 2 * BQ * 4);
-  static_assert(dkdv_lds_bytes<DP>() == 4 * ROWS * 2 + 4 * TR * 4 + 4 * BQ * 4, "LDS size");
+  constexpr int ROWS = BQ * tile_row_bytes<DP>();
+  auto q_rows_s = reinterpret_cast<char(*)[ROWS]>(smem);
+  auto do_rows_s = reinterpret_cast<char(*)[ROWS]>(smem + 2 * ROWS);
+  auto lse_ss = reinterpret_cast<float(*)[BQ]>(smem + 4 * ROWS);
+  auto delta_ss = reinterpret_cast<float(*)[BQ]>(smem + 4 * ROWS + 2 * BQ * 4);
+  static_assert(dkdv_lds_bytes<DP>() == 4 * ROWS + 4 * BQ * 4, "LDS size");
 
   // (batch, head) varies fastest across consecutive workgroups.  Causal: earlier key blocks
   // are seen by more queries; all of them launch first.
@@ -677,6 +650,7 @@ __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, con
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int half = lane / 32;
+  const TileLane<DP> at(lane);
   const int n_wave = kb * BNK + wave * 32;
   const int n = n_wave + lane % 32;
   const int64_t ld = a.ld;
@@ -724,10 +698,8 @@ __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, con
   };
   // Registers -> LDS copy `buf`.
   auto commit_step = [&](int buf) {
-    q_stage.commit_rows(q_rows_s[buf]);
-    q_stage.commit_transposed(q_tr_s[buf]);
-    do_stage.commit_rows(do_rows_s[buf]);
-    do_stage.commit_transposed(do_tr_s[buf]);
+    q_stage.commit(q_rows_s[buf]);
+    do_stage.commit(do_rows_s[buf]);
     if (threadIdx.x < BQ) {
       // Stored negated: they initialise the accumulators of the S and dP products.  Rows
       // past the end carry -lse = -inf (their probabilities vanish) and delta = 0.
@@ -746,10 +718,8 @@ __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, con
       commit_step(cur ^ 1);
       if (m0 + 2 * BQ < a.S) fetch_step(m0 + 2 * BQ);
     }
-    const uint16_t* q_rows = q_rows_s[cur];
-    const uint16_t* do_rows = do_rows_s[cur];
-    const uint32_t* q_tr = q_tr_s[cur];
-    const uint32_t* do_tr = do_tr_s[cur];
+    const char* q_rows = q_rows_s[cur];
+    const char* do_rows = do_rows_s[cur];
     const float* lse_s = lse_ss[cur];
     const float* delta_s = delta_ss[cur];
     if (CAUSAL && m0 + BQ - 1 < n_wave) continue;  // all of this step's queries precede the wave's keys
@@ -775,8 +745,8 @@ __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, con
       }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        s = Mma<T>::run(frag_rows<DP>(q_rows, mt, ks, lane), kf[ks], s);
-        dp = Mma<T>::run(frag_rows<DP>(do_rows, mt, ks, lane), vf[ks], dp);
+        s = Mma<T>::run(frag_rows<DP>(q_rows, at, mt, ks), kf[ks], s);
+        dp = Mma<T>::run(frag_rows<DP>(do_rows, at, mt, ks), vf[ks], dp);
       }
       // The transposed fragments of the second phase are fetched now, so that their LDS
       // latency runs under the exponentials instead of in front of each MFMA.
@@ -785,8 +755,8 @@ __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, con
       for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-          tdo[hf][dt] = frag_transposed<BQ>(do_tr, dt, mt * 2 + hf, lane);
-          tq[hf][dt] = frag_transposed<BQ>(q_tr, dt, mt * 2 + hf, lane);
+          tdo[hf][dt] = frag_transposed<DP>(do_rows, at, dt, mt * 2 + hf);
+          tq[hf][dt] = frag_transposed<DP>(q_rows, at, dt, mt * 2 + hf);
         }
       __builtin_amdgcn_sched_barrier(0);
       if (plain) {
