@@ -103,12 +103,16 @@ __device__ __forceinline__ float fexp2(float v) { return __builtin_amdgcn_exp2f(
 // ---- LDS tiles -------------------------------------------------------------------------
 // A staged tile is R rows x DP columns of T, row-major, rows of DP * 2 bytes without padding.
 // The 16-byte chunk c of row r is stored at chunk position c ^ swz(r) (low three bits), with
-// swz(r) = 2 * (r % 4) + (r / 4) % 2.  Both kinds of fragment read are then free of bank
-// conflicts: eight consecutive rows have eight different swz values (the 128-bit row reads of
-// eight lanes cover all banks), and four consecutive rows starting at a multiple of four move
-// a 32-byte unit to four different units (the transposing 64-bit reads of 16 lanes, four rows
-// x 32 bytes, cover all banks too).  One image serves the products that contract over the
-// tile's columns and those that contract over its rows.
+// swz(r) = 2 * (r % 4) + (r / 4) % 2.  The transposing 64-bit reads (16 lanes: four rows x 32
+// bytes) and the staging stores are free of bank conflicts with it; the 128-bit row reads
+// are served two rows per bank group (LDS has 64 banks and serves 16 lanes of a 128-bit
+// read per clock; timed with four waves reading back to back: 32 clocks per read against
+// 19 for consecutive addresses).  A swizzle over r % 16 that removes that too, 4 * (r/2 % 2)
+// + (r/4 % 4), was measured in these kernels: 25 % fewer LDS-busy cycles, but the two
+// transposing reads of a fragment then need separate address registers and adds, and the
+// forward, which is bound by its VALU work, ran 3-5 % slower (backward within 1 %), so it
+// was not kept.  One image serves the products that contract over the tile's columns and
+// those that contract over its rows.
 template <int DP>
 constexpr int tile_row_bytes() { return DP * 2; }
 __device__ __forceinline__ int tile_swz(int r) { return 2 * (r % 4) + (r / 4) % 2; }

@@ -599,18 +599,18 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
 // and not by the matrix cores.  Operands as above, all extents and strides multiples of 8
 // elements, K (and every K split) a multiple of 64.
 //
-// LDS image of one operand's step (16 KB), chosen per 16-byte chunk by which source chunk
-// each lane names:
-//   k-contiguous: [128 rows][8 chunks], chunk c of row r at position c ^ (r % 8): the 32
-//     rows a fragment read touches spread over all banks;
-//   otherwise: [64 k][16 chunks of 8 rows], chunk c of k-row kk at position
+// LDS image of one operand's step, chosen per 16-byte chunk by which source chunk each lane
+// names (64 banks of four bytes; a 128-bit read is served 16 lanes per clock):
+//   k-contiguous, 64 k per step: [128 rows][8 chunks], chunk c of row r at position
+//     c ^ (r/2 % 8), with 32 k per step [128 rows][4 chunks] and c ^ (r/4 % 4): the sixteen
+//     consecutive rows of a fragment read then hit sixteen different 16-byte bank groups
+//     (timed on the device: 18.5-18.7 clocks per read with four waves reading, as for
+//     consecutive addresses; 32 with c ^ (r % 8));
+//   otherwise: [k][16 chunks of 8 rows], chunk c of k-row kk at position
 //     c ^ (2 * (kk % 4)), read with `ds_read_b64_tr_b16` (within 16 lanes, lane i supplies
 //     the four elements 4*i .. 4*i+3 of a 4 x 16 block and receives column i), which turns
 //     four k-rows of 16 consecutive rows into each lane's four consecutive k.
 // ------------------------------------------------------------------------------------
-
-// (Shown for 64 k per step; with 32 a k-contiguous row is 4 chunks and chunk c of row r
-// sits at c ^ ((r / 2) % 4), the other image simply has 32 k-rows.)
 
 typedef short gemm_i16x4 __attribute__((ext_vector_type(4)));
 
@@ -625,7 +625,7 @@ __device__ __forceinline__ void gemm16_pipe_sources(int64_t ld, int o0, int O, i
   for (int i = 0; i < BK / 16; ++i) {
     const int slot = (i * 4 + wave) * kWave + lane;  // 16-byte position in the LDS image
     if constexpr (KC) {
-      const int r = slot / CPR, c = (slot % CPR) ^ ((r / (8 / CPR)) % CPR);
+      const int r = slot / CPR, c = (slot % CPR) ^ ((r / (16 / CPR)) % CPR);
       src[i] = static_cast<int64_t>(min(o0 + r, O - 1)) * ld + c * 8;  // rows past the edge are never stored
     } else {
       const int kk = slot / 16, c = (slot % 16) ^ (2 * (kk % 4));
@@ -659,7 +659,7 @@ __device__ __forceinline__ uint4 gemm16_pipe_frag(const char* __restrict__ lds_s
     constexpr int CPR = BK / 8;
     const int r = o_base + lane % 32;
     const int g = ks * 2 + lane / 32;
-    return *reinterpret_cast<const uint4*>(lds_step + r * (BK * 2) + ((g ^ ((r / (8 / CPR)) % CPR)) * 16));
+    return *reinterpret_cast<const uint4*>(lds_step + r * (BK * 2) + ((g ^ ((r / (16 / CPR)) % CPR)) * 16));
   } else {
     const int o = o_base + ((lane / 16) % 2) * 16 + 4 * (lane % 4);  // first of the 4 rows this lane supplies
     const int kq = (lane % 16) / 4;                                 // its k-row within a group of 4
