@@ -89,13 +89,16 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
   // products of two k-contiguous operands stay with the register-staged kernel (4-8 %
   // faster there), as does every shape the copy cannot take.  The pair is k per step and
   // copies of the tiles: (32, 2) runs four workgroups per CU, (64, 2) two.
-  // MOGRAD_HIP_GEMM16_PIPE = 0 | 322 | 642 overrides the choice.
+  // MOGRAD_HIP_GEMM16_PIPE = 0 | 322 | 642 | 2322 | 2642 overrides the choice (2xxx: 256 x 128 tiles).
   int pipe = 0;
   if constexpr (!RAGGED) {
     if (g.K % kG16BK == 0 && mult8(g.M) && mult8(g.N)) {
       const int64_t k_wg = ceil_div(g.K, splits);  // the K range one workgroup walks
       if (A_KC && B_KC) pipe = k_wg >= 1024 ? 642 : 0;
       else pipe = k_wg >= 4096 ? 642 : 322;
+      // Large products: 256 x 128 tiles (eight waves), a quarter fewer operand bytes per FLOP
+      // through L2, once they still give every CU two workgroups (4096^3: 3-11 % faster).
+      if (splits <= 1 && g.K >= 1024 && ceil_div(g.M, 256) * tiles_n * g.batch >= 2 * cus) pipe = 2322;
       pipe = static_cast<int>(env_int("MOGRAD_HIP_GEMM16_PIPE", pipe));
     }
   }
@@ -111,6 +114,27 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
     }                                                                                                                  \
     launch(gemm_16bit_mfma_kernel<T, A_KC, B_KC, BIAS_, SPLIT_, RAGGED>);                                              \
   } while (0)
+  if (splits <= 1 && (pipe == 2322 || pipe == 2642)) {
+    // 256 x 128 tiles, eight waves: a quarter fewer operand bytes per FLOP through L2.
+    if constexpr (!RAGGED) {
+      const int tiles_m2 = static_cast<int>(ceil_div(g.M, 256));
+      const dim3 grid2(static_cast<unsigned>(static_cast<int64_t>(tiles_m2) * tiles_n * g.batch));
+      auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid2, dim3(512), 0, stream, a, b, bias, c, static_cast<float*>(nullptr), M, N, K, lda,
+                           ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m2, tiles_n, K, epilogue_of<T>(g));
+      };
+      if (pipe == 2322) {
+        if (bias) launch(gemm_16bit_pipe_kernel<T, A_KC, B_KC, true, false, 32, 2, 256>);
+        else launch(gemm_16bit_pipe_kernel<T, A_KC, B_KC, false, false, 32, 2, 256>);
+      } else {
+        if (bias) launch(gemm_16bit_pipe_kernel<T, A_KC, B_KC, true, false, 64, 2, 256>);
+        else launch(gemm_16bit_pipe_kernel<T, A_KC, B_KC, false, false, 64, 2, 256>);
+      }
+      MG_LAUNCH_CHECK();
+      return MG_OK;
+    }
+  }
+  if (pipe > 1000) pipe -= 2000;  // the split-K launch keeps 128 x 128 tiles
   if (splits <= 1) {
     const dim3 grid(static_cast<unsigned>(blocks));
     float* no_partial = nullptr;

@@ -614,21 +614,26 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
 
 typedef short gemm_i16x4 __attribute__((ext_vector_type(4)));
 
-// The four 16-byte source chunks this thread names for every k-step of one operand, as
-// element offsets from the operand's (batch, k_begin) origin; they advance by BK
+// Copy requests per thread, k-step and operand of ROWS rows, for a workgroup of NW waves.
+constexpr int gemm16_pipe_requests(int rows, int bk, int nw) { return rows * bk * 2 / 16 / (nw * 64); }
+
+// The 16-byte source chunks this thread names for every k-step of one operand of ROWS rows,
+// as element offsets from the operand's (batch, k_begin) origin; they advance by BK
 // (k-contiguous) or BK * ld per step.
-template <bool KC, int BK>
-__device__ __forceinline__ void gemm16_pipe_sources(int64_t ld, int o0, int O, int64_t (&src)[BK / 16]) {
-  constexpr int CPR = BK / 8;  // chunks per k-contiguous row
+template <bool KC, int BK, int ROWS, int NW>
+__device__ __forceinline__ void gemm16_pipe_sources(int64_t ld, int o0, int O,
+                                                    int64_t (&src)[gemm16_pipe_requests(ROWS, BK, NW)]) {
+  constexpr int CPR = BK / 8;     // chunks per k-contiguous row
+  constexpr int CPK = ROWS / 8;   // chunks per k-row of the other image
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
 #pragma unroll
-  for (int i = 0; i < BK / 16; ++i) {
-    const int slot = (i * 4 + wave) * kWave + lane;  // 16-byte position in the LDS image
+  for (int i = 0; i < gemm16_pipe_requests(ROWS, BK, NW); ++i) {
+    const int slot = (i * NW + wave) * kWave + lane;  // 16-byte position in the LDS image
     if constexpr (KC) {
       const int r = slot / CPR, c = (slot % CPR) ^ ((r / (16 / CPR)) % CPR);
       src[i] = static_cast<int64_t>(min(o0 + r, O - 1)) * ld + c * 8;  // rows past the edge are never stored
     } else {
-      const int kk = slot / 16, c = (slot % 16) ^ (2 * (kk % 4));
+      const int kk = slot / CPK, c = (slot % CPK) ^ (2 * (kk % 4));
       const int o = o0 + c * 8;
       src[i] = static_cast<int64_t>(kk) * ld + (o < O ? o : o0);
     }
@@ -640,20 +645,20 @@ __device__ __forceinline__ void gemm16_pipe_sources(int64_t ld, int o0, int O, i
 // wait for *all* outstanding copies, the younger steps' included, which would undo the
 // pipeline; the waits are placed by hand in the kernel instead (MG_WAIT_VMCNT).  m0 (the
 // wave's LDS destination) is written here and used by nothing else in these kernels.
-template <int BK>
+template <int NI, int NW>
 __device__ __forceinline__ void gemm16_pipe_issue(const uint16_t* base, const int64_t* src, char* lds_step) {
   using lds_ptr = __attribute__((address_space(3))) char*;
   const int wave = threadIdx.x / kWave;
   const unsigned dst = static_cast<unsigned>(reinterpret_cast<uintptr_t>((lds_ptr)lds_step)) + wave * 1024;
 #pragma unroll
-  for (int i = 0; i < BK / 16; ++i) {
-    const unsigned dst_i = __builtin_amdgcn_readfirstlane(dst + i * 4096);
+  for (int i = 0; i < NI; ++i) {
+    const unsigned dst_i = __builtin_amdgcn_readfirstlane(dst + i * NW * 1024);
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst_i), "v"(base + src[i]) : "memory");
   }
 }
 
 // MFMA operand fragment: row o_base + lane % 32, k = ks * 16 + (lane / 32) * 8 .. + 7.
-template <bool KC, int BK>
+template <bool KC, int BK, int ROWS>
 __device__ __forceinline__ uint4 gemm16_pipe_frag(const char* __restrict__ lds_step, int o_base, int ks, int lane) {
   if constexpr (KC) {
     constexpr int CPR = BK / 8;
@@ -664,12 +669,12 @@ __device__ __forceinline__ uint4 gemm16_pipe_frag(const char* __restrict__ lds_s
     const int o = o_base + ((lane / 16) % 2) * 16 + 4 * (lane % 4);  // first of the 4 rows this lane supplies
     const int kq = (lane % 16) / 4;                                 // its k-row within a group of 4
     const int kk = ks * 16 + (lane / 32) * 8 + kq;
-    const char* at = lds_step + kk * 256 + (((o / 16) ^ kq) * 32) + (o % 16) * 2;
+    const char* at = lds_step + kk * (ROWS * 2) + (((o / 16) ^ kq) * 32) + (o % 16) * 2;
     using lds_i16x4 = __attribute__((address_space(3))) gemm_i16x4;
     const gemm_i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
         reinterpret_cast<lds_i16x4*>(reinterpret_cast<uintptr_t>(at)));
     const gemm_i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        reinterpret_cast<lds_i16x4*>(reinterpret_cast<uintptr_t>(at + 4 * 256)));
+        reinterpret_cast<lds_i16x4*>(reinterpret_cast<uintptr_t>(at + 4 * (ROWS * 2))));
     uint2 l = __builtin_bit_cast(uint2, lo), h = __builtin_bit_cast(uint2, hi);
     return make_uint4(l.x, l.y, h.x, h.y);
   }
@@ -679,32 +684,37 @@ __device__ __forceinline__ uint4 gemm16_pipe_frag(const char* __restrict__ lds_s
 // 15:14, expcnt 6:4 and lgkmcnt 11:8 left at "no wait").
 #define MG_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0f70)
 
-// Workgroups of the pipelined kernel that fit a CU: by LDS (160 KB) and, at four waves per
-// workgroup, by the register file (at most four).
-constexpr int gemm16_pipe_lds_bytes(int bk, int nstage) {
-  const int stages = nstage * 2 * 128 * bk * 2, out = 4 * 64 * kG16Stride * 2;  // the output tile is transposed here
+// LDS of the pipelined kernel (TM = rows of the A tile: 128 with four waves, 256 with eight) and
+// the workgroups that fit a CU, by LDS (160 KB) and by the register file.
+constexpr int gemm16_pipe_lds_bytes(int bk, int nstage, int tm) {
+  const int stages = nstage * (tm + 128) * bk * 2;
+  const int out = (tm / 32) * 64 * kG16Stride * 2;  // every wave transposes its output tile here
   return stages > out ? stages : out;
 }
-constexpr int gemm16_pipe_occupancy(int bk, int nstage) {
-  const int by_lds = 160 * 1024 / gemm16_pipe_lds_bytes(bk, nstage);
-  return by_lds < 1 ? 1 : (by_lds > 4 ? 4 : by_lds);
+constexpr int gemm16_pipe_occupancy(int bk, int nstage, int tm) {
+  const int by_lds = 160 * 1024 / gemm16_pipe_lds_bytes(bk, nstage, tm);
+  const int by_regs = tm == 128 ? 4 : 2;
+  return by_lds < 1 ? 1 : (by_lds > by_regs ? by_regs : by_lds);
 }
 
-template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, int BK, int NSTAGE>
-__global__ __launch_bounds__(kGemmThreads, gemm16_pipe_occupancy(BK, NSTAGE)) void gemm_16bit_pipe_kernel(
+template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, int BK, int NSTAGE, int TM = 128>
+__global__ __launch_bounds__(TM * 2, gemm16_pipe_occupancy(BK, NSTAGE, TM)) void gemm_16bit_pipe_kernel(
     const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C,
     float* __restrict__ partial, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb,
     int64_t bsc, int tiles_m, int tiles_n, int k_per_split, GemmEpilogue<T> ep) {
-  static_assert(NSTAGE >= 2 && NSTAGE <= 4 && (BK == 32 || BK == 64), "stages");
-  constexpr int NI = BK / 16;  // copy requests per thread, operand and step
-  constexpr int OP = 128 * BK * 2;  // bytes of one operand's step
-  __shared__ __attribute__((aligned(1024))) char lds[gemm16_pipe_lds_bytes(BK, NSTAGE)];
+  static_assert(NSTAGE >= 2 && NSTAGE <= 4 && (BK == 32 || BK == 64) && (TM == 128 || TM == 256), "stages");
+  constexpr int NW = TM / 32;                                 // waves: (TM / 64) x 2 wave tiles of 64 x 64
+  constexpr int NIA = gemm16_pipe_requests(TM, BK, NW);       // copy requests per thread and step
+  constexpr int NIB = gemm16_pipe_requests(kGemmBN, BK, NW);
+  constexpr int OPA = TM * BK * 2, OPB = kGemmBN * BK * 2;    // bytes of an operand's step
+  constexpr int OP = OPA + OPB;
+  __shared__ __attribute__((aligned(1024))) char lds[gemm16_pipe_lds_bytes(BK, NSTAGE, TM)];
 
   const int tiles = tiles_m * tiles_n;
   const int batch = SPLIT_K ? blockIdx.z : blockIdx.x / tiles;
   int tm, tn;
   gemm_tile_of_block(blockIdx.x % tiles, tiles_m, tiles_n, tm, tn);
-  const int m0 = tm * kGemmBM;
+  const int m0 = tm * TM;
   const int n0 = tn * kGemmBN;
   const int k_begin = SPLIT_K ? blockIdx.y * k_per_split : 0;
   const int k_end = SPLIT_K ? min(K, k_begin + k_per_split) : K;
@@ -729,47 +739,47 @@ __global__ __launch_bounds__(kGemmThreads, gemm16_pipe_occupancy(BK, NSTAGE)) vo
 
   const uint16_t* a16 = reinterpret_cast<const uint16_t*>(A);
   const uint16_t* b16 = reinterpret_cast<const uint16_t*>(B);
-  int64_t src_a[NI], src_b[NI];
-  gemm16_pipe_sources<A_KC, BK>(lda, m0, M, src_a);
-  gemm16_pipe_sources<B_KC, BK>(ldb, n0, N, src_b);
+  int64_t src_a[NIA], src_b[NIB];
+  gemm16_pipe_sources<A_KC, BK, TM, NW>(lda, m0, M, src_a);
+  gemm16_pipe_sources<B_KC, BK, kGemmBN, NW>(ldb, n0, N, src_b);
 
   // Steps 0 .. NSTAGE-2 are requested up front; iteration `it` then waits for step `it`
-  // (its own 2 * NI requests; the barrier covers the other waves'), requests step
+  // (its own NIA + NIB requests; the barrier covers the other waves'), requests step
   // it + NSTAGE - 1 into the copy that step it - 1 was just multiplied from, and multiplies.
 #pragma unroll
   for (int s = 0; s < NSTAGE - 1; ++s)
     if (s < steps) {
-      gemm16_pipe_issue<BK>(a16 + s * a_step, src_a, lds + (2 * s) * OP);
-      gemm16_pipe_issue<BK>(b16 + s * b_step, src_b, lds + (2 * s + 1) * OP);
+      gemm16_pipe_issue<NIA, NW>(a16 + s * a_step, src_a, lds + s * OP);
+      gemm16_pipe_issue<NIB, NW>(b16 + s * b_step, src_b, lds + s * OP + OPA);
     }
   int cur = 0, nxt = NSTAGE - 1;
   for (int it = 0; it < steps; ++it) {
-    if (it + NSTAGE - 2 < steps) MG_WAIT_VMCNT(2 * NI * (NSTAGE - 2));  // all but the NSTAGE-2 younger steps
+    if (it + NSTAGE - 2 < steps) MG_WAIT_VMCNT((NIA + NIB) * (NSTAGE - 2));  // all but the NSTAGE-2 younger steps
     else MG_WAIT_VMCNT(0);
     // A plain barrier: __syncthreads() carries a fence that waits for every outstanding
     // copy into LDS, the younger steps' included.
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     if (it + NSTAGE - 1 < steps) {
-      gemm16_pipe_issue<BK>(a16 + (it + NSTAGE - 1) * a_step, src_a, lds + (2 * nxt) * OP);
-      gemm16_pipe_issue<BK>(b16 + (it + NSTAGE - 1) * b_step, src_b, lds + (2 * nxt + 1) * OP);
+      gemm16_pipe_issue<NIA, NW>(a16 + (it + NSTAGE - 1) * a_step, src_a, lds + nxt * OP);
+      gemm16_pipe_issue<NIB, NW>(b16 + (it + NSTAGE - 1) * b_step, src_b, lds + nxt * OP + OPA);
     }
-    const char* la = lds + (2 * cur) * OP;
-    const char* lb = la + OP;
+    const char* la = lds + cur * OP;
+    const char* lb = la + OPA;
     // The fragments of k-slice ks + 1 are requested before the products of slice ks, so
     // their LDS latency runs under four MFMAs.
     uint4 fa[2][2], fb[2][2];
-    fa[0][0] = gemm16_pipe_frag<A_KC, BK>(la, wm, 0, lane);
-    fa[0][1] = gemm16_pipe_frag<A_KC, BK>(la, wm + 32, 0, lane);
-    fb[0][0] = gemm16_pipe_frag<B_KC, BK>(lb, wn, 0, lane);
-    fb[0][1] = gemm16_pipe_frag<B_KC, BK>(lb, wn + 32, 0, lane);
+    fa[0][0] = gemm16_pipe_frag<A_KC, BK, TM>(la, wm, 0, lane);
+    fa[0][1] = gemm16_pipe_frag<A_KC, BK, TM>(la, wm + 32, 0, lane);
+    fb[0][0] = gemm16_pipe_frag<B_KC, BK, kGemmBN>(lb, wn, 0, lane);
+    fb[0][1] = gemm16_pipe_frag<B_KC, BK, kGemmBN>(lb, wn + 32, 0, lane);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       const int c = ks % 2, n = c ^ 1;
       if (ks + 1 < BK / 16) {
-        fa[n][0] = gemm16_pipe_frag<A_KC, BK>(la, wm, ks + 1, lane);
-        fa[n][1] = gemm16_pipe_frag<A_KC, BK>(la, wm + 32, ks + 1, lane);
-        fb[n][0] = gemm16_pipe_frag<B_KC, BK>(lb, wn, ks + 1, lane);
-        fb[n][1] = gemm16_pipe_frag<B_KC, BK>(lb, wn + 32, ks + 1, lane);
+        fa[n][0] = gemm16_pipe_frag<A_KC, BK, TM>(la, wm, ks + 1, lane);
+        fa[n][1] = gemm16_pipe_frag<A_KC, BK, TM>(la, wm + 32, ks + 1, lane);
+        fb[n][0] = gemm16_pipe_frag<B_KC, BK, kGemmBN>(lb, wn, ks + 1, lane);
+        fb[n][1] = gemm16_pipe_frag<B_KC, BK, kGemmBN>(lb, wn + 32, ks + 1, lane);
       }
       acc[0][0] = GemmMma16<T>::run(fa[c][0], fb[c][0], acc[0][0]);
       acc[0][1] = GemmMma16<T>::run(fa[c][0], fb[c][1], acc[0][1]);

@@ -200,11 +200,11 @@ def test_half_precision_mfma_paths(device, dtype, rtol, M, N, K):
 
 @pytest.mark.parametrize("dtype,rtol", [(F16, 2e-3), (BF16, 1.6e-2)])
 @pytest.mark.parametrize("M,N,K", [(256, 384, 512), (384, 128, 1536), (200, 136, 256), (128, 64, 4096), (1024, 384, 1024),
-                                   (72, 1536, 64)])
+                                   (72, 1536, 64), (520, 264, 320)])
 def test_tile_staging_variants_agree(device, monkeypatch, dtype, rtol, M, N, K):
     # The 16-bit products have a register-staged kernel (0) and one whose tiles are copied
-    # straight into LDS, 32 or 64 k per step (322, 642); the library picks by operand layout
-    # and K.  All accumulate each output element over k in the same order on the same MFMA,
+    # straight into LDS, 32 or 64 k per step (322, 642), also with 256 x 128 output tiles
+    # (2322, 2642); the library picks by operand layout, K and size.  All accumulate each output element over k in the same order on the same MFMA,
     # so forcing either must not change a bit, for every operand layout (forward k/k, dX
     # k/n, dW m/n, the last split along K for the tall shapes) and at ragged tile edges.
     x = round_to_dtype(normal(49, 0, (M, K)), dtype)
@@ -212,12 +212,12 @@ def test_tile_staging_variants_agree(device, monkeypatch, dtype, rtol, M, N, K):
     b = round_to_dtype(normal(49, 2, (N,), std=0.1), dtype)
     dy = round_to_dtype(normal(49, 3, (M, N), std=0.5), dtype)
     results = {}
-    for variant in ("0", "322", "642"):
+    for variant in ("0", "322", "642", "2322", "2642"):
         monkeypatch.setenv("MOGRAD_HIP_GEMM16_PIPE", variant)
         results[variant] = _linear_all(device, x, w, b, dy, dtype)
     monkeypatch.delenv("MOGRAD_HIP_GEMM16_PIPE")
     results["auto"] = _linear_all(device, x, w, b, dy, dtype)
-    for variant in ("322", "642", "auto"):
+    for variant in ("322", "642", "2322", "2642", "auto"):
         for got, base, name in zip(results[variant], results["0"], ("y", "dx", "dw", "db")):
             np.testing.assert_array_equal(got, base, err_msg=f"{name}, variant {variant}")
     y, dx, dw, _ = results["auto"]
@@ -263,7 +263,7 @@ def test_batched_projections_share_an_operand(device, dtype, rtol, M, d):
     assert_close(dw.to_numpy((3, d, d)), want_dw, rtol, rtol * np.abs(want_dw).max(), "dw")
 
 
-@pytest.mark.parametrize("variant", ["0", "322", "642"])
+@pytest.mark.parametrize("variant", ["0", "322", "642", "2322", "2642"])
 def test_batched_projections_tile_staging_variants(device, monkeypatch, variant):
     # The same two batched products (batch stride 0 on the shared operand; the second split
     # along K with the batch in the grid's z) through each 16-bit tile-staging variant.
