@@ -263,6 +263,34 @@ def test_batched_projections_share_an_operand(device, dtype, rtol, M, d):
     assert_close(dw.to_numpy((3, d, d)), want_dw, rtol, rtol * np.abs(want_dw).max(), "dw")
 
 
+def test_large_products_agree_with_the_register_staged_kernel(device, monkeypatch):
+    # A product large enough that the library picks 256 x 128 tiles by itself (K >= 1024 and
+    # two such tiles per CU) must equal the register-staged kernel's result bit for bit, for
+    # the forward and both gradient layouts.
+    M, N, K = 8192, 2048, 1024
+    x = round_to_dtype(normal(58, 0, (M, K)), BF16)
+    w = round_to_dtype(normal(58, 1, (N, K), std=0.05), BF16)
+    dy = round_to_dtype(normal(58, 2, (M, N), std=0.5), BF16)
+    lib, st = device.lib, device.stream
+    bx, bw, bdy = (AnyBuffer.from_numpy(device, a, BF16) for a in (x, w, dy))
+
+    def run():
+        y, dx, dw = (AnyBuffer.create(BF16, device, n) for n in (M * N, M * K, N * K))
+        lib.mg_matmul_bt(bx.data_ptr(), bw.data_ptr(), y.data_ptr(), 1, M, N, K, K, 1, K, 1, M * K, N * K, BF16, st)
+        lib.mg_linear_bwd(bdy.data_ptr(), bx.data_ptr(), bw.data_ptr(), dx.data_ptr(), dw.data_ptr(), None, M, N, K, BF16, st)
+        return y.to_numpy((M, N)), dx.to_numpy((M, K)), dw.to_numpy((N, K))
+
+    auto = run()
+    monkeypatch.setenv("MOGRAD_HIP_GEMM16_PIPE", "0")
+    base = run()
+    for got, want, name in zip(auto, base, ("y", "dx", "dw")):
+        np.testing.assert_array_equal(got, want, err_msg=name)
+    # and a spot check of the forward against float64 on a few rows
+    rows = [0, 257, 4095, 8191]
+    want = x[rows].astype(np.float64) @ w.astype(np.float64).T
+    assert_close(auto[0][rows], want, 1.6e-2, 1.6e-2 * np.abs(want).max(), "y rows")
+
+
 @pytest.mark.parametrize("variant", ["0", "322", "642", "2322", "2642"])
 def test_batched_projections_tile_staging_variants(device, monkeypatch, variant):
     # The same two batched products (batch stride 0 on the shared operand; the second split
