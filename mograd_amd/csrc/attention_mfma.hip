@@ -342,12 +342,18 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
     if (CAUSAL && n0 > m_wave + 31) continue;  // every key of the block is in this wave's future
 
     floatx16 s[2];
+    // The forward is bound by its VALU work (32 exponentials and about 150 other VALU
+    // instructions per 16 MFMAs and wave), three waves per SIMD: a wave that is issuing MFMAs
+    // gets priority over the ones doing softmax arithmetic, which keeps the matrix pipe fed
+    // (3-4 % faster; the same hints in the backward kernels measured neutral to slower).
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
       s[nt] = zero16();
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) s[nt] = Mma<T>::run(frag_rows<DP>(k_rows, at, nt, ks), qf[ks], s[nt]);
     }
+    __builtin_amdgcn_s_setprio(0);
     // A block needs per-element masking only at the end of the sequence and, for causal
     // attention, where it crosses the diagonal of this wave's queries.
     const bool plain = !HAS_BIAS && c > 0.f && n0 + BN <= a.S && (!CAUSAL || n0 + BN - 1 <= m_wave);
@@ -410,12 +416,14 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc_o[dt][r] *= corr;
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int t = 0; t < BN / 16; ++t) {
       const uint4 pf = frag_from_acc<T>(s[t / 2], t % 2);
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) acc_o[dt] = Mma<T>::run(frag_transposed<DP>(v_rows, at, dt, t), pf, acc_o[dt]);
     }
+    __builtin_amdgcn_s_setprio(0);
   }
 
   if (m < a.S) {
