@@ -632,13 +632,22 @@ __device__ __forceinline__ void attn_dq_block(const int block, char* smem, const
 // ---- dK, dV ------------------------------------------------------------------------------
 
 // Bytes of LDS the dK/dV walk stages its tiles and row statistics in.
-template <int DP>
+// Bytes of LDS the dK/dV walk stages its tiles and row statistics in, for steps of BQ queries:
+// two copies of a Q tile, a dO tile, lse and delta.
+template <int DP, int BQ>
 constexpr int dkdv_lds_bytes() {
-  return 2 * (2 * 64 * tile_row_bytes<DP>() + 2 * 64 * 4);  // two copies of a Q tile, a dO tile, lse and delta
+  return 2 * (2 * BQ * tile_row_bytes<DP>() + 2 * BQ * 4);
 }
+// Queries per step when the walk has a launch of its own (sequences past 1024 tokens, or head
+// dims above 64): 128 for head dims up to 64, half as many barriers per query (S = 4096
+// 440 -> 430 us, S = 2048 causal 198 -> 191 us; at S = 256 it would cost 3 %, but there the
+// walk shares a launch with dQ and steps by 64).
+template <int DP>
+constexpr int dkdv_long_step() { return DP <= 64 ? 128 : 64; }
 
-// The work of workgroup `block` of a dK/dV launch; `smem` holds dkdv_lds_bytes<DP>() bytes.
-template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
+// The work of workgroup `block` of a dK/dV launch, BQ queries per step; `smem` holds
+// dkdv_lds_bytes<DP, BQ>() bytes.
+template <typename T, int DP, int BQ, bool CAUSAL, bool HAS_BIAS>
 __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, const T* __restrict__ d_o,
                                                 const T* __restrict__ q, const T* __restrict__ k,
                                                 const T* __restrict__ v, const T* __restrict__ mask,
@@ -646,7 +655,6 @@ __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, con
                                                 T* __restrict__ dk, T* __restrict__ dv, const AttnDims& a,
                                                 float scale) {
   constexpr int BNK = 128;                 // keys per workgroup
-  constexpr int BQ = 64;                   // queries per step
   constexpr int MT = BQ / 32, KS = DP / 16, DT = DP / 32;
   // Two copies of every staged tile: step i computes from copy i % 2 while the tile of step
   // i + 1 is written into the other, so one barrier per step suffices.
@@ -655,7 +663,7 @@ __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, con
   auto do_rows_s = reinterpret_cast<char(*)[ROWS]>(smem + 2 * ROWS);
   auto lse_ss = reinterpret_cast<float(*)[BQ]>(smem + 4 * ROWS);
   auto delta_ss = reinterpret_cast<float(*)[BQ]>(smem + 4 * ROWS + 2 * BQ * 4);
-  static_assert(dkdv_lds_bytes<DP>() == 4 * ROWS + 4 * BQ * 4, "LDS size");
+  static_assert(dkdv_lds_bytes<DP, BQ>() == 4 * ROWS + 4 * BQ * 4, "LDS size");
 
   // (batch, head) varies fastest across consecutive workgroups.  Causal: earlier key blocks
   // are seen by more queries; all of them launch first.
@@ -849,8 +857,8 @@ __global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma
     const T* __restrict__ d_o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
     const T* __restrict__ mask, const float* __restrict__ lse, const float* __restrict__ delta, T* __restrict__ dk,
     T* __restrict__ dv, AttnDims a, float scale) {
-  __shared__ __attribute__((aligned(16))) char smem[dkdv_lds_bytes<DP>()];
-  attn_dkdv_block<T, DP, CAUSAL, HAS_BIAS>(blockIdx.x, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
+  __shared__ __attribute__((aligned(16))) char smem[dkdv_lds_bytes<DP, dkdv_long_step<DP>()>()];
+  attn_dkdv_block<T, DP, dkdv_long_step<DP>(), CAUSAL, HAS_BIAS>(blockIdx.x, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
 }
 
 // Both walks in one launch (head dims up to 64, where the two have the same occupancy):
@@ -862,12 +870,12 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_mfma_kernel(
     const T* __restrict__ d_o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
     const T* __restrict__ mask, const float* __restrict__ lse, const float* __restrict__ delta, T* __restrict__ dq,
     T* __restrict__ dk, T* __restrict__ dv, AttnDims a, float scale, int blocks) {
-  constexpr int LDS = dkdv_lds_bytes<DP>() > dq_lds_bytes<DP>() ? dkdv_lds_bytes<DP>() : dq_lds_bytes<DP>();
+  constexpr int LDS = dkdv_lds_bytes<DP, 64>() > dq_lds_bytes<DP>() ? dkdv_lds_bytes<DP, 64>() : dq_lds_bytes<DP>();
   __shared__ __attribute__((aligned(16))) char smem[LDS];
   const int block = (blockIdx.x / 16) * 8 + blockIdx.x % 8;
   if (block >= blocks) return;
   if ((blockIdx.x / 8) % 2 == 0)
-    attn_dkdv_block<T, DP, CAUSAL, HAS_BIAS>(block, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
+    attn_dkdv_block<T, DP, 64, CAUSAL, HAS_BIAS>(block, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
   else
     attn_dq_block<T, DP, 1, CAUSAL, HAS_BIAS>(block, smem, d_o, q, k, v, mask, lse, delta, dq, a, scale);
 }
