@@ -43,6 +43,49 @@ def test_random_linear_shapes(device):
             assert_close(got, want, rt, rt * max(np.abs(want).max(), 1e-3), f"case {case} {(M, N, K)} dtype {dtype} {name}")
 
 
+def test_random_16bit_tile_staging_shapes(device, monkeypatch):
+    # Shapes the LDS-copy GEMM kernels take (extents multiples of 8, K a multiple of 64), with
+    # padded leading dimensions and batches, through every forced variant: all must equal the
+    # register-staged kernel bit for bit, and that one the float64 product.
+    rng = np.random.Generator(np.random.PCG64(95_100))
+    lib, st = device.lib, device.stream
+    for case in range(24):
+        dtype = (F16, BF16)[case % 2]
+        batch = int(rng.integers(1, 4))
+        M, N = (8 * int(v) for v in rng.integers(1, 66, 2))
+        K = 64 * int(rng.integers(1, 33 if case % 4 else 5))
+        lda, ldb = K + 8 * int(rng.integers(0, 3)), K + 8 * int(rng.integers(0, 3))
+        a = round_to_dtype(rng.standard_normal((batch, M, lda)).astype(np.float32), dtype)
+        b = round_to_dtype((rng.standard_normal((batch, N, ldb)) * 0.1).astype(np.float32), dtype)
+        ba, bb = AnyBuffer.from_numpy(device, a, dtype), AnyBuffer.from_numpy(device, b, dtype)
+        results = {}
+        for variant in ("0", "322", "642", "2322", "2642"):
+            monkeypatch.setenv("MOGRAD_HIP_GEMM16_PIPE", variant)
+            nt, nn, tn = (AnyBuffer.create(dtype, device, n) for n in (batch * M * N, batch * M * ldb, batch * lda * N))
+            # C = A B^T over k (both k-contiguous)
+            lib.mg_matmul_bt(ba.data_ptr(), bb.data_ptr(), nt.data_ptr(), batch, M, N, K, lda, 1, ldb, 1, M * lda, N * ldb,
+                             dtype, st)
+            # C2(M, ldb) = C(M, N) B(N, ldb): right operand n-contiguous (the dX layout); K here is N
+            # C3(lda, N) = A^T(lda, M) C(M, N): left operand m-contiguous (the dW layout); K here is M
+            if N % 64 == 0:
+                lib.mg_matmul(nt.data_ptr(), bb.data_ptr(), nn.data_ptr(), batch, M, ldb, N, N, 1, ldb, 1, M * N, N * ldb,
+                              dtype, st)
+            if M % 64 == 0:
+                lib.mg_matmul(ba.data_ptr(), nt.data_ptr(), tn.data_ptr(), batch, lda, N, M, 1, lda, N, 1, M * lda, M * N,
+                              dtype, st)
+            results[variant] = (nt.to_numpy((batch, M, N)), nn.to_numpy((batch, M, ldb)) if N % 64 == 0 else None,
+                                tn.to_numpy((batch, lda, N)) if M % 64 == 0 else None)
+        what = f"case {case} batch {batch} {(M, N, K)} ld {(lda, ldb)} dtype {dtype}"
+        for variant in ("322", "642", "2322", "2642"):
+            for got, base, name in zip(results[variant], results["0"], ("nt", "nn", "tn")):
+                if base is not None:
+                    np.testing.assert_array_equal(got, base, err_msg=f"{what} {name} variant {variant}")
+        want = np.einsum("bmk,bnk->bmn", a[:, :, :K].astype(np.float64), b[:, :, :K].astype(np.float64))
+        rt = RT[dtype]
+        assert_close(results["0"][0], want, rt, rt * max(np.abs(want).max(), 1e-3), what)
+    monkeypatch.delenv("MOGRAD_HIP_GEMM16_PIPE")
+
+
 def test_random_attention_shapes(device):
     rng = np.random.Generator(np.random.PCG64(96_000))
     lib, st = device.lib, device.stream
