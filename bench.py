@@ -256,7 +256,7 @@ def bench_mlp(args, dev) -> int:
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "README MLP fwd+bwd fp32: x (2048,4096) -> Linear 4096 +ReLU -> LayerNorm -> Linear 4096 "
                                "+ReLU -> Linear 10, cross-entropy, labels in [0,10)"},
-        "roofline": {"bound": "mfma", "kernel": "gemm_f32_mfma_kernel, " + dom["name"], "achieved": dom["achieved_TFLOPs"],
+        "roofline": {"bound": "mfma", "kernel": "gemm_f32_pipe_kernel, " + dom["name"], "achieved": dom["achieved_TFLOPs"],
                      "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac_of_mfma_peak"], "traffic": None},
         "kernels": kernels,
     }

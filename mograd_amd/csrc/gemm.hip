@@ -42,6 +42,22 @@ static int launch_f32_mfma(const GemmArgs& g, hipStream_t stream) {
   // Two workgroups are resident per CU; a larger problem is walked by that many workgroups.
   int64_t grid = 2 * static_cast<int64_t>(device_info().cu_count) * env_int("MOGRAD_HIP_GEMM_F32_ROUNDS", 1);
   if (grid > blocks || env_int("MOGRAD_HIP_GEMM_F32_ROUNDS", 1) == 0) grid = blocks;
+  // Tiles copied straight into LDS (gemm_f32_pipe_kernel, same results bit for bit) when K is a
+  // multiple of the 32-deep step; MOGRAD_HIP_GEMM_F32_PIPE=0 keeps the register-staged kernel.
+  if (g.K % kGemmBK == 0 && env_int("MOGRAD_HIP_GEMM_F32_PIPE", 1) != 0) {
+    if (bias)
+      hipLaunchKernelGGL((gemm_f32_pipe_kernel<A_KC, B_KC, true>), dim3(static_cast<unsigned>(grid)),
+                         dim3(kGemmThreads), 0, stream, a, b, bias, c, static_cast<int>(g.M), static_cast<int>(g.N),
+                         static_cast<int>(g.K), lda, ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n,
+                         static_cast<int>(blocks), epilogue_of<float>(g));
+    else
+      hipLaunchKernelGGL((gemm_f32_pipe_kernel<A_KC, B_KC, false>), dim3(static_cast<unsigned>(grid)),
+                         dim3(kGemmThreads), 0, stream, a, b, bias, c, static_cast<int>(g.M), static_cast<int>(g.N),
+                         static_cast<int>(g.K), lda, ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n,
+                         static_cast<int>(blocks), epilogue_of<float>(g));
+    MG_LAUNCH_CHECK();
+    return MG_OK;
+  }
   if (bias)
     hipLaunchKernelGGL((gemm_f32_mfma_kernel<A_KC, B_KC, true>), dim3(static_cast<unsigned>(grid)), dim3(kGemmThreads),
                        0, stream, a, b, bias, c, static_cast<int>(g.M), static_cast<int>(g.N), static_cast<int>(g.K), lda,

@@ -797,6 +797,172 @@ __global__ __launch_bounds__(TM * 2, gemm16_pipe_occupancy(BK, NSTAGE, TM)) void
                                           m0, n0, wm, wn, lane, ep);
 }
 
+// ------------------------------------------------------------------------------------
+// fp32 product with the tiles copied global memory -> LDS by `global_load_lds_dwordx4`, two
+// copies of each 128 x 32 tile: the copy of k-step i + 1 runs under the MFMAs of step i with
+// one barrier per step and no registers or VALU work spent on staging.  Same tiles, same
+// wave layout, same k order inside a step as gemm_f32_mfma_kernel (MFMA j of k-group g
+// multiplies k in {g*8 + j, g*8 + 4 + j}), so the two kernels give identical bits.
+// Requires K % 32 == 0 on top of that kernel's alignment conditions.
+//
+// LDS image of one operand's step (16 KB):
+//   k-contiguous: [128 rows][8 chunks of 4 k], chunk c of row r at position c ^ (r/2 % 8)
+//     (sixteen consecutive rows of a 128-bit fragment read hit sixteen bank groups);
+//   otherwise: [32 k][32 chunks of 4 rows], chunk c of k-row kk at position
+//     c ^ (8 * (kk/4 % 2)): the two halves of a wave read k and k + 4 of the same rows, 128
+//     bytes apart in the banks.
+// ------------------------------------------------------------------------------------
+
+template <bool KC>
+__device__ __forceinline__ void gemm32_pipe_sources(int64_t ld, int o0, int O, int64_t (&src)[4]) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int slot = (i * 4 + wave) * kWave + lane;  // 16-byte position in the LDS image
+    if constexpr (KC) {
+      const int r = slot / 8, c = (slot % 8) ^ ((r / 2) % 8);
+      src[i] = static_cast<int64_t>(min(o0 + r, O - 1)) * ld + c * 4;  // rows past the edge are never stored
+    } else {
+      const int kk = slot / 32, c = (slot % 32) ^ (8 * ((kk / 4) % 2));
+      const int o = o0 + c * 4;
+      src[i] = static_cast<int64_t>(kk) * ld + (o < O ? o : o0);
+    }
+  }
+}
+
+// See gemm16_pipe_issue for why this is assembly.
+__device__ __forceinline__ void gemm32_pipe_issue(const float* base, const int64_t* src, char* lds_step) {
+  using lds_ptr = __attribute__((address_space(3))) char*;
+  const int wave = threadIdx.x / kWave;
+  const unsigned dst = static_cast<unsigned>(reinterpret_cast<uintptr_t>((lds_ptr)lds_step)) + wave * 1024;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const unsigned dst_i = __builtin_amdgcn_readfirstlane(dst + i * 4096);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst_i), "v"(base + src[i]) : "memory");
+  }
+}
+
+// MFMA operand values of one 32-wide tile for k-group g (see gemm_read_frag).
+template <bool KC>
+__device__ __forceinline__ void gemm32_pipe_frag(const char* __restrict__ lds_step, int o_base, int g, int lane,
+                                                 float (&f)[4]) {
+  const int o = o_base + lane % 32;
+  if constexpr (KC) {
+    const int c = g * 2 + lane / 32;
+    const float4 r = *reinterpret_cast<const float4*>(lds_step + o * 128 + ((c ^ ((o / 2) % 8)) * 16));
+    f[0] = r.x; f[1] = r.y; f[2] = r.z; f[3] = r.w;
+  } else {
+    const int kk = g * 8 + (lane / 32) * 4;  // (kk / 4) % 2 == lane / 32 for all four k of this lane
+    const char* at = lds_step + kk * 512 + ((((o / 4) ^ (8 * (lane / 32))) * 16) + (o % 4) * 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) f[j] = *reinterpret_cast<const float*>(at + j * 512);
+  }
+}
+
+template <bool A_KC, bool B_KC, bool HAS_BIAS>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_pipe_kernel(
+    const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias, float* __restrict__ C,
+    int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb, int64_t bsc, int tiles_m,
+    int tiles_n, int total_work, GemmEpilogue<float> ep_in) {
+  constexpr int OP = kGemmBM * kGemmBK * 4;  // bytes of one operand's step
+  __shared__ __attribute__((aligned(1024))) char lds[2][2][OP];
+
+  const int tiles = tiles_m * tiles_n;
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int wm = (wave / 2) * 64;
+  const int wn = (wave % 2) * 64;
+  const int steps = K / kGemmBK;
+  const int64_t a_step = A_KC ? kGemmBK : kGemmBK * lda;
+  const int64_t b_step = B_KC ? kGemmBK : kGemmBK * ldb;
+  // The grid holds at most the workgroups that are resident at once; each takes output tiles
+  // work, work + gridDim.x, ... (see gemm_f32_mfma_kernel).
+  for (int work = blockIdx.x; work < total_work; work += gridDim.x) {
+    const int batch = work / tiles;
+    int tm, tn;
+    gemm_tile_of_block(work % tiles, tiles_m, tiles_n, tm, tn);
+    const int m0 = tm * kGemmBM;
+    const int n0 = tn * kGemmBN;
+    const float* a = A + batch * bsa;
+    const float* b = B + batch * bsb;
+    float* c = C + batch * bsc;
+    GemmEpilogue<float> ep = ep_in;
+    if (ep.residual) ep.residual += batch * bsc;
+    if (ep.relu_mask) ep.relu_mask += batch * bsc;
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    int64_t src_a[4], src_b[4];
+    gemm32_pipe_sources<A_KC>(lda, m0, M, src_a);
+    gemm32_pipe_sources<B_KC>(ldb, n0, N, src_b);
+    gemm32_pipe_issue(a, src_a, lds[0][0]);
+    gemm32_pipe_issue(b, src_b, lds[0][1]);
+    for (int it = 0; it < steps; ++it) {
+      const int cur = it & 1;
+      // This wave's copies of step `it` have landed; the barrier covers the other waves' and
+      // tells that everyone is done reading the other copy.  (A plain barrier: __syncthreads()
+      // would be the same here, every copy being waited for, but costs a fence.)
+      MG_WAIT_VMCNT(0);
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      if (it + 1 < steps) {
+        gemm32_pipe_issue(a + (it + 1) * a_step, src_a, lds[cur ^ 1][0]);
+        gemm32_pipe_issue(b + (it + 1) * b_step, src_b, lds[cur ^ 1][1]);
+      }
+      const char* la = lds[cur][0];
+      const char* lb = lds[cur][1];
+      // The fragments of k-group g + 1 are requested before the products of group g.
+      float fa[2][2][4], fb[2][2][4];
+      gemm32_pipe_frag<A_KC>(la, wm, 0, lane, fa[0][0]);
+      gemm32_pipe_frag<A_KC>(la, wm + 32, 0, lane, fa[0][1]);
+      gemm32_pipe_frag<B_KC>(lb, wn, 0, lane, fb[0][0]);
+      gemm32_pipe_frag<B_KC>(lb, wn + 32, 0, lane, fb[0][1]);
+#pragma unroll
+      for (int g = 0; g < kGemmBK / 8; ++g) {
+        const int p = g % 2, n = p ^ 1;
+        if (g + 1 < kGemmBK / 8) {
+          gemm32_pipe_frag<A_KC>(la, wm, g + 1, lane, fa[n][0]);
+          gemm32_pipe_frag<A_KC>(la, wm + 32, g + 1, lane, fa[n][1]);
+          gemm32_pipe_frag<B_KC>(lb, wn, g + 1, lane, fb[n][0]);
+          gemm32_pipe_frag<B_KC>(lb, wn + 32, g + 1, lane, fb[n][1]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+            for (int tj = 0; tj < 2; ++tj)
+              acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[p][ti][j], fb[p][tj][j], acc[ti][tj], 0, 0, 0);
+      }
+    }
+    // The next tile's first copy goes into lds[0]: every wave must be done reading it.
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+    // Accumulator element r of a lane is row (r/4)*8 + (lane/32)*4 + r%4, column lane%32.
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+      for (int tj = 0; tj < 2; ++tj) {
+        const int col = n0 + wn + tj * 32 + lane % 32;
+        if (col >= N) continue;
+        const float bv = HAS_BIAS ? bias[col] : 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = m0 + wm + ti * 32 + (r / 4) * 8 + (lane / 32) * 4 + (r % 4);
+          if (row < M) {
+            const int64_t at = static_cast<int64_t>(row) * ldc + col;
+            c[at] = gemm_finish<float>(acc[ti][tj][r] + bv, ep, at);
+          }
+        }
+      }
+  }  // tiles of this workgroup
+}
+
 // out[i] = sum_s partial[s][i] (+ bias[i % N]), converted to T.  A workgroup covers 64
 // groups of four consecutive outputs; its four waves each sum every fourth split (eight
 // independent 16-byte loads in flight per thread) and the four sums meet in LDS.  The

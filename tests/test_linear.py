@@ -263,6 +263,27 @@ def test_batched_projections_share_an_operand(device, dtype, rtol, M, d):
     assert_close(dw.to_numpy((3, d, d)), want_dw, rtol, rtol * np.abs(want_dw).max(), "dw")
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 384, 512), (200, 136, 256), (128, 64, 4096), (520, 264, 320), (64, 1000, 32),
+                                   (2048, 512, 1024)])
+def test_f32_tile_staging_variants_agree(device, monkeypatch, M, N, K):
+    # fp32 products have a register-staged kernel and one whose tiles are copied straight into
+    # LDS (K a multiple of 32); same tiles and k order, so the results must be identical bits
+    # for the forward (k/k), dX (k/n) and dW (m/n) operand layouts, ragged tile edges included.
+    x = normal(59, 0, (M, K))
+    w = normal(59, 1, (N, K), std=0.05)
+    b = normal(59, 2, (N,), std=0.1)
+    dy = normal(59, 3, (M, N), std=0.5)
+    monkeypatch.setenv("MOGRAD_HIP_GEMM_F32_PIPE", "0")
+    base = _linear_all(device, x, w, b, dy)
+    monkeypatch.delenv("MOGRAD_HIP_GEMM_F32_PIPE")
+    got = _linear_all(device, x, w, b, dy)
+    for g, want, name in zip(got, base, ("y", "dx", "dw", "db")):
+        np.testing.assert_array_equal(g, want, err_msg=name)
+    assert_sum_close(got[0], O.matmul_bias_bt(x, w, b), np.abs(x) @ np.abs(w).T, what="y")
+    assert_sum_close(got[1], O.linear_grad_x(dy, w), np.abs(dy) @ np.abs(w), what="dx")
+    assert_sum_close(got[2], O.linear_grad_w(dy, x), np.abs(dy).T @ np.abs(x), what="dw")
+
+
 def test_large_products_agree_with_the_register_staged_kernel(device, monkeypatch):
     # A product large enough that the library picks 256 x 128 tiles by itself (K >= 1024 and
     # two such tiles per CU) must equal the register-staged kernel's result bit for bit, for
