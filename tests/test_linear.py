@@ -264,7 +264,9 @@ def test_batched_projections_share_an_operand(device, dtype, rtol, M, d):
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 384, 512), (200, 136, 256), (128, 64, 4096), (520, 264, 320), (64, 1000, 32),
-                                   (2048, 512, 1024)])
+                                   (2048, 512, 1024),
+                                   # 1024 output tiles: more than the resident workgroups, each walks two
+                                   (4096, 4096, 64)])
 def test_f32_tile_staging_variants_agree(device, monkeypatch, M, N, K):
     # fp32 products have a register-staged kernel and one whose tiles are copied straight into
     # LDS (K a multiple of 32); same tiles and k order, so the results must be identical bits
