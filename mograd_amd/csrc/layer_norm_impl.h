@@ -147,29 +147,38 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
   // With narrow per-thread tiles the next row is fetched while this row is reduced;
   // wide tiles would spill, and rely on other resident workgroups to cover the latency.
   constexpr bool PREFETCH = VPT * VEC <= 8;
+  // Rows that several waves share reduce through LDS with workgroup barriers, so when such
+  // rows sit side by side in a workgroup every one of them makes every trip of the loop; a
+  // row slot past the end of the group works on zeros and touches no memory.
+  constexpr bool LOCKSTEP = TPR > kWave && RPW > 1;
   RowTile<T, VEC, TPR, VPT> xv, dyv, xn, dyn;
   int64_t row = r_begin + sub;
   if (PREFETCH && row < r_end) {
     xv.load(x + row * cols, t, cols);
     dyv.load(dy + row * cols, t, cols);
   }
-  for (; row < r_end; row += RPW) {
+  for (; LOCKSTEP ? row - sub < r_end : row < r_end; row += RPW) {
+    const bool active = !LOCKSTEP || row < r_end;
+    if (LOCKSTEP && !active) {
+      xv.zero();
+      dyv.zero();
+    }
     const int64_t next = row + RPW;
     if constexpr (PREFETCH) {
       if (next < r_end) {
         xn.load(x + next * cols, t, cols);
         dyn.load(dy + next * cols, t, cols);
       }
-    } else {
+    } else if (active) {
       xv.load(x + row * cols, t, cols);
       dyv.load(dy + row * cols, t, cols);
     }
     float mu, rstd;
     if constexpr (HAS_STATS) {
-      mu = mean_in[row];
-      rstd = rstd_in[row];
+      mu = active ? mean_in[row] : 0.f;
+      rstd = active ? rstd_in[row] : 0.f;
     } else {
-      const float shift = to_float(x[row * cols]);
+      const float shift = active ? to_float(x[row * cols]) : 0.f;
       row_stats<T, VEC, TPR, VPT, WG>(xv, shift, t, cols, eps, slots, phase, mu, rstd);
     }
     // xhat replaces x; dy*gamma is formed on the fly.  Columns past `cols` hold zeros in
@@ -200,7 +209,7 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
         acc_g.v[i][e] += d * xhat;
         acc_b.v[i][e] += d;
       }
-      if (c < cols) {
+      if (c < cols && active) {
         if (residual != nullptr) {
           // dx = round(gradient) + residual: bit for bit what a separate add of the stored
           // gradient gives.  `residual` may be `dx` itself (each element is read, then written,
@@ -437,6 +446,17 @@ struct LayerNormOps {
   static int launch_bwd(const T* dy, const T* x, const T* gamma, const float* mean, const float* rstd,
                         const T* residual, T* dx, T* dgamma, T* dbeta, int64_t rows, int64_t cols, float eps,
                         hipStream_t stream) {
+    if constexpr (TPR == 512 && VPT * VEC <= 8 && WG_ == 0) {
+      // Rows of 512 threads in pairs, one 1024-thread workgroup per CU instead of two of 512:
+      // as many rows in flight, half as many partial dgamma/dbeta sums to write and read back
+      // ((2048, 4096) fp32: 34.0 -> 32.5 us, (1024, 4096): 18.8 -> 15.8 us).  Only for tiles of
+      // up to 8 values per thread: wider ones do not fit the registers of a 1024-thread
+      // workgroup (16 values: 2 % slower, 32 values: spills, 4x slower).
+      // MOGRAD_HIP_LN_WIDE_PAIR=0 keeps single rows.
+      if (rows >= 4 * static_cast<int64_t>(device_info().cu_count) && env_int("MOGRAD_HIP_LN_WIDE_PAIR", 1) != 0)
+        return launch_bwd<VEC, TPR, VPT, HAS_STATS, 1024>(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows,
+                                                          cols, eps, stream);
+    }
     if constexpr (TPR == 64 && WG_ == 0) {
       const int64_t tall = static_cast<int64_t>(device_info().cu_count) * env_int("MOGRAD_HIP_LN_TALL_ROWS_PER_CU", 16);
       if (rows >= tall)

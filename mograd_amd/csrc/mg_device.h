@@ -189,4 +189,30 @@ __device__ __forceinline__ void block_allreduce(float (&v)[K], float* slots, int
   }
 }
 
+// The same over groups of GW consecutive waves (a row shared by part of the workgroup): every
+// wave publishes its sums, one barrier for the whole workgroup, every thread adds up the GW
+// slots of its own group.  All waves of the workgroup must call it together.
+template <typename Op, int NW, int GW, int K>
+__device__ __forceinline__ void group_allreduce(float (&v)[K], float* slots, int phase) {
+  static_assert(NW % GW == 0, "whole groups");
+#pragma unroll
+  for (int k = 0; k < K; ++k) v[k] = wave_allreduce<Op>(v[k]);
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  float* base = slots + phase * (K * NW);
+  if (lane == 0) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) base[k * NW + wave] = v[k];
+  }
+  __syncthreads();
+  const int first = wave / GW * GW;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    float acc = base[k * NW + first];
+#pragma unroll
+    for (int w = 1; w < GW; ++w) acc = Op::apply(acc, base[k * NW + first + w]);
+    v[k] = acc;
+  }
+}
+
 }  // namespace mg

@@ -63,8 +63,8 @@ struct RowTile {
   }
 };
 
-// Reduction over the TPR threads that share a row: wave-only when TPR == 64, otherwise
-// the whole workgroup (TPR == WG).
+// Reduction over the TPR threads that share a row: wave-only when TPR == 64, the whole
+// workgroup when TPR == WG, otherwise TPR / 64 consecutive waves of it.
 // Position of a thread among the TPR threads of its row, and which of the WG/TPR row
 // slots of the workgroup it serves.  With one row per workgroup the slot is the constant
 // 0, which keeps row addresses wave-uniform (scalar registers).
@@ -84,9 +84,11 @@ __device__ __forceinline__ void row_allreduce_sum(float (&v)[K], float* slots, i
   if constexpr (TPR == kWave) {
 #pragma unroll
     for (int k = 0; k < K; ++k) v[k] = wave_sum(v[k]);
-  } else {
-    static_assert(TPR == WG, "a row is shared by one wave or by the whole workgroup");
+  } else if constexpr (TPR == WG) {
     block_allreduce<SumOp, WG / kWave, K>(v, slots, phase);
+    phase ^= 1;
+  } else {
+    group_allreduce<SumOp, WG / kWave, TPR / kWave, K>(v, slots, phase);
     phase ^= 1;
   }
 }

@@ -61,6 +61,9 @@ def test_bwd_goldens(device, g):
 SHAPES = [
     (1, 4), (3, 7), (5, 65), (33, 130), (64, 384), (16, 1000), (9, 1024), (17, 2048), (6, 4096), (5, 8192),
     (3, 16384), (2, 20000), (4, 1023), (2, 40000), (300, 96), (1, 50000),
+    # tall and wide: the backward pairs 512-thread rows in 1024-thread workgroups (odd row
+    # counts leave a row slot without a row at the end of a group)
+    (1027, 4096), (1025, 3000), (1031, 8192),
 ]
 
 
@@ -149,7 +152,7 @@ def test_saved_statistics_path(device):
 
 
 @pytest.mark.parametrize("dtype", [F32, F16, BF16])
-@pytest.mark.parametrize("rows,cols", [(64, 384), (9, 1000), (33, 4096), (5, 16384), (3, 40000), (7, 129)])
+@pytest.mark.parametrize("rows,cols", [(64, 384), (9, 1000), (33, 4096), (5, 16384), (3, 40000), (7, 129), (1027, 4096)])
 def test_backward_added_to_a_residual_equals_separate_calls(device, dtype, rows, cols):
     # mg_layer_norm_bwd_stats_add: bit for bit mg_layer_norm_bwd_stats followed by mg_add, with
     # the residual in its own buffer and with the residual being dx itself (accumulation in
