@@ -449,7 +449,8 @@ struct LayerNormOps {
     if constexpr (TPR == 512 && VPT * VEC <= 8 && WG_ == 0) {
       // Rows of 512 threads in pairs, one 1024-thread workgroup per CU instead of two of 512:
       // as many rows in flight, half as many partial dgamma/dbeta sums to write and read back
-      // ((2048, 4096) fp32: 34.0 -> 32.5 us, (1024, 4096): 18.8 -> 15.8 us).  Only for tiles of
+      // ((2048, 4096) fp32: 25.2 -> 23.5 us on cached inputs, 1-4 % on cold ones; (1024, 4096):
+      // 18.8 -> 15.8 us).  Only for tiles of
       // up to 8 values per thread: wider ones do not fit the registers of a 1024-thread
       // workgroup (16 values: 2 % slower, 32 values: spills, 4x slower).
       // MOGRAD_HIP_LN_WIDE_PAIR=0 keeps single rows.
