@@ -127,7 +127,7 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
   constexpr int RPW = WG / TPR;
   constexpr int NW = WG / kWave;
   constexpr int TILE_COLS = VPT * TPR * VEC;
-  __shared__ float slots[2 * 2 * NW];
+  __shared__ float slots[2 * 4 * NW];
   // Only used to combine the RPW row slots of one workgroup at the end.
   __shared__ float combine[RPW > 1 ? RPW * TILE_COLS : 1];
 
@@ -173,30 +173,58 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
       xv.load(x + row * cols, t, cols);
       dyv.load(dy + row * cols, t, cols);
     }
-    float mu, rstd;
+    float mu, rstd, c1, c2;
     if constexpr (HAS_STATS) {
       mu = active ? mean_in[row] : 0.f;
       rstd = active ? rstd_in[row] : 0.f;
+      // xhat replaces x; dy*gamma is formed on the fly.  Columns past `cols` hold zeros in
+      // dy and gamma, so they add nothing to the sums.
+      float s[2] = {0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < VPT; ++i)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float xhat = (xv.v[i][e] - mu) * rstd;
+          const float dyg = dyv.v[i][e] * g.v[i][e];
+          xv.v[i][e] = xhat;
+          s[0] += dyg;
+          s[1] += dyg * xhat;
+        }
+      row_allreduce_sum<TPR, WG, 2>(s, slots, phase);
+      c1 = s[0] * inv_n;
+      c2 = s[1] * inv_n;
     } else {
+      // One reduction per row instead of two: with d = x - shift (the shift is the row's
+      // first element, see row_stats) the four sums of d, d^2, dy*gamma and dy*gamma*d give
+      // the statistics and, through xhat = (d - mean_d) * rstd, both row sums of the gradient.
       const float shift = active ? to_float(x[row * cols]) : 0.f;
-      row_stats<T, VEC, TPR, VPT, WG>(xv, shift, t, cols, eps, slots, phase, mu, rstd);
-    }
-    // xhat replaces x; dy*gamma is formed on the fly.  Columns past `cols` hold zeros in
-    // dy and gamma, so they add nothing to the sums.
-    float s[2] = {0.f, 0.f};
+      float s[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < VPT; ++i)
+      for (int i = 0; i < VPT; ++i) {
+        const bool in_row = RowTile<T, VEC, TPR, VPT>::col(i, t) < cols;
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        const float xhat = (xv.v[i][e] - mu) * rstd;
-        const float dyg = dyv.v[i][e] * g.v[i][e];
-        xv.v[i][e] = xhat;
-        s[0] += dyg;
-        s[1] += dyg * xhat;
+        for (int e = 0; e < VEC; ++e) {
+          const float d = in_row ? xv.v[i][e] - shift : 0.f;
+          const float dyg = dyv.v[i][e] * g.v[i][e];
+          xv.v[i][e] = d;
+          s[0] += d;
+          s[1] += d * d;
+          s[2] += dyg;
+          s[3] += dyg * d;
+        }
       }
-    row_allreduce_sum<TPR, WG, 2>(s, slots, phase);
-    const float c1 = s[0] * inv_n;
-    const float c2 = s[1] * inv_n;
+      row_allreduce_sum<TPR, WG, 4>(s, slots, phase);
+      const float md = s[0] * inv_n;
+      const float var = fmaxf(s[1] * inv_n - md * md, 0.f);
+      mu = shift + md;
+      rstd = rsqrtf(var + eps);
+      c1 = s[2] * inv_n;
+      c2 = rstd * (s[3] - md * s[2]) * inv_n;
+#pragma unroll
+      for (int i = 0; i < VPT; ++i)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) xv.v[i][e] = (xv.v[i][e] - md) * rstd;  // xhat
+    }
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
       const int c = RowTile<T, VEC, TPR, VPT>::col(i, t);
