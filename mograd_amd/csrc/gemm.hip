@@ -45,16 +45,50 @@ static int launch_f32_mfma(const GemmArgs& g, hipStream_t stream) {
   // Tiles copied straight into LDS (gemm_f32_pipe_kernel, same results bit for bit) when K is a
   // multiple of the 32-deep step; MOGRAD_HIP_GEMM_F32_PIPE=0 keeps the register-staged kernel.
   if (g.K % kGemmBK == 0 && env_int("MOGRAD_HIP_GEMM_F32_PIPE", 1) != 0) {
+    const int M = static_cast<int>(g.M), N = static_cast<int>(g.N), K = static_cast<int>(g.K);
+    const int batches = static_cast<int>(g.batch);
+    // An output with fewer tiles than CUs (a 10-class head: 2048 x 10 from K = 4096 is 16
+    // tiles) is split along K so that the device is filled; the partial tiles are summed in a
+    // fixed order by the same reduction the 16-bit path uses.
+    const int64_t cus = device_info().cu_count;
+    int splits = 1;
+    if (blocks < cus && g.K >= 1024) {
+      splits = static_cast<int>(ceil_div(env_int("MOGRAD_HIP_GEMM_SPLITK_WG_PER_CU", 2) * cus, blocks));
+      const int max_splits = static_cast<int>(g.K / env_int("MOGRAD_HIP_GEMM_SPLITK_MIN_K", 256));
+      if (splits > max_splits) splits = max_splits;
+      if (splits > 64) splits = 64;
+    }
+    if (splits > 1) {
+      const int k_per_split = static_cast<int>(ceil_div(ceil_div(g.K, splits), kGemmBK) * kGemmBK);
+      splits = static_cast<int>(ceil_div(g.K, k_per_split));
+      const int64_t numel = g.batch * g.M * g.N;
+      Scratch partial;
+      MG_TRY(partial.take(static_cast<int64_t>(splits) * numel * static_cast<int64_t>(sizeof(float))));
+      const int64_t work = blocks * splits;
+      hipLaunchKernelGGL((gemm_f32_pipe_kernel<A_KC, B_KC, false, true>), dim3(static_cast<unsigned>(work)),
+                         dim3(kGemmThreads), 0, stream, a, b, bias, c, partial.as<float>(), M, N, K, lda, ldb, g.N, g.bsa,
+                         g.bsb, g.M * g.N, tiles_m, tiles_n, batches, k_per_split, static_cast<int>(work),
+                         GemmEpilogue<float>{nullptr, nullptr, 0});
+      MG_LAUNCH_CHECK();
+      const unsigned rblocks = static_cast<unsigned>(ceil_div(numel, 256));
+      if (bias)
+        hipLaunchKernelGGL((gemm_splitk_reduce_kernel<float, true>), dim3(rblocks), dim3(256), 0, stream,
+                           partial.as<float>(), bias, c, numel, splits, N, epilogue_of<float>(g));
+      else
+        hipLaunchKernelGGL((gemm_splitk_reduce_kernel<float, false>), dim3(rblocks), dim3(256), 0, stream,
+                           partial.as<float>(), bias, c, numel, splits, N, epilogue_of<float>(g));
+      MG_LAUNCH_CHECK();
+      return MG_OK;
+    }
+    float* no_partial = nullptr;
     if (bias)
-      hipLaunchKernelGGL((gemm_f32_pipe_kernel<A_KC, B_KC, true>), dim3(static_cast<unsigned>(grid)),
-                         dim3(kGemmThreads), 0, stream, a, b, bias, c, static_cast<int>(g.M), static_cast<int>(g.N),
-                         static_cast<int>(g.K), lda, ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n,
-                         static_cast<int>(blocks), epilogue_of<float>(g));
+      hipLaunchKernelGGL((gemm_f32_pipe_kernel<A_KC, B_KC, true, false>), dim3(static_cast<unsigned>(grid)),
+                         dim3(kGemmThreads), 0, stream, a, b, bias, c, no_partial, M, N, K, lda, ldb, g.N, g.bsa, g.bsb,
+                         g.M * g.N, tiles_m, tiles_n, batches, K, static_cast<int>(blocks), epilogue_of<float>(g));
     else
-      hipLaunchKernelGGL((gemm_f32_pipe_kernel<A_KC, B_KC, false>), dim3(static_cast<unsigned>(grid)),
-                         dim3(kGemmThreads), 0, stream, a, b, bias, c, static_cast<int>(g.M), static_cast<int>(g.N),
-                         static_cast<int>(g.K), lda, ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n,
-                         static_cast<int>(blocks), epilogue_of<float>(g));
+      hipLaunchKernelGGL((gemm_f32_pipe_kernel<A_KC, B_KC, false, false>), dim3(static_cast<unsigned>(grid)),
+                         dim3(kGemmThreads), 0, stream, a, b, bias, c, no_partial, M, N, K, lda, ldb, g.N, g.bsa, g.bsb,
+                         g.M * g.N, tiles_m, tiles_n, batches, K, static_cast<int>(blocks), epilogue_of<float>(g));
     MG_LAUNCH_CHECK();
     return MG_OK;
   }
@@ -231,7 +265,8 @@ static int launch_generic(const GemmArgs& g, hipStream_t stream) {
   return MG_OK;
 }
 
-int gemm_dispatch(const char* who, const GemmArgs& g, hipStream_t stream) {
+int gemm_dispatch(const char* who, const GemmArgs& g_in, hipStream_t stream) {
+  const GemmArgs& g = g_in;
   if (!is_float_dtype(g.dtype)) return fail(MG_ERR_INVALID, "%s: unsupported dtype %s", who, dtype_name(g.dtype));
   if (g.batch < 0 || g.M < 0 || g.N < 0 || g.K < 0 || g.M > 0x7fffffffLL || g.N > 0x7fffffffLL || g.K > 0x7fffffffLL)
     return fail(MG_ERR_INVALID, "%s: bad shape batch=%lld M=%lld N=%lld K=%lld", who, static_cast<long long>(g.batch),
@@ -239,16 +274,37 @@ int gemm_dispatch(const char* who, const GemmArgs& g, hipStream_t stream) {
   if (g.batch == 0 || g.M == 0 || g.N == 0) return MG_OK;
   if (!g.a || !g.b || !g.c) return fail(MG_ERR_INVALID, "%s: null pointer argument", who);
 
-  if (g.dtype == MG_F32 && g.K > 0) {
+  if (g_in.dtype == MG_F32 && g_in.K > 0) {
+    GemmArgs g = g_in;
     // Which dimension of each operand is contiguous, and can it be read 16 bytes at a time?
-    const bool a_kc = g.sak == 1 && mult4(g.sam) && mult4(g.K);
-    const bool a_mc = g.sam == 1 && mult4(g.sak) && mult4(g.M);
-    const bool b_kc = g.sbk == 1 && mult4(g.sbn) && mult4(g.K);
-    const bool b_nc = g.sbn == 1 && mult4(g.sbk) && mult4(g.N);
-    const bool aligned = aligned16(g.a) && aligned16(g.b) && mult4(g.bsa) && mult4(g.bsb);
+    bool a_kc = g.sak == 1 && mult4(g.sam) && mult4(g.K) && mult4(g.bsa) && aligned16(g.a);
+    const bool a_mc = g.sam == 1 && mult4(g.sak) && mult4(g.M) && mult4(g.bsa) && aligned16(g.a);
+    bool b_kc = g.sbk == 1 && mult4(g.sbn) && mult4(g.K) && mult4(g.bsb) && aligned16(g.b);
+    const bool b_nc = g.sbn == 1 && mult4(g.sbk) && mult4(g.N) && mult4(g.bsb) && aligned16(g.b);
     // Tiny problems gain nothing from 128x128 tiles.
-    const bool worth_it = g.M * g.N >= 64 * 64 || g.K >= 512;
-    if (aligned && worth_it && (a_kc || a_mc) && (b_kc || b_nc)) {
+    const bool worth_it = g.M * g.N >= 64 * 64 || g.K >= env_int("MOGRAD_HIP_GEMM_F32_MIN_K", 128);
+    // A thin operand that cannot be read 16 bytes at a time as it lies (the (K, 10) gradient
+    // of a 10-class head, read along its 10-wide rows for dW) is first copied k-contiguous:
+    // at most one tile of rows, so the copy is a small fraction of the other operand's bytes.
+    Scratch a_copy, b_copy;
+    const bool deep = g.K >= 512 && mult4(g.K);
+    if (deep && !(a_kc || a_mc) && g.M <= kGemmBM && (b_kc || b_nc || g.N <= kGemmBN)) {
+      MG_TRY(a_copy.take(g.batch * g.M * g.K * static_cast<int64_t>(sizeof(float))));
+      const int64_t shape[3] = {g.batch, g.M, g.K}, strides[3] = {g.bsa, g.sam, g.sak};
+      MG_TRY(mg_contiguous(g.a, a_copy.as<float>(), 3, shape, strides, MG_F32, stream));
+      g.a = a_copy.as<float>();
+      g.sam = g.K, g.sak = 1, g.bsa = g.M * g.K;
+      a_kc = true;
+    }
+    if (deep && !(b_kc || b_nc) && g.N <= kGemmBN && (a_kc || a_mc)) {
+      MG_TRY(b_copy.take(g.batch * g.N * g.K * static_cast<int64_t>(sizeof(float))));
+      const int64_t shape[3] = {g.batch, g.N, g.K}, strides[3] = {g.bsb, g.sbn, g.sbk};
+      MG_TRY(mg_contiguous(g.b, b_copy.as<float>(), 3, shape, strides, MG_F32, stream));
+      g.b = b_copy.as<float>();
+      g.sbn = g.K, g.sbk = 1, g.bsb = g.N * g.K;
+      b_kc = true;
+    }
+    if (worth_it && (a_kc || a_mc) && (b_kc || b_nc)) {
       if (a_kc && b_kc) return launch_f32_mfma<true, true>(g, stream);
       if (a_kc) return launch_f32_mfma<true, false>(g, stream);
       if (b_kc) return launch_f32_mfma<false, true>(g, stream);

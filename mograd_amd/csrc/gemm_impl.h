@@ -859,11 +859,14 @@ __device__ __forceinline__ void gemm32_pipe_frag(const char* __restrict__ lds_st
   }
 }
 
-template <bool A_KC, bool B_KC, bool HAS_BIAS>
+// SPLIT_K: a work item is (K range, batch, tile); the fp32 partial tiles go to
+// partial[(split * batches + batch), M, N] and gemm_splitk_reduce_kernel adds them up in a
+// fixed order (for outputs with too few tiles to fill the device, e.g. a 10-class head).
+template <bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_pipe_kernel(
     const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias, float* __restrict__ C,
-    int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb, int64_t bsc, int tiles_m,
-    int tiles_n, int total_work, GemmEpilogue<float> ep_in) {
+    float* __restrict__ partial, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb,
+    int64_t bsc, int tiles_m, int tiles_n, int batches, int k_per_split, int total_work, GemmEpilogue<float> ep_in) {
   constexpr int OP = kGemmBM * kGemmBK * 4;  // bytes of one operand's step
   __shared__ __attribute__((aligned(1024))) char lds[2][2][OP];
 
@@ -872,19 +875,22 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_pipe_kernel(
   const int lane = threadIdx.x % kWave;
   const int wm = (wave / 2) * 64;
   const int wn = (wave % 2) * 64;
-  const int steps = K / kGemmBK;
   const int64_t a_step = A_KC ? kGemmBK : kGemmBK * lda;
   const int64_t b_step = B_KC ? kGemmBK : kGemmBK * ldb;
   // The grid holds at most the workgroups that are resident at once; each takes output tiles
   // work, work + gridDim.x, ... (see gemm_f32_mfma_kernel).
   for (int work = blockIdx.x; work < total_work; work += gridDim.x) {
-    const int batch = work / tiles;
+    const int split = SPLIT_K ? work / (tiles * batches) : 0;
+    const int in_split = SPLIT_K ? work % (tiles * batches) : work;
+    const int batch = in_split / tiles;
     int tm, tn;
-    gemm_tile_of_block(work % tiles, tiles_m, tiles_n, tm, tn);
+    gemm_tile_of_block(in_split % tiles, tiles_m, tiles_n, tm, tn);
     const int m0 = tm * kGemmBM;
     const int n0 = tn * kGemmBN;
-    const float* a = A + batch * bsa;
-    const float* b = B + batch * bsb;
+    const int k_begin = SPLIT_K ? split * k_per_split : 0;
+    const int steps = (SPLIT_K ? min(K - k_begin, k_per_split) : K) / kGemmBK;
+    const float* a = A + batch * bsa + (A_KC ? static_cast<int64_t>(k_begin) : k_begin * lda);
+    const float* b = B + batch * bsb + (B_KC ? static_cast<int64_t>(k_begin) : k_begin * ldb);
     float* c = C + batch * bsc;
     GemmEpilogue<float> ep = ep_in;
     if (ep.residual) ep.residual += batch * bsc;
@@ -950,13 +956,17 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_pipe_kernel(
       for (int tj = 0; tj < 2; ++tj) {
         const int col = n0 + wn + tj * 32 + lane % 32;
         if (col >= N) continue;
-        const float bv = HAS_BIAS ? bias[col] : 0.f;
+        const float bv = (HAS_BIAS && !SPLIT_K) ? bias[col] : 0.f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int row = m0 + wm + ti * 32 + (r / 4) * 8 + (lane / 32) * 4 + (r % 4);
           if (row < M) {
-            const int64_t at = static_cast<int64_t>(row) * ldc + col;
-            c[at] = gemm_finish<float>(acc[ti][tj][r] + bv, ep, at);
+            if constexpr (SPLIT_K) {
+              partial[((static_cast<int64_t>(split) * batches + batch) * M + row) * N + col] = acc[ti][tj][r];
+            } else {
+              const int64_t at = static_cast<int64_t>(row) * ldc + col;
+              c[at] = gemm_finish<float>(acc[ti][tj][r] + bv, ep, at);
+            }
           }
         }
       }

@@ -42,7 +42,10 @@ def _linear_all(device, x, w, b, dy, dtype=F32):
 
 
 SHAPES = [(64, 10, 256), (64, 256, 784), (128, 128, 128), (256, 384, 512), (200, 136, 260), (130, 65, 384),
-          (1, 8, 16), (33, 7, 5), (512, 1024, 256), (300, 128, 1000)]
+          (1, 8, 16), (33, 7, 5), (512, 1024, 256), (300, 128, 1000),
+          # a 10-class head behind a wide layer: few output tiles (split along K in fp32) and a
+          # 10-wide gradient that is copied k-contiguous before the tiled kernel reads it
+          (2048, 10, 4096), (1024, 6, 1024), (640, 12, 2080)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
@@ -61,7 +64,7 @@ def test_linear_fwd_and_grads_f32(device, M, N, K):
     assert_sum_close(db, O.linear_grad_b(dy), np.abs(dy).sum(axis=0), what="db")
 
 
-@pytest.mark.parametrize("M,N,K", [(128, 256, 512), (200, 136, 260), (64, 10, 256)])
+@pytest.mark.parametrize("M,N,K", [(128, 256, 512), (200, 136, 260), (64, 10, 256), (2048, 10, 4096), (1024, 6, 512)])
 def test_linear_bwd_entry(device, M, N, K):
     x, w, dy = normal(41, 0, (M, K)), normal(41, 1, (N, K)), normal(41, 2, (M, N))
     bx, bw, bdy = (AnyBuffer.from_numpy(device, a) for a in (x, w, dy))
@@ -82,6 +85,26 @@ def test_batched_rank3_and_broadcast_weight(device):
                [(x, Layout(Bt, T, K)), (w, Layout(Bt, N, K, strides=(0, K, 1)))])
     assert_sum_close(out, np.einsum("btk,nk->btn", x.astype(np.float64), w), 
                      np.einsum("btk,nk->btn", np.abs(x), np.abs(w)), what="batched")
+
+
+def test_batched_thin_products_f32(device):
+    # three (T, K) x (K, 10) products and their transposed-operand gradients in one call each:
+    # the split along K and the k-contiguous copy both carry the batch index
+    Bt, T, K, N = 3, 256, 2048, 10
+    x, w, dy = normal(43, 0, (Bt, T, K)), normal(43, 1, (Bt, N, K)), normal(43, 2, (Bt, T, N))
+    y = _run(device, "MATMUL_BT", Layout(Bt, T, N), [(x, Layout(Bt, T, K)), (w, Layout(Bt, N, K))])
+    assert_sum_close(y, np.einsum("btk,bnk->btn", x.astype(np.float64), w),
+                     np.einsum("btk,bnk->btn", np.abs(x), np.abs(w)), what="y")
+    # dW^T = X^T dY per batch: the (T, 10) right operand is read along T
+    dwt = _run(device, "MATMUL", Layout(Bt, K, N),
+               [(x, Layout(Bt, K, T, strides=(T * K, 1, K))), (dy, Layout(Bt, T, N))])
+    assert_sum_close(dwt, np.einsum("btk,btn->bkn", x.astype(np.float64), dy),
+                     np.einsum("btk,btn->bkn", np.abs(x), np.abs(dy)), what="dwt")
+    # dW = dY^T X per batch: the (10, T) left operand is the transposed view of dY
+    dw = _run(device, "MATMUL", Layout(Bt, N, K),
+              [(dy, Layout(Bt, N, T, strides=(T * N, 1, N))), (x, Layout(Bt, T, K))])
+    assert_sum_close(dw, np.einsum("btn,btk->bnk", dy.astype(np.float64), x),
+                     np.einsum("btn,btk->bnk", np.abs(dy), np.abs(x)), what="dw")
 
 
 def test_mlp_chain_matches_oracle(device):
@@ -275,12 +298,17 @@ def test_f32_tile_staging_variants_agree(device, monkeypatch, M, N, K):
     w = normal(59, 1, (N, K), std=0.05)
     b = normal(59, 2, (N,), std=0.1)
     dy = normal(59, 3, (M, N), std=0.5)
+    # (an output of few tiles would be split along K, which changes the order of the sums:
+    # switched off for the bitwise comparison, on again for the comparison with the oracle)
+    monkeypatch.setenv("MOGRAD_HIP_GEMM_SPLITK_MIN_K", str(1 << 30))
     monkeypatch.setenv("MOGRAD_HIP_GEMM_F32_PIPE", "0")
     base = _linear_all(device, x, w, b, dy)
     monkeypatch.delenv("MOGRAD_HIP_GEMM_F32_PIPE")
     got = _linear_all(device, x, w, b, dy)
     for g, want, name in zip(got, base, ("y", "dx", "dw", "db")):
         np.testing.assert_array_equal(g, want, err_msg=name)
+    monkeypatch.delenv("MOGRAD_HIP_GEMM_SPLITK_MIN_K")
+    got = _linear_all(device, x, w, b, dy)
     assert_sum_close(got[0], O.matmul_bias_bt(x, w, b), np.abs(x) @ np.abs(w).T, what="y")
     assert_sum_close(got[1], O.linear_grad_x(dy, w), np.abs(dy) @ np.abs(w), what="dx")
     assert_sum_close(got[2], O.linear_grad_w(dy, x), np.abs(dy).T @ np.abs(x), what="dw")
@@ -336,7 +364,7 @@ def test_batched_projections_tile_staging_variants(device, monkeypatch, variant)
 # ---- fused epilogues: each must give exactly what the separate calls give -----------------
 
 FUSED_SHAPES = [(256, 384, 512), (200, 136, 264), (130, 65, 384), (64, 10, 256), (33, 7, 5), (4096, 128, 128),
-                (128, 64, 4096)]
+                (128, 64, 4096), (256, 10, 2048)]
 
 
 def _ptr(b):
