@@ -43,6 +43,35 @@ def test_random_linear_shapes(device):
             assert_close(got, want, rt, rt * max(np.abs(want).max(), 1e-3), f"case {case} {(M, N, K)} dtype {dtype} {name}")
 
 
+def test_random_thin_f32_products(device):
+    # fp32 heads of a few classes behind wide layers: the forward has fewer output tiles than
+    # the device has CUs (split along K when K is a multiple of 32 and at least 1024), and
+    # dW = dY^T X reads the (M, N) gradient along its N-wide rows (copied k-contiguous when
+    # M is a multiple of 4 and at least 512); neighbouring shapes take the other paths
+    rng = np.random.Generator(np.random.PCG64(95_300))
+    lib, st = device.lib, device.stream
+    for case in range(16):
+        N = int(rng.integers(1, 21))
+        M = int(rng.integers(128, 513)) * 4 if case % 4 != 3 else int(rng.integers(500, 2050))
+        K = int(rng.integers(8, 97)) * 32 if case % 4 != 2 else int(rng.integers(256, 3000))
+        x = rng.standard_normal((M, K)).astype(np.float32)
+        w = (rng.standard_normal((N, K)) * 0.1).astype(np.float32)
+        b = rng.standard_normal(N).astype(np.float32)
+        dy = rng.standard_normal((M, N)).astype(np.float32)
+        bx, bw, bb, bdy = (AnyBuffer.from_numpy(device, a, F32) for a in (x, w, b, dy))
+        y, dx, dw, db = (AnyBuffer.create(F32, device, n) for n in (M * N, M * K, N * K, N))
+        lib.mg_matmul_bias_bt(bx.data_ptr(), bw.data_ptr(), bb.data_ptr(), y.data_ptr(), 1, M, N, K, K, 1, K, 1, M * K,
+                              N * K, F32, st)
+        lib.mg_linear_bwd(bdy.data_ptr(), bx.data_ptr(), bw.data_ptr(), dx.data_ptr(), dw.data_ptr(), db.data_ptr(), M, N,
+                          K, F32, st)
+        rt = RT[F32]
+        for got, want, name in ((y.to_numpy((M, N)), O.matmul_bias_bt(x, w, b), "y"),
+                                (dx.to_numpy((M, K)), O.linear_grad_x(dy, w), "dx"),
+                                (dw.to_numpy((N, K)), O.linear_grad_w(dy, x), "dw"),
+                                (db.to_numpy(), O.linear_grad_b(dy), "db")):
+            assert_close(got, want, rt, rt * max(np.abs(want).max(), 1e-3), f"case {case} {(M, N, K)} {name}")
+
+
 def test_random_16bit_tile_staging_shapes(device, monkeypatch):
     # Shapes the LDS-copy GEMM kernels take (extents multiples of 8, K a multiple of 64), with
     # padded leading dimensions and batches, through every forced variant: all must equal the
