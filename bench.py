@@ -41,9 +41,9 @@ CE_FUSED_BYTES = 2 * CE_ROWS * CE_COLS * 4 + CE_ROWS * 4 + 4          # logits, 
 
 # HBM bytes per launch of the cross-entropy rows kernel, from two `rocprofv3 --pmc` runs
 # (FETCH_SIZE, then WRITE_SIZE) of this same script, each scaled by what the counter reads
-# for the calibration copy below: (805943.2 / 0.50005 + 1610376.8 / 1.0) KiB.  The counter
+# for the calibration copy below: (805943.9 / 0.50005 + 1610378.9 / 1.0) KiB.  The counter
 # runs and the factors are in profiles/ce_rows_kernel_8192x50304_hbm_traffic.md.
-CE_MEASURED_TRAFFIC_BYTES = int((805943.2 / 0.50005 + 1610376.8) * 1024)
+CE_MEASURED_TRAFFIC_BYTES = int((805943.9 / 0.50005 + 1610378.9) * 1024)
 
 
 def _rng(config: int, tensor: int) -> np.random.Generator:
