@@ -61,6 +61,70 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict
   }
 }
 
+// One-launch form for wide matrices: a 1024-thread workgroup owns a 128-byte-wide slab of
+// columns (eight 16-byte pieces) for every row, 128 row lanes deep, so a wave's load reads
+// eight whole 128-byte lines and nothing a workgroup fetches is shared with another.  Each
+// thread sums every 128th row with eight loads in flight; the 128 row lanes are then added
+// through LDS in a fixed order and the result is stored directly: no partial sums in
+// memory, no second launch, no atomics.
+template <typename T, int VEC>
+__global__ __launch_bounds__(1024) void colsum_slab_kernel(const T* __restrict__ a, T* __restrict__ dst,
+                                                           int64_t reduce, int64_t inner) {
+  constexpr int PIECES = 8;             // 16-byte pieces per slab row
+  constexpr int LANES = 1024 / PIECES;  // row lanes
+  constexpr int NCOL = PIECES * VEC;    // columns of a slab
+  constexpr int SL = 1024 / NCOL;       // row-lane groups in the first LDS pass
+  __shared__ float tile[LANES][NCOL + 1];
+  __shared__ float tile2[SL][NCOL + 1];
+  const int cx = threadIdx.x % PIECES;
+  const int ly = threadIdx.x / PIECES;
+  const int64_t col = (static_cast<int64_t>(blockIdx.x) * PIECES + cx) * VEC;
+  const int64_t o = blockIdx.y;
+  float acc[4][VEC];
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[u][e] = 0.f;
+  if (col < inner) {
+    const int64_t step = static_cast<int64_t>(LANES) * inner;
+    const T* p = a + (o * reduce + ly) * inner + col;
+    int64_t r = ly;
+    for (; r + 7 * LANES < reduce; r += 8 * LANES, p += 8 * step) {
+      float v[8][VEC];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) VecIO<T, VEC>::load(p + u * step, v[u]);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[u & 3][e] += v[u][e];
+    }
+    for (; r < reduce; r += LANES, p += step) {
+      float v[VEC];
+      VecIO<T, VEC>::load(p, v);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[0][e] += v[e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) tile[ly][cx * VEC + e] = (acc[0][e] + acc[1][e]) + (acc[2][e] + acc[3][e]);
+  __syncthreads();
+  {
+    const int c = threadIdx.x % NCOL, s = threadIdx.x / NCOL;
+    float t = 0.f;
+#pragma unroll
+    for (int k = 0; k < LANES / SL; ++k) t += tile[s * (LANES / SL) + k][c];
+    tile2[s][c] = t;
+  }
+  __syncthreads();
+  if (threadIdx.x < NCOL) {
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * NCOL + threadIdx.x;
+    float t = 0.f;
+#pragma unroll
+    for (int s = 0; s < SL; ++s) t += tile2[s][threadIdx.x];
+    if (c < inner) dst[o * inner + c] = from_float<T>(t);
+  }
+}
+
 // Sum over the last axis (inner == 1): one wave per output element.
 template <typename T>
 __global__ __launch_bounds__(256) void rowsum_kernel(const T* __restrict__ a, T* __restrict__ dst, int64_t outer,
@@ -109,6 +173,21 @@ static int colsum_typed(const T* a, T* dst, int64_t outer, int64_t reduce, int64
   constexpr int WIDE = WideVec<T>::value;
   const bool wide = inner % WIDE == 0 && aligned16(a) && aligned16(dst);
   const int vec = wide ? WIDE : 1;
+  // Wide matrices take the one-launch kernel: always when there is a 128-byte column slab
+  // for every CU; with slabs for half the CUs only up to 48 MiB of input (half the CUs
+  // stream about 4 TB/s against 5 for the two-stage form on all of them, which outweighs
+  // the saved launch beyond roughly 40 MB).
+  const int64_t slabs = ceil_div(inner, 8 * WIDE) * outer;
+  const int64_t cus = device_info().cu_count;
+  const bool slab_fits = slabs >= cus || (2 * slabs >= cus && outer * reduce * inner * static_cast<int64_t>(sizeof(T)) <=
+                                                                   (int64_t{48} << 20));
+  if (wide && outer <= 65535 && reduce >= 128 && slab_fits && env_int("MOGRAD_HIP_COLSUM_SLAB", 1) != 0) {
+    hipLaunchKernelGGL((colsum_slab_kernel<T, WIDE>),
+                       dim3(static_cast<unsigned>(ceil_div(inner, 8 * WIDE)), static_cast<unsigned>(outer)), dim3(1024),
+                       0, stream, a, dst, reduce, inner);
+    MG_LAUNCH_CHECK();
+    return MG_OK;
+  }
   // Column threads per workgroup: the smallest power of two covering the columns, at most 256.
   int tx_log2 = 3;
   while (tx_log2 < 8 && (int64_t{1} << tx_log2) * vec < inner) ++tx_log2;

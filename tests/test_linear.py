@@ -175,6 +175,27 @@ def test_sum_axis_shapes(device):
         assert_sum_close(got, a.astype(np.float64).sum(axis=axis), np.abs(a).sum(axis=axis), what=f"sum{shape}/{axis}")
 
 
+def test_sum_axis_wide_one_launch(device):
+    # Wide matrices (at least 128 column slabs of 128 bytes) are summed by one launch, a
+    # workgroup per slab: ragged row counts, a ragged last slab, a batch of two, an exact
+    # integer sum, and the same column sums whatever the slab kernel's row order.
+    for shape, axis in [((1000, 4100), 0), ((129, 8200), 0), ((2, 300, 4096), 1), ((2048, 4096), 0)]:
+        a = normal(48, len(shape) * 10 + axis + shape[-1] % 7, shape)
+        out_shape = tuple(s for i, s in enumerate(shape) if i != axis)
+        got = _run(device, "SUM", Layout(*out_shape), [(a, Layout(*shape))], F32, {"axis": axis})
+        assert_sum_close(got, a.astype(np.float64).sum(axis=axis), np.abs(a).sum(axis=axis), what=f"sum{shape}/{axis}")
+    # small integers: every partial sum is exact in fp32, so the result is the integer sum
+    rows, cols = 1153, 4128
+    a = (np.arange(rows * cols, dtype=np.int64).reshape(rows, cols) * 7919 % 17 - 8).astype(np.float32)
+    got = _run(device, "SUM", Layout(cols), [(a, Layout(rows, cols))], F32, {"axis": 0})
+    np.testing.assert_array_equal(got, a.astype(np.int64).sum(axis=0).astype(np.float32))
+    for dtype, rtol in ((F16, 2e-3), (BF16, 1.6e-2)):
+        a = round_to_dtype(normal(48, 5, (1031, 8200)), dtype)
+        got = _run(device, "SUM", Layout(8200), [(a, Layout(1031, 8200))], dtype, {"axis": 0})
+        want = a.astype(np.float64).sum(axis=0)
+        assert_close(got, want, rtol, rtol * np.abs(want).max(), f"sum 16-bit {dtype}")
+
+
 def test_relu_grad(device):
     for n in (1, 7, 4096, 100003):
         out = np.maximum(normal(45, n % 97, (n,)), 0)
