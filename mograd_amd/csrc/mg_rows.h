@@ -133,6 +133,61 @@ __global__ __launch_bounds__(256) void reduce_partials_cw_kernel(const float* __
   if (sy == 0 && c < cols) out[c] = from_float<T>(tile[0][cx]);
 }
 
+// The same sum for wide outputs with many groups: a 1024-thread workgroup owns 32 columns
+// (one 128-byte line of the fp32 partials) and reads them as 16-byte pieces, eight pieces
+// by 128 group lanes, so that a few hundred groups are in flight at once instead of being
+// walked four at a time; the group lanes are then added through LDS in a fixed order.
+// Needs cols % 4 == 0 and 16-byte aligned partials.
+template <typename T>
+__global__ __launch_bounds__(1024) void reduce_partials_slab_kernel(const float* __restrict__ part0, T* __restrict__ out0,
+                                                                    const float* __restrict__ part1, T* __restrict__ out1,
+                                                                    int64_t groups, int64_t cols) {
+  constexpr int LANES = 128, NCOL = 32, SL = 32;
+  __shared__ float tile[LANES][NCOL + 1];
+  __shared__ float tile2[SL][NCOL + 1];
+  const float* part = blockIdx.y == 0 ? part0 : part1;
+  T* out = blockIdx.y == 0 ? out0 : out1;
+  const int cx = threadIdx.x % 8;
+  const int ly = threadIdx.x / 8;
+  const int64_t col = (static_cast<int64_t>(blockIdx.x) * 8 + cx) * 4;
+  float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0;
+  if (col < cols) {
+    const float* p = part + ly * cols + col;
+    const int64_t step = LANES * cols;
+    int64_t g = ly;
+    for (; g + LANES < groups; g += 2 * LANES, p += 2 * step) {
+      const float4 v0 = *reinterpret_cast<const float4*>(p);
+      const float4 v1 = *reinterpret_cast<const float4*>(p + step);
+      a0.x += v0.x; a0.y += v0.y; a0.z += v0.z; a0.w += v0.w;
+      a1.x += v1.x; a1.y += v1.y; a1.z += v1.z; a1.w += v1.w;
+    }
+    if (g < groups) {
+      const float4 v0 = *reinterpret_cast<const float4*>(p);
+      a0.x += v0.x; a0.y += v0.y; a0.z += v0.z; a0.w += v0.w;
+    }
+  }
+  tile[ly][cx * 4 + 0] = a0.x + a1.x;
+  tile[ly][cx * 4 + 1] = a0.y + a1.y;
+  tile[ly][cx * 4 + 2] = a0.z + a1.z;
+  tile[ly][cx * 4 + 3] = a0.w + a1.w;
+  __syncthreads();
+  {
+    const int c = threadIdx.x % NCOL, sl = threadIdx.x / NCOL;
+    float t = 0.f;
+#pragma unroll
+    for (int k = 0; k < LANES / SL; ++k) t += tile[sl * (LANES / SL) + k][c];
+    tile2[sl][c] = t;
+  }
+  __syncthreads();
+  if (threadIdx.x < NCOL) {
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * NCOL + threadIdx.x;
+    float t = 0.f;
+#pragma unroll
+    for (int sl = 0; sl < SL; ++sl) t += tile2[sl][threadIdx.x];
+    if (c < cols) out[c] = from_float<T>(t);
+  }
+}
+
 // Launches the reduction of one or two (groups, cols) partial arrays.  Wide outputs use 64
 // columns x 4 slices per workgroup; narrower ones 32 x 8 (a workgroup still reads whole
 // 128-byte lines of the fp32 partials: with 64-byte pieces the two workgroups that share a
@@ -143,7 +198,12 @@ template <typename T>
 inline void launch_reduce_partials(const float* part0, T* out0, const float* part1, T* out1, int64_t groups, int64_t cols,
                                    int cu_count, hipStream_t stream) {
   const unsigned pairs = part1 ? 2u : 1u;
-  if (ceil_div(cols, 64) * pairs >= static_cast<int64_t>(cu_count)) {
+  const bool slab_ok = cols % 4 == 0 && groups >= 128 && ceil_div(cols, 32) * pairs * 2 >= static_cast<int64_t>(cu_count) &&
+                       aligned16(part0) && (!part1 || aligned16(part1)) && env_int("MOGRAD_HIP_REDUCE_SLAB", 1) != 0;
+  if (slab_ok) {
+    hipLaunchKernelGGL((reduce_partials_slab_kernel<T>), dim3(static_cast<unsigned>(ceil_div(cols, 32)), pairs),
+                       dim3(1024), 0, stream, part0, out0, part1, out1, groups, cols);
+  } else if (ceil_div(cols, 64) * pairs >= static_cast<int64_t>(cu_count)) {
     hipLaunchKernelGGL((reduce_partials_cw_kernel<T, 64>), dim3(static_cast<unsigned>(ceil_div(cols, 64)), pairs),
                        dim3(256), 0, stream, part0, out0, part1, out1, groups, cols);
   } else if (ceil_div(cols, 32) * pairs * 2 >= static_cast<int64_t>(cu_count)) {
