@@ -188,7 +188,10 @@ __global__ __launch_bounds__(1024) void reduce_partials_slab_kernel(const float*
   }
 }
 
-// Launches the reduction of one or two (groups, cols) partial arrays.  Wide outputs use 64
+// Launches the reduction of one or two (groups, cols) partial arrays.  With at least 128
+// groups of 16-byte aligned rows the slab kernel takes it (every partial in flight at once:
+// about 1 us less per call than the forms below at 256 groups, for 384 columns as for
+// 4096).  Otherwise wide outputs use 64
 // columns x 4 slices per workgroup; narrower ones 32 x 8 (a workgroup still reads whole
 // 128-byte lines of the fp32 partials: with 64-byte pieces the two workgroups that share a
 // line sit on different XCDs and each L2 fetches the line, which doubled the kernel's
@@ -198,8 +201,8 @@ template <typename T>
 inline void launch_reduce_partials(const float* part0, T* out0, const float* part1, T* out1, int64_t groups, int64_t cols,
                                    int cu_count, hipStream_t stream) {
   const unsigned pairs = part1 ? 2u : 1u;
-  const bool slab_ok = cols % 4 == 0 && groups >= 128 && ceil_div(cols, 32) * pairs * 2 >= static_cast<int64_t>(cu_count) &&
-                       aligned16(part0) && (!part1 || aligned16(part1)) && env_int("MOGRAD_HIP_REDUCE_SLAB", 1) != 0;
+  const bool slab_ok = cols % 4 == 0 && groups >= 128 && aligned16(part0) && (!part1 || aligned16(part1)) &&
+                       env_int("MOGRAD_HIP_REDUCE_SLAB", 1) != 0;
   if (slab_ok) {
     hipLaunchKernelGGL((reduce_partials_slab_kernel<T>), dim3(static_cast<unsigned>(ceil_div(cols, 32)), pairs),
                        dim3(1024), 0, stream, part0, out0, part1, out1, groups, cols);

@@ -64,6 +64,10 @@ SHAPES = [
     # tall and wide: the backward pairs 512-thread rows in 1024-thread workgroups (odd row
     # counts leave a row slot without a row at the end of a group)
     (1027, 4096), (1025, 3000), (1031, 8192),
+    # 128 or more row groups: the partial dgamma/dbeta rows are summed by the 32-column slab
+    # reduction (133 groups: one full pass of 128 group lanes and a ragged one; 512 groups;
+    # 388 and 644 columns leave the last slab ragged)
+    (530, 644), (2100, 388), (4300, 388),
 ]
 
 
