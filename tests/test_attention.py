@@ -259,3 +259,56 @@ def test_packed_qkv_forms_equal_the_separate_forms(device, dtype, name, causal, 
     got = dqkv.to_numpy((B, S, 3, H, D))
     for i, what in enumerate(("dq", "dk", "dv")):
         np.testing.assert_array_equal(got[:, :, i], g[i].to_numpy((B, S, H, D)), err_msg=what)
+
+
+# The two attention configurations of the benchmark at their own shapes: causal
+# (B8, H12, S1024, D64) runs dK/dV and dQ in one launch of 1536 workgroups; non-causal
+# (B2, H12, S4096, D64) takes the separately launched walks with 128-query steps.
+C4_SHAPES = [("causal", 1, 8, 12, 1024, 64, True, [(0, 0), (3, 7), (7, 11)]),
+             ("full", 2, 2, 12, 4096, 64, False, [(0, 0), (1, 5), (1, 11)])]
+
+
+@pytest.mark.parametrize("name,cfg,B,H,S,D,causal,heads", C4_SHAPES)
+def test_benchmark_shapes_against_oracle(device, name, cfg, B, H, S, D, causal, heads):
+    import os
+
+    q, k, v = (round_to_dtype(normal(4, cfg * 10 + i, (B, S, H, D)), BF16) for i in range(3))
+    do = round_to_dtype(normal(4, cfg * 10 + 3, (B, H, S, D)), BF16)
+    o, lse, dq, dk, dv = _fwd_bwd(device, q, k, v, do, None, causal, dtype=BF16)
+    for t in (o, lse, dq, dk, dv):
+        assert np.all(np.isfinite(t))
+    # float64 oracle on the first, a middle and the last (batch, head)
+    for b, h in heads:
+        sl = lambda t: t[b:b + 1, :, h:h + 1, :]  # noqa: E731
+        ro, rl = O.sdpa_fwd(sl(q), sl(k), sl(v), None, causal)
+        assert _max_err(o[b:b + 1, h:h + 1], ro) <= 1.6e-2, (b, h)
+        assert _max_err(lse[b:b + 1, h:h + 1], rl) <= 1e-3 * max(1.0, float(np.abs(rl).max())), (b, h)
+        want = O.sdpa_bwd(sl(q), sl(k), sl(v), do[b:b + 1, h:h + 1], None, causal)
+        for got, ref, what in zip((dq, dk, dv), want, ("dq", "dk", "dv")):
+            bound = RTOL_BF16_ATTN * (np.abs(ref) + np.abs(ref).max())
+            worst = np.max(np.abs(sl(got) - ref) / bound)
+            assert worst <= 1.0, f"{what} at (b{b}, h{h}): worst {worst:.3g}"
+    # every (batch, head): a second run gives the same bits, and the gradients are linear in
+    # dO exactly for a power-of-two factor (delta, dP and dS double without rounding)
+    o2, lse2, dq2, dk2, dv2 = _fwd_bwd(device, q, k, v, do, None, causal, dtype=BF16)
+    for a, b_, what in zip((o, lse, dq, dk, dv), (o2, lse2, dq2, dk2, dv2), ("o", "lse", "dq", "dk", "dv")):
+        np.testing.assert_array_equal(a, b_, err_msg=what)
+    _, _, dq4, dk4, dv4 = _fwd_bwd(device, q, k, v, do * np.float32(4.0), None, causal, dtype=BF16)
+    for a, b_, what in zip((dq, dk, dv), (dq4, dk4, dv4), ("dq", "dk", "dv")):
+        np.testing.assert_array_equal(a * np.float32(4.0), b_, err_msg=f"{what} not linear in dO")
+    # every (batch, head) against the second formulation in the library: the wave-per-row
+    # kernels that do all arithmetic in fp32 (no matrix cores, no tiles)
+    os.environ["MOGRAD_HIP_ATTN_GENERIC"] = "1"
+    try:
+        og, lg, dqg, dkg, dvg = _fwd_bwd(device, q, k, v, do, None, causal, dtype=BF16)
+    finally:
+        del os.environ["MOGRAD_HIP_ATTN_GENERIC"]
+    assert _max_err(o, og.astype(np.float64)) <= 3.2e-2
+    assert _max_err(lse, lg.astype(np.float64)) <= 2e-3 * max(1.0, float(np.abs(lg).max()))
+    for got, ref, what in zip((dq, dk, dv), (dqg, dkg, dvg), ("dq", "dk", "dv")):
+        ref = ref.astype(np.float64)
+        # per (batch, head) floor: the largest entry of that head's gradient
+        top = np.abs(ref).max(axis=(1, 3), keepdims=True)
+        bound = 2 * RTOL_BF16_ATTN * (np.abs(ref) + top)
+        worst = np.max(np.abs(got - ref) / bound)
+        assert worst <= 1.0, f"{what} vs fp32-arithmetic kernels: worst {worst:.3g}"

@@ -154,6 +154,112 @@ def test_mlp_chain_matches_oracle(device):
         assert_close(got[k], want[k], RTOL_F32, ATOL_F32, k)
 
 
+def test_readme_mlp_square_layer_f32(device):
+    # The 4096 -> 4096 Linear of the README MLP at batch 2048: forward, dX, dW, db at the
+    # size where 1024 output tiles are walked by a grid of 512 resident workgroups.
+    M = 2048
+    N = K = 4096
+    x = normal(3, 30, (M, K))
+    bound = np.sqrt(6.0 / K)
+    w = uniform(3, 31, (N, K), -bound, bound)
+    b = uniform(3, 32, (N,), -bound, bound)
+    dy = normal(3, 33, (M, N))
+    y, dx, dw, db = _linear_all(device, x, w, b, dy)
+    assert_sum_close(y, O.matmul_bias_bt(x, w, b), np.abs(x) @ np.abs(w).T, what="y")
+    assert_sum_close(dx, O.linear_grad_x(dy, w), np.abs(dy) @ np.abs(w), what="dx")
+    assert_sum_close(dw, O.linear_grad_w(dy, x), np.abs(dy).T @ np.abs(x), what="dw")
+    assert_sum_close(db, O.linear_grad_b(dy), np.abs(dy).sum(axis=0), what="db")
+
+
+def test_readme_mlp_chain_matches_oracle(device):
+    # README MLP, fp32: x (2048,4096) -> Linear 4096 +ReLU -> LayerNorm -> Linear 4096 +ReLU ->
+    # Linear 10 -> cross-entropy on integer labels; the call sequence of the benchmark's
+    # MLP step, every gradient against the float64 oracle chain.
+    from mograd_amd import I32
+
+    lib, st = device.lib, device.stream
+    M, D, NC = 2048, 4096, 10
+    bound = np.sqrt(6.0 / D)
+    x = normal(3, 0, (M, D))
+    w1, w2 = (uniform(3, i, (D, D), -bound, bound) for i in (1, 3))
+    b1, b2 = (uniform(3, i, (D,), -bound, bound) for i in (2, 4))
+    w3, b3 = uniform(3, 5, (NC, D), -bound, bound), uniform(3, 6, (NC,), -bound, bound)
+    gamma, beta = np.ones(D, np.float32), np.zeros(D, np.float32)
+    ids = np.random.Generator(np.random.PCG64(3007)).integers(0, NC, M).astype(np.int32)
+    up = lambda a: AnyBuffer.from_numpy(device, a)  # noqa: E731
+    new = lambda n: AnyBuffer.create(F32, device, n)  # noqa: E731
+    P = lambda t: t.data_ptr()  # noqa: E731
+    bx, bw1, bw2, bw3, bb1, bb2, bb3, bg, bbt = (up(a) for a in (x, w1, w2, w3, b1, b2, b3, gamma, beta))
+    bids = AnyBuffer.from_numpy(device, ids, I32)
+    h1p, h1, ln, h2p, h2, logits = new(M * D), new(M * D), new(M * D), new(M * D), new(M * D), new(M * NC)
+    loss, dlogits = new(1), new(M * NC)
+    dh2, dh2p, dln, dh1, dh1p = new(M * D), new(M * D), new(M * D), new(M * D), new(M * D)
+    dw1, dw2, dw3, db1, db2, db3, dg, dbt = new(D * D), new(D * D), new(NC * D), new(D), new(D), new(NC), new(D), new(D)
+
+    def linear(a, w, b, y, n_out, k):
+        lib.mg_matmul_bias_bt(P(a), P(w), P(b), P(y), 1, M, n_out, k, k, 1, k, 1, M * k, n_out * k, F32, st)
+
+    linear(bx, bw1, bb1, h1p, D, D)
+    lib.mg_relu_grad(P(h1p), P(h1p), P(h1), M * D, F32, st)  # relu(v) == relu_grad(v, v)
+    lib.mg_layer_norm_fwd(P(h1), P(bg), P(bbt), P(ln), M, D, 1e-5, F32, st)
+    linear(ln, bw2, bb2, h2p, D, D)
+    lib.mg_relu_grad(P(h2p), P(h2p), P(h2), M * D, F32, st)
+    linear(h2, bw3, bb3, logits, NC, D)
+    lib.mg_cross_entropy_fused_ids(P(logits), P(bids), None, P(loss), P(dlogits), M, NC, F32, I32, st)
+    lib.mg_linear_bwd(P(dlogits), P(h2), P(bw3), P(dh2), P(dw3), P(db3), M, NC, D, F32, st)
+    lib.mg_relu_grad(P(h2), P(dh2), P(dh2p), M * D, F32, st)
+    lib.mg_linear_bwd(P(dh2p), P(ln), P(bw2), P(dln), P(dw2), P(db2), M, D, D, F32, st)
+    lib.mg_layer_norm_bwd(P(dln), P(h1), P(bg), P(dh1), P(dg), P(dbt), M, D, 1e-5, F32, st)
+    lib.mg_relu_grad(P(h1), P(dh1), P(dh1p), M * D, F32, st)
+    lib.mg_linear_bwd(P(dh1p), P(bx), P(bw1), None, P(dw1), P(db1), M, D, D, F32, st)
+
+    # Oracle chain in float64.  A pre-activation within rounding of zero has no determined
+    # sign: there (and only there) the oracle takes the mask the fp32 forward produced.
+    def mask_of(pre64, pre_gpu, what):
+        m64 = pre64 > 0
+        unsure = np.abs(pre64) < 1e-4
+        assert np.array_equal(m64[~unsure], (pre_gpu > 0)[~unsure]), what
+        assert unsure.mean() < 1e-3, what
+        return np.where(unsure, pre_gpu > 0, m64)
+
+    r_h1p = O.matmul_bias_bt(x, w1, b1)
+    g_h1p = h1p.to_numpy((M, D))
+    assert_sum_close(g_h1p, r_h1p, np.abs(x) @ np.abs(w1).T, what="h1 pre-activation")
+    m1 = mask_of(r_h1p, g_h1p, "relu 1 mask")
+    r_h1 = np.where(m1, r_h1p, 0.0)
+    r_ln = O.layer_norm_fwd(r_h1, gamma, beta)
+    # the LayerNorm's input carries the rounding of the product before it, scaled by rstd
+    _, rstd1 = O.layer_norm_stats(r_h1, 1e-5)
+    assert_sum_close(ln.to_numpy((M, D)), r_ln, rstd1 * (np.abs(x) @ np.abs(w1).T), what="layer norm output")
+    r_h2p = O.matmul_bias_bt(r_ln, w2, b2)
+    g_h2p = h2p.to_numpy((M, D))
+    m2 = mask_of(r_h2p, g_h2p, "relu 2 mask")
+    r_h2 = np.where(m2, r_h2p, 0.0)
+    r_logits = O.matmul_bias_bt(r_h2, w3, b3)
+    assert_sum_close(logits.to_numpy((M, NC)), r_logits, np.abs(r_h2) @ np.abs(w3).T, what="logits")
+    assert_close(loss.item(), O.cross_entropy_ids(r_logits, ids), RTOL_F32, ATOL_F32, "loss")
+    r_dlogits = O.cross_entropy_grad_ids(r_logits, ids)
+    a = np.abs
+    assert_sum_close(dw3.to_numpy((NC, D)), O.linear_grad_w(r_dlogits, r_h2), a(r_dlogits).T @ a(r_h2), what="dw3")
+    assert_sum_close(db3.to_numpy(), O.linear_grad_b(r_dlogits), a(r_dlogits).sum(axis=0), what="db3")
+    r_dh2p = np.where(m2, O.linear_grad_x(r_dlogits, w3), 0.0)
+    assert_sum_close(dw2.to_numpy((D, D)), O.linear_grad_w(r_dh2p, r_ln), a(r_dh2p).T @ a(r_ln), what="dw2")
+    assert_sum_close(db2.to_numpy(), O.linear_grad_b(r_dh2p), a(r_dh2p).sum(axis=0), what="db2")
+    r_dln = O.linear_grad_x(r_dh2p, w2)
+    assert_sum_close(dln.to_numpy((M, D)), r_dln, a(r_dh2p) @ a(w2), what="dln")
+    r_dh1, r_dg, r_dbt = O.layer_norm_bwd(r_dln, r_h1, gamma)
+    xhat = O.layer_norm_fwd(r_h1, gamma, beta)
+    assert_sum_close(dg.to_numpy(), r_dg, (a(r_dln) * a(xhat)).sum(axis=0), what="dgamma")
+    assert_sum_close(dbt.to_numpy(), r_dbt, a(r_dln).sum(axis=0), what="dbeta")
+    # dx of a LayerNorm row: rstd * (dy - mean(dy) - xhat * mean(dy * xhat)), each mean a sum of
+    # 4096 terms of the size of dln
+    row = a(r_dln).mean(axis=1, keepdims=True)
+    assert_sum_close(dh1.to_numpy((M, D)), r_dh1, rstd1 * (a(r_dln) + row * (1.0 + a(xhat))), what="dh1")
+    r_dh1p = np.where(m1, r_dh1, 0.0)
+    assert_sum_close(dw1.to_numpy((D, D)), O.linear_grad_w(r_dh1p, x), a(r_dh1p).T @ a(x), what="dw1")
+    assert_sum_close(db1.to_numpy(), O.linear_grad_b(r_dh1p), a(r_dh1p).sum(axis=0), what="db1")
+
+
 @pytest.mark.parametrize("dtype,rtol", [(F16, 2e-3), (BF16, 1.6e-2)])
 def test_half_precision_storage(device, dtype, rtol):
     M, N, K = 96, 80, 136
