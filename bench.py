@@ -91,7 +91,7 @@ def cpu_baseline(sample_ce_rows: int = 256):
         subprocess.run(["make", "-C", str(ROOT / "oracle")], check=True, capture_output=True)
     orc = C.CDLL(str(so))
     orc.orc_num_threads.restype = C.c_int
-    orc.orc_cross_entropy_ids_f32.restype = C.c_float
+    orc.orc_cross_entropy_f32.restype = C.c_float
     cores = int(orc.orc_num_threads())
     p = lambda a: a.ctypes.data_as(C.c_void_p)  # noqa: E731
     L = C.c_int64
@@ -114,10 +114,14 @@ def cpu_baseline(sample_ce_rows: int = 256):
     up = np.ones(1, np.float32)
     dlogits = np.empty_like(logits)
 
+    onehot = np.zeros((n, CE_COLS), np.float32)
+    onehot[np.arange(n), ids] = 1.0
+
     def ce():
-        # the reference runs forward and gradient as separate kernels
-        orc.orc_cross_entropy_ids_f32(p(logits), p(ids), L(n), L(CE_COLS))
-        orc.orc_cross_entropy_grad_ids_f32(p(logits), p(ids), p(up), p(dlogits), L(n), L(CE_COLS))
+        # the reference's structure: forward and gradient as separate passes, each re-deriving
+        # the row maximum and the sum of exponentials, labels dense (one-hot rows)
+        orc.orc_cross_entropy_f32(p(logits), p(onehot), L(n), L(CE_COLS))
+        orc.orc_cross_entropy_grad_f32(p(logits), p(onehot), p(up), p(dlogits), L(n), L(CE_COLS))
 
     def best(fn, reps):
         fn()
@@ -135,8 +139,8 @@ def cpu_baseline(sample_ce_rows: int = 256):
         "unit": "ms",
         "cores": cores,
         "kind": "port",
-        "sample": f"LayerNorm fwd+bwd full (2048x4096) {ln_ms:.2f} ms; cross-entropy fwd+grad on {n} of 8192 rows "
-                  f"scaled x{CE_ROWS // n} = {ce_ms:.1f} ms; best of 3-5 runs, OpenMP on {cores} threads",
+        "sample": f"LayerNorm fwd+bwd full (2048x4096) {ln_ms:.2f} ms; cross-entropy forward and gradient as separate passes with dense "
+                  f"(one-hot) labels on {n} of 8192 rows scaled x{CE_ROWS // n} = {ce_ms:.1f} ms; best of 3-5 runs, OpenMP on {cores} threads",
     }
 
 
@@ -190,7 +194,7 @@ def _kernel_table(dev, entries, iters):
     return out
 
 
-def bench_mlp(args, dev) -> int:
+def bench_mlp(args, dev) -> dict:
     """README MLP, fp32: x (2048,4096) -> Linear 4096->4096 +ReLU -> LayerNorm(4096) -> Linear 4096->4096 +ReLU
     -> Linear 4096->10, cross-entropy on labels in [0,10).  Forward and backward through the C ABI."""
     from mograd_amd import F32, I32, AnyBuffer
@@ -282,11 +286,10 @@ def bench_mlp(args, dev) -> int:
             "value": round(slab_ms * (M / rows), 1), "unit": "ms", "cores": cores, "kind": "port",
             "sample": f"dX + dW + db of one 4096x4096 Linear on {rows} of {M} rows ({slab_ms:.1f} ms) scaled x{M // rows}; "
                       f"one layer, not the whole step; OpenMP on {cores} threads"}
-    print(json.dumps(result))
-    return 0
+    return result
 
 
-def bench_attention(args, dev) -> int:
+def bench_attention(args, dev) -> dict:
     """Flash attention fwd+bwd, bf16 with fp32 accumulation: causal B8 H12 S1024 D64 (the step), and
     non-causal B2 H12 S4096 D64 in the kernel table."""
     from mograd_amd import BF16, F32, AnyBuffer
@@ -366,11 +369,10 @@ def bench_attention(args, dev) -> int:
             "value": round(slab_ms * scale_up, 1), "unit": "ms", "cores": cores, "kind": "port",
             "sample": f"naive fp32 attention fwd+bwd on {Bs * Hs} of {B * H} (batch, head) pairs of the causal "
                       f"configuration ({slab_ms:.1f} ms) scaled x{scale_up}; OpenMP on {cores} threads"}
-    print(json.dumps(result))
-    return 0
+    return result
 
 
-def bench_gpt(args, dev) -> int:
+def bench_gpt(args, dev) -> dict:
     """Character-level GPT training step (examples/tinyshakespear/model.mojo shape): vocab 65, context 256,
     batch 64, 6 layers, d_model 384, 6 heads, MLP 4x, pre-LayerNorm, bf16 activations with fp32 master weights,
     token ids uniform in [0, 65); forward, loss and every parameter gradient."""
@@ -495,8 +497,7 @@ def bench_gpt(args, dev) -> int:
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = _gpt_cpu_baseline(V, d, ff, L, H, B, T)
-    print(json.dumps(result))
-    return 0
+    return result
 
 
 def _gpt_cpu_baseline(V, d, ff, L, H, B, T):
@@ -567,32 +568,12 @@ def _gpt_cpu_baseline(V, d, ff, L, H, B, T):
                       f"(16 batch slices x {L} layers); embedding, lm_head and loss left out; OpenMP on {cores} threads"}
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
-    ap.add_argument("--workload", choices=["ln_ce", "mlp", "attention", "gpt"], default="ln_ce",
-                    help="ln_ce (default): the configuration the metric is quoted on; mlp: README MLP fwd+bwd fp32 "
-                         "(matmul_bias_bt, dX, dW, db); attention: bf16 flash attention fwd+bwd")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this path runs on one GPU; --gpus N with N > 1 is not supported "
-              "(no collective is part of the backward hot path)", file=sys.stderr)
-        return 2
+def bench_ln_ce(args, dev) -> dict:
+    """LayerNorm fwd+bwd fp32 (2048,4096) plus fused softmax-cross-entropy fwd+bwd fp32 (8192,50304), int32 labels."""
+    from mograd_amd import F32, I32, AnyBuffer
 
-    from mograd_amd import F32, I32, AnyBuffer, Device
-
-    dev = Device(0)
     lib = dev.lib
     st = dev.stream
-    if args.workload == "mlp":
-        return bench_mlp(args, dev)
-    if args.workload == "gpt":
-        return bench_gpt(args, dev)
-    if args.workload == "attention":
-        return bench_attention(args, dev)
 
     # ---- inputs, resident in HBM -------------------------------------------------------
     # LayerNorm: four rotating sets (4 x 100 MB) so that no set is still in the 256 MB
@@ -708,6 +689,48 @@ def main() -> int:
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
+    return result
+
+
+WORKLOADS = {"ln_ce": bench_ln_ce, "mlp": bench_mlp, "attention": bench_attention, "gpt": bench_gpt}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
+    ap.add_argument("--workload", choices=["all", *WORKLOADS], default="all",
+                    help="all (default): every configuration in one process, the GPT training step as the headline "
+                         "and the others under 'workloads'; ln_ce: LayerNorm + fused cross-entropy fp32; mlp: README "
+                         "MLP fwd+bwd fp32 (matmul_bias_bt, dX, dW, db); attention: bf16 flash attention fwd+bwd; "
+                         "gpt: the training step alone")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path runs on one GPU; --gpus N with N > 1 is not supported "
+              "(no collective is part of the backward hot path)", file=sys.stderr)
+        return 2
+
+    from mograd_amd import Device
+
+    dev = Device(0)
+    if args.workload != "all":
+        print(json.dumps(WORKLOADS[args.workload](args, dev)))
+        return 0
+    # Every configuration, one after the other on the same device and stream.  The headline
+    # is the GPT training step; each configuration's own step time, roofline, kernel table
+    # and CPU baseline sit under "workloads".
+    per = {}
+    for name in ("ln_ce", "mlp", "attention", "gpt"):
+        print(f"[bench] {name} ...", file=sys.stderr, flush=True)
+        per[name] = WORKLOADS[name](args, dev)
+        dev.synchronize()
+        dev.lib.mg_pool_empty_cache()
+    keep = ("ms_per_step", "dtype", "config", "roofline", "kernels", "cpu_baseline", "phases_ms", "step_roofline")
+    result = dict(per["gpt"])
+    result["workloads"] = {name: {k: r[k] for k in keep if k in r} for name, r in per.items()}
+    result.pop("kernels", None)  # the GPT step's table is under workloads.gpt
     print(json.dumps(result))
     return 0
 
