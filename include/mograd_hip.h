@@ -220,6 +220,21 @@ int mg_cross_entropy_grad_ids(const void* logits, const void* ids, const void* u
 int mg_cross_entropy_fused_ids(const void* logits, const void* ids, const void* upstream,
                                void* loss, void* dlogits, int64_t N, int64_t C, int dtype,
                                int id_dtype, mg_stream stream);
+/* mg_cross_entropy_fused_ids for callers that cannot allocate (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): same arguments, kernels
+ * and results, but the per-row loss terms go to a static device array of
+ * MG_CE_NOALLOC_MAX_ROWS floats (4 MiB per GPU, held until the process ends) instead of a
+ * pool block, and the call makes no hipMalloc/hipFree and takes nothing from the pool.
+ * N above MG_CE_NOALLOC_MAX_ROWS is rejected with MG_ERR_INVALID.  Every call on a GPU
+ * shares that GPU's array: calls that overlap on one GPU (different streams) race; calls
+ * on one stream are ordered.  The array's device address is looked up once per device
+ * (in mg_init, else on the first call there), so call mg_init or make one call before
+ * starting a capture.  No counterpart in the reference. */
+#define MG_CE_NOALLOC_MAX_ROWS (1 << 20)
+int mg_cross_entropy_fused_ids_noalloc(const void* logits, const void* ids, const void* upstream,
+                                       void* loss, void* dlogits, int64_t N, int64_t C, int dtype,
+                                       int id_dtype, mg_stream stream);
+
 /* Dense-label loss and dlogits in one pass. */
 int mg_cross_entropy_fused(const void* logits, const void* labels, const void* upstream,
                            void* loss, void* dlogits, int64_t N, int64_t C, int dtype,

@@ -87,6 +87,7 @@ PROTOTYPES = {
     "mg_cross_entropy_ids": (_i, [_p, _p, _p, _l, _l, _i, _i, _p], True),
     "mg_cross_entropy_grad_ids": (_i, [_p, _p, _p, _p, _l, _l, _i, _i, _p], True),
     "mg_cross_entropy_fused_ids": (_i, [_p, _p, _p, _p, _p, _l, _l, _i, _i, _p], True),
+    "mg_cross_entropy_fused_ids_noalloc": (_i, [_p, _p, _p, _p, _p, _l, _l, _i, _i, _p], True),
     "mg_cross_entropy_fused": (_i, [_p, _p, _p, _p, _p, _l, _l, _i, _p], True),
     "mg_matmul": (_i, [_p, _p, _p] + [_l] * 10 + [_i, _p], True),
     "mg_matmul_bt": (_i, [_p, _p, _p] + [_l] * 10 + [_i, _p], True),

@@ -1,11 +1,13 @@
 // C ABI for softmax cross-entropy: argument checks and dtype dispatch.
+#include <mutex>
+
 #include "mg_internal.h"
 
 namespace mg {
 
 #define MG_DECLARE_CROSS_ENTROPY(SUFFIX)                                                                         \
   int ce_run_##SUFFIX(bool, const void*, const void*, const void*, void*, void*, int64_t, int64_t, int,          \
-                      hipStream_t);                                                                              \
+                      hipStream_t, float*);                                                                            \
   int ce_run_strided_##SUFFIX(const void*, const void*, const void*, void*, void*, int64_t, int64_t,             \
                               const StridedView&, const StridedView&, hipStream_t);
 MG_DECLARE_CROSS_ENTROPY(f32)
@@ -24,7 +26,8 @@ static int check_ce(const char* who, int64_t N, int64_t C, int dtype) {
 }
 
 static int ce_run(const char* who, bool dense, const void* logits, const void* labels, const void* upstream, void* loss,
-                  void* dlogits, int64_t N, int64_t C, int dtype, int id_dtype, mg_stream stream) {
+                  void* dlogits, int64_t N, int64_t C, int dtype, int id_dtype, mg_stream stream,
+                  float* rowloss_ext = nullptr) {
   MG_TRY(check_ce(who, N, C, dtype));
   if (!logits || !labels || (!loss && !dlogits)) return fail(MG_ERR_INVALID, "%s: null pointer argument", who);
   int id64 = 0;
@@ -35,9 +38,9 @@ static int ce_run(const char* who, bool dense, const void* logits, const void* l
   }
   hipStream_t s = to_stream(stream);
   switch (dtype) {
-    case MG_F32: return ce_run_f32(dense, logits, labels, upstream, loss, dlogits, N, C, id64, s);
-    case MG_F16: return ce_run_f16(dense, logits, labels, upstream, loss, dlogits, N, C, id64, s);
-    default: return ce_run_bf16(dense, logits, labels, upstream, loss, dlogits, N, C, id64, s);
+    case MG_F32: return ce_run_f32(dense, logits, labels, upstream, loss, dlogits, N, C, id64, s, rowloss_ext);
+    case MG_F16: return ce_run_f16(dense, logits, labels, upstream, loss, dlogits, N, C, id64, s, rowloss_ext);
+    default: return ce_run_bf16(dense, logits, labels, upstream, loss, dlogits, N, C, id64, s, rowloss_ext);
   }
 }
 
@@ -66,6 +69,35 @@ static int ce_run_strided(const char* who, const void* logits, const void* label
     case MG_F16: return ce_run_strided_f16(logits, labels, upstream, loss, dlogits, N, C, la, lb, s);
     default: return ce_run_strided_bf16(logits, labels, upstream, loss, dlogits, N, C, la, lb, s);
   }
+}
+
+// ---- The entry point that allocates nothing -------------------------------------------
+// Per-row loss terms of mg_cross_entropy_fused_ids_noalloc live in this array instead of a
+// pool block: MG_CE_NOALLOC_MAX_ROWS floats (4 MiB) on every GPU the library runs on, held
+// until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; the device address it resolves to differs per GPU and is what the
+// kernels receive.
+static __device__ __align__(256) float scratch[MG_CE_NOALLOC_MAX_ROWS];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static float* g_scratch_ptr[kMaxDevices] = {};
+
+// Resolves the current device's copy of `scratch` once; later calls return the kept address.
+int ce_noalloc_setup(float** out) {
+  int device = -1;
+  MG_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices)
+    return fail(MG_ERR_UNSUPPORTED, "cross_entropy_fused_ids_noalloc: device ordinal %d not supported", device);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    float* ptr = nullptr;
+    MG_HIP(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) return fail(MG_ERR_HIP, "cross_entropy_fused_ids_noalloc: scratch symbol resolved to null");
+    g_scratch_ptr[device] = ptr;
+  }
+  if (out) *out = g_scratch_ptr[device];
+  return MG_OK;
 }
 
 }  // namespace mg
@@ -118,6 +150,19 @@ int mg_cross_entropy_fused_ids(const void* logits, const void* ids, const void* 
   if (!loss || !dlogits) return mg::fail(MG_ERR_INVALID, "cross_entropy_fused_ids: null output pointer");
   return mg::ce_run("cross_entropy_fused_ids", false, logits, ids, upstream, loss, dlogits, N, C, dtype, id_dtype,
                     stream);
+}
+
+int mg_cross_entropy_fused_ids_noalloc(const void* logits, const void* ids, const void* upstream, void* loss,
+                                       void* dlogits, int64_t N, int64_t C, int dtype, int id_dtype,
+                                       mg_stream stream) {
+  if (!loss || !dlogits) return mg::fail(MG_ERR_INVALID, "cross_entropy_fused_ids_noalloc: null output pointer");
+  if (N > MG_CE_NOALLOC_MAX_ROWS)
+    return mg::fail(MG_ERR_INVALID, "cross_entropy_fused_ids_noalloc: N=%lld exceeds the %d rows of the static scratch",
+                    static_cast<long long>(N), MG_CE_NOALLOC_MAX_ROWS);
+  float* rowloss = nullptr;
+  MG_TRY(mg::ce_noalloc_setup(&rowloss));
+  return mg::ce_run("cross_entropy_fused_ids_noalloc", false, logits, ids, upstream, loss, dlogits, N, C, dtype,
+                    id_dtype, stream, rowloss);
 }
 
 int mg_cross_entropy_fused(const void* logits, const void* labels, const void* upstream, void* loss, void* dlogits,

@@ -514,16 +514,20 @@ struct CrossEntropyOps {
   }
 
   // Gradient and/or loss.  `loss` and `dlogits` may each be null (not both).
+  // `rowloss_ext`, when not null, is a buffer of at least N floats that takes the per-row
+  // loss terms instead of a block from the pool (the entry point that allocates nothing).
   template <bool DENSE>
   static int run(const void* logits_, const void* labels, const void* upstream_, void* loss_, void* dlogits_, int64_t N,
-                 int64_t C, int id64, hipStream_t stream) {
+                 int64_t C, int id64, hipStream_t stream, float* rowloss_ext = nullptr) {
     const T* logits = static_cast<const T*>(logits_);
     const T* upstream = static_cast<const T*>(upstream_);
     T* loss = static_cast<T*>(loss_);
     T* dlogits = static_cast<T*>(dlogits_);
     Scratch rowloss_buf;
     float* rowloss = nullptr;
-    if (loss != nullptr) {
+    if (loss != nullptr && rowloss_ext != nullptr) {
+      rowloss = rowloss_ext;
+    } else if (loss != nullptr) {
       MG_TRY(rowloss_buf.take(N * static_cast<int64_t>(sizeof(float))));
       rowloss = rowloss_buf.as<float>();
     }
@@ -585,10 +589,12 @@ struct CrossEntropyOps {
 #define MG_DEFINE_CROSS_ENTROPY(T, SUFFIX)                                                                          \
   namespace mg {                                                                                                    \
   int ce_run_##SUFFIX(bool dense, const void* logits, const void* labels, const void* upstream, void* loss,         \
-                      void* dlogits, int64_t N, int64_t C, int id64, hipStream_t stream) {                          \
+                      void* dlogits, int64_t N, int64_t C, int id64, hipStream_t stream, float* rowloss_ext) {      \
     if (dense)                                                                                                      \
-      return CrossEntropyOps<T>::template run<true>(logits, labels, upstream, loss, dlogits, N, C, id64, stream);   \
-    return CrossEntropyOps<T>::template run<false>(logits, labels, upstream, loss, dlogits, N, C, id64, stream);    \
+      return CrossEntropyOps<T>::template run<true>(logits, labels, upstream, loss, dlogits, N, C, id64, stream,    \
+                                                    rowloss_ext);                                                   \
+    return CrossEntropyOps<T>::template run<false>(logits, labels, upstream, loss, dlogits, N, C, id64, stream,     \
+                                                   rowloss_ext);                                                    \
   }                                                                                                                 \
   int ce_run_strided_##SUFFIX(const void* logits, const void* labels, const void* upstream, void* loss,             \
                               void* dlogits, int64_t N, int64_t C, const StridedView& la, const StridedView& lb,    \

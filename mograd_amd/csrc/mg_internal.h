@@ -25,6 +25,10 @@ struct DeviceInfo {
 // Properties of the current device, read once per device.
 const DeviceInfo& device_info();
 
+// cross_entropy.hip: address of the current device's static per-row loss scratch (resolved
+// on the first call per device); `out` may be null.
+int ce_noalloc_setup(float** out);
+
 // Pool (runtime.hip).  Thread-safe; see mg_pool_alloc / mg_pool_free.
 int pool_take(void** out, int64_t nbytes);
 int pool_release(void* ptr);

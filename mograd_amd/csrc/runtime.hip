@@ -242,6 +242,9 @@ const char* mg_last_error(void) { return mg::g_last_error.c_str(); }
 int mg_init(int device) {
   MG_HIP(hipSetDevice(device));
   (void)mg::device_info();
+  // the static scratch of the non-allocating entry point: resolve this device's copy now,
+  // so that its first call does no set-up work
+  MG_TRY(mg::ce_noalloc_setup(nullptr));
   return MG_OK;
 }
 
