@@ -66,18 +66,45 @@ __device__ __forceinline__ float dot_rows(const float (&a)[kAttnMaxDPerLane], co
   return wave_sum(s);
 }
 
+// The row statistics in the form the pipelined dK/dV walk copies straight into LDS: -lse in
+// log2 units and -delta, each (B*H, s_pad) with s_pad a multiple of 64 and the rows past S
+// holding -inf and 0 (probabilities of rows that do not exist vanish).  `idx` is the row's
+// index in (B,H,S) order; the thread that owns a sequence's last row writes its padding.
+struct AttnPaddedStats {
+  const float* lse = nullptr;
+  float* nlse = nullptr;    // null: not wanted
+  float* ndelta = nullptr;
+  int s_pad = 0;
+};
+__device__ __forceinline__ void write_padded_stats(const AttnPaddedStats& ps, int64_t idx, int S, float delta) {
+  if (ps.nlse == nullptr) return;
+  const int64_t bh = idx / S;
+  const int s = static_cast<int>(idx - bh * S);
+  ps.nlse[bh * ps.s_pad + s] = -ps.lse[idx] * kAttnLog2e;
+  ps.ndelta[bh * ps.s_pad + s] = -delta;
+  if (s == S - 1)
+    for (int t = S; t < ps.s_pad; ++t) {
+      ps.nlse[bh * ps.s_pad + t] = -INFINITY;
+      ps.ndelta[bh * ps.s_pad + t] = 0.f;
+    }
+}
+
 // delta[b,h,i] = sum_d dO[b,h,i,d] * O[b,h,i,d]
 template <typename T>
 __global__ __launch_bounds__(256) void attn_delta_kernel(const T* __restrict__ d_o, const T* __restrict__ o,
                                                          float* __restrict__ delta, int64_t rows, int D, int S, int H,
-                                                         int o_bshd) {
+                                                         int o_bshd, AttnPaddedStats ps = {}) {
   const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
   if (row >= rows) return;
   const int lane = threadIdx.x % kWave;
   float acc = 0.f;
   for (int d = lane; d < D; d += kWave) acc = fmaf(to_float(d_o[row * D + d]), to_float(o[row * D + d]), acc);
   acc = wave_sum(acc);
-  if (lane == 0) delta[o_row_to_bhs(row, S, H, o_bshd)] = acc;
+  if (lane == 0) {
+    const int64_t idx = o_row_to_bhs(row, S, H, o_bshd);
+    delta[idx] = acc;
+    write_padded_stats(ps, idx, S, acc);
+  }
 }
 
 // Forward: wave = one query row; online softmax in the exp2 domain.

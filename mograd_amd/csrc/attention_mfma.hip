@@ -21,6 +21,8 @@
 //
 // Layouts: Q, K, V, dQ, dK, dV BSHD; O, dO BHSD; mask (B,H,S,S); LSE, delta (B,H,S) fp32.
 #include <cstdlib>
+#include <type_traits>
+#include <utility>
 
 #include "attention_generic.h"
 #include "mg_internal.h"
@@ -839,6 +841,448 @@ __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, con
   }
 }
 
+// ---- dK, dV: software-pipelined walk (head dim <= 64, no bias) ----------------------------
+// Same products and register layouts as attn_dkdv_block, scheduled so that a wave keeps the
+// matrix pipe fed by itself.  The 32-query tiles of a walk form one sequence g = 0, 1, ...;
+// per tile there are five stages:
+//   L1(g)  LDS -> registers: the eight row fragments of Q and dO, and -lse / -delta of the
+//          tile's rows straight into the S and dP accumulators
+//   A(g)   eight MFMAs: S = Q K^T - lse, dP = dO V^T - delta
+//   B(g)   VALU: P = exp2(S), dS = P (dP - delta), both rounded and packed
+//   L2(g)  LDS -> registers: the transposed fragments of dO and Q
+//   C(g)   eight MFMAs: dV^T += dO^T P, dK^T += Q^T dS
+// and iteration g issues  [A(g+1) interleaved with B(g) and L2(g)]  then  [C(g) interleaved
+// with L1(g+2)]: every MFMA's operands were requested a block earlier, and the exponentials
+// of one tile run under the score products of the next.  S and dP alternate between two
+// register sets.  The order is pinned with sched_barrier between MFMA-sized groups.
+//
+// Tiles are copied global memory -> LDS by global_load_lds (no staging registers), 64 queries
+// per step into a ring of three buffers: the copies of step i + 2 are issued right after the
+// barrier that publishes step i + 1, which every wave passes between the two blocks of its
+// first tile of step i.  At that point nobody reads the buffer of step i - 1 any more, and the
+// copies of step i + 1 have had a whole step to land, so one barrier per step suffices and
+// nothing waits on it.  lse and delta arrive pre-negated (lse also in log2 units) and padded
+// per (batch, head) to a multiple of 64 rows with -inf / 0, so that rows past the end of the
+// sequence give P = 0 without any per-element test; their Q / dO rows are copies of the last
+// row.  Causal: wave w's keys meet the diagonal in tile w of the walk (which starts at the
+// workgroup's first key); it starts there, with the masked elements' S accumulators
+// initialised to -inf, and every later tile is unmasked.
+
+// f(integral_constant<int, 0>{}), ..., f(integral_constant<int, N - 1>{}): a loop whose index is a
+// compile-time constant inside the body (DPP controls are instruction immediates).
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+// The value that lane J of this lane's own row of 16 lanes holds (DPP row_newbcast).
+template <int J>
+__device__ __forceinline__ float row_bcast(float v) {
+  return dpp_move<0x150 + J>(v);
+}
+
+// The LDS image of the pipelined walks: as above, but chunk c of row r sits at position
+// c ^ swz16(r) with swz16(r) = 4 * (r/2 % 2) + (r/4 % 2) + 2 * (r/8 % 2).  The 128-bit row reads
+// of sixteen consecutive rows then fall on sixteen different bank groups (the plain swizzle
+// serves them two rows per group, which doubles the cycles of half of all fragment reads),
+// and the transposing reads stay conflict-free.  The price is that rows r and r + 8 no longer
+// swizzle alike, so the second transposing read of a fragment has an address register of its
+// own.  The tiles are written by global_load_lds, a kilobyte (eight rows) per wave
+// instruction, so the image costs nothing on the way in.
+__device__ __forceinline__ int tile_swz16(int r) { return 4 * ((r / 2) % 2) + (r / 4) % 2 + 2 * ((r / 8) % 2); }
+template <int DP>
+__device__ __forceinline__ int tile16_chunk_at(int r, int c) { return r * tile_row_bytes<DP>() + ((c ^ tile_swz16(r)) * 16); }
+template <int DP>
+struct TileLane16 {
+  int rows[DP / 16];
+  int tr_lo[DP / 32], tr_hi[DP / 32];
+  __device__ __forceinline__ explicit TileLane16(int lane) {
+#pragma unroll
+    for (int ks = 0; ks < DP / 16; ++ks) rows[ks] = tile16_chunk_at<DP>(lane % 32, ks * 2 + lane / 32);
+    const int col = ((lane / 16) % 2) * 16 + 4 * (lane % 4);
+    const int r = 4 * (lane / 32) + (lane % 16) / 4;
+#pragma unroll
+    for (int dt = 0; dt < DP / 32; ++dt) {
+      tr_lo[dt] = tile16_chunk_at<DP>(r, (dt * 32 + col) / 8) + (col % 8) * 2;
+      tr_hi[dt] = tile16_chunk_at<DP>(r + 8, (dt * 32 + col) / 8) + (col % 8) * 2;
+    }
+  }
+};
+template <int DP>
+__device__ __forceinline__ uint4 frag_rows(const char* __restrict__ lds, const TileLane16<DP>& at, int rt, int ks) {
+  return *reinterpret_cast<const uint4*>(lds + at.rows[ks] + rt * 32 * tile_row_bytes<DP>());
+}
+template <int DP>
+__device__ __forceinline__ uint4 frag_transposed(const char* __restrict__ lds, const TileLane16<DP>& at, int dt, int t) {
+  using lds_i16x4 = __attribute__((address_space(3))) short4_t;
+  const char* base = lds + t * 16 * tile_row_bytes<DP>();
+  const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      reinterpret_cast<lds_i16x4*>(reinterpret_cast<uintptr_t>(base + at.tr_lo[dt])));
+  const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      reinterpret_cast<lds_i16x4*>(reinterpret_cast<uintptr_t>(base + at.tr_hi[dt])));
+  const uint2 l = __builtin_bit_cast(uint2, lo), h = __builtin_bit_cast(uint2, hi);
+  return make_uint4(l.x, l.y, h.x, h.y);
+}
+
+template <int DP>
+constexpr int dkdv_pipe_buf_bytes() {
+  return 2 * 64 * tile_row_bytes<DP>() + 2 * 64 * 4;  // a Q tile, a dO tile, -lse, -delta of 64 queries
+}
+template <int DP>
+constexpr int dkdv_pipe_lds_bytes() {
+  return 3 * dkdv_pipe_buf_bytes<DP>();
+}
+
+// s_waitcnt with only the vector-memory counter set (vmcnt in bits 3:0 and 15:14, the
+// other counters left at "no wait").
+#define MG_ATTN_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0f70)
+
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+  using lds_ptr = __attribute__((address_space(3))) const char*;
+  return static_cast<unsigned>(reinterpret_cast<uintptr_t>((lds_ptr)p));
+}
+// One wave-wide copy global -> LDS: lane l's 16 (or 4) bytes land at `lds_wave_base` + 16 l
+// (4 l).  Written as assembly so that the compiler does not attach waits for these copies to
+// unrelated LDS reads; m0 is used by nothing else in these kernels.
+__device__ __forceinline__ void copy16_to_lds(unsigned lds_wave_base, const void* src) {
+  const unsigned dst = __builtin_amdgcn_readfirstlane(lds_wave_base);
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(src) : "memory");
+}
+__device__ __forceinline__ void copy4_to_lds(unsigned lds_wave_base, const void* src) {
+  const unsigned dst = __builtin_amdgcn_readfirstlane(lds_wave_base);
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(dst), "v"(src) : "memory");
+}
+
+#ifndef MG_ATTN_STAT_DPP
+#define MG_ATTN_STAT_DPP false
+#endif
+template <typename T, int DP, bool CAUSAL, bool STAT_DPP>
+__device__ __forceinline__ void attn_dkdv_pipe_block(const int block, char* smem, const T* __restrict__ d_o,
+                                                     const T* __restrict__ q, const T* __restrict__ k,
+                                                     const T* __restrict__ v, const float* __restrict__ nlse,
+                                                     const float* __restrict__ ndelta, const int s_pad,
+                                                     T* __restrict__ dk, T* __restrict__ dv, const AttnDims& a,
+                                                     float scale) {
+  static_assert(DP == 64, "tile shapes below are written for a 64-wide head");
+  constexpr int BNK = 128, BQ = 64, KS = DP / 16, DT = DP / 32;
+  constexpr int ROWS = BQ * tile_row_bytes<DP>();
+  constexpr int BUF = dkdv_pipe_buf_bytes<DP>();
+
+  const int n_bh = a.B * a.H;
+  const int kb = block / n_bh;
+  const int h = (block % n_bh) % a.H;
+  const int b = (block % n_bh) / a.H;
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const int half = lane / 32;
+  const TileLane16<DP> at(lane);
+  const int n = kb * BNK + wave * 32 + lane % 32;
+  const int64_t bh = static_cast<int64_t>(b) * a.H + h;
+
+  uint4 kf[KS], vf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d = ks * 16 + half * 8;
+    const bool ok = n < a.S && d < a.D;
+    kf[ks] = ok ? *reinterpret_cast<const uint4*>(k + qkv_at(a, b, n, h) + d) : make_uint4(0, 0, 0, 0);
+    kf[ks] = scale_frag<T>(kf[ks], scale * kAttnLog2e);
+    vf[ks] = ok ? *reinterpret_cast<const uint4*>(v + qkv_at(a, b, n, h) + d) : make_uint4(0, 0, 0, 0);
+  }
+  floatx16 acc_k[DT], acc_v[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    acc_k[dt] = zero16();
+    acc_v[dt] = zero16();
+  }
+
+  const int m_begin = CAUSAL ? kb * BNK : 0;
+  const int nsteps = (a.S - m_begin + BQ - 1) / BQ;
+  const int G = 2 * nsteps;
+
+  // ---- copies: step i -> buffer i % 3 ----
+  // Wave-instruction j of a tile covers its rows 8j .. 8j+7 (1 KB); this wave issues j = wave
+  // and wave + 4 for Q and for dO.  Lane l writes chunk position l % 8 of row 8j + l / 8 and
+  // therefore names the source chunk (l % 8) ^ swz16(row), with row % 16 = 8 (wave % 2) + l / 8.
+  // A copy's address is a scalar base (the step's first row of this (batch, head)) plus a
+  // 32-bit lane offset, so a step's copies cost two VALU operations each: the row, clamped to
+  // the last row of the sequence, times the row pitch.  Chunks of padding columns (head
+  // narrower than the tile) copy the row's chunk 0 instead: whatever lands in a padding column
+  // of Q or dO only ever meets the zeros that K and V hold there.
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int cp_row = lane / 8;
+  const int cp_chunk = (lane % 8) ^ tile_swz16(8 * (wave % 2) + cp_row);  // rows 8j + cp_row, j = wave or wave + 4
+  const unsigned cp_col_bytes = cp_chunk * 8 < a.D ? cp_chunk * 16 : 0;
+  const char* q_bh = reinterpret_cast<const char*>(q + qkv_at(a, b, 0, h));
+  const char* do_bh = reinterpret_cast<const char*>(d_o + o_at(a, b, h, 0));
+  const unsigned q_pitch = static_cast<unsigned>(a.ld) * 2, do_pitch = static_cast<unsigned>(o_ld(a)) * 2;  // bytes per row
+  const char* stat_bh = reinterpret_cast<const char*>((wave_u % 2 == 0 ? nlse : ndelta) + bh * s_pad);
+  const unsigned smem_base = lds_address(smem);
+  // Copy c of 5 of step `step` (clamped to the walk's last step: a copy past the end goes to a
+  // buffer that nobody reads again) into buffer `buf`: Q rows, dO rows, Q rows, dO rows, a statistic.
+  auto issue_piece = [&](int c, int step, int buf) {
+    const int m0 = m_begin + min(step, nsteps - 1) * BQ;
+    const unsigned base = smem_base + buf * BUF;
+    if (c < 4) {
+      const int jj = c / 2;
+      const bool is_do = c % 2;
+      const int j = wave_u + 4 * jj;
+      const int row = min(8 * j + cp_row, a.S - 1 - m0);  // relative to m0
+      const unsigned pitch = is_do ? do_pitch : q_pitch;
+      const char* rows0 = (is_do ? do_bh : q_bh) + static_cast<int64_t>(m0) * pitch;
+      const unsigned dst = __builtin_amdgcn_readfirstlane(base + (is_do ? ROWS : 0) + j * 1024);
+      const unsigned off = row * pitch + cp_col_bytes;
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(rows0) : "memory");
+    } else {
+      const unsigned dst = __builtin_amdgcn_readfirstlane(base + 2 * ROWS + (wave_u % 2) * BQ * 4);
+      const unsigned off = lane * 4;
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(off), "s"(stat_bh + m0 * 4) : "memory");
+    }
+  };
+  auto issue_step = [&](int step, int buf) {
+#pragma unroll
+    for (int c = 0; c < 5; ++c) issue_piece(c, step, buf);
+  };
+
+  // ---- stages ----
+  floatx16 s[2], dp[2];
+  float xs[2], xd[2];  // STAT_DPP: -lse and -delta of the tile's rows, spread over each row of 16 lanes
+  uint4 qr[KS], dor[KS], tq[2][DT], tdo[2][DT], pf[2], dsf[2];
+  uint32_t pw[8], dw[8];
+
+  // LDS addresses of this lane's fragments, as running 32-bit values: `ra` (row fragments)
+  // and `sa` (statistics) point into the buffer of the step that stage L1 reads, `tlo` / `thi`
+  // (transposing reads) into the buffer of the step that stage L2 reads, and all of them
+  // move on by one buffer at the end of every step.  Everything else about a read (Q or dO
+  // tile, which 32 rows, which 16 rows) is an immediate offset of the instruction, so the
+  // walk spends nine additions per step on addresses.
+  typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+  using lds_u4 = __attribute__((address_space(3))) const uintx4*;
+  typedef float floatx4 __attribute__((ext_vector_type(4)));
+  using lds_f4 = __attribute__((address_space(3))) const floatx4*;
+  using lds_f1 = __attribute__((address_space(3))) const float*;
+  using lds_i16x4 = __attribute__((address_space(3))) short4_t*;
+  unsigned ra[KS], sa, tlo[DT], thi[DT];
+  // Accumulator register e of a 32 x 32 tile belongs to row (e/4)*8 + half*4 + e%4.
+  // STAT_DPP: lane j of every row of 16 lanes fetches the statistics of exactly that row for
+  // e = j, and stage B reads "its" value for register e from lane e of its own row of lanes
+  // with a DPP broadcast (one 4-byte LDS read per lane and tile, two more VALU operations per
+  // element).  Otherwise the S and dP accumulators start from -lse and -delta, read as eight
+  // 16-byte broadcasts per tile.
+  const int stat_row = ((lane % 16) / 4) * 8 + half * 4 + lane % 4;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) ra[ks] = smem_base + at.rows[ks];
+  sa = smem_base + 2 * ROWS + (STAT_DPP ? stat_row * 4 : half * 16);
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    tlo[dt] = smem_base + at.tr_lo[dt];
+    thi[dt] = smem_base + at.tr_hi[dt];
+  }
+  int buf_l1 = 0, buf_l2 = 0;  // which buffer each group points into
+  auto advance_l1 = [&]() {
+    const int d = buf_l1 == 2 ? -2 * BUF : BUF;
+    buf_l1 = buf_l1 == 2 ? 0 : buf_l1 + 1;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ra[ks] += d;
+    sa += d;
+  };
+  auto advance_l2 = [&]() {
+    const int d = buf_l2 == 2 ? -2 * BUF : BUF;
+    buf_l2 = buf_l2 == 2 ? 0 : buf_l2 + 1;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      tlo[dt] += d;
+      thi[dt] += d;
+    }
+  };
+  auto read16 = [](unsigned addr) {
+    const uintx4 x = *reinterpret_cast<lds_u4>(static_cast<uintptr_t>(addr));
+    return make_uint4(x[0], x[1], x[2], x[3]);
+  };
+  auto read_tr = [](unsigned lo, unsigned hi) {
+    const short4_t l4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_i16x4>(static_cast<uintptr_t>(lo)));
+    const short4_t h4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_i16x4>(static_cast<uintptr_t>(hi)));
+    const uint2 l = __builtin_bit_cast(uint2, l4), h = __builtin_bit_cast(uint2, h4);
+    return make_uint4(l.x, l.y, h.x, h.y);
+  };
+
+  // L1 piece c of 8 for the tile at rows mt*32 of the buffer `ra` / `sa` point into, into register set P.
+  auto l1_piece = [&](auto PC, int c, int mt) {
+    constexpr int P = decltype(PC)::value;
+    if constexpr (STAT_DPP) {
+      if (c == 0) xs[P] = *reinterpret_cast<lds_f1>(static_cast<uintptr_t>(sa + mt * 128));
+      if (c == 1) xd[P] = *reinterpret_cast<lds_f1>(static_cast<uintptr_t>(sa + BQ * 4 + mt * 128));
+    } else if (c < 4) {
+      const floatx4 x = *reinterpret_cast<lds_f4>(static_cast<uintptr_t>(sa + mt * 128 + c * 32));
+      s[P][c * 4 + 0] = x.x; s[P][c * 4 + 1] = x.y; s[P][c * 4 + 2] = x.z; s[P][c * 4 + 3] = x.w;
+    } else {
+      const floatx4 x = *reinterpret_cast<lds_f4>(static_cast<uintptr_t>(sa + BQ * 4 + mt * 128 + (c - 4) * 32));
+      dp[P][(c - 4) * 4 + 0] = x.x; dp[P][(c - 4) * 4 + 1] = x.y; dp[P][(c - 4) * 4 + 2] = x.z; dp[P][(c - 4) * 4 + 3] = x.w;
+    }
+    if (c % 2 == 0) qr[c / 2] = read16(ra[c / 2] + mt * 32 * tile_row_bytes<DP>());
+    else dor[c / 2] = read16(ra[c / 2] + ROWS + mt * 32 * tile_row_bytes<DP>());
+  };
+  // MFMA c of 8 of stage A into register set P; FRESH: the accumulators start from zero.
+  auto a_piece = [&](auto PC, auto FRESH, int c) {
+    constexpr int P = decltype(PC)::value;
+    constexpr bool Z = decltype(FRESH)::value;
+    if (c % 2 == 0) s[P] = Mma<T>::run(qr[c / 2], kf[c / 2], (Z && c == 0) ? zero16() : s[P]);
+    else dp[P] = Mma<T>::run(dor[c / 2], vf[c / 2], (Z && c == 1) ? zero16() : dp[P]);
+  };
+  // VALU piece C of 8 of stage B on register set P: elements 2C and 2C+1.
+  auto b_piece = [&](auto PC, auto CC) {
+    constexpr int P = decltype(PC)::value;
+    constexpr int c = decltype(CC)::value;
+    float s0 = s[P][2 * c], s1 = s[P][2 * c + 1], d0 = dp[P][2 * c], d1 = dp[P][2 * c + 1];
+    if constexpr (STAT_DPP) {
+      s0 += row_bcast<2 * c>(xs[P]);
+      s1 += row_bcast<2 * c + 1>(xs[P]);
+      d0 += row_bcast<2 * c>(xd[P]);
+      d1 += row_bcast<2 * c + 1>(xd[P]);
+    }
+    const float p0 = fexp2(s0), p1 = fexp2(s1);
+    pw[c] = Mma<T>::pack2(p0, p1);
+    dw[c] = Mma<T>::pack2(p0 * d0, p1 * d1);
+    // Pins the arithmetic here, under the MFMA issued just before it: without a use in this
+    // block the compiler sinks it to the block after the barrier, where the results are read.
+    asm volatile("" : "+v"(pw[c]), "+v"(dw[c]));
+  };
+  // L2 piece c of 4: the transposed fragments of 16 of the tile's rows for one 32-column block.
+  auto l2_piece = [&](int c, int mt) {
+    const int hf = c / 2, dt = c % 2;
+    const int off = (mt * 2 + hf) * 16 * tile_row_bytes<DP>();
+    tdo[hf][dt] = read_tr(tlo[dt] + ROWS + off, thi[dt] + ROWS + off);
+    tq[hf][dt] = read_tr(tlo[dt] + off, thi[dt] + off);
+  };
+  // MFMA c of 8 of stage C.
+  auto c_piece = [&](int c) {
+    const int hf = c / 4, dt = (c % 4) / 2;
+    if (c % 2 == 0) acc_v[dt] = Mma<T>::run(tdo[hf][dt], pf[hf], acc_v[dt]);
+    else acc_k[dt] = Mma<T>::run(tq[hf][dt], dsf[hf], acc_k[dt]);
+  };
+  auto pack_frags = [&]() {
+    pf[0] = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+    pf[1] = make_uint4(pw[4], pw[5], pw[6], pw[7]);
+    dsf[0] = make_uint4(dw[0], dw[1], dw[2], dw[3]);
+    dsf[1] = make_uint4(dw[4], dw[5], dw[6], dw[7]);
+  };
+  // Publishes the next step's buffer (its copies were issued a step ago) and starts the
+  // copies of the step after it into the buffer that the previous step has finished with.
+  // The barrier needs no wait for this wave's LDS reads: the ones still in flight (stage L2 of
+  // the current tile) read the current step's buffer, not the one about to be overwritten.
+  auto publish = [&]() {
+    MG_ATTN_WAIT_VMCNT(0);
+    asm volatile("s_barrier" ::: "memory");
+  };
+  // One iteration of the walk for tile g, whose S / dP are in register set P (= g % 2, the
+  // tile's half of its step).  NEXT: tile g + 1 exists (stage A for it); NEXT2: tile g + 2
+  // exists (stage L1 for it); FRESH: the accumulators of tile g + 1 start from zero (not from
+  // the causal presets).
+  auto iteration = [&](auto PC, auto NEXT, auto NEXT2, auto FRESH, int g) {
+    constexpr int P = decltype(PC)::value;
+    using PN = std::integral_constant<int, P ^ 1>;
+    static_for<8>([&](auto CC) {
+      constexpr int c = decltype(CC)::value;
+      if (decltype(NEXT)::value) a_piece(PN{}, FRESH, c);
+      b_piece(PC, CC);
+      if (c >= 4) l2_piece(c - 4, P);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    pack_frags();
+    if (P == 0) publish();
+    const int step2 = g / 2 + 2;
+    const int buf2 = step2 % 3;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      c_piece(c);
+      if (decltype(NEXT2)::value) l1_piece(PC, c, P);
+      if (P == 0 && c < 5) issue_piece(c, step2, buf2);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (P == 1) {
+      advance_l1();
+      advance_l2();
+    }
+  };
+
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  using Yes = std::true_type;
+  using No = std::false_type;
+
+  issue_step(0, 0);
+  issue_step(1, 1);
+  MG_ATTN_WAIT_VMCNT(5);
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+  // Causal: wave w's keys meet the diagonal in tile w of the walk.  It joins the walk at the
+  // even tile gstart <= w (only the barriers and copies of the steps before that), with the
+  // diagonal folded into the start values of the S accumulators of its first two tiles:
+  // waves 0 and 2 mask the diagonal in their first tile; waves 1 and 3 see nothing in their
+  // first tile and the diagonal in their second.
+  const int gstart = CAUSAL ? min(wave_u & ~1, G) : 0;
+  for (int g = 0; g < gstart; g += 2) {
+    publish();
+    issue_step(g / 2 + 2, (g / 2 + 2) % 3);
+    advance_l1();
+    advance_l2();
+  }
+  if (gstart < G) {
+    const bool odd = CAUSAL && (wave_u & 1);
+    // Stage L1 of the first two tiles; the S accumulators then start from 0 (or -lse) where
+    // the key (column lane % 32) may see the query (row acc_row(r)) and from -inf where not.
+    if (STAT_DPP) {
+      s[0] = zero16(); s[1] = zero16(); dp[0] = zero16(); dp[1] = zero16();
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c) l1_piece(P0{}, c, 0);
+    if (CAUSAL) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[0][r] = (!odd && lane % 32 <= acc_row(r, lane)) ? s[0][r] : -INFINITY;
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c) a_piece(P0{}, No{}, c);
+#pragma unroll
+    for (int c = 0; c < 8; ++c) l1_piece(P1{}, c, 1);
+    if (CAUSAL) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[1][r] = (!odd || lane % 32 <= acc_row(r, lane)) ? s[1][r] : -INFINITY;
+    }
+    advance_l1();
+    using Fresh = std::integral_constant<bool, STAT_DPP>;  // without STAT_DPP stage L1 sets the accumulators
+    int g = gstart;
+    if (g + 2 < G) {
+      iteration(P0{}, Yes{}, Yes{}, No{}, g);
+      iteration(P1{}, Yes{}, Yes{}, Fresh{}, g + 1);
+      for (g += 2; g + 2 < G; g += 2) {
+        iteration(P0{}, Yes{}, Yes{}, Fresh{}, g);
+        iteration(P1{}, Yes{}, Yes{}, Fresh{}, g + 1);
+      }
+      iteration(P0{}, Yes{}, No{}, Fresh{}, g);
+    } else {
+      iteration(P0{}, Yes{}, No{}, No{}, g);
+    }
+    iteration(P1{}, No{}, No{}, Fresh{}, g + 1);
+  }
+
+  if (n < a.S) {
+    T* outk = dk + qkv_at(a, b, n, h);
+    T* outv = dv + qkv_at(a, b, n, h);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d = dt * 32 + g * 8 + half * 4;
+        if (d < a.D) {
+          store4<T>(outk + d, acc_k[dt], g, scale);
+          store4<T>(outv + d, acc_v[dt], g, 1.0f);
+        }
+      }
+  }
+}
+
 // ---- backward launches --------------------------------------------------------------------
 
 template <typename T, int DP, int MQ, bool CAUSAL, bool HAS_BIAS>
@@ -850,6 +1294,16 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
                                                                        T* __restrict__ dq, AttnDims a, float scale) {
   __shared__ __attribute__((aligned(16))) char smem[dq_lds_bytes<DP>()];
   attn_dq_block<T, DP, MQ, CAUSAL, HAS_BIAS>(blockIdx.x, smem, d_o, q, k, v, mask, lse, delta, dq, a, scale);
+}
+
+// The pipelined walk with a launch of its own.
+template <typename T, int DP, bool CAUSAL>
+__global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_pipe_kernel(
+    const T* __restrict__ d_o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+    const float* __restrict__ nlse, const float* __restrict__ ndelta, int s_pad, T* __restrict__ dk, T* __restrict__ dv,
+    AttnDims a, float scale) {
+  __shared__ __attribute__((aligned(1024))) char smem[dkdv_pipe_lds_bytes<DP>()];
+  attn_dkdv_pipe_block<T, DP, CAUSAL, MG_ATTN_STAT_DPP>(blockIdx.x, smem, d_o, q, k, v, nlse, ndelta, s_pad, dk, dv, a, scale);
 }
 
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
@@ -865,18 +1319,23 @@ __global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma
 // groups of eight consecutive workgroups alternate between dK/dV and dQ blocks, so every
 // XCD runs both kinds, and short sequences pay for one launch instead of two.  `blocks` is
 // the block count of each walk; the grid is 2 * round_up(blocks, 8) workgroups.
-template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
+template <typename T, int DP, bool CAUSAL, bool HAS_BIAS, bool PIPE>
 __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_mfma_kernel(
     const T* __restrict__ d_o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
     const T* __restrict__ mask, const float* __restrict__ lse, const float* __restrict__ delta, T* __restrict__ dq,
-    T* __restrict__ dk, T* __restrict__ dv, AttnDims a, float scale, int blocks) {
-  constexpr int LDS = dkdv_lds_bytes<DP, 64>() > dq_lds_bytes<DP>() ? dkdv_lds_bytes<DP, 64>() : dq_lds_bytes<DP>();
-  __shared__ __attribute__((aligned(16))) char smem[LDS];
+    T* __restrict__ dk, T* __restrict__ dv, AttnDims a, float scale, int blocks, const float* __restrict__ nlse,
+    const float* __restrict__ ndelta, int s_pad) {
+  constexpr int DKDV = PIPE ? dkdv_pipe_lds_bytes<DP>() : dkdv_lds_bytes<DP, 64>();
+  constexpr int LDS = DKDV > dq_lds_bytes<DP>() ? DKDV : dq_lds_bytes<DP>();
+  __shared__ __attribute__((aligned(1024))) char smem[LDS];
   const int block = (blockIdx.x / 16) * 8 + blockIdx.x % 8;
   if (block >= blocks) return;
-  if ((blockIdx.x / 8) % 2 == 0)
-    attn_dkdv_block<T, DP, 64, CAUSAL, HAS_BIAS>(block, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
-  else
+  if ((blockIdx.x / 8) % 2 == 0) {
+    if constexpr (PIPE)
+      attn_dkdv_pipe_block<T, DP, CAUSAL, MG_ATTN_STAT_DPP>(block, smem, d_o, q, k, v, nlse, ndelta, s_pad, dk, dv, a, scale);
+    else
+      attn_dkdv_block<T, DP, 64, CAUSAL, HAS_BIAS>(block, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
+  } else
     attn_dq_block<T, DP, 1, CAUSAL, HAS_BIAS>(block, smem, d_o, q, k, v, mask, lse, delta, dq, a, scale);
 }
 
@@ -914,7 +1373,7 @@ static int fwd_typed(const void* q, const void* k, const void* v, const void* ma
 template <typename T, int CPR>
 __global__ __launch_bounds__(256) void attn_delta_rows_kernel(const T* __restrict__ d_o, const T* __restrict__ o,
                                                               float* __restrict__ delta, int64_t rows, int S, int H,
-                                                              int o_bshd) {
+                                                              int o_bshd, AttnPaddedStats ps) {
   const int64_t chunk = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   const int64_t row = chunk / CPR;
   float acc = 0.f;
@@ -927,11 +1386,16 @@ __global__ __launch_bounds__(256) void attn_delta_rows_kernel(const T* __restric
   }
 #pragma unroll
   for (int w = 1; w < CPR; w *= 2) acc += __shfl_xor(acc, w);
-  if (row < rows && threadIdx.x % CPR == 0) delta[o_row_to_bhs(row, S, H, o_bshd)] = acc;
+  if (row < rows && threadIdx.x % CPR == 0) {
+    const int64_t idx = o_row_to_bhs(row, S, H, o_bshd);
+    delta[idx] = acc;
+    write_padded_stats(ps, idx, S, acc);
+  }
 }
 
 template <typename T>
-static int launch_delta(const T* d_o, const T* o, float* delta, int64_t rows, const AttnDims& a, hipStream_t stream) {
+static int launch_delta(const T* d_o, const T* o, float* delta, int64_t rows, const AttnDims& a, hipStream_t stream,
+                        AttnPaddedStats ps = {}) {
   const int D = a.D;
   const int cpr = D / 8;
   const bool vec = D % 8 == 0 && (cpr & (cpr - 1)) == 0 && cpr <= 16;
@@ -939,7 +1403,7 @@ static int launch_delta(const T* d_o, const T* o, float* delta, int64_t rows, co
     const dim3 grid(static_cast<unsigned>(ceil_div(rows * cpr, 256)));
 #define MG_DELTA(CPR_)                                                                                              \
   hipLaunchKernelGGL((attn_delta_rows_kernel<T, CPR_>), grid, dim3(256), 0, stream, d_o, o, delta, rows, a.S, a.H, \
-                     a.o_bshd)
+                     a.o_bshd, ps)
     switch (cpr) {
       case 1: MG_DELTA(1); break;
       case 2: MG_DELTA(2); break;
@@ -950,7 +1414,7 @@ static int launch_delta(const T* d_o, const T* o, float* delta, int64_t rows, co
 #undef MG_DELTA
   } else {
     hipLaunchKernelGGL((attn_delta_kernel<T>), dim3(static_cast<unsigned>(ceil_div(rows, 4))), dim3(256), 0, stream, d_o,
-                       o, delta, rows, D, a.S, a.H, a.o_bshd);
+                       o, delta, rows, D, a.S, a.H, a.o_bshd, ps);
   }
   MG_LAUNCH_CHECK();
   return MG_OK;
@@ -961,9 +1425,25 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
                      const float* lse, void* dq, void* dk, void* dv, AttnDims a, float scale, bool causal, bool has_bias,
                      hipStream_t stream) {
   const int64_t rows = static_cast<int64_t>(a.B) * a.H * a.S;
+  // The pipelined dK/dV walk (head dims up to 64, no bias) reads the row statistics negated
+  // and padded per (batch, head) to a multiple of 64 rows; the delta kernel writes both forms.
+  static const bool pipe_off = [] {
+    const char* e = std::getenv("MOGRAD_HIP_ATTN_DKDV_PIPE");
+    return e && e[0] == '0';
+  }();
+  const bool pipe = DP <= 64 && !has_bias && !pipe_off;
+  const int s_pad = static_cast<int>(ceil_div(a.S, 64) * 64);
+  const int64_t padded = pipe ? static_cast<int64_t>(a.B) * a.H * s_pad : 0;
   Scratch delta;
-  MG_TRY(delta.take(rows * static_cast<int64_t>(sizeof(float))));
-  MG_TRY(launch_delta(static_cast<const T*>(d_o), static_cast<const T*>(o), delta.as<float>(), rows, a, stream));
+  MG_TRY(delta.take((rows + 2 * padded) * static_cast<int64_t>(sizeof(float))));
+  AttnPaddedStats ps;
+  if (pipe) {
+    ps.lse = lse;
+    ps.nlse = delta.as<float>() + rows;
+    ps.ndelta = ps.nlse + padded;
+    ps.s_pad = s_pad;
+  }
+  MG_TRY(launch_delta(static_cast<const T*>(d_o), static_cast<const T*>(o), delta.as<float>(), rows, a, stream, ps));
   const int64_t blocks = static_cast<int64_t>(a.B) * a.H * ceil_div(a.S, 128);
   // One launch for both walks up to this sequence length (measured: 3-5% faster up to 512,
   // even at 1024, 2-3% slower from 2048 on, where the two walks compete for the same CU
@@ -987,10 +1467,24 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
   do {                                                                                                               \
     if constexpr (DP <= 64) {                                                                                        \
       if (fused) {                                                                                                   \
-        hipLaunchKernelGGL((attn_bwd_mfma_kernel<T, DP, C_, B_>), grid_fused, dim3(kAttnThreads), 0, stream, d_o_,   \
-                           q_, k_, v_, mask_, lse, delta.as<float>(), dq_, dk_, dv_, a, scale,                       \
-                           static_cast<int>(blocks));                                                                \
+        if (!B_ && pipe)                                                                                             \
+          hipLaunchKernelGGL((attn_bwd_mfma_kernel<T, DP, C_, B_, !B_>), grid_fused, dim3(kAttnThreads), 0, stream,  \
+                             d_o_, q_, k_, v_, mask_, lse, delta.as<float>(), dq_, dk_, dv_, a, scale,               \
+                             static_cast<int>(blocks), ps.nlse, ps.ndelta, s_pad);                                   \
+        else                                                                                                         \
+          hipLaunchKernelGGL((attn_bwd_mfma_kernel<T, DP, C_, B_, false>), grid_fused, dim3(kAttnThreads), 0,        \
+                             stream, d_o_, q_, k_, v_, mask_, lse, delta.as<float>(), dq_, dk_, dv_, a, scale,       \
+                             static_cast<int>(blocks), ps.nlse, ps.ndelta, s_pad);                                   \
         break;                                                                                                       \
+      }                                                                                                              \
+      if constexpr (!B_) {                                                                                           \
+        if (pipe) {                                                                                                  \
+          hipLaunchKernelGGL((attn_dkdv_pipe_kernel<T, DP, C_>), grid, dim3(kAttnThreads), 0, stream, d_o_, q_, k_,  \
+                             v_, ps.nlse, ps.ndelta, s_pad, dk_, dv_, a, scale);                                     \
+          hipLaunchKernelGGL((attn_dq_mfma_kernel<T, DP, 1, C_, B_>), grid, dim3(kAttnThreads), 0, stream, d_o_, q_, \
+                             k_, v_, mask_, lse, delta.as<float>(), dq_, a, scale);                                  \
+          break;                                                                                                     \
+        }                                                                                                            \
       }                                                                                                              \
     }                                                                                                                \
     hipLaunchKernelGGL((attn_dkdv_mfma_kernel<T, DP, C_, B_>), grid, dim3(kAttnThreads), 0, stream, d_o_, q_, k_,    \
