@@ -1283,6 +1283,279 @@ __device__ __forceinline__ void attn_dkdv_pipe_block(const int block, char* smem
   }
 }
 
+// ---- dQ: software-pipelined walk (head dim <= 64, no bias) -------------------------------
+// The same schedule as attn_dkdv_pipe_block with the roles exchanged: a wave keeps 32 queries
+// (Q pre-scaled and dO as B operands, -lse and -delta as the lane-constant start values of the
+// S^T and dP^T accumulators) and walks the keys in 32-key tiles, 64 keys per step through the
+// ring of three buffers:
+//   L1(g)  the eight row fragments of the K and V tile
+//   A(g)   S^T = K Q^T - lse, dP^T = V dO^T - delta   (eight MFMAs)
+//   B(g)   dS^T = exp2(S^T) dP^T, rounded and packed
+//   L2(g)  the transposed fragments of the K tile
+//   C(g)   dQ^T += K^T dS^T                             (four MFMAs)
+// The keys are walked from the last step down to the first.  The only tiles that need a mask
+// (keys past the end of the sequence; causal: keys after the query) are then in the first step
+// a wave takes part in, where the mask goes into the start values of the S^T accumulators of
+// its first two tiles; every later tile is unmasked.  Causal: a wave joins the walk at the
+// step that holds its last visible key.
+
+template <int DP>
+constexpr int dq_pipe_buf_bytes() {
+  return 2 * 64 * tile_row_bytes<DP>();  // a K tile and a V tile of 64 keys
+}
+template <int DP>
+constexpr int dq_pipe_lds_bytes() {
+  return 3 * dq_pipe_buf_bytes<DP>();
+}
+
+template <typename T, int DP, bool CAUSAL>
+__device__ __forceinline__ void attn_dq_pipe_block(const int block, char* smem, const T* __restrict__ d_o,
+                                                   const T* __restrict__ q, const T* __restrict__ k,
+                                                   const T* __restrict__ v, const float* __restrict__ lse,
+                                                   const float* __restrict__ delta, T* __restrict__ dq,
+                                                   const AttnDims& a, float scale) {
+  static_assert(DP == 64, "tile shapes below are written for a 64-wide head");
+  constexpr int BM = 128, BN = 64, KS = DP / 16, DT = DP / 32;
+  constexpr int ROWS = BN * tile_row_bytes<DP>();
+  constexpr int BUF = dq_pipe_buf_bytes<DP>();
+
+  const int nqb = (a.S + BM - 1) / BM;
+  const int n_bh = a.B * a.H;
+  const int qb = CAUSAL ? nqb - 1 - block / n_bh : block / n_bh;  // heaviest query blocks first
+  const int h = (block % n_bh) % a.H;
+  const int b = (block % n_bh) / a.H;
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int half = lane / 32;
+  const TileLane16<DP> at(lane);
+  const int m_wave = qb * BM + wave_u * 32;
+  const int m = m_wave + lane % 32;
+  const int64_t bh = static_cast<int64_t>(b) * a.H + h;
+
+  const float c = scale * kAttnLog2e;
+  uint4 qf[KS], dof[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d = ks * 16 + half * 8;
+    const bool ok = m < a.S && d < a.D;
+    qf[ks] = ok ? *reinterpret_cast<const uint4*>(q + qkv_at(a, b, m, h) + d) : make_uint4(0, 0, 0, 0);
+    qf[ks] = scale_frag<T>(qf[ks], c);
+    dof[ks] = ok ? *reinterpret_cast<const uint4*>(d_o + o_at(a, b, h, m) + d) : make_uint4(0, 0, 0, 0);
+  }
+  // Rows past the end get lse = +inf so that their probabilities vanish.
+  const float nlse2 = m < a.S ? -lse[bh * a.S + m] * kAttnLog2e : -INFINITY;
+  const float ndl = m < a.S ? -delta[bh * a.S + m] : 0.f;
+  const floatx16 s_init = splat16(nlse2), dp_init = splat16(ndl);
+  floatx16 acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
+
+  // Keys [0, n_end) in steps of 64, walked downwards: step i covers keys n_top - 64 (i + 1) ..
+  const int n_end = CAUSAL ? min(a.S, qb * BM + BM) : a.S;
+  const int nsteps = (n_end + BN - 1) / BN;
+  const int G = 2 * nsteps;
+  auto step_key0 = [&](int step) { return (nsteps - 1 - step) * BN; };
+
+  // ---- copies: step i -> buffer i % 3 (see attn_dkdv_pipe_block) ----
+  const int cp_row = lane / 8;
+  const int cp_chunk = (lane % 8) ^ tile_swz16(8 * (wave % 2) + cp_row);
+  const unsigned cp_col_bytes = cp_chunk * 8 < a.D ? cp_chunk * 16 : 0;
+  const char* k_bh = reinterpret_cast<const char*>(k + qkv_at(a, b, 0, h));
+  const char* v_bh = reinterpret_cast<const char*>(v + qkv_at(a, b, 0, h));
+  const unsigned pitch = static_cast<unsigned>(a.ld) * 2;
+  const unsigned smem_base = lds_address(smem);
+  // Copy c of 4 of step `step` (clamped to the walk's last step) into buffer `buf`: K rows, V
+  // rows, K rows, V rows.  Keys past the end of the sequence copy its last row.
+  auto issue_piece = [&](int c, int step, int buf) {
+    const int n0 = step_key0(min(step, nsteps - 1));
+    const int jj = c / 2;
+    const bool is_v = c % 2;
+    const int j = wave_u + 4 * jj;
+    const int row = min(8 * j + cp_row, a.S - 1 - n0);
+    const char* rows0 = (is_v ? v_bh : k_bh) + static_cast<int64_t>(n0) * pitch;
+    const unsigned dst = __builtin_amdgcn_readfirstlane(smem_base + buf * BUF + (is_v ? ROWS : 0) + j * 1024);
+    const unsigned off = row * pitch + cp_col_bytes;
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(rows0) : "memory");
+  };
+  auto issue_step = [&](int step, int buf) {
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc) issue_piece(cc, step, buf);
+  };
+
+  // ---- stages ----
+  floatx16 s[2], dp[2];
+  uint4 kr[KS], vr[KS], kt[2][DT], dsf[2];
+  uint32_t dw[8];
+  typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+  using lds_u4 = __attribute__((address_space(3))) const uintx4*;
+  using lds_i16x4 = __attribute__((address_space(3))) short4_t*;
+  unsigned ra[KS], tlo[DT], thi[DT];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) ra[ks] = smem_base + at.rows[ks];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    tlo[dt] = smem_base + at.tr_lo[dt];
+    thi[dt] = smem_base + at.tr_hi[dt];
+  }
+  int buf_l1 = 0, buf_l2 = 0;
+  auto advance_l1 = [&]() {
+    const int d = buf_l1 == 2 ? -2 * BUF : BUF;
+    buf_l1 = buf_l1 == 2 ? 0 : buf_l1 + 1;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ra[ks] += d;
+  };
+  auto advance_l2 = [&]() {
+    const int d = buf_l2 == 2 ? -2 * BUF : BUF;
+    buf_l2 = buf_l2 == 2 ? 0 : buf_l2 + 1;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      tlo[dt] += d;
+      thi[dt] += d;
+    }
+  };
+  auto read16 = [](unsigned addr) {
+    const uintx4 x = *reinterpret_cast<lds_u4>(static_cast<uintptr_t>(addr));
+    return make_uint4(x[0], x[1], x[2], x[3]);
+  };
+  auto read_tr = [](unsigned lo, unsigned hi) {
+    const short4_t l4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_i16x4>(static_cast<uintptr_t>(lo)));
+    const short4_t h4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_i16x4>(static_cast<uintptr_t>(hi)));
+    const uint2 l = __builtin_bit_cast(uint2, l4), h2 = __builtin_bit_cast(uint2, h4);
+    return make_uint4(l.x, l.y, h2.x, h2.y);
+  };
+  // L1 piece cc of 8 for the tile at rows mt*32 of the buffer `ra` points into.
+  auto l1_piece = [&](int cc, int mt) {
+    if (cc % 2 == 0) kr[cc / 2] = read16(ra[cc / 2] + mt * 32 * tile_row_bytes<DP>());
+    else vr[cc / 2] = read16(ra[cc / 2] + ROWS + mt * 32 * tile_row_bytes<DP>());
+  };
+  // MFMA cc of 8 of stage A into register set P; FRESH: start from -lse / -delta (not from the presets).
+  auto a_piece = [&](auto PC, auto FRESH, int cc) {
+    constexpr int P = decltype(PC)::value;
+    constexpr bool Z = decltype(FRESH)::value;
+    if (cc % 2 == 0) s[P] = Mma<T>::run(kr[cc / 2], qf[cc / 2], (Z && cc == 0) ? s_init : s[P]);
+    else dp[P] = Mma<T>::run(vr[cc / 2], dof[cc / 2], (Z && cc == 1) ? dp_init : dp[P]);
+  };
+  // VALU piece cc of 8 of stage B on register set P: elements 2cc and 2cc+1.
+  auto b_piece = [&](auto PC, int cc) {
+    constexpr int P = decltype(PC)::value;
+    const float p0 = fexp2(s[P][2 * cc]), p1 = fexp2(s[P][2 * cc + 1]);
+    dw[cc] = Mma<T>::pack2(p0 * dp[P][2 * cc], p1 * dp[P][2 * cc + 1]);
+    asm volatile("" : "+v"(dw[cc]));  // keeps the arithmetic under the MFMA issued before it
+  };
+  // L2 piece cc of 4: the transposed fragment of 16 of the K tile's rows for one 32-column block.
+  auto l2_piece = [&](int cc, int mt) {
+    const int hf = cc / 2, dt = cc % 2;
+    const int off = (mt * 2 + hf) * 16 * tile_row_bytes<DP>();
+    kt[hf][dt] = read_tr(tlo[dt] + off, thi[dt] + off);
+  };
+  // MFMA cc of 4 of stage C.
+  auto c_piece = [&](int cc) {
+    const int hf = cc / 2, dt = cc % 2;
+    acc[dt] = Mma<T>::run(kt[hf][dt], dsf[hf], acc[dt]);
+  };
+  auto publish = [&]() {
+    MG_ATTN_WAIT_VMCNT(0);
+    asm volatile("s_barrier" ::: "memory");
+  };
+  auto iteration = [&](auto PC, auto NEXT, auto NEXT2, auto FRESH, int g) {
+    constexpr int P = decltype(PC)::value;
+    using PN = std::integral_constant<int, P ^ 1>;
+#pragma unroll
+    for (int cc = 0; cc < 8; ++cc) {
+      if (decltype(NEXT)::value) a_piece(PN{}, FRESH, cc);
+      b_piece(PC, cc);
+      if (cc >= 4) l2_piece(cc - 4, P);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    dsf[0] = make_uint4(dw[0], dw[1], dw[2], dw[3]);
+    dsf[1] = make_uint4(dw[4], dw[5], dw[6], dw[7]);
+    if (P == 0) publish();
+    const int step2 = g / 2 + 2;
+    const int buf2 = step2 % 3;
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc) {
+      c_piece(cc);
+      if (decltype(NEXT2)::value) {
+        l1_piece(2 * cc, P);
+        l1_piece(2 * cc + 1, P);
+      }
+      if (P == 0) issue_piece(cc, step2, buf2);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (P == 1) {
+      advance_l1();
+      advance_l2();
+    }
+  };
+
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  using Yes = std::true_type;
+  using No = std::false_type;
+
+  issue_step(0, 0);
+  issue_step(1, 1);
+  MG_ATTN_WAIT_VMCNT(4);
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+  // Causal: the wave joins at the step that holds its last visible key, m_wave + 31.
+  const int first_step = CAUSAL ? max(0, nsteps - 1 - (m_wave + 31) / BN) : 0;
+  const int gstart = min(2 * first_step, G);
+  for (int g = 0; g < gstart; g += 2) {
+    publish();
+    issue_step(g / 2 + 2, (g / 2 + 2) % 3);
+    advance_l1();
+    advance_l2();
+  }
+  if (gstart < G) {
+    // The first two tiles: S^T accumulator r of tile t stands for key n0 + 32 t + acc_row(r); it
+    // starts from -lse if that key exists and (causal) does not come after this lane's query.
+    const int n0 = step_key0(gstart / 2);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = n0 + 32 * t + acc_row(r, lane);
+        const bool ok = key < a.S && (!CAUSAL || key <= m);
+        s[t][r] = ok ? nlse2 : -INFINITY;
+      }
+    dp[0] = dp_init;
+    dp[1] = dp_init;
+#pragma unroll
+    for (int cc = 0; cc < 8; ++cc) l1_piece(cc, 0);
+#pragma unroll
+    for (int cc = 0; cc < 8; ++cc) a_piece(P0{}, No{}, cc);
+#pragma unroll
+    for (int cc = 0; cc < 8; ++cc) l1_piece(cc, 1);
+    advance_l1();
+    int g = gstart;
+    if (g + 2 < G) {
+      iteration(P0{}, Yes{}, Yes{}, No{}, g);
+      iteration(P1{}, Yes{}, Yes{}, Yes{}, g + 1);
+      for (g += 2; g + 2 < G; g += 2) {
+        iteration(P0{}, Yes{}, Yes{}, Yes{}, g);
+        iteration(P1{}, Yes{}, Yes{}, Yes{}, g + 1);
+      }
+      iteration(P0{}, Yes{}, No{}, Yes{}, g);
+    } else {
+      iteration(P0{}, Yes{}, No{}, No{}, g);
+    }
+    iteration(P1{}, No{}, No{}, Yes{}, g + 1);
+  }
+
+  if (m < a.S) {
+    T* out = dq + qkv_at(a, b, m, h);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int d = dt * 32 + g4 * 8 + half * 4;
+        if (d < a.D) store4<T>(out + d, acc[dt], g4, scale);
+      }
+  }
+}
+
 // ---- backward launches --------------------------------------------------------------------
 
 template <typename T, int DP, int MQ, bool CAUSAL, bool HAS_BIAS>
@@ -1294,6 +1567,16 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* 
                                                                        T* __restrict__ dq, AttnDims a, float scale) {
   __shared__ __attribute__((aligned(16))) char smem[dq_lds_bytes<DP>()];
   attn_dq_block<T, DP, MQ, CAUSAL, HAS_BIAS>(blockIdx.x, smem, d_o, q, k, v, mask, lse, delta, dq, a, scale);
+}
+
+template <typename T, int DP, bool CAUSAL>
+__global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_pipe_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
+                                                                       const T* __restrict__ k, const T* __restrict__ v,
+                                                                       const float* __restrict__ lse,
+                                                                       const float* __restrict__ delta,
+                                                                       T* __restrict__ dq, AttnDims a, float scale) {
+  __shared__ __attribute__((aligned(1024))) char smem[dq_pipe_lds_bytes<DP>()];
+  attn_dq_pipe_block<T, DP, CAUSAL>(blockIdx.x, smem, d_o, q, k, v, lse, delta, dq, a, scale);
 }
 
 // The pipelined walk with a launch of its own.
@@ -1335,8 +1618,12 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_mfma_kernel(
       attn_dkdv_pipe_block<T, DP, CAUSAL, MG_ATTN_STAT_DPP>(block, smem, d_o, q, k, v, nlse, ndelta, s_pad, dk, dv, a, scale);
     else
       attn_dkdv_block<T, DP, 64, CAUSAL, HAS_BIAS>(block, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
-  } else
-    attn_dq_block<T, DP, 1, CAUSAL, HAS_BIAS>(block, smem, d_o, q, k, v, mask, lse, delta, dq, a, scale);
+  } else {
+    if constexpr (PIPE)
+      attn_dq_pipe_block<T, DP, CAUSAL>(block, smem, d_o, q, k, v, lse, delta, dq, a, scale);
+    else
+      attn_dq_block<T, DP, 1, CAUSAL, HAS_BIAS>(block, smem, d_o, q, k, v, mask, lse, delta, dq, a, scale);
+  }
 }
 
 // ---- host side ---------------------------------------------------------------------------
@@ -1481,8 +1768,8 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
         if (pipe) {                                                                                                  \
           hipLaunchKernelGGL((attn_dkdv_pipe_kernel<T, DP, C_>), grid, dim3(kAttnThreads), 0, stream, d_o_, q_, k_,  \
                              v_, ps.nlse, ps.ndelta, s_pad, dk_, dv_, a, scale);                                     \
-          hipLaunchKernelGGL((attn_dq_mfma_kernel<T, DP, 1, C_, B_>), grid, dim3(kAttnThreads), 0, stream, d_o_, q_, \
-                             k_, v_, mask_, lse, delta.as<float>(), dq_, a, scale);                                  \
+          hipLaunchKernelGGL((attn_dq_pipe_kernel<T, DP, C_>), grid, dim3(kAttnThreads), 0, stream, d_o_, q_, k_,    \
+                             v_, lse, delta.as<float>(), dq_, a, scale);                                             \
           break;                                                                                                     \
         }                                                                                                            \
       }                                                                                                              \
