@@ -931,9 +931,15 @@ template <int DP>
 constexpr int dkdv_pipe_buf_bytes() {
   return 2 * 64 * tile_row_bytes<DP>() + 2 * 64 * 4;  // a Q tile, a dO tile, -lse, -delta of 64 queries
 }
+// Buffers in the ring of the pipelined walks: the copies of a step are issued kAttnRing - 1
+// steps before the step is read.
+#ifndef MG_ATTN_RING
+#define MG_ATTN_RING 3
+#endif
+constexpr int kAttnRing = MG_ATTN_RING;
 template <int DP>
 constexpr int dkdv_pipe_lds_bytes() {
-  return 3 * dkdv_pipe_buf_bytes<DP>();
+  return kAttnRing * dkdv_pipe_buf_bytes<DP>();
 }
 
 // s_waitcnt with only the vector-memory counter set (vmcnt in bits 3:0 and 15:14, the
@@ -956,9 +962,11 @@ __device__ __forceinline__ void copy4_to_lds(unsigned lds_wave_base, const void*
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(dst), "v"(src) : "memory");
 }
 
-#ifndef MG_ATTN_STAT_DPP
-#define MG_ATTN_STAT_DPP false
-#endif
+// (The row statistics were also tried as one 4-byte LDS read per lane and tile, handed to
+// the accumulator registers' rows by DPP row broadcasts inside stage B: eight fewer 16-byte LDS
+// reads per tile, two more VALU operations per element, 226 us against 209 us for the S = 4096
+// walk: the VALU is the scarcer resource here.)
+constexpr bool kAttnStatDpp = false;
 template <typename T, int DP, bool CAUSAL, bool STAT_DPP>
 __device__ __forceinline__ void attn_dkdv_pipe_block(const int block, char* smem, const T* __restrict__ d_o,
                                                      const T* __restrict__ q, const T* __restrict__ k,
@@ -1002,7 +1010,7 @@ __device__ __forceinline__ void attn_dkdv_pipe_block(const int block, char* smem
   const int nsteps = (a.S - m_begin + BQ - 1) / BQ;
   const int G = 2 * nsteps;
 
-  // ---- copies: step i -> buffer i % 3 ----
+  // ---- copies: step i -> buffer i % kAttnRing ----
   // Wave-instruction j of a tile covers its rows 8j .. 8j+7 (1 KB); this wave issues j = wave
   // and wave + 4 for Q and for dO.  Lane l writes chunk position l % 8 of row 8j + l / 8 and
   // therefore names the source chunk (l % 8) ^ swz16(row), with row % 16 = 8 (wave % 2) + l / 8.
@@ -1082,15 +1090,15 @@ __device__ __forceinline__ void attn_dkdv_pipe_block(const int block, char* smem
   }
   int buf_l1 = 0, buf_l2 = 0;  // which buffer each group points into
   auto advance_l1 = [&]() {
-    const int d = buf_l1 == 2 ? -2 * BUF : BUF;
-    buf_l1 = buf_l1 == 2 ? 0 : buf_l1 + 1;
+    const int d = buf_l1 == kAttnRing - 1 ? -(kAttnRing - 1) * BUF : BUF;
+    buf_l1 = buf_l1 == kAttnRing - 1 ? 0 : buf_l1 + 1;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) ra[ks] += d;
     sa += d;
   };
   auto advance_l2 = [&]() {
-    const int d = buf_l2 == 2 ? -2 * BUF : BUF;
-    buf_l2 = buf_l2 == 2 ? 0 : buf_l2 + 1;
+    const int d = buf_l2 == kAttnRing - 1 ? -(kAttnRing - 1) * BUF : BUF;
+    buf_l2 = buf_l2 == kAttnRing - 1 ? 0 : buf_l2 + 1;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       tlo[dt] += d;
@@ -1173,7 +1181,7 @@ __device__ __forceinline__ void attn_dkdv_pipe_block(const int block, char* smem
   // The barrier needs no wait for this wave's LDS reads: the ones still in flight (stage L2 of
   // the current tile) read the current step's buffer, not the one about to be overwritten.
   auto publish = [&]() {
-    MG_ATTN_WAIT_VMCNT(0);
+    MG_ATTN_WAIT_VMCNT((kAttnRing - 3) * 5);  // all but the younger steps' copies
     asm volatile("s_barrier" ::: "memory");
   };
   // One iteration of the walk for tile g, whose S / dP are in register set P (= g % 2, the
@@ -1192,8 +1200,8 @@ __device__ __forceinline__ void attn_dkdv_pipe_block(const int block, char* smem
     });
     pack_frags();
     if (P == 0) publish();
-    const int step2 = g / 2 + 2;
-    const int buf2 = step2 % 3;
+    const int step2 = g / 2 + kAttnRing - 1;
+    const int buf2 = step2 % kAttnRing;
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
       c_piece(c);
@@ -1212,9 +1220,9 @@ __device__ __forceinline__ void attn_dkdv_pipe_block(const int block, char* smem
   using Yes = std::true_type;
   using No = std::false_type;
 
-  issue_step(0, 0);
-  issue_step(1, 1);
-  MG_ATTN_WAIT_VMCNT(5);
+#pragma unroll
+  for (int st = 0; st < kAttnRing - 1; ++st) issue_step(st, st);
+  MG_ATTN_WAIT_VMCNT((kAttnRing - 2) * 5);
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
   // Causal: wave w's keys meet the diagonal in tile w of the walk.  It joins the walk at the
@@ -1225,7 +1233,7 @@ __device__ __forceinline__ void attn_dkdv_pipe_block(const int block, char* smem
   const int gstart = CAUSAL ? min(wave_u & ~1, G) : 0;
   for (int g = 0; g < gstart; g += 2) {
     publish();
-    issue_step(g / 2 + 2, (g / 2 + 2) % 3);
+    issue_step(g / 2 + kAttnRing - 1, (g / 2 + kAttnRing - 1) % kAttnRing);
     advance_l1();
     advance_l2();
   }
@@ -1305,7 +1313,7 @@ constexpr int dq_pipe_buf_bytes() {
 }
 template <int DP>
 constexpr int dq_pipe_lds_bytes() {
-  return 3 * dq_pipe_buf_bytes<DP>();
+  return kAttnRing * dq_pipe_buf_bytes<DP>();
 }
 
 template <typename T, int DP, bool CAUSAL>
@@ -1357,7 +1365,7 @@ __device__ __forceinline__ void attn_dq_pipe_block(const int block, char* smem, 
   const int G = 2 * nsteps;
   auto step_key0 = [&](int step) { return (nsteps - 1 - step) * BN; };
 
-  // ---- copies: step i -> buffer i % 3 (see attn_dkdv_pipe_block) ----
+  // ---- copies: step i -> buffer i % kAttnRing (see attn_dkdv_pipe_block) ----
   const int cp_row = lane / 8;
   const int cp_chunk = (lane % 8) ^ tile_swz16(8 * (wave % 2) + cp_row);
   const unsigned cp_col_bytes = cp_chunk * 8 < a.D ? cp_chunk * 16 : 0;
@@ -1400,14 +1408,14 @@ __device__ __forceinline__ void attn_dq_pipe_block(const int block, char* smem, 
   }
   int buf_l1 = 0, buf_l2 = 0;
   auto advance_l1 = [&]() {
-    const int d = buf_l1 == 2 ? -2 * BUF : BUF;
-    buf_l1 = buf_l1 == 2 ? 0 : buf_l1 + 1;
+    const int d = buf_l1 == kAttnRing - 1 ? -(kAttnRing - 1) * BUF : BUF;
+    buf_l1 = buf_l1 == kAttnRing - 1 ? 0 : buf_l1 + 1;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) ra[ks] += d;
   };
   auto advance_l2 = [&]() {
-    const int d = buf_l2 == 2 ? -2 * BUF : BUF;
-    buf_l2 = buf_l2 == 2 ? 0 : buf_l2 + 1;
+    const int d = buf_l2 == kAttnRing - 1 ? -(kAttnRing - 1) * BUF : BUF;
+    buf_l2 = buf_l2 == kAttnRing - 1 ? 0 : buf_l2 + 1;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       tlo[dt] += d;
@@ -1455,7 +1463,7 @@ __device__ __forceinline__ void attn_dq_pipe_block(const int block, char* smem, 
     acc[dt] = Mma<T>::run(kt[hf][dt], dsf[hf], acc[dt]);
   };
   auto publish = [&]() {
-    MG_ATTN_WAIT_VMCNT(0);
+    MG_ATTN_WAIT_VMCNT((kAttnRing - 3) * 4);  // all but the younger steps' copies
     asm volatile("s_barrier" ::: "memory");
   };
   auto iteration = [&](auto PC, auto NEXT, auto NEXT2, auto FRESH, int g) {
@@ -1471,8 +1479,8 @@ __device__ __forceinline__ void attn_dq_pipe_block(const int block, char* smem, 
     dsf[0] = make_uint4(dw[0], dw[1], dw[2], dw[3]);
     dsf[1] = make_uint4(dw[4], dw[5], dw[6], dw[7]);
     if (P == 0) publish();
-    const int step2 = g / 2 + 2;
-    const int buf2 = step2 % 3;
+    const int step2 = g / 2 + kAttnRing - 1;
+    const int buf2 = step2 % kAttnRing;
 #pragma unroll
     for (int cc = 0; cc < 4; ++cc) {
       c_piece(cc);
@@ -1494,9 +1502,9 @@ __device__ __forceinline__ void attn_dq_pipe_block(const int block, char* smem, 
   using Yes = std::true_type;
   using No = std::false_type;
 
-  issue_step(0, 0);
-  issue_step(1, 1);
-  MG_ATTN_WAIT_VMCNT(4);
+#pragma unroll
+  for (int st = 0; st < kAttnRing - 1; ++st) issue_step(st, st);
+  MG_ATTN_WAIT_VMCNT((kAttnRing - 2) * 4);
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
   // Causal: the wave joins at the step that holds its last visible key, m_wave + 31.
@@ -1504,7 +1512,7 @@ __device__ __forceinline__ void attn_dq_pipe_block(const int block, char* smem, 
   const int gstart = min(2 * first_step, G);
   for (int g = 0; g < gstart; g += 2) {
     publish();
-    issue_step(g / 2 + 2, (g / 2 + 2) % 3);
+    issue_step(g / 2 + kAttnRing - 1, (g / 2 + kAttnRing - 1) % kAttnRing);
     advance_l1();
     advance_l2();
   }
@@ -1586,7 +1594,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_dkdv_pipe_kernel(
     const float* __restrict__ nlse, const float* __restrict__ ndelta, int s_pad, T* __restrict__ dk, T* __restrict__ dv,
     AttnDims a, float scale) {
   __shared__ __attribute__((aligned(1024))) char smem[dkdv_pipe_lds_bytes<DP>()];
-  attn_dkdv_pipe_block<T, DP, CAUSAL, MG_ATTN_STAT_DPP>(blockIdx.x, smem, d_o, q, k, v, nlse, ndelta, s_pad, dk, dv, a, scale);
+  attn_dkdv_pipe_block<T, DP, CAUSAL, kAttnStatDpp>(blockIdx.x, smem, d_o, q, k, v, nlse, ndelta, s_pad, dk, dv, a, scale);
 }
 
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
@@ -1615,7 +1623,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_mfma_kernel(
   if (block >= blocks) return;
   if ((blockIdx.x / 8) % 2 == 0) {
     if constexpr (PIPE)
-      attn_dkdv_pipe_block<T, DP, CAUSAL, MG_ATTN_STAT_DPP>(block, smem, d_o, q, k, v, nlse, ndelta, s_pad, dk, dv, a, scale);
+      attn_dkdv_pipe_block<T, DP, CAUSAL, kAttnStatDpp>(block, smem, d_o, q, k, v, nlse, ndelta, s_pad, dk, dv, a, scale);
     else
       attn_dkdv_block<T, DP, 64, CAUSAL, HAS_BIAS>(block, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
   } else {
