@@ -3,6 +3,8 @@
 // (mograd/nn/optim/adam.mojo:6-78, sgd.mojo:24-45); the arithmetic and its order are the
 // same here, in one pass: 28 bytes moved per parameter for Adam, 12 for SGD.
 #include "mg_device.h"
+#include <cmath>
+
 #include "mg_internal.h"
 
 // No fused multiply-add contraction in this file: each operation of an update is rounded
@@ -97,12 +99,12 @@ int mg_adam_step(void* w, const void* g, void* m, void* v, int64_t n, float lr, 
   if (!w || !g || !m || !v) return mg::fail(MG_ERR_INVALID, "adam_step: null pointer argument");
   if (!mg::aligned16(w) || !mg::aligned16(g) || !mg::aligned16(m) || !mg::aligned16(v))
     return mg::fail(MG_ERR_INVALID, "adam_step: pointers must be 16-byte aligned");
-  // Bias corrections in fp32 like the reference (`Float32(1.0) - beta1**t`).
-  float b1t = 1.f, b2t = 1.f;
-  for (int64_t i = 0; i < t && (b1t != 0.f || b2t != 0.f); ++i) {
-    b1t *= beta1;
-    b2t *= beta2;
-  }
+  // Bias corrections `Float32(1.0) - beta**t` (mograd/nn/optim/adam.mojo:19-20).  The power is
+  // taken in double and rounded to fp32 once: constant time in t, and within one fp32 rounding
+  // of the exact value however large the step count (a chain of t fp32 multiplications costs
+  // O(t) host time per call and drifts by up to t/2 ulp).
+  const float b1t = static_cast<float>(std::pow(static_cast<double>(beta1), static_cast<double>(t)));
+  const float b2t = static_cast<float>(std::pow(static_cast<double>(beta2), static_cast<double>(t)));
   mg::AdamParams p{lr,
                    beta1,
                    beta2,

@@ -575,6 +575,113 @@ inline Buffers argmax(const OpRef& node, const Buffers& inputs, Device& device) 
   return {out};
 }
 
+// ---- Exec functions of the fused nodes that the gradient rules below emit -----------------------------
+// No counterpart in the reference: its Linear backward is matmul_grad + transpose_grad +
+// expand_grad (mograd/grad.mojo:180-187,278-288), its LAYER_NORM has one output
+// (mograd/runtime/__init__.mojo:425-426) and its labels are dense.  They follow the pattern of
+// its multi-output FLASH_ATTN / FLASH_ATTN_GRAD pair (mograd/grad.mojo:309-344).
+
+// LINEAR_GRAD[dY (.., N), X (.., K), W (N, K)]{has_bias} -> [dX, dW (N, K), db (N)] for Y = X W^T (+ b).
+inline Buffers linear_bwd(const OpRef& node, const Buffers& in, Device& device) {
+  const Layout &ldy = node.src(0).layout(), &lx = node.src(1).layout(), &lw = node.src(2).layout();
+  const Buffers inputs = detail::materialise(node, in, device, 3);
+  detail::require_float(node.dtype(), "linear_bwd");
+  if (lw.rank() != 2) throw Error(MG_ERR_INVALID, "linear_bwd: dY, X and W do not describe Y = X W^T");
+  const int64_t N = lw.shape(0), K = lw.shape(1), M = lx.numel() / K;
+  if (ldy.numel() != M * N) throw Error(MG_ERR_INVALID, "linear_bwd: dY, X and W do not describe Y = X W^T");
+  const bool has_bias = !node.has_attr("has_bias") || node.attr("has_bias") != 0;
+  AnyBuffer dx = AnyBuffer::create(node.dtype(), device, M * K);
+  AnyBuffer dw = AnyBuffer::create(node.dtype(), device, N * K);
+  Buffers out = {dx, dw};
+  void* db_ptr = nullptr;
+  if (has_bias) {
+    out.push_back(AnyBuffer::create(node.dtype(), device, N));
+    db_ptr = out.back().data_ptr();
+  }
+  MOGRAD_CALL(device, mg_linear_bwd, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), dx.data_ptr(),
+              dw.data_ptr(), db_ptr, M, N, K, node.dtype(), device.stream());
+  return out;
+}
+
+// LAYER_NORM_STATS[x, gamma, beta]{eps} -> [y, mean (rows) f32, rstd (rows) f32].
+inline Buffers layer_norm_fwd_stats(const OpRef& node, const Buffers& inputs, Device& device) {
+  const Layout& x = node.src(0).layout();
+  const int64_t cols = x.shape(x.rank() - 1), rows = x.numel() / cols;
+  detail::require_float(node.dtype(), "layer_norm_fwd_stats");
+  AnyBuffer out = AnyBuffer::create(node.dtype(), device, node.numel());
+  AnyBuffer mean = AnyBuffer::create(float32, device, rows);
+  AnyBuffer rstd = AnyBuffer::create(float32, device, rows);
+  MOGRAD_CALL(device, mg_layer_norm_fwd_stats, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+              out.data_ptr(), static_cast<float*>(mean.data_ptr()), static_cast<float*>(rstd.data_ptr()), rows, cols,
+              static_cast<float>(node.attr("eps")),
+              node.dtype(), device.stream());
+  return {out, mean, rstd};
+}
+
+// LAYER_NORM_STATS_GRAD[dy, x, gamma, mean, rstd] -> [dx, dgamma, dbeta].
+inline Buffers layer_norm_bwd_stats(const OpRef& node, const Buffers& inputs, Device& device) {
+  const Layout& x = node.src(1).layout();
+  const Layout& gamma = node.src(2).layout();
+  const int64_t cols = x.shape(x.rank() - 1), rows = x.numel() / cols;
+  detail::require_float(node.dtype(), "layer_norm_bwd_stats");
+  AnyBuffer dx = AnyBuffer::create(node.dtype(), device, x.numel());
+  AnyBuffer dgamma = AnyBuffer::create(node.dtype(), device, gamma.numel());
+  AnyBuffer dbeta = AnyBuffer::create(node.dtype(), device, gamma.numel());
+  MOGRAD_CALL(device, mg_layer_norm_bwd_stats, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+              static_cast<const float*>(inputs[3].data_ptr()), static_cast<const float*>(inputs[4].data_ptr()),
+              dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(), rows, cols, node.dtype(), device.stream());
+  return {dx, dgamma, dbeta};
+}
+
+// CROSS_ENTROPY_IDS[logits (.., C), ids (..) int32/int64] -> (1,).
+inline Buffers cross_entropy_ids(const OpRef& node, const Buffers& in, Device& device) {
+  const Layout& la = node.src(0).layout();
+  const Buffers inputs = detail::materialise(node, in, device, 2);
+  detail::require_float(node.dtype(), "cross_entropy_ids");
+  const int64_t C = la.shape(la.rank() - 1), N = la.numel() / C;
+  AnyBuffer out = AnyBuffer::create(node.dtype(), device, node.numel());
+  MOGRAD_CALL(device, mg_cross_entropy_ids, inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), N, C, node.dtype(),
+              node.src(1).dtype(), device.stream());
+  return {out};
+}
+
+// CROSS_ENTROPY_IDS_GRAD[logits, ids, upstream (1,)] -> dlogits.
+inline Buffers cross_entropy_grad_ids(const OpRef& node, const Buffers& in, Device& device) {
+  const Layout& la = node.src(0).layout();
+  const Buffers inputs = detail::materialise(node, in, device, 2);
+  detail::require_float(node.dtype(), "cross_entropy_grad_ids");
+  const int64_t C = la.shape(la.rank() - 1), N = la.numel() / C;
+  AnyBuffer out = AnyBuffer::create(node.dtype(), device, node.numel());
+  MOGRAD_CALL(device, mg_cross_entropy_grad_ids, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+              out.data_ptr(), N, C, node.dtype(), node.src(1).dtype(), device.stream());
+  return {out};
+}
+
+// ---- Gradient rules (GradFn, mograd/grad.mojo:12): node + upstream -> the multi-output node that
+// computes every source's gradient.  The C++ side keeps the rules that the reference lacks
+// (mograd/grad.mojo:30-65 has none for MATMUL_BT / MATMUL_BIAS_BT); output i of the returned node is
+// the gradient of source i, which the caller selects as the reference selects with GETTUPLE. ----------
+
+// MATMUL_BIAS_BT[X, W, b] or MATMUL_BT[X, W], upstream dY -> LINEAR_GRAD[dY, X, W]{has_bias}.
+inline OpRef linear_grad(const OpRef& node, const OpRef& upstream) {
+  const bool has_bias = node.op_type == "MATMUL_BIAS_BT";
+  return OpRef{"LINEAR_GRAD", node.src(0).layout().as_contiguous(), node.src(0).dtype(),
+               {upstream, node.src(0), node.src(1)}, {{"has_bias", has_bias ? 1.0 : 0.0}}};
+}
+
+// LAYER_NORM_STATS[x, gamma, beta] with its outputs 1 and 2 (mean, rstd) given as leaves ->
+// LAYER_NORM_STATS_GRAD[dy, x, gamma, mean, rstd].
+inline OpRef layer_norm_stats_grad(const OpRef& node, const OpRef& upstream, const OpRef& mean, const OpRef& rstd) {
+  return OpRef{"LAYER_NORM_STATS_GRAD", node.src(0).layout().as_contiguous(), node.src(0).dtype(),
+               {upstream, node.src(0), node.src(1), mean, rstd}, {}};
+}
+
+// CROSS_ENTROPY_IDS[logits, ids], upstream (1,) -> CROSS_ENTROPY_IDS_GRAD[logits, ids, upstream].
+inline OpRef cross_entropy_ids_grad(const OpRef& node, const OpRef& upstream) {
+  return OpRef{"CROSS_ENTROPY_IDS_GRAD", node.src(0).layout().as_contiguous(), node.src(0).dtype(),
+               {node.src(0), node.src(1), upstream}, {}};
+}
+
 // ---- Rule table (mograd/runtime/__init__.mojo:113-167) --------------------------------------------------
 
 struct Rule {
@@ -606,6 +713,12 @@ inline const std::vector<Rule>& scheduler_rules() {
       {"FLASH_ATTN_GRAD", "flash_attn_bwd_sched", flash_attn_bwd_sched},
       {"CROSS_ENTROPY", "cross_entropy", cross_entropy},
       {"CROSS_ENTROPY_GRAD", "cross_entropy_grad", cross_entropy_grad},
+      // fused nodes emitted by the gradient rules above (no counterpart in the reference's table)
+      {"LINEAR_GRAD", "linear_bwd", linear_bwd},
+      {"LAYER_NORM_STATS", "layer_norm_fwd_stats", layer_norm_fwd_stats},
+      {"LAYER_NORM_STATS_GRAD", "layer_norm_bwd_stats", layer_norm_bwd_stats},
+      {"CROSS_ENTROPY_IDS", "cross_entropy_ids", cross_entropy_ids},
+      {"CROSS_ENTROPY_IDS_GRAD", "cross_entropy_grad_ids", cross_entropy_grad_ids},
   };
   return rules;
 }

@@ -25,7 +25,7 @@ from . import _lib
 from ._lib import BF16, F16, F32, I32, I64, MogradError
 
 __all__ = [
-    "Layout", "Device", "AnyBuffer", "Node", "SCHEDULER_RULES", "MogradError",
+    "Layout", "Device", "AnyBuffer", "Node", "SCHEDULER_RULES", "GRAD_RULES", "gradient", "evaluate", "MogradError",
     "float32", "float16", "bfloat16", "int32", "int64",
 ]
 
@@ -291,7 +291,7 @@ class AnyBuffer:
 # --------------------------------------------------------------------------- #
 
 
-@dataclass
+@dataclass(eq=False)
 class Node:
     """Just enough of an op node for the exec functions: its own layout and dtype, the
     layouts of its sources, and its attributes (mograd/op.mojo:124-185)."""
@@ -301,6 +301,9 @@ class Node:
     node_dtype: int
     srcs: List["Node"] = field(default_factory=list)
     node_attrs: Dict[str, object] = field(default_factory=dict)
+    # What the reference keeps in op().buf (mograd/scheduler.mojo:74-78): a leaf's buffer, or
+    # the cached results of an evaluated node (several for a multi-output node).
+    bufs: Optional[List["AnyBuffer"]] = field(default=None, repr=False, compare=False)
 
     def layout(self) -> Layout:
         return self.node_layout
@@ -321,8 +324,14 @@ class Node:
         return self.node_layout.shape(i)
 
     @staticmethod
-    def leaf(layout: Layout, dtype: int = F32) -> "Node":
-        return Node("BUFFER", layout, dtype)
+    def leaf(layout: Layout, dtype: int = F32, buf: Optional["AnyBuffer"] = None) -> "Node":
+        return Node("BUFFER", layout, dtype, bufs=None if buf is None else [buf])
+
+    def __hash__(self) -> int:  # nodes are graph vertices: identity, like OpRef
+        return id(self)
+
+    def __eq__(self, other) -> bool:
+        return self is other
 
 
 def _require_float(dtype: int, who: str) -> None:
@@ -640,6 +649,93 @@ def argmax(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffe
     return [out]
 
 
+# --------------------------------------------------------------------------- #
+# Exec functions for the fused nodes that the gradient rules below emit.  The reference has
+# no counterpart for them: its Linear backward is matmul_grad + transpose_grad + expand_grad
+# (mograd/grad.mojo:180-187,278-288), its LAYER_NORM has one output
+# (mograd/runtime/__init__.mojo:425-426) and its labels are dense.  They follow the pattern
+# of its multi-output FLASH_ATTN / FLASH_ATTN_GRAD pair (mograd/grad.mojo:309-344).
+# --------------------------------------------------------------------------- #
+
+
+def linear_bwd(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """LINEAR_GRAD[dY (.., N), X (.., K), W (N, K)]{has_bias} -> [dX (.., K), dW (N, K), db (N)]
+    for Y = X W^T (+ b): dX = dY W, dW = dY^T X written in W's layout, db = column sums of dY
+    (two results without has_bias).  Leading dimensions collapse into the row count."""
+    ldy, lx, lw = (node.src(i).layout() for i in range(3))
+    inputs = _materialise(node, inputs, device, 3)
+    _require_float(node.dtype(), "linear_bwd")
+    N, K = lw.shape(0), lw.shape(1)
+    M = lx.numel() // K
+    if ldy.numel() != M * N or lw.rank() != 2:
+        raise MogradError(1, "linear_bwd: dY, X and W do not describe Y = X W^T")
+    has_bias = bool(node.attrs().get("has_bias", True))
+    dx = AnyBuffer.create(node.dtype(), device, M * K)
+    dw = AnyBuffer.create(node.dtype(), device, N * K)
+    db = AnyBuffer.create(node.dtype(), device, N) if has_bias else None
+    device.lib.mg_linear_bwd(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), dx.data_ptr(),
+                             dw.data_ptr(), db.data_ptr() if has_bias else None, M, N, K, node.dtype(), device.stream)
+    return [dx, dw, db] if has_bias else [dx, dw]
+
+
+def layer_norm_fwd_stats(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """LAYER_NORM_STATS[x, gamma, beta]{eps} -> [y, mean (rows) f32, rstd (rows) f32]: the
+    forward as a multi-output node, so that the backward reuses the row statistics."""
+    x_layout = node.src(0).layout()
+    cols = x_layout.shape(x_layout.rank() - 1)
+    rows = x_layout.numel() // cols
+    _require_float(node.dtype(), "layer_norm_fwd_stats")
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    mean = AnyBuffer.create(F32, device, rows)
+    rstd = AnyBuffer.create(F32, device, rows)
+    device.lib.mg_layer_norm_fwd_stats(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+                                       out.data_ptr(), mean.data_ptr(), rstd.data_ptr(), rows, cols,
+                                       float(node.attrs()["eps"]), node.dtype(), device.stream)
+    return [out, mean, rstd]
+
+
+def layer_norm_bwd_stats(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """LAYER_NORM_STATS_GRAD[dy, x, gamma, mean, rstd] -> [dx, dgamma, dbeta]."""
+    x_layout = node.src(1).layout()
+    gamma_layout = node.src(2).layout()
+    cols = x_layout.shape(x_layout.rank() - 1)
+    rows = x_layout.numel() // cols
+    _require_float(node.dtype(), "layer_norm_bwd_stats")
+    dx = AnyBuffer.create(node.dtype(), device, x_layout.numel())
+    dgamma = AnyBuffer.create(node.dtype(), device, gamma_layout.numel())
+    dbeta = AnyBuffer.create(node.dtype(), device, gamma_layout.numel())
+    device.lib.mg_layer_norm_bwd_stats(*(inputs[i].data_ptr() for i in range(5)), dx.data_ptr(), dgamma.data_ptr(),
+                                       dbeta.data_ptr(), rows, cols, node.dtype(), device.stream)
+    return [dx, dgamma, dbeta]
+
+
+def cross_entropy_ids(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """CROSS_ENTROPY_IDS[logits (.., C), ids (..) int32/int64] -> (1,): labels as class ids
+    instead of the reference's one_hot(...).cast(f32) rows."""
+    la = node.src(0).layout()
+    inputs = _materialise(node, inputs, device, 2)
+    _require_float(node.dtype(), "cross_entropy_ids")
+    C_ = la.shape(la.rank() - 1)
+    N = la.numel() // C_
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_cross_entropy_ids(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), N, C_, node.dtype(),
+                                    node.src(1).dtype(), device.stream)
+    return [out]
+
+
+def cross_entropy_grad_ids(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """CROSS_ENTROPY_IDS_GRAD[logits, ids, upstream (1,)] -> dlogits."""
+    la = node.src(0).layout()
+    inputs = _materialise(node, inputs, device, 2)
+    _require_float(node.dtype(), "cross_entropy_grad_ids")
+    C_ = la.shape(la.rank() - 1)
+    N = la.numel() // C_
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_cross_entropy_grad_ids(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+                                         out.data_ptr(), N, C_, node.dtype(), node.src(1).dtype(), device.stream)
+    return [out]
+
+
 # Op type -> exec function, the rows of the reference's rule table that belong to this
 # path (mograd/runtime/__init__.mojo:113-167).
 SCHEDULER_RULES = {
@@ -663,6 +759,12 @@ SCHEDULER_RULES = {
     "FLASH_ATTN_GRAD": flash_attn_bwd_sched,
     "CROSS_ENTROPY": cross_entropy,
     "CROSS_ENTROPY_GRAD": cross_entropy_grad,
+    # fused nodes emitted by GRAD_RULES below (no counterpart in the reference's table)
+    "LINEAR_GRAD": linear_bwd,
+    "LAYER_NORM_STATS": layer_norm_fwd_stats,
+    "LAYER_NORM_STATS_GRAD": layer_norm_bwd_stats,
+    "CROSS_ENTROPY_IDS": cross_entropy_ids,
+    "CROSS_ENTROPY_IDS_GRAD": cross_entropy_grad_ids,
 }
 
 
@@ -673,3 +775,155 @@ def run(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     except KeyError:
         raise MogradError(2, f"no scheduler rule for op {node.op_type} on the backward hot path") from None
     return fn(node, inputs, device)
+
+
+# --------------------------------------------------------------------------- #
+# Gradient rules: node + upstream -> one gradient node per source (None: no gradient edge),
+# the GradFn of mograd/grad.mojo:12.  The rules of the reference that lie on this path are
+# restated (layer_norm_grad :296-306, flash_attn_grad :309-344, cross_entropy_grad :224-230,
+# gettuple_grad :291-293); the others are the rules it lacks (mograd/grad.mojo:30-65 has
+# none for MATMUL_BT / MATMUL_BIAS_BT, so its Linear backward is three separate products and
+# a reduction over an unsimplified graph): each emits one multi-output node whose results
+# GETTUPLE selects, the way the reference treats LAYER_NORM_GRAD and FLASH_ATTN_GRAD.
+# --------------------------------------------------------------------------- #
+
+
+def _gettuple(src: Node, index: int, layout: Layout, dtype: int) -> Node:
+    return Node("GETTUPLE", layout, dtype, [src], {"index": index})
+
+
+def _rows_layout(layout: Layout) -> Layout:
+    cols = layout.shape(layout.rank() - 1)
+    return Layout(layout.numel() // cols)
+
+
+def linear_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """MATMUL_BIAS_BT[X, W, b] or MATMUL_BT[X, W] -> LINEAR_GRAD[dY, X, W] -> dX, dW(, db)."""
+    x, w = node.src(0), node.src(1)
+    has_bias = node.op_type == "MATMUL_BIAS_BT"
+    bwd = Node("LINEAR_GRAD", x.layout().as_contiguous(), x.dtype(), [upstream, x, w], {"has_bias": has_bias})
+    grads: List[Optional[Node]] = [_gettuple(bwd, 0, x.layout().as_contiguous(), x.dtype()),
+                                   _gettuple(bwd, 1, w.layout().as_contiguous(), w.dtype())]
+    if has_bias:
+        b = node.src(2)
+        grads.append(_gettuple(bwd, 2, b.layout().as_contiguous(), b.dtype()))
+    return grads
+
+
+def layer_norm_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """mograd/grad.mojo:296-306."""
+    x, gamma = node.src(0), node.src(1)
+    bwd = Node("LAYER_NORM_GRAD", x.layout().as_contiguous(), x.dtype(), [upstream, x, gamma], dict(node.attrs()))
+    return [_gettuple(bwd, 0, x.layout().as_contiguous(), x.dtype()),
+            _gettuple(bwd, 1, gamma.layout().as_contiguous(), gamma.dtype()),
+            _gettuple(bwd, 2, gamma.layout().as_contiguous(), gamma.dtype())]
+
+
+def layer_norm_stats_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """LAYER_NORM_STATS[x, gamma, beta] (outputs y, mean, rstd; `upstream` is dy, passed through
+    GETTUPLE 0 by gettuple_grad) -> LAYER_NORM_STATS_GRAD[dy, x, gamma, mean, rstd]."""
+    x, gamma = node.src(0), node.src(1)
+    rows = _rows_layout(x.layout())
+    mean = _gettuple(node, 1, rows, F32)
+    rstd = _gettuple(node, 2, rows, F32)
+    bwd = Node("LAYER_NORM_STATS_GRAD", x.layout().as_contiguous(), x.dtype(), [upstream, x, gamma, mean, rstd])
+    return [_gettuple(bwd, 0, x.layout().as_contiguous(), x.dtype()),
+            _gettuple(bwd, 1, gamma.layout().as_contiguous(), gamma.dtype()),
+            _gettuple(bwd, 2, gamma.layout().as_contiguous(), gamma.dtype())]
+
+
+def flash_attn_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """mograd/grad.mojo:309-344: O and LSE from the forward's two outputs, LSE (B,H,S) f32."""
+    q, k, v, mask = (node.src(i) for i in range(4))
+    B, S, H = q.layout().shape(0), q.layout().shape(1), q.layout().shape(2)
+    o = _gettuple(node, 0, node.layout(), node.dtype())
+    lse = _gettuple(node, 1, Layout(B, H, S), F32)
+    d_o = upstream if upstream.layout().is_contiguous() else Node("CONTIGUOUS", upstream.layout().as_contiguous(),
+                                                                  upstream.dtype(), [upstream])
+    bwd = Node("FLASH_ATTN_GRAD", q.layout().as_contiguous(), q.dtype(), [d_o, o, q, k, v, mask, lse], dict(node.attrs()))
+    return [_gettuple(bwd, i, t.layout().as_contiguous(), t.dtype()) for i, t in enumerate((q, k, v))] + [None]
+
+
+def cross_entropy_grad_rule(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """mograd/grad.mojo:224-230, and its class-id form."""
+    logits, labels = node.src(0), node.src(1)
+    op = "CROSS_ENTROPY_IDS_GRAD" if node.op_type == "CROSS_ENTROPY_IDS" else "CROSS_ENTROPY_GRAD"
+    return [Node(op, logits.layout().as_contiguous(), logits.dtype(), [logits, labels, upstream]), None]
+
+
+def relu_grad_rule(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """relu_grad: RELU_GRAD[relu_out, upstream]."""
+    return [Node("RELU_GRAD", node.layout().as_contiguous(), node.dtype(), [node, upstream])]
+
+
+def gettuple_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """mograd/grad.mojo:291-293: the upstream passes through to the multi-output source."""
+    return [upstream]
+
+
+GRAD_RULES = {
+    "MATMUL_BT": linear_grad,
+    "MATMUL_BIAS_BT": linear_grad,
+    "LAYER_NORM": layer_norm_grad,
+    "LAYER_NORM_STATS": layer_norm_stats_grad,
+    "FLASH_ATTN": flash_attn_grad,
+    "CROSS_ENTROPY": cross_entropy_grad_rule,
+    "CROSS_ENTROPY_IDS": cross_entropy_grad_rule,
+    "RELU": relu_grad_rule,
+    "GETTUPLE": gettuple_grad,
+}
+
+
+def _toposort(root: Node) -> List[Node]:
+    order: List[Node] = []
+    seen = set()
+
+    def visit(n: Node) -> None:
+        if n in seen:
+            return
+        seen.add(n)
+        for s_ in n.srcs:
+            visit(s_)
+        order.append(n)
+
+    visit(root)
+    return order
+
+
+def gradient(root: Node, initial_grad: Node, targets: Sequence[Node]) -> List[Optional[Node]]:
+    """Grad.compute (mograd/grad.mojo:22-91): walks the graph from `root` in reverse
+    topological order, applies the rule of each node to its accumulated upstream and adds the
+    results to its sources' gradients (ADD nodes where two paths meet).  Returns the gradient
+    node of every target (None if no path reaches it)."""
+    grad_map: Dict[Node, Node] = {root: initial_grad}
+    for node in reversed(_toposort(root)):
+        upstream = grad_map.get(node)
+        if upstream is None or node.dtype() not in (F32, F16, BF16):
+            continue
+        rule = GRAD_RULES.get(node.op_type)
+        if rule is None:
+            if node.srcs:
+                raise MogradError(2, f"no gradient rule for op: {node.op_type}")
+            continue
+        for src, g in zip(node.srcs, rule(node, upstream)):
+            if g is None:
+                continue
+            prev = grad_map.get(src)
+            grad_map[src] = g if prev is None else Node("ADD", g.layout(), g.dtype(), [prev, g])
+    return [grad_map.get(t) for t in targets]
+
+
+def evaluate(node: Node, device: Device) -> AnyBuffer:
+    """Scheduler.run for one result (mograd/scheduler.mojo:40-80): evaluates the sources
+    first, runs the node's rule once and keeps its buffers on the node; GETTUPLE selects an
+    output of a multi-output source."""
+    if node.bufs is None:
+        if node.op_type == "BUFFER":
+            raise MogradError(1, "evaluate: a leaf node without a buffer")
+        if node.op_type == "GETTUPLE":
+            evaluate(node.src(0), device)
+            node.bufs = [node.src(0).bufs[int(node.attrs()["index"])]]
+        else:
+            inputs = [evaluate(s_, device) for s_ in node.srcs]
+            node.bufs = run(node, inputs, device)
+    return node.bufs[0]

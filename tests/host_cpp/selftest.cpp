@@ -287,6 +287,78 @@ int main(int argc, char** argv) {
     return close_to(download(db[0]), want, 0.0, "db");
   });
 
+  // The gradient rule the reference lacks: MATMUL_BIAS_BT -> one LINEAR_GRAD node whose three
+  // outputs are dX, dW (in W's layout) and db.  Same integers as above: exact in fp32.
+  run_case("linear_grad rule: MATMUL_BIAS_BT -> LINEAR_GRAD, exact integers", [&] {
+    const int64_t M = 37, N = 29, K = 53;
+    const auto x = ints(M * K, 2, -4, 4), w = ints(N * K, 3, -4, 4), dy = ints(M * N, 5, -4, 4);
+    const Layout lx{M, K}, lw{N, K}, lb{N}, ly{M, N};
+    const OpRef fwd = node("MATMUL_BIAS_BT", ly, {OpRef::leaf(lx), OpRef::leaf(lw), OpRef::leaf(lb)});
+    const OpRef bwd = linear_grad(fwd, OpRef::leaf(ly));
+    if (bwd.op_type != "LINEAR_GRAD" || bwd.srcs.size() != 3 || bwd.attr("has_bias") != 1) return std::string("wrong node");
+    auto out = run(bwd, {upload(dev, dy), upload(dev, x), upload(dev, w)}, dev);
+    if (out.size() != 3) return std::string("expected three outputs");
+    std::vector<double> want(static_cast<size_t>(M * K), 0.0);
+    for (int64_t m = 0; m < M; ++m)
+      for (int64_t k = 0; k < K; ++k)
+        for (int64_t n = 0; n < N; ++n) want[m * K + k] += static_cast<double>(dy[m * N + n]) * w[n * K + k];
+    std::string why = close_to(download(out[0]), want, 0.0, "dX");
+    if (!why.empty()) return why;
+    want.assign(static_cast<size_t>(N * K), 0.0);
+    for (int64_t n = 0; n < N; ++n)
+      for (int64_t k = 0; k < K; ++k)
+        for (int64_t m = 0; m < M; ++m) want[n * K + k] += static_cast<double>(dy[m * N + n]) * x[m * K + k];
+    why = close_to(download(out[1]), want, 0.0, "dW");
+    if (!why.empty()) return why;
+    want.assign(static_cast<size_t>(N), 0.0);
+    for (int64_t m = 0; m < M; ++m)
+      for (int64_t n = 0; n < N; ++n) want[n] += dy[m * N + n];
+    why = close_to(download(out[2]), want, 0.0, "db");
+    if (!why.empty()) return why;
+    // MATMUL_BT (no bias): two outputs
+    const OpRef bwd2 = linear_grad(node("MATMUL_BT", ly, {OpRef::leaf(lx), OpRef::leaf(lw)}), OpRef::leaf(ly));
+    return std::string(run(bwd2, {upload(dev, dy), upload(dev, x), upload(dev, w)}, dev).size() == 2 ? "" : "expected two outputs");
+  });
+  // LAYER_NORM as a multi-output node whose statistics feed the backward: the golden vectors of
+  // tests/test_nn.mojo:283-324 and tests/test_grad.mojo:776-856 through the new pair.
+  run_case("layer_norm_stats pair reproduces the goldens", [&] {
+    const Layout lx{1, 4}, lv{4}, lr{1};
+    const OpRef fwd = node("LAYER_NORM_STATS", lx, {OpRef::leaf(lx), OpRef::leaf(lv), OpRef::leaf(lv)}, {{"eps", 1e-5}});
+    auto bx = upload(dev, {1, 2, 3, 4}), bg = upload(dev, {1, 2, 1, 2});
+    auto out = run(fwd, {bx, bg, upload(dev, {0.1f, 0.2f, 0.1f, 0.2f})}, dev);
+    if (out.size() != 3) return std::string("expected y, mean, rstd");
+    std::string why = close_to(download(out[0]), {-1.241641, -0.694427, 0.547214, 2.883282}, 1e-4, "y");
+    if (why.empty()) why = close_to(download(out[1]), {2.5}, 1e-6, "mean");
+    if (why.empty()) why = close_to(download(out[2]), {1.0 / std::sqrt(1.25 + 1e-5)}, 1e-5, "rstd");
+    if (!why.empty()) return why;
+    const OpRef bwd = layer_norm_stats_grad(fwd, OpRef::leaf(lx), OpRef::leaf(lr), OpRef::leaf(lr));
+    auto g = run(bwd, {upload(dev, {0.1f, 0.2f, 0.3f, 0.4f}), bx, bg, out[1], out[2]}, dev);
+    why = close_to(download(g[0]), {0.0, 0.089443, -0.178886, 0.089443}, 2e-4, "dx");
+    if (why.empty()) why = close_to(download(g[1]), {-0.134164, -0.089443, 0.134164, 0.536656}, 2e-4, "dgamma");
+    if (why.empty()) why = close_to(download(g[2]), {0.1, 0.2, 0.3, 0.4}, 1e-6, "dbeta");
+    return why;
+  });
+  // Class-id labels: the goldens of tests/test_ops.mojo:155-175 with ids in place of one-hot rows,
+  // and the gradient golden of tests/test_non_contiguous.mojo:302-310 on a contiguous copy.
+  run_case("cross_entropy_ids and its gradient rule", [&] {
+    const Layout la{4, 10}, li{4};
+    const int32_t host_ids[4] = {0, 1, 2, 3};
+    AnyBuffer ids = AnyBuffer::from_host(dev, host_ids, 4, int32);
+    OpRef fwd = node("CROSS_ENTROPY_IDS", Layout{1}, {OpRef::leaf(la), OpRef::leaf(li, int32)});
+    auto loss = run(fwd, {upload(dev, std::vector<float>(40, 0.f)), ids}, dev);
+    std::string why = close_to(download(loss[0]), {2.302585}, 1e-3, "loss");
+    if (!why.empty()) return why;
+    // logits [[1,3],[2,4]], labels (0,1): d/dlogits = (softmax - onehot) / 2
+    const Layout l2{2, 2}, i2{2};
+    const int32_t host_ids2[2] = {0, 1};
+    AnyBuffer ids2 = AnyBuffer::from_host(dev, host_ids2, 2, int32);
+    const OpRef f2 = node("CROSS_ENTROPY_IDS", Layout{1}, {OpRef::leaf(l2), OpRef::leaf(i2, int32)});
+    const OpRef g2 = cross_entropy_ids_grad(f2, OpRef::leaf(Layout{1}));
+    if (g2.op_type != "CROSS_ENTROPY_IDS_GRAD") return std::string("wrong node");
+    auto d = run(g2, {upload(dev, {1, 3, 2, 4}), ids2, upload(dev, {1.0f})}, dev);
+    return close_to(download(d[0]), {-0.440398, 0.440398, 0.059601, -0.059601}, 1e-3, "grad");
+  });
+
   run_case("relu_grad is a bit-exact select", [&] {
     const auto out = ints(1000, 6, -2, 2), up = ints(1000, 7, -9, 9);
     const Layout l{1000};

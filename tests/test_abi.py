@@ -85,4 +85,6 @@ def test_scheduler_rules_cover_the_path():
 
     assert set(SCHEDULER_RULES) == {
         "ADD", "RELU", "CAST", "CONTIGUOUS", "GATHER", "SCATTER_ADD", "RELU_GRAD", "SOFTMAX", "SOFTMAX_GRAD", "ARGMAX", "SUM", "MATMUL", "MATMUL_BT", "MATMUL_BIAS_BT", "LAYER_NORM", "LAYER_NORM_GRAD", "FLASH_ATTN",
-        "FLASH_ATTN_GRAD", "CROSS_ENTROPY", "CROSS_ENTROPY_GRAD"}
+        "FLASH_ATTN_GRAD", "CROSS_ENTROPY", "CROSS_ENTROPY_GRAD",
+        # fused nodes of the gradient rules the reference lacks
+        "LINEAR_GRAD", "LAYER_NORM_STATS", "LAYER_NORM_STATS_GRAD", "CROSS_ENTROPY_IDS", "CROSS_ENTROPY_IDS_GRAD"}

@@ -1,0 +1,195 @@
+"""Gradient rules of the host mirror: the rules of mograd/grad.mojo that lie on the backward
+hot path, and the ones the reference lacks (a fused Linear backward for MATMUL_BT /
+MATMUL_BIAS_BT, LayerNorm as a multi-output node whose statistics feed the backward,
+cross-entropy on class ids), driven the way Tensor.gradient drives them: Grad.compute over
+the graph (mograd/grad.mojo:22-91), then the scheduler's evaluation of the gradient nodes
+(mograd/scheduler.mojo:40-80)."""
+import numpy as np
+import pytest
+
+from helpers import ATOL_F32, RTOL_F32, assert_close, assert_sum_close, integers, normal, uniform
+from oracle import oracle_np as O
+
+from mograd_amd import F32, I32, I64, Layout, Node
+from mograd_amd import runtime as R
+
+
+# ---- graph structure: no GPU ------------------------------------------------------------------
+
+
+def test_linear_rule_emits_one_multi_output_node():
+    x, w, b = Node.leaf(Layout(4, 8)), Node.leaf(Layout(6, 8)), Node.leaf(Layout(6))
+    y = Node("MATMUL_BIAS_BT", Layout(4, 6), F32, [x, w, b])
+    dy = Node.leaf(Layout(4, 6))
+    dx, dw, db = R.gradient(y, dy, [x, w, b])
+    assert [g.op_type for g in (dx, dw, db)] == ["GETTUPLE"] * 3
+    assert [g.attrs()["index"] for g in (dx, dw, db)] == [0, 1, 2]
+    bwd = dx.src(0)
+    assert bwd is dw.src(0) and bwd is db.src(0), "one LINEAR_GRAD node serves all three gradients"
+    assert bwd.op_type == "LINEAR_GRAD" and bwd.srcs == [dy, x, w] and bwd.attrs()["has_bias"] is True
+    assert (dx.layout().shape(), dw.layout().shape(), db.layout().shape()) == ((4, 8), (6, 8), (6,))
+    # without a bias: two gradients
+    y2 = Node("MATMUL_BT", Layout(4, 6), F32, [x, w])
+    g = R.gradient(y2, dy, [x, w])
+    assert g[0].src(0).attrs()["has_bias"] is False and len(R.GRAD_RULES["MATMUL_BT"](y2, dy)) == 2
+
+
+def test_layer_norm_stats_rule_feeds_the_statistics_back():
+    x, g, b = Node.leaf(Layout(3, 5, 16)), Node.leaf(Layout(16)), Node.leaf(Layout(16))
+    ln = Node("LAYER_NORM_STATS", Layout(3, 5, 16), F32, [x, g, b], {"eps": 1e-5})
+    y = Node("GETTUPLE", Layout(3, 5, 16), F32, [ln], {"index": 0})
+    dy = Node.leaf(Layout(3, 5, 16))
+    dx, dg, db = R.gradient(y, dy, [x, g, b])
+    bwd = dx.src(0)
+    assert bwd.op_type == "LAYER_NORM_STATS_GRAD" and bwd is dg.src(0) and bwd is db.src(0)
+    up, bx, bg, mean, rstd = bwd.srcs
+    assert up is dy and bx is x and bg is g
+    assert mean.op_type == rstd.op_type == "GETTUPLE" and mean.src(0) is ln and rstd.src(0) is ln
+    assert (mean.attrs()["index"], rstd.attrs()["index"]) == (1, 2)
+    assert mean.layout().shape() == (15,) and mean.dtype() == F32  # rows = numel / cols
+
+
+def test_reference_rules_on_the_path():
+    # layer_norm_grad (mograd/grad.mojo:296-306) and cross_entropy_grad (:224-230)
+    x, g, b = Node.leaf(Layout(4, 8)), Node.leaf(Layout(8)), Node.leaf(Layout(8))
+    ln = Node("LAYER_NORM", Layout(4, 8), F32, [x, g, b], {"eps": 1e-5, "axis": -1})
+    dx, dg, db = R.gradient(ln, Node.leaf(Layout(4, 8)), [x, g, b])
+    assert dx.src(0).op_type == "LAYER_NORM_GRAD" and dx.src(0).attrs()["eps"] == 1e-5
+    labels = Node.leaf(Layout(4, 8))
+    ce = Node("CROSS_ENTROPY", Layout(1), F32, [ln, labels])
+    one = Node.leaf(Layout(1))
+    dlogits, dlabels = R.GRAD_RULES["CROSS_ENTROPY"](ce, one)
+    assert dlabels is None and dlogits.op_type == "CROSS_ENTROPY_GRAD" and dlogits.srcs == [ln, labels, one]
+    # flash_attn_grad (:309-344): O and LSE from the forward's outputs, LSE (B,H,S) f32, no mask gradient
+    q = Node.leaf(Layout(2, 16, 3, 8))
+    fa = Node("FLASH_ATTN", Layout(2, 3, 16, 8), F32, [q, q, q, Node.leaf(Layout(1))], {"scale": 0.5, "is_causal": True})
+    grads = R.GRAD_RULES["FLASH_ATTN"](fa, Node.leaf(Layout(2, 3, 16, 8)))
+    assert grads[3] is None and grads[0].src(0).op_type == "FLASH_ATTN_GRAD"
+    lse = grads[0].src(0).src(6)
+    assert lse.layout().shape() == (2, 3, 16) and lse.dtype() == F32 and lse.attrs()["index"] == 1
+    # two paths into one node accumulate with ADD (Grad.accum, :93-95)
+    y = Node("MATMUL_BT", Layout(4, 4), F32, [x, x])  # both operands are x
+    gx, = R.gradient(y, Node.leaf(Layout(4, 4)), [x])
+    assert gx.op_type == "ADD"
+    with pytest.raises(R.MogradError, match="no gradient rule for op: CONV2D"):
+        R.gradient(Node("CONV2D", Layout(4, 8), F32, [x]), Node.leaf(Layout(4, 8)), [x])
+
+
+# ---- through the GPU -------------------------------------------------------------------------------
+
+
+def _leaf(device, a, dtype=F32):
+    from mograd_amd import AnyBuffer
+
+    return Node.leaf(Layout(*a.shape), dtype, AnyBuffer.from_numpy(device, a, dtype))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", [(64, 10, 256), (200, 136, 260), (512, 384, 384)])
+def test_linear_gradient_through_the_rule(device, M, N, K):
+    x, w, b, dy = normal(80, 0, (M, K)), normal(80, 1, (N, K)), normal(80, 2, (N,)), normal(80, 3, (M, N))
+    nx, nw, nb, ndy = (_leaf(device, a) for a in (x, w, b, dy))
+    y = Node("MATMUL_BIAS_BT", Layout(M, N), F32, [nx, nw, nb])
+    dx, dw, db = R.gradient(y, ndy, [nx, nw, nb])
+    got = [R.evaluate(g, device).to_numpy(g.layout().shape()) for g in (dx, dw, db)]
+    assert dx.src(0).bufs is not None and len(dx.src(0).bufs) == 3, "LINEAR_GRAD ran once, three outputs"
+    assert_sum_close(got[0], O.linear_grad_x(dy, w), np.abs(dy) @ np.abs(w), what="dx")
+    assert_sum_close(got[1], O.linear_grad_w(dy, x), np.abs(dy).T @ np.abs(x), what="dw")
+    assert_sum_close(got[2], O.linear_grad_b(dy), np.abs(dy).sum(axis=0), what="db")
+    # the node itself through the scheduler entry
+    node = Node("LINEAR_GRAD", Layout(M, K), F32, [Node.leaf(Layout(M, N)), Node.leaf(Layout(M, K)), Node.leaf(Layout(N, K))],
+                {"has_bias": False})
+    out = R.run(node, [ndy.bufs[0], nx.bufs[0], nw.bufs[0]], device)
+    assert len(out) == 2
+    np.testing.assert_array_equal(out[1].to_numpy((N, K)), got[1])
+
+
+@pytest.mark.gpu
+def test_layer_norm_stats_gradient_equals_the_plain_rule(device):
+    rows, cols = 300, 384
+    x, dy = normal(81, 0, (rows, cols), mean=0.3), normal(81, 1, (rows, cols))
+    g, b = uniform(81, 2, (cols,), 0.5, 1.5), normal(81, 3, (cols,), std=0.1)
+    nx, ng, nb, ndy = (_leaf(device, a) for a in (x, g, b, dy))
+    ln = Node("LAYER_NORM_STATS", Layout(rows, cols), F32, [nx, ng, nb], {"eps": 1e-5})
+    y = Node("GETTUPLE", Layout(rows, cols), F32, [ln], {"index": 0})
+    grads = R.gradient(y, ndy, [nx, ng, nb])
+    got = [R.evaluate(t, device).to_numpy(t.layout().shape()) for t in grads]
+    mean, rstd = (ln.bufs[i].to_numpy() for i in (1, 2))
+    rmu, rrs = O.layer_norm_stats(x, 1e-5)
+    assert_close(R.evaluate(y, device).to_numpy((rows, cols)), O.layer_norm_fwd(x, g, b), RTOL_F32, ATOL_F32, "y")
+    assert_close(mean, rmu[:, 0], RTOL_F32, ATOL_F32, "mean")
+    assert_close(rstd, rrs[:, 0], RTOL_F32, ATOL_F32, "rstd")
+    rdx, rdg, rdb = O.layer_norm_bwd(dy, x, g)
+    xhat = (x - rmu) * rrs
+    assert_close(got[0], rdx, RTOL_F32, ATOL_F32, "dx")
+    assert_sum_close(got[1], rdg, (np.abs(dy) * np.abs(xhat)).sum(axis=0), what="dgamma")
+    assert_sum_close(got[2], rdb, np.abs(dy).sum(axis=0), what="dbeta")
+    # the reference's single-output LAYER_NORM with its own rule gives the same gradients
+    ln1 = Node("LAYER_NORM", Layout(rows, cols), F32, [nx, ng, nb], {"eps": 1e-5, "axis": -1})
+    plain = [R.evaluate(t, device).to_numpy(t.layout().shape()) for t in R.gradient(ln1, ndy, [nx, ng, nb])]
+    for a, c, what in zip(got, plain, ("dx", "dgamma", "dbeta")):
+        assert_close(a, c, RTOL_F32, 10 * ATOL_F32, what + " stats vs plain")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("id_dtype,np_id", [(I32, np.int32), (I64, np.int64)])
+def test_cross_entropy_ids_gradient(device, id_dtype, np_id):
+    from mograd_amd import AnyBuffer
+
+    n, c = 257, 1000
+    logits = normal(82, 0, (n, c), std=2.0)
+    ids = integers(82, 1, (n,), 0, c, np_id)
+    nl = _leaf(device, logits)
+    ni = Node.leaf(Layout(n), id_dtype, AnyBuffer.from_numpy(device, ids, id_dtype))
+    loss = Node("CROSS_ENTROPY_IDS", Layout(1), F32, [nl, ni])
+    one = _leaf(device, np.ones(1, np.float32))
+    (dlogits,) = R.gradient(loss, one, [nl])
+    assert dlogits.op_type == "CROSS_ENTROPY_IDS_GRAD"
+    assert_close(R.evaluate(loss, device).item(), O.cross_entropy_ids(logits, ids), RTOL_F32, ATOL_F32, "loss")
+    got = R.evaluate(dlogits, device).to_numpy((n, c))
+    assert_close(got, O.cross_entropy_grad_ids(logits, ids), RTOL_F32, ATOL_F32 / n, "dlogits")
+    neg = got < 0
+    assert np.array_equal(neg.sum(axis=1), np.ones(n, np.int64)) and np.array_equal(np.argmax(neg, axis=1), ids)
+    # equals the dense rule on one-hot rows
+    dense = Node("CROSS_ENTROPY", Layout(1), F32, [nl, _leaf(device, O.one_hot(ids, c).astype(np.float32))])
+    (dl2,) = R.gradient(dense, one, [nl])
+    assert_close(R.evaluate(dl2, device).to_numpy((n, c)), got, RTOL_F32, ATOL_F32 / n, "dense vs ids")
+
+
+@pytest.mark.gpu
+def test_mlp_gradient_through_the_rules(device):
+    # x -> Linear+bias -> ReLU -> LayerNorm (statistics kept) -> Linear+bias -> cross-entropy on ids:
+    # every parameter gradient from gradient() + evaluate(), against the float64 oracle chain.
+    from mograd_amd import AnyBuffer
+
+    M, D0, D1, D2 = 64, 96, 128, 10
+    x = normal(83, 0, (M, D0))
+    w1, b1 = uniform(83, 1, (D1, D0), -0.25, 0.25), uniform(83, 2, (D1,), -0.25, 0.25)
+    g, be = uniform(83, 3, (D1,), 0.5, 1.5), normal(83, 4, (D1,), std=0.1)
+    w2, b2 = uniform(83, 5, (D2, D1), -0.2, 0.2), uniform(83, 6, (D2,), -0.2, 0.2)
+    ids = integers(83, 7, (M,), 0, D2, np.int32)
+    nx, nw1, nb1, ng, nbe, nw2, nb2 = (_leaf(device, a) for a in (x, w1, b1, g, be, w2, b2))
+    ni = Node.leaf(Layout(M), I32, AnyBuffer.from_numpy(device, ids, I32))
+    h_pre = Node("MATMUL_BIAS_BT", Layout(M, D1), F32, [nx, nw1, nb1])
+    h = Node("RELU", Layout(M, D1), F32, [h_pre])
+    ln = Node("LAYER_NORM_STATS", Layout(M, D1), F32, [h, ng, nbe], {"eps": 1e-5})
+    y = Node("GETTUPLE", Layout(M, D1), F32, [ln], {"index": 0})
+    logits = Node("MATMUL_BIAS_BT", Layout(M, D2), F32, [y, nw2, nb2])
+    loss = Node("CROSS_ENTROPY_IDS", Layout(1), F32, [logits, ni])
+    params = [nw1, nb1, ng, nbe, nw2, nb2]
+    grads = R.gradient(loss, _leaf(device, np.ones(1, np.float32)), params)
+    got = [R.evaluate(t, device).to_numpy(t.layout().shape()) for t in grads]
+    # oracle
+    r_hpre = O.matmul_bias_bt(x, w1, b1)
+    r_h = np.maximum(r_hpre, 0)
+    r_y = O.layer_norm_fwd(r_h, g, be)
+    r_logits = O.matmul_bias_bt(r_y, w2, b2)
+    assert_close(R.evaluate(loss, device).item(), O.cross_entropy_ids(r_logits, ids), RTOL_F32, ATOL_F32, "loss")
+    r_dlogits = O.cross_entropy_grad_ids(r_logits, ids)
+    r_dy = O.linear_grad_x(r_dlogits, w2)
+    r_dh, r_dg, r_dbe = O.layer_norm_bwd(r_dy, r_h, g)
+    r_dhpre = O.relu_grad(r_h, r_dh)
+    want = [O.linear_grad_w(r_dhpre, x), O.linear_grad_b(r_dhpre), r_dg, r_dbe, O.linear_grad_w(r_dlogits, r_y),
+            O.linear_grad_b(r_dlogits)]
+    for a, c, what in zip(got, want, ("dw1", "db1", "dgamma", "dbeta", "dw2", "db2")):
+        assert_close(a, c, RTOL_F32, ATOL_F32, what)

@@ -47,4 +47,4 @@ def test_cases_pass_on_the_gpu(driver):
     print(proc.stderr)
     assert proc.returncode == 0, proc.stdout[-2000:]
     lines = proc.stdout.splitlines()
-    assert sum(l.startswith("PASS ") for l in lines) >= 19 and not any(l.startswith("FAIL ") for l in lines)
+    assert sum(l.startswith("PASS ") for l in lines) >= 22 and not any(l.startswith("FAIL ") for l in lines)

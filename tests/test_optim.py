@@ -50,6 +50,37 @@ def test_adam_first_step_moves_by_lr(device):
     np.testing.assert_allclose(bw.to_numpy() - w, -lr * np.sign(g), rtol=1e-4, atol=1e-7)
 
 
+@pytest.mark.parametrize("t", [100_000, 1_000_000])
+def test_adam_late_steps(device, t):
+    # Far into training: the bias corrections 1 - beta**t must still be the fp32 rounding of
+    # the exact power (0.999**100000 = 3.5e-44 is still a nonzero fp32 denormal), and a call
+    # must not cost host time in proportion to t.
+    import time
+
+    lib, st = device.lib, device.stream
+    n = 4096
+    lr, b1, b2, eps = (float(np.float32(h)) for h in (3e-3, 0.9, 0.999, 1e-8))
+    w, g, m, v = normal(83, 0, (n,)), normal(83, 1, (n,)), normal(83, 2, (n,), std=0.1), np.abs(normal(83, 3, (n,), std=0.1))
+    bw, bg, bm, bv = (AnyBuffer.from_numpy(device, a) for a in (w, g, m, v))
+    lib.mg_adam_step(bw.data_ptr(), bg.data_ptr(), bm.data_ptr(), bv.data_ptr(), n, lr, b1, b2, eps, 0.0, t, 0, st)
+    ow, om, ov = O.adam_step(w, g, m, v, lr, b1, b2, eps, 0.0, t, False)
+    assert_close(bw.to_numpy(), ow, RTOL, ATOL, "w")
+    assert_close(bm.to_numpy(), om, RTOL, ATOL, "m")
+
+    def host_seconds(step):
+        device.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(200):
+            lib.mg_adam_step(bw.data_ptr(), bg.data_ptr(), bm.data_ptr(), bv.data_ptr(), n, lr, b1, b2, eps, 0.0, step, 0, st)
+        dt = time.perf_counter() - t0
+        device.synchronize()
+        return dt
+
+    host_seconds(1)
+    early, late = host_seconds(1), host_seconds(t)
+    assert late < 3 * early + 2e-3, f"200 calls: {early * 1e3:.2f} ms at t=1, {late * 1e3:.2f} ms at t={t}"
+
+
 @pytest.mark.parametrize("n", [1, 7, 4096, 100003])
 def test_sgd_step(device, n):
     w, g = normal(82, 0, (n,)), normal(82, 1, (n,))
