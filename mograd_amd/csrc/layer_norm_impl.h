@@ -63,7 +63,7 @@ __global__ __launch_bounds__(WG) void ln_fwd_rows_kernel(const T* __restrict__ x
 
   for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * RPW; row0 < rows; row0 += static_cast<int64_t>(gridDim.x) * RPW) {
     const int64_t row = row0 + sub;
-    if (row >= rows) continue;  // uniform per wave (TPR == 64) or per workgroup (RPW == 1)
+    if (row >= rows) continue;  // uniform per row of 16 lanes (TPR == 16), per wave (64) or per workgroup (RPW == 1)
     RowTile<T, VEC, TPR, VPT> xv;
     xv.load(x + row * cols, t, cols);
     const float shift = to_float(x[row * cols]);
@@ -128,8 +128,10 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
   constexpr int NW = WG / kWave;
   constexpr int TILE_COLS = VPT * TPR * VEC;
   __shared__ float slots[2 * 4 * NW];
-  // Only used to combine the RPW row slots of one workgroup at the end.
-  __shared__ float combine[RPW > 1 ? RPW * TILE_COLS : 1];
+  // Only used to combine the RPW row slots of one workgroup at the end: one set of column sums
+  // per wave (rows narrower than a wave are first added across the wave's rows of lanes).
+  constexpr int SETS = TPR < kWave ? NW : RPW;
+  __shared__ float combine[RPW > 1 ? SETS * TILE_COLS : 1];
 
   int t, sub;
   row_thread<TPR, WG>(t, sub);
@@ -273,24 +275,41 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
       }
     }
   } else {
-    // The RPW waves hold sums for the same columns: add them through LDS, dgamma first,
-    // then dbeta through the same buffer.
+    // The RPW row slots hold sums for the same columns: add them through LDS, dgamma first,
+    // then dbeta through the same buffer.  Rows of 16 lanes: the four rows of a wave are
+    // added inside the wave first (lanes l, l ^ 16, l ^ 32, l ^ 48 hold the same columns).
+    if constexpr (TPR < kWave) {
+#pragma unroll
+      for (int i = 0; i < VPT; ++i)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+#pragma unroll
+          for (int w = TPR; w < kWave; w *= 2) {
+            acc_g.v[i][e] += __shfl_xor(acc_g.v[i][e], w);
+            acc_b.v[i][e] += __shfl_xor(acc_b.v[i][e], w);
+          }
+        }
+    }
+    const int set = TPR < kWave ? static_cast<int>(threadIdx.x / kWave) : sub;
+    const bool writer = TPR >= kWave || threadIdx.x % kWave < TPR;
 #pragma unroll
     for (int which = 0; which < 2; ++which) {
       const RowTile<T, VEC, TPR, VPT>& acc = which == 0 ? acc_g : acc_b;
       float* out = which == 0 ? out_g : out_b;
       if (which == 1) __syncthreads();
+      if (writer) {
 #pragma unroll
-      for (int i = 0; i < VPT; ++i) {
-        const int c = (i * TPR + t) * VEC;
+        for (int i = 0; i < VPT; ++i) {
+          const int c = (i * TPR + t) * VEC;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) combine[sub * TILE_COLS + c + e] = acc.v[i][e];
+          for (int e = 0; e < VEC; ++e) combine[set * TILE_COLS + c + e] = acc.v[i][e];
+        }
       }
       __syncthreads();
       for (int c = threadIdx.x; c < TILE_COLS && c < cols; c += WG) {
         float sum = 0.f;
 #pragma unroll
-        for (int r = 0; r < RPW; ++r) sum += combine[r * TILE_COLS + c];
+        for (int r = 0; r < SETS; ++r) sum += combine[r * TILE_COLS + c];
         out[c] = sum;
       }
     }
@@ -386,8 +405,24 @@ struct LayerNormOps {
   struct Shape {
     int tpr, vpt;
   };
+  // The backward keeps one wave per row from 33 chunks on: with three chunks per lane its five
+  // row tiles no longer fit a 1024-thread workgroup, and sixteen-lane rows in smaller
+  // workgroups measured slower there ((16384, 384) bf16: 17.0 us against 14.3 us).
+  static bool pick_shape_bwd(int64_t chunks, Shape* s) {
+    if (chunks > 32 && chunks <= 64) {
+      *s = {64, 1};
+      return true;
+    }
+    return pick_shape(chunks, s);
+  }
   static bool pick_shape(int64_t chunks, Shape* s) {
-    if (chunks <= 64) *s = {64, 1};
+    // Up to 48 chunks: sixteen lanes per row, four rows per wave (a 384-column 16-bit row is
+    // 48 chunks: one wave per row would leave a quarter of the lanes idle and need the
+    // cross-row steps of the wave reduction).
+    if (chunks <= 16) *s = {16, 1};
+    else if (chunks <= 32) *s = {16, 2};
+    else if (chunks <= 48) *s = {16, 3};
+    else if (chunks <= 64) *s = {64, 1};
     else if (chunks <= 128) *s = {64, 2};
     else if (chunks <= 256) *s = {64, 4};
     else if (chunks <= 512) *s = {256, 2};
@@ -409,7 +444,7 @@ struct LayerNormOps {
   template <int VEC, int TPR, int VPT>
   static int launch_fwd(const T* x, const T* gamma, const T* beta, T* y, float* mean, float* rstd, int64_t rows,
                         int64_t cols, float eps, hipStream_t stream) {
-    constexpr int WG = TPR == 64 ? 256 : TPR;
+    constexpr int WG = TPR <= 64 ? 256 : TPR;
     constexpr int RPW = WG / TPR;
     const int64_t want = ceil_div(rows, RPW);
     const int64_t cap = static_cast<int64_t>(device_info().cu_count) * env_int("MOGRAD_HIP_LN_FWD_WG_PER_CU", 4);
@@ -425,6 +460,9 @@ struct LayerNormOps {
                           int64_t rows, int64_t cols, float eps, hipStream_t stream) {
 #define MG_LN_FWD_CASE(TPR_, VPT_) \
   if (s.tpr == TPR_ && s.vpt == VPT_) return launch_fwd<VEC, TPR_, VPT_>(x, gamma, beta, y, mean, rstd, rows, cols, eps, stream)
+    MG_LN_FWD_CASE(16, 1);
+    MG_LN_FWD_CASE(16, 2);
+    MG_LN_FWD_CASE(16, 3);
     MG_LN_FWD_CASE(64, 1);
     MG_LN_FWD_CASE(64, 2);
     MG_LN_FWD_CASE(64, 4);
@@ -486,13 +524,16 @@ struct LayerNormOps {
         return launch_bwd<VEC, TPR, VPT, HAS_STATS, 1024>(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows,
                                                           cols, eps, stream);
     }
-    if constexpr (TPR == 64 && WG_ == 0) {
+    if constexpr (TPR <= 64 && WG_ == 0) {
+      // The largest workgroup whose register budget holds the five row tiles: 1024 threads
+      // (128 registers) up to 8 values per tile, 512 up to 16, 256 beyond.
+      constexpr int TALL_WG = VPT * VEC <= 8 ? 1024 : (VPT * VEC <= 16 ? 512 : 256);
       const int64_t tall = static_cast<int64_t>(device_info().cu_count) * env_int("MOGRAD_HIP_LN_TALL_ROWS_PER_CU", 16);
-      if (rows >= tall)
-        return launch_bwd<VEC, TPR, VPT, HAS_STATS, 1024>(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows,
-                                                          cols, eps, stream);
+      if (rows >= tall && TALL_WG > 256)
+        return launch_bwd<VEC, TPR, VPT, HAS_STATS, TALL_WG>(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta,
+                                                             rows, cols, eps, stream);
     }
-    constexpr int WG = WG_ != 0 ? WG_ : (TPR == 64 ? 256 : TPR);
+    constexpr int WG = WG_ != 0 ? WG_ : (TPR <= 64 ? 256 : TPR);
     constexpr int RPW = WG / TPR;
     int64_t groups = bwd_groups(rows, RPW, WG);
     int64_t rows_per_group = ceil_div(ceil_div(rows, groups), RPW) * RPW;
@@ -519,6 +560,8 @@ struct LayerNormOps {
   if (s.tpr == TPR_ && s.vpt == VPT_)    \
   return launch_bwd<VEC, TPR_, VPT_, HAS_STATS>(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows, cols, eps, \
                                                 stream)
+    MG_LN_BWD_CASE(16, 1);
+    MG_LN_BWD_CASE(16, 2);
     MG_LN_BWD_CASE(64, 1);
     MG_LN_BWD_CASE(64, 2);
     MG_LN_BWD_CASE(64, 4);
@@ -574,10 +617,10 @@ struct LayerNormOps {
     // The backward keeps five row tiles per thread: at most 16 elements per tile with
     // 1024 threads (128 registers each), 32 with fewer threads.  Wider rows stream.
     auto fits = [](const Shape& sh, int vec) { return sh.vpt * vec <= (sh.tpr == 1024 ? 16 : 32); };
-    if (can_vectorise(cols, {dy, x, gamma, dx, residual}) && pick_shape(cols / WIDE, &s) && fits(s, WIDE))
+    if (can_vectorise(cols, {dy, x, gamma, dx, residual}) && pick_shape_bwd(cols / WIDE, &s) && fits(s, WIDE))
       return dispatch_bwd<WIDE, HAS_STATS>(s, dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows, cols, eps,
                                            stream);
-    if (pick_shape(cols, &s) && fits(s, 1))
+    if (pick_shape_bwd(cols, &s) && fits(s, 1))
       return dispatch_bwd<1, HAS_STATS>(s, dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows, cols, eps, stream);
     if (residual == nullptr)
       return bwd_stream<HAS_STATS>(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, rows, cols, eps, stream);

@@ -157,6 +157,17 @@ __device__ __forceinline__ float wave_allreduce(float v) {
   return Op::apply(lo, hi);
 }
 
+// Every lane returns the reduction over its own row of 16 lanes (lanes 16j .. 16j+15): the
+// first four DPP steps of wave_allreduce, which never leave a row.
+template <typename Op>
+__device__ __forceinline__ float row16_allreduce(float v) {
+  v = Op::apply(v, dpp_move<kDppQuadXor1>(v));
+  v = Op::apply(v, dpp_move<kDppQuadXor2>(v));
+  v = Op::apply(v, dpp_move<kDppRowHalfMirror>(v));
+  v = Op::apply(v, dpp_move<kDppRowMirror>(v));
+  return v;
+}
+
 __device__ __forceinline__ float wave_sum(float v) { return wave_allreduce<SumOp>(v); }
 __device__ __forceinline__ float wave_max(float v) { return wave_allreduce<MaxOp>(v); }
 

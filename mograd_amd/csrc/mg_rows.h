@@ -81,7 +81,11 @@ __device__ __forceinline__ void row_thread(int& t, int& sub) {
 
 template <int TPR, int WG, int K>
 __device__ __forceinline__ void row_allreduce_sum(float (&v)[K], float* slots, int& phase) {
-  if constexpr (TPR == kWave) {
+  if constexpr (TPR == 16) {
+    // four rows side by side in a wave, each on one row of 16 lanes
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = row16_allreduce<SumOp>(v[k]);
+  } else if constexpr (TPR == kWave) {
 #pragma unroll
     for (int k = 0; k < K; ++k) v[k] = wave_sum(v[k]);
   } else if constexpr (TPR == WG) {
