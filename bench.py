@@ -642,7 +642,20 @@ def bench_ln_ce(args, dev) -> dict:
     iters = max(10, min(args.steps, 100))
     timer = EventTimer(dev, iters)
     kernels = []
+    # Calibration of the HBM roofline on this box, one read-dominated and one write-only
+    # stream over the same 1.65 GB buffer (outside the step): the loss-only cross-entropy reads
+    # the logits once and writes 32 KB; the fill writes the buffer once.
+    def ce_loss_only(i):
+        lib.mg_cross_entropy_ids(logits.data_ptr(), ids.data_ptr(), loss.data_ptr(), CE_ROWS, CE_COLS, F32, I32, st)
+
+    def fill_only(i):
+        lib.mg_fill(dlogits.data_ptr(), 0.0, CE_ROWS * CE_COLS, F32, st)
+
+    ce_read_bytes = CE_ROWS * CE_COLS * 4 + CE_ROWS * 4 + 4
     for name, fn, nbytes in (("layer_norm_fwd", ln_fwd, LN_FWD_BYTES), ("layer_norm_bwd", ln_bwd, LN_BWD_BYTES),
+                             ("calibration: cross_entropy_ids, loss only (reads 1.65 GB, writes 32 KB)", ce_loss_only,
+                              ce_read_bytes),
+                             ("calibration: fill (writes 1.65 GB)", fill_only, CE_ROWS * CE_COLS * 4),
                              ("cross_entropy_fused_ids", ce_fused, CE_FUSED_BYTES)):
         fn(0)
         dev.synchronize()

@@ -108,6 +108,24 @@ static int launch_f32_mfma(const GemmArgs& g, hipStream_t stream) {
 
 static bool mult8(int64_t v) { return (v & 7) == 0; }
 
+// Into how many K ranges a 16-bit product of `blocks` output tiles is split (1: not at all):
+// enough for `wg_per_cu` workgroups per CU, each with at least 256 of K.
+static int splitk_16bit_splits(int64_t blocks, int64_t K, int wg_per_cu) {
+  const int64_t cus = device_info().cu_count;
+  if (blocks >= cus || K < 1024) return 1;
+  int splits = static_cast<int>(ceil_div(wg_per_cu * cus, blocks));
+  const int max_splits = static_cast<int>(K / env_int("MOGRAD_HIP_GEMM_SPLITK_MIN_K", 256));
+  if (splits > max_splits) splits = max_splits;
+  if (splits > 64) splits = 64;
+  return splits < 1 ? 1 : splits;
+}
+// The K range of one workgroup, a multiple of the k-step, and the number of ranges that leaves.
+static int splitk_16bit_range(int64_t K, int* splits) {
+  const int k_per_split = static_cast<int>(ceil_div(ceil_div(K, *splits), kG16BK) * kG16BK);
+  *splits = static_cast<int>(ceil_div(K, k_per_split));
+  return k_per_split;
+}
+
 // 16-bit MFMA path, optionally split along K when the output has too few tiles to fill
 // the device (dW of a narrow layer: reduction over thousands of rows into a small matrix).
 template <typename T, bool A_KC, bool B_KC, bool RAGGED>
@@ -125,13 +143,7 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
   T* c = static_cast<T*>(g.c);
   const int M = static_cast<int>(g.M), N = static_cast<int>(g.N), K = static_cast<int>(g.K);
   const int64_t cus = device_info().cu_count;
-  int splits = 1;
-  if (g.batch <= 65535 && blocks < cus && g.K >= 1024) {
-    splits = static_cast<int>(ceil_div(env_int("MOGRAD_HIP_GEMM_SPLITK_WG_PER_CU", 2) * cus, blocks));
-    const int max_splits = static_cast<int>(g.K / env_int("MOGRAD_HIP_GEMM_SPLITK_MIN_K", 256));
-    if (splits > max_splits) splits = max_splits;
-    if (splits > 64) splits = 64;
-  }
+  int splits = splitk_16bit_splits(blocks, g.K, env_int("MOGRAD_HIP_GEMM_SPLITK_WG_PER_CU", 2));
   // Tiles copied straight into LDS (gemm_16bit_pipe_kernel) where that measured faster: an
   // operand that is not k-contiguous is transposed by the LDS read instead of in registers
   // (dX 15-25 %, dW 5-20 % faster at Linear-layer shapes, 20-30 % at 4096^3 and up), and long
@@ -152,11 +164,11 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
       pipe = static_cast<int>(env_int("MOGRAD_HIP_GEMM16_PIPE", pipe));
     }
   }
-#define MG_GEMM16_LAUNCH(BIAS_, SPLIT_, GRID_, PARTIAL_, KPS_, EP_)                                                     \
+#define MG_GEMM16_LAUNCH(BIAS_, SPLIT_, GRID_, PARTIAL_, KPS_, NSPLIT_, EP_)                                                   \
   do {                                                                                                                 \
     auto launch = [&](auto kernel) {                                                                                   \
       hipLaunchKernelGGL(kernel, GRID_, dim3(kGemmThreads), 0, stream, a, b, bias, c, PARTIAL_, M, N, K, lda, ldb, g.N,  \
-                         g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n, KPS_, EP_);                                        \
+                         g.bsa, g.bsb, g.M * g.N, tiles_m, tiles_n, KPS_, NSPLIT_, static_cast<int>(g.batch), EP_);   \
     };                                                                                                                 \
     if constexpr (!RAGGED) {                                                                                           \
       if (pipe == 322) { launch(gemm_16bit_pipe_kernel<T, A_KC, B_KC, BIAS_, SPLIT_, 32, 2>); break; }                 \
@@ -171,7 +183,8 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
       const dim3 grid2(static_cast<unsigned>(static_cast<int64_t>(tiles_m2) * tiles_n * g.batch));
       auto launch = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, grid2, dim3(512), 0, stream, a, b, bias, c, static_cast<float*>(nullptr), M, N, K, lda,
-                           ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m2, tiles_n, K, epilogue_of<T>(g));
+                           ldb, g.N, g.bsa, g.bsb, g.M * g.N, tiles_m2, tiles_n, K, 1, static_cast<int>(g.batch),
+                           epilogue_of<T>(g));
       };
       if (pipe == 2322) {
         if (bias) launch(gemm_16bit_pipe_kernel<T, A_KC, B_KC, true, false, 32, 2, 256>);
@@ -188,20 +201,21 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
   if (splits <= 1) {
     const dim3 grid(static_cast<unsigned>(blocks));
     float* no_partial = nullptr;
-    if (bias) MG_GEMM16_LAUNCH(true, false, grid, no_partial, K, epilogue_of<T>(g));
-    else MG_GEMM16_LAUNCH(false, false, grid, no_partial, K, epilogue_of<T>(g));
+    if (bias) MG_GEMM16_LAUNCH(true, false, grid, no_partial, K, 1, epilogue_of<T>(g));
+    else MG_GEMM16_LAUNCH(false, false, grid, no_partial, K, 1, epilogue_of<T>(g));
     MG_LAUNCH_CHECK();
     return MG_OK;
   }
-  const int k_per_split = static_cast<int>(ceil_div(ceil_div(g.K, splits), kG16BK) * kG16BK);
-  splits = static_cast<int>(ceil_div(g.K, k_per_split));
+  const int k_per_split = splitk_16bit_range(g.K, &splits);
   // The batches of C are contiguous ((batch, M, N) row-major), so partials and the reduction
   // treat them as one array of batch * M * N elements.
   Scratch partial;
   const int64_t numel = g.batch * g.M * g.N;
   MG_TRY(partial.take(static_cast<int64_t>(splits) * numel * static_cast<int64_t>(sizeof(float))));
-  const dim3 grid(static_cast<unsigned>(tiles), static_cast<unsigned>(splits), static_cast<unsigned>(g.batch));
-  MG_GEMM16_LAUNCH(false, true, grid, partial.as<float>(), k_per_split, (GemmEpilogue<T>{nullptr, nullptr, 0}));
+  const int64_t split_grid = gemm_split_grid(tiles, splits, g.batch);
+  if (split_grid > 0x7fffffffLL) return fail(MG_ERR_INVALID, "matmul: too many output tiles");
+  const dim3 grid(static_cast<unsigned>(split_grid));
+  MG_GEMM16_LAUNCH(false, true, grid, partial.as<float>(), k_per_split, splits, (GemmEpilogue<T>{nullptr, nullptr, 0}));
 #undef MG_GEMM16_LAUNCH
   MG_LAUNCH_CHECK();
   const unsigned rblocks = static_cast<unsigned>(ceil_div(numel, 256));
@@ -327,6 +341,74 @@ int gemm_dispatch(const char* who, const GemmArgs& g_in, hipStream_t stream) {
 int colsum_dispatch(const void* a, void* dst, int64_t outer, int64_t reduce, int64_t inner, int dtype,
                     hipStream_t stream);  // reduce.hip
 
+// dX (M,K) = dY (M,N) W (N,K) and dW (N,K) = dY^T X of a 16-bit Linear layer in one launch
+// (linear_bwd_16bit_kernel), for the shapes at which launch_16bit_mfma would give both the
+// pipelined kernel with 32 k per step and split dW along the rows.  dW comes out bit for bit
+// as from its own launch with the same number of K ranges, and so does dX unless its own launch would split it along N (fewer
+// dX tiles than CUs): here dX is never split, the dW workgroups fill the device.
+// *done = false: not such a shape, nothing launched.
+// MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH=0 switches it off (benchmarks, tests of the equivalence).
+template <typename T>
+static int linear_bwd_one_launch(const void* dy, const void* x, const void* w, void* dx, void* dw, int64_t M, int64_t N,
+                                 int64_t K, const void* relu_mask, bool dx_accumulate, hipStream_t stream, bool* done) {
+  *done = false;
+  if (env_int("MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH", 1) == 0 || std::getenv("MOGRAD_HIP_GEMM16_PIPE")) return MG_OK;
+  if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return MG_OK;
+  if (M % kG16BK || N % kG16BK || !mult8(K)) return MG_OK;
+  if (!aligned16(dy) || !aligned16(x) || !aligned16(w) || !aligned16(dx) || !aligned16(dw)) return MG_OK;
+  if (M * K < 64 * 64 || N * K < 64 * 64) return MG_OK;
+  const int64_t cus = device_info().cu_count;
+  const int tiles_kk = static_cast<int>(ceil_div(K, kGemmBN));
+  // dW: must be split, each workgroup's rows short enough for the 32-k variant.
+  const int w_tiles_m = static_cast<int>(ceil_div(N, kGemmBM));
+  const int64_t w_tiles = static_cast<int64_t>(w_tiles_m) * tiles_kk;
+  // One workgroup per CU is enough here: the dX tiles fill the rest of the device, and half
+  // the K ranges are half the partial tiles to write and sum (GPT step 3.06 -> 3.00 ms).
+  int splits = splitk_16bit_splits(w_tiles, M, env_int("MOGRAD_HIP_LINEAR_BWD_SPLIT_WG_PER_CU", 1));
+  if (splits <= 1 || ceil_div(M, splits) >= 4096) return MG_OK;
+  const int k_per_split = splitk_16bit_range(M, &splits);
+  // dX: the 32-k variant with 128 x 128 tiles.
+  const int x_tiles_m = static_cast<int>(ceil_div(M, kGemmBM));
+  const int64_t x_tiles = static_cast<int64_t>(x_tiles_m) * tiles_kk;
+  if (N >= 4096 || (N >= 1024 && ceil_div(M, 256) * tiles_kk >= 2 * cus)) return MG_OK;
+  const int64_t n_dw = gemm_split_grid(w_tiles, splits, 1);
+  if (n_dw + x_tiles > 0x7fffffffLL) return MG_OK;
+
+  Scratch partial;
+  const int64_t numel = N * K;
+  MG_TRY(partial.take(static_cast<int64_t>(splits) * numel * static_cast<int64_t>(sizeof(float))));
+  const T* dyt = static_cast<const T*>(dy);
+  const Gemm16Problem<T> pw{dyt, static_cast<const T*>(x), nullptr, static_cast<T*>(dw), partial.as<float>(),
+                            static_cast<int>(N), static_cast<int>(K), static_cast<int>(M),
+                            N, K, K, 0, 0, numel, w_tiles_m, tiles_kk, k_per_split, splits, 1,
+                            GemmEpilogue<T>{nullptr, nullptr, 0}};
+  const Gemm16Problem<T> px{dyt, static_cast<const T*>(w), nullptr, static_cast<T*>(dx), nullptr,
+                            static_cast<int>(M), static_cast<int>(K), static_cast<int>(N),
+                            N, K, K, 0, 0, M * K, x_tiles_m, tiles_kk, static_cast<int>(N), 1, 1,
+                            GemmEpilogue<T>{dx_accumulate ? static_cast<const T*>(dx) : nullptr,
+                                            static_cast<const T*>(relu_mask), 0}};
+  hipLaunchKernelGGL((linear_bwd_16bit_kernel<T>), dim3(static_cast<unsigned>(n_dw + x_tiles)), dim3(kGemmThreads), 0,
+                     stream, pw, px, static_cast<int>(n_dw));
+  MG_LAUNCH_CHECK();
+  const unsigned rblocks = static_cast<unsigned>(ceil_div(numel, 256));
+  hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, false>), dim3(rblocks), dim3(256), 0, stream, partial.as<float>(),
+                     static_cast<const T*>(nullptr), static_cast<T*>(dw), numel, splits, static_cast<int>(K),
+                     GemmEpilogue<T>{nullptr, nullptr, 0});
+  MG_LAUNCH_CHECK();
+  *done = true;
+  return MG_OK;
+}
+
+int linear_bwd_products(const void* dy, const void* x, const void* w, void* dx, void* dw, int64_t M, int64_t N, int64_t K,
+                        const void* relu_mask, bool dx_accumulate, int dtype, hipStream_t stream, bool* done) {
+  *done = false;
+  if (dtype == MG_BF16)
+    return linear_bwd_one_launch<bf16_t>(dy, x, w, dx, dw, M, N, K, relu_mask, dx_accumulate, stream, done);
+  if (dtype == MG_F16)
+    return linear_bwd_one_launch<f16_t>(dy, x, w, dx, dw, M, N, K, relu_mask, dx_accumulate, stream, done);
+  return MG_OK;
+}
+
 }  // namespace mg
 
 extern "C" {
@@ -375,6 +457,16 @@ int mg_matmul_bias_relu_bt(const void* a, const void* b, const void* bias, void*
 static int linear_bwd_impl(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db, int64_t M,
                            int64_t N, int64_t K, bool dx_accumulate, bool x_is_relu_output, int dtype, mg_stream stream) {
   hipStream_t s = mg::to_stream(stream);
+  if (x_is_relu_output && dx && !x) return mg::fail(MG_ERR_INVALID, "linear_bwd: x is needed as the relu mask");
+  if (dx && dw && dy && x && w) {
+    bool done = false;
+    MG_TRY(mg::linear_bwd_products(dy, x, w, dx, dw, M, N, K, x_is_relu_output ? x : nullptr, dx_accumulate, dtype, s,
+                                   &done));
+    if (done) {
+      if (db) MG_TRY(mg::colsum_dispatch(dy, db, 1, M, N, dtype, s));
+      return MG_OK;
+    }
+  }
   if (dx) {  // dX (M,K) = dY (M,N) x W (N,K): reduction over N, W read as an n-contiguous right operand
     mg::GemmArgs g{dy, w, nullptr, dx, 1, M, K, N, N, 1, K, 1, 0, 0, dtype};
     if (x_is_relu_output) {

@@ -31,11 +31,12 @@ constexpr int kKcStride = kGemmBK + 4;  // floats per LDS row of a k-contiguous 
 // Workgroup -> output tile.  Consecutive workgroup ids go to different XCDs (id % 8), each
 // with its own L2; ids are regrouped so that one XCD works on a compact block of tiles
 // that share operand rows and columns.
-__device__ __forceinline__ void gemm_tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+constexpr int kXcd = 8;
+__device__ __forceinline__ void gemm_tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn,
+                                                   bool regroup = true) {
   const int total = tiles_m * tiles_n;
-  constexpr int kXcd = 8;
   int id = bid;
-  if (total % kXcd == 0) id = (bid % kXcd) * (total / kXcd) + bid / kXcd;
+  if (regroup && total % kXcd == 0) id = (bid % kXcd) * (total / kXcd) + bid / kXcd;
   // Raster in bands of 4 tile-rows so that a band's A rows stay in L2.
   constexpr int kBand = 4;
   const int band_tiles = kBand * tiles_n;
@@ -44,6 +45,25 @@ __device__ __forceinline__ void gemm_tile_of_block(int bid, int tiles_m, int til
   const int rows_here = min(kBand, tiles_m - band * kBand);
   tm = band * kBand + in_band % rows_here;
   tn = in_band / rows_here;
+}
+
+// Split-K launches use one grid axis of kXcd * ceil(groups / kXcd) * tiles workgroups, a group
+// being one (batch, K range).  All output tiles of a group read the same K range of both
+// operands, so a group's workgroups are given ids of one residue mod kXcd: they run on one
+// XCD and the range is fetched into one L2 instead of all eight (the dW of a 384 -> 1536
+// layer over 16384 rows fetched 240 MB for 63 MB of operands with tiles dealt out round
+// robin).  Returns false for the padding workgroups of the last, partial round of groups.
+__device__ __forceinline__ bool gemm_split_work(int bid, int tiles, int splits, int batches, int& tile, int& split,
+                                                int& batch) {
+  const int j = bid / kXcd;
+  const int group = (j / tiles) * kXcd + bid % kXcd;
+  tile = j % tiles;
+  split = group % splits;
+  batch = group / splits;
+  return group < splits * batches;
+}
+inline int64_t gemm_split_grid(int64_t tiles, int64_t splits, int64_t batches) {
+  return kXcd * ((splits * batches + kXcd - 1) / kXcd) * tiles;
 }
 
 // What happens to a product element after the bias: v = acc + bias; relu: v = max(v, 0);
@@ -296,7 +316,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
 // wants (8 consecutive k per lane).  A k-contiguous operand is copied as is; an
 // m/n-contiguous operand is transposed on the way in: a thread loads 8 columns of two
 // consecutive k rows and stores 8 dwords, each packing (k, k+1) for one column.
-// SPLIT_K: blockIdx.y selects a K range and fp32 partial tiles go to scratch
+// SPLIT_K: a workgroup takes one K range (gemm_split_work) and fp32 partial tiles go to scratch
 // (splits, M, N); gemm_splitk_reduce_kernel sums them in a fixed order.
 // ------------------------------------------------------------------------------------
 
@@ -529,20 +549,23 @@ template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, bool RA
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
     const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C,
     float* __restrict__ partial, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb,
-    int64_t bsc, int tiles_m, int tiles_n, int k_per_split, GemmEpilogue<T> ep) {
+    int64_t bsc, int tiles_m, int tiles_n, int k_per_split, int splits, int batches, GemmEpilogue<T> ep) {
   __shared__ __attribute__((aligned(16))) uint16_t lds_a[kGemmBM * kG16Stride];
   __shared__ __attribute__((aligned(16))) uint16_t lds_b[kGemmBN * kG16Stride];
 
   const int tiles = tiles_m * tiles_n;
-  // Split along K: grid (tiles, splits, batch).  Otherwise the batch index is folded into x.
-  const int batch = SPLIT_K ? blockIdx.z : blockIdx.x / tiles;
+  // Split along K: see gemm_split_work.  Otherwise the batch index is folded into the tile id.
+  int batch = blockIdx.x / tiles, tile = blockIdx.x % tiles, split = 0;
+  if constexpr (SPLIT_K) {
+    if (!gemm_split_work(blockIdx.x, tiles, splits, batches, tile, split, batch)) return;
+  }
   int tm, tn;
-  gemm_tile_of_block(blockIdx.x % tiles, tiles_m, tiles_n, tm, tn);
+  gemm_tile_of_block(tile, tiles_m, tiles_n, tm, tn, !SPLIT_K);
   const int m0 = tm * kGemmBM;
   const int n0 = tn * kGemmBN;
   A += batch * bsa;
   B += batch * bsb;
-  const int k_begin = SPLIT_K ? blockIdx.y * k_per_split : 0;
+  const int k_begin = SPLIT_K ? split * k_per_split : 0;
   const int k_end = SPLIT_K ? min(K, k_begin + k_per_split) : K;
 
   const int wave = threadIdx.x / kWave;
@@ -586,7 +609,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
 
   uint16_t* mine = (wave < 2 ? lds_a : lds_b) + (wave % 2) * 64 * kG16Stride;  // staging memory, idle now
   gemm16_write_tile<T, HAS_BIAS, SPLIT_K>(acc, mine, bias, C, partial, M, N, ldc, bsc, batch,
-                                          SPLIT_K ? static_cast<int>(blockIdx.y) : 0, SPLIT_K ? static_cast<int>(gridDim.z) : 1,
+                                          split, SPLIT_K ? batches : 1,
                                           m0, n0, wm, wn, lane, ep);
 }
 
@@ -697,26 +720,51 @@ constexpr int gemm16_pipe_occupancy(int bk, int nstage, int tm) {
   return by_lds < 1 ? 1 : (by_lds > by_regs ? by_regs : by_lds);
 }
 
+// One product's arguments, as the kernels below take them.
+template <typename T>
+struct Gemm16Problem {
+  const T* A;
+  const T* B;
+  const T* bias;
+  T* C;
+  float* partial;
+  int M, N, K;
+  int64_t lda, ldb, ldc, bsa, bsb, bsc;
+  int tiles_m, tiles_n, k_per_split, splits, batches;
+  GemmEpilogue<T> ep;
+};
+
+// The work of workgroup `bid` of a launch for one product; `lds` is the workgroup's
+// gemm16_pipe_lds_bytes(BK, NSTAGE, TM) bytes, aligned to 1024.
 template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, int BK, int NSTAGE, int TM = 128>
-__global__ __launch_bounds__(TM * 2, gemm16_pipe_occupancy(BK, NSTAGE, TM)) void gemm_16bit_pipe_kernel(
-    const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C,
-    float* __restrict__ partial, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb,
-    int64_t bsc, int tiles_m, int tiles_n, int k_per_split, GemmEpilogue<T> ep) {
+__device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm16Problem<T>& pr) {
   static_assert(NSTAGE >= 2 && NSTAGE <= 4 && (BK == 32 || BK == 64) && (TM == 128 || TM == 256), "stages");
   constexpr int NW = TM / 32;                                 // waves: (TM / 64) x 2 wave tiles of 64 x 64
   constexpr int NIA = gemm16_pipe_requests(TM, BK, NW);       // copy requests per thread and step
   constexpr int NIB = gemm16_pipe_requests(kGemmBN, BK, NW);
   constexpr int OPA = TM * BK * 2, OPB = kGemmBN * BK * 2;    // bytes of an operand's step
   constexpr int OP = OPA + OPB;
-  __shared__ __attribute__((aligned(1024))) char lds[gemm16_pipe_lds_bytes(BK, NSTAGE, TM)];
+  const T* __restrict__ A = pr.A;
+  const T* __restrict__ B = pr.B;
+  const T* __restrict__ bias = pr.bias;
+  T* __restrict__ C = pr.C;
+  float* __restrict__ partial = pr.partial;
+  const int M = pr.M, N = pr.N, K = pr.K;
+  const int64_t lda = pr.lda, ldb = pr.ldb, ldc = pr.ldc, bsa = pr.bsa, bsb = pr.bsb, bsc = pr.bsc;
+  const int tiles_m = pr.tiles_m, tiles_n = pr.tiles_n, k_per_split = pr.k_per_split, splits = pr.splits,
+            batches = pr.batches;
+  const GemmEpilogue<T> ep = pr.ep;
 
   const int tiles = tiles_m * tiles_n;
-  const int batch = SPLIT_K ? blockIdx.z : blockIdx.x / tiles;
+  int batch = bid / tiles, tile = bid % tiles, split = 0;
+  if constexpr (SPLIT_K) {
+    if (!gemm_split_work(bid, tiles, splits, batches, tile, split, batch)) return;
+  }
   int tm, tn;
-  gemm_tile_of_block(blockIdx.x % tiles, tiles_m, tiles_n, tm, tn);
+  gemm_tile_of_block(tile, tiles_m, tiles_n, tm, tn, !SPLIT_K);
   const int m0 = tm * TM;
   const int n0 = tn * kGemmBN;
-  const int k_begin = SPLIT_K ? blockIdx.y * k_per_split : 0;
+  const int k_begin = SPLIT_K ? split * k_per_split : 0;
   const int k_end = SPLIT_K ? min(K, k_begin + k_per_split) : K;
   const int steps = (k_end - k_begin) / BK;
   A += batch * bsa + (A_KC ? static_cast<int64_t>(k_begin) : k_begin * lda);
@@ -793,8 +841,33 @@ __global__ __launch_bounds__(TM * 2, gemm16_pipe_occupancy(BK, NSTAGE, TM)) void
 
   uint16_t* mine = reinterpret_cast<uint16_t*>(lds) + wave * 64 * kG16Stride;
   gemm16_write_tile<T, HAS_BIAS, SPLIT_K>(acc, mine, bias, C, partial, M, N, ldc, bsc, batch,
-                                          SPLIT_K ? static_cast<int>(blockIdx.y) : 0, SPLIT_K ? static_cast<int>(gridDim.z) : 1,
+                                          split, SPLIT_K ? batches : 1,
                                           m0, n0, wm, wn, lane, ep);
+}
+
+template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, int BK, int NSTAGE, int TM = 128>
+__global__ __launch_bounds__(TM * 2, gemm16_pipe_occupancy(BK, NSTAGE, TM)) void gemm_16bit_pipe_kernel(
+    const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C,
+    float* __restrict__ partial, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb,
+    int64_t bsc, int tiles_m, int tiles_n, int k_per_split, int splits, int batches, GemmEpilogue<T> ep) {
+  __shared__ __attribute__((aligned(1024))) char lds[gemm16_pipe_lds_bytes(BK, NSTAGE, TM)];
+  const Gemm16Problem<T> pr{A, B, bias, C, partial, M, N, K, lda, ldb, ldc, bsa, bsb, bsc,
+                            tiles_m, tiles_n, k_per_split, splits, batches, ep};
+  gemm16_pipe_block<T, A_KC, B_KC, HAS_BIAS, SPLIT_K, BK, NSTAGE, TM>(lds, blockIdx.x, pr);
+}
+
+// Both products of a Linear layer's backward in one launch: workgroups [0, n_dw) take the
+// K ranges of dW = dY^T X (their partial tiles are summed by gemm_splitk_reduce_kernel
+// afterwards), the rest the tiles of dX = dY W.  The longer-running dW ranges start first
+// and the dX tiles fill the CUs as those drain, where two launches each end in a tail of
+// half-empty CUs (384 dX tiles on 256 CUs) and pay a launch apiece.
+template <typename T>
+__global__ __launch_bounds__(256, gemm16_pipe_occupancy(32, 2, 128)) void linear_bwd_16bit_kernel(
+    Gemm16Problem<T> dw, Gemm16Problem<T> dx, int n_dw) {
+  __shared__ __attribute__((aligned(1024))) char lds[gemm16_pipe_lds_bytes(32, 2, 128)];
+  const int bid = blockIdx.x;
+  if (bid < n_dw) gemm16_pipe_block<T, false, false, false, true, 32, 2, 128>(lds, bid, dw);
+  else gemm16_pipe_block<T, true, false, false, false, 32, 2, 128>(lds, bid - n_dw, dx);
 }
 
 // ------------------------------------------------------------------------------------

@@ -553,6 +553,48 @@ def test_fused_epilogues_equal_separate_calls(device, dtype, M, N, K):
     np.testing.assert_array_equal(acc.to_numpy(), dx_ref.to_numpy())
 
 
+@pytest.mark.parametrize("dtype,rtol", [(F16, 2e-3), (BF16, 1.6e-2)])
+@pytest.mark.parametrize("M,N,K", [(2048, 384, 384), (4096, 1152, 384), (2048, 1536, 384), (4096, 384, 1536),
+                                   (1056, 96, 200), (1024, 64, 72)])
+def test_linear_bwd_one_launch_matches_two(device, monkeypatch, dtype, rtol, M, N, K):
+    # dX and dW of a 16-bit layer whose dW is split along the rows go out as one launch
+    # (workgroups of both products in one grid); MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH=0 keeps the
+    # two launches.  Same tiles, same k order: no bit may differ, also with the relu mask and
+    # with accumulation into dx, and at ragged tile edges (K = 200, 72).
+    lib, st = device.lib, device.stream
+    x = np.maximum(round_to_dtype(normal(52, 0, (M, K)), dtype), 0)
+    w = round_to_dtype(normal(52, 1, (N, K), std=0.05), dtype)
+    dy = round_to_dtype(normal(52, 2, (M, N), std=0.5), dtype)
+    prior = round_to_dtype(normal(52, 3, (M, K)), dtype)
+    bx, bw, bdy = (AnyBuffer.from_numpy(device, a, dtype) for a in (x, w, dy))
+    results = {}
+    # the common launch splits dW for one workgroup per CU; ask the separate launch for the same
+    monkeypatch.setenv("MOGRAD_HIP_GEMM_SPLITK_WG_PER_CU", "1")
+    for mode in ("0", "1"):
+        monkeypatch.setenv("MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH", mode)
+        out = []
+        for accumulate, masked in ((0, 0), (1, 1)):
+            dx = AnyBuffer.from_numpy(device, prior, dtype)
+            dw, db = AnyBuffer.create(dtype, device, N * K), AnyBuffer.create(dtype, device, N)
+            lib.mg_linear_bwd_fused(_ptr(bdy), _ptr(bx), _ptr(bw), _ptr(dx), _ptr(dw), _ptr(db), M, N, K, accumulate,
+                                    masked, dtype, st)
+            out += [dx.to_numpy((M, K)), dw.to_numpy((N, K)), db.to_numpy()]
+        results[mode] = out
+    # Launched alone, a dX with fewer tiles than CUs and a long reduction is itself split along
+    # N (fp32 partials, another summation order); inside the common launch it never is.
+    dx_split_alone = -(-M // 128) * -(-K // 128) < 256 and N >= 1024
+    for got, base, name in zip(results["1"], results["0"], ("dx", "dw", "db", "dx masked+acc", "dw'", "db'")):
+        if name.startswith("dx") and dx_split_alone:
+            assert_close(got, base, rtol, rtol * np.abs(base).max(), name)
+        else:
+            np.testing.assert_array_equal(got, base, err_msg=name)
+    dx, dw = results["1"][0], results["1"][1]
+    for got, want, name in ((dx, O.linear_grad_x(dy, w), "dx"), (dw, O.linear_grad_w(dy, x), "dw")):
+        assert_close(got, want, rtol, rtol * np.abs(want).max(), name)
+    masked = results["1"][3]
+    assert_close(masked, prior + O.linear_grad_x(dy, w) * (x > 0), 2 * rtol, 2 * rtol * np.abs(dx).max(), "dx masked+acc")
+
+
 def test_fused_entry_errors(device):
     buf = AnyBuffer.create(F32, device, 16)
     p = buf.data_ptr()
