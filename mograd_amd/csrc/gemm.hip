@@ -73,10 +73,10 @@ static int launch_f32_mfma(const GemmArgs& g, hipStream_t stream) {
       const unsigned rblocks = static_cast<unsigned>(ceil_div(numel, 256));
       if (bias)
         hipLaunchKernelGGL((gemm_splitk_reduce_kernel<float, true>), dim3(rblocks), dim3(256), 0, stream,
-                           partial.as<float>(), bias, c, numel, splits, N, epilogue_of<float>(g));
+                           partial.as<float>(), bias, c, numel, numel, splits, N, epilogue_of<float>(g));
       else
         hipLaunchKernelGGL((gemm_splitk_reduce_kernel<float, false>), dim3(rblocks), dim3(256), 0, stream,
-                           partial.as<float>(), bias, c, numel, splits, N, epilogue_of<float>(g));
+                           partial.as<float>(), bias, c, numel, numel, splits, N, epilogue_of<float>(g));
       MG_LAUNCH_CHECK();
       return MG_OK;
     }
@@ -221,10 +221,10 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
   const unsigned rblocks = static_cast<unsigned>(ceil_div(numel, 256));
   if (bias)
     hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, true>), dim3(rblocks), dim3(256), 0, stream, partial.as<float>(),
-                       bias, c, numel, splits, N, epilogue_of<T>(g));
+                       bias, c, numel, numel, splits, N, epilogue_of<T>(g));
   else
     hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, false>), dim3(rblocks), dim3(256), 0, stream, partial.as<float>(),
-                       bias, c, numel, splits, N, epilogue_of<T>(g));
+                       bias, c, numel, numel, splits, N, epilogue_of<T>(g));
   MG_LAUNCH_CHECK();
   return MG_OK;
 }
@@ -350,8 +350,10 @@ int colsum_dispatch(const void* a, void* dst, int64_t outer, int64_t reduce, int
 // MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH=0 switches it off (benchmarks, tests of the equivalence).
 template <typename T>
 static int linear_bwd_one_launch(const void* dy, const void* x, const void* w, void* dx, void* dw, int64_t M, int64_t N,
-                                 int64_t K, const void* relu_mask, bool dx_accumulate, hipStream_t stream, bool* done) {
+                                 int64_t K, const void* relu_mask, bool dx_accumulate, hipStream_t stream, bool* done,
+                                 int64_t dw_rows = -1) {
   *done = false;
+  if (dw_rows < 0) dw_rows = N;  // rows of dW to write: fewer than N when dY and W came zero-padded
   if (env_int("MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH", 1) == 0 || std::getenv("MOGRAD_HIP_GEMM16_PIPE")) return MG_OK;
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return MG_OK;
   if (M % kG16BK || N % kG16BK || !mult8(K)) return MG_OK;
@@ -390,22 +392,70 @@ static int linear_bwd_one_launch(const void* dy, const void* x, const void* w, v
   hipLaunchKernelGGL((linear_bwd_16bit_kernel<T>), dim3(static_cast<unsigned>(n_dw + x_tiles)), dim3(kGemmThreads), 0,
                      stream, pw, px, static_cast<int>(n_dw));
   MG_LAUNCH_CHECK();
-  const unsigned rblocks = static_cast<unsigned>(ceil_div(numel, 256));
+  const unsigned rblocks = static_cast<unsigned>(ceil_div(dw_rows * K, 256));
   hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, false>), dim3(rblocks), dim3(256), 0, stream, partial.as<float>(),
-                     static_cast<const T*>(nullptr), static_cast<T*>(dw), numel, splits, static_cast<int>(K),
+                     static_cast<const T*>(nullptr), static_cast<T*>(dw), dw_rows * K, numel, splits, static_cast<int>(K),
                      GemmEpilogue<T>{nullptr, nullptr, 0});
   MG_LAUNCH_CHECK();
   *done = true;
   return MG_OK;
 }
 
+// dst (rows, cols_to) = src (rows, cols) with zero columns appended; cols_to is a multiple of 8
+// and dst 16-byte aligned.  One thread per 8 output columns.
+template <typename T>
+__global__ __launch_bounds__(256) void pad_columns_kernel(const T* __restrict__ src, T* __restrict__ dst, int64_t rows,
+                                                          int cols, int cols_to) {
+  const int chunks = cols_to / 8;
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= rows * chunks) return;
+  const int64_t r = i / chunks;
+  const int c0 = static_cast<int>(i % chunks) * 8;
+  T v[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = c0 + e < cols ? src[r * cols + c0 + e] : from_float<T>(0.f);
+  *reinterpret_cast<uint4*>(dst + r * cols_to + c0) = *reinterpret_cast<const uint4*>(v);
+}
+
+// A layer whose width N is not a multiple of the k-step (a 65-symbol vocabulary) cannot take
+// the pipelined kernels as it lies: rows of dY start at odd addresses, and both products
+// would go to the element-staged kernel (3-4 % of the matrix cores busy).  Here dY gets
+// zero columns and W zero rows up to the next multiple of 32 (copies of M x N and N x K
+// elements, small beside X and dX), the padded layer goes through the common launch, and
+// only the first N rows of dW are written.  The padding adds exact zeros to every sum.
+template <typename T>
+static int linear_bwd_padded(const void* dy, const void* x, const void* w, void* dx, void* dw, int64_t M, int64_t N,
+                             int64_t K, const void* relu_mask, bool dx_accumulate, hipStream_t stream, bool* done) {
+  *done = false;
+  const int64_t n_to = ceil_div(N, kG16BK) * kG16BK;
+  if (N % kG16BK == 0 || n_to > 2 * N || M % kG16BK || !mult8(K) || M < 1024 || n_to * K > 0x7fffffffLL) return MG_OK;
+  if (env_int("MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH", 1) == 0 || std::getenv("MOGRAD_HIP_GEMM16_PIPE")) return MG_OK;
+  Scratch dy_pad, w_pad;
+  MG_TRY(dy_pad.take(M * n_to * static_cast<int64_t>(sizeof(T))));
+  MG_TRY(w_pad.take(n_to * K * static_cast<int64_t>(sizeof(T))));
+  // W: rows appended to a row-major array, i.e. one row of N * K elements padded to n_to * K
+  const int64_t w_chunks = n_to * K / 8, dy_chunks = M * (n_to / 8);
+  hipLaunchKernelGGL((pad_columns_kernel<T>), dim3(static_cast<unsigned>(ceil_div(w_chunks, 256))), dim3(256), 0, stream,
+                     static_cast<const T*>(w), w_pad.as<T>(), static_cast<int64_t>(1), static_cast<int>(N * K),
+                     static_cast<int>(n_to * K));
+  MG_LAUNCH_CHECK();
+  hipLaunchKernelGGL((pad_columns_kernel<T>), dim3(static_cast<unsigned>(ceil_div(dy_chunks, 256))), dim3(256), 0, stream,
+                     static_cast<const T*>(dy), dy_pad.as<T>(), M, static_cast<int>(N), static_cast<int>(n_to));
+  MG_LAUNCH_CHECK();
+  return linear_bwd_one_launch<T>(dy_pad.as<T>(), x, w_pad.as<T>(), dx, dw, M, n_to, K, relu_mask, dx_accumulate, stream,
+                                  done, N);
+}
+
 int linear_bwd_products(const void* dy, const void* x, const void* w, void* dx, void* dw, int64_t M, int64_t N, int64_t K,
                         const void* relu_mask, bool dx_accumulate, int dtype, hipStream_t stream, bool* done) {
   *done = false;
-  if (dtype == MG_BF16)
-    return linear_bwd_one_launch<bf16_t>(dy, x, w, dx, dw, M, N, K, relu_mask, dx_accumulate, stream, done);
-  if (dtype == MG_F16)
-    return linear_bwd_one_launch<f16_t>(dy, x, w, dx, dw, M, N, K, relu_mask, dx_accumulate, stream, done);
+  if (dtype == MG_BF16) {
+    MG_TRY(linear_bwd_one_launch<bf16_t>(dy, x, w, dx, dw, M, N, K, relu_mask, dx_accumulate, stream, done));
+    if (!*done) MG_TRY(linear_bwd_padded<bf16_t>(dy, x, w, dx, dw, M, N, K, relu_mask, dx_accumulate, stream, done));
+  } else if (dtype == MG_F16) {
+    MG_TRY(linear_bwd_one_launch<f16_t>(dy, x, w, dx, dw, M, N, K, relu_mask, dx_accumulate, stream, done));
+    if (!*done) MG_TRY(linear_bwd_padded<f16_t>(dy, x, w, dx, dw, M, N, K, relu_mask, dx_accumulate, stream, done));
+  }
   return MG_OK;
 }
 

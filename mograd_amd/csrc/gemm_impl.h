@@ -1046,14 +1046,15 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_pipe_kernel(
   }  // tiles of this workgroup
 }
 
-// out[i] = sum_s partial[s][i] (+ bias[i % N]), converted to T.  A workgroup covers 64
+// out[i] = sum_s partial[s * slice + i] (+ bias[i % N]) for i < numel <= slice, converted to T.  A workgroup covers 64
 // groups of four consecutive outputs; its four waves each sum every fourth split (eight
 // independent 16-byte loads in flight per thread) and the four sums meet in LDS.  The
 // order of the additions is fixed, so the result is deterministic.
 template <typename T, bool HAS_BIAS>
 __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ partial,
                                                                  const T* __restrict__ bias, T* __restrict__ out,
-                                                                 int64_t numel, int splits, int N, GemmEpilogue<T> ep) {
+                                                                 int64_t numel, int64_t slice, int splits, int N,
+                                                                 GemmEpilogue<T> ep) {
   __shared__ float4 tile[4][64];
   const int cx = threadIdx.x % 64;
   const int sl = threadIdx.x / 64;
@@ -1064,18 +1065,18 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
     int s = sl;
     if (full) {
       for (; s + 4 < splits; s += 8) {
-        const float4 u = *reinterpret_cast<const float4*>(partial + static_cast<int64_t>(s) * numel + i);
-        const float4 w = *reinterpret_cast<const float4*>(partial + static_cast<int64_t>(s + 4) * numel + i);
+        const float4 u = *reinterpret_cast<const float4*>(partial + static_cast<int64_t>(s) * slice + i);
+        const float4 w = *reinterpret_cast<const float4*>(partial + static_cast<int64_t>(s + 4) * slice + i);
         acc0.x += u.x; acc0.y += u.y; acc0.z += u.z; acc0.w += u.w;
         acc1.x += w.x; acc1.y += w.y; acc1.z += w.z; acc1.w += w.w;
       }
       for (; s < splits; s += 4) {
-        const float4 u = *reinterpret_cast<const float4*>(partial + static_cast<int64_t>(s) * numel + i);
+        const float4 u = *reinterpret_cast<const float4*>(partial + static_cast<int64_t>(s) * slice + i);
         acc0.x += u.x; acc0.y += u.y; acc0.z += u.z; acc0.w += u.w;
       }
     } else {
       for (; s < splits; s += 4) {
-        const float* p = partial + static_cast<int64_t>(s) * numel + i;
+        const float* p = partial + static_cast<int64_t>(s) * slice + i;
         acc0.x += p[0];
         if (i + 1 < numel) acc0.y += p[1];
         if (i + 2 < numel) acc0.z += p[2];

@@ -595,6 +595,39 @@ def test_linear_bwd_one_launch_matches_two(device, monkeypatch, dtype, rtol, M, 
     assert_close(masked, prior + O.linear_grad_x(dy, w) * (x > 0), 2 * rtol, 2 * rtol * np.abs(dx).max(), "dx masked+acc")
 
 
+@pytest.mark.parametrize("dtype,rtol", [(F16, 2e-3), (BF16, 1.6e-2)])
+@pytest.mark.parametrize("M,N,K", [(4096, 65, 384), (1024, 72, 64), (2048, 100, 200), (1056, 33, 136)])
+def test_linear_bwd_ragged_width(device, monkeypatch, dtype, rtol, M, N, K):
+    # A width that is no multiple of 32 (the 65-symbol head): dY and W are zero-padded to the
+    # next multiple inside the call and go through the common launch; without it
+    # (MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH=0) the element-staged kernels take both products.
+    # Both against the oracle; dX also bit for bit (the padding adds exact zeros, same k order).
+    lib, st = device.lib, device.stream
+    x = np.maximum(round_to_dtype(normal(53, 0, (M, K)), dtype), 0)
+    w = round_to_dtype(normal(53, 1, (N, K), std=0.05), dtype)
+    dy = round_to_dtype(normal(53, 2, (M, N), std=0.5), dtype)
+    prior = round_to_dtype(normal(53, 3, (M, K)), dtype)
+    bx, bw, bdy = (AnyBuffer.from_numpy(device, a, dtype) for a in (x, w, dy))
+    results = {}
+    for mode in ("0", "1"):
+        monkeypatch.setenv("MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH", mode)
+        dx = AnyBuffer.from_numpy(device, prior, dtype)
+        # canaries behind dW: only N rows may be written although the padded product has more
+        dw = AnyBuffer.from_numpy(device, np.full((N + 32) * K, 7.0, np.float32), dtype)
+        db = AnyBuffer.create(dtype, device, N)
+        lib.mg_linear_bwd_fused(_ptr(bdy), _ptr(bx), _ptr(bw), _ptr(dx), _ptr(dw), _ptr(db), M, N, K, 1, 1, dtype, st)
+        dw_all = dw.to_numpy((N + 32, K))
+        assert (dw_all[N:] == 7.0).all()
+        results[mode] = (dx.to_numpy((M, K)), dw_all[:N], db.to_numpy())
+    np.testing.assert_array_equal(results["1"][0], results["0"][0], err_msg="dx")
+    np.testing.assert_array_equal(results["1"][2], results["0"][2], err_msg="db")
+    want_dx = prior + O.linear_grad_x(dy, w) * (x > 0)
+    want_dw = O.linear_grad_w(dy, x)
+    for mode in ("0", "1"):
+        assert_close(results[mode][0], want_dx, 2 * rtol, 2 * rtol * np.abs(want_dx).max(), "dx " + mode)
+        assert_close(results[mode][1], want_dw, rtol, rtol * np.abs(want_dw).max(), "dw " + mode)
+
+
 def test_fused_entry_errors(device):
     buf = AnyBuffer.create(F32, device, 16)
     p = buf.data_ptr()
