@@ -33,12 +33,17 @@ template <>
 __device__ __forceinline__ f16_t from_float<f16_t>(float v) {
   return static_cast<f16_t>(v);
 }
-// Round to nearest even; NaN stays NaN.
+// fp32 -> bf16, round to nearest even, NaN stays NaN: the hardware conversion
+// (v_cvt_pk_bf16_f32, one instruction for two values; the bit arithmetic it replaces took
+// seven per value, which showed in every 16-bit kernel's output loop).
+typedef __bf16 hw_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float hw_f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t bf16_pack2_rne(float lo, float hi) {
+  const hw_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, hw_bf16x2));
+}
 __device__ __forceinline__ uint16_t bf16_bits_rne(float v) {
-  uint32_t u = __float_as_uint(v);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(v));
 }
 template <>
 __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) {
@@ -111,7 +116,7 @@ struct VecIO<bf16_t, 8> {
     uint32_t w[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      w[i] = static_cast<uint32_t>(bf16_bits_rne(v[2 * i])) | (static_cast<uint32_t>(bf16_bits_rne(v[2 * i + 1])) << 16);
+      w[i] = bf16_pack2_rne(v[2 * i], v[2 * i + 1]);
     *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
   }
 };
