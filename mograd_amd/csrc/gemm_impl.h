@@ -328,6 +328,19 @@ typedef __bf16 gemm_bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 gemm_f16x2 __attribute__((ext_vector_type(2)));
 typedef float gemm_f32x2 __attribute__((ext_vector_type(2)));
 
+// Two fp32 values rounded to T (nearest even), the first in the low half.
+template <typename T>
+__device__ __forceinline__ uint32_t gemm16_pack2(float lo, float hi);
+template <>
+__device__ __forceinline__ uint32_t gemm16_pack2<bf16_t>(float lo, float hi) {
+  return bf16_pack2_rne(lo, hi);
+}
+template <>
+__device__ __forceinline__ uint32_t gemm16_pack2<f16_t>(float lo, float hi) {
+  const gemm_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, gemm_f16x2));
+}
+
 template <typename T>
 struct GemmMma16;
 template <>
@@ -471,20 +484,32 @@ __device__ __forceinline__ void gemm16_write_tile(const floatx16 (&acc)[2][2], u
   if constexpr (!SPLIT_K) {
     const bool wide_out = (N % 8 == 0) && (ldc % 8 == 0) && (bsc % 8 == 0) && (reinterpret_cast<uintptr_t>(C) % 16 == 0);
     if (wide_out) {
+      // An accumulator holds one column and, per group of four registers, four consecutive
+      // rows.  Two lanes with neighbouring columns swap packed pairs of rows, so that the even
+      // lane holds (own, neighbour) of the first row of a pair and the odd lane (neighbour,
+      // own) of the second: 32 four-byte LDS writes per thread instead of 64 two-byte ones,
+      // and three VALU instructions per pair (convert, swap, byte select).
+      const int odd = lane & 1;
+      const uint32_t select = odd ? 0x03020706u : 0x05040100u;
+      uint32_t* const base32 =
+          reinterpret_cast<uint32_t*>(mine + ((lane / 32) * 4 + odd) * kG16Stride + (lane % 32 - odd));
 #pragma unroll
       for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
         for (int tj = 0; tj < 2; ++tj) {
-          const int cl = tj * 32 + lane % 32;
-          const int col = n0 + wn + cl;
+          const int col = n0 + wn + tj * 32 + lane % 32;
           const float bv = (HAS_BIAS && col < N) ? to_float(bias[col]) : 0.f;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int rl = ti * 32 + (r / 4) * 8 + (lane / 32) * 4 + (r % 4);
-            float f = acc[ti][tj][r] + bv;
-            if (ep.relu) f = f > 0.f ? f : 0.f;
-            const T v = from_float<T>(f);
-            mine[rl * kG16Stride + cl] = __builtin_bit_cast(uint16_t, v);
+          for (int rp = 0; rp < 8; ++rp) {  // rows 2 rp and 2 rp + 1 of the sixteen
+            float f0 = acc[ti][tj][2 * rp] + bv, f1 = acc[ti][tj][2 * rp + 1] + bv;
+            if (ep.relu) {
+              f0 = f0 > 0.f ? f0 : 0.f;
+              f1 = f1 > 0.f ? f1 : 0.f;
+            }
+            const uint32_t w = gemm16_pack2<T>(f0, f1);
+            const uint32_t y = __builtin_amdgcn_update_dpp(0, w, kDppQuadXor1, 0xf, 0xf, false);
+            const int rl = ti * 32 + (rp / 2) * 8 + (rp % 2) * 2;  // without the lane's own (lane / 32) * 4 + odd
+            base32[(rl * kG16Stride + tj * 32) / 2] = __builtin_amdgcn_perm(y, w, select);
           }
         }
       __syncthreads();
