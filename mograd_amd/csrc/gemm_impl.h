@@ -14,6 +14,8 @@
 // chunk overlaps the MFMAs of the current one) -> LDS -> MFMA operands.
 #pragma once
 
+#include <type_traits>
+
 #include "mg_device.h"
 #include "mg_internal.h"
 
@@ -493,57 +495,76 @@ __device__ __forceinline__ void gemm16_write_tile(const floatx16 (&acc)[2][2], u
       const uint32_t select = odd ? 0x03020706u : 0x05040100u;
       uint32_t* const base32 =
           reinterpret_cast<uint32_t*>(mine + ((lane / 32) * 4 + odd) * kG16Stride + (lane % 32 - odd));
+      // (One copy of the loop per setting of the relu flag: inside the loop the flag would
+      // cost two more instructions per value.)
+      auto stage = [&](auto relu) {
 #pragma unroll
-      for (int ti = 0; ti < 2; ++ti)
+        for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
-        for (int tj = 0; tj < 2; ++tj) {
-          const int col = n0 + wn + tj * 32 + lane % 32;
-          const float bv = (HAS_BIAS && col < N) ? to_float(bias[col]) : 0.f;
-#pragma unroll
-          for (int rp = 0; rp < 8; ++rp) {  // rows 2 rp and 2 rp + 1 of the sixteen
-            float f0 = acc[ti][tj][2 * rp] + bv, f1 = acc[ti][tj][2 * rp + 1] + bv;
-            if (ep.relu) {
-              f0 = f0 > 0.f ? f0 : 0.f;
-              f1 = f1 > 0.f ? f1 : 0.f;
+          for (int tj = 0; tj < 2; ++tj) {
+            float bv = 0.f;
+            if constexpr (HAS_BIAS) {
+              const int col = n0 + wn + tj * 32 + lane % 32;
+              bv = col < N ? to_float(bias[col]) : 0.f;
             }
-            const uint32_t w = gemm16_pack2<T>(f0, f1);
-            const uint32_t y = __builtin_amdgcn_update_dpp(0, w, kDppQuadXor1, 0xf, 0xf, false);
-            const int rl = ti * 32 + (rp / 2) * 8 + (rp % 2) * 2;  // without the lane's own (lane / 32) * 4 + odd
-            base32[(rl * kG16Stride + tj * 32) / 2] = __builtin_amdgcn_perm(y, w, select);
+#pragma unroll
+            for (int rp = 0; rp < 8; ++rp) {  // rows 2 rp and 2 rp + 1 of the sixteen
+              float f0 = acc[ti][tj][2 * rp], f1 = acc[ti][tj][2 * rp + 1];
+              if constexpr (HAS_BIAS) f0 += bv, f1 += bv;
+              if constexpr (decltype(relu)::value) {
+                f0 = f0 > 0.f ? f0 : 0.f;
+                f1 = f1 > 0.f ? f1 : 0.f;
+              }
+              const uint32_t w = gemm16_pack2<T>(f0, f1);
+              const uint32_t y = __builtin_amdgcn_update_dpp(w, w, kDppQuadXor1, 0xf, 0xf, false);
+              const int rl = ti * 32 + (rp / 2) * 8 + (rp % 2) * 2;  // without the lane's own (lane / 32) * 4 + odd
+              base32[(rl * kG16Stride + tj * 32) / 2] = __builtin_amdgcn_perm(y, w, select);
+            }
           }
-        }
+      };
+      if (ep.relu) stage(std::true_type{});
+      else stage(std::false_type{});
       __syncthreads();
-      T* cbase = C + batch * bsc;
-      const T* rbase = ep.residual ? ep.residual + batch * bsc : nullptr;
-      const T* mbase = ep.relu_mask ? ep.relu_mask + batch * bsc : nullptr;
+      // Rows of the wave's 64 x 64 tile go out 16 bytes per lane, eight lanes to a row, eight
+      // rows per store: one address per thread, stepped by eight rows.
+      const int rl0 = lane / 8, ch = lane % 8;
+      const int row0 = m0 + wm + rl0;
+      const int col = n0 + wn + ch * 8;
+      if (col >= N) return;
+      const int64_t at0 = batch * bsc + static_cast<int64_t>(row0) * ldc + col;
+      const int64_t step = 8 * ldc;
+      const uint16_t* src = mine + rl0 * kG16Stride + ch * 8;
+      const T* rbase = ep.residual;
+      const T* mbase = ep.relu_mask;
+      if (!rbase && !mbase) {
+        T* dst = C + at0;
+        uint4 v[8];  // all eight LDS reads first: their latencies overlap
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<const uint4*>(src + i * 8 * kG16Stride);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (row0 + 8 * i < M) *reinterpret_cast<uint4*>(dst + i * step) = v[i];
+        return;
+      }
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const int chunk = lane + i * kWave;
-        const int rl = chunk / 8, ch = chunk % 8;
-        const int row = m0 + wm + rl;
-        const int col = n0 + wn + ch * 8;
-        if (row < M && col < N) {
-          const int64_t at = static_cast<int64_t>(row) * ldc + col;
-          if (rbase || mbase) {
-            float v[8];
-            VecIO<T, 8>::load(reinterpret_cast<const T*>(mine + rl * kG16Stride + ch * 8), v);
-            if (mbase) {
-              float mk[8];
-              VecIO<T, 8>::load(mbase + at, mk);
+        if (row0 + 8 * i >= M) break;
+        const int64_t at = at0 + i * step;
+        float v[8];
+        VecIO<T, 8>::load(reinterpret_cast<const T*>(src + i * 8 * kG16Stride), v);
+        if (mbase) {
+          float mk[8];
+          VecIO<T, 8>::load(mbase + at, mk);
 #pragma unroll
-              for (int e = 0; e < 8; ++e) v[e] = mk[e] > 0.f ? v[e] : 0.f;
-            }
-            if (rbase) {
-              float rs[8];
-              VecIO<T, 8>::load(rbase + at, rs);
-#pragma unroll
-              for (int e = 0; e < 8; ++e) v[e] += rs[e];
-            }
-            VecIO<T, 8>::store(cbase + at, v);
-          } else {
-            *reinterpret_cast<uint4*>(cbase + at) = *reinterpret_cast<const uint4*>(mine + rl * kG16Stride + ch * 8);
-          }
+          for (int e = 0; e < 8; ++e) v[e] = mk[e] > 0.f ? v[e] : 0.f;
         }
+        if (rbase) {
+          float rs[8];
+          VecIO<T, 8>::load(rbase + at, rs);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] += rs[e];
+        }
+        VecIO<T, 8>::store(C + at, v);
       }
       return;
     }
