@@ -39,11 +39,20 @@ LN_FWD_BYTES = 2 * LN_ROWS * LN_COLS * 4 + 2 * LN_COLS * 4            # x, y, ga
 LN_BWD_BYTES = 3 * LN_ROWS * LN_COLS * 4 + 3 * LN_COLS * 4            # dy, x, dx, gamma, dgamma, dbeta
 CE_FUSED_BYTES = 2 * CE_ROWS * CE_COLS * 4 + CE_ROWS * 4 + 4          # logits, dlogits, labels, loss
 
-# HBM bytes per launch of the cross-entropy rows kernel, from two `rocprofv3 --pmc` runs
-# (FETCH_SIZE, then WRITE_SIZE) of this same script, each scaled by what the counter reads
-# for the calibration copy below: (805943.9 / 0.50005 + 1610378.9 / 1.0) KiB.  The counter
-# runs and the factors are in profiles/ce_rows_kernel_8192x50304_hbm_traffic.md.
-CE_MEASURED_TRAFFIC_BYTES = int((805943.9 / 0.50005 + 1610378.9) * 1024)
+def _measured_traffic(key: str):
+    """HBM bytes per launch of one kernel, from the counter figures committed beside the
+    profiles (profiles/hbm_traffic.json: per-dispatch means of FETCH_SIZE and WRITE_SIZE in
+    KiB from two `rocprofv3 --pmc` runs of this script, and what each counter reads per true
+    KiB for the plain copy of known size that the ln_ce workload performs).  None when the
+    file has no such entry."""
+    try:
+        with open(ROOT / "profiles" / "hbm_traffic.json") as f:
+            entry = json.load(f).get(key)
+    except (OSError, ValueError):
+        return None
+    if not entry:
+        return None
+    return int((entry["fetch_kib"] / entry["fetch_factor"] + entry["write_kib"] / entry["write_factor"]) * 1024)
 
 
 def _rng(config: int, tensor: int) -> np.random.Generator:
@@ -261,7 +270,8 @@ def bench_mlp(args, dev) -> dict:
         "config": {"workload": "README MLP fwd+bwd fp32: x (2048,4096) -> Linear 4096 +ReLU -> LayerNorm -> Linear 4096 "
                                "+ReLU -> Linear 10, cross-entropy, labels in [0,10)"},
         "roofline": {"bound": "mfma", "kernel": "gemm_f32_pipe_kernel, " + dom["name"], "achieved": dom["achieved_TFLOPs"],
-                     "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac_of_mfma_peak"], "traffic": None},
+                     "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac_of_mfma_peak"],
+                     "traffic": _measured_traffic("gemm_f32_pipe_kernel_mlp_step")},
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:
@@ -344,7 +354,7 @@ def bench_attention(args, dev) -> dict:
         "roofline": {"bound": "mfma", "kernel": "attn_bwd_mfma_kernel (dK/dV and dQ walks) + attn_delta_rows_kernel "
                                                 "(mg_flash_attn_bwd, causal S1024)",
                      "achieved": dom["achieved_TFLOPs"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": dom["frac_of_mfma_peak"], "traffic": None},
+                     "frac": dom["frac_of_mfma_peak"], "traffic": _measured_traffic("attn_bwd_mfma_kernel_b8h12s1024")},
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:
@@ -501,7 +511,8 @@ def bench_gpt(args, dev) -> dict:
                      "kernel": "linear_bwd_16bit_kernel (+ gemm_splitk_reduce_kernel): mg_linear_bwd at the block's four "
                                "layer shapes, 4 M N K FLOP each, mean over the four",
                      "achieved": round(lin_tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(lin_tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "frac": round(lin_tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": _measured_traffic("linear_bwd_16bit_kernel_gpt_step"),
                      "algorithmic_flops": lin_flops / 4, "launch_ms": round(lin_ms / 4, 5),
                      "share_of_step": round(L * lin_ms / ms, 3)},
         "whole_step": {"algorithmic_flops": flops, "achieved_TFLOPs": round(tf, 1),
@@ -709,7 +720,7 @@ def bench_ln_ce(args, dev) -> dict:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(dominant["achieved_GBps"] / HBM_PEAK_GBS, 4),
-            "traffic": CE_MEASURED_TRAFFIC_BYTES,
+            "traffic": _measured_traffic("ce_rows_kernel_8192x50304_f32"),
         },
         "kernels": kernels,
     }

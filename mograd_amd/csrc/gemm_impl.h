@@ -676,12 +676,23 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
 //     (timed on the device: 18.5-18.7 clocks per read with four waves reading, as for
 //     consecutive addresses; 32 with c ^ (r % 8));
 //   otherwise: [k][16 chunks of 8 rows], chunk c of k-row kk at position
-//     c ^ (2 * (kk % 4)), read with `ds_read_b64_tr_b16` (within 16 lanes, lane i supplies
+//     c ^ gemm16_tr_swizzle(kk), read with `ds_read_b64_tr_b16` (within 16 lanes, lane i supplies
 //     the four elements 4*i .. 4*i+3 of a 4 x 16 block and receives column i), which turns
 //     four k-rows of 16 consecutive rows into each lane's four consecutive k.
 // ------------------------------------------------------------------------------------
 
 typedef short gemm_i16x4 __attribute__((ext_vector_type(4)));
+
+// Where 16-byte chunk c of k-row kk of an m/n-contiguous operand sits in its LDS row:
+// c ^ swizzle(kk).  A k-row is 256 or 512 bytes, a whole number of trips round the 64 banks,
+// so without it every k-row would start on bank 0.  A transposing read takes 32 bytes of each
+// of four k-rows (kk % 4 = 0..3) per sixteen lanes: 4 * (kk % 4) puts those on four different
+// 32-byte bank groups that leave the neighbouring sixteen lanes' groups (chunk + 2) free, and
+// 2 * (kk / 8 % 2) moves the upper half-wave (k-rows + 8) onto the remaining groups, so that
+// whichever 32 lanes the LDS serves together touch every bank once.  (With c ^ 2 * (kk % 4),
+// two sixteen-lane groups shared their bank groups: 43 % of the LDS cycles of the Linear
+// backward kernel were conflict cycles.)
+__device__ __forceinline__ constexpr int gemm16_tr_swizzle(int kk) { return 4 * (kk % 4) ^ 2 * ((kk / 8) % 2); }
 
 // Copy requests per thread, k-step and operand of ROWS rows, for a workgroup of NW waves.
 constexpr int gemm16_pipe_requests(int rows, int bk, int nw) { return rows * bk * 2 / 16 / (nw * 64); }
@@ -702,7 +713,7 @@ __device__ __forceinline__ void gemm16_pipe_sources(int64_t ld, int o0, int O,
       const int r = slot / CPR, c = (slot % CPR) ^ ((r / (16 / CPR)) % CPR);
       src[i] = static_cast<int64_t>(min(o0 + r, O - 1)) * ld + c * 8;  // rows past the edge are never stored
     } else {
-      const int kk = slot / CPK, c = (slot % CPK) ^ (2 * (kk % 4));
+      const int kk = slot / CPK, c = (slot % CPK) ^ gemm16_tr_swizzle(kk);
       const int o = o0 + c * 8;
       src[i] = static_cast<int64_t>(kk) * ld + (o < O ? o : o0);
     }
@@ -738,7 +749,7 @@ __device__ __forceinline__ uint4 gemm16_pipe_frag(const char* __restrict__ lds_s
     const int o = o_base + ((lane / 16) % 2) * 16 + 4 * (lane % 4);  // first of the 4 rows this lane supplies
     const int kq = (lane % 16) / 4;                                 // its k-row within a group of 4
     const int kk = ks * 16 + (lane / 32) * 8 + kq;
-    const char* at = lds_step + kk * (ROWS * 2) + (((o / 16) ^ kq) * 32) + (o % 16) * 2;
+    const char* at = lds_step + kk * (ROWS * 2) + (((o / 8) ^ gemm16_tr_swizzle(kk)) * 16) + (o % 8) * 2;
     using lds_i16x4 = __attribute__((address_space(3))) gemm_i16x4;
     const gemm_i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
         reinterpret_cast<lds_i16x4*>(reinterpret_cast<uintptr_t>(at)));
