@@ -16,8 +16,13 @@
 // atomics, so every output is written once and results are reproducible.
 //
 // A product that contracts over the streamed index needs the streamed tile transposed
-// ([d][row]); tiles are staged in LDS in both orientations, the transposed one written as
-// packed pairs of rows so that the LDS stores are full dwords.
+// ([d][row]).  A tile is staged in LDS once, row-major with its 16-byte chunks swizzled; the
+// products that contract over its columns read it with ds_read_b128, the ones that contract
+// over its rows with ds_read_b64_tr_b16, which transposes 4 x 16 blocks on the way out.
+// For head dims up to 64 without a bias the backward walks are software-pipelined
+// (attn_dkdv_pipe_block, attn_dq_pipe_block): tiles copied global -> LDS by
+// global_load_lds_dwordx4 into a ring of three buffers, the exponentials of one tile issued
+// between the matrix instructions of its neighbours.
 //
 // Layouts: Q, K, V, dQ, dK, dV BSHD; O, dO BHSD; mask (B,H,S,S); LSE, delta (B,H,S) fp32.
 #include <cstdlib>
