@@ -789,6 +789,10 @@ struct Gemm16Problem {
   int64_t lda, ldb, ldc, bsa, bsb, bsc;
   int tiles_m, tiles_n, k_per_split, splits, batches;
   GemmEpilogue<T> ep;
+  // Split along K with an m-contiguous A only (dW = dY^T X): when set, the workgroups of the
+  // first tile column also sum their A tiles over k, i.e. dY over its rows, and leave one
+  // partial row of the bias gradient per K range at colsum_part[split * M + m].
+  float* colsum_part = nullptr;
 };
 
 // The work of workgroup `bid` of a launch for one product; `lds` is the workgroup's
@@ -842,6 +846,15 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+  // Column sums of the A tiles (see Gemm16Problem::colsum_part): a thread takes one 16-byte
+  // chunk (8 of the tile's 128 m) of every 16th k-row.
+  constexpr bool CAN_COLSUM = SPLIT_K && !A_KC && TM == 128;
+  const bool colsum = CAN_COLSUM && pr.colsum_part != nullptr && tn == 0;
+  const int cs_chunk = threadIdx.x % 16, cs_row = threadIdx.x / 16;
+  float cs_acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) cs_acc[e] = 0.f;
+
   const uint16_t* a16 = reinterpret_cast<const uint16_t*>(A);
   const uint16_t* b16 = reinterpret_cast<const uint16_t*>(B);
   int64_t src_a[NIA], src_b[NIB];
@@ -870,6 +883,18 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
     }
     const char* la = lds + cur * OP;
     const char* lb = la + OPA;
+    if constexpr (CAN_COLSUM) {
+      if (colsum) {
+#pragma unroll
+        for (int j = 0; j < BK / 16; ++j) {
+          const int kk = cs_row + 16 * j;
+          float v[8];
+          VecIO<T, 8>::load(reinterpret_cast<const T*>(la + kk * (TM * 2) + ((cs_chunk ^ gemm16_tr_swizzle(kk)) * 16)), v);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) cs_acc[e] += v[e];
+        }
+      }
+    }
     // The fragments of k-slice ks + 1 are requested before the products of slice ks, so
     // their LDS latency runs under four MFMAs.
     uint4 fa[2][2], fb[2][2];
@@ -896,6 +921,25 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
   }
   __syncthreads();  // every wave is done with the staged tiles: their memory serves the output
 
+  if constexpr (CAN_COLSUM) {
+    if (colsum) {
+      // sixteen threads hold sums for the same 8 columns (k-rows 0, 16, ... / 1, 17, ... / ...):
+      // added in a fixed order through LDS, one thread per column
+      constexpr int kPitch = 128 + 4;
+      float* red = reinterpret_cast<float*>(lds);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) red[cs_row * kPitch + cs_chunk * 8 + e] = cs_acc[e];
+      __syncthreads();
+      if (threadIdx.x < 128 && m0 + static_cast<int>(threadIdx.x) < M) {
+        float sum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sum += red[r * kPitch + threadIdx.x];
+        pr.colsum_part[static_cast<int64_t>(split) * M + m0 + threadIdx.x] = sum;
+      }
+      __syncthreads();
+    }
+  }
+
   uint16_t* mine = reinterpret_cast<uint16_t*>(lds) + wave * 64 * kG16Stride;
   gemm16_write_tile<T, HAS_BIAS, SPLIT_K>(acc, mine, bias, C, partial, M, N, ldc, bsc, batch,
                                           split, SPLIT_K ? batches : 1,
@@ -914,10 +958,12 @@ __global__ __launch_bounds__(TM * 2, gemm16_pipe_occupancy(BK, NSTAGE, TM)) void
 }
 
 // Both products of a Linear layer's backward in one launch: workgroups [0, n_dw) take the
-// K ranges of dW = dY^T X (their partial tiles are summed by gemm_splitk_reduce_kernel
+// K ranges of dW = dY^T X (their partial tiles are summed by linear_bwd_finish_kernel
 // afterwards), the rest the tiles of dX = dY W.  The longer-running dW ranges start first
 // and the dX tiles fill the CUs as those drain, where two launches each end in a tail of
-// half-empty CUs (384 dX tiles on 256 CUs) and pay a launch apiece.
+// half-empty CUs (384 dX tiles on 256 CUs) and pay a launch apiece.  With
+// dw.colsum_part set, the dW workgroups of the first tile column also produce the bias
+// gradient's partial rows from the dY tiles they hold anyway.
 template <typename T>
 __global__ __launch_bounds__(256, gemm16_pipe_occupancy(32, 2, 128)) void linear_bwd_16bit_kernel(
     Gemm16Problem<T> dw, Gemm16Problem<T> dx, int n_dw) {
@@ -1108,14 +1154,13 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_pipe_kernel(
 // independent 16-byte loads in flight per thread) and the four sums meet in LDS.  The
 // order of the additions is fixed, so the result is deterministic.
 template <typename T, bool HAS_BIAS>
-__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ partial,
-                                                                 const T* __restrict__ bias, T* __restrict__ out,
-                                                                 int64_t numel, int64_t slice, int splits, int N,
-                                                                 GemmEpilogue<T> ep) {
-  __shared__ float4 tile[4][64];
+__device__ __forceinline__ void gemm_splitk_reduce_block(float4 (&tile)[4][64], int64_t bid,
+                                                         const float* __restrict__ partial, const T* __restrict__ bias,
+                                                         T* __restrict__ out, int64_t numel, int64_t slice, int splits,
+                                                         int N, const GemmEpilogue<T>& ep) {
   const int cx = threadIdx.x % 64;
   const int sl = threadIdx.x / 64;
-  const int64_t i = (static_cast<int64_t>(blockIdx.x) * 64 + cx) * 4;
+  const int64_t i = (bid * 64 + cx) * 4;
   float4 acc0 = make_float4(0.f, 0.f, 0.f, 0.f), acc1 = acc0;
   if (i < numel) {
     const bool full = i + 3 < numel;
@@ -1150,6 +1195,48 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
     const float bv = HAS_BIAS ? to_float(bias[(i + e) % N]) : 0.f;
     out[i + e] = gemm_finish<T>(r[e] + bv, ep, i + e);
   }
+}
+
+template <typename T, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ partial,
+                                                                 const T* __restrict__ bias, T* __restrict__ out,
+                                                                 int64_t numel, int64_t slice, int splits, int N,
+                                                                 GemmEpilogue<T> ep) {
+  __shared__ float4 tile[4][64];
+  gemm_splitk_reduce_block<T, HAS_BIAS>(tile, blockIdx.x, partial, bias, out, numel, slice, splits, N, ep);
+}
+
+// What follows the common launch of a Linear layer's backward: workgroups [0, dw_blocks) sum
+// the K ranges of dW (gemm_splitk_reduce_block), the rest sum the `groups` partial rows of
+// the bias gradient that the launch left (one per K range), 64 columns per workgroup,
+// every fourth row per 64 threads, then (t0 + t1) + (t2 + t3).  Fixed order, no atomics.
+template <typename T>
+__global__ __launch_bounds__(256) void linear_bwd_finish_kernel(const float* __restrict__ partial, T* __restrict__ dw,
+                                                                int64_t numel, int64_t slice, int splits, int K,
+                                                                int dw_blocks, const float* __restrict__ db_part,
+                                                                T* __restrict__ db, int groups, int N) {
+  __shared__ float4 tile[4][64];
+  const int bid = blockIdx.x;
+  if (bid < dw_blocks) {
+    gemm_splitk_reduce_block<T, false>(tile, bid, partial, static_cast<const T*>(nullptr), dw, numel, slice, splits, K,
+                                       GemmEpilogue<T>{nullptr, nullptr, 0});
+    return;
+  }
+  float(&sums)[4][64] = *reinterpret_cast<float(*)[4][64]>(&tile[0][0]);
+  const int cx = threadIdx.x % 64, sl = threadIdx.x / 64;
+  const int c = (bid - dw_blocks) * 64 + cx;
+  float a0 = 0.f, a1 = 0.f;
+  if (c < N) {
+    int g = sl;
+    for (; g + 4 < groups; g += 8) {
+      a0 += db_part[static_cast<int64_t>(g) * N + c];
+      a1 += db_part[static_cast<int64_t>(g + 4) * N + c];
+    }
+    for (; g < groups; g += 4) a0 += db_part[static_cast<int64_t>(g) * N + c];
+  }
+  sums[sl][cx] = a0 + a1;
+  __syncthreads();
+  if (sl == 0 && c < N) db[c] = from_float<T>((sums[0][cx] + sums[1][cx]) + (sums[2][cx] + sums[3][cx]));
 }
 
 }  // namespace mg

@@ -583,11 +583,16 @@ def test_linear_bwd_one_launch_matches_two(device, monkeypatch, dtype, rtol, M, 
     # Launched alone, a dX with fewer tiles than CUs and a long reduction is itself split along
     # N (fp32 partials, another summation order); inside the common launch it never is.
     dx_split_alone = -(-M // 128) * -(-K // 128) < 256 and N >= 1024
+    # In the common launch the bias gradient comes from the dW workgroups' dY tiles, one partial
+    # row per K range: another (fixed) summation order than mg_sum_axis on its own.
     for got, base, name in zip(results["1"], results["0"], ("dx", "dw", "db", "dx masked+acc", "dw'", "db'")):
-        if name.startswith("dx") and dx_split_alone:
+        if (name.startswith("dx") and dx_split_alone) or name.startswith("db"):
             assert_close(got, base, rtol, rtol * np.abs(base).max(), name)
         else:
             np.testing.assert_array_equal(got, base, err_msg=name)
+    np.testing.assert_array_equal(results["1"][2], results["1"][5], err_msg="db, second call")
+    want_db = O.linear_grad_b(dy)
+    assert_close(results["1"][2], want_db, rtol, rtol * np.abs(want_db).max(), "db")
     dx, dw = results["1"][0], results["1"][1]
     for got, want, name in ((dx, O.linear_grad_x(dy, w), "dx"), (dw, O.linear_grad_w(dy, x), "dw")):
         assert_close(got, want, rtol, rtol * np.abs(want).max(), name)
