@@ -1571,6 +1571,250 @@ __device__ __forceinline__ void attn_dq_pipe_block(const int block, char* smem, 
 
 // ---- backward launches --------------------------------------------------------------------
 
+// ---- whole heads in LDS (sequences up to 256, head dim 64, no bias) -----------------------
+// At short sequences the walks above are all prologue: a workgroup runs two to four steps
+// after loading its resident operand and filling its ring, four workgroups per (batch, head)
+// each read Q, K, V and dO again, and delta needs a launch of its own.  But the four tensors
+// of one (batch, head) are then at most 4 x 256 x 128 bytes = 128 KB and fit one CU's LDS.
+// Here one workgroup of eight waves copies them in once (global_load_lds, the conflict-free
+// image of the pipelined walks), computes delta = rowsum(dO o O) itself, and after one barrier
+// every wave runs, straight from LDS, first the dK/dV products of its own 32 keys over the
+// query tiles and then the dQ products of its own 32 queries over the key tiles: the per-tile
+// arithmetic of attn_dkdv_block and attn_dq_block, with no streaming and no further barrier.
+// Causal: wave w meets 8 - w query tiles in the first pass and w + 1 key tiles in the second,
+// so the waves carry equal loads without waiting for each other between the passes.
+constexpr int kResidentS = 256;
+constexpr int kResidentTensor = kResidentS * 128;                        // bytes of one tensor's image
+constexpr int kResidentLds = 4 * kResidentTensor + 2 * kResidentS * 4;   // Q, K, V, dO, -lse, -delta
+
+template <typename T, bool CAUSAL>
+__global__ __launch_bounds__(512, 1) void attn_bwd_resident_kernel(
+    const T* __restrict__ d_o, const T* __restrict__ o, const T* __restrict__ q, const T* __restrict__ k,
+    const T* __restrict__ v, const float* __restrict__ lse, T* __restrict__ dq, T* __restrict__ dk, T* __restrict__ dv,
+    AttnDims a, float scale) {
+  constexpr int DP = 64, KS = DP / 16, DT = DP / 32;
+  __shared__ __attribute__((aligned(1024))) char smem[kResidentLds];
+  const char* const q_rows = smem;
+  const char* const k_rows = smem + kResidentTensor;
+  const char* const v_rows = smem + 2 * kResidentTensor;
+  const char* const do_rows = smem + 3 * kResidentTensor;
+  float* const nlse_s = reinterpret_cast<float*>(smem + 4 * kResidentTensor);
+  float* const ndelta_s = nlse_s + kResidentS;
+
+  const int bh = blockIdx.x;
+  const int b = bh / a.H, h = bh % a.H;
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int half = lane / 32;
+  const int n_tiles = (a.S + 31) / 32;
+
+  // ---- copies: wave instruction j of a tensor covers its rows 8j .. 8j+7 (1 KB); this wave
+  // issues j = wave, wave + 8, ...  Lane l writes chunk position l % 8 of row 8j + l / 8 and
+  // therefore names the source chunk (l % 8) ^ swz16(row), with row % 16 = 8 (wave % 2) + l / 8.
+  // Rows past the end of the sequence (up to the end of its last 32-row tile) copy the last row.
+  {
+    const unsigned smem_base = lds_address(smem);
+    const int cp_row = lane / 8;
+    const unsigned cp_col = static_cast<unsigned>(((lane % 8) ^ tile_swz16(8 * (wave % 2) + cp_row)) * 16);
+    const unsigned qkv_pitch = static_cast<unsigned>(a.ld) * 2, do_pitch = static_cast<unsigned>(o_ld(a)) * 2;
+    const char* const src[4] = {reinterpret_cast<const char*>(q + qkv_at(a, b, 0, h)),
+                                reinterpret_cast<const char*>(k + qkv_at(a, b, 0, h)),
+                                reinterpret_cast<const char*>(v + qkv_at(a, b, 0, h)),
+                                reinterpret_cast<const char*>(d_o + o_at(a, b, h, 0))};
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int jj = 0; jj < kResidentS / 64; ++jj) {
+        const int j = wave + 8 * jj;
+        if (8 * j < n_tiles * 32) {
+          const int row = min(8 * j + cp_row, a.S - 1);
+          const unsigned off = row * (t == 3 ? do_pitch : qkv_pitch) + cp_col;
+          const unsigned dst = __builtin_amdgcn_readfirstlane(smem_base + t * kResidentTensor + j * 1024);
+          asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(src[t]) : "memory");
+        }
+      }
+  }
+  // ---- delta and the statistics: two threads per row, 32 columns each; O comes from global
+  // memory, dO from its LDS image once the copies have landed.  Stored negated, lse in log2
+  // units: they start the accumulators of the S and dP products.  Rows past the end carry
+  // -lse = -inf (their probabilities vanish) and delta = 0.
+  {
+    const int i = threadIdx.x / 2, part = threadIdx.x % 2;
+    const int ic = min(i, a.S - 1);
+    uint4 ow[4];
+    const T* orow = o + o_at(a, b, h, ic) + part * 32;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) ow[c] = *reinterpret_cast<const uint4*>(orow + 8 * c);
+    const float nl = i < a.S ? -lse[static_cast<int64_t>(bh) * a.S + i] * kAttnLog2e : -INFINITY;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies have landed
+    __syncthreads();
+    float dot = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      float x[8], y[8];
+      VecIO<T, 8>::load(reinterpret_cast<const T*>(&ow[c]), x);
+      VecIO<T, 8>::load(reinterpret_cast<const T*>(do_rows + tile16_chunk_at<DP>(i, part * 4 + c)), y);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dot = fmaf(x[e], y[e], dot);
+    }
+    dot += dpp_move<kDppQuadXor1>(dot);
+    if (part == 0) {
+      nlse_s[i] = nl;
+      ndelta_s[i] = i < a.S ? -dot : 0.f;
+    }
+  }
+  __syncthreads();
+
+  const TileLane16<DP> at(lane);
+  const float c = scale * kAttnLog2e;
+  if (wave >= n_tiles) return;  // no keys and no queries for this wave
+
+  // ---- pass 1: dK, dV of keys 32 wave .. 32 wave + 31
+  {
+    const int n_wave = wave * 32;
+    const int n = n_wave + lane % 32;
+    uint4 kf[KS], vf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      kf[ks] = scale_frag<T>(frag_rows<DP>(k_rows, at, wave, ks), c);
+      vf[ks] = frag_rows<DP>(v_rows, at, wave, ks);
+    }
+    floatx16 acc_k[DT], acc_v[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      acc_k[dt] = zero16();
+      acc_v[dt] = zero16();
+    }
+    for (int mt = CAUSAL ? wave : 0; mt < n_tiles; ++mt) {
+      const int m0 = mt * 32;
+      const bool plain = n_wave + 31 < a.S && (!CAUSAL || mt > wave);
+      floatx16 s, dp;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const float4 l4 = *reinterpret_cast<const float4*>(&nlse_s[m0 + g * 8 + half * 4]);
+        const float4 d4 = *reinterpret_cast<const float4*>(&ndelta_s[m0 + g * 8 + half * 4]);
+        s[g * 4 + 0] = l4.x; s[g * 4 + 1] = l4.y; s[g * 4 + 2] = l4.z; s[g * 4 + 3] = l4.w;
+        dp[g * 4 + 0] = d4.x; dp[g * 4 + 1] = d4.y; dp[g * 4 + 2] = d4.z; dp[g * 4 + 3] = d4.w;
+      }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        s = Mma<T>::run(frag_rows<DP>(q_rows, at, mt, ks), kf[ks], s);
+        dp = Mma<T>::run(frag_rows<DP>(do_rows, at, mt, ks), vf[ks], dp);
+      }
+      uint4 tq[2][DT], tdo[2][DT];
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          tdo[hf][dt] = frag_transposed<DP>(do_rows, at, dt, mt * 2 + hf);
+          tq[hf][dt] = frag_transposed<DP>(q_rows, at, dt, mt * 2 + hf);
+        }
+      __builtin_amdgcn_sched_barrier(0);
+      if (plain) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float p = fexp2(s[r]);
+          s[r] = p;
+          dp[r] = p * dp[r];
+        }
+      } else {
+        const bool col_ok = n < a.S;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          bool valid = col_ok;
+          if (CAUSAL) valid = valid && n <= m0 + acc_row(r, lane);
+          float p = fexp2(s[r]);  // rows past the end started from -inf: p = 0
+          p = valid ? p : 0.f;
+          s[r] = p;
+          dp[r] = p * dp[r];
+        }
+      }
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        const uint4 pf = frag_from_acc<T>(s, hf);
+        const uint4 dsf = frag_from_acc<T>(dp, hf);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          acc_v[dt] = Mma<T>::run(tdo[hf][dt], pf, acc_v[dt]);
+          acc_k[dt] = Mma<T>::run(tq[hf][dt], dsf, acc_k[dt]);
+        }
+      }
+    }
+    if (n < a.S) {
+      T* outk = dk + qkv_at(a, b, n, h);
+      T* outv = dv + qkv_at(a, b, n, h);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int d = dt * 32 + g * 8 + half * 4;
+          store4<T>(outk + d, acc_k[dt], g, scale);
+          store4<T>(outv + d, acc_v[dt], g, 1.0f);
+        }
+    }
+  }
+
+  // ---- pass 2: dQ of queries 32 wave .. 32 wave + 31
+  {
+    const int m_wave = wave * 32;
+    const int m = m_wave + lane % 32;
+    uint4 qf[KS], dof[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[ks] = scale_frag<T>(frag_rows<DP>(q_rows, at, wave, ks), c);
+      dof[ks] = frag_rows<DP>(do_rows, at, wave, ks);
+    }
+    const floatx16 s_init = splat16(nlse_s[m]), dp_init = splat16(ndelta_s[m]);
+    floatx16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
+    const int nt_end = CAUSAL ? wave + 1 : n_tiles;
+    for (int nt = 0; nt < nt_end; ++nt) {
+      const int nb = nt * 32;
+      floatx16 s = s_init, dp = dp_init;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        s = Mma<T>::run(frag_rows<DP>(k_rows, at, nt, ks), qf[ks], s);
+        dp = Mma<T>::run(frag_rows<DP>(v_rows, at, nt, ks), dof[ks], dp);
+      }
+      uint4 kt[2][DT];
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) kt[hf][dt] = frag_transposed<DP>(k_rows, at, dt, nt * 2 + hf);
+      __builtin_amdgcn_sched_barrier(0);
+      const bool plain = nb + 32 <= a.S && (!CAUSAL || nt < wave);
+      if (plain) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = fexp2(s[r]) * dp[r];
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int n = nb + acc_row(r, lane);
+          bool valid = n < a.S;
+          if (CAUSAL) valid = valid && n <= m;
+          float p = fexp2(s[r]);
+          p = valid ? p : 0.f;
+          s[r] = p * dp[r];  // dS^T
+        }
+      }
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        const uint4 dsf = frag_from_acc<T>(s, hf);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[dt] = Mma<T>::run(kt[hf][dt], dsf, acc[dt]);
+      }
+    }
+    if (m < a.S) {
+      T* out = dq + qkv_at(a, b, m, h);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) store4<T>(out + dt * 32 + g * 8 + half * 4, acc[dt], g, scale);
+    }
+  }
+}
+
 template <typename T, int DP, int MQ, bool CAUSAL, bool HAS_BIAS>
 __global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
                                                                        const T* __restrict__ k, const T* __restrict__ v,
@@ -1725,6 +1969,26 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
                      const float* lse, void* dq, void* dk, void* dv, AttnDims a, float scale, bool causal, bool has_bias,
                      hipStream_t stream) {
   const int64_t rows = static_cast<int64_t>(a.B) * a.H * a.S;
+  // Short sequences of 64-wide heads: one workgroup per (batch, head) with the whole head in
+  // LDS (attn_bwd_resident_kernel); no delta launch, no scratch.
+  if constexpr (DP == 64) {
+    if (a.D == 64 && a.S <= kResidentS && !has_bias && env_int("MOGRAD_HIP_ATTN_RESIDENT", 1) != 0 &&
+        static_cast<int64_t>(a.S) * a.ld * 2 < 0x7fffffffLL) {
+      const dim3 grid(static_cast<unsigned>(a.B * a.H));
+      if (causal)
+        hipLaunchKernelGGL((attn_bwd_resident_kernel<T, true>), grid, dim3(512), 0, stream, static_cast<const T*>(d_o),
+                           static_cast<const T*>(o), static_cast<const T*>(q), static_cast<const T*>(k),
+                           static_cast<const T*>(v), lse, static_cast<T*>(dq), static_cast<T*>(dk), static_cast<T*>(dv), a,
+                           scale);
+      else
+        hipLaunchKernelGGL((attn_bwd_resident_kernel<T, false>), grid, dim3(512), 0, stream, static_cast<const T*>(d_o),
+                           static_cast<const T*>(o), static_cast<const T*>(q), static_cast<const T*>(k),
+                           static_cast<const T*>(v), lse, static_cast<T*>(dq), static_cast<T*>(dk), static_cast<T*>(dv), a,
+                           scale);
+      MG_LAUNCH_CHECK();
+      return MG_OK;
+    }
+  }
   // The pipelined dK/dV walk (head dims up to 64, no bias) reads the row statistics negated
   // and padded per (batch, head) to a multiple of 64 rows; the delta kernel writes both forms.
   static const bool pipe_off = [] {

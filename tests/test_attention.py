@@ -129,6 +129,35 @@ def test_bf16_gradients_rtol(device, causal):
         assert np.all(np.abs(got - want) <= bound), f"{what}: worst {np.max(np.abs(got - want) / bound):.3g}"
 
 
+@pytest.mark.parametrize("dtype,rtol", [(F16, RTOL_BF16_ATTN / 8), (BF16, RTOL_BF16_ATTN)])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,S", [(3, 2, 256), (2, 3, 200), (1, 2, 33), (2, 2, 1), (4, 3, 128), (1, 1, 225)])
+def test_whole_head_in_lds_backward(device, monkeypatch, dtype, rtol, causal, B, H, S):
+    # Sequences up to 256 tokens of 64-wide heads: the backward keeps a (batch, head)'s Q, K, V
+    # and dO in LDS and computes delta itself, one workgroup per head
+    # (MOGRAD_HIP_ATTN_RESIDENT=0: the streaming walks).  Both against the oracle, at every
+    # length class: full tiles, a ragged last tile, fewer tiles than waves, a single token.
+    D = 64
+    q, k, v, do, _ = _inputs(57, B, S, H, D, dtype, False)
+    want = O.sdpa_bwd(q, k, v, do, None, causal)
+    results = {}
+    for mode in ("0", "1"):
+        monkeypatch.setenv("MOGRAD_HIP_ATTN_RESIDENT", mode)
+        results[mode] = _fwd_bwd(device, q, k, v, do, None, causal, dtype=dtype)[2:]
+        for got, ref, what in zip(results[mode], want, ("dq", "dk", "dv")):
+            # (a single token has dq = dk = 0 exactly; the kernels leave the rounding of dP - delta)
+            bound = rtol * (np.abs(ref) + max(np.abs(ref).max(), 1e-2))
+            assert np.all(np.isfinite(got)), what
+            assert np.all(np.abs(got - ref) <= bound), f"{what} ({mode}): worst {np.max(np.abs(got - ref) / bound):.3g}"
+    # the two paths round P and dS to 16 bits at the same points: they differ by summation order only
+    for a, b_, ref, what in zip(results["1"], results["0"], want, ("dq", "dk", "dv")):
+        assert np.max(np.abs(a - b_)) <= 0.5 * rtol * max(np.abs(ref).max(), 1e-2), what
+    # and the resident path is deterministic
+    again = _fwd_bwd(device, q, k, v, do, None, causal, dtype=dtype)[2:]
+    for a, b_ in zip(again, results["1"]):
+        np.testing.assert_array_equal(a, b_)
+
+
 def test_closed_forms(device):
     B, S, H, D = 1, 128, 1, 8
     z = np.zeros((B, S, H, D), np.float32)
