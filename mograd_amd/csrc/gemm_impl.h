@@ -964,13 +964,13 @@ __global__ __launch_bounds__(TM * 2, gemm16_pipe_occupancy(BK, NSTAGE, TM)) void
 // half-empty CUs (384 dX tiles on 256 CUs) and pay a launch apiece.  With
 // dw.colsum_part set, the dW workgroups of the first tile column also produce the bias
 // gradient's partial rows from the dY tiles they hold anyway.
-template <typename T>
-__global__ __launch_bounds__(256, gemm16_pipe_occupancy(32, 2, 128)) void linear_bwd_16bit_kernel(
+template <typename T, int NSTAGE = 2>
+__global__ __launch_bounds__(256, gemm16_pipe_occupancy(32, NSTAGE, 128)) void linear_bwd_16bit_kernel(
     Gemm16Problem<T> dw, Gemm16Problem<T> dx, int n_dw) {
-  __shared__ __attribute__((aligned(1024))) char lds[gemm16_pipe_lds_bytes(32, 2, 128)];
+  __shared__ __attribute__((aligned(1024))) char lds[gemm16_pipe_lds_bytes(32, NSTAGE, 128)];
   const int bid = blockIdx.x;
-  if (bid < n_dw) gemm16_pipe_block<T, false, false, false, true, 32, 2, 128>(lds, bid, dw);
-  else gemm16_pipe_block<T, true, false, false, false, 32, 2, 128>(lds, bid - n_dw, dx);
+  if (bid < n_dw) gemm16_pipe_block<T, false, false, false, true, 32, NSTAGE, 128>(lds, bid, dw);
+  else gemm16_pipe_block<T, true, false, false, false, 32, NSTAGE, 128>(lds, bid - n_dw, dx);
 }
 
 // ------------------------------------------------------------------------------------
