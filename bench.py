@@ -429,6 +429,8 @@ def bench_gpt(args, dev) -> dict:
     bias_f, gam, bet = rnd(ff, 8), rnd(d, 9), rnd(d, 10)
     out_d, out_ff, out_v, dlog = new(n * d), new(n * ff), new(n * V), new(n * V)
     dw_big, db_big, dgam, dbet = new(ff * d), new(ff), new(d), new(d)
+    big_ids = AnyBuffer.from_numpy(dev, _rng(5, 9).integers(0, 50304, 8192).astype(np.int32), I32)
+    big_table = new(50304 * 768)
     mean, rstd, lse, loss1 = new(n, F32), new(n, F32), new(B * H * T, F32), new(1)
     qkv, o, do, dqkv = rnd(3 * n * d, 11), new(n * d), rnd(n * d, 14), rnd(3 * n * d, 15)  # Q | K | V per token
     w_qkv = rnd(3 * d * d, 12)  # the stacked (3d, d) projection weight
@@ -485,6 +487,10 @@ def bench_gpt(args, dev) -> dict:
          n * d * e2 + n * 4, "B", None),
         ("scatter_add bf16 16384 rows into (65, 384)", lambda i: lib.mg_scatter_add(P(ids), P(dy_d), P(dw_big), n, V, d, I32, BF16, st),
          n * d * e2 + n * 4 + V * d * e2, "B", None),
+        ("scatter_add bf16 8192 rows of 768 into a (50304, 768) table (not in the step: a GPT-2-sized embedding gradient, "
+         "indices bucketed by row first)",
+         lambda i: lib.mg_scatter_add(P(big_ids), P(x_ff), P(big_table), 8192, 50304, 768, I32, BF16, st),
+         8192 * 768 * e2 + 8192 * 4 + 50304 * 768 * e2, "B", None),
         ("cast fp32 -> bf16 parameter arena", lambda i: lib.mg_cast(P(model.master), P(model.work), model.total, F32, BF16, st),
          model.total * 6, "B", None),
     ]

@@ -142,6 +142,50 @@ def test_scatter_add_vs_oracle(device, dtype, idx_dtype, V, d, n):
     assert not got[untouched].any()
 
 
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("idx_dtype", [I32, I64])
+@pytest.mark.parametrize("V,d,n", [(2048, 64, 3000), (5000, 72, 700), (1024, 5, 1)])
+def test_scatter_add_large_table_buckets(device, monkeypatch, dtype, idx_dtype, V, d, n):
+    # From a thousand rows on the indices are bucketed by destination row (a stable sort of
+    # (row, position) pairs) and a wave adds only its own row's run, in the same ascending
+    # position order as the scanning kernel: forcing either path gives the same bits.  Indices
+    # outside the table, repeated heavily and absent rows are all in the mix.
+    y = round_to_dtype(normal(70, 0, (n, d)), dtype)
+    idx = integers(70, 1, (n,), -3, V + 3, np.int32 if idx_dtype == I32 else np.int64)
+    idx[: n // 4] = idx[0] if 0 <= idx[0] < V else 7  # one heavy row
+    operands = [(idx, Layout(n), idx_dtype), (y, Layout(n, d), dtype)]
+    monkeypatch.setenv("MOGRAD_HIP_SCATTER_BUCKET_MIN_ROWS", "1")
+    got = _run(device, "SCATTER_ADD", Layout(V, d), operands, dtype)
+    keep = (idx >= 0) & (idx < V)
+    want = O.scatter_add(idx[keep], y[keep], V)
+    mass = O.scatter_add(idx[keep], np.abs(y[keep]), V)
+    eps = {F32: 0.0, F16: 2.0 ** -11, BF16: 2.0 ** -8}[dtype]
+    assert np.all(np.abs(got - want) <= RTOL_F32 * np.abs(want) + eps * np.abs(want) + 16 * 2.0 ** -24 * mass + 1e-30)
+    assert not got[np.setdiff1d(np.arange(V), idx[keep])].any()
+    if n <= 1024:  # one slab of the scanning kernel: the same order of additions
+        monkeypatch.setenv("MOGRAD_HIP_SCATTER_BUCKET_MIN_ROWS", "1000000000")
+        np.testing.assert_array_equal(got, _run(device, "SCATTER_ADD", Layout(V, d), operands, dtype))
+
+
+def test_scatter_add_vocabulary_sized_table(device):
+    # A GPT-2 embedding gradient: 8192 tokens into (50304, 768) bf16.  Histogram exactly, the
+    # adjoint identity with gather, untouched rows zero, two runs identical.
+    V, d, n = 50304, 768, 8192
+    idx = integers(71, 0, (n,), 0, V, np.int32)
+    idx[:512] = 11  # a frequent token
+    y = round_to_dtype(normal(71, 1, (n, d)), BF16)
+    operands = [(idx, Layout(n), I32), (y, Layout(n, d), BF16)]
+    got = _run(device, "SCATTER_ADD", Layout(V, d), operands, BF16)
+    np.testing.assert_array_equal(got, _run(device, "SCATTER_ADD", Layout(V, d), operands, BF16))
+    assert not got[np.setdiff1d(np.arange(V), idx)].any()
+    rows = np.unique(idx)[:200]
+    want = O.scatter_add(idx, y, V)[rows]
+    assert np.all(np.abs(got[rows] - want) <= 2.0 ** -8 * np.abs(want) + 1e-3)
+    ones = np.ones((n, 8), np.float32)
+    hist = _run(device, "SCATTER_ADD", Layout(V, 8), [(idx, Layout(n), I32), (ones, Layout(n, 8), F32)], F32)
+    np.testing.assert_array_equal(hist[:, 0], np.bincount(idx, minlength=V).astype(np.float32))
+
+
 def test_scatter_add_ignores_bad_indices_and_checks_rank(device):
     V, d, n = 5, 8, 6
     y = normal(67, 0, (n, d))
