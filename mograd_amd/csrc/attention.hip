@@ -1,6 +1,7 @@
 // C ABI for flash attention: argument checks, routing between the MFMA kernels (16-bit
 // storage, head dimension up to 128) and the general fp32-arithmetic kernels.
 #include "attention_generic.h"
+#include "attention_tiled.h"
 #include "mg_internal.h"
 
 namespace mg {
@@ -25,10 +26,60 @@ static int check_attn(const char* who, int64_t B, int64_t S, int64_t H, int64_t 
   return MG_OK;
 }
 
+// The row-per-thread kernels (attention_tiled.h) take head dimensions up to 128 once a sequence
+// has rows for a workgroup; MOGRAD_HIP_ATTN_TILED=0 keeps the wave-per-row kernels.
+static bool attn_tiled_ok(const AttnDims& a) {
+  return a.D <= 128 && a.S >= 64 && static_cast<int64_t>(a.B) * a.H <= 65535 && env_int("MOGRAD_HIP_ATTN_TILED", 1) != 0;
+}
+
+template <typename T, int NT, int DL>
+static void fwd_tiled_launch(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse,
+                             const AttnDims& a, float scale, bool causal, bool has_bias, hipStream_t stream) {
+  const dim3 grid(static_cast<unsigned>(ceil_div(a.S, 256 / NT)), static_cast<unsigned>(a.B * a.H));
+#define MG_FWD(C_, B_)                                                                                               \
+  hipLaunchKernelGGL((attn_fwd_tiled_kernel<T, NT, DL, C_, B_>), grid, dim3(256), 0, stream, static_cast<const T*>(q), \
+                     static_cast<const T*>(k), static_cast<const T*>(v), static_cast<const T*>(mask),                \
+                     static_cast<T*>(o), lse, a, scale)
+  if (causal) MG_FWD(true, false);
+  else if (has_bias) MG_FWD(false, true);
+  else MG_FWD(false, false);
+#undef MG_FWD
+}
+
+template <typename T, int NT, int DL, int NTK, int DLK>
+static void bwd_tiled_launch(const void* d_o, const void* q, const void* k, const void* v, const void* mask,
+                             const float* lse, const float* delta, void* dq, void* dk, void* dv, const AttnDims& a,
+                             float scale, bool causal, bool has_bias, hipStream_t stream) {
+  const dim3 grid_q(static_cast<unsigned>(ceil_div(a.S, 256 / NT)), static_cast<unsigned>(a.B * a.H));
+  const dim3 grid_k(static_cast<unsigned>(ceil_div(a.S, 256 / NTK)), static_cast<unsigned>(a.B * a.H));
+#define MG_BWD(C_, B_)                                                                                                \
+  do {                                                                                                                \
+    hipLaunchKernelGGL((attn_dq_tiled_kernel<T, NT, DL, C_, B_>), grid_q, dim3(256), 0, stream,                       \
+                       static_cast<const T*>(d_o), static_cast<const T*>(q), static_cast<const T*>(k),                \
+                       static_cast<const T*>(v), static_cast<const T*>(mask), lse, delta, static_cast<T*>(dq), a,     \
+                       scale);                                                                                        \
+    hipLaunchKernelGGL((attn_dkdv_tiled_kernel<T, NTK, DLK, C_, B_>), grid_k, dim3(256), 0, stream,                   \
+                       static_cast<const T*>(d_o), static_cast<const T*>(q), static_cast<const T*>(k),                \
+                       static_cast<const T*>(v), static_cast<const T*>(mask), lse, delta, static_cast<T*>(dk),        \
+                       static_cast<T*>(dv), a, scale);                                                                \
+  } while (0)
+  if (causal) MG_BWD(true, false);
+  else if (has_bias) MG_BWD(false, true);
+  else MG_BWD(false, false);
+#undef MG_BWD
+}
+
 template <typename T>
 static int fwd_generic(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, AttnDims a,
                        float scale, bool causal, bool has_bias, hipStream_t stream) {
   const int64_t rows = static_cast<int64_t>(a.B) * a.H * a.S;
+  if (attn_tiled_ok(a)) {
+    if (a.D <= 32) fwd_tiled_launch<T, 1, 32>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
+    else if (a.D <= 64) fwd_tiled_launch<T, 2, 32>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
+    else fwd_tiled_launch<T, 4, 32>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
+    MG_LAUNCH_CHECK();
+    return MG_OK;
+  }
   const dim3 grid(static_cast<unsigned>(ceil_div(rows, 4)));
 #define MG_FWD(C_, B_)                                                                                              \
   hipLaunchKernelGGL((attn_fwd_generic_kernel<T, C_, B_>), grid, dim3(256), 0, stream, static_cast<const T*>(q),    \
@@ -53,6 +104,14 @@ static int bwd_generic(const void* d_o, const void* o, const void* q, const void
   hipLaunchKernelGGL((attn_delta_kernel<T>), grid, dim3(256), 0, stream, static_cast<const T*>(d_o),
                      static_cast<const T*>(o), delta.as<float>(), rows, a.D, a.S, a.H, a.o_bshd);
   MG_LAUNCH_CHECK();
+  if (attn_tiled_ok(a)) {
+    const float* dl = delta.as<float>();
+    if (a.D <= 32) bwd_tiled_launch<T, 1, 32, 1, 32>(d_o, q, k, v, mask, lse, dl, dq, dk, dv, a, scale, causal, has_bias, stream);
+    else if (a.D <= 64) bwd_tiled_launch<T, 2, 32, 2, 32>(d_o, q, k, v, mask, lse, dl, dq, dk, dv, a, scale, causal, has_bias, stream);
+    else bwd_tiled_launch<T, 4, 32, 4, 32>(d_o, q, k, v, mask, lse, dl, dq, dk, dv, a, scale, causal, has_bias, stream);
+    MG_LAUNCH_CHECK();
+    return MG_OK;
+  }
 #define MG_BWD(C_, B_)                                                                                                \
   do {                                                                                                                \
     hipLaunchKernelGGL((attn_dq_generic_kernel<T, C_, B_>), grid, dim3(256), 0, stream, static_cast<const T*>(d_o),   \

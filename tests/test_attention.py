@@ -79,6 +79,24 @@ def test_f32_error_budget(device, name, causal, with_mask, D, budget):
     assert _max_err(dq, rdq) <= budget and _max_err(dk, rdk) <= budget and _max_err(dv, rdv) <= budget
 
 
+@pytest.mark.parametrize("name,causal,with_mask", MODES)
+@pytest.mark.parametrize("B,H,S,D,budget", [(1, 2, 300, 64, 5e-6), (2, 1, 100, 128, 1e-5), (1, 3, 64, 24, 5e-6),
+                                            (1, 1, 257, 72, 1e-5), (2, 2, 130, 32, 5e-6)])
+def test_f32_row_per_thread_and_wave_per_row_kernels(device, monkeypatch, name, causal, with_mask, B, H, S, D, budget):
+    # fp32 tensors with head dims up to 128 and at least 64 tokens take kernels that keep a row
+    # per thread (or per 2 / 4 neighbouring threads) and stage the other side through LDS;
+    # MOGRAD_HIP_ATTN_TILED=0 keeps a wave per row.  Both must meet the reference's fp32 budget
+    # against the f64 oracle, at sequence lengths that leave ragged tiles and idle threads.
+    q, k, v, do, m = _inputs(58, B, S, H, D, F32, with_mask)
+    ro, rl = O.sdpa_fwd(q, k, v, m, causal)
+    want = (ro, rl) + tuple(O.sdpa_bwd(q, k, v, do, m, causal))
+    for mode in ("0", "1"):
+        monkeypatch.setenv("MOGRAD_HIP_ATTN_TILED", mode)
+        got = _fwd_bwd(device, q, k, v, do, m, causal)
+        for g, w, what in zip(got, want, ("o", "lse", "dq", "dk", "dv")):
+            assert _max_err(g, w) <= budget, f"{what} (tiled={mode}): {_max_err(g, w)}"
+
+
 HALF_SHAPES = [(2, 2, 96, 64), (1, 3, 200, 64), (2, 1, 128, 128), (1, 2, 257, 32), (1, 1, 4, 8), (1, 2, 96, 256),
                (1, 2, 130, 72)]
 
