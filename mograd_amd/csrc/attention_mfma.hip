@@ -1890,7 +1890,7 @@ bool attn_mfma_supported(int dtype, int64_t D, const void* const* ptrs, int nptr
   if (D % 8 != 0 || D > 128) return false;  // rows are read 16 bytes at a time
   for (int i = 0; i < nptrs; ++i)
     if (ptrs[i] != nullptr && !aligned16(ptrs[i])) return false;
-  const char* force = std::getenv("MOGRAD_HIP_ATTN_GENERIC");
+  const char* force = env_str("MOGRAD_HIP_ATTN_GENERIC");
   if (force && force[0] == '1') return false;
   return true;
 }
@@ -1992,7 +1992,7 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
   // The pipelined dK/dV walk (head dims up to 64, no bias) reads the row statistics negated
   // and padded per (batch, head) to a multiple of 64 rows; the delta kernel writes both forms.
   static const bool pipe_off = [] {
-    const char* e = std::getenv("MOGRAD_HIP_ATTN_DKDV_PIPE");
+    const char* e = env_str("MOGRAD_HIP_ATTN_DKDV_PIPE");
     return e && e[0] == '0';
   }();
   const bool pipe = DP <= 64 && !has_bias && !pipe_off;
@@ -2014,7 +2014,7 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
   // instead of filling each other's gaps).  MOGRAD_HIP_ATTN_FUSED_BWD_MAX_S overrides it; 0
   // always launches dK/dV and dQ separately.
   static const int fused_max_s = [] {
-    const char* e = std::getenv("MOGRAD_HIP_ATTN_FUSED_BWD_MAX_S");
+    const char* e = env_str("MOGRAD_HIP_ATTN_FUSED_BWD_MAX_S");
     return e && e[0] ? std::atoi(e) : 1024;
   }();
   const bool fused = DP <= 64 && a.S <= fused_max_s && 2 * (blocks + 7) < 0x7fffffffLL;

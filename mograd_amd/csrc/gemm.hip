@@ -355,7 +355,7 @@ static int linear_bwd_one_launch(const void* dy, const void* x, const void* w, v
   *done = false;
   if (db_done) *db_done = false;
   if (dw_rows < 0) dw_rows = N;  // rows of dW to write: fewer than N when dY and W came zero-padded
-  if (env_int("MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH", 1) == 0 || std::getenv("MOGRAD_HIP_GEMM16_PIPE")) return MG_OK;
+  if (env_int("MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH", 1) == 0 || env_str("MOGRAD_HIP_GEMM16_PIPE")) return MG_OK;
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return MG_OK;
   if (M % kG16BK || N % kG16BK || !mult8(K)) return MG_OK;
   if (!aligned16(dy) || !aligned16(x) || !aligned16(w) || !aligned16(dx) || !aligned16(dw)) return MG_OK;
@@ -451,7 +451,7 @@ static int linear_bwd_padded(const void* dy, const void* x, const void* w, void*
   *done = false;
   const int64_t n_to = ceil_div(N, kG16BK) * kG16BK;
   if (N % kG16BK == 0 || n_to > 2 * N || M % kG16BK || !mult8(K) || M < 1024 || n_to * K > 0x7fffffffLL) return MG_OK;
-  if (env_int("MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH", 1) == 0 || std::getenv("MOGRAD_HIP_GEMM16_PIPE")) return MG_OK;
+  if (env_int("MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH", 1) == 0 || env_str("MOGRAD_HIP_GEMM16_PIPE")) return MG_OK;
   Scratch dy_pad, w_pad;
   MG_TRY(dy_pad.take(M * n_to * static_cast<int64_t>(sizeof(T))));
   MG_TRY(w_pad.take(n_to * K * static_cast<int64_t>(sizeof(T))));

@@ -87,11 +87,27 @@ inline const char* dtype_name(int dtype) {
   }
 }
 
-// Integer tuning knob from the environment (read on every call; used by benchmarks to
-// compare kernel layouts without rebuilding).
-inline int env_int(const char* name, int fallback) {
+// The MOGRAD_HIP_* tuning knobs (kernel layout choices that benchmarks and equivalence tests
+// flip without rebuilding) are honoured only in a process that sets MOGRAD_HIP_TUNING=1, so
+// that the library's behaviour in a host application does not depend on stray variables of
+// its environment.  Read once.
+inline bool tuning_enabled() {
+  static const bool on = [] {
+    const char* v = std::getenv("MOGRAD_HIP_TUNING");
+    return v && v[0] == '1';
+  }();
+  return on;
+}
+// A tuning knob's raw value, or null when unset or when tuning is off.
+inline const char* env_str(const char* name) {
+  if (!tuning_enabled()) return nullptr;
   const char* v = std::getenv(name);
-  return (v && *v) ? std::atoi(v) : fallback;
+  return (v && *v) ? v : nullptr;
+}
+// Integer tuning knob (looked up on every call).
+inline int env_int(const char* name, int fallback) {
+  const char* v = env_str(name);
+  return v ? std::atoi(v) : fallback;
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
