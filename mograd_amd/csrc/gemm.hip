@@ -207,24 +207,25 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
     return MG_OK;
   }
   const int k_per_split = splitk_16bit_range(g.K, &splits);
-  // The batches of C are contiguous ((batch, M, N) row-major), so partials and the reduction
-  // treat them as one array of batch * M * N elements.
+  // Partial tiles: whole 128 x 128 tiles in accumulator order (gemm16_partial_floats); the
+  // reduction maps them back onto the contiguous (batch, M, N) output.
   Scratch partial;
-  const int64_t numel = g.batch * g.M * g.N;
-  MG_TRY(partial.take(static_cast<int64_t>(splits) * numel * static_cast<int64_t>(sizeof(float))));
+  const int64_t slice = gemm16_partial_floats(g.M, g.N, g.batch, 1);
+  MG_TRY(partial.take(static_cast<int64_t>(splits) * slice * static_cast<int64_t>(sizeof(float))));
   const int64_t split_grid = gemm_split_grid(tiles, splits, g.batch);
   if (split_grid > 0x7fffffffLL) return fail(MG_ERR_INVALID, "matmul: too many output tiles");
   const dim3 grid(static_cast<unsigned>(split_grid));
   MG_GEMM16_LAUNCH(false, true, grid, partial.as<float>(), k_per_split, splits, (GemmEpilogue<T>{nullptr, nullptr, 0}));
 #undef MG_GEMM16_LAUNCH
   MG_LAUNCH_CHECK();
-  const unsigned rblocks = static_cast<unsigned>(ceil_div(numel, 256));
+  if (slice / 256 > 0x7fffffffLL) return fail(MG_ERR_INVALID, "matmul: too many output tiles");
+  const unsigned rblocks = static_cast<unsigned>(slice / 256);
   if (bias)
-    hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, true>), dim3(rblocks), dim3(256), 0, stream, partial.as<float>(),
-                       bias, c, numel, numel, splits, N, epilogue_of<T>(g));
+    hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, true, true>), dim3(rblocks), dim3(256), 0, stream,
+                       partial.as<float>(), bias, c, slice, slice, splits, N, epilogue_of<T>(g), M, tiles_n);
   else
-    hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, false>), dim3(rblocks), dim3(256), 0, stream, partial.as<float>(),
-                       bias, c, numel, numel, splits, N, epilogue_of<T>(g));
+    hipLaunchKernelGGL((gemm_splitk_reduce_kernel<T, false, true>), dim3(rblocks), dim3(256), 0, stream,
+                       partial.as<float>(), bias, c, slice, slice, splits, N, epilogue_of<T>(g), M, tiles_n);
   MG_LAUNCH_CHECK();
   return MG_OK;
 }
@@ -361,25 +362,47 @@ static int linear_bwd_one_launch(const void* dy, const void* x, const void* w, v
   if (!aligned16(dy) || !aligned16(x) || !aligned16(w) || !aligned16(dx) || !aligned16(dw)) return MG_OK;
   if (M * K < 64 * 64 || N * K < 64 * 64) return MG_OK;
   const int64_t cus = device_info().cu_count;
-  const int tiles_kk = static_cast<int>(ceil_div(K, kGemmBN));
+  // Input widths that are multiples of 384 take 128 x 384 output tiles (twelve waves, one
+  // workgroup per CU): the three column tiles of a row block share one copy of the dY tile,
+  // a third fewer bytes from L2 per FLOP.  MOGRAD_HIP_LINEAR_BWD_WIDE=0: 128 x 128 tiles.
+  // Taken when those tiles leave CUs free for dW's K ranges, so that the whole launch is one
+  // workgroup per CU, and the layer is wide enough to pay for the larger partial tiles.
+  const bool wide = K % kGemmWideBN == 0 && ceil_div(M, kGemmBM) * (K / kGemmWideBN) < cus && N >= 768 &&
+                    env_int("MOGRAD_HIP_LINEAR_BWD_WIDE", 1) != 0;
+  const int tiles_kk = static_cast<int>(ceil_div(K, wide ? kGemmWideBN : kGemmBN));
   // dW: must be split, each workgroup's rows short enough for the 32-k variant.
   const int w_tiles_m = static_cast<int>(ceil_div(N, kGemmBM));
   const int64_t w_tiles = static_cast<int64_t>(w_tiles_m) * tiles_kk;
-  // One workgroup per CU is enough here: the dX tiles fill the rest of the device, and half
-  // the K ranges are half the partial tiles to write and sum (GPT step 3.06 -> 3.00 ms).
-  int splits = splitk_16bit_splits(w_tiles, M, env_int("MOGRAD_HIP_LINEAR_BWD_SPLIT_WG_PER_CU", 1));
-  if (splits <= 1 || ceil_div(M, splits) >= 4096) return MG_OK;
-  const int k_per_split = splitk_16bit_range(M, &splits);
-  // dX: the 32-k variant with 128 x 128 tiles.
   const int x_tiles_m = static_cast<int>(ceil_div(M, kGemmBM));
   const int64_t x_tiles = static_cast<int64_t>(x_tiles_m) * tiles_kk;
+  int splits;
+  if (wide) {
+    // Every workgroup step is the same work (a 128 x 384 x 32 product), so the K ranges of dW
+    // are cut to what a CU's share of all steps comes to: with fewer dX tiles than CUs the
+    // ranges take the CUs that the tiles leave free, all in one round; otherwise the ranges
+    // start first and the tiles fill in behind them.
+    const int64_t steps_w = M / kG16BK, steps_x = N / kG16BK;
+    const int64_t share = ceil_div(x_tiles * steps_x + w_tiles * steps_w, cus);
+    int64_t want = x_tiles < cus ? (cus - x_tiles) / w_tiles : 0;
+    if (want < 2) want = ceil_div(steps_w, share);
+    const int64_t most = std::min<int64_t>(64, M / 256);
+    splits = static_cast<int>(std::max<int64_t>(1, std::min(want, most)));
+  } else {
+    // One workgroup per CU is enough here: the dX tiles fill the rest of the device, and half
+    // the K ranges are half the partial tiles to write and sum (GPT step 3.06 -> 3.00 ms).
+    splits = splitk_16bit_splits(w_tiles, M, env_int("MOGRAD_HIP_LINEAR_BWD_SPLIT_WG_PER_CU", 1));
+  }
+  if (splits <= 1 || ceil_div(M, splits) >= 4096) return MG_OK;
+  const int k_per_split = splitk_16bit_range(M, &splits);
+  // dX: the 32-k variant.
   if (N >= 4096 || (N >= 1024 && ceil_div(M, 256) * tiles_kk >= 2 * cus)) return MG_OK;
   const int64_t n_dw = gemm_split_grid(w_tiles, splits, 1);
   if (n_dw + x_tiles > 0x7fffffffLL) return MG_OK;
 
   Scratch partial;
   const int64_t numel = N * K;
-  MG_TRY(partial.take(static_cast<int64_t>(splits) * numel * static_cast<int64_t>(sizeof(float))));
+  const int64_t slice = gemm16_partial_floats(N, K, 1, 1);  // whole tiles per K range
+  MG_TRY(partial.take(static_cast<int64_t>(splits) * slice * static_cast<int64_t>(sizeof(float))));
   const T* dyt = static_cast<const T*>(dy);
   const Gemm16Problem<T> pw{dyt, static_cast<const T*>(x), nullptr, static_cast<T*>(dw), partial.as<float>(),
                             static_cast<int>(N), static_cast<int>(K), static_cast<int>(M),
@@ -405,18 +428,25 @@ static int linear_bwd_one_launch(const void* dy, const void* x, const void* w, v
   // Three copies of the tiles (two k-steps in flight per workgroup, three workgroups per CU)
   // measured 1 % faster on the GPT step than two copies and four workgroups; four copies no
   // better than two.  MOGRAD_HIP_LINEAR_BWD_STAGES=2 selects two.
-  if (env_int("MOGRAD_HIP_LINEAR_BWD_STAGES", 3) == 2)
+  if (wide && env_int("MOGRAD_HIP_LINEAR_BWD_STAGES", 2) == 3)  // 32 k per step, three copies: 3-4 % slower
+    hipLaunchKernelGGL((linear_bwd_16bit_kernel<T, 3, kGemmWideBN>), dim3(static_cast<unsigned>(n_dw + x_tiles)),
+                       dim3(2 * kGemmWideBN), 0, stream, pw2, px, static_cast<int>(n_dw));
+  else if (wide)  // 64 k per step, two copies (128 KB of LDS): half the barriers, whole cache lines of dY
+    hipLaunchKernelGGL((linear_bwd_16bit_kernel<T, 2, kGemmWideBN, 64>), dim3(static_cast<unsigned>(n_dw + x_tiles)),
+                       dim3(2 * kGemmWideBN), 0, stream, pw2, px, static_cast<int>(n_dw));
+  else if (env_int("MOGRAD_HIP_LINEAR_BWD_STAGES", 3) == 2)
     hipLaunchKernelGGL((linear_bwd_16bit_kernel<T, 2>), dim3(static_cast<unsigned>(n_dw + x_tiles)), dim3(kGemmThreads), 0,
                        stream, pw2, px, static_cast<int>(n_dw));
   else
     hipLaunchKernelGGL((linear_bwd_16bit_kernel<T, 3>), dim3(static_cast<unsigned>(n_dw + x_tiles)), dim3(kGemmThreads), 0,
                        stream, pw2, px, static_cast<int>(n_dw));
   MG_LAUNCH_CHECK();
-  const int dw_blocks = static_cast<int>(ceil_div(dw_rows * K, 256));
+  const int dw_blocks = static_cast<int>(slice / 256);
   const int db_blocks = groups > 0 ? static_cast<int>(ceil_div(N, 64)) : 0;
   hipLaunchKernelGGL((linear_bwd_finish_kernel<T>), dim3(static_cast<unsigned>(dw_blocks + db_blocks)), dim3(256), 0,
-                     stream, partial.as<float>(), static_cast<T*>(dw), dw_rows * K, numel, splits, static_cast<int>(K),
-                     dw_blocks, db_part.as<float>(), static_cast<T*>(db), groups, static_cast<int>(N));
+                     stream, partial.as<float>(), static_cast<T*>(dw), static_cast<int>(dw_rows), slice, splits,
+                     static_cast<int>(K), dw_blocks, db_part.as<float>(), static_cast<T*>(db), groups,
+                     static_cast<int>(N));
   MG_LAUNCH_CHECK();
   if (db_done) *db_done = groups > 0;
   *done = true;
@@ -572,3 +602,15 @@ int mg_linear_bwd_fused(const void* dy, const void* x, const void* w, void* dx, 
 }
 
 }  // extern "C"
+
+#ifdef MG_TIMELINE
+namespace mg { __device__ long long mg_timeline[16384 * 8]; }
+extern "C" int mg_debug_timeline(void* out, long long count, int clear) {
+  if (clear) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(mg::mg_timeline)) != hipSuccess) return 1;
+    return hipMemset(p, 0, sizeof(long long) * 16384 * 8) == hipSuccess ? 0 : 1;
+  }
+  return hipMemcpyFromSymbol(out, HIP_SYMBOL(mg::mg_timeline), sizeof(long long) * count) == hipSuccess ? 0 : 1;
+}
+#endif

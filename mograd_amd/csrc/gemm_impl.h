@@ -49,23 +49,29 @@ __device__ __forceinline__ void gemm_tile_of_block(int bid, int tiles_m, int til
   tn = in_band / rows_here;
 }
 
-// Split-K launches use one grid axis of kXcd * ceil(groups / kXcd) * tiles workgroups, a group
-// being one (batch, K range).  All output tiles of a group read the same K range of both
-// operands, so a group's workgroups are given ids of one residue mod kXcd: they run on one
-// XCD and the range is fetched into one L2 instead of all eight (the dW of a 384 -> 1536
-// layer over 16384 rows fetched 240 MB for 63 MB of operands with tiles dealt out round
-// robin).  Returns false for the padding workgroups of the last, partial round of groups.
+// Split-K launches use one grid axis.  The work items, one per (batch, K range, output tile),
+// are numbered with the tile varying fastest, and XCD x (the workgroups whose id is x mod kXcd)
+// takes the contiguous block [x n / kXcd, (x + 1) n / kXcd) of the n items: every XCD gets the
+// same number of items to within one (dealing out whole K ranges left two XCDs with twice the
+// work of the others whenever the ranges were no multiple of eight), and an XCD's items are
+// mostly whole K ranges, whose tiles read the same rows of both operands, so a range is fetched
+// into one or two L2s instead of all eight (the dW of a 384 -> 1536 layer over 16384 rows
+// fetched 240 MB for 63 MB of operands with tiles dealt out round robin).  Returns false for
+// the few padding workgroups at the end of the shorter blocks.
 __device__ __forceinline__ bool gemm_split_work(int bid, int tiles, int splits, int batches, int& tile, int& split,
                                                 int& batch) {
-  const int j = bid / kXcd;
-  const int group = (j / tiles) * kXcd + bid % kXcd;
-  tile = j % tiles;
+  const int64_t n = static_cast<int64_t>(tiles) * splits * batches;
+  const int x = bid % kXcd;
+  const int64_t item = x * n / kXcd + bid / kXcd;
+  if (item >= (x + 1) * n / kXcd) return false;
+  const int group = static_cast<int>(item / tiles);
+  tile = static_cast<int>(item % tiles);
   split = group % splits;
   batch = group / splits;
-  return group < splits * batches;
+  return true;
 }
 inline int64_t gemm_split_grid(int64_t tiles, int64_t splits, int64_t batches) {
-  return kXcd * ((splits * batches + kXcd - 1) / kXcd) * tiles;
+  return kXcd * ((tiles * splits * batches + kXcd - 1) / kXcd);
 }
 
 // What happens to a product element after the bias: v = acc + bias; relu: v = max(v, 0);
@@ -362,6 +368,17 @@ struct GemmMma16<f16_t> {
 
 constexpr int kG16BK = 64;
 constexpr int kG16Stride = kG16BK + 8;  // elements per LDS row: 144 bytes, 16-byte aligned, bank-spreading
+// fp32 partial tiles of a product split along K: [K range][batch][tile_m][tile_n] tiles of
+// 128 x 128 values, each stored as its four waves' accumulators,
+//   [wave][ti][tj][g][lane][j]  =  row (wave / 2) * 64 + ti * 32 + g * 8 + (lane / 32) * 4 + j,
+//                                  column (wave % 2) * 64 + tj * 32 + lane % 32
+// of the tile.  Tiles are stored whole; rows and columns past the matrix hold whatever the
+// clamped operand rows produced and are dropped by the reduction.
+constexpr int kG16PartialTile = kGemmBM * kGemmBN;
+constexpr int kGemmWideBN = 384;  // columns of the wide tile of linear_bwd_16bit_kernel
+inline int64_t gemm16_partial_floats(int64_t M, int64_t N, int64_t batches, int64_t splits) {
+  return splits * batches * ((M + kGemmBM - 1) / kGemmBM) * ((N + kGemmBN - 1) / kGemmBN) * kG16PartialTile;
+}
 
 struct Gemm16Stage {
   uint4 v[4];
@@ -483,7 +500,26 @@ __device__ __forceinline__ void gemm16_write_tile(const floatx16 (&acc)[2][2], u
                                                   float* __restrict__ partial, int M, int N, int64_t ldc, int64_t bsc,
                                                   int batch, int split, int batches, int m0, int n0, int wm, int wn,
                                                   int lane, const GemmEpilogue<T>& ep) {
-  if constexpr (!SPLIT_K) {
+  if constexpr (SPLIT_K) {
+    // A K range's partial tile goes out as the accumulators lie in the registers: sixteen
+    // unguarded 16-byte stores per thread, each a contiguous kilobyte of the wave
+    // (see gemm16_partial_floats for the layout; gemm_splitk_reduce_block undoes it).
+    const int tiles_n = (N + kGemmBN - 1) / kGemmBN, tiles_m = (M + kGemmBM - 1) / kGemmBM;
+    const int col0 = n0 + wn;  // a multiple of 64; the workgroup's tile may span several partial tiles
+    const int64_t tile_at = (static_cast<int64_t>(split) * batches + batch) * tiles_m * tiles_n +
+                            static_cast<int64_t>(m0 / kGemmBM) * tiles_n + col0 / kGemmBN;
+    float4* dst = reinterpret_cast<float4*>(partial) + tile_at * (kG16PartialTile / 4) +
+                  ((wm / 64) * 2 + (col0 / 64) % 2) * 1024 + lane;
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+      for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          dst[((ti * 2 + tj) * 4 + g) * 64] = make_float4(acc[ti][tj][4 * g], acc[ti][tj][4 * g + 1],
+                                                          acc[ti][tj][4 * g + 2], acc[ti][tj][4 * g + 3]);
+    return;
+  } else {
     const bool wide_out = (N % 8 == 0) && (ldc % 8 == 0) && (bsc % 8 == 0) && (reinterpret_cast<uintptr_t>(C) % 16 == 0);
     if (wide_out) {
       // An accumulator holds one column and, per group of four registers, four consecutive
@@ -575,17 +611,13 @@ __device__ __forceinline__ void gemm16_write_tile(const floatx16 (&acc)[2][2], u
     for (int tj = 0; tj < 2; ++tj) {
       const int col = n0 + wn + tj * 32 + lane % 32;
       if (col >= N) continue;
-      const float bv = (HAS_BIAS && !SPLIT_K) ? to_float(bias[col]) : 0.f;
+      const float bv = HAS_BIAS ? to_float(bias[col]) : 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm + ti * 32 + (r / 4) * 8 + (lane / 32) * 4 + (r % 4);
         if (row < M) {
-          if constexpr (SPLIT_K)
-            partial[((static_cast<int64_t>(split) * batches + batch) * M + row) * N + col] = acc[ti][tj][r];
-          else {
-            const int64_t at = batch * bsc + static_cast<int64_t>(row) * ldc + col;
-            C[at] = gemm_finish<T>(acc[ti][tj][r] + bv, ep, at);
-          }
+          const int64_t at = batch * bsc + static_cast<int64_t>(row) * ldc + col;
+          C[at] = gemm_finish<T>(acc[ti][tj][r] + bv, ep, at);
         }
       }
     }
@@ -694,13 +726,23 @@ typedef short gemm_i16x4 __attribute__((ext_vector_type(4)));
 // backward kernel were conflict cycles.)
 __device__ __forceinline__ constexpr int gemm16_tr_swizzle(int kk) { return 4 * (kk % 4) ^ 2 * ((kk / 8) % 2); }
 
-// Copy requests per thread, k-step and operand of ROWS rows, for a workgroup of NW waves.
-constexpr int gemm16_pipe_requests(int rows, int bk, int nw) { return rows * bk * 2 / 16 / (nw * 64); }
+// Copying one k-step of an operand of ROWS rows in a workgroup of NW waves: the waves that
+// take part (all of them, unless the step has fewer kilobytes than the workgroup has waves)
+// and the 16-byte requests of each of their threads.
+constexpr int gemm16_pipe_waves(int rows, int bk, int nw) {
+  const int kb = rows * bk * 2 / 1024;
+  int w = kb < nw ? kb : nw;
+  while (kb % w) --w;  // every taking wave the same number of kilobytes
+  return w;
+}
+constexpr int gemm16_pipe_requests(int rows, int bk, int nw) {
+  return rows * bk * 2 / 16 / (gemm16_pipe_waves(rows, bk, nw) * 64);
+}
 
 // The 16-byte source chunks this thread names for every k-step of one operand of ROWS rows,
 // as element offsets from the operand's (batch, k_begin) origin; they advance by BK
 // (k-contiguous) or BK * ld per step.
-template <bool KC, int BK, int ROWS, int NW>
+template <bool KC, int BK, int ROWS, int NW>  // NW: the waves that take part in this operand's copy
 __device__ __forceinline__ void gemm16_pipe_sources(int64_t ld, int o0, int O,
                                                     int64_t (&src)[gemm16_pipe_requests(ROWS, BK, NW)]) {
   constexpr int CPR = BK / 8;     // chunks per k-contiguous row
@@ -766,14 +808,14 @@ __device__ __forceinline__ uint4 gemm16_pipe_frag(const char* __restrict__ lds_s
 
 // LDS of the pipelined kernel (TM = rows of the A tile: 128 with four waves, 256 with eight) and
 // the workgroups that fit a CU, by LDS (160 KB) and by the register file.
-constexpr int gemm16_pipe_lds_bytes(int bk, int nstage, int tm) {
-  const int stages = nstage * (tm + 128) * bk * 2;
-  const int out = (tm / 32) * 64 * kG16Stride * 2;  // every wave transposes its output tile here
+constexpr int gemm16_pipe_lds_bytes(int bk, int nstage, int tm, int tn = 128) {
+  const int stages = nstage * (tm + tn) * bk * 2;
+  const int out = (tm / 64) * (tn / 64) * 64 * kG16Stride * 2;  // every wave transposes its output tile here
   return stages > out ? stages : out;
 }
-constexpr int gemm16_pipe_occupancy(int bk, int nstage, int tm) {
-  const int by_lds = 160 * 1024 / gemm16_pipe_lds_bytes(bk, nstage, tm);
-  const int by_regs = tm == 128 ? 4 : 2;
+constexpr int gemm16_pipe_occupancy(int bk, int nstage, int tm, int tn = 128) {
+  const int by_lds = 160 * 1024 / gemm16_pipe_lds_bytes(bk, nstage, tm, tn);
+  const int by_regs = 16 / ((tm / 64) * (tn / 64));  // four waves per SIMD at most
   return by_lds < 1 ? 1 : (by_lds > by_regs ? by_regs : by_lds);
 }
 
@@ -795,15 +837,23 @@ struct Gemm16Problem {
   float* colsum_part = nullptr;
 };
 
+#ifdef MG_TIMELINE
+extern __device__ long long mg_timeline[16384 * 8];
+#endif
 // The work of workgroup `bid` of a launch for one product; `lds` is the workgroup's
-// gemm16_pipe_lds_bytes(BK, NSTAGE, TM) bytes, aligned to 1024.
-template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, int BK, int NSTAGE, int TM = 128>
+// gemm16_pipe_lds_bytes(BK, NSTAGE, TM, TN) bytes, aligned to 1024.  The output tile is
+// TM x TN, (TM / 64) x (TN / 64) waves with 64 x 64 each; pr.tiles_n counts tiles of TN columns.
+template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, int BK, int NSTAGE, int TM = 128,
+          int TN = kGemmBN>
 __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm16Problem<T>& pr) {
   static_assert(NSTAGE >= 2 && NSTAGE <= 4 && (BK == 32 || BK == 64) && (TM == 128 || TM == 256), "stages");
-  constexpr int NW = TM / 32;                                 // waves: (TM / 64) x 2 wave tiles of 64 x 64
+  static_assert(TN % 128 == 0 && (!SPLIT_K || TM == 128), "partial tiles are 128 x 128");
+  constexpr int WN = TN / 64;                                 // waves side by side
+  constexpr int NW = (TM / 64) * WN;
+  constexpr int NWA = gemm16_pipe_waves(TM, BK, NW), NWB = gemm16_pipe_waves(TN, BK, NW);  // waves that copy A, B
   constexpr int NIA = gemm16_pipe_requests(TM, BK, NW);       // copy requests per thread and step
-  constexpr int NIB = gemm16_pipe_requests(kGemmBN, BK, NW);
-  constexpr int OPA = TM * BK * 2, OPB = kGemmBN * BK * 2;    // bytes of an operand's step
+  constexpr int NIB = gemm16_pipe_requests(TN, BK, NW);
+  constexpr int OPA = TM * BK * 2, OPB = TN * BK * 2;         // bytes of an operand's step
   constexpr int OP = OPA + OPB;
   const T* __restrict__ A = pr.A;
   const T* __restrict__ B = pr.B;
@@ -817,6 +867,10 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
   const GemmEpilogue<T> ep = pr.ep;
 
   const int tiles = tiles_m * tiles_n;
+#ifdef MG_TIMELINE
+  const long long tl_entry = wall_clock64();
+  long long tl_wait = 0, tl_first = 0;
+#endif
   int batch = bid / tiles, tile = bid % tiles, split = 0;
   if constexpr (SPLIT_K) {
     if (!gemm_split_work(bid, tiles, splits, batches, tile, split, batch)) return;
@@ -824,7 +878,7 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
   int tm, tn;
   gemm_tile_of_block(tile, tiles_m, tiles_n, tm, tn, !SPLIT_K);
   const int m0 = tm * TM;
-  const int n0 = tn * kGemmBN;
+  const int n0 = tn * TN;
   const int k_begin = SPLIT_K ? split * k_per_split : 0;
   const int k_end = SPLIT_K ? min(K, k_begin + k_per_split) : K;
   const int steps = (k_end - k_begin) / BK;
@@ -835,8 +889,11 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
 
   const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
-  const int wm = (wave / 2) * 64;
-  const int wn = (wave % 2) * 64;
+  const int wm = (wave / WN) * 64;
+  const int wn = (wave % WN) * 64;
+  // Waves that copy fewer requests per step have fewer outstanding at the waits below.
+  const bool copies_a = NWA == NW || wave < NWA, copies_b = NWB == NW || wave < NWB;
+  const int per_step = (copies_a ? NIA : 0) + (copies_b ? NIB : 0);
 
   floatx16 acc[2][2];
 #pragma unroll
@@ -846,10 +903,11 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // Column sums of the A tiles (see Gemm16Problem::colsum_part): a thread takes one 16-byte
-  // chunk (8 of the tile's 128 m) of every 16th k-row.
+  // Column sums of the A tiles (see Gemm16Problem::colsum_part): a thread of the first four
+  // waves takes one 16-byte chunk (8 of the tile's 128 m) of every 16th k-row.
   constexpr bool CAN_COLSUM = SPLIT_K && !A_KC && TM == 128;
   const bool colsum = CAN_COLSUM && pr.colsum_part != nullptr && tn == 0;
+  const bool cs_thread = threadIdx.x < 256;
   const int cs_chunk = threadIdx.x % 16, cs_row = threadIdx.x / 16;
   float cs_acc[8];
 #pragma unroll
@@ -858,33 +916,44 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
   const uint16_t* a16 = reinterpret_cast<const uint16_t*>(A);
   const uint16_t* b16 = reinterpret_cast<const uint16_t*>(B);
   int64_t src_a[NIA], src_b[NIB];
-  gemm16_pipe_sources<A_KC, BK, TM, NW>(lda, m0, M, src_a);
-  gemm16_pipe_sources<B_KC, BK, kGemmBN, NW>(ldb, n0, N, src_b);
+  gemm16_pipe_sources<A_KC, BK, TM, NWA>(lda, m0, M, src_a);
+  gemm16_pipe_sources<B_KC, BK, TN, NWB>(ldb, n0, N, src_b);
+  auto request = [&](int step, int copy) {
+    if (copies_a) gemm16_pipe_issue<NIA, NWA>(a16 + step * a_step, src_a, lds + copy * OP);
+    if (copies_b) gemm16_pipe_issue<NIB, NWB>(b16 + step * b_step, src_b, lds + copy * OP + OPA);
+  };
 
   // Steps 0 .. NSTAGE-2 are requested up front; iteration `it` then waits for step `it`
   // (its own NIA + NIB requests; the barrier covers the other waves'), requests step
   // it + NSTAGE - 1 into the copy that step it - 1 was just multiplied from, and multiplies.
 #pragma unroll
   for (int s = 0; s < NSTAGE - 1; ++s)
-    if (s < steps) {
-      gemm16_pipe_issue<NIA, NW>(a16 + s * a_step, src_a, lds + s * OP);
-      gemm16_pipe_issue<NIB, NW>(b16 + s * b_step, src_b, lds + s * OP + OPA);
-    }
+    if (s < steps) request(s, s);
+#ifdef MG_TIMELINE
+  const long long tl_pro = wall_clock64();
+#endif
   int cur = 0, nxt = NSTAGE - 1;
   for (int it = 0; it < steps; ++it) {
-    if (it + NSTAGE - 2 < steps) MG_WAIT_VMCNT((NIA + NIB) * (NSTAGE - 2));  // all but the NSTAGE-2 younger steps
-    else MG_WAIT_VMCNT(0);
+#ifdef MG_TIMELINE
+    const long long tl_c0 = clock64();
+#endif
+    // all but the NSTAGE - 2 younger steps' requests
+    if (it + NSTAGE - 2 >= steps || NSTAGE == 2) MG_WAIT_VMCNT(0);
+    else if (per_step == NIA + NIB) MG_WAIT_VMCNT((NIA + NIB) * (NSTAGE - 2));
+    else if (per_step == NIB) MG_WAIT_VMCNT(NIB * (NSTAGE - 2));
+    else if (per_step == NIA) MG_WAIT_VMCNT(NIA * (NSTAGE - 2));
     // A plain barrier: __syncthreads() carries a fence that waits for every outstanding
     // copy into LDS, the younger steps' included.
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    if (it + NSTAGE - 1 < steps) {
-      gemm16_pipe_issue<NIA, NW>(a16 + (it + NSTAGE - 1) * a_step, src_a, lds + nxt * OP);
-      gemm16_pipe_issue<NIB, NW>(b16 + (it + NSTAGE - 1) * b_step, src_b, lds + nxt * OP + OPA);
-    }
+#ifdef MG_TIMELINE
+    tl_wait += clock64() - tl_c0;
+    if (it == 0) tl_first = wall_clock64();
+#endif
+    if (it + NSTAGE - 1 < steps) request(it + NSTAGE - 1, nxt);
     const char* la = lds + cur * OP;
     const char* lb = la + OPA;
     if constexpr (CAN_COLSUM) {
-      if (colsum) {
+      if (colsum && cs_thread) {
 #pragma unroll
         for (int j = 0; j < BK / 16; ++j) {
           const int kk = cs_row + 16 * j;
@@ -900,16 +969,16 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
     uint4 fa[2][2], fb[2][2];
     fa[0][0] = gemm16_pipe_frag<A_KC, BK, TM>(la, wm, 0, lane);
     fa[0][1] = gemm16_pipe_frag<A_KC, BK, TM>(la, wm + 32, 0, lane);
-    fb[0][0] = gemm16_pipe_frag<B_KC, BK, kGemmBN>(lb, wn, 0, lane);
-    fb[0][1] = gemm16_pipe_frag<B_KC, BK, kGemmBN>(lb, wn + 32, 0, lane);
+    fb[0][0] = gemm16_pipe_frag<B_KC, BK, TN>(lb, wn, 0, lane);
+    fb[0][1] = gemm16_pipe_frag<B_KC, BK, TN>(lb, wn + 32, 0, lane);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       const int c = ks % 2, n = c ^ 1;
       if (ks + 1 < BK / 16) {
         fa[n][0] = gemm16_pipe_frag<A_KC, BK, TM>(la, wm, ks + 1, lane);
         fa[n][1] = gemm16_pipe_frag<A_KC, BK, TM>(la, wm + 32, ks + 1, lane);
-        fb[n][0] = gemm16_pipe_frag<B_KC, BK, kGemmBN>(lb, wn, ks + 1, lane);
-        fb[n][1] = gemm16_pipe_frag<B_KC, BK, kGemmBN>(lb, wn + 32, ks + 1, lane);
+        fb[n][0] = gemm16_pipe_frag<B_KC, BK, TN>(lb, wn, ks + 1, lane);
+        fb[n][1] = gemm16_pipe_frag<B_KC, BK, TN>(lb, wn + 32, ks + 1, lane);
       }
       acc[0][0] = GemmMma16<T>::run(fa[c][0], fb[c][0], acc[0][0]);
       acc[0][1] = GemmMma16<T>::run(fa[c][0], fb[c][1], acc[0][1]);
@@ -919,6 +988,10 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
     cur = cur + 1 == NSTAGE ? 0 : cur + 1;
     nxt = nxt + 1 == NSTAGE ? 0 : nxt + 1;
   }
+#ifdef MG_TIMELINE
+  const long long tl_loop = wall_clock64();
+  const long long tl_loop_c = clock64();
+#endif
   __syncthreads();  // every wave is done with the staged tiles: their memory serves the output
 
   if constexpr (CAN_COLSUM) {
@@ -927,8 +1000,10 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
       // added in a fixed order through LDS, one thread per column
       constexpr int kPitch = 128 + 4;
       float* red = reinterpret_cast<float*>(lds);
+      if (cs_thread) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) red[cs_row * kPitch + cs_chunk * 8 + e] = cs_acc[e];
+        for (int e = 0; e < 8; ++e) red[cs_row * kPitch + cs_chunk * 8 + e] = cs_acc[e];
+      }
       __syncthreads();
       if (threadIdx.x < 128 && m0 + static_cast<int>(threadIdx.x) < M) {
         float sum = 0.f;
@@ -944,6 +1019,15 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
   gemm16_write_tile<T, HAS_BIAS, SPLIT_K>(acc, mine, bias, C, partial, M, N, ldc, bsc, batch,
                                           split, SPLIT_K ? batches : 1,
                                           m0, n0, wm, wn, lane, ep);
+#ifdef MG_TIMELINE
+  if (threadIdx.x == 0 && blockIdx.x < 16384) {
+    long long* t = mg_timeline + static_cast<long long>(blockIdx.x) * 8;
+    t[0] = tl_entry; t[1] = tl_pro; t[2] = tl_first; t[3] = tl_loop; t[4] = wall_clock64();
+    t[5] = tl_wait; t[6] = steps | (SPLIT_K ? 1 << 20 : 0);
+    t[7] = (static_cast<long long>(__builtin_amdgcn_s_getreg(63508)) << 32) | static_cast<unsigned>(__builtin_amdgcn_s_getreg(63492));
+    (void)tl_loop_c;
+  }
+#endif
 }
 
 template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, int BK, int NSTAGE, int TM = 128>
@@ -964,13 +1048,13 @@ __global__ __launch_bounds__(TM * 2, gemm16_pipe_occupancy(BK, NSTAGE, TM)) void
 // half-empty CUs (384 dX tiles on 256 CUs) and pay a launch apiece.  With
 // dw.colsum_part set, the dW workgroups of the first tile column also produce the bias
 // gradient's partial rows from the dY tiles they hold anyway.
-template <typename T, int NSTAGE = 2>
-__global__ __launch_bounds__(256, gemm16_pipe_occupancy(32, NSTAGE, 128)) void linear_bwd_16bit_kernel(
+template <typename T, int NSTAGE = 2, int TN = kGemmBN, int BK = 32>
+__global__ __launch_bounds__(2 * TN, gemm16_pipe_occupancy(BK, NSTAGE, 128, TN)) void linear_bwd_16bit_kernel(
     Gemm16Problem<T> dw, Gemm16Problem<T> dx, int n_dw) {
-  __shared__ __attribute__((aligned(1024))) char lds[gemm16_pipe_lds_bytes(32, NSTAGE, 128)];
+  __shared__ __attribute__((aligned(1024))) char lds[gemm16_pipe_lds_bytes(BK, NSTAGE, 128, TN)];
   const int bid = blockIdx.x;
-  if (bid < n_dw) gemm16_pipe_block<T, false, false, false, true, 32, NSTAGE, 128>(lds, bid, dw);
-  else gemm16_pipe_block<T, true, false, false, false, 32, NSTAGE, 128>(lds, bid - n_dw, dx);
+  if (bid < n_dw) gemm16_pipe_block<T, false, false, false, true, BK, NSTAGE, 128, TN>(lds, bid, dw);
+  else gemm16_pipe_block<T, true, false, false, false, BK, NSTAGE, 128, TN>(lds, bid - n_dw, dx);
 }
 
 // ------------------------------------------------------------------------------------
@@ -1153,17 +1237,22 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_pipe_kernel(
 // groups of four consecutive outputs; its four waves each sum every fourth split (eight
 // independent 16-byte loads in flight per thread) and the four sums meet in LDS.  The
 // order of the additions is fixed, so the result is deterministic.
-template <typename T, bool HAS_BIAS>
+// TILED: the partials are whole 128 x 128 tiles in accumulator order (kG16PartialTile), numel
+// = slice = their count per K range, and a group of four is four consecutive rows of one
+// column of `out` (rows x N per batch; tiles_n tile columns; rows and columns past the matrix
+// are dropped).
+template <typename T, bool HAS_BIAS, bool TILED = false>
 __device__ __forceinline__ void gemm_splitk_reduce_block(float4 (&tile)[4][64], int64_t bid,
                                                          const float* __restrict__ partial, const T* __restrict__ bias,
                                                          T* __restrict__ out, int64_t numel, int64_t slice, int splits,
-                                                         int N, const GemmEpilogue<T>& ep) {
+                                                         int N, const GemmEpilogue<T>& ep, int rows = 0,
+                                                         int tiles_n = 0) {
   const int cx = threadIdx.x % 64;
   const int sl = threadIdx.x / 64;
   const int64_t i = (bid * 64 + cx) * 4;
   float4 acc0 = make_float4(0.f, 0.f, 0.f, 0.f), acc1 = acc0;
   if (i < numel) {
-    const bool full = i + 3 < numel;
+    const bool full = TILED || i + 3 < numel;
     int s = sl;
     if (full) {
       for (; s + 4 < splits; s += 8) {
@@ -1191,19 +1280,39 @@ __device__ __forceinline__ void gemm_splitk_reduce_block(float4 (&tile)[4][64], 
   const float4 t0 = tile[0][cx], t1 = tile[1][cx], t2 = tile[2][cx], t3 = tile[3][cx];
   const float r[4] = {(t0.x + t1.x) + (t2.x + t3.x), (t0.y + t1.y) + (t2.y + t3.y), (t0.z + t1.z) + (t2.z + t3.z),
                       (t0.w + t1.w) + (t2.w + t3.w)};
-  for (int e = 0; e < 4 && i + e < numel; ++e) {
-    const float bv = HAS_BIAS ? to_float(bias[(i + e) % N]) : 0.f;
-    out[i + e] = gemm_finish<T>(r[e] + bv, ep, i + e);
+  if constexpr (TILED) {
+    // bid * 64 + cx = ((((t * 4 + wave) * 2 + ti) * 2 + tj) * 4 + g) * 64 + lane, and cx = lane
+    const int64_t q = bid * 64;
+    const int g = static_cast<int>(q / 64 % 4), tj = static_cast<int>(q / 256 % 2), ti = static_cast<int>(q / 512 % 2);
+    const int wave = static_cast<int>(q / 1024 % 4);
+    const int64_t t = q / 4096;  // tile over (batch, tile row, tile column)
+    const int tiles_m = (rows + kGemmBM - 1) / kGemmBM;
+    const int tn = static_cast<int>(t % tiles_n), tm = static_cast<int>(t / tiles_n % tiles_m);
+    const int64_t batch = t / tiles_n / tiles_m;
+    const int row = tm * kGemmBM + (wave / 2) * 64 + ti * 32 + g * 8 + (cx / 32) * 4;
+    const int col = tn * kGemmBN + (wave % 2) * 64 + tj * 32 + cx % 32;
+    if (col >= N) return;
+    const float bv = HAS_BIAS ? to_float(bias[col]) : 0.f;
+    for (int e = 0; e < 4 && row + e < rows; ++e) {
+      const int64_t at = (batch * rows + row + e) * N + col;
+      out[at] = gemm_finish<T>(r[e] + bv, ep, at);
+    }
+  } else {
+    for (int e = 0; e < 4 && i + e < numel; ++e) {
+      const float bv = HAS_BIAS ? to_float(bias[(i + e) % N]) : 0.f;
+      out[i + e] = gemm_finish<T>(r[e] + bv, ep, i + e);
+    }
   }
 }
 
-template <typename T, bool HAS_BIAS>
+template <typename T, bool HAS_BIAS, bool TILED = false>
 __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ partial,
                                                                  const T* __restrict__ bias, T* __restrict__ out,
                                                                  int64_t numel, int64_t slice, int splits, int N,
-                                                                 GemmEpilogue<T> ep) {
+                                                                 GemmEpilogue<T> ep, int rows = 0, int tiles_n = 0) {
   __shared__ float4 tile[4][64];
-  gemm_splitk_reduce_block<T, HAS_BIAS>(tile, blockIdx.x, partial, bias, out, numel, slice, splits, N, ep);
+  gemm_splitk_reduce_block<T, HAS_BIAS, TILED>(tile, blockIdx.x, partial, bias, out, numel, slice, splits, N, ep, rows,
+                                               tiles_n);
 }
 
 // What follows the common launch of a Linear layer's backward: workgroups [0, dw_blocks) sum
@@ -1212,14 +1321,16 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
 // every fourth row per 64 threads, then (t0 + t1) + (t2 + t3).  Fixed order, no atomics.
 template <typename T>
 __global__ __launch_bounds__(256) void linear_bwd_finish_kernel(const float* __restrict__ partial, T* __restrict__ dw,
-                                                                int64_t numel, int64_t slice, int splits, int K,
+                                                                int dw_rows, int64_t slice, int splits, int K,
                                                                 int dw_blocks, const float* __restrict__ db_part,
                                                                 T* __restrict__ db, int groups, int N) {
   __shared__ float4 tile[4][64];
   const int bid = blockIdx.x;
   if (bid < dw_blocks) {
-    gemm_splitk_reduce_block<T, false>(tile, bid, partial, static_cast<const T*>(nullptr), dw, numel, slice, splits, K,
-                                       GemmEpilogue<T>{nullptr, nullptr, 0});
+    // dW is (dw_rows, K); the partial tiles cover the (N, K) product of the launch
+    gemm_splitk_reduce_block<T, false, true>(tile, bid, partial, static_cast<const T*>(nullptr), dw, slice, slice,
+                                             splits, K, GemmEpilogue<T>{nullptr, nullptr, 0}, dw_rows,
+                                             (K + kGemmBN - 1) / kGemmBN);
     return;
   }
   float(&sums)[4][64] = *reinterpret_cast<float(*)[4][64]>(&tile[0][0]);

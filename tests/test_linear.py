@@ -570,8 +570,12 @@ def test_linear_bwd_one_launch_matches_two(device, monkeypatch, dtype, rtol, M, 
     results = {}
     # the common launch splits dW for one workgroup per CU; ask the separate launch for the same
     monkeypatch.setenv("MOGRAD_HIP_GEMM_SPLITK_WG_PER_CU", "1")
-    for mode in ("0", "1"):
-        monkeypatch.setenv("MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH", mode)
+    # Input widths that are multiples of 384 take 128 x 384 tiles in the common launch, with dW's
+    # K ranges cut differently: "wide" is compared within the tolerance, the 128 x 128 form bitwise.
+    modes = ("0", "1", "wide") if K % 384 == 0 else ("0", "1")
+    for mode in modes:
+        monkeypatch.setenv("MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH", "0" if mode == "0" else "1")
+        monkeypatch.setenv("MOGRAD_HIP_LINEAR_BWD_WIDE", "1" if mode == "wide" else "0")
         out = []
         for accumulate, masked in ((0, 0), (1, 1)):
             dx = AnyBuffer.from_numpy(device, prior, dtype)
@@ -590,14 +594,20 @@ def test_linear_bwd_one_launch_matches_two(device, monkeypatch, dtype, rtol, M, 
             assert_close(got, base, rtol, rtol * np.abs(base).max(), name)
         else:
             np.testing.assert_array_equal(got, base, err_msg=name)
-    np.testing.assert_array_equal(results["1"][2], results["1"][5], err_msg="db, second call")
-    want_db = O.linear_grad_b(dy)
-    assert_close(results["1"][2], want_db, rtol, rtol * np.abs(want_db).max(), "db")
-    dx, dw = results["1"][0], results["1"][1]
-    for got, want, name in ((dx, O.linear_grad_x(dy, w), "dx"), (dw, O.linear_grad_w(dy, x), "dw")):
-        assert_close(got, want, rtol, rtol * np.abs(want).max(), name)
-    masked = results["1"][3]
-    assert_close(masked, prior + O.linear_grad_x(dy, w) * (x > 0), 2 * rtol, 2 * rtol * np.abs(dx).max(), "dx masked+acc")
+    want_db, want_dx, want_dw = O.linear_grad_b(dy), O.linear_grad_x(dy, w), O.linear_grad_w(dy, x)
+    for mode in modes[1:]:
+        res = results[mode]
+        np.testing.assert_array_equal(res[2], res[5], err_msg="db, second call")
+        np.testing.assert_array_equal(res[1], res[4], err_msg="dw, second call")
+        assert_close(res[2], want_db, rtol, rtol * np.abs(want_db).max(), "db")
+        for got, want, name in ((res[0], want_dx, "dx"), (res[1], want_dw, "dw")):
+            assert_close(got, want, rtol, rtol * np.abs(want).max(), f"{name} ({mode})")
+        assert_close(res[3], prior + want_dx * (x > 0), 2 * rtol, 2 * rtol * np.abs(want_dx).max(), "dx masked+acc")
+    if "wide" in results:
+        # same dX tiles' k order (one tile is three of the narrow ones side by side): bitwise
+        if not dx_split_alone:
+            np.testing.assert_array_equal(results["wide"][0], results["0"][0], err_msg="dx wide")
+            np.testing.assert_array_equal(results["wide"][3], results["0"][3], err_msg="dx masked+acc wide")
 
 
 @pytest.mark.parametrize("dtype,rtol", [(F16, 2e-3), (BF16, 1.6e-2)])
