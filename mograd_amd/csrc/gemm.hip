@@ -602,15 +602,3 @@ int mg_linear_bwd_fused(const void* dy, const void* x, const void* w, void* dx, 
 }
 
 }  // extern "C"
-
-#ifdef MG_TIMELINE
-namespace mg { __device__ long long mg_timeline[16384 * 8]; }
-extern "C" int mg_debug_timeline(void* out, long long count, int clear) {
-  if (clear) {
-    void* p = nullptr;
-    if (hipGetSymbolAddress(&p, HIP_SYMBOL(mg::mg_timeline)) != hipSuccess) return 1;
-    return hipMemset(p, 0, sizeof(long long) * 16384 * 8) == hipSuccess ? 0 : 1;
-  }
-  return hipMemcpyFromSymbol(out, HIP_SYMBOL(mg::mg_timeline), sizeof(long long) * count) == hipSuccess ? 0 : 1;
-}
-#endif

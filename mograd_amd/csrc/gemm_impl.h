@@ -837,9 +837,6 @@ struct Gemm16Problem {
   float* colsum_part = nullptr;
 };
 
-#ifdef MG_TIMELINE
-extern __device__ long long mg_timeline[16384 * 8];
-#endif
 // The work of workgroup `bid` of a launch for one product; `lds` is the workgroup's
 // gemm16_pipe_lds_bytes(BK, NSTAGE, TM, TN) bytes, aligned to 1024.  The output tile is
 // TM x TN, (TM / 64) x (TN / 64) waves with 64 x 64 each; pr.tiles_n counts tiles of TN columns.
@@ -867,10 +864,6 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
   const GemmEpilogue<T> ep = pr.ep;
 
   const int tiles = tiles_m * tiles_n;
-#ifdef MG_TIMELINE
-  const long long tl_entry = wall_clock64();
-  long long tl_wait = 0, tl_first = 0;
-#endif
   int batch = bid / tiles, tile = bid % tiles, split = 0;
   if constexpr (SPLIT_K) {
     if (!gemm_split_work(bid, tiles, splits, batches, tile, split, batch)) return;
@@ -929,14 +922,8 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
 #pragma unroll
   for (int s = 0; s < NSTAGE - 1; ++s)
     if (s < steps) request(s, s);
-#ifdef MG_TIMELINE
-  const long long tl_pro = wall_clock64();
-#endif
   int cur = 0, nxt = NSTAGE - 1;
   for (int it = 0; it < steps; ++it) {
-#ifdef MG_TIMELINE
-    const long long tl_c0 = clock64();
-#endif
     // all but the NSTAGE - 2 younger steps' requests
     if (it + NSTAGE - 2 >= steps || NSTAGE == 2) MG_WAIT_VMCNT(0);
     else if (per_step == NIA + NIB) MG_WAIT_VMCNT((NIA + NIB) * (NSTAGE - 2));
@@ -945,10 +932,6 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
     // A plain barrier: __syncthreads() carries a fence that waits for every outstanding
     // copy into LDS, the younger steps' included.
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-#ifdef MG_TIMELINE
-    tl_wait += clock64() - tl_c0;
-    if (it == 0) tl_first = wall_clock64();
-#endif
     if (it + NSTAGE - 1 < steps) request(it + NSTAGE - 1, nxt);
     const char* la = lds + cur * OP;
     const char* lb = la + OPA;
@@ -988,10 +971,6 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
     cur = cur + 1 == NSTAGE ? 0 : cur + 1;
     nxt = nxt + 1 == NSTAGE ? 0 : nxt + 1;
   }
-#ifdef MG_TIMELINE
-  const long long tl_loop = wall_clock64();
-  const long long tl_loop_c = clock64();
-#endif
   __syncthreads();  // every wave is done with the staged tiles: their memory serves the output
 
   if constexpr (CAN_COLSUM) {
@@ -1019,15 +998,6 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
   gemm16_write_tile<T, HAS_BIAS, SPLIT_K>(acc, mine, bias, C, partial, M, N, ldc, bsc, batch,
                                           split, SPLIT_K ? batches : 1,
                                           m0, n0, wm, wn, lane, ep);
-#ifdef MG_TIMELINE
-  if (threadIdx.x == 0 && blockIdx.x < 16384) {
-    long long* t = mg_timeline + static_cast<long long>(blockIdx.x) * 8;
-    t[0] = tl_entry; t[1] = tl_pro; t[2] = tl_first; t[3] = tl_loop; t[4] = wall_clock64();
-    t[5] = tl_wait; t[6] = steps | (SPLIT_K ? 1 << 20 : 0);
-    t[7] = (static_cast<long long>(__builtin_amdgcn_s_getreg(63508)) << 32) | static_cast<unsigned>(__builtin_amdgcn_s_getreg(63492));
-    (void)tl_loop_c;
-  }
-#endif
 }
 
 template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, int BK, int NSTAGE, int TM = 128>
