@@ -26,10 +26,10 @@ static int check_attn(const char* who, int64_t B, int64_t S, int64_t H, int64_t 
   return MG_OK;
 }
 
-// The row-per-thread kernels (attention_tiled.h) take head dimensions up to 128 once a sequence
-// has rows for a workgroup; MOGRAD_HIP_ATTN_TILED=0 keeps the wave-per-row kernels.
+// The row-per-thread kernels (attention_tiled.h) take over once a sequence has rows for a
+// workgroup; MOGRAD_HIP_ATTN_TILED=0 keeps the wave-per-row kernels.
 static bool attn_tiled_ok(const AttnDims& a) {
-  return a.D <= 128 && a.S >= 64 && static_cast<int64_t>(a.B) * a.H <= 65535 && env_int("MOGRAD_HIP_ATTN_TILED", 1) != 0;
+  return a.D <= 512 && a.S >= 64 && static_cast<int64_t>(a.B) * a.H <= 65535 && env_int("MOGRAD_HIP_ATTN_TILED", 1) != 0;
 }
 
 template <typename T, int NT, int DL>
@@ -76,7 +76,9 @@ static int fwd_generic(const void* q, const void* k, const void* v, const void* 
   if (attn_tiled_ok(a)) {
     if (a.D <= 32) fwd_tiled_launch<T, 1, 32>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
     else if (a.D <= 64) fwd_tiled_launch<T, 2, 32>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
-    else fwd_tiled_launch<T, 4, 32>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
+    else if (a.D <= 128) fwd_tiled_launch<T, 4, 32>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
+    else if (a.D <= 256) fwd_tiled_launch<T, 8, 32>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
+    else fwd_tiled_launch<T, 16, 32>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
     MG_LAUNCH_CHECK();
     return MG_OK;
   }
@@ -108,7 +110,9 @@ static int bwd_generic(const void* d_o, const void* o, const void* q, const void
     const float* dl = delta.as<float>();
     if (a.D <= 32) bwd_tiled_launch<T, 1, 32, 1, 32>(d_o, q, k, v, mask, lse, dl, dq, dk, dv, a, scale, causal, has_bias, stream);
     else if (a.D <= 64) bwd_tiled_launch<T, 2, 32, 2, 32>(d_o, q, k, v, mask, lse, dl, dq, dk, dv, a, scale, causal, has_bias, stream);
-    else bwd_tiled_launch<T, 4, 32, 4, 32>(d_o, q, k, v, mask, lse, dl, dq, dk, dv, a, scale, causal, has_bias, stream);
+    else if (a.D <= 128) bwd_tiled_launch<T, 4, 32, 4, 32>(d_o, q, k, v, mask, lse, dl, dq, dk, dv, a, scale, causal, has_bias, stream);
+    else if (a.D <= 256) bwd_tiled_launch<T, 8, 32, 8, 32>(d_o, q, k, v, mask, lse, dl, dq, dk, dv, a, scale, causal, has_bias, stream);
+    else bwd_tiled_launch<T, 16, 32, 16, 32>(d_o, q, k, v, mask, lse, dl, dq, dk, dv, a, scale, causal, has_bias, stream);
     MG_LAUNCH_CHECK();
     return MG_OK;
   }

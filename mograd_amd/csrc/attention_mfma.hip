@@ -277,7 +277,7 @@ __device__ __forceinline__ void store4(T* dst, const floatx16& acc, int g, float
 // ---- forward -----------------------------------------------------------------------------
 
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
-__global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T* __restrict__ q, const T* __restrict__ k,
+__global__ __launch_bounds__(kAttnThreads, DP <= 128 ? 2 : 1) void attn_fwd_mfma_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                                         const T* __restrict__ v,
                                                                         const T* __restrict__ mask, T* __restrict__ o,
                                                                         float* __restrict__ lse, AttnDims a, float scale) {
@@ -451,6 +451,10 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_mfma_kernel(const T*
 // A wave owns MQ tiles of 32 queries; every A fragment read from LDS (K rows, V rows,
 // K^T) feeds MQ MFMAs, which is what keeps LDS bandwidth below the MFMA rate.
 
+// Head dims above 128 (the 256 bucket): the backward walks of a block run as this many
+// workgroups, each producing one part of the head dimension of its gradients.
+constexpr int kAttnWideSplit = 2;
+
 // Bytes of LDS the dQ walk stages its tiles in.
 template <int DP>
 constexpr int dq_lds_bytes() {
@@ -458,13 +462,17 @@ constexpr int dq_lds_bytes() {
 }
 
 // The work of workgroup `block` of a dQ launch; `smem` holds dq_lds_bytes<DP>() bytes.
-template <typename T, int DP, int MQ, bool CAUSAL, bool HAS_BIAS>
+// DSPLIT > 1: the workgroup produces only part DPART of the head dimension's DSPLIT equal
+// parts of dQ (the score products still run over the whole head), so that the accumulators of a
+// 256-wide head fit the register file; the parts are separate workgroups.
+template <typename T, int DP, int MQ, bool CAUSAL, bool HAS_BIAS, int DSPLIT = 1, int DPART = 0>
 __device__ __forceinline__ void attn_dq_block(const int block, char* smem, const T* __restrict__ d_o,
                                               const T* __restrict__ q, const T* __restrict__ k,
                                               const T* __restrict__ v, const T* __restrict__ mask,
                                               const float* __restrict__ lse, const float* __restrict__ delta,
                                               T* __restrict__ dq, const AttnDims& a, float scale) {
-  constexpr int BM = 128 * MQ, BN = 64, KS = DP / 16, DT = DP / 32;
+  constexpr int BM = 128 * MQ, BN = 64, KS = DP / 16, DT = DP / 32 / DSPLIT, DT0 = DPART * DT;
+  static_assert((DP / 32) % DSPLIT == 0 && DPART < DSPLIT, "parts of the head dimension");
   // Two copies of each staged tile (step i computes from copy i % 2 while the tile of step
   // i + 1 is written into the other: one barrier per step) for head dims up to 64.  Above,
   // one copy and two barriers per step: the two-copy schedule spills more there (68-108 bytes
@@ -613,7 +621,7 @@ __device__ __forceinline__ void attn_dq_block(const int block, char* smem, const
         for (int mq = 0; mq < MQ; ++mq) dsf[mq] = frag_from_acc<T>(s[mq], hf);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-          const uint4 kt = frag_transposed<DP>(k_rows, at, dt, t);
+          const uint4 kt = frag_transposed<DP>(k_rows, at, DT0 + dt, t);
 #pragma unroll
           for (int mq = 0; mq < MQ; ++mq) acc[mq][dt] = Mma<T>::run(kt, dsf[mq], acc[mq][dt]);
         }
@@ -629,7 +637,7 @@ __device__ __forceinline__ void attn_dq_block(const int block, char* smem, const
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const int d = dt * 32 + g * 8 + half * 4;
+          const int d = (DT0 + dt) * 32 + g * 8 + half * 4;
           if (d < a.D) store4<T>(out + d, acc[mq][dt], g, scale);
         }
     }
@@ -654,7 +662,8 @@ constexpr int dkdv_long_step() { return DP <= 64 ? 128 : 64; }
 
 // The work of workgroup `block` of a dK/dV launch, BQ queries per step; `smem` holds
 // dkdv_lds_bytes<DP, BQ>() bytes.
-template <typename T, int DP, int BQ, bool CAUSAL, bool HAS_BIAS>
+// DSPLIT, DPART: as for attn_dq_block, for dK and dV.
+template <typename T, int DP, int BQ, bool CAUSAL, bool HAS_BIAS, int DSPLIT = 1, int DPART = 0>
 __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, const T* __restrict__ d_o,
                                                 const T* __restrict__ q, const T* __restrict__ k,
                                                 const T* __restrict__ v, const T* __restrict__ mask,
@@ -662,7 +671,8 @@ __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, con
                                                 T* __restrict__ dk, T* __restrict__ dv, const AttnDims& a,
                                                 float scale) {
   constexpr int BNK = 128;                 // keys per workgroup
-  constexpr int MT = BQ / 32, KS = DP / 16, DT = DP / 32;
+  constexpr int MT = BQ / 32, KS = DP / 16, DT = DP / 32 / DSPLIT, DT0 = DPART * DT;
+  static_assert((DP / 32) % DSPLIT == 0 && DPART < DSPLIT, "parts of the head dimension");
   // Two copies of every staged tile: step i computes from copy i % 2 while the tile of step
   // i + 1 is written into the other, so one barrier per step suffices.
   constexpr int ROWS = BQ * tile_row_bytes<DP>();
@@ -786,8 +796,8 @@ __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, con
       for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-          tdo[hf][dt] = frag_transposed<DP>(do_rows, at, dt, mt * 2 + hf);
-          tq[hf][dt] = frag_transposed<DP>(q_rows, at, dt, mt * 2 + hf);
+          tdo[hf][dt] = frag_transposed<DP>(do_rows, at, DT0 + dt, mt * 2 + hf);
+          tq[hf][dt] = frag_transposed<DP>(q_rows, at, DT0 + dt, mt * 2 + hf);
         }
       __builtin_amdgcn_sched_barrier(0);
       if (plain) {
@@ -837,7 +847,7 @@ __device__ __forceinline__ void attn_dkdv_block(const int block, char* smem, con
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const int d = dt * 32 + g * 8 + half * 4;
+        const int d = (DT0 + dt) * 32 + g * 8 + half * 4;
         if (d < a.D) {
           store4<T>(outk + d, acc_k[dt], g, scale);
           store4<T>(outv + d, acc_v[dt], g, 1.0f);
@@ -1816,14 +1826,23 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_resident_kernel(
 }
 
 template <typename T, int DP, int MQ, bool CAUSAL, bool HAS_BIAS>
-__global__ __launch_bounds__(kAttnThreads, 2) void attn_dq_mfma_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
+__global__ __launch_bounds__(kAttnThreads, DP <= 128 ? 2 : 1) void attn_dq_mfma_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
                                                                        const T* __restrict__ k, const T* __restrict__ v,
                                                                        const T* __restrict__ mask,
                                                                        const float* __restrict__ lse,
                                                                        const float* __restrict__ delta,
                                                                        T* __restrict__ dq, AttnDims a, float scale) {
   __shared__ __attribute__((aligned(16))) char smem[dq_lds_bytes<DP>()];
-  attn_dq_block<T, DP, MQ, CAUSAL, HAS_BIAS>(blockIdx.x, smem, d_o, q, k, v, mask, lse, delta, dq, a, scale);
+  if constexpr (DP <= 128) {
+    attn_dq_block<T, DP, MQ, CAUSAL, HAS_BIAS>(blockIdx.x, smem, d_o, q, k, v, mask, lse, delta, dq, a, scale);
+  } else {
+    // wider heads: each half of the head dimension of a query block is a workgroup of its own
+    const int block = blockIdx.x / kAttnWideSplit;
+    if (blockIdx.x % kAttnWideSplit == 0)
+      attn_dq_block<T, DP, MQ, CAUSAL, HAS_BIAS, kAttnWideSplit, 0>(block, smem, d_o, q, k, v, mask, lse, delta, dq, a, scale);
+    else
+      attn_dq_block<T, DP, MQ, CAUSAL, HAS_BIAS, kAttnWideSplit, 1>(block, smem, d_o, q, k, v, mask, lse, delta, dq, a, scale);
+  }
 }
 
 template <typename T, int DP, bool CAUSAL>
@@ -1852,7 +1871,15 @@ __global__ __launch_bounds__(kAttnThreads, DP <= 64 ? 2 : 1) void attn_dkdv_mfma
     const T* __restrict__ mask, const float* __restrict__ lse, const float* __restrict__ delta, T* __restrict__ dk,
     T* __restrict__ dv, AttnDims a, float scale) {
   __shared__ __attribute__((aligned(16))) char smem[dkdv_lds_bytes<DP, dkdv_long_step<DP>()>()];
-  attn_dkdv_block<T, DP, dkdv_long_step<DP>(), CAUSAL, HAS_BIAS>(blockIdx.x, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
+  if constexpr (DP <= 128) {
+    attn_dkdv_block<T, DP, dkdv_long_step<DP>(), CAUSAL, HAS_BIAS>(blockIdx.x, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
+  } else {
+    const int block = blockIdx.x / kAttnWideSplit;
+    if (blockIdx.x % kAttnWideSplit == 0)
+      attn_dkdv_block<T, DP, 32, CAUSAL, HAS_BIAS, kAttnWideSplit, 0>(block, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
+    else
+      attn_dkdv_block<T, DP, 32, CAUSAL, HAS_BIAS, kAttnWideSplit, 1>(block, smem, d_o, q, k, v, mask, lse, delta, dk, dv, a, scale);
+  }
 }
 
 // Both walks in one launch (head dims up to 64, where the two have the same occupancy):
@@ -1887,7 +1914,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_bwd_mfma_kernel(
 
 bool attn_mfma_supported(int dtype, int64_t D, const void* const* ptrs, int nptrs) {
   if (dtype != MG_F16 && dtype != MG_BF16) return false;
-  if (D % 8 != 0 || D > 128) return false;  // rows are read 16 bytes at a time
+  if (D % 8 != 0 || D > 256) return false;  // rows are read 16 bytes at a time
   for (int i = 0; i < nptrs; ++i)
     if (ptrs[i] != nullptr && !aligned16(ptrs[i])) return false;
   const char* force = env_str("MOGRAD_HIP_ATTN_GENERIC");
@@ -2027,6 +2054,7 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
   T* dk_ = static_cast<T*>(dk);
   T* dv_ = static_cast<T*>(dv);
   const dim3 grid(static_cast<unsigned>(blocks)), grid_fused(static_cast<unsigned>(2 * ((blocks + 7) / 8 * 8)));
+  const dim3 grid_plain(static_cast<unsigned>(blocks * (DP > 128 ? kAttnWideSplit : 1)));
 #define MG_LAUNCH(C_, B_)                                                                                            \
   do {                                                                                                               \
     if constexpr (DP <= 64) {                                                                                        \
@@ -2051,10 +2079,10 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
         }                                                                                                            \
       }                                                                                                              \
     }                                                                                                                \
-    hipLaunchKernelGGL((attn_dkdv_mfma_kernel<T, DP, C_, B_>), grid, dim3(kAttnThreads), 0, stream, d_o_, q_, k_,    \
-                       v_, mask_, lse, delta.as<float>(), dk_, dv_, a, scale);                                       \
-    hipLaunchKernelGGL((attn_dq_mfma_kernel<T, DP, 1, C_, B_>), grid, dim3(kAttnThreads), 0, stream, d_o_, q_, k_,   \
-                       v_, mask_, lse, delta.as<float>(), dq_, a, scale);                                            \
+    hipLaunchKernelGGL((attn_dkdv_mfma_kernel<T, DP, C_, B_>), grid_plain, dim3(kAttnThreads), 0, stream, d_o_, q_,  \
+                       k_, v_, mask_, lse, delta.as<float>(), dk_, dv_, a, scale);                                   \
+    hipLaunchKernelGGL((attn_dq_mfma_kernel<T, DP, 1, C_, B_>), grid_plain, dim3(kAttnThreads), 0, stream, d_o_, q_, \
+                       k_, v_, mask_, lse, delta.as<float>(), dq_, a, scale);                                        \
   } while (0)
   if (causal) MG_LAUNCH(true, false);
   else if (has_bias) MG_LAUNCH(false, true);
@@ -2067,6 +2095,9 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
 int attn_fwd_mfma(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, AttnDims a,
                   float scale, bool causal, bool has_bias, int dtype, hipStream_t stream) {
   const bool small = a.D <= 64;
+  if (a.D > 128)
+    return dtype == MG_BF16 ? fwd_typed<bf16_t, 256>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream)
+                            : fwd_typed<f16_t, 256>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
   if (dtype == MG_BF16)
     return small ? fwd_typed<bf16_t, 64>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream)
                  : fwd_typed<bf16_t, 128>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
@@ -2078,6 +2109,10 @@ int attn_bwd_mfma(const void* d_o, const void* o, const void* q, const void* k, 
                   const float* lse, void* dq, void* dk, void* dv, AttnDims a, float scale, bool causal, bool has_bias,
                   int dtype, hipStream_t stream) {
   const bool small = a.D <= 64;
+  if (a.D > 128)
+    return dtype == MG_BF16
+               ? bwd_typed<bf16_t, 256>(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal, has_bias, stream)
+               : bwd_typed<f16_t, 256>(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal, has_bias, stream);
   if (dtype == MG_BF16)
     return small ? bwd_typed<bf16_t, 64>(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal, has_bias, stream)
                  : bwd_typed<bf16_t, 128>(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal, has_bias, stream);

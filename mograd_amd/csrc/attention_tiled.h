@@ -1,6 +1,6 @@
-// Flash attention in fp32 arithmetic for head dimensions up to 128, a row per thread (or per
-// two or four neighbouring threads): the form the general path takes when a sequence is long
-// enough to fill workgroups.
+// Flash attention in fp32 arithmetic for head dimensions up to 512, a row per thread (or per
+// two to sixteen neighbouring threads): the form the general path takes when a sequence is
+// long enough to fill workgroups.
 //
 // attention_generic.h gives every row a whole wave, one element of the head per lane, so each
 // (query, key) pair costs a wave-wide reduction: about thirty instructions for 64 products.
@@ -17,17 +17,22 @@
 
 namespace mg {
 
-// Sum over the NT neighbouring lanes that share a row (NT = 1, 2 or 4: inside a quad).
+// Sum over the NT neighbouring lanes that share a row (NT = 1 .. 16, a power of two: inside a
+// quad, then across the quads of eight and of sixteen lanes by the mirrored moves).
 template <int NT>
 __device__ __forceinline__ float row_lanes_sum(float v) {
+  static_assert(NT == 1 || NT == 2 || NT == 4 || NT == 8 || NT == 16, "lanes per row");
   if constexpr (NT >= 2) v += dpp_move<kDppQuadXor1>(v);
   if constexpr (NT >= 4) v += dpp_move<kDppQuadXor2>(v);
+  if constexpr (NT >= 8) v += dpp_move<kDppRowHalfMirror>(v);
+  if constexpr (NT >= 16) v += dpp_move<kDppRowMirror>(v);
   return v;
 }
 
-// Rows of a staged tile: 2048 / (NT * DL) of them, so that a tile is 8 KB per tensor.
+// Rows of a staged tile: 2048 / (NT * DL) of them, so that a tile is 8 KB per tensor, and at
+// least the eight keys that the forward handles at a time.
 template <int NT, int DL>
-constexpr int tiled_rows() { return 2048 / (NT * DL); }
+constexpr int tiled_rows() { return 2048 / (NT * DL) < 8 ? 8 : 2048 / (NT * DL); }
 
 // Stage TK rows (first row j0, row stride `ld` elements, rows >= S and columns >= D as zeros)
 // of `src` into `dst` [TK][NT * DL] as fp32, all 256 threads taking part.

@@ -81,10 +81,11 @@ def test_f32_error_budget(device, name, causal, with_mask, D, budget):
 
 @pytest.mark.parametrize("name,causal,with_mask", MODES)
 @pytest.mark.parametrize("B,H,S,D,budget", [(1, 2, 300, 64, 5e-6), (2, 1, 100, 128, 1e-5), (1, 3, 64, 24, 5e-6),
-                                            (1, 1, 257, 72, 1e-5), (2, 2, 130, 32, 5e-6)])
+                                            (1, 1, 257, 72, 1e-5), (2, 2, 130, 32, 5e-6), (1, 2, 150, 256, 2e-5),
+                                            (1, 1, 97, 200, 2e-5), (1, 2, 70, 512, 4e-5), (1, 1, 131, 328, 4e-5)])
 def test_f32_row_per_thread_and_wave_per_row_kernels(device, monkeypatch, name, causal, with_mask, B, H, S, D, budget):
-    # fp32 tensors with head dims up to 128 and at least 64 tokens take kernels that keep a row
-    # per thread (or per 2 / 4 neighbouring threads) and stage the other side through LDS;
+    # fp32 tensors with at least 64 tokens take kernels that keep a row per thread (or per 2 to
+    # 16 neighbouring threads, 32 elements of the head each) and stage the other side through LDS;
     # MOGRAD_HIP_ATTN_TILED=0 keeps a wave per row.  Both must meet the reference's fp32 budget
     # against the f64 oracle, at sequence lengths that leave ragged tiles and idle threads.
     q, k, v, do, m = _inputs(58, B, S, H, D, F32, with_mask)
@@ -98,7 +99,7 @@ def test_f32_row_per_thread_and_wave_per_row_kernels(device, monkeypatch, name, 
 
 
 HALF_SHAPES = [(2, 2, 96, 64), (1, 3, 200, 64), (2, 1, 128, 128), (1, 2, 257, 32), (1, 1, 4, 8), (1, 2, 96, 256),
-               (1, 2, 130, 72)]
+               (1, 2, 130, 72), (1, 1, 80, 512), (1, 2, 40, 192), (1, 2, 300, 256), (2, 1, 130, 200), (1, 1, 129, 136)]
 
 
 @pytest.mark.parametrize("dtype,budget_fwd,budget_bwd", [(F16, 2e-3, 8e-3), (BF16, 1.6e-2, 6.4e-2)])
