@@ -203,6 +203,64 @@ def _kernel_table(dev, entries, iters):
     return out
 
 
+# --------------------------------------------------------------------------- #
+# Sanity checks before timing: a few sampled rows of each workload's outputs
+# against plain float64 numpy, so that the timed numbers rest on checked
+# results.  (The parity tests proper, against the oracle, are under tests/.)
+# A mismatch raises; nothing here runs inside a timed region.
+# --------------------------------------------------------------------------- #
+
+
+def _check(name: str, got, want, rtol: float, floor: float = 1e-30) -> None:
+    """|got - want| <= rtol * (|want| + max(largest |want|, floor)), elementwise."""
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    bound = rtol * (np.abs(want) + max(float(np.abs(want).max()), floor))
+    bad = ~(np.abs(got - want) <= bound)  # NaN counts as bad
+    if bad.any():
+        k = int(np.argmax(np.abs(got - want) / bound))
+        raise RuntimeError(f"bench.py sanity check failed: {name}: got {got.flat[k]!r}, want {want.flat[k]!r} "
+                           f"(rtol {rtol}, {int(bad.sum())} of {bad.size} values off)")
+
+
+def _rows_to_host(dev, buf, rows, cols: int, np_dtype=np.float32) -> np.ndarray:
+    """Rows `rows` of a contiguous fp32 (rows, cols) device buffer, one small copy per row."""
+    out = np.empty((len(rows), cols), np_dtype)
+    for i, r in enumerate(rows):
+        dev.lib.mg_copy_to_host(out[i].ctypes.data_as(C.c_void_p), C.c_void_p(buf.data_ptr().value + r * cols * out.itemsize),
+                                cols * out.itemsize, dev.stream)
+    dev.synchronize()
+    return out
+
+
+def _verify_attention(q, k, v, do, o, lse, dq, dk, dv, B, H, S, D, causal: bool, rtol: float = 3e-2) -> None:
+    """O, lse, dQ for sampled queries and dK, dV for sampled keys of two (batch, head) pairs.  Q, K, V and
+    their gradients are (B, S, H, D); O and dO (B, H, S, D); lse (B, H, S).  (A causal query that sees one
+    key has dQ = 0 exactly and the kernels leave the rounding of dP - delta: hence the absolute floor.)"""
+    sc = 1.0 / np.sqrt(D)
+    for (b, h) in ((0, 0), (B - 1, H - 1)):
+        Q, K, V = (t[b, :, h, :].astype(np.float64) for t in (q, k, v))
+        Oh, dO, L = o[b, h].astype(np.float64), do[b, h].astype(np.float64), lse[b, h].astype(np.float64)
+        for i in (0, S // 2 + 1, S - 1):
+            s = sc * (K @ Q[i])
+            if causal:
+                s[i + 1:] = -np.inf
+            m = s.max()
+            p = np.exp(s - m)
+            l_ref = m + np.log(p.sum())
+            p /= p.sum()
+            _check(f"attention O[{b},{h},{i}]", Oh[i], p @ V, rtol)
+            _check(f"attention lse[{b},{h},{i}]", [L[i]], [l_ref], 1e-3)
+            ds = p * (V @ dO[i] - dO[i] @ Oh[i])
+            _check(f"attention dQ[{b},{i},{h}]", dq[b, i, h], sc * (ds @ K), rtol, 1e-2)
+        delta = np.einsum("sd,sd->s", dO, Oh)
+        for j in (0, S // 2 - 1, S - 1):
+            pj = np.exp(sc * (Q @ K[j]) - L)
+            if causal:
+                pj[:j] = 0.0
+            _check(f"attention dV[{b},{j},{h}]", dv[b, j, h], pj @ dO, rtol, 1e-2)
+            _check(f"attention dK[{b},{j},{h}]", dk[b, j, h], sc * ((pj * (dO @ V[j] - delta)) @ Q), rtol, 1e-2)
+
+
 def bench_mlp(args, dev) -> dict:
     """README MLP, fp32: x (2048,4096) -> Linear 4096->4096 +ReLU -> LayerNorm(4096) -> Linear 4096->4096 +ReLU
     -> Linear 4096->10, cross-entropy on labels in [0,10).  Forward and backward through the C ABI."""
@@ -249,6 +307,17 @@ def bench_mlp(args, dev) -> dict:
     def step(i):
         fwd(i)
         bwd(i)
+
+    # sampled rows of the second 4096 x 4096 layer's three products, and its db
+    step(0)
+    rows = [0, M // 3, M - 1]
+    w2_h, b2_h = w2.to_numpy((D, D)).astype(np.float64), b2.to_numpy().astype(np.float64)
+    ln_h, dy_h = ln.to_numpy((M, D)).astype(np.float64), dh2p.to_numpy((M, D)).astype(np.float64)
+    _check("mlp Y = X W^T + b", _rows_to_host(dev, h2p, rows, D), ln_h[rows] @ w2_h.T + b2_h, 1e-4)
+    _check("mlp dX = dY W", _rows_to_host(dev, dln, rows, D), dy_h[rows] @ w2_h, 1e-4)
+    _check("mlp dW = dY^T X", _rows_to_host(dev, dw2, rows, D), dy_h[:, rows].T @ ln_h, 1e-4)
+    _check("mlp db", db2.to_numpy(), dy_h.sum(axis=0), 1e-4)
+    del w2_h, ln_h, dy_h
 
     ms = _time_steps(dev, step, args.warmup, args.steps)
     fl = 2.0 * M * D * D
@@ -325,8 +394,17 @@ def bench_attention(args, dev) -> dict:
 
     c1 = (8, 12, 1024, 64)
     c2 = (2, 12, 4096, 64)
-    f1, b1 = runner(*c1, 1, make(*c1, 1))
-    f2, b2 = runner(*c2, 0, make(*c2, 2))
+    bufs1, bufs2 = make(*c1, 1), make(*c2, 2)
+    f1, b1 = runner(*c1, 1, bufs1)
+    f2, b2 = runner(*c2, 0, bufs2)
+    for (Bc, Hc, Sc, Dc), causal, bufs, f, b in ((c1, True, bufs1, f1, b1), (c2, False, bufs2, f2, b2)):
+        f(0)
+        b(0)
+        q_, k_, v_, do_, o_, dq_, dk_, dv_, lse_ = bufs
+        bshd, bhsd = (Bc, Sc, Hc, Dc), (Bc, Hc, Sc, Dc)
+        _verify_attention(q_.to_numpy(bshd), k_.to_numpy(bshd), v_.to_numpy(bshd), do_.to_numpy(bhsd), o_.to_numpy(bhsd),
+                          lse_.to_numpy((Bc, Hc, Sc)), dq_.to_numpy(bshd), dk_.to_numpy(bshd), dv_.to_numpy(bshd),
+                          Bc, Hc, Sc, Dc, causal)
 
     def step(i):
         f1(i)
@@ -396,6 +474,27 @@ def bench_gpt(args, dev) -> dict:
     model.load_params(init_params(_rng(5, 0), V, d, ff, L))
     ids = AnyBuffer.from_numpy(dev, _rng(5, 1).integers(0, V, (B, T)).astype(np.int32))
     labels = AnyBuffer.from_numpy(dev, _rng(5, 2).integers(0, V, (B, T)).astype(np.int32))
+
+    # the end of the chain on this step's own tensors: the loss from the logits, sampled rows of
+    # dlogits, the 65-symbol head's weight gradient from dlogits and the last hidden state, and
+    # every gradient finite
+    model.step(ids, labels, B, T)
+    lg = model.tmp["logits"].to_numpy((n, V)).astype(np.float64)
+    lab = labels.to_numpy().reshape(-1)
+    lsm = lg - lg.max(axis=1, keepdims=True)
+    lsm -= np.log(np.exp(lsm).sum(axis=1, keepdims=True))
+    _check("gpt loss", [model.loss.item()], [-lsm[np.arange(n), lab].mean()], 2e-3)
+    dl = model.tmp["dlogits"].to_numpy((n, V)).astype(np.float64)
+    rows = [0, n // 2 + 5, n - 1]
+    want = np.exp(lsm[rows])
+    for n_, r in enumerate(rows):
+        want[n_, lab[r]] -= 1.0
+    _check("gpt dlogits", dl[rows], want / n, 1e-2)
+    grads = model.gradients()
+    _check("gpt d lm_head", grads["lm_head"], dl.T @ model.h[L].to_numpy((n, d)).astype(np.float64), 2e-2)
+    if not np.all(np.isfinite(model.grads.to_numpy())):
+        raise RuntimeError("bench.py sanity check failed: gpt gradients are not all finite")
+    del lg, lsm, dl, grads
 
     ms = _time_steps(dev, lambda i: model.step(ids, labels, B, T), args.warmup, args.steps)
     loss = model.loss.item()
@@ -651,6 +750,29 @@ def bench_ln_ce(args, dev) -> dict:
         ln_fwd(i)
         ln_bwd(i)
         ce_fused(i)
+
+    # sampled rows of the cross-entropy gradient and of the LayerNorm outputs
+    step(0)
+    rows = [0, CE_ROWS // 2 + 3, CE_ROWS - 1]
+    lg = _rows_to_host(dev, logits, rows, CE_COLS).astype(np.float64)
+    idh = ids.to_numpy()
+    pr = np.exp(lg - lg.max(axis=1, keepdims=True))
+    pr /= pr.sum(axis=1, keepdims=True)
+    for n_, r in enumerate(rows):
+        pr[n_, idh[r]] -= 1.0
+    _check("cross-entropy dlogits", _rows_to_host(dev, dlogits, rows, CE_COLS), pr / CE_ROWS, 1e-4)
+    if not np.isfinite(loss.item()) or loss.item() <= 0.0:
+        raise RuntimeError(f"bench.py sanity check failed: cross-entropy loss {loss.item()!r}")
+    x0, dy0, y0, dx0 = ln_sets[0]
+    lrows = [0, LN_ROWS // 2, LN_ROWS - 1]
+    xh, dyh = (_rows_to_host(dev, t, lrows, LN_COLS).astype(np.float64) for t in (x0, dy0))
+    gh, bh_ = gamma.to_numpy().astype(np.float64), beta.to_numpy().astype(np.float64)
+    mu, var = xh.mean(axis=1, keepdims=True), xh.var(axis=1, keepdims=True)
+    xhat = (xh - mu) / np.sqrt(var + 1e-5)
+    _check("layer_norm y", _rows_to_host(dev, y0, lrows, LN_COLS), xhat * gh + bh_, 1e-4)
+    dyg = dyh * gh
+    dx_ref = (dyg - dyg.mean(axis=1, keepdims=True) - xhat * (dyg * xhat).mean(axis=1, keepdims=True)) / np.sqrt(var + 1e-5)
+    _check("layer_norm dx", _rows_to_host(dev, dx0, lrows, LN_COLS), dx_ref, 1e-4)
 
     # One plain device-to-device copy of known size (logits -> dlogits, 1.648 GB each way),
     # outside every timed region: under `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` it is the
