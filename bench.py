@@ -613,7 +613,7 @@ def bench_gpt(args, dev) -> dict:
                    "tokens_per_step": n, "loss": round(loss, 4)},
         "phases_ms": {"forward": round(float(np.mean(fwd_ms)), 4), "backward": round(float(np.mean(bwd_ms)), 4)},
         "roofline": {"bound": "mfma",
-                     "kernel": "linear_bwd_16bit_kernel (+ gemm_splitk_reduce_kernel): mg_linear_bwd at the block's four "
+                     "kernel": "linear_bwd_16bit_kernel (+ linear_bwd_finish_kernel): mg_linear_bwd at the block's four "
                                "layer shapes, 4 M N K FLOP each, mean over the four",
                      "achieved": round(lin_tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(lin_tf / MFMA_BF16_PEAK_TFLOPS, 4),
