@@ -40,7 +40,6 @@ template <typename T, int NT, int DL>
 __device__ __forceinline__ void tiled_stage(const T* __restrict__ src, int64_t ld, int j0, int S, int D,
                                             float* __restrict__ dst) {
   constexpr int DP = NT * DL, TK = tiled_rows<NT, DL>();
-#pragma unroll
   for (int e = threadIdx.x; e < TK * DP; e += 256) {
     const int jj = e / DP, d = e % DP;
     const int j = j0 + jj;
