@@ -555,7 +555,7 @@ def test_fused_epilogues_equal_separate_calls(device, dtype, M, N, K):
 
 @pytest.mark.parametrize("dtype,rtol", [(F16, 2e-3), (BF16, 1.6e-2)])
 @pytest.mark.parametrize("M,N,K", [(2048, 384, 384), (4096, 1152, 384), (2048, 1536, 384), (4096, 384, 1536),
-                                   (1056, 96, 200), (1024, 64, 72)])
+                                   (1056, 96, 200), (1024, 64, 72), (2048, 832, 768)])
 def test_linear_bwd_one_launch_matches_two(device, monkeypatch, dtype, rtol, M, N, K):
     # dX and dW of a 16-bit layer whose dW is split along the rows go out as one launch
     # (workgroups of both products in one grid); MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH=0 keeps the
