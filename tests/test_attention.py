@@ -123,10 +123,12 @@ def test_half_error_budget(device, dtype, budget_fwd, budget_bwd, name, causal, 
 
 
 @pytest.mark.parametrize("causal", [True, False])
-def test_long_ragged_sequence(device, causal):
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_long_ragged_sequence(device, causal, D):
     # Past 1024 tokens the head-dim-64 backward launches its dK/dV and dQ walks separately
-    # (one launch below that); 1100 is not a multiple of any tile.
-    B, H, S, D = 1, 2, 1100, 64
+    # (one launch below that); 1100 is not a multiple of any tile.  Head dims 128 and 256: the
+    # unpipelined walks, at 256 with the head dimension of the gradients split over two workgroups.
+    B, H, S = 1, 2, 1100
     q, k, v, do, _ = _inputs(56, B, S, H, D, BF16, False)
     o, lse, dq, dk, dv = _fwd_bwd(device, q, k, v, do, None, causal, dtype=BF16)
     ro, rl = O.sdpa_fwd(q, k, v, None, causal)
