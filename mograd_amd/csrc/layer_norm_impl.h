@@ -246,8 +246,13 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
           // by the same thread).
           float rs[VEC];
           VecIO<T, VEC>::load(residual + row * cols + c, rs);
+          {
+            // a plain addition, as the separate add kernel performs it: not to be contracted
+            // with the multiplication that produced the gradient
+#pragma clang fp contract(off)
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) out[e] = to_float(from_float<T>(out[e])) + rs[e];
+            for (int e = 0; e < VEC; ++e) out[e] = to_float(from_float<T>(out[e])) + rs[e];
+          }
         }
         VecIO<T, VEC>::store(dx + row * cols + c, out);
       }
