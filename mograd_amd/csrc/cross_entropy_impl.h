@@ -25,11 +25,15 @@ __device__ __forceinline__ float fast_exp2(float v) { return __builtin_amdgcn_ex
 
 template <int TPR, int WG, int K>
 __device__ __forceinline__ void row_allreduce_max(float (&v)[K], float* slots, int& phase) {
-  if constexpr (TPR == kWave) {
+  if constexpr (TPR == 16) {
+    // four rows side by side in a wave, each on one row of 16 lanes
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = row16_allreduce<MaxOp>(v[k]);
+  } else if constexpr (TPR == kWave) {
 #pragma unroll
     for (int k = 0; k < K; ++k) v[k] = wave_max(v[k]);
   } else {
-    static_assert(TPR == WG, "a row is shared by one wave or by the whole workgroup");
+    static_assert(TPR == WG, "a row is shared by sixteen lanes, one wave or the whole workgroup");
     block_allreduce<MaxOp, WG / kWave, K>(v, slots, phase);
     phase ^= 1;
   }
@@ -63,7 +67,7 @@ __global__ __launch_bounds__(WG, (TPR == 256 && VPT * VEC > 128) ? 2 : 1) void c
   // row's loads before this row's stores and double the register footprint.
   {
     const int64_t row = static_cast<int64_t>(blockIdx.x) * RPW + sub;
-    if (row >= N) return;  // uniform per wave (TPR == 64) or per workgroup (RPW == 1); no barrier follows for TPR == 64
+    if (row >= N) return;  // per 16-lane row, per wave or per workgroup (RPW == 1); no barrier follows for TPR <= 64
     const T* xr = logits + row * C;
     Tile x;
     x.load(xr, t, C);
@@ -436,7 +440,10 @@ struct CrossEntropyOps {
 
   // Thread layout for a row of `chunks` chunks held in registers; false if too wide.
   static bool pick_shape(int64_t chunks, bool wide, Shape* s) {
-    if (chunks <= 64) *s = {64, 1};
+    // Rows of up to 80 unaligned elements (a 65-symbol vocabulary): sixteen lanes per row, four
+    // rows per wave; one wave per row left most lanes idle and a latency per 130 bytes.
+    if (!wide && chunks <= 80 && env_int("MOGRAD_HIP_CE_NARROW", 1) != 0) *s = {16, 5};
+    else if (chunks <= 64) *s = {64, 1};
     else if (chunks <= 128) *s = {64, 2};
     else if (chunks <= 256) *s = {64, 4};
     else if (chunks <= 1024) *s = {256, 4};
@@ -474,7 +481,7 @@ struct CrossEntropyOps {
   template <int VEC, int TPR, int VPT, bool DENSE>
   static int launch_rows(const T* logits, const void* labels, const T* upstream, float* rowloss, T* dlogits, int64_t N,
                          int64_t C, int id64, hipStream_t stream) {
-    constexpr int WG = TPR == 64 ? 256 : TPR;
+    constexpr int WG = TPR <= 64 ? 256 : TPR;
     hipLaunchKernelGGL((ce_rows_kernel<T, VEC, TPR, VPT, WG, DENSE>), dim3(row_grid(N, WG / TPR)), dim3(WG), 0, stream,
                        logits, labels, upstream, rowloss, dlogits, N, static_cast<int>(C), id64);
     MG_LAUNCH_CHECK();
@@ -487,6 +494,7 @@ struct CrossEntropyOps {
 #define MG_CE_CASE(TPR_, VPT_)        \
   if (s.tpr == TPR_ && s.vpt == VPT_) \
   return launch_rows<VEC, TPR_, VPT_, DENSE>(logits, labels, upstream, rowloss, dlogits, N, C, id64, stream)
+    MG_CE_CASE(16, 5);
     MG_CE_CASE(64, 1);
     MG_CE_CASE(64, 2);
     MG_CE_CASE(64, 4);
