@@ -394,6 +394,54 @@ int mg_adam_step(void* w, const void* g, void* m, void* v, int64_t n, float lr, 
 int mg_sgd_step(void* w, const void* g, int64_t n, float lr, mg_stream stream);
 
 /* ------------------------------------------------------------------------------------ */
+/* Deferred second-stage reductions.  No counterpart in the reference, which runs every   */
+/* reduction where its graph node is evaluated.                                           */
+/*                                                                                        */
+/* mg_linear_bwd, mg_layer_norm_bwd_stats(_add) and mg_scatter_add each end in a short     */
+/* second kernel that adds fp32 partial results in a fixed order (the K ranges of dW and   */
+/* the partial rows of db; the row groups of dgamma/dbeta; the index slabs of the table).  */
+/* Nothing in a backward pass reads those sums, so a training step can leave them all to   */
+/* one launch at its end.  The `_deferred` forms take the same arguments plus              */
+/*   grad_dtype  element type of the parameter gradients this call produces (dw and db;    */
+/*               dgamma and dbeta; dst): the tensors' `dtype`, or MG_F32 to get the fp32   */
+/*               sums unrounded (fp32 master gradients of a 16-bit layer);                 */
+/*   list        an mg_deferred the pending sums are recorded on.                          */
+/* They enqueue the first-stage kernels (dx is complete when those are) and return; the    */
+/* parameter gradients are valid only after mg_finish_deferred(list, stream), called on    */
+/* the same stream, which sums everything on the list in one launch and empties it.  The   */
+/* sums use the code of the immediate forms: with grad_dtype == dtype the results are      */
+/* bit-identical to them, with MG_F32 they are the same fp32 sums before rounding.  A      */
+/* shape whose immediate form has no second stage, or none that can be deferred, is        */
+/* computed at once (and converted if grad_dtype differs).  The list keeps the partial     */
+/* results' pool blocks until it is finished or destroyed.  One list serves one stream     */
+/* and one host thread at a time.                                                          */
+/* ------------------------------------------------------------------------------------ */
+
+typedef void* mg_deferred;
+int mg_deferred_create(mg_deferred* out);
+/* Drops pending sums (their outputs stay unwritten) and frees the list. */
+int mg_deferred_destroy(mg_deferred list);
+/* Number of sums waiting on the list. */
+int mg_deferred_pending(mg_deferred list);
+/* Runs every pending sum of `list` in one launch on `stream` and empties the list. */
+int mg_finish_deferred(mg_deferred list, mg_stream stream);
+
+/* mg_linear_bwd_fused with dw and db of `grad_dtype`, their sums deferred. */
+int mg_linear_bwd_deferred(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db,
+                           int64_t M, int64_t N, int64_t K, int dx_accumulate, int x_is_relu_output,
+                           int dtype, int grad_dtype, mg_deferred list, mg_stream stream);
+/* mg_layer_norm_bwd_stats_add (`residual` may be NULL: mg_layer_norm_bwd_stats) with dgamma
+ * and dbeta of `grad_dtype`, their sums deferred. */
+int mg_layer_norm_bwd_stats_deferred(const void* dy, const void* x, const void* gamma, const float* mean,
+                                     const float* rstd, const void* residual, void* dx, void* dgamma,
+                                     void* dbeta, int64_t rows, int64_t cols, int dtype, int grad_dtype,
+                                     mg_deferred list, mg_stream stream);
+/* mg_scatter_add with dst of `grad_dtype`, the sum over the index slabs deferred. */
+int mg_scatter_add_deferred(const void* indices, const void* values, void* dst, int64_t n_idx,
+                            int64_t num_rows, int64_t row_size, int idx_dtype, int dtype, int grad_dtype,
+                            mg_deferred list, mg_stream stream);
+
+/* ------------------------------------------------------------------------------------ */
 /* Flash attention.  Q, K, V, dQ, dK, dV are BSHD; O and dO are BHSD; mask is            */
 /* (B,H,S,S) additive bias in natural-log units, of `dtype`; LSE is (B,H,S) fp32 natural  */
 /* log (kernels/attention/generic.mojo:29-35).  dtype in {F32, F16, BF16}.                */

@@ -109,6 +109,13 @@ PROTOTYPES = {
     "mg_contiguous": (_i, [_p, _p, _i, _pl, _pl, _i, _p], True),
     "mg_gather": (_i, [_p, _p, _p, _l, _l, _l, _l, _l, _i, _i, _p], True),
     "mg_scatter_add": (_i, [_p, _p, _p, _l, _l, _l, _i, _i, _p], True),
+    "mg_deferred_create": (_i, [C.POINTER(_p)], True),
+    "mg_deferred_destroy": (_i, [_p], True),
+    "mg_deferred_pending": (_i, [_p], False),
+    "mg_finish_deferred": (_i, [_p, _p], True),
+    "mg_linear_bwd_deferred": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _l, _i, _i, _i, _i, _p, _p], True),
+    "mg_layer_norm_bwd_stats_deferred": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _l, _l, _i, _i, _p, _p], True),
+    "mg_scatter_add_deferred": (_i, [_p, _p, _p, _l, _l, _l, _i, _i, _i, _p, _p], True),
     "mg_flash_attn_fwd": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _l, _l, _f, _i, _i, _i, _p], True),
     "mg_flash_attn_bwd": (_i, [_p] * 10 + [_l, _l, _l, _l, _f, _i, _i, _i, _p], True),
     "mg_flash_attn_fwd_bshd": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _l, _l, _f, _i, _i, _i, _p], True),

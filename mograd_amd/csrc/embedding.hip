@@ -224,7 +224,7 @@ static int scatter_launch(const I* indices, const T* values, T* dst, int64_t n_i
                      dst, n_idx, num_rows, row_size, slab_len);
   MG_LAUNCH_CHECK();
   const int64_t cols = num_rows * row_size;
-  launch_reduce_partials<T>(part.as<float>(), dst, nullptr, nullptr, slabs, cols, device_info().cu_count, s);
+  reduce_partials_or_defer<T>(part, dst, nullptr, static_cast<T*>(nullptr), slabs, cols, device_info().cu_count, s);
   MG_LAUNCH_CHECK();
   return MG_OK;
 }
@@ -281,6 +281,20 @@ int mg_gather(const void* src, const void* indices, void* dst, int64_t n_idx, in
       return mg::gather_by_index<mg::bf16_t>(src, indices, dst, n_idx, num_rows, row_size, src_row_stride,
                                              src_col_stride, idx_dtype, s);
   }
+}
+
+int mg_scatter_add_deferred(const void* indices, const void* values, void* dst, int64_t n_idx, int64_t num_rows,
+                            int64_t row_size, int idx_dtype, int dtype, int grad_dtype, mg_deferred list,
+                            mg_stream stream) {
+  if (!mg::is_float_dtype(dtype))
+    return mg::fail(MG_ERR_INVALID, "scatter_add_deferred: unsupported dtype %s", mg::dtype_name(dtype));
+  MG_TRY(mg::deferred_check("scatter_add_deferred", list, dtype, grad_dtype));
+  if (num_rows < 0 || row_size < 0) return mg::fail(MG_ERR_INVALID, "scatter_add_deferred: negative size");
+  mg::DeferredScope scope(static_cast<mg::DeferredList*>(list), dtype, grad_dtype);
+  void* dst_use;
+  MG_TRY(scope.substitute(dst, num_rows * row_size, &dst_use));
+  MG_TRY(mg_scatter_add(indices, values, dst_use, n_idx, num_rows, row_size, idx_dtype, dtype, stream));
+  return scope.finish(mg::to_stream(stream));
 }
 
 int mg_scatter_add(const void* indices, const void* values, void* dst, int64_t n_idx, int64_t num_rows,

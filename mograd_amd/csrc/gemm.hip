@@ -1,5 +1,6 @@
 // C ABI for the matmul family: operand classification, kernel choice, launches.
 #include "gemm_impl.h"
+#include "mg_deferred.h"
 
 namespace mg {
 
@@ -443,6 +444,19 @@ static int linear_bwd_one_launch(const void* dy, const void* x, const void* w, v
   MG_LAUNCH_CHECK();
   const int dw_blocks = static_cast<int>(slice / 256);
   const int db_blocks = groups > 0 ? static_cast<int>(ceil_div(N, 64)) : 0;
+  if (DeferredList* dl = deferred_current()) {
+    // The sums of the K ranges are left to mg_finish_deferred (same code, same order).
+    dl->push(kDeferSplitK, partial.as<float>(), dw, slice, static_cast<int>(dw_rows), static_cast<int>(K), splits,
+             ceil_div(dw_blocks, 4));
+    dl->hold(partial);
+    if (groups > 0) {
+      dl->push(kDeferBiasRows, db_part.as<float>(), db, 0, 0, static_cast<int>(N), groups, ceil_div(db_blocks, 4));
+      dl->hold(db_part);
+    }
+    if (db_done) *db_done = groups > 0;
+    *done = true;
+    return MG_OK;
+  }
   hipLaunchKernelGGL((linear_bwd_finish_kernel<T>), dim3(static_cast<unsigned>(dw_blocks + db_blocks)), dim3(256), 0,
                      stream, partial.as<float>(), static_cast<T*>(dw), static_cast<int>(dw_rows), slice, splits,
                      static_cast<int>(K), dw_blocks, db_part.as<float>(), static_cast<T*>(db), groups,
@@ -599,6 +613,21 @@ int mg_linear_bwd(const void* dy, const void* x, const void* w, void* dx, void* 
 int mg_linear_bwd_fused(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db, int64_t M, int64_t N,
                         int64_t K, int dx_accumulate, int x_is_relu_output, int dtype, mg_stream stream) {
   return linear_bwd_impl(dy, x, w, dx, dw, db, M, N, K, dx_accumulate != 0, x_is_relu_output != 0, dtype, stream);
+}
+
+int mg_linear_bwd_deferred(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db, int64_t M,
+                           int64_t N, int64_t K, int dx_accumulate, int x_is_relu_output, int dtype, int grad_dtype,
+                           mg_deferred list, mg_stream stream) {
+  if (!mg::is_float_dtype(dtype))
+    return mg::fail(MG_ERR_INVALID, "linear_bwd_deferred: unsupported dtype %s", mg::dtype_name(dtype));
+  MG_TRY(mg::deferred_check("linear_bwd_deferred", list, dtype, grad_dtype));
+  if (M < 0 || N < 0 || K < 0) return mg::fail(MG_ERR_INVALID, "linear_bwd_deferred: negative size");
+  mg::DeferredScope scope(static_cast<mg::DeferredList*>(list), dtype, grad_dtype);
+  void *dw_use, *db_use;
+  MG_TRY(scope.substitute(dw, N * K, &dw_use));
+  MG_TRY(scope.substitute(db, N, &db_use));
+  MG_TRY(linear_bwd_impl(dy, x, w, dx, dw_use, db_use, M, N, K, dx_accumulate != 0, x_is_relu_output != 0, dtype, stream));
+  return scope.finish(mg::to_stream(stream));
 }
 
 }  // extern "C"

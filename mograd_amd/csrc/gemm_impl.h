@@ -1212,13 +1212,13 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_pipe_kernel(
 // column of `out` (rows x N per batch; tiles_n tile columns; rows and columns past the matrix
 // are dropped).
 template <typename T, bool HAS_BIAS, bool TILED = false>
-__device__ __forceinline__ void gemm_splitk_reduce_block(float4 (&tile)[4][64], int64_t bid,
+__device__ __forceinline__ void gemm_splitk_reduce_block(float4 (&tile)[4][64], int tid, int64_t bid,
                                                          const float* __restrict__ partial, const T* __restrict__ bias,
                                                          T* __restrict__ out, int64_t numel, int64_t slice, int splits,
                                                          int N, const GemmEpilogue<T>& ep, int rows = 0,
                                                          int tiles_n = 0) {
-  const int cx = threadIdx.x % 64;
-  const int sl = threadIdx.x / 64;
+  const int cx = tid % 64;  // tid: this thread among the 256 that share `tile`
+  const int sl = tid / 64;
   const int64_t i = (bid * 64 + cx) * 4;
   float4 acc0 = make_float4(0.f, 0.f, 0.f, 0.f), acc1 = acc0;
   if (i < numel) {
@@ -1281,8 +1281,32 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
                                                                  int64_t numel, int64_t slice, int splits, int N,
                                                                  GemmEpilogue<T> ep, int rows = 0, int tiles_n = 0) {
   __shared__ float4 tile[4][64];
-  gemm_splitk_reduce_block<T, HAS_BIAS, TILED>(tile, blockIdx.x, partial, bias, out, numel, slice, splits, N, ep, rows,
+  gemm_splitk_reduce_block<T, HAS_BIAS, TILED>(tile, threadIdx.x, blockIdx.x, partial, bias, out, numel, slice, splits, N, ep, rows,
                                                tiles_n);
+}
+
+// db[c] = sum over the `groups` partial rows db_part[g][c], 64 columns per 256 threads (`tid`
+// of them, column block `bx`): every fourth row per 64 threads, then (t0 + t1) + (t2 + t3).
+// `sums_` is 256 floats of LDS; every one of the 256 threads must make the call.
+template <typename T>
+__device__ __forceinline__ void linear_bwd_db_block(float* __restrict__ sums_, int tid, int bx,
+                                                    const float* __restrict__ db_part, T* __restrict__ db, int groups,
+                                                    int N) {
+  float(&sums)[4][64] = *reinterpret_cast<float(*)[4][64]>(sums_);
+  const int cx = tid % 64, sl = tid / 64;
+  const int c = bx * 64 + cx;
+  float a0 = 0.f, a1 = 0.f;
+  if (c < N) {
+    int g = sl;
+    for (; g + 4 < groups; g += 8) {
+      a0 += db_part[static_cast<int64_t>(g) * N + c];
+      a1 += db_part[static_cast<int64_t>(g + 4) * N + c];
+    }
+    for (; g < groups; g += 4) a0 += db_part[static_cast<int64_t>(g) * N + c];
+  }
+  sums[sl][cx] = a0 + a1;
+  __syncthreads();
+  if (sl == 0 && c < N) db[c] = from_float<T>((sums[0][cx] + sums[1][cx]) + (sums[2][cx] + sums[3][cx]));
 }
 
 // What follows the common launch of a Linear layer's backward: workgroups [0, dw_blocks) sum
@@ -1298,26 +1322,13 @@ __global__ __launch_bounds__(256) void linear_bwd_finish_kernel(const float* __r
   const int bid = blockIdx.x;
   if (bid < dw_blocks) {
     // dW is (dw_rows, K); the partial tiles cover the (N, K) product of the launch
-    gemm_splitk_reduce_block<T, false, true>(tile, bid, partial, static_cast<const T*>(nullptr), dw, slice, slice,
+    gemm_splitk_reduce_block<T, false, true>(tile, threadIdx.x, bid, partial, static_cast<const T*>(nullptr), dw, slice,
+                                             slice,
                                              splits, K, GemmEpilogue<T>{nullptr, nullptr, 0}, dw_rows,
                                              (K + kGemmBN - 1) / kGemmBN);
     return;
   }
-  float(&sums)[4][64] = *reinterpret_cast<float(*)[4][64]>(&tile[0][0]);
-  const int cx = threadIdx.x % 64, sl = threadIdx.x / 64;
-  const int c = (bid - dw_blocks) * 64 + cx;
-  float a0 = 0.f, a1 = 0.f;
-  if (c < N) {
-    int g = sl;
-    for (; g + 4 < groups; g += 8) {
-      a0 += db_part[static_cast<int64_t>(g) * N + c];
-      a1 += db_part[static_cast<int64_t>(g + 4) * N + c];
-    }
-    for (; g < groups; g += 4) a0 += db_part[static_cast<int64_t>(g) * N + c];
-  }
-  sums[sl][cx] = a0 + a1;
-  __syncthreads();
-  if (sl == 0 && c < N) db[c] = from_float<T>((sums[0][cx] + sums[1][cx]) + (sums[2][cx] + sums[3][cx]));
+  linear_bwd_db_block<T>(reinterpret_cast<float*>(&tile[0][0]), threadIdx.x, bid - dw_blocks, db_part, db, groups, N);
 }
 
 }  // namespace mg

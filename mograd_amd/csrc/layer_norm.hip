@@ -1,4 +1,5 @@
 // C ABI for LayerNorm: argument checks and dtype dispatch.
+#include "mg_deferred.h"
 #include "mg_internal.h"
 
 namespace mg {
@@ -86,6 +87,22 @@ int mg_layer_norm_bwd_stats_add(const void* dy, const void* x, const void* gamma
   if (!mean || !rstd) return mg::fail(MG_ERR_INVALID, "layer_norm_bwd_stats_add: null statistics pointer");
   if (!residual && rows > 0) return mg::fail(MG_ERR_INVALID, "layer_norm_bwd_stats_add: null residual pointer");
   return mg::ln_bwd(dy, x, gamma, mean, rstd, residual, dx, dgamma, dbeta, rows, cols, 0.f, dtype, stream);
+}
+
+int mg_layer_norm_bwd_stats_deferred(const void* dy, const void* x, const void* gamma, const float* mean,
+                                     const float* rstd, const void* residual, void* dx, void* dgamma, void* dbeta,
+                                     int64_t rows, int64_t cols, int dtype, int grad_dtype, mg_deferred list,
+                                     mg_stream stream) {
+  if (!mean || !rstd) return mg::fail(MG_ERR_INVALID, "layer_norm_bwd_stats_deferred: null statistics pointer");
+  MG_TRY(mg::check_ln("layer_norm_bwd_stats_deferred", rows, cols, dtype));
+  MG_TRY(mg::deferred_check("layer_norm_bwd_stats_deferred", list, dtype, grad_dtype));
+  if (!dgamma || !dbeta) return mg::fail(MG_ERR_INVALID, "layer_norm_bwd_stats_deferred: null pointer argument");
+  mg::DeferredScope scope(static_cast<mg::DeferredList*>(list), dtype, grad_dtype);
+  void *dg_use, *db_use;
+  MG_TRY(scope.substitute(dgamma, cols, &dg_use));
+  MG_TRY(scope.substitute(dbeta, cols, &db_use));
+  MG_TRY(mg::ln_bwd(dy, x, gamma, mean, rstd, residual, dx, dg_use, db_use, rows, cols, 0.f, dtype, stream));
+  return scope.finish(mg::to_stream(stream));
 }
 
 }  // extern "C"

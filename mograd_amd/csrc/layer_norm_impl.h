@@ -551,8 +551,7 @@ struct LayerNormOps {
                        part_b.as<float>(), rows,
                        static_cast<int>(cols), eps, rows_per_group);
     MG_LAUNCH_CHECK();
-    launch_reduce_partials<T>(part_g.as<float>(), dgamma, part_b.as<float>(), dbeta, groups, cols,
-                              device_info().cu_count, stream);
+    reduce_partials_or_defer<T>(part_g, dgamma, &part_b, dbeta, groups, cols, device_info().cu_count, stream);
     MG_LAUNCH_CHECK();
     return MG_OK;
   }
@@ -600,8 +599,7 @@ struct LayerNormOps {
                        dim3(256), 0, stream, dy, x, stat_mean.as<float>(), stat_rstd.as<float>(), part_g.as<float>(),
                        part_b.as<float>(), rows, cols, rows_per_group);
     MG_LAUNCH_CHECK();
-    launch_reduce_partials<T>(part_g.as<float>(), dgamma, part_b.as<float>(), dbeta, groups, cols,
-                              device_info().cu_count, stream);
+    reduce_partials_or_defer<T>(part_g, dgamma, &part_b, dbeta, groups, cols, device_info().cu_count, stream);
     MG_LAUNCH_CHECK();
     return MG_OK;
   }

@@ -45,6 +45,12 @@ class Scratch {
   Scratch(const Scratch&) = delete;
   Scratch& operator=(const Scratch&) = delete;
   int take(int64_t nbytes) { return pool_take(&ptr_, nbytes); }
+  // Gives the block up without returning it to the pool: the caller now owns it.
+  void* detach() {
+    void* p = ptr_;
+    ptr_ = nullptr;
+    return p;
+  }
   template <typename T>
   T* as() const {
     return static_cast<T*>(ptr_);

@@ -3,6 +3,7 @@
 // the second stage of the two-stage column reduction.
 #pragma once
 
+#include "mg_deferred.h"
 #include "mg_device.h"
 
 namespace mg {
@@ -104,17 +105,18 @@ __device__ __forceinline__ void row_allreduce_sum(float (&v)[K], float* slots, i
 // (partials, output) pairs to reduce.
 // ------------------------------------------------------------------------------------
 
+// One workgroup's share (256 threads, `tid` of them; column block `bx`) of the sum below.
+// `tile` is SL x CW floats of LDS.  Every thread of the 256 must make the call: it holds
+// barriers.
 template <typename T, int CW>
-__global__ __launch_bounds__(256) void reduce_partials_cw_kernel(const float* __restrict__ part0, T* __restrict__ out0,
-                                                                 const float* __restrict__ part1, T* __restrict__ out1,
-                                                                 int64_t groups, int64_t cols) {
+__device__ __forceinline__ void reduce_partials_cw_block(float* __restrict__ tile_, int tid, int64_t bx,
+                                                         const float* __restrict__ part, T* __restrict__ out,
+                                                         int64_t groups, int64_t cols) {
   constexpr int SL = 256 / CW;  // row slices per workgroup
-  __shared__ float tile[SL][CW];
-  const float* part = blockIdx.y == 0 ? part0 : part1;
-  T* out = blockIdx.y == 0 ? out0 : out1;
-  const int cx = threadIdx.x % CW;
-  const int sy = threadIdx.x / CW;
-  const int64_t c = static_cast<int64_t>(blockIdx.x) * CW + cx;
+  float(&tile)[SL][CW] = *reinterpret_cast<float(*)[SL][CW]>(tile_);
+  const int cx = tid % CW;
+  const int sy = tid / CW;
+  const int64_t c = bx * CW + cx;
   float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
   if (c < cols) {
     int64_t g = sy;
@@ -137,23 +139,33 @@ __global__ __launch_bounds__(256) void reduce_partials_cw_kernel(const float* __
   if (sy == 0 && c < cols) out[c] = from_float<T>(tile[0][cx]);
 }
 
+template <typename T, int CW>
+__global__ __launch_bounds__(256) void reduce_partials_cw_kernel(const float* __restrict__ part0, T* __restrict__ out0,
+                                                                 const float* __restrict__ part1, T* __restrict__ out1,
+                                                                 int64_t groups, int64_t cols) {
+  __shared__ float tile[256];
+  reduce_partials_cw_block<T, CW>(tile, threadIdx.x, blockIdx.x, blockIdx.y == 0 ? part0 : part1,
+                                  blockIdx.y == 0 ? out0 : out1, groups, cols);
+}
+
 // The same sum for wide outputs with many groups: a 1024-thread workgroup owns 32 columns
 // (one 128-byte line of the fp32 partials) and reads them as 16-byte pieces, eight pieces
 // by 128 group lanes, so that a few hundred groups are in flight at once instead of being
 // walked four at a time; the group lanes are then added through LDS in a fixed order.
 // Needs cols % 4 == 0 and 16-byte aligned partials.
+constexpr int kSlabLanes = 128, kSlabCols = 32, kSlabSlices = 32;
+constexpr int kSlabLdsFloats = (kSlabLanes + kSlabSlices) * (kSlabCols + 1);
+// One 1024-thread workgroup's share (column block `bx`); `lds` is kSlabLdsFloats floats.
 template <typename T>
-__global__ __launch_bounds__(1024) void reduce_partials_slab_kernel(const float* __restrict__ part0, T* __restrict__ out0,
-                                                                    const float* __restrict__ part1, T* __restrict__ out1,
-                                                                    int64_t groups, int64_t cols) {
-  constexpr int LANES = 128, NCOL = 32, SL = 32;
-  __shared__ float tile[LANES][NCOL + 1];
-  __shared__ float tile2[SL][NCOL + 1];
-  const float* part = blockIdx.y == 0 ? part0 : part1;
-  T* out = blockIdx.y == 0 ? out0 : out1;
+__device__ __forceinline__ void reduce_partials_slab_block(float* __restrict__ lds, int64_t bx,
+                                                           const float* __restrict__ part, T* __restrict__ out,
+                                                           int64_t groups, int64_t cols) {
+  constexpr int LANES = kSlabLanes, NCOL = kSlabCols, SL = kSlabSlices;
+  float(&tile)[LANES][NCOL + 1] = *reinterpret_cast<float(*)[LANES][NCOL + 1]>(lds);
+  float(&tile2)[SL][NCOL + 1] = *reinterpret_cast<float(*)[SL][NCOL + 1]>(lds + LANES * (NCOL + 1));
   const int cx = threadIdx.x % 8;
   const int ly = threadIdx.x / 8;
-  const int64_t col = (static_cast<int64_t>(blockIdx.x) * 8 + cx) * 4;
+  const int64_t col = (bx * 8 + cx) * 4;
   float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0;
   if (col < cols) {
     const float* p = part + ly * cols + col;
@@ -184,12 +196,21 @@ __global__ __launch_bounds__(1024) void reduce_partials_slab_kernel(const float*
   }
   __syncthreads();
   if (threadIdx.x < NCOL) {
-    const int64_t c = static_cast<int64_t>(blockIdx.x) * NCOL + threadIdx.x;
+    const int64_t c = bx * NCOL + threadIdx.x;
     float t = 0.f;
 #pragma unroll
     for (int sl = 0; sl < SL; ++sl) t += tile2[sl][threadIdx.x];
     if (c < cols) out[c] = from_float<T>(t);
   }
+}
+
+template <typename T>
+__global__ __launch_bounds__(1024) void reduce_partials_slab_kernel(const float* __restrict__ part0, T* __restrict__ out0,
+                                                                    const float* __restrict__ part1, T* __restrict__ out1,
+                                                                    int64_t groups, int64_t cols) {
+  __shared__ float lds[kSlabLdsFloats];
+  reduce_partials_slab_block<T>(lds, blockIdx.x, blockIdx.y == 0 ? part0 : part1, blockIdx.y == 0 ? out0 : out1, groups,
+                                cols);
 }
 
 // Launches the reduction of one or two (groups, cols) partial arrays.  With at least 128
@@ -201,25 +222,58 @@ __global__ __launch_bounds__(1024) void reduce_partials_slab_kernel(const float*
 // line sit on different XCDs and each L2 fetches the line, which doubled the kernel's
 // fetched bytes at 4096 columns); a few hundred columns use 16 x 16 so that they still
 // spread over enough workgroups to hide the load latency.
+// Which form sums (groups, cols) partials: 0 the slab kernel, else the column width of
+// reduce_partials_cw_kernel.
+inline int reduce_partials_variant(const float* part0, const float* part1, int64_t groups, int64_t cols, int cu_count) {
+  const int64_t pairs = part1 ? 2 : 1;
+  const bool slab_ok = cols % 4 == 0 && groups >= 128 && aligned16(part0) && (!part1 || aligned16(part1)) &&
+                       env_int("MOGRAD_HIP_REDUCE_SLAB", 1) != 0;
+  if (slab_ok) return 0;
+  if (ceil_div(cols, 64) * pairs >= static_cast<int64_t>(cu_count)) return 64;
+  if (ceil_div(cols, 32) * pairs * 2 >= static_cast<int64_t>(cu_count)) return 32;
+  return 16;
+}
+
 template <typename T>
 inline void launch_reduce_partials(const float* part0, T* out0, const float* part1, T* out1, int64_t groups, int64_t cols,
                                    int cu_count, hipStream_t stream) {
   const unsigned pairs = part1 ? 2u : 1u;
-  const bool slab_ok = cols % 4 == 0 && groups >= 128 && aligned16(part0) && (!part1 || aligned16(part1)) &&
-                       env_int("MOGRAD_HIP_REDUCE_SLAB", 1) != 0;
-  if (slab_ok) {
+  const int variant = reduce_partials_variant(part0, part1, groups, cols, cu_count);
+  if (variant == 0) {
     hipLaunchKernelGGL((reduce_partials_slab_kernel<T>), dim3(static_cast<unsigned>(ceil_div(cols, 32)), pairs),
                        dim3(1024), 0, stream, part0, out0, part1, out1, groups, cols);
-  } else if (ceil_div(cols, 64) * pairs >= static_cast<int64_t>(cu_count)) {
+  } else if (variant == 64) {
     hipLaunchKernelGGL((reduce_partials_cw_kernel<T, 64>), dim3(static_cast<unsigned>(ceil_div(cols, 64)), pairs),
                        dim3(256), 0, stream, part0, out0, part1, out1, groups, cols);
-  } else if (ceil_div(cols, 32) * pairs * 2 >= static_cast<int64_t>(cu_count)) {
+  } else if (variant == 32) {
     hipLaunchKernelGGL((reduce_partials_cw_kernel<T, 32>), dim3(static_cast<unsigned>(ceil_div(cols, 32)), pairs),
                        dim3(256), 0, stream, part0, out0, part1, out1, groups, cols);
   } else {
     hipLaunchKernelGGL((reduce_partials_cw_kernel<T, 16>), dim3(static_cast<unsigned>(ceil_div(cols, 16)), pairs),
                        dim3(256), 0, stream, part0, out0, part1, out1, groups, cols);
   }
+}
+
+// launch_reduce_partials, unless a `_deferred` entry point is running on this thread: then the
+// sums are recorded on its list (same form, hence the same order of additions) together with
+// the partials' pool blocks, and nothing is launched here.
+template <typename T>
+inline void reduce_partials_or_defer(Scratch& part0, T* out0, Scratch* part1, T* out1, int64_t groups, int64_t cols,
+                                     int cu_count, hipStream_t stream) {
+  const float* p0 = part0.as<float>();
+  const float* p1 = part1 ? part1->as<float>() : nullptr;
+  DeferredList* dl = deferred_current();
+  if (!dl || cols > 0x7fffffffLL || groups > 0x7fffffffLL) {
+    launch_reduce_partials<T>(p0, out0, p1, out1, groups, cols, cu_count, stream);
+    return;
+  }
+  const int variant = reduce_partials_variant(p0, p1, groups, cols, cu_count);
+  const int kind = variant == 0 ? kDeferSlab : variant == 64 ? kDeferCw64 : variant == 32 ? kDeferCw32 : kDeferCw16;
+  const int64_t blocks = deferred_column_blocks(variant, cols);
+  dl->push(kind, p0, out0, 0, 0, static_cast<int>(cols), static_cast<int>(groups), blocks);
+  if (p1) dl->push(kind, p1, out1, 0, 0, static_cast<int>(cols), static_cast<int>(groups), blocks);
+  dl->hold(part0);
+  if (part1) dl->hold(*part1);
 }
 
 }  // namespace mg

@@ -18,11 +18,16 @@ mg_cross_entropy_fused_ids, mg_scatter_add for the embedding; in the forward the
 that feed them (mg_matmul_bt_add, mg_matmul_bias_relu_bt).
 
 Mixed precision: the parameters live in one fp32 arena (master weights); each step casts
-the whole arena once to the compute dtype (bf16 by default), runs every kernel in that
-dtype with fp32 accumulation, writes the weight gradients into a compute-dtype arena of
-the same layout and casts that once to an fp32 gradient arena.  All activations and
-temporaries are allocated once per (batch, context) shape, so a step performs no
-allocation.  This module contains no arithmetic; there is no CPU fallback.
+the whole arena once to the compute dtype (bf16 by default) and runs every kernel in that
+dtype with fp32 accumulation.  The parameter gradients are sums of fp32 partial results
+(the K ranges of a split dW, the row groups of dgamma/dbeta, the slabs of the embedding
+gradient) that nothing in the backward pass reads, so the step records them on an
+mg_deferred list and one launch at its end (mg_finish_deferred) writes them all, in fp32,
+straight into the gradient arena: no 16-bit rounding of the weight gradients and no cast.
+`deferred=False` keeps the earlier sequence (each sum where it arises, gradients rounded to
+the compute dtype in an arena of their own, one cast to fp32), which the tests compare with.
+All activations and temporaries are allocated once per (batch, context) shape.  This module
+contains no arithmetic; there is no CPU fallback.
 """
 from __future__ import annotations
 
@@ -51,7 +56,7 @@ class _Slice:
 
 class TinyTransformer:
     def __init__(self, device: Device, vocab_size: int, d_model: int, d_ff: int, n_layers: int, n_heads: int,
-                 compute_dtype: int = BF16, eps: float = 1e-5):
+                 compute_dtype: int = BF16, eps: float = 1e-5, deferred: bool = True):
         if d_model % n_heads:
             raise MogradError(1, "d_model must be a multiple of n_heads")
         self.device, self.lib, self.stream = device, device.lib, device.stream
@@ -59,6 +64,7 @@ class TinyTransformer:
         self.dh = d_model // n_heads
         self.cd = compute_dtype
         self.eps = eps
+        self.deferred = deferred
         self.slices: Dict[str, _Slice] = {}
         off = 0
 
@@ -86,8 +92,16 @@ class TinyTransformer:
         self.master = AnyBuffer.create(F32, device, self.total, fill=0.0)  # fp32 master weights
         self.grads = AnyBuffer.create(F32, device, self.total, fill=0.0)   # fp32 gradients, same layout
         self.work = AnyBuffer.create(self.cd, device, self.total)          # weights in the compute dtype
-        self.wgrad = AnyBuffer.create(self.cd, device, self.total, fill=0.0)
+        self.wgrad = None if deferred else AnyBuffer.create(self.cd, device, self.total, fill=0.0)
+        self.pending = C.c_void_p()
+        if deferred:
+            self.lib.mg_deferred_create(C.byref(self.pending))
         self._plan_key = None
+
+    def __del__(self):
+        if getattr(self, "pending", None):
+            self.lib.mg_deferred_destroy(self.pending)
+            self.pending = None
 
     # ------------------------------------------------------------------ parameters
 
@@ -122,6 +136,10 @@ class TinyTransformer:
         return C.c_void_p(self.work.storage.ptr + self.slices[name].offset * DTYPE_SIZE[self.cd])
 
     def _g(self, name: str) -> C.c_void_p:
+        """Where a parameter's gradient is written: the fp32 arena (deferred sums) or the
+        compute-dtype one."""
+        if self.deferred:
+            return C.c_void_p(self.grads.storage.ptr + self.slices[name].offset * 4)
         return C.c_void_p(self.wgrad.storage.ptr + self.slices[name].offset * DTYPE_SIZE[self.cd])
 
     # ------------------------------------------------------------------ workspace
@@ -204,29 +222,45 @@ class TinyTransformer:
 
         # ---- backward
         t = {k: P(v) for k, v in self.tmp.items()}
-        lib.mg_linear_bwd(t["dlogits"], P(self.h[self.L]), self._w("lm_head"), t["dh"], self._g("lm_head"), None, n, V,
-                          d, cd, s)
+        if self.deferred:
+            q = self.pending
+
+            def lin_bwd(dy, x, w, dx, dw, db, N, K, accumulate=0, relu=0):
+                lib.mg_linear_bwd_deferred(dy, x, w, dx, dw, db, n, N, K, accumulate, relu, cd, F32, q, s)
+
+            def ln_bwd(dy, x, gam, mean, rstd, dg, db):  # dh += LayerNorm backward
+                lib.mg_layer_norm_bwd_stats_deferred(dy, x, gam, mean, rstd, t["dh"], t["dh"], dg, db, n, d, cd, F32, q, s)
+        else:
+            def lin_bwd(dy, x, w, dx, dw, db, N, K, accumulate=0, relu=0):
+                lib.mg_linear_bwd_fused(dy, x, w, dx, dw, db, n, N, K, accumulate, relu, cd, s)
+
+            def ln_bwd(dy, x, gam, mean, rstd, dg, db):
+                lib.mg_layer_norm_bwd_stats_add(dy, x, gam, mean, rstd, t["dh"], t["dh"], dg, db, n, d, cd, s)
+
+        lin_bwd(t["dlogits"], P(self.h[self.L]), self._w("lm_head"), t["dh"], self._g("lm_head"), None, V, d)
         for l in reversed(range(self.L)):
             c = self.saved[l]
             w = lambda name, l=l: self._w(f"blocks.{l}.{name}")
             g = lambda name, l=l: self._g(f"blocks.{l}.{name}")
-            # h_out = h_mid + W2 a
-            lib.mg_linear_bwd_fused(t["dh"], P(c["a"]), w("w2"), t["da"], g("w2"), None, n, d, ff, 0, 1, cd, s)
-            lib.mg_linear_bwd(t["da"], P(c["x2"]), w("w1"), t["dx_a"], g("w1"), g("b1"), n, ff, d, cd, s)
+            # h_out = h_mid + W2 a; the ReLU's gradient rides on the dX product
+            lin_bwd(t["dh"], P(c["a"]), w("w2"), t["da"], g("w2"), None, d, ff, relu=1)
+            lin_bwd(t["da"], P(c["x2"]), w("w1"), t["dx_a"], g("w1"), g("b1"), ff, d)
             # dh += LayerNorm backward: the skip connection's share is already in dh
-            lib.mg_layer_norm_bwd_stats_add(t["dx_a"], P(c["h_mid"]), w("ln2_g"), P(c["mean2"]), P(c["rstd2"]), t["dh"],
-                                            t["dh"], g("ln2_g"), g("ln2_b"), n, d, cd, s)
+            ln_bwd(t["dx_a"], P(c["h_mid"]), w("ln2_g"), P(c["mean2"]), P(c["rstd2"]), g("ln2_g"), g("ln2_b"))
             # h_mid = h_in + W_O ctx
-            lib.mg_linear_bwd(t["dh"], P(c["ctx"]), w("wo"), t["dctx"], g("wo"), None, n, d, d, cd, s)
+            lin_bwd(t["dh"], P(c["ctx"]), w("wo"), t["dctx"], g("wo"), None, d, d)
             # dctx and ctx are (B, T, H, dh); dQ | dK | dV come back as one (n, 3d) tensor
             lib.mg_flash_attn_bwd_packed(t["dctx"], P(c["ctx"]), P(c["qkv"]), None, P(c["lse"]), t["dqkv"], B, T, H, dh,
                                          scale, 1, 0, cd, s)
             # gradient of the stacked projection: dx1 (n, d) and dW (3d, d) = dwq | dwk | dwv
-            lib.mg_linear_bwd(t["dqkv"], P(c["x1"]), w("wq"), t["dx_a"], g("wq"), None, n, 3 * d, d, cd, s)
-            lib.mg_layer_norm_bwd_stats_add(t["dx_a"], P(self.h[l]), w("ln1_g"), P(c["mean1"]), P(c["rstd1"]), t["dh"],
-                                            t["dh"], g("ln1_g"), g("ln1_b"), n, d, cd, s)
-        lib.mg_scatter_add(P(ids), t["dh"], self._g("embed"), n, V, d, ids.dtype, cd, s)
-        lib.mg_cast(P(self.wgrad), P(self.grads), self.total, cd, F32, s)
+            lin_bwd(t["dqkv"], P(c["x1"]), w("wq"), t["dx_a"], g("wq"), None, 3 * d, d)
+            ln_bwd(t["dx_a"], P(self.h[l]), w("ln1_g"), P(c["mean1"]), P(c["rstd1"]), g("ln1_g"), g("ln1_b"))
+        if self.deferred:
+            lib.mg_scatter_add_deferred(P(ids), t["dh"], self._g("embed"), n, V, d, ids.dtype, cd, F32, self.pending, s)
+            lib.mg_finish_deferred(self.pending, s)
+        else:
+            lib.mg_scatter_add(P(ids), t["dh"], self._g("embed"), n, V, d, ids.dtype, cd, s)
+            lib.mg_cast(P(self.wgrad), P(self.grads), self.total, cd, F32, s)
         if marks:
             marks("backward")
         return self.loss

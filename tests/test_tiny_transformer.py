@@ -132,3 +132,50 @@ def test_training_reduces_the_loss(device):
         model.adam_step(lr=3e-3, weight_decay=0.01, decoupled=True)
     last = loss.item()
     assert first > math.log(V) - 0.5 and last < 0.5 * first, (first, last)
+
+
+@pytest.mark.parametrize("V,d,ff,L,H,B,T", [(65, 128, 512, 2, 2, 8, 128), (65, 384, 1536, 2, 6, 16, 256)])
+def test_deferred_sums_equal_the_immediate_sequence(device, V, d, ff, L, H, B, T):
+    # The default step leaves every parameter gradient's second-stage sum to one launch at its
+    # end and writes it in fp32; `deferred=False` sums where the partial results arise, rounds to
+    # bf16 and casts.  Same kernels and same order of additions: the fp32 gradients, rounded to
+    # bf16, are the other sequence's bit for bit, and so are the loss and the activations' path.
+    rng = np.random.Generator(np.random.PCG64(73_000 + d))
+    params = _perturb_norms(init_params(rng, V, d, ff, L), rng)
+    ids = AnyBuffer.from_numpy(device, integers(73, 1, (B, T), 0, V, np.int32))
+    labels = AnyBuffer.from_numpy(device, integers(73, 2, (B, T), 0, V, np.int32))
+    grads, losses = [], []
+    for deferred in (True, False):
+        model = TinyTransformer(device, V, d, ff, L, H, deferred=deferred)
+        model.load_params(params)
+        losses.append(model.step(ids, labels, B, T).item())
+        grads.append(_flatten(model.gradients()))
+    assert losses[0] == losses[1]
+    for name, g32 in grads[0].items():
+        np.testing.assert_array_equal(round_to_dtype(g32, BF16), grads[1][name], err_msg=name)
+        assert (g32 != grads[1][name]).any(), f"{name}: the fp32 sums carry bits that bf16 drops"
+
+
+def test_weight_gradient_at_fp32_precision(device):
+    # With fp32 parameter gradients the only 16-bit roundings left in dW are those of its
+    # operands.  For the first block's MLP input layer the operands of the last backward launch
+    # are still in the step's buffers (dY in `da`, X in the saved LayerNorm output): dW1 and db1
+    # must equal their float64 products to fp32-accumulation accuracy, not to bf16's.
+    V, d, ff, L, H, B, T = 65, 384, 1536, 2, 6, 16, 256
+    rng = np.random.Generator(np.random.PCG64(74_000))
+    model = TinyTransformer(device, V, d, ff, L, H)
+    model.load_params(init_params(rng, V, d, ff, L))
+    ids = AnyBuffer.from_numpy(device, integers(74, 1, (B, T), 0, V, np.int32))
+    labels = AnyBuffer.from_numpy(device, integers(74, 2, (B, T), 0, V, np.int32))
+    model.step(ids, labels, B, T)
+    g = model.gradients()["blocks"][0]
+    n = B * T
+    dy = model.tmp["da"].to_numpy((n, ff)).astype(np.float64)
+    x = model.saved[0]["x2"].to_numpy((n, d)).astype(np.float64)
+    want_w, want_b = dy.T @ x, dy.sum(axis=0)
+    mass_w, mass_b = np.abs(dy).T @ np.abs(x), np.abs(dy).sum(axis=0)
+    # 2^-24 per addition against the mass summed; bf16 rounding of the result would be 2^-9 of it
+    assert np.abs(g["w1"] - want_w).max() <= 32 * 2.0 ** -24 * mass_w.max()
+    assert (np.abs(g["w1"] - want_w) <= 32 * 2.0 ** -24 * mass_w + 1e-12).all()
+    assert (np.abs(g["b1"] - want_b) <= 32 * 2.0 ** -24 * mass_b + 1e-12).all()
+    assert np.abs(round_to_dtype(g["w1"], BF16) - g["w1"]).max() > 0, "dW1 is not a bf16-rounded value"
