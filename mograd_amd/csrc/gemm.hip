@@ -109,6 +109,12 @@ static int launch_f32_mfma(const GemmArgs& g, hipStream_t stream) {
 
 static bool mult8(int64_t v) { return (v & 7) == 0; }
 
+// gemm_big.hip: the 256 x 256-tile kernel for large 16-bit products (variant 4ksn: k per step,
+// copies of the tiles).
+int gemm16_big_launch(int dtype, bool a_kc, bool b_kc, int variant, const void* a, const void* b, const void* bias,
+                      void* c, int64_t batch, int M, int N, int K, int64_t lda, int64_t ldb, int64_t bsa, int64_t bsb,
+                      const void* residual, const void* relu_mask, int relu, hipStream_t stream);
+
 // Into how many K ranges a 16-bit product of `blocks` output tiles is split (1: not at all):
 // enough for `wg_per_cu` workgroups per CU, each with at least 256 of K.
 static int splitk_16bit_splits(int64_t blocks, int64_t K, int wg_per_cu) {
@@ -162,9 +168,19 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
       // Large products: 256 x 128 tiles (eight waves), a quarter fewer operand bytes per FLOP
       // through L2, once they still give every CU two workgroups (4096^3: 3-11 % faster).
       if (splits <= 1 && g.K >= 1024 && ceil_div(g.M, 256) * tiles_n * g.batch >= 2 * cus) pipe = 2322;
+      // Products with a 256 x 256 tile for every CU: four waves of 128 x 128 each, one workgroup
+      // per CU (gemm_16bit_big_kernel; 4642: 64 k per step and two copies of the tiles, 4324: 32 k
+      // and four; 4096^3 forward 147 -> 121 us, 8192^3 dW 1016 -> 887 us, bit-identical results).
+      if (splits <= 1 && g.K >= 1024 && ceil_div(g.M, kGemmBigT) * ceil_div(g.N, kGemmBigT) * g.batch >= cus) pipe = 4642;
       pipe = static_cast<int>(env_int("MOGRAD_HIP_GEMM16_PIPE", pipe));
     }
   }
+  if (splits <= 1 && pipe >= 4000) {
+    if constexpr (!RAGGED)
+      return gemm16_big_launch(g.dtype, A_KC, B_KC, pipe, g.a, g.b, g.bias, g.c, g.batch, M, N, K, lda, ldb, g.bsa, g.bsb,
+                               g.residual, g.relu_mask, g.relu, stream);
+  }
+  if (pipe >= 4000) pipe = 322;
 #define MG_GEMM16_LAUNCH(BIAS_, SPLIT_, GRID_, PARTIAL_, KPS_, NSPLIT_, EP_)                                                   \
   do {                                                                                                                 \
     auto launch = [&](auto kernel) {                                                                                   \

@@ -1011,6 +1011,170 @@ __global__ __launch_bounds__(TM * 2, gemm16_pipe_occupancy(BK, NSTAGE, TM)) void
   gemm16_pipe_block<T, A_KC, B_KC, HAS_BIAS, SPLIT_K, BK, NSTAGE, TM>(lds, blockIdx.x, pr);
 }
 
+// ------------------------------------------------------------------------------------
+// Large products: 256 x 256 output tile per workgroup of four waves, one wave per SIMD, each
+// wave a 128 x 128 tile as 4 x 4 v_mfma_f32_32x32x16 accumulators (256 accumulator registers
+// of the 512 a lone wave may use).  A k-slice of 16 takes four A and four B fragments for
+// sixteen MFMAs, i.e. half a kilobyte of LDS reads per MFMA where the 64 x 64 wave tile of
+// the kernels above needs a whole one: with four SIMDs issuing MFMAs back to back those
+// kernels ask the LDS for exactly its 128 bytes per clock, this one for half of that, and a
+// 256 x 256 tile also halves the operand bytes a FLOP pulls through L2.  The price is one
+// workgroup per CU: no second wave hides a wait, so the fragments of slice ks + 1 are read
+// while slice ks is multiplied and the tiles are copied NSTAGE steps ahead.  Taken for
+// products with at least one such tile per CU; tiles, copy and LDS images are those of
+// gemm16_pipe_block, and so is the order of every sum (results are bit-identical).
+// 8192^3 bf16 forward / dX / dW: 1.26 / 1.11 / 1.02 ms with 256 x 128 tiles of 64 x 64 wave
+// tiles -> 1.06 / 0.95 / 0.89 ms; matrix pipe busy 64 % of the CU-busy cycles (44-49 % before).
+// With the copies compiled out the same loop takes 0.79 / 0.73 / 0.70 ms, with the MFMAs
+// compiled out 0.63-0.72 / 0.63 / 0.57-0.64 ms: the L2 -> LDS copy of 8.6 GB per launch is as
+// long as the arithmetic and the two do not overlap fully.
+// ------------------------------------------------------------------------------------
+constexpr int kGemmBigT = 256;
+constexpr int gemm16_big_lds_bytes(int bk, int nstage) {
+  const int stages = nstage * 2 * kGemmBigT * bk * 2;
+  const int out = 4 * 64 * kG16Stride * 2;
+  return stages > out ? stages : out;
+}
+
+template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, int BK, int NSTAGE>
+__global__ __launch_bounds__(256, 1) void gemm_16bit_big_kernel(
+    const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C, int M, int N, int K,
+    int64_t lda, int64_t ldb, int64_t ldc, int64_t bsa, int64_t bsb, int64_t bsc, int tiles_m, int tiles_n,
+    GemmEpilogue<T> ep) {
+  static_assert(NSTAGE >= 2 && NSTAGE <= 4 && (BK == 32 || BK == 64), "stages");
+  constexpr int TT = kGemmBigT, NW = 4;
+  constexpr int NI = gemm16_pipe_requests(TT, BK, NW);  // copy requests per thread, operand and step
+  constexpr int OPB = TT * BK * 2;                      // bytes of an operand's step
+  constexpr int OP = 2 * OPB;
+  __shared__ __attribute__((aligned(1024))) char lds[gemm16_big_lds_bytes(BK, NSTAGE)];
+
+  const int tiles = tiles_m * tiles_n;
+  const int batch = blockIdx.x / tiles, tile = blockIdx.x % tiles;
+  int tm, tn;
+  gemm_tile_of_block(tile, tiles_m, tiles_n, tm, tn, true);
+  const int m0 = tm * TT, n0 = tn * TT;
+  const int steps = K / BK;
+  A += batch * bsa;
+  B += batch * bsb;
+  const int64_t a_step = A_KC ? BK : BK * lda;
+  const int64_t b_step = B_KC ? BK : BK * ldb;
+
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int wm = (wave / 2) * 128;
+  const int wn = (wave % 2) * 128;
+
+  floatx16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const uint16_t* a16 = reinterpret_cast<const uint16_t*>(A);
+  const uint16_t* b16 = reinterpret_cast<const uint16_t*>(B);
+  int64_t src_a[NI], src_b[NI];
+  gemm16_pipe_sources<A_KC, BK, TT, NW>(lda, m0, M, src_a);
+  gemm16_pipe_sources<B_KC, BK, TT, NW>(ldb, n0, N, src_b);
+  auto request = [&](int step, int copy) {
+    gemm16_pipe_issue<NI, NW>(a16 + step * a_step, src_a, lds + copy * OP);
+    gemm16_pipe_issue<NI, NW>(b16 + step * b_step, src_b, lds + copy * OP + OPB);
+  };
+
+  // The k loop is one stream of 16-deep slices.  While the sixteen MFMAs of a slice run, the
+  // eight fragments of the next slice are read into the other half of `f` (the reads are dealt
+  // out between the MFMAs with sched_group_barrier: left to itself the compiler reads each
+  // fragment right before its use and waits for it).  Before the last slice of a step comes
+  // the step's one synchronisation: the data of the next step has arrived (all but the
+  // NSTAGE - 2 younger steps' copies), no wave reads the current step's tiles any more (their
+  // last fragments are in registers), so the copy of step it + NSTAGE may overwrite them.
+  constexpr int NS = BK / 16;
+  constexpr int RA = A_KC ? 1 : 2, RB = B_KC ? 1 : 2;  // LDS reads per fragment
+  uint4 f[2][8];
+  auto read_frags = [&](int buf, int step, int ks) {  // B first: every MFMA group needs all four
+    const char* la = lds + (step % NSTAGE) * OP;
+    const char* lb = la + OPB;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[buf][4 + i] = gemm16_pipe_frag<B_KC, BK, TT>(lb, wn + 32 * i, ks, lane);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[buf][i] = gemm16_pipe_frag<A_KC, BK, TT>(la, wm + 32 * i, ks, lane);
+  };
+  auto multiply = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = GemmMma16<T>::run(f[buf][i], f[buf][4 + j], acc[i][j]);
+  };
+  // Slice ks of step `it`.  MODE 0: steady state (a copy is requested at the step's
+  // synchronisation, the next step exists); 1: the product's last steps (nothing left to
+  // request, every copy is waited for); 2: the very last slice (nothing left to read either).
+  auto slice = [&](int it, int ks, auto mode) {
+    constexpr int MODE = decltype(mode)::value;
+    const int buf = ks % 2;
+    if (ks == NS - 1) {
+      if constexpr (MODE != 0 || NSTAGE == 2) MG_WAIT_VMCNT(0);
+      else MG_WAIT_VMCNT(2 * NI * (NSTAGE - 2));
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      if constexpr (MODE == 0) request(it + NSTAGE, it % NSTAGE);
+      if constexpr (MODE != 2) read_frags(buf ^ 1, it + 1, 0);
+    } else {
+      read_frags(buf ^ 1, it, ks + 1);
+    }
+    multiply(buf);
+    if constexpr (MODE != 2) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {  // four groups of (4 MFMAs, a quarter of the reads)
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, RA + RB, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  static_assert(NS % 2 == 0, "a step ends on the second fragment buffer");
+#pragma unroll
+  for (int s = 0; s < NSTAGE; ++s)
+    if (s < steps) request(s, s);
+  if (steps > NSTAGE - 1) MG_WAIT_VMCNT(2 * NI * (NSTAGE - 1));
+  else MG_WAIT_VMCNT(0);
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  read_frags(0, 0, 0);
+  // The loop body starts at a step's synchronisation (where nothing is outstanding anyway, so
+  // what the compiler assumes at a loop head costs nothing) and runs on through the first
+  // slices of the next step.
+#pragma unroll
+  for (int ks = 0; ks < NS - 1; ++ks) slice(0, ks, std::integral_constant<int, 0>{});
+  int it = 0;
+  for (; it < steps - NSTAGE; ++it) {
+    slice(it, NS - 1, std::integral_constant<int, 0>{});
+#pragma unroll
+    for (int ks = 0; ks < NS - 1; ++ks) slice(it + 1, ks, std::integral_constant<int, 0>{});
+  }
+  for (; it < steps - 1; ++it) {
+    slice(it, NS - 1, std::integral_constant<int, 1>{});
+#pragma unroll
+    for (int ks = 0; ks < NS - 1; ++ks) slice(it + 1, ks, std::integral_constant<int, 1>{});
+  }
+  slice(steps - 1, NS - 1, std::integral_constant<int, 2>{});
+  __syncthreads();  // every wave is done with the staged tiles: their memory serves the output
+
+  // The wave's 128 x 128 tile goes out as four 64 x 64 quadrants through its own strip of LDS.
+  uint16_t* mine = reinterpret_cast<uint16_t*>(lds) + wave * 64 * kG16Stride;
+#pragma unroll
+  for (int qi = 0; qi < 2; ++qi)
+#pragma unroll
+    for (int qj = 0; qj < 2; ++qj) {
+      floatx16 quad[2][2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) quad[i][j] = acc[2 * qi + i][2 * qj + j];
+      gemm16_write_tile<T, HAS_BIAS, false>(quad, mine, bias, C, nullptr, M, N, ldc, bsc, batch, 0, 1, m0, n0,
+                                            wm + 64 * qi, wn + 64 * qj, lane, ep);
+      __syncthreads();  // the strip is read out before the next quadrant is written into it
+    }
+}
+
 // Both products of a Linear layer's backward in one launch: workgroups [0, n_dw) take the
 // K ranges of dW = dY^T X (their partial tiles are summed by linear_bwd_finish_kernel
 // afterwards), the rest the tiles of dX = dY W.  The longer-running dW ranges start first

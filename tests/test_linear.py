@@ -354,7 +354,7 @@ def test_half_precision_mfma_paths(device, dtype, rtol, M, N, K):
 def test_tile_staging_variants_agree(device, monkeypatch, dtype, rtol, M, N, K):
     # The 16-bit products have a register-staged kernel (0) and one whose tiles are copied
     # straight into LDS, 32 or 64 k per step (322, 642), also with 256 x 128 output tiles
-    # (2322, 2642); the library picks by operand layout, K and size.  All accumulate each output element over k in the same order on the same MFMA,
+    # (2322, 2642) or 256 x 256 tiles of 128 x 128 wave tiles (4324, 4642); the library picks by operand layout, K and size.  All accumulate each output element over k in the same order on the same MFMA,
     # so forcing either must not change a bit, for every operand layout (forward k/k, dX
     # k/n, dW m/n, the last split along K for the tall shapes) and at ragged tile edges.
     x = round_to_dtype(normal(49, 0, (M, K)), dtype)
@@ -362,12 +362,12 @@ def test_tile_staging_variants_agree(device, monkeypatch, dtype, rtol, M, N, K):
     b = round_to_dtype(normal(49, 2, (N,), std=0.1), dtype)
     dy = round_to_dtype(normal(49, 3, (M, N), std=0.5), dtype)
     results = {}
-    for variant in ("0", "322", "642", "2322", "2642"):
+    for variant in ("0", "322", "642", "2322", "2642", "4324", "4642"):
         monkeypatch.setenv("MOGRAD_HIP_GEMM16_PIPE", variant)
         results[variant] = _linear_all(device, x, w, b, dy, dtype)
     monkeypatch.delenv("MOGRAD_HIP_GEMM16_PIPE")
     results["auto"] = _linear_all(device, x, w, b, dy, dtype)
-    for variant in ("322", "642", "2322", "2642", "auto"):
+    for variant in ("322", "642", "2322", "2642", "4324", "4642", "auto"):
         for got, base, name in zip(results[variant], results["0"], ("y", "dx", "dw", "db")):
             np.testing.assert_array_equal(got, base, err_msg=f"{name}, variant {variant}")
     y, dx, dw, _ = results["auto"]
@@ -441,11 +441,11 @@ def test_f32_tile_staging_variants_agree(device, monkeypatch, M, N, K):
     assert_sum_close(got[2], O.linear_grad_w(dy, x), np.abs(dy).T @ np.abs(x), what="dw")
 
 
-def test_large_products_agree_with_the_register_staged_kernel(device, monkeypatch):
-    # A product large enough that the library picks 256 x 128 tiles by itself (K >= 1024 and
-    # two such tiles per CU) must equal the register-staged kernel's result bit for bit, for
-    # the forward and both gradient layouts.
-    M, N, K = 8192, 2048, 1024
+@pytest.mark.parametrize("M,N,K", [(8192, 2048, 1024), (4104, 4000, 1088), (2048, 8192, 2048)])
+def test_large_products_agree_with_the_register_staged_kernel(device, monkeypatch, M, N, K):
+    # A product large enough that the library picks 256 x 256 tiles by itself (K >= 1024 and
+    # a tile for every CU) must equal the register-staged kernel's result bit for bit, for
+    # the forward and both gradient layouts, also with ragged last tiles in both directions.
     x = round_to_dtype(normal(58, 0, (M, K)), BF16)
     w = round_to_dtype(normal(58, 1, (N, K), std=0.05), BF16)
     dy = round_to_dtype(normal(58, 2, (M, N), std=0.5), BF16)
@@ -464,7 +464,7 @@ def test_large_products_agree_with_the_register_staged_kernel(device, monkeypatc
     for got, want, name in zip(auto, base, ("y", "dx", "dw")):
         np.testing.assert_array_equal(got, want, err_msg=name)
     # and a spot check of the forward against float64 on a few rows
-    rows = [0, 257, 4095, 8191]
+    rows = [0, 257, M // 2 - 1, M - 1]
     want = x[rows].astype(np.float64) @ w.astype(np.float64).T
     assert_close(auto[0][rows], want, 1.6e-2, 1.6e-2 * np.abs(want).max(), "y rows")
 
