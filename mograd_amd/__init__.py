@@ -6,6 +6,7 @@ Importing the package does not load the library; constructing a `Device` does, a
 if it is missing.
 """
 from ._lib import BF16, F16, F32, I32, I64, LibraryMissing, MogradError, load  # noqa: F401
-from .runtime import GRAD_RULES, SCHEDULER_RULES, AnyBuffer, Device, Layout, Node, evaluate, gradient, run  # noqa: F401
+from .runtime import (GRAD_RULES, SCHEDULER_RULES, AnyBuffer, Device, Layout, Node, evaluate, evaluate_many,  # noqa: F401
+                      gradient, run)
 
 __version__ = "0.1"

@@ -26,6 +26,7 @@
 #include <cstdint>
 #include <cstdlib>
 #include <map>
+#include <optional>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -168,6 +169,9 @@ class Device {
   }
 
   mg_stream stream() const { return stream_; }
+  // While set (DeferredSums below), the exec functions of LINEAR_GRAD, LAYER_NORM_STATS_GRAD(_ADD)
+  // and SCATTER_ADD leave their second-stage sums on this list.
+  mg_deferred pending = nullptr;
   void synchronize() { check(fn<decltype(&::mg_stream_sync)>("mg_stream_sync")(stream_)); }  // ctx.synchronize()
   void empty_cache() { check(fn<decltype(&::mg_pool_empty_cache)>("mg_pool_empty_cache")()); }
   mg_pool_stats memory_stats() {
@@ -237,6 +241,7 @@ class AnyBuffer {
   void* data_ptr() const { return static_cast<char*>(storage_->ptr()) + offset_elems_ * dtype_size(dtype_); }
   DType dtype() const { return dtype_; }
   int64_t numel() const { return numel_; }
+  int64_t offset_elems() const { return offset_elems_; }
   // Shares storage; the element count and base offset come from `layout`.
   AnyBuffer view(const Layout& layout) const {
     AnyBuffer b = *this;
@@ -275,6 +280,9 @@ struct OpRef {
   }
   static OpRef leaf(const Layout& layout, DType dtype = float32) { return OpRef{"BUFFER", layout, dtype, {}, {}}; }
 };
+
+// Value of a FLASH_ATTN / FLASH_ATTN_GRAD node's "layout" attribute when O and dO are (B, S, H, D).
+constexpr double kLayoutBshd = 1.0;
 
 using Buffers = std::vector<AnyBuffer>;
 using BoundExecFn = Buffers (*)(const OpRef& node, const Buffers& inputs, Device& device);
@@ -363,9 +371,15 @@ inline Buffers flash_attn_fwd_sched(const OpRef& node, const Buffers& inputs, De
   detail::require_float(node.dtype(), "flash_attn_fwd");
   AnyBuffer dst = AnyBuffer::create(node.dtype(), device, node.numel());
   AnyBuffer lse = AnyBuffer::create(float32, device, B * H * S);
-  MOGRAD_CALL(device, mg_flash_attn_fwd, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
-              inputs[3].data_ptr(), dst.data_ptr(), static_cast<float*>(lse.data_ptr()), B, S, H, D,
-              static_cast<float>(node.attr("scale")), is_causal, has_bias, node.dtype(), device.stream());
+  // {layout: kLayoutBshd} (set by fuse_attention_output_layout): O is written (B, S, H, D) like Q
+  if (node.has_attr("layout") && node.attr("layout") == kLayoutBshd)
+    MOGRAD_CALL(device, mg_flash_attn_fwd_bshd, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+                inputs[3].data_ptr(), dst.data_ptr(), static_cast<float*>(lse.data_ptr()), B, S, H, D,
+                static_cast<float>(node.attr("scale")), is_causal, has_bias, node.dtype(), device.stream());
+  else
+    MOGRAD_CALL(device, mg_flash_attn_fwd, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+                inputs[3].data_ptr(), dst.data_ptr(), static_cast<float*>(lse.data_ptr()), B, S, H, D,
+                static_cast<float>(node.attr("scale")), is_causal, has_bias, node.dtype(), device.stream());
   return {dst, lse};
 }
 
@@ -380,10 +394,16 @@ inline Buffers flash_attn_bwd_sched(const OpRef& node, const Buffers& inputs, De
   AnyBuffer dq = AnyBuffer::create(node.dtype(), device, q.numel());
   AnyBuffer dk = AnyBuffer::create(node.dtype(), device, q.numel());
   AnyBuffer dv = AnyBuffer::create(node.dtype(), device, q.numel());
-  MOGRAD_CALL(device, mg_flash_attn_bwd, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
-              inputs[3].data_ptr(), inputs[4].data_ptr(), inputs[5].data_ptr(),
-              static_cast<const float*>(inputs[6].data_ptr()), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, S, H, D,
-              static_cast<float>(node.attr("scale")), is_causal, has_bias, node.dtype(), device.stream());
+  if (node.has_attr("layout") && node.attr("layout") == kLayoutBshd)
+    MOGRAD_CALL(device, mg_flash_attn_bwd_bshd, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+                inputs[3].data_ptr(), inputs[4].data_ptr(), inputs[5].data_ptr(),
+                static_cast<const float*>(inputs[6].data_ptr()), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, S, H, D,
+                static_cast<float>(node.attr("scale")), is_causal, has_bias, node.dtype(), device.stream());
+  else
+    MOGRAD_CALL(device, mg_flash_attn_bwd, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+                inputs[3].data_ptr(), inputs[4].data_ptr(), inputs[5].data_ptr(),
+                static_cast<const float*>(inputs[6].data_ptr()), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, S, H, D,
+                static_cast<float>(node.attr("scale")), is_causal, has_bias, node.dtype(), device.stream());
   return {dq, dk, dv};
 }
 
@@ -534,8 +554,13 @@ inline Buffers scatter_add(const OpRef& node, const Buffers& inputs, Device& dev
     throw Error(MG_ERR_INVALID, "scatter_add expects values shaped [*indices.shape, row_size]");
   const Buffers in = detail::materialise(node, inputs, device, 2);
   AnyBuffer out = AnyBuffer::create(node.dtype(), device, node.numel());
-  MOGRAD_CALL(device, mg_scatter_add, in[0].data_ptr(), in[1].data_ptr(), out.data_ptr(), la.numel(), node.shape(0),
-              lb.shape(lb.rank() - 1), node.src(0).dtype(), node.dtype(), device.stream());
+  if (device.pending)
+    MOGRAD_CALL(device, mg_scatter_add_deferred, in[0].data_ptr(), in[1].data_ptr(), out.data_ptr(), la.numel(),
+                node.shape(0), lb.shape(lb.rank() - 1), node.src(0).dtype(), node.dtype(), node.dtype(), device.pending,
+                device.stream());
+  else
+    MOGRAD_CALL(device, mg_scatter_add, in[0].data_ptr(), in[1].data_ptr(), out.data_ptr(), la.numel(), node.shape(0),
+                lb.shape(lb.rank() - 1), node.src(0).dtype(), node.dtype(), device.stream());
   return {out};
 }
 
@@ -581,16 +606,21 @@ inline Buffers argmax(const OpRef& node, const Buffers& inputs, Device& device) 
 // (mograd/runtime/__init__.mojo:425-426) and its labels are dense.  They follow the pattern of
 // its multi-output FLASH_ATTN / FLASH_ATTN_GRAD pair (mograd/grad.mojo:309-344).
 
-// LINEAR_GRAD[dY (.., N), X (.., K), W (N, K)]{has_bias} -> [dX, dW (N, K), db (N)] for Y = X W^T (+ b).
+// LINEAR_GRAD[dY (.., N), X (.., K), W (N, K)(, prior)]{has_bias, relu_mask, accumulate} -> [dX, dW (N, K), db (N)]
+// for Y = X W^T (+ b).  relu_mask: X is a ReLU's output and dX is zeroed where X <= 0; accumulate: dX = prior + dY W.
 inline Buffers linear_bwd(const OpRef& node, const Buffers& in, Device& device) {
   const Layout &ldy = node.src(0).layout(), &lx = node.src(1).layout(), &lw = node.src(2).layout();
-  const Buffers inputs = detail::materialise(node, in, device, 3);
+  const bool accumulate = node.has_attr("accumulate") && node.attr("accumulate") != 0;
+  const bool relu_mask = node.has_attr("relu_mask") && node.attr("relu_mask") != 0;
+  const Buffers inputs = detail::materialise(node, in, device, accumulate ? 4 : 3);
   detail::require_float(node.dtype(), "linear_bwd");
   if (lw.rank() != 2) throw Error(MG_ERR_INVALID, "linear_bwd: dY, X and W do not describe Y = X W^T");
   const int64_t N = lw.shape(0), K = lw.shape(1), M = lx.numel() / K;
   if (ldy.numel() != M * N) throw Error(MG_ERR_INVALID, "linear_bwd: dY, X and W do not describe Y = X W^T");
   const bool has_bias = !node.has_attr("has_bias") || node.attr("has_bias") != 0;
   AnyBuffer dx = AnyBuffer::create(node.dtype(), device, M * K);
+  if (accumulate)  // the kernel adds into dx: start it from the prior gradient
+    MOGRAD_CALL(device, mg_copy_device, dx.data_ptr(), inputs[3].data_ptr(), M * K * dtype_size(node.dtype()), device.stream());
   AnyBuffer dw = AnyBuffer::create(node.dtype(), device, N * K);
   Buffers out = {dx, dw};
   void* db_ptr = nullptr;
@@ -598,8 +628,16 @@ inline Buffers linear_bwd(const OpRef& node, const Buffers& in, Device& device) 
     out.push_back(AnyBuffer::create(node.dtype(), device, N));
     db_ptr = out.back().data_ptr();
   }
-  MOGRAD_CALL(device, mg_linear_bwd, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), dx.data_ptr(),
-              dw.data_ptr(), db_ptr, M, N, K, node.dtype(), device.stream());
+  if (device.pending)
+    MOGRAD_CALL(device, mg_linear_bwd_deferred, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+                dx.data_ptr(), dw.data_ptr(), db_ptr, M, N, K, accumulate, relu_mask, node.dtype(), node.dtype(),
+                device.pending, device.stream());
+  else if (accumulate || relu_mask)
+    MOGRAD_CALL(device, mg_linear_bwd_fused, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), dx.data_ptr(),
+                dw.data_ptr(), db_ptr, M, N, K, accumulate, relu_mask, node.dtype(), device.stream());
+  else
+    MOGRAD_CALL(device, mg_linear_bwd, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), dx.data_ptr(),
+                dw.data_ptr(), db_ptr, M, N, K, node.dtype(), device.stream());
   return out;
 }
 
@@ -618,19 +656,102 @@ inline Buffers layer_norm_fwd_stats(const OpRef& node, const Buffers& inputs, De
   return {out, mean, rstd};
 }
 
-// LAYER_NORM_STATS_GRAD[dy, x, gamma, mean, rstd] -> [dx, dgamma, dbeta].
-inline Buffers layer_norm_bwd_stats(const OpRef& node, const Buffers& inputs, Device& device) {
+// LAYER_NORM_STATS_GRAD[dy, x, gamma, mean, rstd] -> [dx, dgamma, dbeta], and
+// LAYER_NORM_STATS_GRAD_ADD[dy, x, gamma, mean, rstd, residual]: dx = gradient + residual.
+inline Buffers layer_norm_bwd_stats(const OpRef& node, const Buffers& in, Device& device) {
   const Layout& x = node.src(1).layout();
   const Layout& gamma = node.src(2).layout();
   const int64_t cols = x.shape(x.rank() - 1), rows = x.numel() / cols;
   detail::require_float(node.dtype(), "layer_norm_bwd_stats");
+  const bool with_residual = node.op_type == "LAYER_NORM_STATS_GRAD_ADD";
+  const Buffers inputs = with_residual ? detail::materialise(node, in, device, 6) : in;
   AnyBuffer dx = AnyBuffer::create(node.dtype(), device, x.numel());
   AnyBuffer dgamma = AnyBuffer::create(node.dtype(), device, gamma.numel());
   AnyBuffer dbeta = AnyBuffer::create(node.dtype(), device, gamma.numel());
-  MOGRAD_CALL(device, mg_layer_norm_bwd_stats, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
-              static_cast<const float*>(inputs[3].data_ptr()), static_cast<const float*>(inputs[4].data_ptr()),
-              dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(), rows, cols, node.dtype(), device.stream());
+  const void* residual = with_residual ? inputs[5].data_ptr() : nullptr;
+  const float* mean = static_cast<const float*>(inputs[3].data_ptr());
+  const float* rstd = static_cast<const float*>(inputs[4].data_ptr());
+  if (device.pending)
+    MOGRAD_CALL(device, mg_layer_norm_bwd_stats_deferred, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+                mean, rstd, residual, dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(), rows, cols, node.dtype(),
+                node.dtype(), device.pending, device.stream());
+  else if (with_residual)
+    MOGRAD_CALL(device, mg_layer_norm_bwd_stats_add, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), mean,
+                rstd, residual, dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(), rows, cols, node.dtype(),
+                device.stream());
+  else
+    MOGRAD_CALL(device, mg_layer_norm_bwd_stats, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), mean,
+                rstd, dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(), rows, cols, node.dtype(), device.stream());
   return {dx, dgamma, dbeta};
+}
+
+// MATMUL_BT_ADD[A, B (N, K), R] = A B^T + R, R laid out like the result.
+inline Buffers matmul_bt_add(const OpRef& node, const Buffers& inputs, Device& device) {
+  const int64_t N = node.shape(node.layout().rank() - 1);
+  const detail::MatmulDims d = detail::matmul_dims(node.src(0).layout(), node.src(1).layout(), N, true, "matmul");
+  AnyBuffer residual = inputs[2];
+  if (!node.src(2).layout().is_contiguous()) {
+    const OpRef wrap{"ADD", node.layout(), node.dtype(), {node.src(2)}, {}};
+    residual = detail::materialise(wrap, {inputs[2]}, device, 1)[0];
+  }
+  AnyBuffer out = AnyBuffer::create(node.dtype(), device, node.numel());
+  MOGRAD_CALL(device, mg_matmul_bt_add, inputs[0].data_ptr(), inputs[1].data_ptr(), residual.data_ptr(), out.data_ptr(),
+              d.batch, d.M, N, d.K, d.lda0, d.lda1, d.ldb0, d.ldb1, d.bsa, d.bsb, node.dtype(), device.stream());
+  return {out};
+}
+
+// MATMUL_BIAS_RELU_BT[A, B (N, K), bias (N)] = max(A B^T + bias, 0).
+inline Buffers matmul_bias_relu_bt(const OpRef& node, const Buffers& inputs, Device& device) {
+  const int64_t N = node.shape(node.layout().rank() - 1);
+  const detail::MatmulDims d = detail::matmul_dims(node.src(0).layout(), node.src(1).layout(), N, true, "matmul_bias");
+  AnyBuffer out = AnyBuffer::create(node.dtype(), device, node.numel());
+  MOGRAD_CALL(device, mg_matmul_bias_relu_bt, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+              out.data_ptr(), d.batch, d.M, N, d.K, d.lda0, d.lda1, d.ldb0, d.ldb1, d.bsa, d.bsb, node.dtype(),
+              device.stream());
+  return {out};
+}
+
+// RESHAPE[a]: a contiguous tensor under another shape, a view (a strided source is materialised first).
+inline Buffers reshape(const OpRef& node, const Buffers& inputs, Device& device) {
+  const Buffers in = detail::materialise(node, inputs, device, 1);
+  const Layout rows = node.layout().as_contiguous();
+  return {in[0].view(Layout(rows.shape(), rows.stride(), in[0].offset_elems()))};
+}
+
+// TRANSPOSE[a]{dim0, dim1}: a strided view of the same storage.
+inline Buffers transpose(const OpRef& node, const Buffers& inputs, Device&) { return {inputs[0].view(node.layout())}; }
+
+// FLASH_ATTN_PACKED[qkv (B, S, 3, H, D)(, mask)]{scale, is_causal, has_bias} -> [O (B, S, H, D), LSE (B, H, S) f32].
+inline Buffers flash_attn_packed_fwd(const OpRef& node, const Buffers& inputs, Device& device) {
+  const Layout& q = node.src(0).layout();
+  if (q.rank() != 5 || q.shape(2) != 3) throw Error(MG_ERR_INVALID, "flash_attn_packed: qkv must be (B, S, 3, H, D)");
+  const int64_t B = q.shape(0), S = q.shape(1), H = q.shape(3), D = q.shape(4);
+  const bool is_causal = node.attr("is_causal") != 0;
+  const bool has_bias = node.has_attr("has_bias") ? node.attr("has_bias") != 0 : true;
+  detail::require_float(node.dtype(), "flash_attn_fwd");
+  AnyBuffer dst = AnyBuffer::create(node.dtype(), device, node.numel());
+  AnyBuffer lse = AnyBuffer::create(float32, device, B * H * S);
+  const void* mask = inputs.size() > 1 ? inputs[1].data_ptr() : nullptr;
+  MOGRAD_CALL(device, mg_flash_attn_fwd_packed, inputs[0].data_ptr(), mask, dst.data_ptr(),
+              static_cast<float*>(lse.data_ptr()), B, S, H, D, static_cast<float>(node.attr("scale")), is_causal, has_bias,
+              node.dtype(), device.stream());
+  return {dst, lse};
+}
+
+// FLASH_ATTN_PACKED_GRAD[dO, O, qkv, LSE(, mask)] -> dqkv (B, S, 3, H, D).
+inline Buffers flash_attn_packed_bwd(const OpRef& node, const Buffers& in, Device& device) {
+  const Layout& q = node.src(2).layout();
+  const int64_t B = q.shape(0), S = q.shape(1), H = q.shape(3), D = q.shape(4);
+  const bool is_causal = node.attr("is_causal") != 0;
+  const bool has_bias = node.has_attr("has_bias") ? node.attr("has_bias") != 0 : !is_causal;
+  detail::require_float(node.dtype(), "flash_attn_bwd");
+  const Buffers inputs = detail::materialise(node, in, device, 1);
+  AnyBuffer dqkv = AnyBuffer::create(node.dtype(), device, node.numel());
+  const void* mask = inputs.size() > 4 ? inputs[4].data_ptr() : nullptr;
+  MOGRAD_CALL(device, mg_flash_attn_bwd_packed, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), mask,
+              static_cast<const float*>(inputs[3].data_ptr()), dqkv.data_ptr(), B, S, H, D,
+              static_cast<float>(node.attr("scale")), is_causal, has_bias, node.dtype(), device.stream());
+  return {dqkv};
 }
 
 // CROSS_ENTROPY_IDS[logits (.., C), ids (..) int32/int64] -> (1,).
@@ -682,6 +803,109 @@ inline OpRef cross_entropy_ids_grad(const OpRef& node, const OpRef& upstream) {
                {node.src(0), node.src(1), upstream}, {}};
 }
 
+// ---- Rewrite rules (RewriteFn, mograd/simplify/__init__.mojo:9): node -> the fused node, or nothing.  The
+// fusions of a transformer training step that this library adds to the reference's GPU_REWRITES
+// (mograd/runtime/gpu/rewrites.mojo:13-34).  A multi-output node's result i is selected by
+// GETTUPLE{index: i}[node], as in the reference. -------------------------------------------------------------
+
+inline OpRef gettuple(const OpRef& src, int index, const Layout& layout, DType dtype) {
+  return OpRef{"GETTUPLE", layout, dtype, {src}, {{"index", static_cast<double>(index)}}};
+}
+inline bool is_output0_of(const OpRef& n, const char* op) {
+  return n.op_type == "GETTUPLE" && n.attr("index") == 0 && n.src(0).op_type == op;
+}
+
+// ADD(MATMUL_BT(a, w), r), either operand order -> MATMUL_BT_ADD[a, w, r].
+inline std::optional<OpRef> fuse_matmul_add(const OpRef& node) {
+  if (node.op_type != "ADD") return std::nullopt;
+  for (int i = 0; i < 2; ++i) {
+    const OpRef &mm = node.src(i), &other = node.src(1 - i);
+    if (mm.op_type == "MATMUL_BT" && mm.layout().shape() == other.layout().shape() && mm.dtype() == other.dtype())
+      return OpRef{"MATMUL_BT_ADD", mm.layout(), node.dtype(), {mm.src(0), mm.src(1), other}, {}};
+  }
+  return std::nullopt;
+}
+
+// RELU(MATMUL_BIAS_BT(a, w, b)) -> MATMUL_BIAS_RELU_BT[a, w, b].
+inline std::optional<OpRef> fuse_matmul_bias_relu(const OpRef& node) {
+  if (node.op_type != "RELU" || node.src(0).op_type != "MATMUL_BIAS_BT") return std::nullopt;
+  return OpRef{"MATMUL_BIAS_RELU_BT", node.src(0).layout(), node.dtype(), node.src(0).srcs, {}};
+}
+
+// RELU_GRAD(y, GETTUPLE0(LINEAR_GRAD(dy, y, w))) -> GETTUPLE0(LINEAR_GRAD{relu_mask}(dy, y, w)); `same` tells
+// whether two operand positions hold the same tensor (nodes here are values, not graph vertices).
+inline std::optional<OpRef> fuse_relu_grad_into_linear_grad(const OpRef& node, bool x_is_the_relu_output) {
+  if (node.op_type != "RELU_GRAD" || !is_output0_of(node.src(1), "LINEAR_GRAD") || !x_is_the_relu_output) return std::nullopt;
+  OpRef lin = node.src(1).src(0);
+  if (lin.has_attr("relu_mask") || lin.has_attr("accumulate")) return std::nullopt;
+  lin.node_attrs["relu_mask"] = 1.0;
+  return gettuple(lin, 0, node.src(1).layout(), node.src(1).dtype());
+}
+
+// ADD(p, GETTUPLE0(LINEAR_GRAD(dy, x, w))) -> GETTUPLE0(LINEAR_GRAD{accumulate}(dy, x, w, p)).
+inline std::optional<OpRef> fuse_add_into_linear_grad(const OpRef& node) {
+  if (node.op_type != "ADD") return std::nullopt;
+  for (int i = 0; i < 2; ++i) {
+    const OpRef &sel = node.src(i), &other = node.src(1 - i);
+    if (!is_output0_of(sel, "LINEAR_GRAD") || sel.src(0).has_attr("accumulate")) continue;
+    if (sel.layout().shape() != other.layout().shape() || sel.dtype() != other.dtype()) continue;
+    OpRef lin = sel.src(0);
+    lin.srcs.push_back(other);
+    lin.node_attrs["accumulate"] = 1.0;
+    return gettuple(lin, 0, sel.layout(), sel.dtype());
+  }
+  return std::nullopt;
+}
+
+// ADD(r, GETTUPLE0(LAYER_NORM_STATS_GRAD(dy, x, g, mean, rstd))) -> GETTUPLE0(LAYER_NORM_STATS_GRAD_ADD(.., r)).
+inline std::optional<OpRef> fuse_add_into_layer_norm_grad(const OpRef& node) {
+  if (node.op_type != "ADD") return std::nullopt;
+  for (int i = 0; i < 2; ++i) {
+    const OpRef &sel = node.src(i), &other = node.src(1 - i);
+    if (!is_output0_of(sel, "LAYER_NORM_STATS_GRAD")) continue;
+    if (sel.layout().shape() != other.layout().shape() || sel.dtype() != other.dtype()) continue;
+    OpRef ln = sel.src(0);
+    ln.op_type = "LAYER_NORM_STATS_GRAD_ADD";
+    ln.srcs.push_back(other);
+    return gettuple(ln, 0, sel.layout(), sel.dtype());
+  }
+  return std::nullopt;
+}
+
+// CONTIGUOUS(TRANSPOSE{1,2}(GETTUPLE0(FLASH_ATTN(q, k, v, mask)))) -> GETTUPLE0(FLASH_ATTN{layout: bshd}(...)).
+inline std::optional<OpRef> fuse_attention_output_layout(const OpRef& node) {
+  if (node.op_type != "CONTIGUOUS" || node.src(0).op_type != "TRANSPOSE" || !is_output0_of(node.src(0).src(0), "FLASH_ATTN"))
+    return std::nullopt;
+  const OpRef& tr = node.src(0);
+  const OpRef& sel = tr.src(0);
+  const int d0 = (static_cast<int>(tr.has_attr("dim0") ? tr.attr("dim0") : -2) + 4) % 4;
+  const int d1 = (static_cast<int>(tr.has_attr("dim1") ? tr.attr("dim1") : -1) + 4) % 4;
+  if (tr.layout().rank() != 4 || !((d0 == 1 && d1 == 2) || (d0 == 2 && d1 == 1))) return std::nullopt;
+  OpRef attn = sel.src(0);
+  if (attn.has_attr("layout")) return std::nullopt;
+  attn.node_attrs["layout"] = kLayoutBshd;
+  const Layout bshd({sel.shape(0), sel.shape(2), sel.shape(1), sel.shape(3)});
+  attn.node_layout = bshd;
+  return gettuple(attn, 0, bshd, sel.dtype());
+}
+
+// Leaves the second-stage sums of the exec functions that run inside its lifetime on one mg_deferred list
+// and finishes them with a single launch (finish()), as a training step does at its end.
+class DeferredSums {
+ public:
+  explicit DeferredSums(Device& device) : device_(device) {
+    MOGRAD_CALL(device_, mg_deferred_create, &device_.pending);
+  }
+  ~DeferredSums() {
+    if (device_.pending) device_.fn<decltype(&::mg_deferred_destroy)>("mg_deferred_destroy")(device_.pending);
+    device_.pending = nullptr;
+  }
+  void finish() { MOGRAD_CALL(device_, mg_finish_deferred, device_.pending, device_.stream()); }
+
+ private:
+  Device& device_;
+};
+
 // ---- Rule table (mograd/runtime/__init__.mojo:113-167) --------------------------------------------------
 
 struct Rule {
@@ -719,6 +943,14 @@ inline const std::vector<Rule>& scheduler_rules() {
       {"LAYER_NORM_STATS_GRAD", "layer_norm_bwd_stats", layer_norm_bwd_stats},
       {"CROSS_ENTROPY_IDS", "cross_entropy_ids", cross_entropy_ids},
       {"CROSS_ENTROPY_IDS_GRAD", "cross_entropy_grad_ids", cross_entropy_grad_ids},
+      // views, and the fused nodes that the rewrite rules below create
+      {"RESHAPE", "reshape", reshape},
+      {"TRANSPOSE", "transpose", transpose},
+      {"MATMUL_BT_ADD", "matmul_bt_add", matmul_bt_add},
+      {"MATMUL_BIAS_RELU_BT", "matmul_bias_relu_bt", matmul_bias_relu_bt},
+      {"LAYER_NORM_STATS_GRAD_ADD", "layer_norm_bwd_stats", layer_norm_bwd_stats},
+      {"FLASH_ATTN_PACKED", "flash_attn_packed_fwd", flash_attn_packed_fwd},
+      {"FLASH_ATTN_PACKED_GRAD", "flash_attn_packed_bwd", flash_attn_packed_bwd},
   };
   return rules;
 }

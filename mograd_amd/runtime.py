@@ -171,6 +171,10 @@ class Device:
     def synchronize(self) -> None:
         self.lib.mg_stream_sync(self.stream)
 
+    # The list on which the exec functions of LINEAR_GRAD, LAYER_NORM_STATS_GRAD(_ADD) and
+    # SCATTER_ADD leave their second-stage sums while it is set (see `deferred_sums`).
+    pending = None
+
     def empty_cache(self) -> None:
         self.lib.mg_pool_empty_cache()
 
@@ -384,9 +388,10 @@ def flash_attn_fwd_sched(node: Node, inputs: List[AnyBuffer], device: Device) ->
     _require_float(node.dtype(), "flash_attn_fwd")
     dst = AnyBuffer.create(node.dtype(), device, node.numel())
     lse = AnyBuffer.create(F32, device, B * H * S)
-    device.lib.mg_flash_attn_fwd(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
-                                 inputs[3].data_ptr(), dst.data_ptr(), lse.data_ptr(), B, S, H, D, scale,
-                                 int(is_causal), int(has_bias), node.dtype(), device.stream)
+    # {layout: "bshd"} (set by fuse_attention_output_layout): O is written (B, S, H, D) like Q
+    fwd = device.lib.mg_flash_attn_fwd_bshd if node.attrs().get("layout") == "bshd" else device.lib.mg_flash_attn_fwd
+    fwd(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), inputs[3].data_ptr(), dst.data_ptr(),
+        lse.data_ptr(), B, S, H, D, scale, int(is_causal), int(has_bias), node.dtype(), device.stream)
     return [dst, lse]
 
 
@@ -403,9 +408,9 @@ def flash_attn_bwd_sched(node: Node, inputs: List[AnyBuffer], device: Device) ->
     dq = AnyBuffer.create(node.dtype(), device, numel)
     dk = AnyBuffer.create(node.dtype(), device, numel)
     dv = AnyBuffer.create(node.dtype(), device, numel)
-    device.lib.mg_flash_attn_bwd(*(inputs[i].data_ptr() for i in range(7)), dq.data_ptr(), dk.data_ptr(),
-                                 dv.data_ptr(), B, S, H, D, scale, int(is_causal), int(has_bias), node.dtype(),
-                                 device.stream)
+    bwd = device.lib.mg_flash_attn_bwd_bshd if node.attrs().get("layout") == "bshd" else device.lib.mg_flash_attn_bwd
+    bwd(*(inputs[i].data_ptr() for i in range(7)), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, S, H, D, scale,
+        int(is_causal), int(has_bias), node.dtype(), device.stream)
     return [dq, dk, dv]
 
 
@@ -603,8 +608,13 @@ def scatter_add(node: Node, inputs: List[AnyBuffer], device: Device) -> List[Any
     inputs = _materialise(node, inputs, device, 2)
     row_size = lb.shape(lb.rank() - 1)
     out = AnyBuffer.create(node.dtype(), device, node.numel())
-    device.lib.mg_scatter_add(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), la.numel(),
-                              node.shape(0), row_size, node.src(0).dtype(), node.dtype(), device.stream)
+    if device.pending is not None:
+        device.lib.mg_scatter_add_deferred(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), la.numel(),
+                                           node.shape(0), row_size, node.src(0).dtype(), node.dtype(), node.dtype(),
+                                           device.pending, device.stream)
+    else:
+        device.lib.mg_scatter_add(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), la.numel(),
+                                  node.shape(0), row_size, node.src(0).dtype(), node.dtype(), device.stream)
     return [out]
 
 
@@ -659,11 +669,16 @@ def argmax(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffe
 
 
 def linear_bwd(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
-    """LINEAR_GRAD[dY (.., N), X (.., K), W (N, K)]{has_bias} -> [dX (.., K), dW (N, K), db (N)]
-    for Y = X W^T (+ b): dX = dY W, dW = dY^T X written in W's layout, db = column sums of dY
-    (two results without has_bias).  Leading dimensions collapse into the row count."""
+    """LINEAR_GRAD[dY (.., N), X (.., K), W (N, K)(, prior)]{has_bias, relu_mask, accumulate}
+    -> [dX (.., K), dW (N, K), db (N)] for Y = X W^T (+ b): dX = dY W, dW = dY^T X written in W's
+    layout, db = column sums of dY (two results without has_bias).  relu_mask: X is a ReLU's
+    output and dX is zeroed where X <= 0 (the RELU_GRAD of the layer below, folded in);
+    accumulate: dX = prior + dY W with `prior` the fourth source.  Leading dimensions collapse
+    into the row count."""
     ldy, lx, lw = (node.src(i).layout() for i in range(3))
-    inputs = _materialise(node, inputs, device, 3)
+    accumulate = bool(node.attrs().get("accumulate", False))
+    relu_mask = bool(node.attrs().get("relu_mask", False))
+    inputs = _materialise(node, inputs, device, 4 if accumulate else 3)
     _require_float(node.dtype(), "linear_bwd")
     N, K = lw.shape(0), lw.shape(1)
     M = lx.numel() // K
@@ -671,10 +686,19 @@ def linear_bwd(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyB
         raise MogradError(1, "linear_bwd: dY, X and W do not describe Y = X W^T")
     has_bias = bool(node.attrs().get("has_bias", True))
     dx = AnyBuffer.create(node.dtype(), device, M * K)
+    if accumulate:  # the kernel adds into dx: start it from the prior gradient
+        device.lib.mg_copy_device(dx.data_ptr(), inputs[3].data_ptr(), dx.size_bytes(), device.stream)
     dw = AnyBuffer.create(node.dtype(), device, N * K)
     db = AnyBuffer.create(node.dtype(), device, N) if has_bias else None
-    device.lib.mg_linear_bwd(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), dx.data_ptr(),
-                             dw.data_ptr(), db.data_ptr() if has_bias else None, M, N, K, node.dtype(), device.stream)
+    args = (inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), dx.data_ptr(), dw.data_ptr(),
+            db.data_ptr() if has_bias else None, M, N, K)
+    if device.pending is not None:
+        device.lib.mg_linear_bwd_deferred(*args, int(accumulate), int(relu_mask), node.dtype(), node.dtype(),
+                                          device.pending, device.stream)
+    elif accumulate or relu_mask:
+        device.lib.mg_linear_bwd_fused(*args, int(accumulate), int(relu_mask), node.dtype(), device.stream)
+    else:
+        device.lib.mg_linear_bwd(*args, node.dtype(), device.stream)
     return [dx, dw, db] if has_bias else [dx, dw]
 
 
@@ -695,18 +719,104 @@ def layer_norm_fwd_stats(node: Node, inputs: List[AnyBuffer], device: Device) ->
 
 
 def layer_norm_bwd_stats(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
-    """LAYER_NORM_STATS_GRAD[dy, x, gamma, mean, rstd] -> [dx, dgamma, dbeta]."""
+    """LAYER_NORM_STATS_GRAD[dy, x, gamma, mean, rstd] -> [dx, dgamma, dbeta], and
+    LAYER_NORM_STATS_GRAD_ADD[dy, x, gamma, mean, rstd, residual]: dx = gradient + residual (the
+    gradient that reaches x along another path, e.g. a skip connection)."""
     x_layout = node.src(1).layout()
     gamma_layout = node.src(2).layout()
     cols = x_layout.shape(x_layout.rank() - 1)
     rows = x_layout.numel() // cols
     _require_float(node.dtype(), "layer_norm_bwd_stats")
+    with_residual = node.op_type == "LAYER_NORM_STATS_GRAD_ADD"
+    if with_residual:
+        inputs = _materialise(node, inputs, device, 6)
     dx = AnyBuffer.create(node.dtype(), device, x_layout.numel())
     dgamma = AnyBuffer.create(node.dtype(), device, gamma_layout.numel())
     dbeta = AnyBuffer.create(node.dtype(), device, gamma_layout.numel())
-    device.lib.mg_layer_norm_bwd_stats(*(inputs[i].data_ptr() for i in range(5)), dx.data_ptr(), dgamma.data_ptr(),
-                                       dbeta.data_ptr(), rows, cols, node.dtype(), device.stream)
+    residual = inputs[5].data_ptr() if with_residual else None
+    ptrs = [inputs[i].data_ptr() for i in range(5)]
+    if device.pending is not None:
+        device.lib.mg_layer_norm_bwd_stats_deferred(*ptrs, residual, dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(),
+                                                    rows, cols, node.dtype(), node.dtype(), device.pending, device.stream)
+    elif with_residual:
+        device.lib.mg_layer_norm_bwd_stats_add(*ptrs, residual, dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(), rows,
+                                               cols, node.dtype(), device.stream)
+    else:
+        device.lib.mg_layer_norm_bwd_stats(*ptrs, dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(), rows, cols,
+                                           node.dtype(), device.stream)
     return [dx, dgamma, dbeta]
+
+
+def matmul_bt_add(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """MATMUL_BT_ADD[A, B (N, K), R] = A B^T + R (R laid out like the result): the residual
+    addition of a transformer block on the product that feeds it."""
+    la, lb = node.src(0).layout(), node.src(1).layout()
+    N = node.shape(node.layout().rank() - 1)
+    batch, M, K, lda0, lda1, ldb0, ldb1, bsa, bsb = _matmul_dims(la, lb, N, True, "matmul")
+    residual = inputs[2]
+    if not node.src(2).layout().is_contiguous():
+        residual = _materialise(Node("ADD", node.layout(), node.dtype(), [node.src(2)]), [inputs[2]], device, 1)[0]
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_matmul_bt_add(inputs[0].data_ptr(), inputs[1].data_ptr(), residual.data_ptr(), out.data_ptr(), batch, M,
+                                N, K, lda0, lda1, ldb0, ldb1, bsa, bsb, node.dtype(), device.stream)
+    return [out]
+
+
+def matmul_bias_relu_bt(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """MATMUL_BIAS_RELU_BT[A, B (N, K), bias (N)] = max(A B^T + bias, 0)."""
+    la, lb = node.src(0).layout(), node.src(1).layout()
+    N = node.shape(node.layout().rank() - 1)
+    batch, M, K, lda0, lda1, ldb0, ldb1, bsa, bsb = _matmul_dims(la, lb, N, True, "matmul_bias")
+    out = AnyBuffer.create(node.dtype(), device, node.numel())
+    device.lib.mg_matmul_bias_relu_bt(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), out.data_ptr(),
+                                      batch, M, N, K, lda0, lda1, ldb0, ldb1, bsa, bsb, node.dtype(), device.stream)
+    return [out]
+
+
+def reshape(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """RESHAPE[a]: a contiguous tensor under another shape, a view (mograd/op.mojo:335-337 folds
+    the identity; a strided source is materialised first, like the reference's reshape)."""
+    (src,) = _materialise(node, inputs, device, 1)
+    return [src.view(Layout(*node.layout().shape(), base_offset=src.offset_elems))]
+
+
+def transpose(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """TRANSPOSE[a]{dim0, dim1}: a strided view of the same storage (runtime/__init__.mojo:157)."""
+    return [inputs[0].view(node.layout())]
+
+
+def flash_attn_packed_fwd(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """FLASH_ATTN_PACKED[qkv (B, S, 3, H, D), mask]{scale, is_causal, has_bias} -> [O (B, S, H, D),
+    LSE (B, H, S) f32]: Q, K and V are the three slices of one projection's output, and O comes out
+    in the layout the next projection reads."""
+    B, S, three, H, D = (node.src(0).layout().shape(i) for i in range(5))
+    if three != 3:
+        raise MogradError(1, "flash_attn_packed: qkv must be (B, S, 3, H, D)")
+    is_causal = bool(node.attrs()["is_causal"])
+    has_bias = bool(node.attrs().get("has_bias", True))
+    _require_float(node.dtype(), "flash_attn_fwd")
+    dst = AnyBuffer.create(node.dtype(), device, node.numel())
+    lse = AnyBuffer.create(F32, device, B * H * S)
+    mask = inputs[1].data_ptr() if len(inputs) > 1 else None
+    device.lib.mg_flash_attn_fwd_packed(inputs[0].data_ptr(), mask, dst.data_ptr(), lse.data_ptr(), B, S, H, D,
+                                        float(node.attrs()["scale"]), int(is_causal), int(has_bias), node.dtype(),
+                                        device.stream)
+    return [dst, lse]
+
+
+def flash_attn_packed_bwd(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """FLASH_ATTN_PACKED_GRAD[dO, O, qkv, LSE(, mask)] -> dqkv (B, S, 3, H, D)."""
+    B, S, _, H, D = (node.src(2).layout().shape(i) for i in range(5))
+    is_causal = bool(node.attrs()["is_causal"])
+    has_bias = bool(node.attrs().get("has_bias", not is_causal))
+    _require_float(node.dtype(), "flash_attn_bwd")
+    inputs = _materialise(node, inputs, device, 1)  # dO contiguous, as flash_attn_grad makes it
+    dqkv = AnyBuffer.create(node.dtype(), device, node.numel())
+    mask = inputs[4].data_ptr() if len(inputs) > 4 else None
+    device.lib.mg_flash_attn_bwd_packed(inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(), mask,
+                                        inputs[3].data_ptr(), dqkv.data_ptr(), B, S, H, D, float(node.attrs()["scale"]),
+                                        int(is_causal), int(has_bias), node.dtype(), device.stream)
+    return [dqkv]
 
 
 def cross_entropy_ids(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
@@ -765,6 +875,14 @@ SCHEDULER_RULES = {
     "LAYER_NORM_STATS_GRAD": layer_norm_bwd_stats,
     "CROSS_ENTROPY_IDS": cross_entropy_ids,
     "CROSS_ENTROPY_IDS_GRAD": cross_entropy_grad_ids,
+    # views, and the fused nodes that mograd_amd.rewrites.GPU_REWRITES creates
+    "RESHAPE": reshape,
+    "TRANSPOSE": transpose,
+    "MATMUL_BT_ADD": matmul_bt_add,
+    "MATMUL_BIAS_RELU_BT": matmul_bias_relu_bt,
+    "LAYER_NORM_STATS_GRAD_ADD": layer_norm_bwd_stats,
+    "FLASH_ATTN_PACKED": flash_attn_packed_fwd,
+    "FLASH_ATTN_PACKED_GRAD": flash_attn_packed_bwd,
 }
 
 
@@ -861,6 +979,66 @@ def gettuple_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
     return [upstream]
 
 
+def add_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """mograd/grad.mojo:126-127: both sources receive the upstream (same shapes on this path;
+    the reference's un-broadcast of an EXPAND source is expand_grad, outside it)."""
+    for src in node.srcs:
+        if src.layout().shape() != node.layout().shape():
+            raise MogradError(2, "add_grad: broadcast operands are outside the backward hot path")
+    return [upstream, upstream]
+
+
+def contiguous_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """mograd/grad.mojo:269: a copy's gradient is the upstream itself."""
+    return [upstream]
+
+
+def cast_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """mograd/grad.mojo:237: the upstream cast back to the source's dtype."""
+    src = node.src(0)
+    if src.dtype() not in (F32, F16, BF16):
+        return [None]
+    return [Node("CAST", upstream.layout().as_contiguous(), src.dtype(), [upstream])]
+
+
+def gather_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """mograd/grad.mojo:190: SCATTER_ADD[indices, upstream] in the table's shape; no gradient for
+    the indices."""
+    table, indices = node.src(0), node.src(1)
+    return [Node("SCATTER_ADD", table.layout().as_contiguous(), table.dtype(), [indices, upstream]), None]
+
+
+def softmax_grad_rule(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """mograd/grad.mojo:232-234: SOFTMAX_GRAD[y, upstream]."""
+    return [Node("SOFTMAX_GRAD", node.layout().as_contiguous(), node.dtype(), [node, upstream])]
+
+
+def reshape_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """mograd/grad.mojo (reshape_grad): the upstream under the source's shape."""
+    src = node.src(0)
+    return [Node("RESHAPE", src.layout().as_contiguous(), upstream.dtype(), [upstream])]
+
+
+def transpose_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """mograd/grad.mojo:186-187: the same two dimensions swapped back (a view)."""
+    d0, d1 = int(node.attrs().get("dim0", -2)), int(node.attrs().get("dim1", -1))
+    return [Node("TRANSPOSE", upstream.layout().transpose(d0, d1), upstream.dtype(), [upstream], dict(node.attrs()))]
+
+
+def flash_attn_packed_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """FLASH_ATTN_PACKED[qkv(, mask)] -> FLASH_ATTN_PACKED_GRAD[dO, O, qkv, LSE(, mask)] -> dqkv: the
+    packed form of flash_attn_grad (mograd/grad.mojo:309-344); the mask gets no gradient."""
+    qkv = node.src(0)
+    B, S, _, H, _ = qkv.layout().shape()
+    o = _gettuple(node, 0, node.layout(), node.dtype())
+    lse = _gettuple(node, 1, Layout(B, H, S), F32)
+    d_o = upstream if upstream.layout().is_contiguous() else Node("CONTIGUOUS", upstream.layout().as_contiguous(),
+                                                                  upstream.dtype(), [upstream])
+    bwd = Node("FLASH_ATTN_PACKED_GRAD", qkv.layout().as_contiguous(), qkv.dtype(), [d_o, o, qkv, lse] + node.srcs[1:],
+               dict(node.attrs()))
+    return [bwd] + [None] * (len(node.srcs) - 1)
+
+
 GRAD_RULES = {
     "MATMUL_BT": linear_grad,
     "MATMUL_BIAS_BT": linear_grad,
@@ -871,22 +1049,34 @@ GRAD_RULES = {
     "CROSS_ENTROPY_IDS": cross_entropy_grad_rule,
     "RELU": relu_grad_rule,
     "GETTUPLE": gettuple_grad,
+    "ADD": add_grad,
+    "CONTIGUOUS": contiguous_grad,
+    "CAST": cast_grad,
+    "GATHER": gather_grad,
+    "SOFTMAX": softmax_grad_rule,
+    "RESHAPE": reshape_grad,
+    "TRANSPOSE": transpose_grad,
+    "FLASH_ATTN_PACKED": flash_attn_packed_grad,
 }
 
 
 def _toposort(root: Node) -> List[Node]:
+    """Sources before consumers, each node once (GraphUtils.toposort); iterative, so that deep
+    training graphs do not run into the interpreter's recursion limit."""
     order: List[Node] = []
     seen = set()
-
-    def visit(n: Node) -> None:
-        if n in seen:
-            return
-        seen.add(n)
-        for s_ in n.srcs:
-            visit(s_)
-        order.append(n)
-
-    visit(root)
+    stack = [(root, 0)]
+    seen.add(root)
+    while stack:
+        n, i = stack.pop()
+        if i < len(n.srcs):
+            stack.append((n, i + 1))
+            child = n.srcs[i]
+            if child not in seen:
+                seen.add(child)
+                stack.append((child, 0))
+        else:
+            order.append(n)
     return order
 
 
@@ -917,13 +1107,36 @@ def evaluate(node: Node, device: Device) -> AnyBuffer:
     """Scheduler.run for one result (mograd/scheduler.mojo:40-80): evaluates the sources
     first, runs the node's rule once and keeps its buffers on the node; GETTUPLE selects an
     output of a multi-output source."""
-    if node.bufs is None:
-        if node.op_type == "BUFFER":
+    for n in _toposort(node):
+        if n.bufs is not None:
+            continue
+        if n.op_type == "BUFFER":
             raise MogradError(1, "evaluate: a leaf node without a buffer")
-        if node.op_type == "GETTUPLE":
-            evaluate(node.src(0), device)
-            node.bufs = [node.src(0).bufs[int(node.attrs()["index"])]]
+        if n.op_type == "GETTUPLE":
+            n.bufs = [n.src(0).bufs[int(n.attrs()["index"])]]
         else:
-            inputs = [evaluate(s_, device) for s_ in node.srcs]
-            node.bufs = run(node, inputs, device)
+            n.bufs = run(n, [s_.bufs[0] for s_ in n.srcs], device)
     return node.bufs[0]
+
+
+def evaluate_many(nodes: Sequence[Node], device: Device, deferred_sums: bool = False) -> List[AnyBuffer]:
+    """Scheduler.run_many (mograd/scheduler.mojo:39-82): every node of `nodes` in one walk, shared
+    sub-graphs evaluated once.  With `deferred_sums` the second-stage sums of the parameter
+    gradients (LINEAR_GRAD, LAYER_NORM_STATS_GRAD(_ADD), SCATTER_ADD) are left on one mg_deferred
+    list and finished by a single launch after the walk: same bits, fewer launches."""
+    sink = Node("SINK", Layout(1), F32, list(nodes))
+    order = _toposort(sink)[:-1]
+    if deferred_sums:
+        pending = C.c_void_p()
+        device.lib.mg_deferred_create(C.byref(pending))
+        device.pending = pending
+    try:
+        for n in order:
+            evaluate(n, device)
+        if deferred_sums:
+            device.lib.mg_finish_deferred(device.pending, device.stream)
+    finally:
+        if deferred_sums:
+            device.lib.mg_deferred_destroy(device.pending)
+            device.pending = None
+    return [n.bufs[0] for n in nodes]

@@ -265,6 +265,74 @@ class TinyTransformer:
             marks("backward")
         return self.loss
 
+    # ------------------------------------------------------------------ the same step through the rule tables
+
+    def graph(self, ids: AnyBuffer, labels: AnyBuffer, B: int, T: int):
+        """The forward pass as a node graph over the compute-dtype parameters (leaves bound to the
+        slices of `self.work`), written with plain ops the way the reference's model writes it
+        (examples/tinyshakespear/model.mojo): GATHER, LAYER_NORM_STATS, MATMUL_BT, ADD, RELU,
+        MATMUL_BIAS_BT, attention on the stacked projection's (B, T, 3, H, dh) output, and
+        cross-entropy on class ids.  Returns (loss node, {parameter name: leaf node})."""
+        from .runtime import Layout, Node
+
+        n, d, ff, V, H, dh, cd = B * T, self.d, self.ff, self.V, self.H, self.dh, self.cd
+        leaves = {}
+
+        def param(name, shape=None):
+            sl = self.slices[name]
+            shape = shape or sl.shape
+            numel = int(np.prod(shape))
+            leaf = Node.leaf(Layout(*shape), cd, AnyBuffer(self.work.storage, cd, numel, sl.offset))
+            leaves[name] = leaf
+            return leaf
+
+        get = lambda node, i, layout, dtype=cd: Node("GETTUPLE", layout, dtype, [node], {"index": i})
+        ids_leaf = Node.leaf(Layout(n), ids.dtype, ids)
+        labels_leaf = Node.leaf(Layout(n), labels.dtype, labels)
+        h = Node("GATHER", Layout(n, d), cd, [param("embed"), ids_leaf])
+        for l in range(self.L):
+            w = lambda name, shape=None, l=l: param(f"blocks.{l}.{name}", shape)
+
+            def norm(x, g, b):
+                ln = Node("LAYER_NORM_STATS", Layout(n, d), cd, [x, g, b], {"eps": self.eps})
+                return get(ln, 0, Layout(n, d))
+
+            x1 = norm(h, w("ln1_g"), w("ln1_b"))
+            # wq | wk | wv lie back to back: one (3d, d) weight whose product is Q | K | V per token
+            wqkv = w("wq", (3 * d, d))
+            qkv = Node("MATMUL_BT", Layout(n, 3 * d), cd, [x1, wqkv])
+            qkv5 = Node("RESHAPE", Layout(B, T, 3, H, dh), cd, [qkv])
+            attn = Node("FLASH_ATTN_PACKED", Layout(B, T, H, dh), cd, [qkv5],
+                        {"scale": 1.0 / math.sqrt(dh), "is_causal": True, "has_bias": False})
+            ctx = Node("RESHAPE", Layout(n, d), cd, [get(attn, 0, Layout(B, T, H, dh))])
+            h_mid = Node("ADD", Layout(n, d), cd, [Node("MATMUL_BT", Layout(n, d), cd, [ctx, w("wo")]), h])
+            x2 = norm(h_mid, w("ln2_g"), w("ln2_b"))
+            a = Node("RELU", Layout(n, ff), cd, [Node("MATMUL_BIAS_BT", Layout(n, ff), cd, [x2, w("w1"), w("b1")])])
+            h = Node("ADD", Layout(n, d), cd, [Node("MATMUL_BT", Layout(n, d), cd, [a, w("w2")]), h_mid])
+        logits = Node("MATMUL_BT", Layout(n, V), cd, [h, param("lm_head")])
+        loss = Node("CROSS_ENTROPY_IDS", Layout(1), cd, [logits, labels_leaf])
+        return loss, leaves
+
+    def step_via_rules(self, ids: AnyBuffer, labels: AnyBuffer, B: int, T: int, deferred_sums: bool = True):
+        """The training step as the rule tables produce it: the forward graph of `graph`, its
+        gradient graph from runtime.gradient (GRAD_RULES), both rewritten by
+        Simplifier(GPU_REWRITES()) into the fused nodes, evaluated by runtime.evaluate_many.  Returns
+        (loss buffer, {parameter name: gradient buffer in the compute dtype}).  The kernels and
+        their operands are those of `step`, so the results equal `step`'s bit for bit (its
+        gradients before the cast to fp32)."""
+        from .rewrites import GPU_REWRITES, Simplifier
+        from .runtime import evaluate_many, gradient
+
+        self.lib.mg_cast(self.master.data_ptr(), self.work.data_ptr(), self.total, F32, self.cd, self.stream)
+        loss, leaves = self.graph(ids, labels, B, T)
+        names = [k for k in leaves if not k.endswith((".wk", ".wv"))]
+        one = AnyBuffer.create(self.cd, self.device, 1, fill=1.0)
+        from .runtime import Layout, Node
+        grads = gradient(loss, Node.leaf(Layout(1), self.cd, one), [leaves[k] for k in names])
+        roots = Simplifier(GPU_REWRITES()).run_many([loss] + grads)
+        bufs = evaluate_many(roots, self.device, deferred_sums=deferred_sums)
+        return bufs[0], dict(zip(names, bufs[1:])), roots
+
     # ------------------------------------------------------------------ optimizer
 
     def adam_step(self, lr: float = 1e-3, beta1: float = 0.9, beta2: float = 0.999, eps: float = 1e-8,

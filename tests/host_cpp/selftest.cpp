@@ -401,6 +401,106 @@ int main(int argc, char** argv) {
     return "no error raised";
   });
 
+  // The fused nodes that the rewrite rules create, against the nodes they replace, on small
+  // integers (every sum exact in fp32, so equality is exact whatever the order): a block's
+  // residual product, its ReLU product, the ReLU gradient folded into LINEAR_GRAD, LayerNorm's
+  // gradient added to the skip connection's, and the same gradients with their second-stage sums
+  // deferred to one launch.
+  run_case("rewrites: fused nodes equal the nodes they replace", [&]() -> std::string {
+    const int64_t M = 64, N = 24, K = 40;
+    const Layout lx{M, K}, lw{N, K}, ly{M, N}, lb{N};
+    const auto x = ints(M * K, 21, -3, 3), w = ints(N * K, 22, -2, 2), b = ints(N, 23, -4, 4), r = ints(M * N, 24, -9, 9);
+    Buffers in = {upload(dev, x), upload(dev, w), upload(dev, b), upload(dev, r)};
+    const OpRef nx = OpRef::leaf(lx), nw = OpRef::leaf(lw), nb = OpRef::leaf(lb), nr = OpRef::leaf(ly);
+    // ADD(MATMUL_BT, r) -> MATMUL_BT_ADD
+    const OpRef mm = node("MATMUL_BT", ly, {nx, nw});
+    const auto fused_add = fuse_matmul_add(node("ADD", ly, {nr, mm}));
+    if (!fused_add || fused_add->op_type != "MATMUL_BT_ADD") return "ADD(r, MATMUL_BT) was not rewritten";
+    auto y0 = run(mm, {in[0], in[1]}, dev);
+    auto y1 = run(node("ADD", ly, {nr, mm}), {in[3], y0[0]}, dev);
+    auto y2 = run(*fused_add, {in[0], in[1], in[3]}, dev);
+    if (download(y1[0]) != download(y2[0])) return "MATMUL_BT_ADD differs from MATMUL_BT + ADD";
+    // RELU(MATMUL_BIAS_BT) -> MATMUL_BIAS_RELU_BT
+    const OpRef mb = node("MATMUL_BIAS_BT", ly, {nx, nw, nb});
+    const auto fused_relu = fuse_matmul_bias_relu(node("RELU", ly, {mb}));
+    if (!fused_relu || fused_relu->op_type != "MATMUL_BIAS_RELU_BT") return "RELU(MATMUL_BIAS_BT) was not rewritten";
+    auto a0 = run(mb, {in[0], in[1], in[2]}, dev);
+    auto a1 = run(node("RELU", ly, {mb}), {a0[0]}, dev);
+    auto a2 = run(*fused_relu, {in[0], in[1], in[2]}, dev);
+    if (download(a1[0]) != download(a2[0])) return "MATMUL_BIAS_RELU_BT differs from MATMUL_BIAS_BT + RELU";
+    // RELU_GRAD(y, LINEAR_GRAD[0]) -> LINEAR_GRAD{relu_mask}: here x plays the ReLU's output
+    std::vector<float> xr = x;
+    for (auto& v : xr) v = v > 0 ? v : 0;
+    AnyBuffer bx = upload(dev, xr), bdy = upload(dev, r);
+    const OpRef lin = linear_grad(node("MATMUL_BT", ly, {nx, nw}), nr);
+    const OpRef sel = gettuple(lin, 0, lx, float32);
+    const auto masked = fuse_relu_grad_into_linear_grad(node("RELU_GRAD", lx, {nx, sel}), true);
+    if (!masked || masked->src(0).attr("relu_mask") != 1) return "RELU_GRAD(y, LINEAR_GRAD[0]) was not rewritten";
+    auto g0 = run(lin, {bdy, bx, in[1]}, dev);
+    auto g1 = run(node("RELU_GRAD", lx, {nx, sel}), {bx, g0[0]}, dev);
+    auto g2 = run(masked->src(0), {bdy, bx, in[1]}, dev);
+    if (download(g1[0]) != download(g2[0])) return "LINEAR_GRAD{relu_mask} differs from LINEAR_GRAD + RELU_GRAD";
+    if (download(g0[1]) != download(g2[1])) return "dW changed under relu_mask";
+    // ADD(p, LINEAR_GRAD[0]) -> LINEAR_GRAD{accumulate}
+    const auto accum = fuse_add_into_linear_grad(node("ADD", lx, {nx, sel}));
+    if (!accum || accum->src(0).srcs.size() != 4) return "ADD(p, LINEAR_GRAD[0]) was not rewritten";
+    auto p1 = run(node("ADD", lx, {nx, sel}), {in[0], g0[0]}, dev);
+    auto p2 = run(accum->src(0), {bdy, bx, in[1], in[0]}, dev);
+    if (download(p1[0]) != download(p2[0])) return "LINEAR_GRAD{accumulate} differs from LINEAR_GRAD + ADD";
+    // the same LINEAR_GRAD with its second-stage sums deferred
+    {
+      DeferredSums sums(dev);
+      auto d2 = run(masked->src(0), {bdy, bx, in[1]}, dev);
+      sums.finish();
+      if (download(d2[0]) != download(g2[0]) || download(d2[1]) != download(g2[1])) return "deferred LINEAR_GRAD differs";
+    }
+    return "";
+  });
+  run_case("rewrites: LayerNorm gradient added to the skip connection's", [&]() -> std::string {
+    const int64_t rows = 48, cols = 32;
+    const Layout lx{rows, cols}, lv{cols}, lr{rows};
+    const auto x = ints(rows * cols, 31, -5, 5), dy = ints(rows * cols, 32, -3, 3), res = ints(rows * cols, 33, -7, 7);
+    std::vector<float> g(cols, 1.f), b(cols, 0.f);
+    for (int64_t c = 0; c < cols; ++c) g[c] = 0.5f + 0.125f * static_cast<float>(c % 8);
+    const OpRef fwd = node("LAYER_NORM_STATS", lx, {OpRef::leaf(lx), OpRef::leaf(lv), OpRef::leaf(lv)}, {{"eps", 1e-5}});
+    AnyBuffer bx = upload(dev, x), bg = upload(dev, g), bdy = upload(dev, dy), bres = upload(dev, res);
+    auto f = run(fwd, {bx, bg, upload(dev, b)}, dev);
+    const OpRef bwd = layer_norm_stats_grad(fwd, OpRef::leaf(lx), OpRef::leaf(lr), OpRef::leaf(lr));
+    const OpRef sel = gettuple(bwd, 0, lx, float32);
+    const auto fused = fuse_add_into_layer_norm_grad(node("ADD", lx, {OpRef::leaf(lx), sel}));
+    if (!fused || fused->src(0).op_type != "LAYER_NORM_STATS_GRAD_ADD") return "ADD(r, LAYER_NORM_STATS_GRAD[0]) was not rewritten";
+    auto g0 = run(bwd, {bdy, bx, bg, f[1], f[2]}, dev);
+    auto g1 = run(node("ADD", lx, {OpRef::leaf(lx), sel}), {bres, g0[0]}, dev);
+    auto g2 = run(fused->src(0), {bdy, bx, bg, f[1], f[2], bres}, dev);
+    if (download(g1[0]) != download(g2[0])) return "dx differs from LAYER_NORM_STATS_GRAD + ADD";
+    if (download(g0[1]) != download(g2[1]) || download(g0[2]) != download(g2[2])) return "dgamma / dbeta changed";
+    DeferredSums sums(dev);
+    auto g3 = run(fused->src(0), {bdy, bx, bg, f[1], f[2], bres}, dev);
+    sums.finish();
+    if (download(g3[0]) != download(g2[0]) || download(g3[1]) != download(g2[1]) || download(g3[2]) != download(g2[2]))
+      return "deferred sums differ";
+    return "";
+  });
+  run_case("rewrites: attention output written (B, S, H, D)", [&]() -> std::string {
+    const int64_t B = 1, S = 8, H = 2, D = 8;
+    const Layout bshd{B, S, H, D}, bhsd{B, H, S, D};
+    const auto q = ints(B * S * H * D, 41, -2, 2), k = ints(B * S * H * D, 42, -2, 2), v = ints(B * S * H * D, 43, -3, 3);
+    Buffers in = {upload(dev, q), upload(dev, k), upload(dev, v), upload(dev, std::vector<float>(1, 0.f))};
+    const OpRef attn = node("FLASH_ATTN", bhsd, {OpRef::leaf(bshd), OpRef::leaf(bshd), OpRef::leaf(bshd), OpRef::leaf(Layout{1})},
+                            {{"scale", 0.25}, {"is_causal", 1}, {"has_bias", 0}});
+    const OpRef o = gettuple(attn, 0, bhsd, float32);
+    const OpRef tr = node("TRANSPOSE", bhsd.transpose(1, 2), {o}, {{"dim0", 1}, {"dim1", 2}});
+    const OpRef copy = node("CONTIGUOUS", bshd, {tr});
+    const auto fused = fuse_attention_output_layout(copy);
+    if (!fused || fused->src(0).attr("layout") != kLayoutBshd) return "CONTIGUOUS(TRANSPOSE(FLASH_ATTN[0])) was not rewritten";
+    auto a0 = run(attn, in, dev);
+    auto t0 = run(tr, {a0[0]}, dev);
+    auto c0 = run(copy, {t0[0]}, dev);
+    auto a1 = run(fused->src(0), in, dev);
+    if (download(c0[0]) != download(a1[0])) return "FLASH_ATTN{layout: bshd} differs from the copy";
+    return "";
+  });
+
   // Pool behaviour seen through AnyBuffer (tests/test_memory.mojo:18-60): a freed block of the
   // 1024-byte class serves the next request that rounds to the same class.
   run_case("pool reuses a size class", [&]() -> std::string {

@@ -10,8 +10,9 @@ import pytest
 from helpers import ATOL_F32, RTOL_F32, assert_close, assert_sum_close, integers, normal, uniform
 from oracle import oracle_np as O
 
-from mograd_amd import F32, I32, I64, Layout, Node
+from mograd_amd import BF16, F32, I32, I64, AnyBuffer, Layout, Node
 from mograd_amd import runtime as R
+from mograd_amd.runtime import round_to_dtype
 
 
 # ---- graph structure: no GPU ------------------------------------------------------------------
@@ -193,3 +194,138 @@ def test_mlp_gradient_through_the_rules(device):
             O.linear_grad_b(r_dlogits)]
     for a, c, what in zip(got, want, ("dw1", "db1", "dgamma", "dbeta", "dw2", "db2")):
         assert_close(a, c, RTOL_F32, ATOL_F32, what)
+
+
+# --------------------------------------------------------------------------- #
+# The transformer step through gradient() + Simplifier(GPU_REWRITES()) + evaluate_many()
+# --------------------------------------------------------------------------- #
+
+
+def _op_counts(roots):
+    from mograd_amd.runtime import _toposort
+
+    counts = {}
+    for n in _toposort(Node("SINK", Layout(1), F32, list(roots)))[:-1]:
+        counts[n.op_type] = counts.get(n.op_type, 0) + 1
+    return counts
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [BF16, F32])
+@pytest.mark.parametrize("V,d,ff,L,H,B,T", [(65, 128, 512, 2, 2, 4, 64), (65, 384, 1536, 1, 6, 16, 256)])
+def test_transformer_step_through_the_rule_tables(device, dtype, V, d, ff, L, H, B, T):
+    # The forward graph in plain ops (GATHER, LAYER_NORM_STATS, MATMUL_BT, ADD, RELU, MATMUL_BIAS_BT,
+    # packed attention, cross-entropy on ids), differentiated by gradient() over GRAD_RULES, rewritten
+    # into the fused nodes and evaluated: every parameter gradient and the loss must equal the
+    # hand-sequenced TinyTransformer.step bit for bit, and the rewritten graph must consist of the
+    # fused nodes that step calls (no separate ADD / RELU / RELU_GRAD left in a block).
+    from helpers import integers
+    from mograd_amd.tiny_transformer import TinyTransformer, init_params
+
+    rng = np.random.Generator(np.random.PCG64(75_000 + d))
+    params = init_params(rng, V, d, ff, L)
+    for b in params["blocks"]:
+        for g, be in (("ln1_g", "ln1_b"), ("ln2_g", "ln2_b")):
+            b[g] = rng.uniform(0.5, 1.5, b[g].shape).astype(np.float32)
+            b[be] = rng.normal(0, 0.1, b[be].shape).astype(np.float32)
+    ids = AnyBuffer.from_numpy(device, integers(75, 1, (B, T), 0, V, np.int32))
+    labels = AnyBuffer.from_numpy(device, integers(75, 2, (B, T), 0, V, np.int32))
+    model = TinyTransformer(device, V, d, ff, L, H, compute_dtype=dtype, deferred=False)
+    model.load_params(params)
+    want_loss = model.step(ids, labels, B, T).item()
+    want = model.gradients()
+    for deferred_sums in (False, True):
+        loss, grads, roots = model.step_via_rules(ids, labels, B, T, deferred_sums=deferred_sums)
+        assert loss.item() == want_loss
+        for name, buf in grads.items():
+            parts = name.split(".")
+            ref = want["blocks"][int(parts[1])] if parts[0] == "blocks" else want
+            key = parts[-1]
+            if key == "wq":  # the stacked (3d, d) projection: wq | wk | wv
+                blk = want["blocks"][int(parts[1])]
+                expect = np.concatenate([blk["wq"], blk["wk"], blk["wv"]], axis=0)
+            else:
+                expect = ref[key]
+            np.testing.assert_array_equal(buf.to_numpy(expect.shape), expect, err_msg=f"{name} (deferred {deferred_sums})")
+    counts = _op_counts(roots)
+    assert counts.get("MATMUL_BT_ADD") == 2 * L and counts.get("MATMUL_BIAS_RELU_BT") == L
+    assert counts.get("LAYER_NORM_STATS_GRAD_ADD") == 2 * L and "LAYER_NORM_STATS_GRAD" not in counts
+    assert counts.get("LINEAR_GRAD") == 4 * L + 1
+    for gone in ("ADD", "RELU", "RELU_GRAD"):
+        assert gone not in counts, f"{gone} survived the rewrites: {counts}"
+
+
+@pytest.mark.gpu
+def test_rewrites_attention_copy_and_shared_input_accumulation(device):
+    # (i) CONTIGUOUS(TRANSPOSE(FLASH_ATTN[0])) -> FLASH_ATTN{layout: bshd}, and its gradient node
+    # follows; (ii) three projections of one input: their input gradients ADD(ADD(dx_q, dx_k), dx_v)
+    # become accumulating LINEAR_GRAD nodes.  The rewritten graph must give the same bits as the
+    # graph as written.
+    from mograd_amd.rewrites import GPU_REWRITES, Simplifier
+    from mograd_amd.runtime import evaluate_many
+
+    B, S, H, D, dtype = 2, 96, 2, 64, BF16
+    n, d = B * S, H * D
+    x = round_to_dtype(normal(76, 0, (n, d)), dtype)
+    ws = [round_to_dtype(normal(76, 1 + i, (d, d), std=0.05), dtype) for i in range(4)]
+    up = round_to_dtype(normal(76, 9, (n, d)), dtype)
+
+    def build():
+        leaf = lambda a: Node.leaf(Layout(*a.shape), dtype, AnyBuffer.from_numpy(device, a, dtype))
+        lx, (lq, lk, lv, lo) = leaf(x), [leaf(w) for w in ws]
+        proj = lambda w: Node("RESHAPE", Layout(B, S, H, D), dtype, [Node("MATMUL_BT", Layout(n, d), dtype, [lx, w])])
+        mask = Node.leaf(Layout(1), dtype, AnyBuffer.create(dtype, device, 1, fill=0.0))
+        attn = Node("FLASH_ATTN", Layout(B, H, S, D), dtype, [proj(lq), proj(lk), proj(lv), mask],
+                    {"scale": 0.125, "is_causal": True, "has_bias": False})
+        o = Node("GETTUPLE", Layout(B, H, S, D), dtype, [attn], {"index": 0})
+        tr = Node("TRANSPOSE", Layout(B, H, S, D).transpose(1, 2), dtype, [o], {"dim0": 1, "dim1": 2})
+        ctx = Node("RESHAPE", Layout(n, d), dtype, [Node("CONTIGUOUS", Layout(B, S, H, D), dtype, [tr])])
+        y = Node("MATMUL_BT", Layout(n, d), dtype, [ctx, lo])
+        grads = R.gradient(y, leaf(up), [lx, lq, lk, lv, lo])
+        return [y] + grads
+
+    plain = [b.to_numpy() for b in evaluate_many(build(), device)]
+    roots = Simplifier(GPU_REWRITES()).run_many(build())
+    fused = [b.to_numpy() for b in evaluate_many(roots, device)]
+    for a, b, name in zip(fused, plain, ("y", "dx", "dwq", "dwk", "dwv", "dwo")):
+        np.testing.assert_array_equal(a, b, err_msg=name)
+    counts = _op_counts(roots)
+    assert "CONTIGUOUS" not in counts and "TRANSPOSE" not in counts, counts
+    assert "ADD" not in counts, counts
+    from mograd_amd.runtime import _toposort
+    nodes = _toposort(Node("SINK", Layout(1), F32, list(roots)))
+    assert all(nd.attrs().get("layout") == "bshd" for nd in nodes if nd.op_type in ("FLASH_ATTN", "FLASH_ATTN_GRAD"))
+    assert sum(1 for nd in nodes if nd.op_type == "LINEAR_GRAD" and nd.attrs().get("accumulate")) == 2
+
+
+def test_rewrite_rules_on_graph_structure():
+    # no GPU: patterns, refusal when the folded tensor has another reader, redirection of the other
+    # selectors of a refitted multi-output node
+    from mograd_amd.rewrites import GPU_REWRITES, Simplifier
+
+    x, w, b, r = Node.leaf(Layout(4, 8)), Node.leaf(Layout(6, 8)), Node.leaf(Layout(6)), Node.leaf(Layout(4, 6))
+    mm = Node("MATMUL_BT", Layout(4, 6), F32, [x, w])
+    out = Simplifier(GPU_REWRITES()).run(Node("ADD", Layout(4, 6), F32, [r, mm]))
+    assert out.op_type == "MATMUL_BT_ADD" and out.srcs == [x, w, r]
+    # the product has a second reader: it must stay a node of its own
+    both = Simplifier(GPU_REWRITES()).run_many([Node("ADD", Layout(4, 6), F32, [mm, r]), mm])
+    assert both[0].op_type == "ADD" and both[1] is mm
+    act = Node("RELU", Layout(4, 6), F32, [Node("MATMUL_BIAS_BT", Layout(4, 6), F32, [x, w, b])])
+    assert Simplifier(GPU_REWRITES()).run(act).op_type == "MATMUL_BIAS_RELU_BT"
+    # RELU_GRAD folded into the LINEAR_GRAD that reads the ReLU's output: dW's selector follows
+    y = Node("RELU", Layout(4, 8), F32, [x])
+    z = Node("MATMUL_BT", Layout(4, 6), F32, [y, w])
+    dx, dw = R.gradient(z, Node.leaf(Layout(4, 6)), [x, w])
+    assert dx.op_type == "RELU_GRAD"
+    dx2, dw2 = Simplifier(GPU_REWRITES()).run_many([dx, dw])
+    assert dx2.op_type == "GETTUPLE" and dx2.src(0).op_type == "LINEAR_GRAD" and dx2.src(0).attrs()["relu_mask"] is True
+    assert dw2.src(0) is dx2.src(0), "dW reads the refitted node, not a second copy of the product"
+    # the gradient rules added for residual and embedding graphs
+    emb, idx = Node.leaf(Layout(10, 8)), Node.leaf(Layout(4), I32)
+    h = Node("GATHER", Layout(4, 8), F32, [emb, idx])
+    s2 = Node("ADD", Layout(4, 8), F32, [h, Node("CONTIGUOUS", Layout(4, 8), F32, [h])])
+    (g,) = R.gradient(s2, Node.leaf(Layout(4, 8)), [emb])
+    assert g.op_type == "SCATTER_ADD" and g.src(0) is idx and g.src(1).op_type == "ADD"
+    c = Node("CAST", Layout(4, 8), BF16, [x])
+    (gc,) = R.gradient(c, Node.leaf(Layout(4, 8), BF16), [x])
+    assert gc.op_type == "CAST" and gc.dtype() == F32
