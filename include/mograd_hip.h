@@ -12,8 +12,13 @@
  *     taken from the library's pool and returned before the call returns; this is safe
  *     because all work of one call is enqueued on the one stream passed in, and the pool
  *     hands memory back out only to later calls (the reference's single in-order-stream
- *     contract, mograd/memory.mojo:27-31).  Calls on different streams that overlap in
- *     time must not share the pool's scratch: serialise them or use one stream.
+ *     contract, mograd/memory.mojo:27-31).  This makes the library a one-stream-per-device
+ *     library: every entry point that takes scratch (the LayerNorm, cross-entropy, Linear
+ *     and attention backward entries, split products, mg_sum_axis, mg_scatter_add and the
+ *     `_deferred` forms) returns its blocks to the pool while its kernels are still queued,
+ *     untagged by stream, so calls issued on two streams of one device that overlap in
+ *     time may be handed the same block.  Use one stream per device, or order the streams
+ *     with events so that such calls never overlap.
  *   - `stream` is a hipStream_t passed as void*; NULL is the default stream.  No function
  *     synchronises the host unless its comment says so.
  *   - The symbols are new names: the reference's own `mograd_*` exports use the Mojo ABI

@@ -2018,11 +2018,7 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
   }
   // The pipelined dK/dV walk (head dims up to 64, no bias) reads the row statistics negated
   // and padded per (batch, head) to a multiple of 64 rows; the delta kernel writes both forms.
-  static const bool pipe_off = [] {
-    const char* e = env_str("MOGRAD_HIP_ATTN_DKDV_PIPE");
-    return e && e[0] == '0';
-  }();
-  const bool pipe = DP <= 64 && !has_bias && !pipe_off;
+  const bool pipe = DP <= 64 && !has_bias && env_int("MOGRAD_HIP_ATTN_DKDV_PIPE", 1) != 0;
   const int s_pad = static_cast<int>(ceil_div(a.S, 64) * 64);
   const int64_t padded = pipe ? static_cast<int64_t>(a.B) * a.H * s_pad : 0;
   Scratch delta;
@@ -2040,10 +2036,7 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
   // even at 1024, 2-3% slower from 2048 on, where the two walks compete for the same CU
   // instead of filling each other's gaps).  MOGRAD_HIP_ATTN_FUSED_BWD_MAX_S overrides it; 0
   // always launches dK/dV and dQ separately.
-  static const int fused_max_s = [] {
-    const char* e = env_str("MOGRAD_HIP_ATTN_FUSED_BWD_MAX_S");
-    return e && e[0] ? std::atoi(e) : 1024;
-  }();
+  const int fused_max_s = env_int("MOGRAD_HIP_ATTN_FUSED_BWD_MAX_S", 1024);
   const bool fused = DP <= 64 && a.S <= fused_max_s && 2 * (blocks + 7) < 0x7fffffffLL;
   const T* d_o_ = static_cast<const T*>(d_o);
   const T* q_ = static_cast<const T*>(q);

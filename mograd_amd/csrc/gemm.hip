@@ -411,6 +411,10 @@ static int linear_bwd_one_launch(const void* dy, const void* x, const void* w, v
   }
   if (splits <= 1 || ceil_div(M, splits) >= 4096) return MG_OK;
   const int k_per_split = splitk_16bit_range(M, &splits);
+  // Every K range of dW and the whole reduction of dX must be whole k-steps (of 32 or 64): the
+  // kernels drop a remainder.  Guaranteed by M % kG16BK == 0, N % kG16BK == 0 and ranges cut in
+  // units of kG16BK; checked here so that a change to either cannot lose rows silently.
+  if (k_per_split % kG16BK != 0 || M % kG16BK != 0 || N % kG16BK != 0) return MG_OK;
   // dX: the 32-k variant.
   if (N >= 4096 || (N >= 1024 && ceil_div(M, 256) * tiles_kk >= 2 * cus)) return MG_OK;
   const int64_t n_dw = gemm_split_grid(w_tiles, splits, 1);
@@ -502,7 +506,7 @@ __global__ __launch_bounds__(256) void pad_columns_kernel(const T* __restrict__ 
 // A layer whose width N is not a multiple of the k-step (a 65-symbol vocabulary) cannot take
 // the pipelined kernels as it lies: rows of dY start at odd addresses, and both products
 // would go to the element-staged kernel (3-4 % of the matrix cores busy).  Here dY gets
-// zero columns and W zero rows up to the next multiple of 32 (copies of M x N and N x K
+// zero columns and W zero rows up to the next multiple of 64 (copies of M x N and N x K
 // elements, small beside X and dX), the padded layer goes through the common launch, and
 // only the first N rows of dW are written.  The padding adds exact zeros to every sum.
 template <typename T>

@@ -845,6 +845,8 @@ template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, int BK,
 __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm16Problem<T>& pr) {
   static_assert(NSTAGE >= 2 && NSTAGE <= 4 && (BK == 32 || BK == 64) && (TM == 128 || TM == 256), "stages");
   static_assert(TN % 128 == 0 && (!SPLIT_K || TM == 128), "partial tiles are 128 x 128");
+  // The host cuts K ranges and checks K in units of kG16BK: every range is then whole steps of BK.
+  static_assert(kG16BK % BK == 0, "K ranges are multiples of kG16BK, which must be whole steps");
   constexpr int WN = TN / 64;                                 // waves side by side
   constexpr int NW = (TM / 64) * WN;
   constexpr int NWA = gemm16_pipe_waves(TM, BK, NW), NWB = gemm16_pipe_waves(TN, BK, NW);  // waves that copy A, B

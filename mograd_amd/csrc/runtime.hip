@@ -242,9 +242,11 @@ const char* mg_last_error(void) { return mg::g_last_error.c_str(); }
 int mg_init(int device) {
   MG_HIP(hipSetDevice(device));
   (void)mg::device_info();
-  // the static scratch of the non-allocating entry point: resolve this device's copy now,
-  // so that its first call does no set-up work
-  MG_TRY(mg::ce_noalloc_setup(nullptr));
+  // The static scratch of the non-allocating entry point: resolve this device's copy now, so
+  // that its first call does no set-up work.  A failure here (a device ordinal beyond its
+  // table, say) concerns that one optional entry point, which reports it when called: the rest
+  // of the library stays usable.
+  if (mg::ce_noalloc_setup(nullptr) != MG_OK) mg::clear_error();
   return MG_OK;
 }
 

@@ -15,6 +15,25 @@ RTOL_F32, ATOL_F32 = 1e-4, 1e-5       # fp32 reductions
 RTOL_BF16_ATTN = 2e-2                 # bf16 attention gradients
 
 
+# bf16 attention gradients (B, S, H, D): rtol 2e-2 of the entry plus a floor for entries that
+# cancel to ~0, taken per (batch, head) and not per tensor: 7.5e-3 of that head's largest entry.
+# Observed on the MI355X over (B2,H3,S256,D64), (B1,H2,S1100,D64/128/256) and three heads each of
+# the two benchmark shapes, causal and not: the part of |err| that rtol*|ref| does not cover is at
+# most 3.8e-3 of the head's largest entry (dq, non-causal S256), typically 1-2.5e-3; the floor is
+# twice the worst observation.  (|err| itself stays under 1.03e-2 of the head's largest entry.)
+ATTN_BF16_FLOOR = 7.5e-3
+
+
+def assert_attn_grad_close(got, ref, what, rtol=RTOL_BF16_ATTN, floor=ATTN_BF16_FLOOR, min_top=0.0):
+    """|got - ref| <= rtol |ref| + floor * (largest |ref| of the same batch and head), tensors (B, S, H, D)."""
+    ref = np.asarray(ref, dtype=np.float64)
+    assert np.all(np.isfinite(got)), what
+    top = np.maximum(np.abs(ref).max(axis=(1, 3), keepdims=True), min_top)
+    bound = rtol * np.abs(ref) + floor * top
+    worst = float(np.max(np.abs(got - ref) / bound))
+    assert worst <= 1.0, f"{what}: worst |err| / (rtol |ref| + floor * head max) = {worst:.3g}"
+
+
 def rng_for(config: int, tensor: int) -> np.random.Generator:
     return np.random.Generator(np.random.PCG64(1000 * config + tensor))
 
