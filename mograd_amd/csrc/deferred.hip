@@ -17,23 +17,20 @@ struct DeferredTable {
 };
 
 // LDS of a finishing workgroup: the largest of the forms' needs.
-constexpr int kDeferredLdsBytes = kSlabLdsFloats * 4 > 4 * 4 * 64 * 16 ? kSlabLdsFloats * 4 : 4 * 4 * 64 * 16;
+constexpr int kDeferredLdsBytes = kSlabLdsFloats * 4 > 4096 ? kSlabLdsFloats * 4 : 4096;
 
 template <typename OutT>
 __device__ __forceinline__ void deferred_run(char* lds, const DeferredJob& j, int local_block) {
   OutT* out = static_cast<OutT*>(j.out);
   const int sub = threadIdx.x / 256, tid = threadIdx.x % 256;
   switch (j.kind) {
-    case kDeferSplitK: {
-      // four 256-thread pieces of gemm_splitk_reduce_block's work per workgroup; a piece past
-      // the end does no loads or stores but keeps the barrier
-      float4(&tile)[4][64] = reinterpret_cast<float4(*)[4][64]>(lds)[sub];
-      gemm_splitk_reduce_block<OutT, false, true>(tile, tid, static_cast<int64_t>(local_block) * 4 + sub, j.part,
+    case kDeferSplitK:
+      // a thread sums four consecutive values of a partial tile over the K ranges
+      gemm_splitk_reduce_group<OutT, false, true, true>(static_cast<int64_t>(local_block) * 1024 + threadIdx.x, j.part,
                                                   static_cast<const OutT*>(nullptr), out, j.slice, j.slice, j.groups,
                                                   j.cols, GemmEpilogue<OutT>{nullptr, nullptr, 0}, j.rows,
                                                   (j.cols + kGemmBN - 1) / kGemmBN);
       break;
-    }
     case kDeferBiasRows:
       linear_bwd_db_block<OutT>(reinterpret_cast<float*>(lds) + sub * 256, tid, local_block * 4 + sub, j.part, out,
                                 j.groups, j.cols);

@@ -499,7 +499,7 @@ __device__ __forceinline__ void gemm16_write_tile(const floatx16 (&acc)[2][2], u
                                                   const T* __restrict__ bias, T* __restrict__ C,
                                                   float* __restrict__ partial, int M, int N, int64_t ldc, int64_t bsc,
                                                   int batch, int split, int batches, int m0, int n0, int wm, int wn,
-                                                  int lane, const GemmEpilogue<T>& ep) {
+                                                  int lane, const GemmEpilogue<T>& ep, bool partial_stream = false) {
   if constexpr (SPLIT_K) {
     // A K range's partial tile goes out as the accumulators lie in the registers: sixteen
     // unguarded 16-byte stores per thread, each a contiguous kilobyte of the wave
@@ -510,6 +510,18 @@ __device__ __forceinline__ void gemm16_write_tile(const floatx16 (&acc)[2][2], u
                             static_cast<int64_t>(m0 / kGemmBM) * tiles_n + col0 / kGemmBN;
     float4* dst = reinterpret_cast<float4*>(partial) + tile_at * (kG16PartialTile / 4) +
                   ((wm / 64) * 2 + (col0 / 64) % 2) * 1024 + lane;
+    if (partial_stream) {
+#pragma unroll
+      for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+        for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const floatx4 v = {acc[ti][tj][4 * g], acc[ti][tj][4 * g + 1], acc[ti][tj][4 * g + 2], acc[ti][tj][4 * g + 3]};
+            __builtin_nontemporal_store(v, reinterpret_cast<floatx4*>(dst + ((ti * 2 + tj) * 4 + g) * 64));
+          }
+      return;
+    }
 #pragma unroll
     for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
@@ -835,6 +847,9 @@ struct Gemm16Problem {
   // first tile column also sum their A tiles over k, i.e. dY over its rows, and leave one
   // partial row of the bias gradient per K range at colsum_part[split * M + m].
   float* colsum_part = nullptr;
+  // The partial tiles are read back much later (their sum is deferred to the end of a training
+  // step): store them past the caches.
+  bool partial_stream = false;
 };
 
 // The work of workgroup `bid` of a launch for one product; `lds` is the workgroup's
@@ -999,7 +1014,7 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
   uint16_t* mine = reinterpret_cast<uint16_t*>(lds) + wave * 64 * kG16Stride;
   gemm16_write_tile<T, HAS_BIAS, SPLIT_K>(acc, mine, bias, C, partial, M, N, ldc, bsc, batch,
                                           split, SPLIT_K ? batches : 1,
-                                          m0, n0, wm, wn, lane, ep);
+                                          m0, n0, wm, wn, lane, ep, pr.partial_stream);
 }
 
 template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, int BK, int NSTAGE, int TM = 128>
@@ -1369,64 +1384,93 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_f32_pipe_kernel(
   }  // tiles of this workgroup
 }
 
-// out[i] = sum_s partial[s * slice + i] (+ bias[i % N]) for i < numel <= slice, converted to T.  A workgroup covers 64
-// groups of four consecutive outputs; its four waves each sum every fourth split (eight
-// independent 16-byte loads in flight per thread) and the four sums meet in LDS.  The
-// order of the additions is fixed, so the result is deterministic.
+// out[i] = sum_s partial[s * slice + i] (+ bias[i % N]) for i < numel <= slice, converted to T.  One thread
+// sums group g, four consecutive outputs, over all K ranges: range s goes to one of eight
+// running sums, number (s / 4 % 2, s % 4), in increasing s, and the eight meet as
+// ((a00 + a10) + (a01 + a11)) + ((a02 + a12) + (a03 + a13)).  The order is fixed, so the result is
+// deterministic; it is the order of an earlier form of this reduction (four waves summing
+// every fourth range each and meeting in LDS), kept so that results did not change, with
+// eight independent 16-byte loads in flight per thread and no barrier.
 // TILED: the partials are whole 128 x 128 tiles in accumulator order (kG16PartialTile), numel
 // = slice = their count per K range, and a group of four is four consecutive rows of one
 // column of `out` (rows x N per batch; tiles_n tile columns; rows and columns past the matrix
 // are dropped).
-template <typename T, bool HAS_BIAS, bool TILED = false>
-__device__ __forceinline__ void gemm_splitk_reduce_block(float4 (&tile)[4][64], int tid, int64_t bid,
-                                                         const float* __restrict__ partial, const T* __restrict__ bias,
-                                                         T* __restrict__ out, int64_t numel, int64_t slice, int splits,
-                                                         int N, const GemmEpilogue<T>& ep, int rows = 0,
-                                                         int tiles_n = 0) {
-  const int cx = tid % 64;  // tid: this thread among the 256 that share `tile`
-  const int sl = tid / 64;
-  const int64_t i = (bid * 64 + cx) * 4;
-  float4 acc0 = make_float4(0.f, 0.f, 0.f, 0.f), acc1 = acc0;
-  if (i < numel) {
-    const bool full = TILED || i + 3 < numel;
-    int s = sl;
-    if (full) {
-      for (; s + 4 < splits; s += 8) {
-        const float4 u = *reinterpret_cast<const float4*>(partial + static_cast<int64_t>(s) * slice + i);
-        const float4 w = *reinterpret_cast<const float4*>(partial + static_cast<int64_t>(s + 4) * slice + i);
-        acc0.x += u.x; acc0.y += u.y; acc0.z += u.z; acc0.w += u.w;
-        acc1.x += w.x; acc1.y += w.y; acc1.z += w.z; acc1.w += w.w;
-      }
-      for (; s < splits; s += 4) {
-        const float4 u = *reinterpret_cast<const float4*>(partial + static_cast<int64_t>(s) * slice + i);
-        acc0.x += u.x; acc0.y += u.y; acc0.z += u.z; acc0.w += u.w;
-      }
-    } else {
-      for (; s < splits; s += 4) {
-        const float* p = partial + static_cast<int64_t>(s) * slice + i;
-        acc0.x += p[0];
-        if (i + 1 < numel) acc0.y += p[1];
-        if (i + 2 < numel) acc0.z += p[2];
+template <typename T, bool HAS_BIAS, bool TILED = false, bool STREAM = false>
+__device__ __forceinline__ void gemm_splitk_reduce_group(int64_t g, const float* __restrict__ partial,
+                                                         const T* __restrict__ bias, T* __restrict__ out, int64_t numel,
+                                                         int64_t slice, int splits, int N, const GemmEpilogue<T>& ep,
+                                                         int rows = 0, int tiles_n = 0) {
+  const int64_t i = g * 4;
+  if (i >= numel) return;
+  float r[4];
+  if (TILED || i + 3 < numel) {
+    float4 acc[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[h][j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const float* p = partial + i;
+    constexpr int NB = 8;  // K ranges in flight per thread (2 or 1 measured 2-7 % slower on a step's sums)
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+#pragma unroll
+      for (int h = 0; h < 8; h += NB) {
+        float4 v[NB];
+#pragma unroll
+        for (int e = 0; e < NB; ++e)
+          if (s0 + h + e >= splits) {
+            v[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+          } else if constexpr (STREAM) {
+            // read once, long after it was written: a streaming load that leaves the caches to
+            // the tensors of the next step (a step's deferred sums: 137 -> 103 us)
+            const floatx4 nt =
+                __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(p + static_cast<int64_t>(s0 + h + e) * slice));
+            v[e] = make_float4(nt[0], nt[1], nt[2], nt[3]);
+          } else {
+            v[e] = *reinterpret_cast<const float4*>(p + static_cast<int64_t>(s0 + h + e) * slice);
+          }
+#pragma unroll
+        for (int e = 0; e < NB; ++e) {
+          if (s0 + h + e < splits) {  // (adding the zero would turn a -0 sum into +0)
+            float4& a = acc[(h + e) / 4][(h + e) % 4];
+            a.x += v[e].x; a.y += v[e].y; a.z += v[e].z; a.w += v[e].w;
+          }
+        }
       }
     }
+    float4 t[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      t[j] = make_float4(acc[0][j].x + acc[1][j].x, acc[0][j].y + acc[1][j].y, acc[0][j].z + acc[1][j].z,
+                         acc[0][j].w + acc[1][j].w);
+    r[0] = (t[0].x + t[1].x) + (t[2].x + t[3].x);
+    r[1] = (t[0].y + t[1].y) + (t[2].y + t[3].y);
+    r[2] = (t[0].z + t[1].z) + (t[2].z + t[3].z);
+    r[3] = (t[0].w + t[1].w) + (t[2].w + t[3].w);
+  } else {
+    // the last, partial group of an untiled slice: element by element, four running sums
+    float a[4][3];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) a[j][0] = a[j][1] = a[j][2] = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float* p = partial + static_cast<int64_t>(s) * slice + i;
+      a[s % 4][0] += p[0];
+      if (i + 1 < numel) a[s % 4][1] += p[1];
+      if (i + 2 < numel) a[s % 4][2] += p[2];
+    }
+#pragma unroll
+    for (int e = 0; e < 3; ++e) r[e] = ((a[0][e] + 0.f) + (a[1][e] + 0.f)) + ((a[2][e] + 0.f) + (a[3][e] + 0.f));
+    r[3] = 0.f;
   }
-  tile[sl][cx] = make_float4(acc0.x + acc1.x, acc0.y + acc1.y, acc0.z + acc1.z, acc0.w + acc1.w);
-  __syncthreads();
-  if (sl != 0 || i >= numel) return;
-  const float4 t0 = tile[0][cx], t1 = tile[1][cx], t2 = tile[2][cx], t3 = tile[3][cx];
-  const float r[4] = {(t0.x + t1.x) + (t2.x + t3.x), (t0.y + t1.y) + (t2.y + t3.y), (t0.z + t1.z) + (t2.z + t3.z),
-                      (t0.w + t1.w) + (t2.w + t3.w)};
   if constexpr (TILED) {
-    // bid * 64 + cx = ((((t * 4 + wave) * 2 + ti) * 2 + tj) * 4 + g) * 64 + lane, and cx = lane
-    const int64_t q = bid * 64;
-    const int g = static_cast<int>(q / 64 % 4), tj = static_cast<int>(q / 256 % 2), ti = static_cast<int>(q / 512 % 2);
-    const int wave = static_cast<int>(q / 1024 % 4);
-    const int64_t t = q / 4096;  // tile over (batch, tile row, tile column)
+    // g = ((((t * 4 + wave) * 2 + ti) * 2 + tj) * 4 + q) * 64 + lane
+    const int lane = static_cast<int>(g % 64), q = static_cast<int>(g / 64 % 4), tj = static_cast<int>(g / 256 % 2),
+              ti = static_cast<int>(g / 512 % 2), wave = static_cast<int>(g / 1024 % 4);
+    const int64_t t = g / 4096;  // tile over (batch, tile row, tile column)
     const int tiles_m = (rows + kGemmBM - 1) / kGemmBM;
     const int tn = static_cast<int>(t % tiles_n), tm = static_cast<int>(t / tiles_n % tiles_m);
     const int64_t batch = t / tiles_n / tiles_m;
-    const int row = tm * kGemmBM + (wave / 2) * 64 + ti * 32 + g * 8 + (cx / 32) * 4;
-    const int col = tn * kGemmBN + (wave % 2) * 64 + tj * 32 + cx % 32;
+    const int row = tm * kGemmBM + (wave / 2) * 64 + ti * 32 + q * 8 + (lane / 32) * 4;
+    const int col = tn * kGemmBN + (wave % 2) * 64 + tj * 32 + lane % 32;
     if (col >= N) return;
     const float bv = HAS_BIAS ? to_float(bias[col]) : 0.f;
     for (int e = 0; e < 4 && row + e < rows; ++e) {
@@ -1446,9 +1490,8 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
                                                                  const T* __restrict__ bias, T* __restrict__ out,
                                                                  int64_t numel, int64_t slice, int splits, int N,
                                                                  GemmEpilogue<T> ep, int rows = 0, int tiles_n = 0) {
-  __shared__ float4 tile[4][64];
-  gemm_splitk_reduce_block<T, HAS_BIAS, TILED>(tile, threadIdx.x, blockIdx.x, partial, bias, out, numel, slice, splits, N, ep, rows,
-                                               tiles_n);
+  gemm_splitk_reduce_group<T, HAS_BIAS, TILED>(static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x, partial, bias, out,
+                                               numel, slice, splits, N, ep, rows, tiles_n);
 }
 
 // db[c] = sum over the `groups` partial rows db_part[g][c], 64 columns per 256 threads (`tid`
@@ -1479,22 +1522,22 @@ __device__ __forceinline__ void linear_bwd_db_block(float* __restrict__ sums_, i
 // the K ranges of dW (gemm_splitk_reduce_block), the rest sum the `groups` partial rows of
 // the bias gradient that the launch left (one per K range), 64 columns per workgroup,
 // every fourth row per 64 threads, then (t0 + t1) + (t2 + t3).  Fixed order, no atomics.
+// dw_blocks = ceil(slice / 1024): a thread sums four consecutive values of a partial tile.
 template <typename T>
 __global__ __launch_bounds__(256) void linear_bwd_finish_kernel(const float* __restrict__ partial, T* __restrict__ dw,
                                                                 int dw_rows, int64_t slice, int splits, int K,
                                                                 int dw_blocks, const float* __restrict__ db_part,
                                                                 T* __restrict__ db, int groups, int N) {
-  __shared__ float4 tile[4][64];
+  __shared__ float sums[256];
   const int bid = blockIdx.x;
   if (bid < dw_blocks) {
     // dW is (dw_rows, K); the partial tiles cover the (N, K) product of the launch
-    gemm_splitk_reduce_block<T, false, true>(tile, threadIdx.x, bid, partial, static_cast<const T*>(nullptr), dw, slice,
-                                             slice,
-                                             splits, K, GemmEpilogue<T>{nullptr, nullptr, 0}, dw_rows,
-                                             (K + kGemmBN - 1) / kGemmBN);
+    gemm_splitk_reduce_group<T, false, true>(static_cast<int64_t>(bid) * 256 + threadIdx.x, partial,
+                                             static_cast<const T*>(nullptr), dw, slice, slice, splits, K,
+                                             GemmEpilogue<T>{nullptr, nullptr, 0}, dw_rows, (K + kGemmBN - 1) / kGemmBN);
     return;
   }
-  linear_bwd_db_block<T>(reinterpret_cast<float*>(&tile[0][0]), threadIdx.x, bid - dw_blocks, db_part, db, groups, N);
+  linear_bwd_db_block<T>(sums, threadIdx.x, bid - dw_blocks, db_part, db, groups, N);
 }
 
 }  // namespace mg

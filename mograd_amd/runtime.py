@@ -1108,15 +1108,20 @@ def evaluate(node: Node, device: Device) -> AnyBuffer:
     first, runs the node's rule once and keeps its buffers on the node; GETTUPLE selects an
     output of a multi-output source."""
     for n in _toposort(node):
-        if n.bufs is not None:
-            continue
-        if n.op_type == "BUFFER":
-            raise MogradError(1, "evaluate: a leaf node without a buffer")
-        if n.op_type == "GETTUPLE":
-            n.bufs = [n.src(0).bufs[int(n.attrs()["index"])]]
-        else:
-            n.bufs = run(n, [s_.bufs[0] for s_ in n.srcs], device)
+        _evaluate_node(n, device)
     return node.bufs[0]
+
+
+def _evaluate_node(n: Node, device: Device) -> None:
+    """One node whose sources have their buffers."""
+    if n.bufs is not None:
+        return
+    if n.op_type == "BUFFER":
+        raise MogradError(1, "evaluate: a leaf node without a buffer")
+    if n.op_type == "GETTUPLE":
+        n.bufs = [n.src(0).bufs[int(n.attrs()["index"])]]
+    else:
+        n.bufs = run(n, [s_.bufs[0] for s_ in n.srcs], device)
 
 
 def evaluate_many(nodes: Sequence[Node], device: Device, deferred_sums: bool = False) -> List[AnyBuffer]:
@@ -1132,7 +1137,7 @@ def evaluate_many(nodes: Sequence[Node], device: Device, deferred_sums: bool = F
         device.pending = pending
     try:
         for n in order:
-            evaluate(n, device)
+            _evaluate_node(n, device)
         if deferred_sums:
             device.lib.mg_finish_deferred(device.pending, device.stream)
     finally:

@@ -313,23 +313,33 @@ class TinyTransformer:
         loss = Node("CROSS_ENTROPY_IDS", Layout(1), cd, [logits, labels_leaf])
         return loss, leaves
 
-    def step_via_rules(self, ids: AnyBuffer, labels: AnyBuffer, B: int, T: int, deferred_sums: bool = True):
+    def step_via_rules(self, ids: AnyBuffer, labels: AnyBuffer, B: int, T: int, deferred_sums: bool = True,
+                       reuse_graph: bool = False):
         """The training step as the rule tables produce it: the forward graph of `graph`, its
         gradient graph from runtime.gradient (GRAD_RULES), both rewritten by
         Simplifier(GPU_REWRITES()) into the fused nodes, evaluated by runtime.evaluate_many.  Returns
-        (loss buffer, {parameter name: gradient buffer in the compute dtype}).  The kernels and
-        their operands are those of `step`, so the results equal `step`'s bit for bit (its
-        gradients before the cast to fp32)."""
+        (loss buffer, {parameter name: gradient buffer in the compute dtype}, rewritten roots).  The
+        kernels and their operands are those of `step`, so the results equal `step`'s bit for bit
+        (its gradients before the cast to fp32).  The reference builds its graph anew every step
+        (lazy tensors); `reuse_graph` keeps the rewritten graph of the first call with the same
+        (ids, labels, B, T) and only evaluates it again."""
         from .rewrites import GPU_REWRITES, Simplifier
-        from .runtime import evaluate_many, gradient
+        from .runtime import Layout, Node, _toposort, evaluate_many, gradient
 
         self.lib.mg_cast(self.master.data_ptr(), self.work.data_ptr(), self.total, F32, self.cd, self.stream)
-        loss, leaves = self.graph(ids, labels, B, T)
-        names = [k for k in leaves if not k.endswith((".wk", ".wv"))]
-        one = AnyBuffer.create(self.cd, self.device, 1, fill=1.0)
-        from .runtime import Layout, Node
-        grads = gradient(loss, Node.leaf(Layout(1), self.cd, one), [leaves[k] for k in names])
-        roots = Simplifier(GPU_REWRITES()).run_many([loss] + grads)
+        key = (id(ids), id(labels), B, T)
+        if reuse_graph and getattr(self, "_rules_graph", None) and self._rules_graph[0] == key:
+            _, names, roots, interior = self._rules_graph
+            for node in interior:  # forget last step's results; the leaves keep their buffers
+                node.bufs = None
+        else:
+            loss, leaves = self.graph(ids, labels, B, T)
+            names = [k for k in leaves if not k.endswith((".wk", ".wv"))]
+            one = AnyBuffer.create(self.cd, self.device, 1, fill=1.0)
+            grads = gradient(loss, Node.leaf(Layout(1), self.cd, one), [leaves[k] for k in names])
+            roots = Simplifier(GPU_REWRITES()).run_many([loss] + grads)
+            interior = [n for n in _toposort(Node("SINK", Layout(1), F32, list(roots)))[:-1] if n.op_type != "BUFFER"]
+            self._rules_graph = (key, names, roots, interior) if reuse_graph else None
         bufs = evaluate_many(roots, self.device, deferred_sums=deferred_sums)
         return bufs[0], dict(zip(names, bufs[1:])), roots
 
