@@ -18,7 +18,7 @@ __global__ __launch_bounds__(256) void add_kernel(const T* __restrict__ a, const
       VecIO<T, VEC>::load(b + i, y);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) x[e] += y[e];
-      VecIO<T, VEC>::store(dst + i, x);
+      VecIO<T, VEC>::store_stream(dst + i, x);
     } else {
       for (int64_t j = i; j < n; ++j) dst[j] = from_float<T>(to_float(a[j]) + to_float(b[j]));
     }
@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void relu_kernel(const T* __restrict__ a, T* _
       VecIO<T, VEC>::load(a + i, x);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) x[e] = x[e] > 0.f ? x[e] : 0.f;
-      VecIO<T, VEC>::store(dst + i, x);
+      VecIO<T, VEC>::store_stream(dst + i, x);
     } else {
       for (int64_t j = i; j < n; ++j) dst[j] = to_float(a[j]) > 0.f ? a[j] : from_float<T>(0.f);
     }

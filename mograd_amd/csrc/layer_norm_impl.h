@@ -73,7 +73,7 @@ __global__ __launch_bounds__(WG) void ln_fwd_rows_kernel(const T* __restrict__ x
     for (int i = 0; i < VPT; ++i)
 #pragma unroll
       for (int e = 0; e < VEC; ++e) xv.v[i][e] = (xv.v[i][e] - mu) * rstd * g.v[i][e] + b.v[i][e];
-    xv.store(y + row * cols, t, cols);
+    xv.store_stream(y + row * cols, t, cols);
     if (mean_out != nullptr && t == 0) {
       mean_out[row] = mu;
       rstd_out[row] = rstd;
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
                                                          const float* __restrict__ rstd_in, const T* residual,
                                                          T* dx, float* __restrict__ part_g,
                                                          float* __restrict__ part_b, int64_t rows, int cols, float eps,
-                                                         int64_t rows_per_group) {
+                                                         int64_t rows_per_group, int64_t row_step) {
   constexpr int RPW = WG / TPR;
   constexpr int NW = WG / kWave;
   constexpr int TILE_COLS = VPT * TPR * VEC;
@@ -142,8 +142,11 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
   acc_g.zero();
   acc_b.zero();
 
-  const int64_t r_begin = static_cast<int64_t>(blockIdx.x) * rows_per_group;
-  const int64_t r_end = min(r_begin + rows_per_group, rows);
+  // row_step == RPW: the group's rows are consecutive; otherwise its rows lie row_step apart
+  // (the groups interleaved, every trip of the loop reading one contiguous band of the matrix).
+  const int64_t r_begin = row_step == RPW ? static_cast<int64_t>(blockIdx.x) * rows_per_group
+                                          : static_cast<int64_t>(blockIdx.x) * RPW;
+  const int64_t r_end = row_step == RPW ? min(r_begin + rows_per_group, rows) : rows;
   const float inv_n = 1.0f / static_cast<float>(cols);
 
   // With narrow per-thread tiles the next row is fetched while this row is reduced;
@@ -155,30 +158,44 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
   constexpr bool LOCKSTEP = TPR > kWave && RPW > 1;
   RowTile<T, VEC, TPR, VPT> xv, dyv, xn, dyn;
   int64_t row = r_begin + sub;
+  // The row's scalars travel with its tile: the saved statistics, or the row's first element
+  // (the shift of the one-pass sums), fetched a trip ahead like the tile itself.
+  float sc0 = 0.f, sc1 = 0.f, sc0_n = 0.f, sc1_n = 0.f;
+  auto load_scalars = [&](int64_t r, float& a, float& b) {
+    if constexpr (HAS_STATS) {
+      a = mean_in[r];
+      b = rstd_in[r];
+    } else {
+      a = to_float(x[r * cols]);
+    }
+  };
   if (PREFETCH && row < r_end) {
     xv.load(x + row * cols, t, cols);
     dyv.load(dy + row * cols, t, cols);
+    load_scalars(row, sc0, sc1);
   }
-  for (; LOCKSTEP ? row - sub < r_end : row < r_end; row += RPW) {
+  for (; LOCKSTEP ? row - sub < r_end : row < r_end; row += row_step) {
     const bool active = !LOCKSTEP || row < r_end;
     if (LOCKSTEP && !active) {
       xv.zero();
       dyv.zero();
     }
-    const int64_t next = row + RPW;
+    const int64_t next = row + row_step;
     if constexpr (PREFETCH) {
       if (next < r_end) {
         xn.load(x + next * cols, t, cols);
         dyn.load(dy + next * cols, t, cols);
+        load_scalars(next, sc0_n, sc1_n);
       }
     } else if (active) {
       xv.load(x + row * cols, t, cols);
       dyv.load(dy + row * cols, t, cols);
+      load_scalars(row, sc0, sc1);
     }
     float mu, rstd, c1, c2;
     if constexpr (HAS_STATS) {
-      mu = active ? mean_in[row] : 0.f;
-      rstd = active ? rstd_in[row] : 0.f;
+      mu = active ? sc0 : 0.f;
+      rstd = active ? sc1 : 0.f;
       // xhat replaces x; dy*gamma is formed on the fly.  Columns past `cols` hold zeros in
       // dy and gamma, so they add nothing to the sums.
       float s[2] = {0.f, 0.f};
@@ -199,7 +216,7 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
       // One reduction per row instead of two: with d = x - shift (the shift is the row's
       // first element, see row_stats) the four sums of d, d^2, dy*gamma and dy*gamma*d give
       // the statistics and, through xhat = (d - mean_d) * rstd, both row sums of the gradient.
-      const float shift = active ? to_float(x[row * cols]) : 0.f;
+      const float shift = active ? sc0 : 0.f;
       float s[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int i = 0; i < VPT; ++i) {
@@ -254,13 +271,15 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
             for (int e = 0; e < VEC; ++e) out[e] = to_float(from_float<T>(out[e])) + rs[e];
           }
         }
-        VecIO<T, VEC>::store(dx + row * cols + c, out);
+        VecIO<T, VEC>::store_stream(dx + row * cols + c, out);
       }
     }
     if constexpr (PREFETCH) {
       if (next < r_end) {
         xv = xn;
         dyv = dyn;
+        sc0 = sc0_n;
+        sc1 = sc1_n;
       }
     }
   }
@@ -315,7 +334,7 @@ __global__ __launch_bounds__(WG) void ln_bwd_rows_kernel(const T* __restrict__ d
         float sum = 0.f;
 #pragma unroll
         for (int r = 0; r < SETS; ++r) sum += combine[r * TILE_COLS + c];
-        out[c] = sum;
+        __builtin_nontemporal_store(sum, out + c);
       }
     }
   }
@@ -412,7 +431,8 @@ struct LayerNormOps {
   };
   // The backward keeps one wave per row from 33 chunks on: with three chunks per lane its five
   // row tiles no longer fit a 1024-thread workgroup, and sixteen-lane rows in smaller
-  // workgroups measured slower there ((16384, 384) bf16: 17.0 us against 14.3 us).
+  // workgroups measured slower there ((16384, 384) bf16, row kernel alone: 16.7 us with 256
+  // threads and 20.4 us with 512 against 13.8 us).
   static bool pick_shape_bwd(int64_t chunks, Shape* s) {
     if (chunks > 32 && chunks <= 64) {
       *s = {64, 1};
@@ -543,13 +563,22 @@ struct LayerNormOps {
     int64_t groups = bwd_groups(rows, RPW, WG);
     int64_t rows_per_group = ceil_div(ceil_div(rows, groups), RPW) * RPW;
     groups = ceil_div(rows, rows_per_group);
+    // Matrices of 16 MiB and more: the groups' rows interleaved, so that the workgroups of one
+    // trip read a contiguous band of x and dy and write one of dx (DRAM pages shared between
+    // neighbours: (16384, 1024) fp32 47.4 -> 43.6 us, (4096, 8192) bf16 62.8 -> 59.3 us,
+    // (2048, 4096) fp32 29.6 -> 28.5 us).  Smaller, cache-resident ones measure 1 % slower that
+    // way and keep consecutive rows.  MOGRAD_HIP_LN_INTERLEAVE=0/1 forces either.
+    const int il_knob = env_int("MOGRAD_HIP_LN_INTERLEAVE", -1);
+    const bool interleave =
+        il_knob < 0 ? rows * cols * static_cast<int64_t>(sizeof(T)) >= (int64_t{16} << 20) : il_knob != 0;
     Scratch part_g, part_b;
     MG_TRY(part_g.take(groups * cols * static_cast<int64_t>(sizeof(float))));
     MG_TRY(part_b.take(groups * cols * static_cast<int64_t>(sizeof(float))));
     hipLaunchKernelGGL((ln_bwd_rows_kernel<T, VEC, TPR, VPT, WG, HAS_STATS>), dim3(static_cast<unsigned>(groups)),
                        dim3(WG), 0, stream, dy, x, gamma, mean, rstd, residual, dx, part_g.as<float>(),
                        part_b.as<float>(), rows,
-                       static_cast<int>(cols), eps, rows_per_group);
+                       static_cast<int>(cols), eps, rows_per_group,
+                       interleave ? groups * RPW : static_cast<int64_t>(RPW));
     MG_LAUNCH_CHECK();
     reduce_partials_or_defer<T>(part_g, dgamma, &part_b, dbeta, groups, cols, device_info().cu_count, stream);
     MG_LAUNCH_CHECK();

@@ -58,6 +58,15 @@ __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) {
 template <typename T, int VEC>
 struct VecIO;
 
+// `store_stream` writes past the caches (a non-temporal store): for outputs that are written
+// once and read by a later kernel.  On buffers that are not cache-resident it is the faster form
+// for the row and elementwise kernels (LayerNorm backward (2048, 4096) fp32: 33.9 -> 28.8 us, a
+// 100 MB add 19.9 -> 15.6 us; no difference on cache-resident ones), but not for the
+// cross-entropy kernels, whose workgroups write a long row each (631 -> 889 us at (8192, 50304)),
+// and they keep the plain store.
+typedef float mg_f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t mg_u4 __attribute__((ext_vector_type(4)));
+
 template <>
 struct VecIO<float, 4> {
   static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
@@ -67,12 +76,17 @@ struct VecIO<float, 4> {
   static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
     *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
   }
+  static __device__ __forceinline__ void store_stream(float* p, const float (&v)[4]) {
+    const mg_f4 r = {v[0], v[1], v[2], v[3]};
+    __builtin_nontemporal_store(r, reinterpret_cast<mg_f4*>(p));
+  }
 };
 
 template <typename T>
 struct VecIO<T, 1> {
   static __device__ __forceinline__ void load(const T* p, float (&v)[1]) { v[0] = to_float(*p); }
   static __device__ __forceinline__ void store(T* p, const float (&v)[1]) { *p = from_float<T>(v[0]); }
+  static __device__ __forceinline__ void store_stream(T* p, const float (&v)[1]) { *p = from_float<T>(v[0]); }
 };
 
 template <>
@@ -99,6 +113,17 @@ struct VecIO<f16_t, 8> {
     }
     *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
   }
+  static __device__ __forceinline__ void store_stream(f16_t* p, const float (&v)[8]) {
+    mg_u4 w;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      union { uint32_t u; f16_t h[2]; } cv;
+      cv.h[0] = static_cast<f16_t>(v[2 * i]);
+      cv.h[1] = static_cast<f16_t>(v[2 * i + 1]);
+      w[i] = cv.u;
+    }
+    __builtin_nontemporal_store(w, reinterpret_cast<mg_u4*>(p));
+  }
 };
 
 template <>
@@ -118,6 +143,13 @@ struct VecIO<bf16_t, 8> {
     for (int i = 0; i < 4; ++i)
       w[i] = bf16_pack2_rne(v[2 * i], v[2 * i + 1]);
     *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+  static __device__ __forceinline__ void store_stream(bf16_t* p, const float (&v)[8]) {
+    mg_u4 w;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      w[i] = bf16_pack2_rne(v[2 * i], v[2 * i + 1]);
+    __builtin_nontemporal_store(w, reinterpret_cast<mg_u4*>(p));
   }
 };
 

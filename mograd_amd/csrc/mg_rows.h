@@ -56,6 +56,20 @@ struct RowTile {
       }
     }
   }
+  // The same with stores that bypass the caches (see VecIO::store_stream).
+  __device__ __forceinline__ void store_stream(T* row_ptr, int t, int cols) const {
+    const unsigned lane_off = static_cast<unsigned>(t) * VEC;
+    const int nfull = full_chunks(cols);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      T* chunk_base = row_ptr + i * (TPR * VEC);
+      if (i < nfull) {
+        VecIO<T, VEC>::store_stream(chunk_base + lane_off, v[i]);
+      } else if (i == nfull && col(i, t) < cols) {
+        VecIO<T, VEC>::store_stream(chunk_base + lane_off, v[i]);
+      }
+    }
+  }
   __device__ __forceinline__ void zero() {
 #pragma unroll
     for (int i = 0; i < VPT; ++i)
@@ -172,13 +186,13 @@ __device__ __forceinline__ void reduce_partials_slab_block(float* __restrict__ l
     const int64_t step = LANES * cols;
     int64_t g = ly;
     for (; g + LANES < groups; g += 2 * LANES, p += 2 * step) {
-      const float4 v0 = *reinterpret_cast<const float4*>(p);
-      const float4 v1 = *reinterpret_cast<const float4*>(p + step);
+      const mg_f4 v0 = __builtin_nontemporal_load(reinterpret_cast<const mg_f4*>(p));
+      const mg_f4 v1 = __builtin_nontemporal_load(reinterpret_cast<const mg_f4*>(p + step));
       a0.x += v0.x; a0.y += v0.y; a0.z += v0.z; a0.w += v0.w;
       a1.x += v1.x; a1.y += v1.y; a1.z += v1.z; a1.w += v1.w;
     }
     if (g < groups) {
-      const float4 v0 = *reinterpret_cast<const float4*>(p);
+      const mg_f4 v0 = __builtin_nontemporal_load(reinterpret_cast<const mg_f4*>(p));
       a0.x += v0.x; a0.y += v0.y; a0.z += v0.z; a0.w += v0.w;
     }
   }
