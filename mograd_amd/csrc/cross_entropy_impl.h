@@ -176,6 +176,92 @@ __global__ __launch_bounds__(WG, (TPR == 256 && VPT * VEC > 128) ? 2 : 1) void c
   }
 }
 
+// Integer labels, 16-bit logits, rows of thousands of columns: the row stays in
+// registers as loaded (eight 16-bit values per 128-bit register quad) and is unpacked in each of
+// its three passes (maximum, sum of exponentials, gradient), so a thread holds VPT * 4 registers
+// for VPT * 8 columns instead of VPT * 8: 200 fp32 values per thread next to the 100 registers
+// they were loaded into spill (656 bytes per lane at 50304 columns: 1.36 TB/s).  The second
+// exponential per element is free in a kernel that waits for memory.  The arithmetic per element
+// is that of ce_rows_kernel, so are the bits.  One row per workgroup.
+template <typename T, int TPR, int VPT>
+__global__ __launch_bounds__(TPR, TPR <= 256 ? 4 : (TPR <= 512 ? 2 : 1)) void ce_rows_packed_kernel(
+    const T* __restrict__ logits, const void* __restrict__ labels, const T* __restrict__ upstream,
+    float* __restrict__ rowloss, T* __restrict__ dlogits, int64_t N, int C, int id64) {
+  static_assert(sizeof(T) == 2, "16-bit element types");
+  constexpr int VEC = 8;
+  __shared__ float slots[2 * (TPR / kWave)];
+  const int t = threadIdx.x;
+  int phase = 0;
+  const float inv_rows = 1.0f / static_cast<float>(N);
+  const float scale = (upstream != nullptr ? to_float(upstream[0]) : 1.0f) * inv_rows;
+  const int64_t row = blockIdx.x;
+  const T* xr = logits + row * C;
+  T* out_row = dlogits + row * C;
+  const int nfull = (C / VEC) / TPR;  // chunk indices below it exist for every thread
+  const bool tail = (nfull * TPR + t) * VEC < C;  // this thread's chunk `nfull` exists
+
+  uint4 raw[VPT];
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    raw[i] = make_uint4(0, 0, 0, 0);
+    if (i < nfull || (i == nfull && tail)) raw[i] = *reinterpret_cast<const uint4*>(xr + (i * TPR + t) * VEC);
+  }
+  float m[1] = {-INFINITY};
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    if (i < nfull || (i == nfull && tail)) {
+      float x[VEC];
+      VecIO<T, VEC>::load(reinterpret_cast<const T*>(&raw[i]), x);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) m[0] = fmaxf(m[0], x[e]);
+    }
+  }
+  row_allreduce_max<TPR, TPR, 1>(m, slots, phase);
+  const float m2 = m[0] * kLog2e;
+  // Between the passes the packed registers are made opaque to the compiler, which would
+  // otherwise keep the unpacked values of one pass for the next.
+  auto forget = [&]() {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) asm volatile("" : "+v"(raw[i].x), "+v"(raw[i].y), "+v"(raw[i].z), "+v"(raw[i].w));
+  };
+  forget();
+  float s[1] = {0.f};
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    if (i < nfull || (i == nfull && tail)) {
+      float x[VEC];
+      VecIO<T, VEC>::load(reinterpret_cast<const T*>(&raw[i]), x);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) s[0] += fast_exp2(fmaf(x[e], kLog2e, -m2));
+    }
+  }
+  row_allreduce_sum<TPR, TPR, 1>(s, slots, phase);
+  const float k = scale / s[0];
+  forget();
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    if (i < nfull || (i == nfull && tail)) {
+      float x[VEC];
+      VecIO<T, VEC>::load(reinterpret_cast<const T*>(&raw[i]), x);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) x[e] = fast_exp2(fmaf(x[e], kLog2e, -m2)) * k;
+      VecIO<T, VEC>::store(out_row + (i * TPR + t) * VEC, x);
+    }
+  }
+  // the "- 1" at the label column: a scalar store by the thread that owns the column, after its
+  // vector stores (same thread, same address: program order holds)
+  const int64_t id = load_id(labels, row, id64 != 0);
+  const bool id_ok = id >= 0 && id < C;
+  if (id_ok && (static_cast<int>(id) / VEC) % TPR == t) {
+    const float xl = to_float(xr[id]);
+    const float lp = xl - m[0] - logf(s[0]);  // log softmax at the label
+    out_row[id] = from_float<T>((fast_exp2(fmaf(xl, kLog2e, -m2)) / s[0] - 1.0f) * scale);
+    if (rowloss != nullptr) rowloss[row] = -lp * inv_rows;
+  }
+  // An id outside [0, C) selects no column: the row's loss term is flagged NaN.
+  if (rowloss != nullptr && !id_ok && t == 0) rowloss[row] = NAN;
+}
+
 // ------------------------------------------------------------------------------------
 // Streaming kernels: any C, any alignment.  One workgroup per row.
 // ------------------------------------------------------------------------------------
@@ -552,6 +638,37 @@ struct CrossEntropyOps {
       return finish_loss(rowloss, loss, N, stream);
     }
     Shape s;
+    if constexpr (sizeof(T) == 2 && !DENSE) {
+      // 16-bit rows of more than 512 chunks (4096 columns) with integer labels: the packed row
+      // kernel ((8192, 50304) bf16 1220 -> 344 us, (16384, 16392) 415 -> 209 us, (65536, 4104)
+      // 275 -> 205 us, (32768, 8192) 197 us either way).  MOGRAD_HIP_CE_PACKED=0: the fp32 tiles.
+      const int64_t chunks = C / WIDE;
+      if (wide && chunks > 512 && chunks <= 16384 && dlogits != nullptr && env_int("MOGRAD_HIP_CE_PACKED", 1) != 0) {
+        const unsigned grid = static_cast<unsigned>(N);
+        const int Ci = static_cast<int>(C);
+        if (chunks <= 1024)
+          hipLaunchKernelGGL((ce_rows_packed_kernel<T, 256, 4>), dim3(grid), dim3(256), 0, stream, logits, labels, upstream,
+                             rowloss, dlogits, N, Ci, id64);
+        else if (chunks <= 2048)
+          hipLaunchKernelGGL((ce_rows_packed_kernel<T, 256, 8>), dim3(grid), dim3(256), 0, stream, logits, labels, upstream,
+                             rowloss, dlogits, N, Ci, id64);
+        else if (chunks <= 4096)
+          hipLaunchKernelGGL((ce_rows_packed_kernel<T, 256, 16>), dim3(grid), dim3(256), 0, stream, logits, labels, upstream,
+                             rowloss, dlogits, N, Ci, id64);
+        else if (chunks <= 6400)
+          hipLaunchKernelGGL((ce_rows_packed_kernel<T, 256, 25>), dim3(grid), dim3(256), 0, stream, logits, labels, upstream,
+                             rowloss, dlogits, N, Ci, id64);
+        else if (chunks <= 12800)
+          hipLaunchKernelGGL((ce_rows_packed_kernel<T, 512, 25>), dim3(grid), dim3(512), 0, stream, logits, labels, upstream,
+                             rowloss, dlogits, N, Ci, id64);
+        else
+          hipLaunchKernelGGL((ce_rows_packed_kernel<T, 1024, 16>), dim3(grid), dim3(1024), 0, stream, logits, labels,
+                             upstream, rowloss, dlogits, N, Ci, id64);
+        MG_LAUNCH_CHECK();
+        if (loss != nullptr) return finish_loss(rowloss, loss, N, stream);
+        return MG_OK;
+      }
+    }
     if (wide && pick_shape(C / WIDE, true, &s)) {
       MG_TRY((dispatch_rows<WIDE, DENSE>(s, logits, labels, upstream, rowloss, dlogits, N, C, id64, stream)));
     } else if (!wide && pick_shape(C, false, &s)) {

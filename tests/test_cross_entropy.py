@@ -221,6 +221,30 @@ def test_half_precision_storage(device, dtype, rtol, N, Cc):
     assert_close(_ce_grad(device, x, one_hot, up, dtype=dtype), want, rtol, floor, "dense dlogits")
 
 
+@pytest.mark.parametrize("dtype,rtol", [(F16, 2e-3), (BF16, 1.6e-2)])
+@pytest.mark.parametrize("N,Cc", [(5, 50304), (3, 40008), (2, 70000), (2, 110000), (3, 32776), (9, 4104), (7, 12000),
+                                  (4, 24000), (6, 8192)])
+def test_wide_16bit_rows_stay_packed(device, monkeypatch, dtype, rtol, N, Cc):
+    # 16-bit rows of 4104 to 131072 columns with integer labels stay in registers as loaded
+    # and are unpacked once per pass (256, 512 or 1024 threads per row); MOGRAD_HIP_CE_PACKED=0
+    # holds them as fp32.  The arithmetic per element is the same: same bits; both meet the oracle.
+    x = round_to_dtype(normal(35, 0, (N, Cc), std=2.0), dtype)
+    ids = integers(35, 1, (N,), 0, Cc)
+    ids[0] = Cc - 1  # a label in the row's last, possibly partial, chunk
+    got = {}
+    for knob in ("1", "0"):
+        monkeypatch.setenv("MOGRAD_HIP_CE_PACKED", knob)
+        got[knob] = _ids_calls(device, x, ids, 1.0, I32, dtype)
+    want_loss, want = O.cross_entropy_ids(x, ids), O.cross_entropy_grad_ids(x, ids, 1.0)
+    for knob, (loss, grad, loss2, grad2) in got.items():
+        assert_close(loss2, want_loss, rtol, rtol, f"fused loss ({knob})")
+        assert_close(grad, want, rtol, rtol / N, f"dlogits ({knob})")
+        assert_close(grad2, want, rtol, rtol / N, f"fused dlogits ({knob})")
+    np.testing.assert_array_equal(got["1"][1], got["0"][1])
+    np.testing.assert_array_equal(got["1"][3], got["0"][3])
+    assert got["1"][2] == got["0"][2]
+
+
 def test_out_of_range_id_flags_loss(device):
     x = normal(34, 0, (4, 100))
     ids = np.array([0, 5, 100, 7], np.int32)
