@@ -184,7 +184,7 @@ __global__ __launch_bounds__(WG, (TPR == 256 && VPT * VEC > 128) ? 2 : 1) void c
 // exponential per element is free in a kernel that waits for memory.  The arithmetic per element
 // is that of ce_rows_kernel, so are the bits.  One row per workgroup.
 template <typename T, int TPR, int VPT>
-__global__ __launch_bounds__(TPR, TPR <= 256 ? 4 : (TPR <= 512 ? 2 : 1)) void ce_rows_packed_kernel(
+__global__ __launch_bounds__(TPR, TPR <= 256 ? (VPT > 16 ? 3 : 4) : (TPR <= 512 ? 2 : 1)) void ce_rows_packed_kernel(
     const T* __restrict__ logits, const void* __restrict__ labels, const T* __restrict__ upstream,
     float* __restrict__ rowloss, T* __restrict__ dlogits, int64_t N, int C, int id64) {
   static_assert(sizeof(T) == 2, "16-bit element types");
