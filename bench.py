@@ -1013,7 +1013,62 @@ def bench_ln_ce(args, dev) -> dict:
     return result
 
 
-WORKLOADS = {"ln_ce": bench_ln_ce, "mlp": bench_mlp, "attention": bench_attention, "gpt": bench_gpt}
+def bench_gemm16(args, dev) -> dict:
+    """The 16-bit GEMM core away from the GPT step's short shapes: forward, dX and dW of a square
+    bf16 Linear layer at 8192 and 4096 (no BASELINE configuration; `--workload gemm16` only, not
+    part of the default run).  A step is the three products at 8192."""
+    from mograd_amd import BF16, AnyBuffer
+
+    lib, st = dev.lib, dev.stream
+    P = lambda b: b.data_ptr()  # noqa: E731
+    entries, keep = [], []
+    for n in (8192, 4096):
+        x, w, dy = (AnyBuffer.from_numpy(dev, _rng(6, 10 * i + n % 7).standard_normal(n * n, dtype=np.float32) * sc, BF16)
+                    for i, sc in ((0, 1.0), (1, 0.02), (2, 1.0)))
+        y, dx, dw = (AnyBuffer.create(BF16, dev, n * n) for _ in range(3))
+        keep += [x, w, dy, y, dx, dw]
+        fl = 2.0 * n * n * n
+        entries += [
+            (f"Y = X W^T bf16 {n}^3 (mg_matmul_bt)",
+             lambda i, x=x, w=w, y=y, n=n: lib.mg_matmul_bt(P(x), P(w), P(y), 1, n, n, n, n, 1, n, 1, n * n, n * n, BF16, st),
+             fl, "F", MFMA_BF16_PEAK_TFLOPS),
+            (f"dX = dY W bf16 {n}^3 (mg_linear_bwd, dx only)",
+             lambda i, x=x, w=w, dy=dy, dx=dx, n=n: lib.mg_linear_bwd(P(dy), P(x), P(w), P(dx), None, None, n, n, n, BF16, st),
+             fl, "F", MFMA_BF16_PEAK_TFLOPS),
+            (f"dW = dY^T X bf16 {n}^3 (mg_linear_bwd, dw only)",
+             lambda i, x=x, w=w, dy=dy, dw=dw, n=n: lib.mg_linear_bwd(P(dy), P(x), P(w), None, P(dw), None, n, n, n, BF16, st),
+             fl, "F", MFMA_BF16_PEAK_TFLOPS),
+        ]
+    # sampled rows of the 4096^3 forward against float64
+    n = 4096
+    x, w, y = keep[6], keep[7], keep[9]
+    entries[3][1](0)
+    dev.synchronize()
+    rows = [0, n // 3, n - 1]
+    want = x.to_numpy((n, n))[rows].astype(np.float64) @ w.to_numpy((n, n)).astype(np.float64).T
+    _check("gemm16 Y = X W^T", y.to_numpy((n, n))[rows], want, 2e-2)
+
+    def step(i):
+        for e in entries[:3]:
+            e[1](i)
+
+    ms = _time_steps(dev, step, min(args.warmup, 3), min(args.steps, 20))
+    kernels = _kernel_table(dev, entries, 10)
+    dom = min(kernels[:3], key=lambda r: r["frac_of_mfma_peak"])
+    return {
+        "metric": "fwd+bwd step ms; per-bwd-kernel HBM GB/s or MFMA % of MI355X peak", "value": round(ms, 4), "unit": "ms",
+        "n_gpus": 1, "steps": min(args.steps, 20), "warmup": min(args.warmup, 3), "ms_per_step": round(ms, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "bf16 Linear 8192 -> 8192 on 8192 rows: forward, dX and dW products (gemm_16bit_big_kernel), "
+                               "N(0,1) activations and gradients; the same at 4096 in the kernel table"},
+        "roofline": {"bound": "mfma", "kernel": "gemm_16bit_big_kernel, " + dom["name"], "achieved": dom["achieved_TFLOPs"],
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac_of_mfma_peak"], "traffic": None},
+        "kernels": kernels,
+    }
+
+
+# "all" runs the four BASELINE configurations; gemm16 is an extra, by name only.
+WORKLOADS = {"ln_ce": bench_ln_ce, "mlp": bench_mlp, "attention": bench_attention, "gpt": bench_gpt, "gemm16": bench_gemm16}
 
 
 def main() -> int:
@@ -1026,7 +1081,7 @@ def main() -> int:
                     help="all (default): every configuration in one process, the GPT training step as the headline "
                          "and the others under 'workloads'; ln_ce: LayerNorm + fused cross-entropy fp32; mlp: README "
                          "MLP fwd+bwd fp32 (matmul_bias_bt, dX, dW, db); attention: bf16 flash attention fwd+bwd; "
-                         "gpt: the training step alone")
+                         "gpt: the training step alone; gemm16: large square bf16 products (an extra, not in 'all')")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path runs on one GPU; --gpus N with N > 1 is not supported "
