@@ -720,6 +720,9 @@ inline Buffers reshape(const OpRef& node, const Buffers& inputs, Device& device)
 
 // TRANSPOSE[a]{dim0, dim1}: a strided view of the same storage.
 inline Buffers transpose(const OpRef& node, const Buffers& inputs, Device&) { return {inputs[0].view(node.layout())}; }
+// EXPAND[a]: a broadcast view, stride 0 along the expanded axes (what grad.mojo:156-177 builds as
+// the gradient of SUM); consumers materialise it with mg_contiguous.
+inline Buffers expand(const OpRef& node, const Buffers& inputs, Device&) { return {inputs[0].view(node.layout())}; }
 
 // FLASH_ATTN_PACKED[qkv (B, S, 3, H, D)(, mask)]{scale, is_causal, has_bias} -> [O (B, S, H, D), LSE (B, H, S) f32].
 inline Buffers flash_attn_packed_fwd(const OpRef& node, const Buffers& inputs, Device& device) {
@@ -946,6 +949,7 @@ inline const std::vector<Rule>& scheduler_rules() {
       // views, and the fused nodes that the rewrite rules below create
       {"RESHAPE", "reshape", reshape},
       {"TRANSPOSE", "transpose", transpose},
+      {"EXPAND", "expand", expand},
       {"MATMUL_BT_ADD", "matmul_bt_add", matmul_bt_add},
       {"MATMUL_BIAS_RELU_BT", "matmul_bias_relu_bt", matmul_bias_relu_bt},
       {"LAYER_NORM_STATS_GRAD_ADD", "layer_norm_bwd_stats", layer_norm_bwd_stats},

@@ -785,6 +785,13 @@ def transpose(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBu
     return [inputs[0].view(node.layout())]
 
 
+def expand(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """EXPAND[a]: a broadcast view, stride 0 along the expanded axes (runtime/__init__.mojo, the view
+    ops; grad.mojo:156-177 builds it as the gradient of SUM).  A consumer that needs rows in memory
+    materialises it with mg_contiguous, which reads stride-0 views."""
+    return [inputs[0].view(node.layout())]
+
+
 def flash_attn_packed_fwd(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     """FLASH_ATTN_PACKED[qkv (B, S, 3, H, D), mask]{scale, is_causal, has_bias} -> [O (B, S, H, D),
     LSE (B, H, S) f32]: Q, K and V are the three slices of one projection's output, and O comes out
@@ -878,6 +885,7 @@ SCHEDULER_RULES = {
     # views, and the fused nodes that mograd_amd.rewrites.GPU_REWRITES creates
     "RESHAPE": reshape,
     "TRANSPOSE": transpose,
+    "EXPAND": expand,
     "MATMUL_BT_ADD": matmul_bt_add,
     "MATMUL_BIAS_RELU_BT": matmul_bias_relu_bt,
     "LAYER_NORM_STATS_GRAD_ADD": layer_norm_bwd_stats,
@@ -1013,6 +1021,39 @@ def softmax_grad_rule(node: Node, upstream: Node) -> List[Optional[Node]]:
     return [Node("SOFTMAX_GRAD", node.layout().as_contiguous(), node.dtype(), [node, upstream])]
 
 
+def sum_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """mograd/grad.mojo:156-177: the upstream broadcast back over the summed axis, an EXPAND view
+    with stride 0 there (every stride 0 for the full reduction)."""
+    shape = node.src(0).layout().shape()
+    up = upstream.layout()
+    if "axis" not in node.attrs():
+        strides = [0] * len(shape)
+    else:
+        ax = int(node.attrs()["axis"]) % len(shape)
+        if up.rank() == len(shape):  # keepdim: the size-1 axis is expanded in place
+            strides = [0 if i == ax else up.stride(i) for i in range(len(shape))]
+        else:
+            strides = list(up.stride())
+            strides.insert(ax, 0)
+    return [Node("EXPAND", Layout(*shape, strides=strides, base_offset=up.base_offset), node.dtype(), [upstream])]
+
+
+def expand_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
+    """mograd/grad.mojo:278-288: the upstream summed over the leading axes that EXPAND added and,
+    keeping the dimension, over every axis it widened."""
+    src, out = node.src(0).layout(), node.layout()
+    grad = upstream
+    for _ in range(out.rank() - src.rank()):
+        dims = grad.layout().shape()
+        grad = Node("SUM", Layout(*dims[1:]), grad.dtype(), [grad], {"axis": 0})
+    for i in range(src.rank()):
+        if src.shape(i) != grad.layout().shape(i):
+            dims = list(grad.layout().shape())
+            dims[i] = 1
+            grad = Node("SUM", Layout(*dims), grad.dtype(), [grad], {"axis": i, "keepdim": True})
+    return [grad]
+
+
 def reshape_grad(node: Node, upstream: Node) -> List[Optional[Node]]:
     """mograd/grad.mojo (reshape_grad): the upstream under the source's shape."""
     src = node.src(0)
@@ -1056,6 +1097,8 @@ GRAD_RULES = {
     "SOFTMAX": softmax_grad_rule,
     "RESHAPE": reshape_grad,
     "TRANSPOSE": transpose_grad,
+    "SUM": sum_grad,
+    "EXPAND": expand_grad,
     "FLASH_ATTN_PACKED": flash_attn_packed_grad,
 }
 

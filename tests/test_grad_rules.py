@@ -85,6 +85,51 @@ def _leaf(device, a, dtype=F32):
     return Node.leaf(Layout(*a.shape), dtype, AnyBuffer.from_numpy(device, a, dtype))
 
 
+def test_sum_and_expand_rules_are_each_others_gradient():
+    # sum_grad (mograd/grad.mojo:156-177): the upstream as an EXPAND view with stride 0 along the
+    # summed axis; expand_grad (:278-288): sums back over what EXPAND added or widened.
+    x = Node.leaf(Layout(5, 7, 3))
+    for axis, keep, up_shape, strides in ((1, False, (5, 3), (3, 0, 1)), (0, False, (7, 3), (0, 3, 1)),
+                                          (2, True, (5, 7, 1), (7, 1, 0))):
+        attrs = {"axis": axis, "keepdim": True} if keep else {"axis": axis}
+        y = Node("SUM", Layout(*up_shape), F32, [x], attrs)
+        (dx,) = R.gradient(y, Node.leaf(Layout(*up_shape)), [x])
+        assert dx.op_type == "EXPAND" and dx.layout().shape() == (5, 7, 3) and dx.layout().stride() == strides
+    full = Node("SUM", Layout(1), F32, [x])
+    (dx,) = R.gradient(full, Node.leaf(Layout(1)), [x])
+    assert dx.layout().stride() == (0, 0, 0)
+    # EXPAND of a bias row over the rows of a matrix: its gradient is the column sum
+    b = Node.leaf(Layout(6))
+    e = Node("EXPAND", Layout(4, 6, strides=(0, 1)), F32, [b])
+    (db,) = R.gradient(e, Node.leaf(Layout(4, 6)), [b])
+    assert db.op_type == "SUM" and db.attrs()["axis"] == 0 and db.layout().shape() == (6,)
+    # a widened size-1 axis keeps its dimension
+    c = Node.leaf(Layout(4, 1))
+    e2 = Node("EXPAND", Layout(4, 6, strides=(1, 0)), F32, [c])
+    (dc,) = R.gradient(e2, Node.leaf(Layout(4, 6)), [c])
+    assert dc.op_type == "SUM" and dc.attrs()["axis"] == 1 and dc.layout().shape() == (4, 1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", [(64, 40, 256), (300, 136, 72)])
+def test_sum_gradient_through_a_linear_layer(device, M, N, K):
+    # s = sum over rows of (X W^T); ds/dX and ds/dW for an upstream g over the N columns: the
+    # EXPAND view that sum_grad builds is materialised by the Linear backward's exec function.
+    x, w, g = normal(66, 0, (M, K)), normal(66, 1, (N, K), std=0.1), normal(66, 2, (N,))
+    nx, nw = (Node.leaf(Layout(*a.shape), F32, AnyBuffer.from_numpy(device, a)) for a in (x, w))
+    h = Node("MATMUL_BT", Layout(M, N), F32, [nx, nw])
+    s_ = Node("SUM", Layout(N), F32, [h], {"axis": 0})
+    up = Node.leaf(Layout(N), F32, AnyBuffer.from_numpy(device, g))
+    dx, dw = R.gradient(s_, up, [nx, nw])
+    got_dx, got_dw = (b.to_numpy(shape) for b, shape in zip(R.evaluate_many([dx, dw], device), ((M, K), (N, K))))
+    g64, x64, w64 = g.astype(np.float64), x.astype(np.float64), w.astype(np.float64)
+    want_dx = np.broadcast_to(g64 @ w64, (M, K))
+    want_dw = np.outer(g64, x64.sum(axis=0))
+    assert_close(got_dx, want_dx, RTOL_F32, RTOL_F32 * np.abs(want_dx).max(), "dx")
+    assert_close(got_dw, want_dw, RTOL_F32, RTOL_F32 * np.abs(want_dw).max(), "dw")
+    assert_close(R.evaluate(s_, device).to_numpy(), (x64 @ w64.T).sum(axis=0), RTOL_F32, RTOL_F32 * M, "sum")
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("M,N,K", [(64, 10, 256), (200, 136, 260), (512, 384, 384)])
 def test_linear_gradient_through_the_rule(device, M, N, K):
