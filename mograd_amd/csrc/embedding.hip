@@ -6,9 +6,9 @@
 // That costs rows x indices comparisons, fine for a 65-row table and hopeless for a 50304-row
 // one; large tables first sort (row, position) pairs by row (a stable radix sort, so
 // positions stay ascending inside a row), and a wave then adds only its own row's run.
+#include <algorithm>
 #include <cstring>
-
-#include <rocprim/device/device_radix_sort.hpp>
+#include <utility>
 
 #include "mg_device.h"
 #include "mg_internal.h"
@@ -99,6 +99,122 @@ __global__ __launch_bounds__(256) void scatter_keys_kernel(const I* __restrict__
   pos[i] = static_cast<uint32_t>(i);
 }
 
+// ---- stable radix sort of (key, pos) pairs, eight bits of the key per pass --------------------
+// A pass is three steps: the digit histogram of every tile of the list, an exclusive scan of
+// the histograms in (digit, tile) order (per digit over the tiles, then over the digits'
+// totals), and the scatter, in which a tile places its pairs behind its digit's offset in their
+// order of appearance.  Counts are integer sums, so nothing
+// depends on scheduling; equal keys keep their order in every pass, so after the last one the
+// positions are ascending inside a key.
+
+// hist[d * tiles + tile] = number of keys of the tile (256 * items consecutive pairs) with digit d
+__global__ __launch_bounds__(256) void sort_hist_kernel(const uint32_t* __restrict__ key, uint32_t* __restrict__ hist,
+                                                        int64_t n, int shift, int items, int tiles) {
+  __shared__ uint32_t h[256];
+  h[threadIdx.x] = 0;
+  __syncthreads();
+  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * 256 * items;
+  for (int e = 0; e < items; ++e) {
+    const int64_t i = t0 + static_cast<int64_t>(e) * 256 + threadIdx.x;
+    if (i < n) atomicAdd(&h[(key[i] >> shift) & 255u], 1u);
+  }
+  __syncthreads();
+  hist[static_cast<int64_t>(threadIdx.x) * tiles + blockIdx.x] = h[threadIdx.x];
+}
+
+// Workgroup d turns digit d's row of counts, hist[d * tiles ..], into its exclusive scan over
+// the tiles, 256 at a time, and leaves the digit's total in hist[256 * tiles + d].
+__global__ __launch_bounds__(256) void sort_scan_kernel(uint32_t* __restrict__ hist, int tiles) {
+  __shared__ uint32_t part[256];
+  uint32_t* row = hist + static_cast<int64_t>(blockIdx.x) * tiles;
+  uint32_t carry = 0;
+  for (int t0 = 0; t0 < tiles; t0 += 256) {
+    const int t = t0 + threadIdx.x;
+    const uint32_t c = t < tiles ? row[t] : 0u;
+    part[threadIdx.x] = c;
+    __syncthreads();
+    for (int d = 1; d < 256; d *= 2) {  // inclusive scan of the 256 counts
+      const uint32_t v = threadIdx.x >= static_cast<unsigned>(d) ? part[threadIdx.x - d] : 0u;
+      __syncthreads();
+      part[threadIdx.x] += v;
+      __syncthreads();
+    }
+    if (t < tiles) row[t] = carry + part[threadIdx.x] - c;
+    carry += part[255];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) hist[static_cast<int64_t>(256) * tiles + blockIdx.x] = carry;
+}
+
+// The pairs of a tile go behind hist[digit * tiles + tile], 256 at a time in their order: a
+// pair's rank among the round's pairs with its digit is the number of lower lanes of its wave
+// with that digit (eight ballots) plus the lower waves' counts of it.  The digit's offset is the
+// total of the lower digits plus the digit's count in the tiles before; with RAW the histograms
+// are still counts and every workgroup sums them itself (lists of few tiles: 256 * tiles reads
+// a workgroup cost less than a launch of the scan).
+template <bool RAW>
+__global__ __launch_bounds__(256) void sort_scatter_kernel(const uint32_t* __restrict__ key, const uint32_t* __restrict__ pos,
+                                                           uint32_t* __restrict__ key_out, uint32_t* __restrict__ pos_out,
+                                                           const uint32_t* __restrict__ hist, int64_t n, int shift,
+                                                           int items, int tiles) {
+  __shared__ uint32_t base[256];
+  __shared__ uint32_t wcount[4][256];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  {
+    uint32_t total = 0, before = 0;  // of this thread's digit: in all tiles, in the tiles before this one
+    if constexpr (RAW) {
+      for (int t = 0; t < tiles; ++t) {
+        const uint32_t c = hist[static_cast<int64_t>(threadIdx.x) * tiles + t];
+        total += c;
+        before += t < static_cast<int>(blockIdx.x) ? c : 0u;
+      }
+    } else {
+      total = hist[static_cast<int64_t>(256) * tiles + threadIdx.x];
+      before = hist[static_cast<int64_t>(threadIdx.x) * tiles + blockIdx.x];
+    }
+    uint32_t* scan = wcount[0];
+    scan[threadIdx.x] = total;
+    __syncthreads();
+    for (int d = 1; d < 256; d *= 2) {
+      const uint32_t v = threadIdx.x >= static_cast<unsigned>(d) ? scan[threadIdx.x - d] : 0u;
+      __syncthreads();
+      scan[threadIdx.x] += v;
+      __syncthreads();
+    }
+    base[threadIdx.x] = scan[threadIdx.x] - total + before;
+    __syncthreads();
+  }
+  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * 256 * items;
+  for (int e = 0; e < items; ++e) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) wcount[w][threadIdx.x] = 0;
+    __syncthreads();
+    const int64_t i = t0 + static_cast<int64_t>(e) * 256 + threadIdx.x;
+    const bool valid = i < n;
+    const uint32_t k = valid ? key[i] : 0u;
+    const uint32_t d = (k >> shift) & 255u;
+    uint64_t same = __ballot(valid);
+#pragma unroll
+    for (int bit = 0; bit < 8; ++bit) {
+      const bool one = (d >> bit) & 1u;
+      const uint64_t m = __ballot(one);
+      same &= one ? m : ~m;
+    }
+    const uint32_t below = static_cast<uint32_t>(__popcll(same & ((uint64_t{1} << lane) - 1)));
+    if (valid && below == 0) wcount[wave][d] = static_cast<uint32_t>(__popcll(same));
+    __syncthreads();
+    if (valid) {
+      uint32_t r = base[d] + below;
+      for (int w = 0; w < wave; ++w) r += wcount[w][d];
+      key_out[r] = k;
+      pos_out[r] = pos[i];
+    }
+    __syncthreads();
+    base[threadIdx.x] += wcount[0][threadIdx.x] + wcount[1][threadIdx.x] + wcount[2][threadIdx.x] + wcount[3][threadIdx.x];
+    __syncthreads();
+  }
+}
+
 // Runs of equal keys in the sorted list: row k's value rows are pos[first[k] .. last[k]).
 // `first` and `last` hold zeros on entry, so a row without values gets an empty run.
 __global__ __launch_bounds__(256) void scatter_runs_kernel(const uint32_t* __restrict__ key, uint32_t* __restrict__ first,
@@ -138,29 +254,46 @@ __global__ __launch_bounds__(64) void scatter_runs_sum_kernel(const uint32_t* __
 template <typename T, typename I, int VEC>
 static int scatter_bucketed(const I* indices, const T* values, T* dst, int64_t n_idx, int64_t num_rows, int64_t row_size,
                             hipStream_t s) {
-  const unsigned n = static_cast<unsigned>(n_idx);
-  unsigned bits = 1;
+  int bits = 1;
   while (bits < 32 && (int64_t{1} << bits) <= num_rows) ++bits;  // keys are 0 .. num_rows
-  size_t sort_bytes = 0;
-  MG_HIP(rocprim::radix_sort_pairs(nullptr, sort_bytes, static_cast<uint32_t*>(nullptr), static_cast<uint32_t*>(nullptr),
-                                   static_cast<uint32_t*>(nullptr), static_cast<uint32_t*>(nullptr), n, 0, bits, s));
-  // one block: key, pos, sorted key, sorted pos (n each), first, last (num_rows + 1 each), sort scratch
-  const int64_t ints = 4 * n_idx + 2 * (num_rows + 1);
-  const int64_t ints_padded = ceil_div(ints, 64) * 64;
+  const int passes = (bits + 7) / 8;
+  // tiles of 256 * items pairs: four pairs per thread while that fills the chip, more for long
+  // lists (a tile's pairs of one digit land next to each other, and every tile costs 256
+  // counters); MOGRAD_HIP_SCATTER_SORT_MAX_TILES moves the limit
+  const int64_t max_tiles = std::max(1, env_int("MOGRAD_HIP_SCATTER_SORT_MAX_TILES", 1024));
+  const int items = static_cast<int>(std::max<int64_t>(4, ceil_div(n_idx, 256 * max_tiles)));
+  const int tiles = static_cast<int>(ceil_div(n_idx, int64_t{256} * items));
+  // one block: key, pos, their second copies (n each), first, last (num_rows + 1 each), the histograms
+  const int64_t ints = 4 * n_idx + 2 * (num_rows + 1) + int64_t{256} * (tiles + 1);
   Scratch work;
-  MG_TRY(work.take(ints_padded * 4 + static_cast<int64_t>(sort_bytes)));
+  MG_TRY(work.take(ints * 4));
   uint32_t* key = work.as<uint32_t>();
   uint32_t* pos = key + n_idx;
-  uint32_t* key_sorted = pos + n_idx;
-  uint32_t* pos_sorted = key_sorted + n_idx;
-  uint32_t* first = pos_sorted + n_idx;
+  uint32_t* key2 = pos + n_idx;
+  uint32_t* pos2 = key2 + n_idx;
+  uint32_t* first = pos2 + n_idx;
   uint32_t* last = first + num_rows + 1;
-  void* sort_tmp = key + ints_padded;
+  uint32_t* hist = last + num_rows + 1;
   const unsigned blocks = static_cast<unsigned>(ceil_div(n_idx, 256));
   MG_TRY(mg_fill(first, 0.0, 2 * (num_rows + 1), MG_I32, s));
   hipLaunchKernelGGL((scatter_keys_kernel<I>), dim3(blocks), dim3(256), 0, s, indices, key, pos, n_idx, num_rows);
   MG_LAUNCH_CHECK();
-  MG_HIP(rocprim::radix_sort_pairs(sort_tmp, sort_bytes, key, key_sorted, pos, pos_sorted, n, 0, bits, s));
+  for (int p = 0; p < passes; ++p) {
+    hipLaunchKernelGGL(sort_hist_kernel, dim3(tiles), dim3(256), 0, s, key, hist, n_idx, 8 * p, items, tiles);
+    if (tiles <= 64) {
+      hipLaunchKernelGGL(sort_scatter_kernel<true>, dim3(tiles), dim3(256), 0, s, key, pos, key2, pos2, hist, n_idx, 8 * p,
+                         items, tiles);
+    } else {
+      hipLaunchKernelGGL(sort_scan_kernel, dim3(256), dim3(256), 0, s, hist, tiles);
+      hipLaunchKernelGGL(sort_scatter_kernel<false>, dim3(tiles), dim3(256), 0, s, key, pos, key2, pos2, hist, n_idx, 8 * p,
+                         items, tiles);
+    }
+    MG_LAUNCH_CHECK();
+    std::swap(key, key2);
+    std::swap(pos, pos2);
+  }
+  uint32_t* key_sorted = key;
+  uint32_t* pos_sorted = pos;
   hipLaunchKernelGGL(scatter_runs_kernel, dim3(blocks), dim3(256), 0, s, key_sorted, first, last, n_idx);
   MG_LAUNCH_CHECK();
   const dim3 grid(static_cast<unsigned>(num_rows), static_cast<unsigned>(ceil_div(row_size, 64 * VEC)));

@@ -186,6 +186,26 @@ def test_scatter_add_vocabulary_sized_table(device):
     np.testing.assert_array_equal(hist[:, 0], np.bincount(idx, minlength=V).astype(np.float32))
 
 
+@pytest.mark.parametrize("max_tiles", [16384, 5, 1])
+@pytest.mark.parametrize("idx_dtype", [I32, I64])
+@pytest.mark.parametrize("V,n", [(70000, 200000), (300, 1031), (65536, 40000), (1 << 16 | 1, 9000)])
+def test_scatter_add_sort_places_every_pair_once(device, monkeypatch, idx_dtype, V, n, max_tiles):
+    # The bucketing sort is a radix sort of (row, position) pairs, eight bits a pass: tables of
+    # up to 256, 65536 and more rows take one, two and three passes, a list of more than 1024
+    # pairs takes several tiles, and the tile limit lowered to 5 and 1 makes a thread carry more
+    # than four pairs.  Small integer values sum exactly in fp32 in any order, so the result
+    # equals the oracle's bit for bit only if every pair reached its own row exactly once.
+    d = 8
+    y = integers(72, 0, (n, d), -8, 9, np.int32).astype(np.float32)
+    idx = integers(72, 1, (n,), -2, V + 2, np.int32 if idx_dtype == I32 else np.int64)
+    idx[: n // 8] = V - 1  # one heavy row, in the last bucket of every pass
+    keep = (idx >= 0) & (idx < V)
+    monkeypatch.setenv("MOGRAD_HIP_SCATTER_BUCKET_MIN_ROWS", "1")
+    monkeypatch.setenv("MOGRAD_HIP_SCATTER_SORT_MAX_TILES", str(max_tiles))
+    got = _run(device, "SCATTER_ADD", Layout(V, d), [(idx, Layout(n), idx_dtype), (y, Layout(n, d), F32)], F32)
+    np.testing.assert_array_equal(got, O.scatter_add(idx[keep], y[keep], V).astype(np.float32))
+
+
 def test_scatter_add_ignores_bad_indices_and_checks_rank(device):
     V, d, n = 5, 8, 6
     y = normal(67, 0, (n, d))
