@@ -7,6 +7,7 @@
 // one; large tables first sort (row, position) pairs by row (a stable radix sort, so
 // positions stay ascending inside a row), and a wave then adds only its own row's run.
 #include <algorithm>
+#include <atomic>
 #include <cstring>
 #include <utility>
 
@@ -85,7 +86,270 @@ __global__ __launch_bounds__(64) void scatter_rows_kernel(const I* __restrict__ 
   }
 }
 
-// ---- large tables: bucket the indices by destination row first ---------------------------
+// VEC elements of a value row as loaded, unpacked to floats only when they are added: eight
+// of them wait in registers for the loads of a long run.
+template <typename T, int VEC>
+struct PackedChunk {
+  static constexpr int kBytes = sizeof(T) * VEC;
+  static_assert(kBytes == 16 || kBytes == 4 || kBytes == 2, "a chunk is one 16-byte load or one element");
+  uint32_t w[kBytes == 16 ? 4 : 1];
+  __device__ __forceinline__ void load(const T* p) {
+    if constexpr (kBytes == 16) {
+      const mg_u4 r = *reinterpret_cast<const mg_u4*>(p);
+      w[0] = r[0]; w[1] = r[1]; w[2] = r[2]; w[3] = r[3];
+    } else if constexpr (kBytes == 4) {
+      w[0] = *reinterpret_cast<const uint32_t*>(p);
+    } else {
+      w[0] = *reinterpret_cast<const uint16_t*>(p);
+    }
+  }
+  __device__ __forceinline__ void unpack(float (&v)[VEC]) {
+#pragma unroll
+    for (int i = 0; i < (kBytes == 16 ? 4 : 1); ++i) asm volatile("" : "+v"(w[i]));  // not before this point
+    if constexpr (kBytes == 2) {
+      const uint16_t bits = static_cast<uint16_t>(w[0]);
+      T t;
+      __builtin_memcpy(&t, &bits, 2);
+      v[0] = to_float(t);
+    } else {
+      VecIO<T, VEC>::load(reinterpret_cast<const T*>(w), v);
+    }
+  }
+};
+
+// ---- large tables, short index lists: one launch ------------------------------------------
+// A workgroup owns 4 * rows_per_wave consecutive destination rows and one block of 64 * VEC
+// columns.  Its four waves read a quarter of the index list each and keep, in position order,
+// the (row, position) pairs that fall into the workgroup's rows; the four lists one after the
+// other are then the workgroup's pairs in position order.  After that a wave walks the lists
+// once per row of its own and adds the value rows it finds, in that order, in fp32 from zero
+// (the order of scatter_rows_kernel with one slab: the same bits), and writes the row, zeros if
+// it found none.  Every workgroup reads the whole index list, which is what limits this form
+// to short lists; it needs no sort and no second launch.
+constexpr int kRangeCap = 512;      // pairs of a wave's list kept in LDS
+constexpr int kRangePosBits = 25;   // a pair is (row - first row) << 25 | position
+constexpr uint32_t kRangePosMask = (1u << kRangePosBits) - 1;
+
+// The pairs of positions [i0, i1) with a row in [r0, r1), written to out[0 .. cap) in position
+// order; returns their number, which may exceed cap (the pairs beyond it are then not kept).
+// A lane reads 16 bytes of indices at once where it can.
+template <typename I>
+__device__ __forceinline__ uint32_t range_collect(const I* __restrict__ indices, int64_t i0, int64_t i1, int64_t r0, int64_t r1,
+                                                  uint32_t* out, uint32_t cap, bool vec_ok, int lane) {
+  constexpr int K = 16 / sizeof(I);
+  constexpr int U = 4;  // loads in flight
+  struct alignas(16) Pack {
+    I v[K];
+  };
+  const uint64_t lower = (uint64_t{1} << lane) - 1;
+  uint32_t cnt = 0;
+  for (int64_t base = i0; base < i1; base += 64 * K * U) {
+    Pack pk[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t p = base + (u * 64 + lane) * K;
+      if (vec_ok && p + K <= i1) {
+        pk[u] = *reinterpret_cast<const Pack*>(indices + p);
+      } else {
+#pragma unroll
+        for (int c = 0; c < K; ++c) pk[u].v[c] = p + c < i1 ? indices[p + c] : static_cast<I>(-1);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t p = base + (u * 64 + lane) * K;
+      bool hit[K];
+      uint64_t found[K], any = 0;
+#pragma unroll
+      for (int c = 0; c < K; ++c) {
+        const int64_t v = static_cast<int64_t>(pk[u].v[c]);
+        hit[c] = v >= r0 && v < r1;
+        found[c] = __ballot(hit[c]);
+        any |= found[c];
+      }
+      if (any) {  // wave-uniform; a lane's pairs follow those of the lower lanes
+        uint32_t slot = cnt;
+#pragma unroll
+        for (int c = 0; c < K; ++c) {
+          slot += static_cast<uint32_t>(__popcll(found[c] & lower));
+          cnt += static_cast<uint32_t>(__popcll(found[c]));
+        }
+#pragma unroll
+        for (int c = 0; c < K; ++c) {
+          if (hit[c]) {
+            if (slot < cap)
+              out[slot] = (static_cast<uint32_t>(static_cast<int64_t>(pk[u].v[c]) - r0) << kRangePosBits) |
+                          static_cast<uint32_t>(p + c);
+            ++slot;
+          }
+        }
+      }
+    }
+  }
+  return cnt;
+}
+
+// grid (row ranges, column blocks).  `quarter` is the share of the index list a wave reads, a
+// multiple of 256.  A workgroup whose lists outgrow LDS (a row that a large part of the list
+// points at) keeps them in one of the `slots` areas of 4 * quarter pairs behind the `slots`
+// owner words at `spill`: it claims an area by writing `tag`, a number no earlier launch on
+// this memory has used, over an owner word that does not hold it yet, so the words need no
+// clearing, and which area it gets does not change what it computes.  More than
+// n_idx / (kRangeCap + 1) workgroups per column block cannot outgrow LDS, so with that many
+// areas a free one is always found; a workgroup that finds none (fewer areas, or stale words
+// that happen to equal the tag) reads the whole index list once per row instead.
+template <typename T, typename I, int VEC, bool STREAM>
+__global__ __launch_bounds__(256) void scatter_ranges_kernel(const I* __restrict__ indices, const T* __restrict__ values,
+                                                             T* __restrict__ dst, uint32_t* __restrict__ spill, uint32_t slots,
+                                                             uint32_t tag, int64_t n_idx, int64_t num_rows, int64_t row_size,
+                                                             int rows_per_wave, int64_t quarter, bool vec_ok) {
+  __shared__ uint32_t lds_list[4 * kRangeCap];
+  __shared__ uint32_t counts[4];
+  __shared__ int claimed;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * 4 * rows_per_wave;
+  const int64_t r1 = min(r0 + 4 * rows_per_wave, num_rows);
+  const int64_t i0 = min(wave * quarter, n_idx), i1 = min(i0 + quarter, n_idx);
+  {
+    const uint32_t cnt = range_collect<I>(indices, i0, i1, r0, r1, lds_list + wave * kRangeCap, kRangeCap, vec_ok, lane);
+    if (lane == 0) counts[wave] = cnt;
+  }
+  __syncthreads();
+  const uint32_t c0 = counts[0], c1 = counts[1], c2 = counts[2], c3 = counts[3];
+  const uint32_t* list = lds_list;  // LDS or global memory
+  int64_t stride = kRangeCap;
+  const int64_t col = (static_cast<int64_t>(blockIdx.y) * 64 + lane) * VEC;
+  const bool active = col < row_size;
+  const uint32_t col32 = static_cast<uint32_t>(col);  // a row holds fewer than 2^22 columns
+  auto put = [&](int64_t row, const float (&acc)[VEC]) {
+    if constexpr (STREAM) VecIO<T, VEC>::store_stream(dst + row * row_size + col, acc);
+    else VecIO<T, VEC>::store(dst + row * row_size + col, acc);
+  };
+  if (max(max(c0, c1), max(c2, c3)) > kRangeCap) {  // the same for the whole workgroup
+    if (threadIdx.x == 0) {
+      int got = -1;
+      uint32_t at = slots ? (blockIdx.y * gridDim.x + blockIdx.x) % slots : 0;
+      for (uint32_t tries = 0; tries < slots && got < 0; ++tries) {
+        uint32_t seen = __hip_atomic_load(spill + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        while (seen != tag) {  // free: claim it unless another workgroup does first
+          const uint32_t before = atomicCAS(spill + at, seen, tag);
+          if (before == seen) {
+            got = static_cast<int>(at);
+            break;
+          }
+          seen = before;
+        }
+        at = at + 1 == slots ? 0 : at + 1;
+      }
+      claimed = got;
+    }
+    __syncthreads();
+    if (claimed < 0) {  // no area: a wave reads the whole list for each row of its own
+      for (int k = 0; k < rows_per_wave; ++k) {
+        const int64_t row = r0 + wave * rows_per_wave + k;
+        if (row >= r1) break;
+        float acc[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+        for (int64_t base = 0; base < n_idx; base += 64) {
+          const int64_t at = base + lane;
+          uint64_t hits = __ballot(at < n_idx && static_cast<int64_t>(indices[at]) == row);
+          while (hits) {
+            const int bit = __ffsll(static_cast<long long>(hits)) - 1;
+            hits &= hits - 1;
+            if (active) {
+              float v[VEC];
+              VecIO<T, VEC>::load(values + (base + bit) * row_size + col, v);
+#pragma unroll
+              for (int e = 0; e < VEC; ++e) acc[e] += v[e];
+            }
+          }
+        }
+        if (active) put(row, acc);
+      }
+      return;
+    }
+    uint32_t* mine = spill + slots + static_cast<int64_t>(claimed) * 4 * quarter;
+    range_collect<I>(indices, i0, i1, r0, r1, mine + wave * quarter, static_cast<uint32_t>(quarter), vec_ok, lane);
+    __threadfence();
+    __syncthreads();
+    list = mine;
+    stride = quarter;
+  }
+  const uint32_t off1 = c0, off2 = off1 + c1, off3 = off2 + c2, total = off3 + c3;
+  auto pair_at = [&](uint32_t t) -> uint32_t {  // the t-th pair of the four lists in a row
+    if (t >= total) return 0xffffffffu;          // row field 127: no row of the workgroup
+    const int l = (t >= off1) + (t >= off2) + (t >= off3);
+    const uint32_t first = l == 0 ? 0u : (l == 1 ? off1 : (l == 2 ? off2 : off3));
+    return list[l * stride + (t - first)];
+  };
+  const uint32_t head = pair_at(lane);  // most workgroups hold fewer than 64 pairs
+  for (int k = 0; k < rows_per_wave; ++k) {
+    const uint32_t local = static_cast<uint32_t>(wave * rows_per_wave + k);
+    const int64_t row = r0 + local;
+    if (row >= r1) break;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+    for (uint32_t b = 0; b < total; b += 64) {
+      const uint32_t pair = b == 0 ? head : pair_at(b + lane);
+      uint64_t hits = __ballot((pair >> kRangePosBits) == local);
+      while (hits) {  // wave-uniform; eight value rows in flight, added in position order
+        constexpr int U = 8;
+        uint32_t pos[U];
+        int got = 0;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          pos[u] = 0;
+          if (hits) {
+            const int bit = __ffsll(static_cast<long long>(hits)) - 1;
+            hits &= hits - 1;
+            pos[u] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(pair), bit)) & kRangePosMask;
+            got = u + 1;
+          }
+        }
+        if (active) {
+          PackedChunk<T, VEC> chunk[U];
+#pragma unroll
+          for (int u = 0; u < U; ++u)
+            if (u < got) chunk[u].load(values + static_cast<int64_t>(pos[u]) * row_size + col32);
+#pragma unroll
+          for (int u = 0; u < U; ++u)
+            if (u < got) {
+              float v[VEC];
+              chunk[u].unpack(v);
+#pragma unroll
+              for (int e = 0; e < VEC; ++e) acc[e] += v[e];
+            }
+        }
+      }
+    }
+    if (active) put(row, acc);
+  }
+}
+
+template <typename T, typename I, int VEC>
+static int scatter_ranges(const I* indices, const T* values, T* dst, int64_t n_idx, int64_t num_rows, int64_t row_size,
+                          int rows_per_wave, int64_t quarter, hipStream_t s) {
+  const int64_t ranges = ceil_div(num_rows, 4 * rows_per_wave), col_blocks = ceil_div(row_size, 64 * VEC);
+  static std::atomic<uint32_t> launches{0};
+  const uint32_t tag = ++launches;
+  // as many areas as workgroups can need, within 64 MiB
+  int64_t slots = std::min(col_blocks * (n_idx / (kRangeCap + 1) + 1) + 8, std::max<int64_t>(8, (int64_t{4} << 20) / quarter));
+  const int slots_knob = env_int("MOGRAD_HIP_SCATTER_SPILL_SLOTS", -1);  // tests: 0 = no areas
+  if (slots_knob >= 0) slots = slots_knob;
+  Scratch spill;
+  MG_TRY(spill.take((slots + slots * 4 * quarter + 1) * 4));
+  const dim3 grid(static_cast<unsigned>(ranges), static_cast<unsigned>(col_blocks));
+  const bool stream_out = env_int("MOGRAD_HIP_SCATTER_STREAM", 1) != 0;
+  auto kernel = stream_out ? scatter_ranges_kernel<T, I, VEC, true> : scatter_ranges_kernel<T, I, VEC, false>;
+  hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, indices, values, dst, spill.as<uint32_t>(), static_cast<uint32_t>(slots), tag, n_idx,
+                     num_rows, row_size, rows_per_wave, quarter, aligned16(indices));
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+// ---- large tables, long index lists: bucket the indices by destination row first -------------
 
 // key[i] = destination row of value row i (num_rows for an index outside the table: a bucket
 // that nobody sums), pos[i] = i.
@@ -241,14 +505,24 @@ __global__ __launch_bounds__(64) void scatter_runs_sum_kernel(const uint32_t* __
   float acc[VEC];
 #pragma unroll
   for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+  const uint32_t col32 = static_cast<uint32_t>(col);
   const uint32_t p1 = last[row];
-  for (uint32_t p = first[row]; p < p1; ++p) {
-    float v[VEC];
-    VecIO<T, VEC>::load(values + static_cast<int64_t>(pos[p]) * row_size + col, v);
+  for (uint32_t p = first[row]; p < p1; p += 8) {  // eight value rows in flight
+    const int got = static_cast<int>(min(p1 - p, 8u));
+    PackedChunk<T, VEC> chunk[8];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) acc[e] += v[e];
+    for (int u = 0; u < 8; ++u)
+      if (u < got) chunk[u].load(values + static_cast<int64_t>(pos[p + u]) * row_size + col32);
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (u < got) {
+        float v[VEC];
+        chunk[u].unpack(v);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] += v[e];
+      }
   }
-  VecIO<T, VEC>::store(dst + row * row_size + col, acc);
+  VecIO<T, VEC>::store_stream(dst + row * row_size + col, acc);
 }
 
 template <typename T, typename I, int VEC>
@@ -330,8 +604,20 @@ static int scatter_launch(const I* indices, const T* values, T* dst, int64_t n_i
   // Tables of a thousand rows and more: bucket first (MOGRAD_HIP_SCATTER_BUCKET_MIN_ROWS moves
   // the threshold; (50304, 768) from 8192 rows took 5 ms by scanning).
   if (num_rows >= env_int("MOGRAD_HIP_SCATTER_BUCKET_MIN_ROWS", 1024) && n_idx > 0 && n_idx < 0x7fffffffLL &&
-      num_rows < 0x7fffffffLL)
+      num_rows < 0x7fffffffLL) {
+    // Short lists: every workgroup of a row range reads the whole list, up to 2^(the knob)
+    // index reads in all (MOGRAD_HIP_SCATTER_RANGE_READS_LOG2; 0 switches the form off), and a
+    // wave's list should hold 128 pairs at most when the indices are spread evenly.
+    const int rows_per_wave = static_cast<int>(std::min<int64_t>(16, std::max<int64_t>(1, num_rows / 4096)));
+    constexpr int64_t kStep = 64 * (16 / sizeof(I)) * 4;  // positions a wave reads in one step
+    const int64_t quarter = ceil_div(ceil_div(n_idx, 4), kStep) * kStep;
+    const int64_t reads = ceil_div(num_rows, 4 * rows_per_wave) * ceil_div(row_size, 64 * VEC) * 4 * quarter;
+    const int reads_log2 = env_int("MOGRAD_HIP_SCATTER_RANGE_READS_LOG2", 27);
+    if (reads_log2 > 0 && reads_log2 < 40 && reads <= (int64_t{1} << reads_log2) && n_idx < (int64_t{1} << kRangePosBits) &&
+        n_idx * rows_per_wave <= 128 * num_rows)
+      return scatter_ranges<T, I, VEC>(indices, values, dst, n_idx, num_rows, row_size, rows_per_wave, quarter, s);
     return scatter_bucketed<T, I, VEC>(indices, values, dst, n_idx, num_rows, row_size, s);
+  }
   const int64_t col_blocks = ceil_div(row_size, 64 * VEC);
   // Slabs of the index list: enough waves to fill the device, at least 256 indices each,
   // partial sums capped at 64 MiB.

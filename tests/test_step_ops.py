@@ -201,9 +201,56 @@ def test_scatter_add_sort_places_every_pair_once(device, monkeypatch, idx_dtype,
     idx[: n // 8] = V - 1  # one heavy row, in the last bucket of every pass
     keep = (idx >= 0) & (idx < V)
     monkeypatch.setenv("MOGRAD_HIP_SCATTER_BUCKET_MIN_ROWS", "1")
+    monkeypatch.setenv("MOGRAD_HIP_SCATTER_RANGE_READS_LOG2", "0")  # the sort, whatever the list's length
     monkeypatch.setenv("MOGRAD_HIP_SCATTER_SORT_MAX_TILES", str(max_tiles))
     got = _run(device, "SCATTER_ADD", Layout(V, d), [(idx, Layout(n), idx_dtype), (y, Layout(n, d), F32)], F32)
     np.testing.assert_array_equal(got, O.scatter_add(idx[keep], y[keep], V).astype(np.float32))
+
+
+@pytest.mark.parametrize("areas", [-1, 1, 0])
+@pytest.mark.parametrize("idx_dtype", [I32, I64])
+@pytest.mark.parametrize("V,d,n,heavy", [(50304, 8, 8192, 512), (70000, 8, 5000, 3000), (300, 24, 1031, 128),
+                                         (4096 * 9 + 5, 8, 1, 0), (2048, 520, 2500, 2500), (65, 8, 700, 0)])
+def test_scatter_add_row_ranges_place_every_pair_once(device, monkeypatch, idx_dtype, V, d, n, heavy, areas):
+    # Short lists into large tables take one launch: a workgroup per range of rows collects the
+    # pairs of its rows from the whole list.  A row that more than 512 pairs of one quarter of
+    # the list point at makes its workgroup keep its lists in global memory instead of LDS; the
+    # last range of a table is shorter than the others; 520 columns leave the second column
+    # block mostly empty.  With one area for the two workgroups that need one, or none, the
+    # workgroups left without read the whole list once per row.  Exact for the same reason as above.
+    y = integers(73, 0, (n, d), -8, 9, np.int32).astype(np.float32)
+    idx = integers(73, 1, (n,), -2, V + 2, np.int32 if idx_dtype == I32 else np.int64)
+    idx[:heavy] = V - 1
+    keep = (idx >= 0) & (idx < V)
+    monkeypatch.setenv("MOGRAD_HIP_SCATTER_BUCKET_MIN_ROWS", "1")
+    monkeypatch.setenv("MOGRAD_HIP_SCATTER_RANGE_READS_LOG2", "30")
+    if areas >= 0:
+        monkeypatch.setenv("MOGRAD_HIP_SCATTER_SPILL_SLOTS", str(areas))
+    got = _run(device, "SCATTER_ADD", Layout(V, d), [(idx, Layout(n), idx_dtype), (y, Layout(n, d), F32)], F32)
+    np.testing.assert_array_equal(got, O.scatter_add(idx[keep], y[keep], V).astype(np.float32))
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("V,d,n", [(2048, 64, 3000), (50304, 136, 4000)])
+def test_scatter_add_forms_agree_bit_for_bit(device, monkeypatch, dtype, V, d, n):
+    # Row ranges, the sort and (one slab) the scanning kernel all add a row's values in
+    # ascending position order in fp32 from zero: the same bits, with and without streaming stores.
+    y = round_to_dtype(normal(74, 0, (n, d)), dtype)
+    idx = integers(74, 1, (n,), -3, V + 3, np.int32)
+    idx[: n // 3] = 17
+    operands = [(idx, Layout(n), I32), (y, Layout(n, d), dtype)]
+    monkeypatch.setenv("MOGRAD_HIP_SCATTER_RANGE_READS_LOG2", "30")
+    ranges = _run(device, "SCATTER_ADD", Layout(V, d), operands, dtype)
+    monkeypatch.setenv("MOGRAD_HIP_SCATTER_STREAM", "0")
+    np.testing.assert_array_equal(ranges, _run(device, "SCATTER_ADD", Layout(V, d), operands, dtype))
+    monkeypatch.setenv("MOGRAD_HIP_SCATTER_RANGE_READS_LOG2", "0")
+    np.testing.assert_array_equal(ranges, _run(device, "SCATTER_ADD", Layout(V, d), operands, dtype))
+    if n <= 1024 * 3 and V <= 2048:
+        monkeypatch.setenv("MOGRAD_HIP_SCATTER_BUCKET_MIN_ROWS", "1000000000")
+        # several slabs here: partial sums are regrouped, so only to the summation tolerance
+        scan = _run(device, "SCATTER_ADD", Layout(V, d), operands, dtype)
+        eps = {F32: 2.0 ** -20, F16: 2.0 ** -10, BF16: 2.0 ** -7}[dtype]
+        assert np.all(np.abs(scan - ranges) <= eps * (np.abs(ranges) + 64.0))
 
 
 def test_scatter_add_ignores_bad_indices_and_checks_rank(device):
