@@ -441,6 +441,26 @@ int mg_layer_norm_bwd_stats_deferred(const void* dy, const void* x, const void* 
                                      const float* rstd, const void* residual, void* dx, void* dgamma,
                                      void* dbeta, int64_t rows, int64_t cols, int dtype, int grad_dtype,
                                      mg_deferred list, mg_stream stream);
+/* A Linear layer's backward continued through the LayerNorm that produced the layer's input:
+ * for Y = LN(h) W^T (+ b) with LN(h) = x, given dY,
+ *   dW = dY^T x, db = column sums of dY (db may be NULL),
+ *   dh = LayerNorm backward of dY W at h with the saved statistics (dx_accumulate != 0: added
+ *        to what `dh` holds, the gradient reaching h along a skip connection), dgamma, dbeta,
+ * i.e. mg_linear_bwd(dy, x, w, t, dw, db) followed by mg_layer_norm_bwd_stats(_add)(t, h, gamma,
+ * mean, rstd, dh, ..) without the (M, K) tensor t = dY W: for 16-bit layers with K == 384 input
+ * columns whose backward takes the single launch with 128 x 384 tiles, a tile holds whole rows
+ * of t and continues as the LayerNorm backward from LDS; t is rounded to the tensors' type on
+ * the way, as storing it would, so only the order of the row and column sums differs from the
+ * two separate calls.  Every other shape and dtype runs those two calls with t in a pool block.
+ * `list` may be NULL (sums at once, grad_dtype == dtype); otherwise dw, db, dgamma and dbeta
+ * are of `grad_dtype` and their sums are deferred as in the `_deferred` forms.  No counterpart
+ * in the reference, whose graph evaluates LINEAR_GRAD and the LayerNorm gradient as separate
+ * nodes (mograd/grad.mojo:296-344). */
+int mg_linear_bwd_layer_norm_bwd(const void* dy, const void* x, const void* w, const void* h,
+                                 const void* gamma, const float* mean, const float* rstd, void* dh,
+                                 void* dw, void* db, void* dgamma, void* dbeta, int64_t M, int64_t N,
+                                 int64_t K, int dx_accumulate, int dtype, int grad_dtype,
+                                 mg_deferred list, mg_stream stream);
 /* mg_scatter_add with dst of `grad_dtype`, the sum over the index slabs deferred. */
 int mg_scatter_add_deferred(const void* indices, const void* values, void* dst, int64_t n_idx,
                             int64_t num_rows, int64_t row_size, int idx_dtype, int dtype, int grad_dtype,

@@ -115,6 +115,7 @@ PROTOTYPES = {
     "mg_finish_deferred": (_i, [_p, _p], True),
     "mg_linear_bwd_deferred": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _l, _i, _i, _i, _i, _p, _p], True),
     "mg_layer_norm_bwd_stats_deferred": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _l, _l, _i, _i, _p, _p], True),
+    "mg_linear_bwd_layer_norm_bwd": (_i, [_p] * 12 + [_l, _l, _l, _i, _i, _i, _p, _p], True),
     "mg_scatter_add_deferred": (_i, [_p, _p, _p, _l, _l, _l, _i, _i, _i, _p, _p], True),
     "mg_flash_attn_fwd": (_i, [_p, _p, _p, _p, _p, _p, _l, _l, _l, _l, _f, _i, _i, _i, _p], True),
     "mg_flash_attn_bwd": (_i, [_p] * 10 + [_l, _l, _l, _l, _f, _i, _i, _i, _p], True),

@@ -1,6 +1,7 @@
 // C ABI for the matmul family: operand classification, kernel choice, launches.
 #include "gemm_impl.h"
 #include "mg_deferred.h"
+#include "mg_rows.h"
 
 namespace mg {
 
@@ -358,6 +359,9 @@ int gemm_dispatch(const char* who, const GemmArgs& g_in, hipStream_t stream) {
 
 int colsum_dispatch(const void* a, void* dst, int64_t outer, int64_t reduce, int64_t inner, int dtype,
                     hipStream_t stream);  // reduce.hip
+int ln_bwd(const void* dy, const void* x, const void* gamma, const float* mean, const float* rstd, const void* residual,
+           void* dx, void* dgamma, void* dbeta, int64_t rows, int64_t cols, float eps, int dtype,
+           mg_stream stream);  // layer_norm.hip
 
 // dX (M,K) = dY (M,N) W (N,K) and dW (N,K) = dY^T X of a 16-bit Linear layer in one launch
 // (linear_bwd_16bit_kernel), for the shapes at which launch_16bit_mfma would give both the
@@ -366,10 +370,25 @@ int colsum_dispatch(const void* a, void* dst, int64_t outer, int64_t reduce, int
 // dX tiles than CUs): here dX is never split, the dW workgroups fill the device.
 // *done = false: not such a shape, nothing launched.
 // MOGRAD_HIP_LINEAR_BWD_ONE_LAUNCH=0 switches it off (benchmarks, tests of the equivalence).
+// With `ln`, the launch's dX tiles continue as the backward of the LayerNorm whose output X is
+// (linear_bwd_ln_16bit_kernel): `dx` then receives that LayerNorm's input gradient (added to
+// what it holds when dx_accumulate), dY W itself is not stored, and the LayerNorm's dgamma and
+// dbeta follow from one partial row per tile of 128 rows.  Only for the wide tiles of a
+// 384-wide input (K == 384); otherwise *done stays false.
+struct LinearBwdLayerNorm {
+  const void* x;       // the LayerNorm's input (M, K)
+  const void* gamma;   // (K)
+  const float* mean;   // (M)
+  const float* rstd;
+  void* dgamma;        // (K)
+  void* dbeta;
+};
+
 template <typename T>
 static int linear_bwd_one_launch(const void* dy, const void* x, const void* w, void* dx, void* dw, int64_t M, int64_t N,
                                  int64_t K, const void* relu_mask, bool dx_accumulate, hipStream_t stream, bool* done,
-                                 int64_t dw_rows = -1, void* db = nullptr, bool* db_done = nullptr) {
+                                 int64_t dw_rows = -1, void* db = nullptr, bool* db_done = nullptr,
+                                 const LinearBwdLayerNorm* ln = nullptr) {
   *done = false;
   if (db_done) *db_done = false;
   if (dw_rows < 0) dw_rows = N;  // rows of dW to write: fewer than N when dY and W came zero-padded
@@ -386,6 +405,9 @@ static int linear_bwd_one_launch(const void* dy, const void* x, const void* w, v
   // workgroup per CU, and the layer is wide enough to pay for the larger partial tiles.
   const bool wide = K % kGemmWideBN == 0 && ceil_div(M, kGemmBM) * (K / kGemmWideBN) < cus && N >= 768 &&
                     env_int("MOGRAD_HIP_LINEAR_BWD_WIDE", 1) != 0;
+  if (ln && (!wide || K != kGemmWideBN || relu_mask || env_int("MOGRAD_HIP_LINEAR_BWD_STAGES", 2) == 3 ||
+             !aligned16(ln->x) || !aligned16(ln->gamma)))
+    return MG_OK;
   const int tiles_kk = static_cast<int>(ceil_div(K, wide ? kGemmWideBN : kGemmBN));
   // dW: must be split, each workgroup's rows short enough for the 32-k variant.
   const int w_tiles_m = static_cast<int>(ceil_div(N, kGemmBM));
@@ -453,7 +475,16 @@ static int linear_bwd_one_launch(const void* dy, const void* x, const void* w, v
   // Three copies of the tiles (two k-steps in flight per workgroup, three workgroups per CU)
   // measured 1 % faster on the GPT step than two copies and four workgroups; four copies no
   // better than two.  MOGRAD_HIP_LINEAR_BWD_STAGES=2 selects two.
-  if (wide && env_int("MOGRAD_HIP_LINEAR_BWD_STAGES", 2) == 3)  // 32 k per step, three copies: 3-4 % slower
+  Scratch ln_part_g, ln_part_b;
+  if (ln) {
+    MG_TRY(ln_part_g.take(static_cast<int64_t>(x_tiles_m) * K * static_cast<int64_t>(sizeof(float))));
+    MG_TRY(ln_part_b.take(static_cast<int64_t>(x_tiles_m) * K * static_cast<int64_t>(sizeof(float))));
+    Gemm16Problem<T> px2 = px;
+    px2.ln = Gemm16LayerNormBwd<T>{static_cast<const T*>(ln->x), static_cast<const T*>(ln->gamma), ln->mean, ln->rstd,
+                                   ln_part_g.as<float>(), ln_part_b.as<float>()};
+    hipLaunchKernelGGL((linear_bwd_ln_16bit_kernel<T>), dim3(static_cast<unsigned>(n_dw + x_tiles)), dim3(2 * kGemmWideBN),
+                       0, stream, pw2, px2, static_cast<int>(n_dw));
+  } else if (wide && env_int("MOGRAD_HIP_LINEAR_BWD_STAGES", 2) == 3)  // 32 k per step, three copies: 3-4 % slower
     hipLaunchKernelGGL((linear_bwd_16bit_kernel<T, 3, kGemmWideBN>), dim3(static_cast<unsigned>(n_dw + x_tiles)),
                        dim3(2 * kGemmWideBN), 0, stream, pw2, px, static_cast<int>(n_dw));
   else if (wide)  // 64 k per step, two copies (128 KB of LDS): half the barriers, whole cache lines of dY
@@ -466,6 +497,11 @@ static int linear_bwd_one_launch(const void* dy, const void* x, const void* w, v
     hipLaunchKernelGGL((linear_bwd_16bit_kernel<T, 3>), dim3(static_cast<unsigned>(n_dw + x_tiles)), dim3(kGemmThreads), 0,
                        stream, pw2, px, static_cast<int>(n_dw));
   MG_LAUNCH_CHECK();
+  if (ln) {  // the tiles' partial rows of dgamma / dbeta: summed now, or left on the deferred list
+    reduce_partials_or_defer<T>(ln_part_g, static_cast<T*>(ln->dgamma), &ln_part_b, static_cast<T*>(ln->dbeta), x_tiles_m,
+                                K, static_cast<int>(cus), stream);
+    MG_LAUNCH_CHECK();
+  }
   const int dw_blocks = static_cast<int>(slice / 1024);  // 256 threads, four consecutive partial values each
   const int db_blocks = groups > 0 ? static_cast<int>(ceil_div(N, 64)) : 0;
   if (DeferredList* dl = deferred_current()) {
@@ -539,9 +575,18 @@ static int linear_bwd_padded(const void* dy, const void* x, const void* w, void*
 // *done: dX and dW are on their way; *db_done: so is db (else the caller sums dY's columns).
 int linear_bwd_products(const void* dy, const void* x, const void* w, void* dx, void* dw, void* db, int64_t M, int64_t N,
                         int64_t K, const void* relu_mask, bool dx_accumulate, int dtype, hipStream_t stream, bool* done,
-                        bool* db_done) {
+                        bool* db_done, const LinearBwdLayerNorm* ln = nullptr) {
   *done = false;
   *db_done = false;
+  if (ln) {  // only the one launch has the LayerNorm continuation
+    if (dtype == MG_BF16)
+      return linear_bwd_one_launch<bf16_t>(dy, x, w, dx, dw, M, N, K, relu_mask, dx_accumulate, stream, done, -1, db,
+                                           db_done, ln);
+    if (dtype == MG_F16)
+      return linear_bwd_one_launch<f16_t>(dy, x, w, dx, dw, M, N, K, relu_mask, dx_accumulate, stream, done, -1, db,
+                                          db_done, ln);
+    return MG_OK;
+  }
   if (dtype == MG_BF16) {
     MG_TRY(linear_bwd_one_launch<bf16_t>(dy, x, w, dx, dw, M, N, K, relu_mask, dx_accumulate, stream, done, -1, db,
                                          db_done));
@@ -652,6 +697,45 @@ int mg_linear_bwd_deferred(const void* dy, const void* x, const void* w, void* d
   MG_TRY(scope.substitute(db, N, &db_use));
   MG_TRY(linear_bwd_impl(dy, x, w, dx, dw_use, db_use, M, N, K, dx_accumulate != 0, x_is_relu_output != 0, dtype, stream));
   return scope.finish(mg::to_stream(stream));
+}
+
+int mg_linear_bwd_layer_norm_bwd(const void* dy, const void* x, const void* w, const void* ln_x, const void* gamma,
+                                 const float* mean, const float* rstd, void* dx, void* dw, void* db, void* dgamma,
+                                 void* dbeta, int64_t M, int64_t N, int64_t K, int dx_accumulate, int dtype,
+                                 int grad_dtype, mg_deferred list, mg_stream stream) {
+  const char* who = "linear_bwd_layer_norm_bwd";
+  if (!mg::is_float_dtype(dtype)) return mg::fail(MG_ERR_INVALID, "%s: unsupported dtype %s", who, mg::dtype_name(dtype));
+  if (M < 0 || N < 0 || K <= 0) return mg::fail(MG_ERR_INVALID, "%s: bad size", who);
+  if (!dy || !x || !w || !ln_x || !gamma || !mean || !rstd || !dx || !dw || !dgamma || !dbeta)
+    return mg::fail(MG_ERR_INVALID, "%s: null pointer argument", who);
+  if (list) MG_TRY(mg::deferred_check(who, list, dtype, grad_dtype));
+  else if (grad_dtype != dtype) return mg::fail(MG_ERR_INVALID, "%s: without a deferred list the gradients have the tensors' dtype", who);
+  hipStream_t s = mg::to_stream(stream);
+  auto run = [&](void* dw_use, void* db_use, void* dg_use, void* dbt_use) -> int {
+    bool done = false, db_done = false;
+    const mg::LinearBwdLayerNorm ln{ln_x, gamma, mean, rstd, dg_use, dbt_use};
+    MG_TRY(mg::linear_bwd_products(dy, x, w, dx, dw_use, db_use, M, N, K, nullptr, dx_accumulate != 0, dtype, s, &done,
+                                   &db_done, &ln));
+    if (done) {
+      if (db_use && !db_done) MG_TRY(mg::colsum_dispatch(dy, db_use, 1, M, N, dtype, s));
+      return MG_OK;
+    }
+    // Other shapes: dY W into a scratch tensor with the separate entry's kernels, then the LayerNorm backward.
+    mg::Scratch dy_ln;
+    MG_TRY(dy_ln.take(M * K * static_cast<int64_t>(mg::dtype_size(dtype))));
+    MG_TRY(linear_bwd_impl(dy, x, w, dy_ln.as<char>(), dw_use, db_use, M, N, K, false, false, dtype, stream));
+    return mg::ln_bwd(dy_ln.as<char>(), ln_x, gamma, mean, rstd, dx_accumulate ? dx : nullptr, dx, dg_use, dbt_use, M, K,
+                      0.f, dtype, stream);
+  };
+  if (!list) return run(dw, db, dgamma, dbeta);
+  mg::DeferredScope scope(static_cast<mg::DeferredList*>(list), dtype, grad_dtype);
+  void *dw_use, *db_use, *dg_use, *dbt_use;
+  MG_TRY(scope.substitute(dw, N * K, &dw_use));
+  MG_TRY(scope.substitute(db, N, &db_use));
+  MG_TRY(scope.substitute(dgamma, K, &dg_use));
+  MG_TRY(scope.substitute(dbeta, K, &dbt_use));
+  MG_TRY(run(dw_use, db_use, dg_use, dbt_use));
+  return scope.finish(s);
 }
 
 }  // extern "C"

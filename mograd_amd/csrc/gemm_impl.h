@@ -635,6 +635,153 @@ __device__ __forceinline__ void gemm16_write_tile(const floatx16 (&acc)[2][2], u
     }
 }
 
+// What a product's output tile needs to continue as a LayerNorm backward (see gemm16_ln_bwd_tile).
+template <typename T>
+struct Gemm16LayerNormBwd {
+  const T* x = nullptr;         // the LayerNorm's input, laid out like the product's output
+  const T* gamma = nullptr;     // (cols)
+  const float* mean = nullptr;  // (rows) saved by the forward
+  const float* rstd = nullptr;
+  float* part_g = nullptr;      // (row tiles, cols) partial column sums of dy * xhat and of dy
+  float* part_b = nullptr;
+};
+
+// Output of a 128 x (64 WN) tile whose rows are whole rows of the result (N = 64 WN), when the
+// result dY is only wanted as the upstream of a LayerNorm backward: the tile is staged in LDS
+// as the rounded 16-bit values a store would have written, and the workgroup then computes,
+// from LDS and the matching rows of the LayerNorm's input x,
+//   dx = rstd (dY gamma - mean_n(dY gamma) - xhat mean_n(dY gamma xhat)),  xhat = (x - mean) rstd,
+// written to C as round(dx) (+ the residual, as the separate kernels give it), and the tile's
+// column sums of dY xhat and dY as one row of part_g / part_b.  dY itself never reaches memory.
+// A lane owns 8 columns of rows rl0 + 8 i of its wave's 64 x 64 tile (the layout of the plain
+// store); a row's sums go over the 8 lanes of its 64 columns by DPP and over the WN waves that
+// share the row through LDS, in a fixed order, and the column sums over the 8 row lanes by
+// shuffles and over the two row waves through LDS.  `free_lds` is LDS behind the waves' strips:
+// 128 * WN * 8 bytes for the row sums and 2 * 64 * WN * 8 for the column sums.
+template <typename T, int WN>
+__device__ __forceinline__ void gemm16_ln_bwd_tile(const floatx16 (&acc)[2][2], uint16_t* __restrict__ mine,
+                                                   float* __restrict__ free_lds, T* C, int M, int64_t ldc, int tile_m,
+                                                   int m0, int wm, int wn, int lane, const T* residual,
+                                                   const Gemm16LayerNormBwd<T>& ln) {  // residual may be C itself
+  constexpr int COLS = 64 * WN;
+  {  // the staging of gemm16_write_tile (no bias, no ReLU)
+    const int odd = lane & 1;
+    const uint32_t select = odd ? 0x03020706u : 0x05040100u;
+    uint32_t* const base32 = reinterpret_cast<uint32_t*>(mine + ((lane / 32) * 4 + odd) * kG16Stride + (lane % 32 - odd));
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+      for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+        for (int rp = 0; rp < 8; ++rp) {
+          const uint32_t w = gemm16_pack2<T>(acc[ti][tj][2 * rp], acc[ti][tj][2 * rp + 1]);
+          const uint32_t y = __builtin_amdgcn_update_dpp(w, w, kDppQuadXor1, 0xf, 0xf, false);
+          const int rl = ti * 32 + (rp / 2) * 8 + (rp % 2) * 2;
+          base32[(rl * kG16Stride + tj * 32) / 2] = __builtin_amdgcn_perm(y, w, select);
+        }
+  }
+  float2* row_sums = reinterpret_cast<float2*>(free_lds);               // [128][WN]
+  float* col_sums = free_lds + 128 * WN * 2;                             // [2 row waves][which][COLS]
+  const int rl0 = lane / 8, ch = lane % 8;
+  const int col = wn + ch * 8;
+  const uint16_t* src = mine + rl0 * kG16Stride + ch * 8;
+  float gam[8];
+  VecIO<T, 8>::load(ln.gamma + col, gam);
+  uint4 xraw[8], rraw[8];
+  float mu[8], rs[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = min(m0 + wm + rl0 + 8 * i, M - 1);  // rows past the end: computed, never stored or summed
+    const int64_t at = static_cast<int64_t>(row) * ldc + col;
+    xraw[i] = *reinterpret_cast<const uint4*>(ln.x + at);
+    rraw[i] = residual ? *reinterpret_cast<const uint4*>(residual + at) : make_uint4(0, 0, 0, 0);
+    mu[i] = ln.mean[row];
+    rs[i] = ln.rstd[row];
+  }
+  __syncthreads();  // the strips are complete
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float dy[8], xv[8];
+    VecIO<T, 8>::load(reinterpret_cast<const T*>(src + i * 8 * kG16Stride), dy);
+    VecIO<T, 8>::load(reinterpret_cast<const T*>(&xraw[i]), xv);
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float xhat = (xv[e] - mu[i]) * rs[i];
+      const float dyg = dy[e] * gam[e];
+      s0 += dyg;
+      s1 += dyg * xhat;
+    }
+    s0 += dpp_move<kDppQuadXor1>(s0);
+    s1 += dpp_move<kDppQuadXor1>(s1);
+    s0 += dpp_move<kDppQuadXor2>(s0);
+    s1 += dpp_move<kDppQuadXor2>(s1);
+    s0 += dpp_move<kDppRowHalfMirror>(s0);
+    s1 += dpp_move<kDppRowHalfMirror>(s1);
+    if (ch == 0) row_sums[(wm + rl0 + 8 * i) * WN + wn / 64] = make_float2(s0, s1);
+  }
+  __syncthreads();
+  const float inv_n = 1.0f / static_cast<float>(COLS);
+  float acc_g[8], acc_b[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc_g[e] = acc_b[e] = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = m0 + wm + rl0 + 8 * i;
+    float c1 = 0.f, c2 = 0.f;
+#pragma unroll
+    for (int w = 0; w < WN; ++w) {
+      const float2 p = row_sums[(wm + rl0 + 8 * i) * WN + w];
+      c1 += p.x;
+      c2 += p.y;
+    }
+    c1 *= inv_n;
+    c2 *= inv_n;
+    float dy[8], xv[8], rv[8], out[8];
+    VecIO<T, 8>::load(reinterpret_cast<const T*>(src + i * 8 * kG16Stride), dy);
+    VecIO<T, 8>::load(reinterpret_cast<const T*>(&xraw[i]), xv);
+    VecIO<T, 8>::load(reinterpret_cast<const T*>(&rraw[i]), rv);
+    const bool ok = row < M;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float xhat = (xv[e] - mu[i]) * rs[i];
+      const float d = ok ? dy[e] : 0.f;
+      out[e] = rs[i] * (d * gam[e] - c1 - xhat * c2);
+      acc_g[e] += d * xhat;
+      acc_b[e] += d;
+    }
+    if (residual) {
+      // round(gradient) + residual: a plain addition, as the separate add performs it
+#pragma clang fp contract(off)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) out[e] = to_float(from_float<T>(out[e])) + rv[e];
+    }
+    if (ok) VecIO<T, 8>::store(C + static_cast<int64_t>(row) * ldc + col, out);
+  }
+  // column sums over the wave's 64 rows: the 8 lanes with this lane's columns
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+#pragma unroll
+    for (int w = 8; w < kWave; w *= 2) {
+      acc_g[e] += __shfl_xor(acc_g[e], w);
+      acc_b[e] += __shfl_xor(acc_b[e], w);
+    }
+  }
+  if (rl0 == 0) {
+    float* mine_g = col_sums + (wm / 64) * 2 * COLS + col;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      mine_g[e] = acc_g[e];
+      mine_g[COLS + e] = acc_b[e];
+    }
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < COLS; c += blockDim.x) {
+    ln.part_g[static_cast<int64_t>(tile_m) * COLS + c] = col_sums[c] + col_sums[2 * COLS + c];
+    ln.part_b[static_cast<int64_t>(tile_m) * COLS + c] = col_sums[COLS + c] + col_sums[3 * COLS + c];
+  }
+}
+
 template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, bool RAGGED>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_16bit_mfma_kernel(
     const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ bias, T* __restrict__ C,
@@ -850,13 +997,15 @@ struct Gemm16Problem {
   // The partial tiles are read back much later (their sum is deferred to the end of a training
   // step): store them past the caches.
   bool partial_stream = false;
+  // The output continues as a LayerNorm backward inside the launch (gemm16_pipe_block<.., LN_BWD>).
+  Gemm16LayerNormBwd<T> ln;
 };
 
 // The work of workgroup `bid` of a launch for one product; `lds` is the workgroup's
 // gemm16_pipe_lds_bytes(BK, NSTAGE, TM, TN) bytes, aligned to 1024.  The output tile is
 // TM x TN, (TM / 64) x (TN / 64) waves with 64 x 64 each; pr.tiles_n counts tiles of TN columns.
 template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, int BK, int NSTAGE, int TM = 128,
-          int TN = kGemmBN>
+          int TN = kGemmBN, bool LN_BWD = false>
 __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm16Problem<T>& pr) {
   static_assert(NSTAGE >= 2 && NSTAGE <= 4 && (BK == 32 || BK == 64) && (TM == 128 || TM == 256), "stages");
   static_assert(TN % 128 == 0 && (!SPLIT_K || TM == 128), "partial tiles are 128 x 128");
@@ -1012,9 +1161,18 @@ __device__ __forceinline__ void gemm16_pipe_block(char* lds, int bid, const Gemm
   }
 
   uint16_t* mine = reinterpret_cast<uint16_t*>(lds) + wave * 64 * kG16Stride;
-  gemm16_write_tile<T, HAS_BIAS, SPLIT_K>(acc, mine, bias, C, partial, M, N, ldc, bsc, batch,
-                                          split, SPLIT_K ? batches : 1,
-                                          m0, n0, wm, wn, lane, ep, pr.partial_stream);
+  if constexpr (LN_BWD) {
+    // whole rows per tile, and room behind the strips for the row and column sums
+    static_assert(!SPLIT_K && !HAS_BIAS && TM == 128, "the LayerNorm epilogue takes a plain 128-row tile");
+    static_assert(gemm16_pipe_lds_bytes(BK, NSTAGE, TM, TN) >= NW * 64 * kG16Stride * 2 + 128 * WN * 8 + 2 * 64 * WN * 8,
+                  "LDS behind the output strips");
+    float* free_lds = reinterpret_cast<float*>(lds + NW * 64 * kG16Stride * 2);
+    gemm16_ln_bwd_tile<T, WN>(acc, mine, free_lds, C + batch * bsc, M, ldc, tm, m0, wm, wn, lane, ep.residual, pr.ln);
+  } else {
+    gemm16_write_tile<T, HAS_BIAS, SPLIT_K>(acc, mine, bias, C, partial, M, N, ldc, bsc, batch,
+                                            split, SPLIT_K ? batches : 1,
+                                            m0, n0, wm, wn, lane, ep, pr.partial_stream);
+  }
 }
 
 template <typename T, bool A_KC, bool B_KC, bool HAS_BIAS, bool SPLIT_K, int BK, int NSTAGE, int TM = 128>
@@ -1206,6 +1364,17 @@ __global__ __launch_bounds__(2 * TN, gemm16_pipe_occupancy(BK, NSTAGE, 128, TN))
   const int bid = blockIdx.x;
   if (bid < n_dw) gemm16_pipe_block<T, false, false, false, true, BK, NSTAGE, 128, TN>(lds, bid, dw);
   else gemm16_pipe_block<T, true, false, false, false, BK, NSTAGE, 128, TN>(lds, bid - n_dw, dx);
+}
+
+// The same launch with the dX tiles (128 x 384: whole rows of a 384-wide layer input) continuing
+// as the backward of the LayerNorm that produced the layer's input (gemm16_ln_bwd_tile).
+template <typename T>
+__global__ __launch_bounds__(2 * kGemmWideBN, 1) void linear_bwd_ln_16bit_kernel(Gemm16Problem<T> dw, Gemm16Problem<T> dx,
+                                                                                 int n_dw) {
+  __shared__ __attribute__((aligned(1024))) char lds[gemm16_pipe_lds_bytes(64, 2, 128, kGemmWideBN)];
+  const int bid = blockIdx.x;
+  if (bid < n_dw) gemm16_pipe_block<T, false, false, false, true, 64, 2, 128, kGemmWideBN>(lds, bid, dw);
+  else gemm16_pipe_block<T, true, false, false, false, 64, 2, 128, kGemmWideBN, true>(lds, bid - n_dw, dx);
 }
 
 // ------------------------------------------------------------------------------------

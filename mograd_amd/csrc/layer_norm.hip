@@ -34,8 +34,9 @@ static int ln_fwd(const void* x, const void* gamma, const void* beta, void* y, f
   }
 }
 
-static int ln_bwd(const void* dy, const void* x, const void* gamma, const float* mean, const float* rstd,
-                  const void* residual, void* dx, void* dgamma, void* dbeta, int64_t rows, int64_t cols, float eps,
+// (also the second half of mg_linear_bwd_layer_norm_bwd when its shapes take separate kernels)
+int ln_bwd(const void* dy, const void* x, const void* gamma, const float* mean, const float* rstd,
+           const void* residual, void* dx, void* dgamma, void* dbeta, int64_t rows, int64_t cols, float eps,
                   int dtype, mg_stream stream) {
   MG_TRY(check_ln("layer_norm_bwd", rows, cols, dtype));
   if (!dgamma || !dbeta) return fail(MG_ERR_INVALID, "layer_norm_bwd: null pointer argument");

@@ -685,6 +685,38 @@ inline Buffers layer_norm_bwd_stats(const OpRef& node, const Buffers& in, Device
   return {dx, dgamma, dbeta};
 }
 
+// LINEAR_LAYER_NORM_GRAD[dY (.., N), x (.., K), W (N, K), h (.., K), gamma, mean, rstd(, prior)]{has_bias, accumulate}
+// -> [dh, dgamma, dbeta, dW, db] for Y = x W^T (+ b) with x = LayerNorm(h): the layer's LINEAR_GRAD and the
+// LAYER_NORM_STATS_GRAD(_ADD) of the LayerNorm that feeds it as one node; dY W is never stored.
+inline Buffers linear_layer_norm_bwd(const OpRef& node, const Buffers& in, Device& device) {
+  const Layout &ldy = node.src(0).layout(), &lx = node.src(1).layout(), &lw = node.src(2).layout();
+  const bool accumulate = node.has_attr("accumulate") && node.attr("accumulate") != 0;
+  const bool has_bias = !node.has_attr("has_bias") || node.attr("has_bias") != 0;
+  const Buffers inputs = detail::materialise(node, in, device, accumulate ? 8 : 7);
+  detail::require_float(node.dtype(), "linear_layer_norm_bwd");
+  if (lw.rank() != 2) throw Error(MG_ERR_INVALID, "linear_layer_norm_bwd: W is not a matrix");
+  const int64_t N = lw.shape(0), K = lw.shape(1), M = lx.numel() / K;
+  if (ldy.numel() != M * N || node.src(3).layout().numel() != M * K)
+    throw Error(MG_ERR_INVALID, "linear_layer_norm_bwd: dY, x, W and h do not describe Y = LayerNorm(h) W^T");
+  AnyBuffer dh = AnyBuffer::create(node.dtype(), device, M * K);
+  if (accumulate)  // the kernel adds into dh: start it from the prior gradient
+    MOGRAD_CALL(device, mg_copy_device, dh.data_ptr(), inputs[7].data_ptr(), M * K * dtype_size(node.dtype()), device.stream());
+  AnyBuffer dgamma = AnyBuffer::create(node.dtype(), device, K);
+  AnyBuffer dbeta = AnyBuffer::create(node.dtype(), device, K);
+  AnyBuffer dw = AnyBuffer::create(node.dtype(), device, N * K);
+  Buffers out = {dh, dgamma, dbeta, dw};
+  void* db_ptr = nullptr;
+  if (has_bias) {
+    out.push_back(AnyBuffer::create(node.dtype(), device, N));
+    db_ptr = out.back().data_ptr();
+  }
+  MOGRAD_CALL(device, mg_linear_bwd_layer_norm_bwd, inputs[0].data_ptr(), inputs[1].data_ptr(), inputs[2].data_ptr(),
+              inputs[3].data_ptr(), inputs[4].data_ptr(), static_cast<const float*>(inputs[5].data_ptr()),
+              static_cast<const float*>(inputs[6].data_ptr()), dh.data_ptr(), dw.data_ptr(), db_ptr, dgamma.data_ptr(),
+              dbeta.data_ptr(), M, N, K, accumulate, node.dtype(), node.dtype(), device.pending, device.stream());
+  return out;
+}
+
 // MATMUL_BT_ADD[A, B (N, K), R] = A B^T + R, R laid out like the result.
 inline Buffers matmul_bt_add(const OpRef& node, const Buffers& inputs, Device& device) {
   const int64_t N = node.shape(node.layout().rank() - 1);
@@ -875,6 +907,42 @@ inline std::optional<OpRef> fuse_add_into_layer_norm_grad(const OpRef& node) {
   return std::nullopt;
 }
 
+// LAYER_NORM_STATS_GRAD(_ADD)(GETTUPLE0(LINEAR_GRAD(dy, x, w)), h, g, mean, rstd(, r)) ->
+// LINEAR_LAYER_NORM_GRAD[dy, x, w, h, g, mean, rstd(, r)]: outputs [dh, dgamma, dbeta, dW, db], so the selectors
+// of the LayerNorm node keep their indices and the product's dW and db are read at 3 and 4.  The caller
+// applies it only where nothing else reads the product's dX.
+inline std::optional<OpRef> fuse_linear_grad_into_layer_norm_grad(const OpRef& node) {
+  const bool with_residual = node.op_type == "LAYER_NORM_STATS_GRAD_ADD";
+  if ((node.op_type != "LAYER_NORM_STATS_GRAD" && !with_residual) || !is_output0_of(node.src(0), "LINEAR_GRAD"))
+    return std::nullopt;
+  const OpRef& lin = node.src(0).src(0);
+  if (lin.has_attr("relu_mask") || lin.has_attr("accumulate") || lin.dtype() != node.dtype()) return std::nullopt;
+  if (node.src(1).layout().numel() != node.src(0).layout().numel()) return std::nullopt;
+  OpRef fused{"LINEAR_LAYER_NORM_GRAD", node.layout(), node.dtype(),
+              {lin.src(0), lin.src(1), lin.src(2), node.src(1), node.src(2), node.src(3), node.src(4)},
+              {{"has_bias", !lin.has_attr("has_bias") || lin.attr("has_bias") != 0 ? 1.0 : 0.0}}};
+  if (with_residual) {
+    fused.srcs.push_back(node.src(5));
+    fused.node_attrs["accumulate"] = 1.0;
+  }
+  return fused;
+}
+
+// ADD(r, GETTUPLE0(LINEAR_LAYER_NORM_GRAD(..))) -> GETTUPLE0(LINEAR_LAYER_NORM_GRAD{accumulate}(.., r)).
+inline std::optional<OpRef> fuse_add_into_linear_layer_norm_grad(const OpRef& node) {
+  if (node.op_type != "ADD") return std::nullopt;
+  for (int i = 0; i < 2; ++i) {
+    const OpRef &sel = node.src(i), &other = node.src(1 - i);
+    if (!is_output0_of(sel, "LINEAR_LAYER_NORM_GRAD") || sel.src(0).has_attr("accumulate")) continue;
+    if (sel.layout().shape() != other.layout().shape() || sel.dtype() != other.dtype()) continue;
+    OpRef fused = sel.src(0);
+    fused.srcs.push_back(other);
+    fused.node_attrs["accumulate"] = 1.0;
+    return gettuple(fused, 0, sel.layout(), sel.dtype());
+  }
+  return std::nullopt;
+}
+
 // CONTIGUOUS(TRANSPOSE{1,2}(GETTUPLE0(FLASH_ATTN(q, k, v, mask)))) -> GETTUPLE0(FLASH_ATTN{layout: bshd}(...)).
 inline std::optional<OpRef> fuse_attention_output_layout(const OpRef& node) {
   if (node.op_type != "CONTIGUOUS" || node.src(0).op_type != "TRANSPOSE" || !is_output0_of(node.src(0).src(0), "FLASH_ATTN"))
@@ -953,6 +1021,7 @@ inline const std::vector<Rule>& scheduler_rules() {
       {"MATMUL_BT_ADD", "matmul_bt_add", matmul_bt_add},
       {"MATMUL_BIAS_RELU_BT", "matmul_bias_relu_bt", matmul_bias_relu_bt},
       {"LAYER_NORM_STATS_GRAD_ADD", "layer_norm_bwd_stats", layer_norm_bwd_stats},
+      {"LINEAR_LAYER_NORM_GRAD", "linear_layer_norm_bwd", linear_layer_norm_bwd},
       {"FLASH_ATTN_PACKED", "flash_attn_packed_fwd", flash_attn_packed_fwd},
       {"FLASH_ATTN_PACKED_GRAD", "flash_attn_packed_bwd", flash_attn_packed_bwd},
   };

@@ -119,6 +119,8 @@ class Simplifier:
         for r in roots:  # a root is read by the caller
             self.uses[r] = self.uses.get(r, 0) + 1
         for node in topo:
+            if node in self.subst:  # a rule that ran on another node has already replaced this one
+                continue
             node_r = self._with_subst(node)
             for _ in range(64):
                 progressed = False
@@ -247,6 +249,48 @@ def fuse_add_into_layer_norm_grad(node: Node, sim: Simplifier) -> Optional[Node]
     return None
 
 
+def fuse_linear_grad_into_layer_norm_grad(node: Node, sim: Simplifier) -> Optional[Node]:
+    """LAYER_NORM_STATS_GRAD(GETTUPLE0(LINEAR_GRAD(dy, x, w)), h, g, mean, rstd) ->
+    LINEAR_LAYER_NORM_GRAD[dy, x, w, h, g, mean, rstd] with outputs [dh, dgamma, dbeta, dW, db]: the input
+    gradient of a Linear layer that only the backward of the LayerNorm feeding the layer reads.  The
+    LayerNorm node's selectors keep their indices; the product's dW and db selectors move to 3 and 4."""
+    sel = node.src(0)
+    if sel.op_type != "GETTUPLE" or int(sel.attrs().get("index", -1)) != 0 or sel.src(0).op_type != "LINEAR_GRAD":
+        return None
+    lin = sel.src(0)
+    if lin.attrs().get("relu_mask") or lin.attrs().get("accumulate") or not sim.single_use(sel):
+        return None
+    if node.src(1).layout().numel() != sel.layout().numel() or node.dtype() != lin.dtype():
+        return None
+    attrs = {"has_bias": bool(lin.attrs().get("has_bias", True))}
+    srcs = list(lin.srcs[:3]) + list(node.srcs[1:5])
+    if node.op_type == "LAYER_NORM_STATS_GRAD_ADD":
+        srcs.append(node.src(5))
+        attrs["accumulate"] = True
+    new = Node("LINEAR_LAYER_NORM_GRAD", node.node_layout, node.node_dtype, srcs, attrs)
+    for c in sim.consumers_of(lin):  # dW and db of the product now come from the new node
+        index = int(c.attrs().get("index", -1)) if c.op_type == "GETTUPLE" else -1
+        if index in (1, 2):
+            moved = Node("GETTUPLE", c.node_layout, c.node_dtype, [new], {"index": index + 2})
+            sim.replace(sim.resolve(c), moved)
+    return new
+
+
+def fuse_add_into_linear_layer_norm_grad(node: Node, sim: Simplifier) -> Optional[Node]:
+    """ADD(r, GETTUPLE0(LINEAR_LAYER_NORM_GRAD(..))) -> GETTUPLE0(LINEAR_LAYER_NORM_GRAD{accumulate}(.., r))."""
+    for sel, other in ((node.src(0), node.src(1)), (node.src(1), node.src(0))):
+        if sel.op_type != "GETTUPLE" or sel.src(0).op_type != "LINEAR_LAYER_NORM_GRAD":
+            continue
+        fused = sel.src(0)
+        if int(sel.attrs().get("index", -1)) != 0 or fused.attrs().get("accumulate") or not sim.single_use(sel):
+            continue
+        if not _same_shape(sel, other) or other.dtype() != sel.dtype() or fused in _toposort(other):
+            continue
+        new = _refit(fused, "LINEAR_LAYER_NORM_GRAD", list(fused.srcs) + [other], {**fused.attrs(), "accumulate": True}, sim)
+        return Node("GETTUPLE", sel.node_layout, sel.node_dtype, [new], {"index": 0})
+    return None
+
+
 def _is_bhsd_to_bshd(tr: Node) -> bool:
     d0, d1 = int(tr.attrs().get("dim0", -2)) % 4, int(tr.attrs().get("dim1", -1)) % 4
     return tr.layout().rank() == 4 and {d0, d1} == {1, 2}
@@ -307,7 +351,12 @@ def GPU_REWRITES() -> List[Rule]:
         Rule(Pat("CONTIGUOUS", [Pat("TRANSPOSE", [get0("FLASH_ATTN")])]), fuse_attention_output_layout,
              "fuse_attention_output_layout"),
         Rule(Pat("FLASH_ATTN_GRAD"), fuse_attention_grad_layout, "fuse_attention_grad_layout"),
+        Rule(Pat("LAYER_NORM_STATS_GRAD", [get0("LINEAR_GRAD")]), fuse_linear_grad_into_layer_norm_grad,
+             "fuse_linear_grad_into_layer_norm_grad"),
+        Rule(Pat("LAYER_NORM_STATS_GRAD_ADD", [get0("LINEAR_GRAD")]), fuse_linear_grad_into_layer_norm_grad,
+             "fuse_linear_grad_into_layer_norm_grad"),
         Rule(Pat("ADD"), fuse_matmul_add, "fuse_matmul_add"),
         Rule(Pat("ADD"), fuse_add_into_layer_norm_grad, "fuse_add_into_layer_norm_grad"),
+        Rule(Pat("ADD"), fuse_add_into_linear_layer_norm_grad, "fuse_add_into_linear_layer_norm_grad"),
         Rule(Pat("ADD"), fuse_add_into_linear_grad, "fuse_add_into_linear_grad"),
     ]

@@ -747,6 +747,35 @@ def layer_norm_bwd_stats(node: Node, inputs: List[AnyBuffer], device: Device) ->
     return [dx, dgamma, dbeta]
 
 
+def linear_layer_norm_bwd(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
+    """LINEAR_LAYER_NORM_GRAD[dY (.., N), x (.., K), W (N, K), h (.., K), gamma, mean, rstd(, prior)]{has_bias,
+    accumulate} -> [dh, dgamma, dbeta, dW, db] for Y = x W^T (+ b) with x = LayerNorm(h): the
+    LINEAR_GRAD of the layer and the LAYER_NORM_STATS_GRAD(_ADD) of the LayerNorm that feeds it as
+    one node (mg_linear_bwd_layer_norm_bwd), dY W never stored.  accumulate: dh = prior + the
+    LayerNorm's input gradient, `prior` the eighth source."""
+    ldy, lx, lw = (node.src(i).layout() for i in range(3))
+    accumulate = bool(node.attrs().get("accumulate", False))
+    has_bias = bool(node.attrs().get("has_bias", True))
+    inputs = _materialise(node, inputs, device, 8 if accumulate else 7)
+    _require_float(node.dtype(), "linear_layer_norm_bwd")
+    N, K = lw.shape(0), lw.shape(1)
+    M = lx.numel() // K
+    if ldy.numel() != M * N or lw.rank() != 2 or node.src(3).layout().numel() != M * K:
+        raise MogradError(1, "linear_layer_norm_bwd: dY, x, W and h do not describe Y = LayerNorm(h) W^T")
+    dh = AnyBuffer.create(node.dtype(), device, M * K)
+    if accumulate:  # the kernel adds into dh: start it from the prior gradient
+        device.lib.mg_copy_device(dh.data_ptr(), inputs[7].data_ptr(), dh.size_bytes(), device.stream)
+    dgamma = AnyBuffer.create(node.dtype(), device, K)
+    dbeta = AnyBuffer.create(node.dtype(), device, K)
+    dw = AnyBuffer.create(node.dtype(), device, N * K)
+    db = AnyBuffer.create(node.dtype(), device, N) if has_bias else None
+    device.lib.mg_linear_bwd_layer_norm_bwd(*(inputs[i].data_ptr() for i in range(7)), dh.data_ptr(), dw.data_ptr(),
+                                            db.data_ptr() if has_bias else None, dgamma.data_ptr(), dbeta.data_ptr(),
+                                            M, N, K, int(accumulate), node.dtype(), node.dtype(), device.pending,
+                                            device.stream)
+    return [dh, dgamma, dbeta, dw, db] if has_bias else [dh, dgamma, dbeta, dw]
+
+
 def matmul_bt_add(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     """MATMUL_BT_ADD[A, B (N, K), R] = A B^T + R (R laid out like the result): the residual
     addition of a transformer block on the product that feeds it."""
@@ -889,6 +918,7 @@ SCHEDULER_RULES = {
     "MATMUL_BT_ADD": matmul_bt_add,
     "MATMUL_BIAS_RELU_BT": matmul_bias_relu_bt,
     "LAYER_NORM_STATS_GRAD_ADD": layer_norm_bwd_stats,
+    "LINEAR_LAYER_NORM_GRAD": linear_layer_norm_bwd,
     "FLASH_ATTN_PACKED": flash_attn_packed_fwd,
     "FLASH_ATTN_PACKED_GRAD": flash_attn_packed_bwd,
 }

@@ -11,7 +11,8 @@ The backward pass is the graph mograd/grad.mojo builds for that forward, with th
 entries in place of their unfused chains: mg_linear_bwd(_fused) for every Linear (with the
 ReLU gradient folded into the dX product; the Q, K and V projections are one Linear with
 the stacked (3d, d) weight, so their input and weight gradients are one product each),
-mg_layer_norm_bwd_stats_add (the gradient added to the skip connection's in place),
+mg_linear_bwd_layer_norm_bwd where a LayerNorm feeds a Linear (the LayerNorm's backward rides on
+the product's dX tiles and its result is added to the skip connection's gradient in place),
 mg_flash_attn_bwd_packed (Q | K | V and dQ | dK | dV as one (B,T,3,H,dh) tensor each, O and
 dO in the projections' (B,T,H,dh) layout, so no transposing copies),
 mg_cross_entropy_fused_ids, mg_scatter_add for the embedding; in the forward the residual additions and the ReLU ride on the products
@@ -160,7 +161,7 @@ class TinyTransformer:
                 "h_mid": new(n * d), "x2": new(n * d), "a": new(n * ff),
                 "mean1": new(n, F32), "rstd1": new(n, F32), "mean2": new(n, F32), "rstd2": new(n, F32),
             })
-        self.tmp = {name: new(n * d) for name in ("dh", "dctx", "dx_a")}
+        self.tmp = {name: new(n * d) for name in ("dh", "dctx")}
         self.tmp["dqkv"] = new(3 * n * d)  # dQ | dK | dV per token
         self.tmp["da"] = new(n * ff)
         self.tmp["logits"] = new(n * V)
@@ -228,14 +229,16 @@ class TinyTransformer:
             def lin_bwd(dy, x, w, dx, dw, db, N, K, accumulate=0, relu=0):
                 lib.mg_linear_bwd_deferred(dy, x, w, dx, dw, db, n, N, K, accumulate, relu, cd, F32, q, s)
 
-            def ln_bwd(dy, x, gam, mean, rstd, dg, db):  # dh += LayerNorm backward
-                lib.mg_layer_norm_bwd_stats_deferred(dy, x, gam, mean, rstd, t["dh"], t["dh"], dg, db, n, d, cd, F32, q, s)
+            def lin_ln_bwd(dy, x, w, dw, db, N, h, gam, mean, rstd, dg, dbt):  # dh += LayerNorm backward of dY W
+                lib.mg_linear_bwd_layer_norm_bwd(dy, x, w, h, gam, mean, rstd, t["dh"], dw, db, dg, dbt, n, N, d, 1, cd,
+                                                 F32, q, s)
         else:
             def lin_bwd(dy, x, w, dx, dw, db, N, K, accumulate=0, relu=0):
                 lib.mg_linear_bwd_fused(dy, x, w, dx, dw, db, n, N, K, accumulate, relu, cd, s)
 
-            def ln_bwd(dy, x, gam, mean, rstd, dg, db):
-                lib.mg_layer_norm_bwd_stats_add(dy, x, gam, mean, rstd, t["dh"], t["dh"], dg, db, n, d, cd, s)
+            def lin_ln_bwd(dy, x, w, dw, db, N, h, gam, mean, rstd, dg, dbt):
+                lib.mg_linear_bwd_layer_norm_bwd(dy, x, w, h, gam, mean, rstd, t["dh"], dw, db, dg, dbt, n, N, d, 1, cd,
+                                                 cd, None, s)
 
         lin_bwd(t["dlogits"], P(self.h[self.L]), self._w("lm_head"), t["dh"], self._g("lm_head"), None, V, d)
         for l in reversed(range(self.L)):
@@ -244,17 +247,18 @@ class TinyTransformer:
             g = lambda name, l=l: self._g(f"blocks.{l}.{name}")
             # h_out = h_mid + W2 a; the ReLU's gradient rides on the dX product
             lin_bwd(t["dh"], P(c["a"]), w("w2"), t["da"], g("w2"), None, d, ff, relu=1)
-            lin_bwd(t["da"], P(c["x2"]), w("w1"), t["dx_a"], g("w1"), g("b1"), ff, d)
-            # dh += LayerNorm backward: the skip connection's share is already in dh
-            ln_bwd(t["dx_a"], P(c["h_mid"]), w("ln2_g"), P(c["mean2"]), P(c["rstd2"]), g("ln2_g"), g("ln2_b"))
+            # the layer's input is LayerNorm(h_mid): its backward rides on the dX tiles, dh += the result
+            # (the skip connection's share is already in dh)
+            lin_ln_bwd(t["da"], P(c["x2"]), w("w1"), g("w1"), g("b1"), ff, P(c["h_mid"]), w("ln2_g"), P(c["mean2"]),
+                       P(c["rstd2"]), g("ln2_g"), g("ln2_b"))
             # h_mid = h_in + W_O ctx
             lin_bwd(t["dh"], P(c["ctx"]), w("wo"), t["dctx"], g("wo"), None, d, d)
             # dctx and ctx are (B, T, H, dh); dQ | dK | dV come back as one (n, 3d) tensor
             lib.mg_flash_attn_bwd_packed(t["dctx"], P(c["ctx"]), P(c["qkv"]), None, P(c["lse"]), t["dqkv"], B, T, H, dh,
                                          scale, 1, 0, cd, s)
             # gradient of the stacked projection: dx1 (n, d) and dW (3d, d) = dwq | dwk | dwv
-            lin_bwd(t["dqkv"], P(c["x1"]), w("wq"), t["dx_a"], g("wq"), None, 3 * d, d)
-            ln_bwd(t["dx_a"], P(self.h[l]), w("ln1_g"), P(c["mean1"]), P(c["rstd1"]), g("ln1_g"), g("ln1_b"))
+            lin_ln_bwd(t["dqkv"], P(c["x1"]), w("wq"), g("wq"), None, 3 * d, P(self.h[l]), w("ln1_g"), P(c["mean1"]),
+                       P(c["rstd1"]), g("ln1_g"), g("ln1_b"))
         if self.deferred:
             lib.mg_scatter_add_deferred(P(ids), t["dh"], self._g("embed"), n, V, d, ids.dtype, cd, F32, self.pending, s)
             lib.mg_finish_deferred(self.pending, s)

@@ -481,6 +481,41 @@ int main(int argc, char** argv) {
       return "deferred sums differ";
     return "";
   });
+  run_case("rewrites: a Linear layer's backward continued through the LayerNorm that feeds it", [&]() -> std::string {
+    // fp32 tensors take the separate kernels inside the one entry: the same bits as the two nodes
+    const int64_t rows = 48, cols = 32, N = 24;
+    const Layout lh{rows, cols}, lv{cols}, lr{rows}, lw{N, cols}, ldy{rows, N};
+    const auto h = ints(rows * cols, 51, -5, 5), dy = ints(rows * N, 52, -3, 3), w = ints(N * cols, 53, -2, 2),
+               res = ints(rows * cols, 54, -7, 7);
+    std::vector<float> g(cols, 1.f), b(cols, 0.f);
+    for (int64_t c = 0; c < cols; ++c) g[c] = 0.5f + 0.125f * static_cast<float>(c % 8);
+    const OpRef fwd = node("LAYER_NORM_STATS", lh, {OpRef::leaf(lh), OpRef::leaf(lv), OpRef::leaf(lv)}, {{"eps", 1e-5}});
+    AnyBuffer bh = upload(dev, h), bg = upload(dev, g), bdy = upload(dev, dy), bw = upload(dev, w), bres = upload(dev, res);
+    auto f = run(fwd, {bh, bg, upload(dev, b)}, dev);
+    const OpRef x = gettuple(fwd, 0, lh, float32);
+    const OpRef y = node("MATMUL_BIAS_BT", ldy, {x, OpRef::leaf(lw), OpRef::leaf(Layout{N})});
+    const OpRef lin = linear_grad(y, OpRef::leaf(ldy));
+    const OpRef ln = layer_norm_stats_grad(fwd, gettuple(lin, 0, lh, float32), OpRef::leaf(lr), OpRef::leaf(lr));
+    const auto fused = fuse_linear_grad_into_layer_norm_grad(ln);
+    if (!fused || fused->op_type != "LINEAR_LAYER_NORM_GRAD" || fused->srcs.size() != 7)
+      return "LAYER_NORM_STATS_GRAD(LINEAR_GRAD[0], ..) was not rewritten";
+    const auto accum = fuse_add_into_linear_layer_norm_grad(node("ADD", lh, {OpRef::leaf(lh), gettuple(*fused, 0, lh, float32)}));
+    if (!accum || accum->src(0).srcs.size() != 8) return "ADD(r, LINEAR_LAYER_NORM_GRAD[0]) was not rewritten";
+    auto l0 = run(lin, {bdy, f[0], bw}, dev);
+    auto n0 = run(ln, {l0[0], bh, bg, f[1], f[2]}, dev);
+    auto a0 = run(node("ADD", lh, {OpRef::leaf(lh), OpRef::leaf(lh)}), {bres, n0[0]}, dev);
+    auto f1 = run(*fused, {bdy, f[0], bw, bh, bg, f[1], f[2]}, dev);
+    auto f2 = run(accum->src(0), {bdy, f[0], bw, bh, bg, f[1], f[2], bres}, dev);
+    if (download(f1[0]) != download(n0[0]) || download(f2[0]) != download(a0[0])) return "dh differs from the two nodes";
+    if (download(f1[1]) != download(n0[1]) || download(f1[2]) != download(n0[2])) return "dgamma / dbeta differ";
+    if (download(f1[3]) != download(l0[1]) || download(f1[4]) != download(l0[2])) return "dW / db differ";
+    DeferredSums sums(dev);
+    auto f3 = run(accum->src(0), {bdy, f[0], bw, bh, bg, f[1], f[2], bres}, dev);
+    sums.finish();
+    for (size_t i = 0; i < 5; ++i)
+      if (download(f3[i]) != download(f2[i])) return "deferred sums differ";
+    return "";
+  });
   run_case("rewrites: attention output written (B, S, H, D)", [&]() -> std::string {
     const int64_t B = 1, S = 8, H = 2, D = 8;
     const Layout bshd{B, S, H, D}, bhsd{B, H, S, D};

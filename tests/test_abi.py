@@ -89,5 +89,6 @@ def test_scheduler_rules_cover_the_path():
         # fused nodes of the gradient rules the reference lacks
         "LINEAR_GRAD", "LAYER_NORM_STATS", "LAYER_NORM_STATS_GRAD", "CROSS_ENTROPY_IDS", "CROSS_ENTROPY_IDS_GRAD",
         # views, and the fused nodes of mograd_amd.rewrites.GPU_REWRITES
-        "RESHAPE", "TRANSPOSE", "EXPAND", "MATMUL_BT_ADD", "MATMUL_BIAS_RELU_BT", "LAYER_NORM_STATS_GRAD_ADD", "FLASH_ATTN_PACKED",
+        "RESHAPE", "TRANSPOSE", "EXPAND", "MATMUL_BT_ADD", "MATMUL_BIAS_RELU_BT", "LAYER_NORM_STATS_GRAD_ADD", "LINEAR_LAYER_NORM_GRAD",
+        "FLASH_ATTN_PACKED",
         "FLASH_ATTN_PACKED_GRAD"}

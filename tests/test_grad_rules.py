@@ -294,8 +294,12 @@ def test_transformer_step_through_the_rule_tables(device, dtype, V, d, ff, L, H,
             np.testing.assert_array_equal(buf.to_numpy(expect.shape), expect, err_msg=f"{name} (deferred {deferred_sums})")
     counts = _op_counts(roots)
     assert counts.get("MATMUL_BT_ADD") == 2 * L and counts.get("MATMUL_BIAS_RELU_BT") == L
-    assert counts.get("LAYER_NORM_STATS_GRAD_ADD") == 2 * L and "LAYER_NORM_STATS_GRAD" not in counts
-    assert counts.get("LINEAR_GRAD") == 4 * L + 1
+    # both LayerNorms of a block feed a Linear layer: their backward rides on that layer's
+    assert counts.get("LINEAR_LAYER_NORM_GRAD") == 2 * L and counts.get("LINEAR_GRAD") == 2 * L + 1
+    assert "LAYER_NORM_STATS_GRAD" not in counts and "LAYER_NORM_STATS_GRAD_ADD" not in counts
+    from mograd_amd.runtime import _toposort
+    assert all(nd.attrs().get("accumulate") for nd in _toposort(Node("SINK", Layout(1), F32, list(roots)))
+               if nd.op_type == "LINEAR_LAYER_NORM_GRAD")
     for gone in ("ADD", "RELU", "RELU_GRAD"):
         assert gone not in counts, f"{gone} survived the rewrites: {counts}"
 
@@ -365,6 +369,27 @@ def test_rewrite_rules_on_graph_structure():
     dx2, dw2 = Simplifier(GPU_REWRITES()).run_many([dx, dw])
     assert dx2.op_type == "GETTUPLE" and dx2.src(0).op_type == "LINEAR_GRAD" and dx2.src(0).attrs()["relu_mask"] is True
     assert dw2.src(0) is dx2.src(0), "dW reads the refitted node, not a second copy of the product"
+    # a LayerNorm that feeds a Linear layer on a skip connection: h2 = h + Linear(LayerNorm(h)).  The
+    # LayerNorm's backward and the ADD of the skip connection's share fold into the layer's backward;
+    # dW and db move to the new node's outputs 3 and 4, and the product is not computed twice.
+    hh, gam, bet, wl, bl = (Node.leaf(Layout(*sh)) for sh in ((4, 8), (8,), (8,), (6, 8), (6,)))
+    ln = Node("LAYER_NORM_STATS", Layout(4, 8), F32, [hh, gam, bet], {"eps": 1e-5})
+    xn = Node("GETTUPLE", Layout(4, 8), F32, [ln], {"index": 0})
+    lin_out = Node("MATMUL_BIAS_BT", Layout(4, 6), F32, [xn, wl, bl])
+    w_back = Node.leaf(Layout(8, 6))
+    h2 = Node("ADD", Layout(4, 8), F32, [hh, Node("MATMUL_BT", Layout(4, 8), F32, [lin_out, w_back])])
+    grads = R.gradient(h2, Node.leaf(Layout(4, 8)), [hh, gam, bet, wl, bl])
+    dh, dgam, dbet, dwl, dbl = Simplifier(GPU_REWRITES()).run_many(grads)
+    fused = dh.src(0)
+    assert dh.op_type == "GETTUPLE" and fused.op_type == "LINEAR_LAYER_NORM_GRAD" and fused.attrs()["accumulate"] is True
+    assert len(fused.srcs) == 8 and fused.srcs[1] is xn and fused.srcs[2] is wl and fused.srcs[3] is hh
+    for sel, index in ((dh, 0), (dgam, 1), (dbet, 2), (dwl, 3), (dbl, 4)):
+        assert sel.op_type == "GETTUPLE" and sel.src(0) is fused and sel.attrs()["index"] == index
+    assert _op_counts([dh, dgam, dbet, dwl, dbl]).get("LINEAR_GRAD") == 1  # only the one of w_back is left
+    # dX of the product has a second reader: the two nodes stay apart
+    grads = R.gradient(h2, Node.leaf(Layout(4, 8)), [hh, xn])
+    kept = Simplifier(GPU_REWRITES()).run_many(grads)
+    assert kept[0].src(0).op_type == "LAYER_NORM_STATS_GRAD_ADD" and kept[1].src(0).op_type == "LINEAR_GRAD"
     # the gradient rules added for residual and embedding graphs
     emb, idx = Node.leaf(Layout(10, 8)), Node.leaf(Layout(4), I32)
     h = Node("GATHER", Layout(4, 8), F32, [emb, idx])

@@ -5,6 +5,8 @@ The operand layouts are the ones mograd's graph produces for a Linear layer
 X W^T + b, dX = MATMUL_BT(dY, TRANSPOSE(W)) with a strided right operand, and
 dW^T = MATMUL(TRANSPOSE(X), dY) with a strided left operand; db = SUM(axis=0).
 """
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -641,6 +643,77 @@ def test_linear_bwd_ragged_width(device, monkeypatch, dtype, rtol, M, N, K):
     for mode in ("0", "1"):
         assert_close(results[mode][0], want_dx, 2 * rtol, 2 * rtol * np.abs(want_dx).max(), "dx " + mode)
         assert_close(results[mode][1], want_dw, rtol, rtol * np.abs(want_dw).max(), "dw " + mode)
+
+
+LN_CONT_SHAPES = [(4096, 1152, 384), (2048, 1536, 384), (2112, 768, 384), (16384, 1536, 384),  # one launch, whole rows
+                  (1024, 384, 384), (512, 96, 200), (2048, 832, 768)]                              # separate kernels
+
+
+@pytest.mark.parametrize("deferred", [False, True])
+@pytest.mark.parametrize("dtype", [BF16, F16, F32])
+@pytest.mark.parametrize("M,N,K", LN_CONT_SHAPES)
+def test_linear_bwd_continues_as_layer_norm_bwd(device, dtype, M, N, K, deferred):
+    # Y = LN(h) W^T + b: the layer's backward and the LayerNorm's in one entry.  For 16-bit layers
+    # of 384 input columns the dX tiles hold whole rows and finish as the LayerNorm backward
+    # inside the launch ((2112, ..): the last tile is half empty); other shapes and fp32 run the
+    # two separate entries on a scratch tensor.  Either way dW and db are the separate entry's
+    # bits, and dh, dgamma and dbeta differ from the separate calls only by the order of their
+    # fp32 sums; the oracle gets the same dY W rounded to the tensors' type.
+    if dtype == F32 and M * N * K > 2048 * 1536 * 384:
+        pytest.skip("the fp32 path is the two separate entries: one large case is enough")
+    lib, st = device.lib, device.stream
+    h = round_to_dtype(normal(81, 0, (M, K), std=1.5) + 0.3, dtype)
+    gamma = round_to_dtype(uniform(81, 1, (K,), 0.5, 1.5), dtype)
+    beta = round_to_dtype(normal(81, 2, (K,), std=0.1), dtype)
+    w = round_to_dtype(normal(81, 3, (N, K), std=0.1), dtype)
+    dy = round_to_dtype(normal(81, 4, (M, N), std=0.5), dtype)
+    prior = round_to_dtype(normal(81, 5, (M, K)), dtype)
+    bh, bg, bbeta, bw, bdy, bprior = (AnyBuffer.from_numpy(device, a, dtype) for a in (h, gamma, beta, w, dy, prior))
+    new = lambda n, dt=dtype: AnyBuffer.create(dt, device, n)  # noqa: E731
+    x, mean, rstd = new(M * K), new(M, F32), new(M, F32)
+    lib.mg_layer_norm_fwd_stats(_ptr(bh), _ptr(bg), _ptr(bbeta), _ptr(x), _ptr(mean), _ptr(rstd), M, K, 1e-5, dtype, st)
+    # the two separate entries
+    t, dh_ref, dw_ref, db_ref, dg_ref, dbt_ref = new(M * K), new(M * K), new(N * K), new(N), new(K), new(K)
+    lib.mg_linear_bwd(_ptr(bdy), _ptr(x), _ptr(bw), _ptr(t), _ptr(dw_ref), _ptr(db_ref), M, N, K, dtype, st)
+    lib.mg_layer_norm_bwd_stats_add(_ptr(t), _ptr(bh), _ptr(bg), _ptr(mean), _ptr(rstd), _ptr(bprior), _ptr(dh_ref),
+                                    _ptr(dg_ref), _ptr(dbt_ref), M, K, dtype, st)
+    # the one entry, dh in place on top of the prior gradient
+    gdt = F32 if deferred else dtype
+    dh = AnyBuffer.from_numpy(device, prior, dtype)
+    dw, db, dg, dbt = new(N * K, gdt), new(N, gdt), new(K, gdt), new(K, gdt)
+    pending = C.c_void_p()
+    if deferred:
+        lib.mg_deferred_create(C.byref(pending))
+    try:
+        lib.mg_linear_bwd_layer_norm_bwd(_ptr(bdy), _ptr(x), _ptr(bw), _ptr(bh), _ptr(bg), _ptr(mean), _ptr(rstd), _ptr(dh),
+                                         _ptr(dw), _ptr(db), _ptr(dg), _ptr(dbt), M, N, K, 1, dtype, gdt,
+                                         pending if deferred else None, st)
+        if deferred:
+            lib.mg_finish_deferred(pending, st)
+    finally:
+        if deferred:
+            lib.mg_deferred_destroy(pending)
+    ulp = {F32: 2.0 ** -21, F16: 2.0 ** -9, BF16: 2.0 ** -6}[dtype]  # two units in the last place
+    if deferred:  # fp32 sums before the rounding of the immediate forms
+        np.testing.assert_array_equal(round_to_dtype(dw.to_numpy(), dtype), dw_ref.to_numpy())
+        np.testing.assert_array_equal(round_to_dtype(db.to_numpy(), dtype), db_ref.to_numpy())
+    else:
+        np.testing.assert_array_equal(dw.to_numpy(), dw_ref.to_numpy())
+        np.testing.assert_array_equal(db.to_numpy(), db_ref.to_numpy())
+    got, ref = dh.to_numpy((M, K)).astype(np.float64), dh_ref.to_numpy((M, K)).astype(np.float64)
+    # (the gradient is rounded before the prior is added: a unit in its last place, not the sum's)
+    assert np.all(np.abs(got - ref) <= ulp * (np.abs(ref) + np.abs(prior)) + 1e-5 * np.abs(ref).max())
+    assert np.mean(got == ref) > 0.98
+    tv = t.to_numpy((M, K)).astype(np.float64)
+    for g_, r_, mass in ((dg, dg_ref, np.abs(tv).sum(axis=0) * 4.0), (dbt, dbt_ref, np.abs(tv).sum(axis=0))):
+        gv, rv = g_.to_numpy().astype(np.float64), r_.to_numpy().astype(np.float64)
+        assert np.all(np.abs(gv - rv) <= ulp * np.abs(rv) + 2.0 ** -20 * mass)
+    if M <= 4096:  # and the oracle, from the rounded dY W the kernels saw
+        odx, odg, odb = O.layer_norm_bwd(tv, h, gamma)
+        rt = {F32: 1e-4, F16: 2e-3, BF16: 1.6e-2}[dtype]
+        assert_close(got, round_to_dtype(odx, dtype).astype(np.float64) + prior, rt, rt * np.abs(odx).max(), "dh")
+        assert_close(dg.to_numpy(), odg, rt, rt * np.abs(odg).max(), "dgamma")
+        assert_close(dbt.to_numpy(), odb, rt, rt * np.abs(odb).max(), "dbeta")
 
 
 def test_fused_entry_errors(device):
