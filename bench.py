@@ -649,11 +649,20 @@ def bench_gpt(args, dev) -> dict:
          5.0 * attn_fl, "F", PF),
         ("flash_attn_fwd_packed bf16 causal B64 H6 S256 D64 (2 B H S^2 D)",
          lambda i: lib.mg_flash_attn_fwd_packed(P(qkv), None, P(o), P(lse), B, T, H, dh, sc, 1, 0, BF16, st), 2.0 * attn_fl, "F", PF),
-        ("layer_norm_bwd_stats_deferred bf16 (16384, 384), dx accumulated in place, dgamma/dbeta sums deferred; "
-         + CACHED,
+        ("layer_norm_bwd_stats_deferred bf16 (16384, 384), dx accumulated in place, dgamma/dbeta sums deferred (not in "
+         "the step since the Linear backward after each LayerNorm carries it: the next two rows); " + CACHED,
          lambda i: lib.mg_layer_norm_bwd_stats_deferred(P(dy_d), P(x_d), P(gam), P(mean), P(rstd), P(out_d), P(out_d), P(dg32),
                                                         P(dbt32), n, d, BF16, F32, pending, st),
          4 * n * d * e2 + 2 * n * 4 + 3 * d * e2, "B", None),
+        ("linear_bwd_layer_norm_bwd bf16, stacked Q|K|V projection (16384, 1152<-384): linear_bwd_deferred plus the "
+         "backward of the LayerNorm that feeds the layer, from the dX tiles (4 M N K FLOP counted; in the step)",
+         lambda i: lib.mg_linear_bwd_layer_norm_bwd(P(dqkv), P(x_d), P(w_qkv), P(x_ff), P(gam), P(mean), P(rstd), P(out_d),
+                                                    P(dw32), None, P(dg32), P(dbt32), n, 3 * d, d, 1, BF16, F32, pending, st),
+         12.0 * n * d * d, "F", PF),
+        ("linear_bwd_layer_norm_bwd bf16 (16384, 1536<-384) with db: likewise (in the step)",
+         lambda i: lib.mg_linear_bwd_layer_norm_bwd(P(dy_ff), P(x_d), P(w_fd), P(x_ff), P(gam), P(mean), P(rstd), P(out_d),
+                                                    P(dw32), P(db32), P(dg32), P(dbt32), n, ff, d, 1, BF16, F32, pending, st),
+         4.0 * n * d * ff, "F", PF),
         ("layer_norm_fwd_stats bf16 (16384, 384); " + CACHED,
          lambda i: lib.mg_layer_norm_fwd_stats(P(x_d), P(gam), P(bet), P(out_d), P(mean), P(rstd), n, d, 1e-5, BF16, st),
          2 * n * d * e2 + 2 * n * 4 + 2 * d * e2, "B", None),
