@@ -649,9 +649,13 @@ LN_CONT_SHAPES = [(4096, 1152, 384), (2048, 1536, 384), (2112, 768, 384), (16384
                   (1024, 384, 384), (512, 96, 200), (2048, 832, 768)]                              # separate kernels
 
 
+# fp32 always takes the two separate entries: the largest shapes add nothing there
+LN_CONT_CASES = [(dt, *shape) for dt in (BF16, F16, F32) for shape in LN_CONT_SHAPES
+                 if dt != F32 or shape[0] * shape[1] * shape[2] <= 2048 * 1536 * 384]
+
+
 @pytest.mark.parametrize("deferred", [False, True])
-@pytest.mark.parametrize("dtype", [BF16, F16, F32])
-@pytest.mark.parametrize("M,N,K", LN_CONT_SHAPES)
+@pytest.mark.parametrize("dtype,M,N,K", LN_CONT_CASES)
 def test_linear_bwd_continues_as_layer_norm_bwd(device, dtype, M, N, K, deferred):
     # Y = LN(h) W^T + b: the layer's backward and the LayerNorm's in one entry.  For 16-bit layers
     # of 384 input columns the dX tiles hold whole rows and finish as the LayerNorm backward
@@ -659,8 +663,6 @@ def test_linear_bwd_continues_as_layer_norm_bwd(device, dtype, M, N, K, deferred
     # two separate entries on a scratch tensor.  Either way dW and db are the separate entry's
     # bits, and dh, dgamma and dbeta differ from the separate calls only by the order of their
     # fp32 sums; the oracle gets the same dY W rounded to the tensors' type.
-    if dtype == F32 and M * N * K > 2048 * 1536 * 384:
-        pytest.skip("the fp32 path is the two separate entries: one large case is enough")
     lib, st = device.lib, device.stream
     h = round_to_dtype(normal(81, 0, (M, K), std=1.5) + 0.3, dtype)
     gamma = round_to_dtype(uniform(81, 1, (K,), 0.5, 1.5), dtype)
