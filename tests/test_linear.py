@@ -718,6 +718,42 @@ def test_linear_bwd_continues_as_layer_norm_bwd(device, dtype, M, N, K, deferred
         assert_close(dbt.to_numpy(), odb, rt, rt * np.abs(odb).max(), "dbeta")
 
 
+@pytest.mark.parametrize("M,N,K", [(2048, 1152, 384), (1024, 384, 384)])
+def test_linear_bwd_layer_norm_bwd_without_prior_and_bias(device, M, N, K):
+    # dx_accumulate = 0 (dh is written, whatever it held) and db = NULL, in the one launch and in
+    # the separate-kernels form.
+    dtype = BF16
+    lib, st = device.lib, device.stream
+    h = round_to_dtype(normal(82, 0, (M, K), std=2.0), dtype)
+    gamma = round_to_dtype(uniform(82, 1, (K,), 0.5, 1.5), dtype)
+    w = round_to_dtype(normal(82, 3, (N, K), std=0.1), dtype)
+    dy = round_to_dtype(normal(82, 4, (M, N), std=0.5), dtype)
+    bh, bg, bw, bdy = (AnyBuffer.from_numpy(device, a, dtype) for a in (h, gamma, w, dy))
+    new = lambda n, dt=dtype: AnyBuffer.create(dt, device, n)  # noqa: E731
+    x, mean, rstd = new(M * K), new(M, F32), new(M, F32)
+    lib.mg_layer_norm_fwd_stats(_ptr(bh), _ptr(bg), _ptr(bg), _ptr(x), _ptr(mean), _ptr(rstd), M, K, 1e-5, dtype, st)
+    t, dh_ref, dw_ref, dg_ref, dbt_ref = new(M * K), new(M * K), new(N * K), new(K), new(K)
+    lib.mg_linear_bwd(_ptr(bdy), _ptr(x), _ptr(bw), _ptr(t), _ptr(dw_ref), None, M, N, K, dtype, st)
+    lib.mg_layer_norm_bwd_stats(_ptr(t), _ptr(bh), _ptr(bg), _ptr(mean), _ptr(rstd), _ptr(dh_ref), _ptr(dg_ref),
+                                _ptr(dbt_ref), M, K, dtype, st)
+    dh = AnyBuffer.create(dtype, device, M * K, fill=123.0)  # must be overwritten, not added to
+    dw, dg, dbt = new(N * K), new(K), new(K)
+    lib.mg_linear_bwd_layer_norm_bwd(_ptr(bdy), _ptr(x), _ptr(bw), _ptr(bh), _ptr(bg), _ptr(mean), _ptr(rstd), _ptr(dh),
+                                     _ptr(dw), None, _ptr(dg), _ptr(dbt), M, N, K, 0, dtype, dtype, None, st)
+    np.testing.assert_array_equal(dw.to_numpy(), dw_ref.to_numpy())
+    got, ref = dh.to_numpy().astype(np.float64), dh_ref.to_numpy().astype(np.float64)
+    assert np.all(np.abs(got - ref) <= 2.0 ** -6 * np.abs(ref) + 1e-5 * np.abs(ref).max()) and np.mean(got == ref) > 0.98
+    for g_, r_ in ((dg, dg_ref), (dbt, dbt_ref)):
+        gv, rv = g_.to_numpy().astype(np.float64), r_.to_numpy().astype(np.float64)
+        assert np.all(np.abs(gv - rv) <= 2.0 ** -6 * np.abs(rv) + 1e-3 * np.abs(rv).max())
+    with pytest.raises(MogradError):  # dgamma is not optional
+        lib.mg_linear_bwd_layer_norm_bwd(_ptr(bdy), _ptr(x), _ptr(bw), _ptr(bh), _ptr(bg), _ptr(mean), _ptr(rstd), _ptr(dh),
+                                         _ptr(dw), None, None, _ptr(dbt), M, N, K, 0, dtype, dtype, None, st)
+    with pytest.raises(MogradError):  # without a list the gradients have the tensors' type
+        lib.mg_linear_bwd_layer_norm_bwd(_ptr(bdy), _ptr(x), _ptr(bw), _ptr(bh), _ptr(bg), _ptr(mean), _ptr(rstd), _ptr(dh),
+                                         _ptr(dw), None, _ptr(dg), _ptr(dbt), M, N, K, 0, dtype, F32, None, st)
+
+
 def test_fused_entry_errors(device):
     buf = AnyBuffer.create(F32, device, 16)
     p = buf.data_ptr()
