@@ -328,14 +328,17 @@ __global__ __launch_bounds__(256) void scatter_ranges_kernel(const I* __restrict
   }
 }
 
+// One count for every instantiation below: a tag must differ from those of all earlier launches
+// that may have used the same pool block.
+static std::atomic<uint32_t> g_range_launches{0};
+
 template <typename T, typename I, int VEC>
 static int scatter_ranges(const I* indices, const T* values, T* dst, int64_t n_idx, int64_t num_rows, int64_t row_size,
                           int rows_per_wave, int64_t quarter, hipStream_t s) {
   const int64_t ranges = ceil_div(num_rows, 4 * rows_per_wave), col_blocks = ceil_div(row_size, 64 * VEC);
-  static std::atomic<uint32_t> launches{0};
-  const uint32_t tag = ++launches;
+  const uint32_t tag = ++g_range_launches;
   // as many areas as workgroups can need, within 64 MiB
-  int64_t slots = std::min(col_blocks * (n_idx / (kRangeCap + 1) + 1) + 8, std::max<int64_t>(8, (int64_t{4} << 20) / quarter));
+  int64_t slots = std::min(col_blocks * (n_idx / (kRangeCap + 1) + 1) + 8, std::max<int64_t>(1, (int64_t{4} << 20) / quarter));
   const int slots_knob = env_int("MOGRAD_HIP_SCATTER_SPILL_SLOTS", -1);  // tests: 0 = no areas
   if (slots_knob >= 0) slots = slots_knob;
   Scratch spill;

@@ -754,6 +754,25 @@ def test_linear_bwd_layer_norm_bwd_without_prior_and_bias(device, M, N, K):
                                          _ptr(dw), None, _ptr(dg), _ptr(dbt), M, N, K, 0, dtype, F32, None, st)
 
 
+@pytest.mark.parametrize("M,N,acc", [(0, 64, 1), (128, 0, 1), (128, 0, 0)])
+def test_linear_bwd_layer_norm_bwd_empty_sides(device, M, N, acc):
+    # No rows: every sum is zero and dh is left alone.  No output features: dY W is zero, so dh
+    # keeps its prior (or becomes zero), and the LayerNorm's sums are zero.
+    dtype, K = BF16, 384
+    lib, st = device.lib, device.stream
+    new = lambda n, fill, dt=dtype: AnyBuffer.create(dt, device, max(n, 1), fill=fill)  # noqa: E731
+    dy, x, w, h, g = new(M * N, 0.5), new(M * K, 0.25), new(N * K, 0.125), new(M * K, 1.0), new(K, 1.0)
+    mean, rstd = new(M, 0.0, F32), new(M, 1.0, F32)
+    dh, dw, db, dg, dbt = new(M * K, 3.0), new(N * K, 7.0), new(N, 7.0), new(K, 7.0), new(K, 7.0)
+    lib.mg_linear_bwd_layer_norm_bwd(_ptr(dy), _ptr(x), _ptr(w), _ptr(h), _ptr(g), _ptr(mean), _ptr(rstd), _ptr(dh),
+                                     _ptr(dw), _ptr(db), _ptr(dg), _ptr(dbt), M, N, K, acc, dtype, dtype, None, st)
+    assert np.all(dg.to_numpy() == 0) and np.all(dbt.to_numpy() == 0)
+    if M:
+        assert np.all(dh.to_numpy() == (3.0 if acc else 0.0))
+    if N:
+        assert np.all(dw.to_numpy() == 0) and np.all(db.to_numpy() == 0)
+
+
 def test_fused_entry_errors(device):
     buf = AnyBuffer.create(F32, device, 16)
     p = buf.data_ptr()
