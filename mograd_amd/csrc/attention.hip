@@ -148,8 +148,8 @@ static int flash_attn_fwd_impl(int o_bshd, int64_t ld, const void* q, const void
   const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D),
                        o_bshd,              ld ? ld : H * D};
   hipStream_t s = mg::to_stream(stream);
-  const void* ptrs[] = {q, k, v, o, has_bias ? mask : nullptr};
-  if (mg::attn_mfma_supported(dtype, D, ptrs, 5))
+  const void* ptrs[] = {q, k, v, o};  // the bias may start at any element
+  if (mg::attn_mfma_supported(dtype, D, ptrs, 4))
     return mg::attn_fwd_mfma(q, k, v, mask, o, lse, a, scale, causal != 0, has_bias != 0, dtype, s);
   switch (dtype) {
     case MG_F32: return mg::fwd_generic<float>(q, k, v, mask, o, lse, a, scale, causal != 0, has_bias != 0, s);
@@ -168,8 +168,8 @@ static int flash_attn_bwd_impl(int o_bshd, int64_t ld, const void* d_o, const vo
   const mg::AttnDims a{static_cast<int>(B), static_cast<int>(S), static_cast<int>(H), static_cast<int>(D),
                        o_bshd,              ld ? ld : H * D};
   hipStream_t s = mg::to_stream(stream);
-  const void* ptrs[] = {d_o, o, q, k, v, dq, dk, dv, has_bias ? mask : nullptr};
-  if (mg::attn_mfma_supported(dtype, D, ptrs, 9))
+  const void* ptrs[] = {d_o, o, q, k, v, dq, dk, dv};  // the bias may start at any element
+  if (mg::attn_mfma_supported(dtype, D, ptrs, 8))
     return mg::attn_bwd_mfma(d_o, o, q, k, v, mask, lse, dq, dk, dv, a, scale, causal != 0, has_bias != 0, dtype, s);
   switch (dtype) {
     case MG_F32:

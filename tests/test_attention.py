@@ -20,23 +20,26 @@ from mograd_amd import runtime as R  # noqa: E402
 from mograd_amd.runtime import round_to_dtype  # noqa: E402
 
 
-def _fwd(device, q, k, v, mask, causal, scale, dtype):
+def _fwd(device, q, k, v, mask, causal, scale, dtype, mask_offset=0):
     B, S, H, D = q.shape
     attrs = {"scale": scale, "is_causal": causal, "has_bias": mask is not None}
     m = mask if mask is not None else np.zeros(8, np.float32)  # placeholder the kernels never read
     srcs = [Node.leaf(Layout(B, S, H, D), dtype)] * 3 + [Node.leaf(Layout(*m.shape), dtype)]
     node = Node("FLASH_ATTN", Layout(B, H, S, D), dtype, srcs, attrs)
     bufs = [AnyBuffer.from_numpy(device, a, dtype) for a in (q, k, v, m)]
+    if mask_offset:  # the same bias, `mask_offset` elements into a larger allocation
+        padded = np.concatenate([np.zeros(mask_offset, m.dtype), m.ravel()])
+        bufs[3] = AnyBuffer.from_numpy(device, padded, dtype).view(Layout(m.size, base_offset=mask_offset))
     o, lse = R.run(node, bufs, device)
     return o, lse, bufs
 
 
-def _fwd_bwd(device, q, k, v, do, mask=None, causal=False, scale=None, dtype=F32):
+def _fwd_bwd(device, q, k, v, do, mask=None, causal=False, scale=None, dtype=F32, mask_offset=0):
     """Forward for O/LSE chained into the backward, as the reference's run_bwd does
     (tests/kernels/attention/harness.mojo:266-344)."""
     B, S, H, D = q.shape
     scale = scale if scale is not None else 1.0 / math.sqrt(D)
-    o, lse, (bq, bk, bv, bm) = _fwd(device, q, k, v, mask, causal, scale, dtype)
+    o, lse, (bq, bk, bv, bm) = _fwd(device, q, k, v, mask, causal, scale, dtype, mask_offset)
     attrs = {"scale": scale, "is_causal": causal, "has_bias": mask is not None}
     leaf = Node.leaf(Layout(B, S, H, D), dtype)
     srcs = [Node.leaf(Layout(B, H, S, D), dtype), Node.leaf(Layout(B, H, S, D), dtype), leaf, leaf, leaf,
@@ -193,6 +196,20 @@ def test_closed_forms(device):
     o, lse, *_ = _fwd_bwd(device, z, z, v, np.ones((B, H, S, D), np.float32), None, False)
     np.testing.assert_allclose(o[0, 0], np.repeat(v[0, :, 0].mean(axis=0)[None], S, axis=0), atol=1e-6)
     np.testing.assert_allclose(lse, math.log(S), rtol=1e-6)
+
+
+@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("S", [96, 200])
+def test_bias_at_any_alignment(device, D, S):
+    # A bias whose rows are whole 8-byte groups is read a group at a time; one that starts at an
+    # odd element of its allocation (or has S % 4 != 0, which the shapes above cover) is read element
+    # by element into the same form.  The results must be the same bits.
+    q, k, v, do, m = _inputs(59, 1, S, 2, D, BF16, True)
+    aligned = _fwd_bwd(device, q, k, v, do, m, False, dtype=BF16)
+    for offset in (1, 2, 3):
+        shifted = _fwd_bwd(device, q, k, v, do, m, False, dtype=BF16, mask_offset=offset)
+        for a, b_, what in zip(aligned, shifted, ("o", "lse", "dq", "dk", "dv")):
+            np.testing.assert_array_equal(a, b_, err_msg=f"{what} at offset {offset}")
 
 
 def test_bias_shift_invariance(device):
