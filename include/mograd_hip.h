@@ -341,6 +341,26 @@ int mg_cast(const void* a, void* dst, int64_t n, int in_dtype, int out_dtype, mg
 int mg_contiguous(const void* a, void* dst, int rank, const int64_t* shape, const int64_t* strides,
                   int dtype, mg_stream stream);
 
+/* The four maps above over strided views: the operands are views of dst's shape (host arrays
+ * of `rank` <= 8 extents) with their own element strides, >= 0, 0 along a broadcast axis, base
+ * offsets already applied to the pointers; dst is row-major, contiguous, and overlaps neither
+ * operand.  Any alignment; views whose innermost axis is contiguous (or constant) and whose
+ * rows start on 16-byte boundaries are read 16 bytes at a time, others element by element.
+ * The values equal mg_contiguous of each operand followed by the contiguous entry, without
+ * the copy (a broadcast bias is never written out).
+ * Replace mograd_add_strided (kernels/__init__.mojo:474-487), mograd_relu (:274-286),
+ * mograd_relu_grad (:546-560) and mograd_cast (:304-335) for non-contiguous layouts
+ * (kernels/strided.mojo:54-114, kernels/elementwise.mojo:75-90). */
+int mg_add_strided(const void* a, const void* b, void* dst, int rank, const int64_t* shape,
+                   const int64_t* strides_a, const int64_t* strides_b, int dtype, mg_stream stream);
+int mg_relu_strided(const void* a, void* dst, int rank, const int64_t* shape, const int64_t* strides,
+                    int dtype, mg_stream stream);
+int mg_relu_grad_strided(const void* out, const void* upstream, void* dst, int rank,
+                         const int64_t* shape, const int64_t* strides_out,
+                         const int64_t* strides_upstream, int dtype, mg_stream stream);
+int mg_cast_strided(const void* a, void* dst, int rank, const int64_t* shape, const int64_t* strides,
+                    int in_dtype, int out_dtype, mg_stream stream);
+
 /* dst(i, :) = src(indices[i], :), i < n_idx; src is (num_rows, row_size) with the given
  * element strides, dst and indices contiguous, idx_dtype MG_I32 or MG_I64 (the reference
  * takes int64 only).  An index outside [0, num_rows) yields a row of zeros (the reference
@@ -366,6 +386,13 @@ int mg_scatter_add(const void* indices, const void* values, void* dst, int64_t n
 /* y = softmax over the last axis of (rows, cols).  Replaces mograd_softmax for a
  * contiguous source, kernels/__init__.mojo:1015-1030 (kernels/softmax.mojo:19-38). */
 int mg_softmax(const void* x, void* y, int64_t rows, int64_t cols, int dtype, mg_stream stream);
+
+/* Row softmax over the last axis of a strided view (`rank` >= 1 extents and element strides
+ * >= 0, base offset applied to `x`); y is row-major, contiguous.  Same arithmetic as mg_softmax;
+ * rows that are contiguous and start on 16-byte boundaries are read 16 bytes at a time.
+ * Replaces mograd_softmax_strided, kernels/__init__.mojo:1033-1060 (kernels/softmax.mojo:40-68). */
+int mg_softmax_strided(const void* x, void* y, int rank, const int64_t* shape, const int64_t* strides,
+                       int dtype, mg_stream stream);
 
 /* dst = y * (upstream - sum over the row of y * upstream).  Replaces mograd_softmax_grad,
  * kernels/__init__.mojo:1062-1090 (kernels/softmax.mojo:76-98). */

@@ -107,6 +107,11 @@ PROTOTYPES = {
     "mg_relu": (_i, [_p, _p, _l, _i, _p], True),
     "mg_cast": (_i, [_p, _p, _l, _i, _i, _p], True),
     "mg_contiguous": (_i, [_p, _p, _i, _pl, _pl, _i, _p], True),
+    "mg_add_strided": (_i, [_p, _p, _p, _i, _pl, _pl, _pl, _i, _p], True),
+    "mg_relu_strided": (_i, [_p, _p, _i, _pl, _pl, _i, _p], True),
+    "mg_relu_grad_strided": (_i, [_p, _p, _p, _i, _pl, _pl, _pl, _i, _p], True),
+    "mg_cast_strided": (_i, [_p, _p, _i, _pl, _pl, _i, _i, _p], True),
+    "mg_softmax_strided": (_i, [_p, _p, _i, _pl, _pl, _i, _p], True),
     "mg_gather": (_i, [_p, _p, _p, _l, _l, _l, _l, _l, _i, _i, _p], True),
     "mg_scatter_add": (_i, [_p, _p, _p, _l, _l, _l, _i, _i, _p], True),
     "mg_deferred_create": (_i, [C.POINTER(_p)], True),

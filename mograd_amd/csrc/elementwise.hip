@@ -1,6 +1,7 @@
 // Elementwise maps of the training step around the backward kernels: residual and gradient
-// adds, relu, dtype casts, and the copy that makes a strided view contiguous.  All are
-// HBM-bound streaming kernels with 16-byte accesses.
+// adds, relu, dtype casts, and the copy that makes a strided view contiguous, plus the same
+// maps over strided (transposed, sliced, broadcast) views.  All are HBM-bound streaming kernels
+// with 16-byte accesses where the views allow them.
 #include "mg_device.h"
 #include "mg_internal.h"
 
@@ -99,6 +100,99 @@ __global__ __launch_bounds__(256) void contiguous_kernel(const V* __restrict__ s
     }
     off += rem * static_cast<Index>(v.stride[0]);
     dst[flat] = src[off];
+  }
+}
+
+// ---- the same maps over strided views -----------------------------------------------------
+// dst (row-major) = op(a[view a], b[view b]): both operands are views of dst's shape with their
+// own element strides (0 along a broadcast axis).  A thread takes VEC consecutive elements of
+// the innermost axis; an operand whose innermost stride is 1 is read with 16-byte loads, one
+// whose innermost stride is 0 is read once and repeated; VEC = 1 serves every other view
+// element by element.  `shape` holds the innermost extent in units of VEC, `sa`/`sb` the
+// innermost strides times VEC.
+enum MapOp { kMapAdd = 0, kMapRelu = 1, kMapReluGrad = 2, kMapCast = 3 };
+
+struct MapView {
+  int rank;
+  int64_t shape[kMaxRank];
+  int64_t sa[kMaxRank];
+  int64_t sb[kMaxRank];
+};
+
+// Elements per thread of the wide form: one 16-byte access on each side, two on the fp32 side
+// of a cast to or from 16 bits.
+template <typename S, typename D>
+struct MapWide {
+  static constexpr int value = sizeof(S) == 4 && sizeof(D) == 4 ? 4 : 8;
+};
+
+template <typename T, int VEC>
+__device__ __forceinline__ void map_load(const T* __restrict__ p, bool unit, float (&v)[VEC]) {
+  if constexpr (VEC == 1) {
+    v[0] = to_float(*p);
+  } else if (unit) {
+    if constexpr (sizeof(T) == 4 && VEC == 8) {
+      float lo[4], hi[4];
+      VecIO<T, 4>::load(p, lo);
+      VecIO<T, 4>::load(p + 4, hi);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[e] = lo[e];
+        v[4 + e] = hi[e];
+      }
+    } else {
+      VecIO<T, VEC>::load(p, v);
+    }
+  } else {
+    const float x = to_float(*p);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) v[e] = x;
+  }
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void map_store(T* __restrict__ p, const float (&v)[VEC]) {
+  if constexpr (VEC == 1) {
+    *p = from_float<T>(v[0]);
+  } else if constexpr (sizeof(T) == 4 && VEC == 8) {
+    const float lo[4] = {v[0], v[1], v[2], v[3]};
+    const float hi[4] = {v[4], v[5], v[6], v[7]};
+    VecIO<T, 4>::store(p, lo);
+    VecIO<T, 4>::store(p + 4, hi);
+  } else {
+    VecIO<T, VEC>::store(p, v);
+  }
+}
+
+template <typename S, typename D, int OP, int VEC, typename Index>
+__global__ __launch_bounds__(256) void map_strided_kernel(const S* __restrict__ a, const S* __restrict__ b,
+                                                          D* __restrict__ dst, MapView v, int64_t n, bool a_unit,
+                                                          bool b_unit) {
+  constexpr bool kBinary = OP == kMapAdd || OP == kMapReluGrad;
+  const int64_t step = static_cast<int64_t>(gridDim.x) * 256;
+  for (int64_t flat = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; flat < n; flat += step) {
+    Index rem = static_cast<Index>(flat);
+    Index off_a = 0, off_b = 0;
+    for (int d = v.rank - 1; d > 0; --d) {
+      const Index extent = static_cast<Index>(v.shape[d]);
+      const Index q = rem / extent;
+      const Index idx = rem - q * extent;
+      off_a += idx * static_cast<Index>(v.sa[d]);
+      if constexpr (kBinary) off_b += idx * static_cast<Index>(v.sb[d]);
+      rem = q;
+    }
+    off_a += rem * static_cast<Index>(v.sa[0]);
+    if constexpr (kBinary) off_b += rem * static_cast<Index>(v.sb[0]);
+    float x[VEC], y[VEC];
+    map_load<S, VEC>(a + off_a, a_unit, x);
+    if constexpr (kBinary) map_load<S, VEC>(b + off_b, b_unit, y);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      if constexpr (OP == kMapAdd) x[e] += y[e];
+      else if constexpr (OP == kMapRelu) x[e] = x[e] > 0.f ? x[e] : 0.f;
+      else if constexpr (OP == kMapReluGrad) x[e] = x[e] > 0.f ? y[e] : 0.f;
+    }
+    map_store<D, VEC>(dst + flat * VEC, x);
   }
 }
 
@@ -221,6 +315,125 @@ static int contiguous_dispatch(const void* src, void* dst, int rank, const int64
   }
 }
 
+template <typename S, typename D, int OP>
+static int map_strided_typed(const void* a, const void* b, void* dst, const MapView& v, int64_t n, int vec, bool narrow,
+                             bool a_unit, bool b_unit, hipStream_t s) {
+  const dim3 grid(stream_blocks(n, 1));
+  const S* pa = static_cast<const S*>(a);
+  const S* pb = static_cast<const S*>(b);
+  D* pd = static_cast<D*>(dst);
+#define MG_MAP_LAUNCH(VEC_, INDEX_) \
+  hipLaunchKernelGGL((map_strided_kernel<S, D, OP, VEC_, INDEX_>), grid, dim3(256), 0, s, pa, pb, pd, v, n, a_unit, b_unit)
+  if (vec > 1) {
+    constexpr int kWide = MapWide<S, D>::value;
+    if (narrow) MG_MAP_LAUNCH(kWide, uint32_t);
+    else MG_MAP_LAUNCH(kWide, int64_t);
+  } else {
+    if (narrow) MG_MAP_LAUNCH(1, uint32_t);
+    else MG_MAP_LAUNCH(1, int64_t);
+  }
+#undef MG_MAP_LAUNCH
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+template <int OP>
+static int map_strided_dtypes(const void* a, const void* b, void* dst, const MapView& v, int64_t n, int vec, bool narrow,
+                              bool a_unit, bool b_unit, int in_dtype, int out_dtype, hipStream_t s) {
+#define MG_MAP_TYPED(S_, D_) return map_strided_typed<S_, D_, OP>(a, b, dst, v, n, vec, narrow, a_unit, b_unit, s)
+  if constexpr (OP == kMapCast) {
+    if (in_dtype == MG_F32) {
+      if (out_dtype == MG_F32) MG_MAP_TYPED(float, float);
+      if (out_dtype == MG_F16) MG_MAP_TYPED(float, f16_t);
+      MG_MAP_TYPED(float, bf16_t);
+    }
+    if (in_dtype == MG_F16) {
+      if (out_dtype == MG_F32) MG_MAP_TYPED(f16_t, float);
+      if (out_dtype == MG_F16) MG_MAP_TYPED(f16_t, f16_t);
+      MG_MAP_TYPED(f16_t, bf16_t);
+    }
+    if (out_dtype == MG_F32) MG_MAP_TYPED(bf16_t, float);
+    if (out_dtype == MG_F16) MG_MAP_TYPED(bf16_t, f16_t);
+    MG_MAP_TYPED(bf16_t, bf16_t);
+  } else {
+    if (in_dtype == MG_F32) MG_MAP_TYPED(float, float);
+    if (in_dtype == MG_F16) MG_MAP_TYPED(f16_t, f16_t);
+    MG_MAP_TYPED(bf16_t, bf16_t);
+  }
+#undef MG_MAP_TYPED
+}
+
+// Checks the views, drops unit dims, merges neighbours that are contiguous with each other in
+// both operands, picks 4 or 8 elements per thread where every operand allows it, and launches.
+template <int OP>
+static int map_strided_dispatch(const char* who, const void* a, const void* b, void* dst, int rank, const int64_t* shape,
+                                const int64_t* strides_a, const int64_t* strides_b, int in_dtype, int out_dtype,
+                                hipStream_t s) {
+  constexpr bool kBinary = OP == kMapAdd || OP == kMapReluGrad;
+  if (!is_float_dtype(in_dtype) || !is_float_dtype(out_dtype))
+    return fail(MG_ERR_INVALID, "%s: unsupported dtype %s", who, dtype_name(is_float_dtype(in_dtype) ? out_dtype : in_dtype));
+  if (rank < 0 || rank > kMaxRank) return fail(MG_ERR_INVALID, "%s: rank %d outside 0..%d", who, rank, kMaxRank);
+  if (rank > 0 && (!shape || !strides_a || (kBinary && !strides_b)))
+    return fail(MG_ERR_INVALID, "%s: null shape or strides", who);
+  int64_t n = 1;
+  for (int d = 0; d < rank; ++d) {
+    if (shape[d] < 0 || strides_a[d] < 0 || (kBinary && strides_b[d] < 0))
+      return fail(MG_ERR_INVALID, "%s: negative extent or stride at dim %d", who, d);
+    n *= shape[d];
+  }
+  if (n == 0) return MG_OK;
+  if (!a || (kBinary && !b) || !dst) return fail(MG_ERR_INVALID, "%s: null pointer argument", who);
+  int64_t sh[kMaxRank], sa[kMaxRank], sb[kMaxRank];
+  int r = 0;
+  for (int d = 0; d < rank; ++d) {
+    if (shape[d] == 1) continue;
+    const int64_t tb = kBinary ? strides_b[d] : 0;
+    if (r > 0 && sa[r - 1] == shape[d] * strides_a[d] && sb[r - 1] == shape[d] * tb) {
+      sh[r - 1] *= shape[d];
+      sa[r - 1] = strides_a[d];
+      sb[r - 1] = tb;
+    } else {
+      sh[r] = shape[d];
+      sa[r] = strides_a[d];
+      sb[r] = tb;
+      ++r;
+    }
+  }
+  if (r == 0) {
+    sh[0] = 1;
+    sa[0] = sb[0] = 1;
+    r = 1;
+  }
+  // A group per thread: the innermost extent in whole groups, dst and every unit-stride operand
+  // on 16-byte boundaries at every group (base pointer and outer strides), any other operand
+  // constant along the innermost axis.
+  const int in_size = dtype_size(in_dtype);
+  auto wide_operand = [&](const void* p, const int64_t* st) {
+    if (st[r - 1] == 0) return true;
+    if (st[r - 1] != 1 || !aligned16(p)) return false;
+    for (int d = 0; d + 1 < r; ++d)
+      if (st[d] * in_size % 16 != 0) return false;
+    return true;
+  };
+  const int group = dtype_size(in_dtype) == 4 && dtype_size(out_dtype) == 4 ? 4 : 8;  // MapWide
+  const bool wide = sh[r - 1] % group == 0 && aligned16(dst) && wide_operand(a, sa) && (!kBinary || wide_operand(b, sb));
+  const int vec = wide ? group : 1;
+  MapView v;
+  v.rank = r;
+  int64_t max_a = 0, max_b = 0;
+  for (int d = 0; d < r; ++d) {
+    const bool inner = d == r - 1;
+    v.shape[d] = inner ? sh[d] / vec : sh[d];
+    v.sa[d] = inner ? sa[d] * vec : sa[d];
+    v.sb[d] = inner ? sb[d] * vec : sb[d];
+    max_a += (v.shape[d] - 1) * v.sa[d];
+    max_b += (v.shape[d] - 1) * v.sb[d];
+  }
+  const int64_t chunks = n / vec;
+  const bool narrow = n < (int64_t{1} << 31) && max_a < (int64_t{1} << 31) && max_b < (int64_t{1} << 31);
+  return map_strided_dtypes<OP>(a, b, dst, v, chunks, vec, narrow, sa[r - 1] == 1, sb[r - 1] == 1, in_dtype, out_dtype, s);
+}
+
 }  // namespace mg
 
 extern "C" {
@@ -277,6 +490,30 @@ int mg_cast(const void* a, void* dst, int64_t n, int in_dtype, int out_dtype, mg
 int mg_contiguous(const void* a, void* dst, int rank, const int64_t* shape, const int64_t* strides, int dtype,
                   mg_stream stream) {
   return mg::contiguous_dispatch(a, dst, rank, shape, strides, dtype, mg::to_stream(stream));
+}
+
+int mg_add_strided(const void* a, const void* b, void* dst, int rank, const int64_t* shape, const int64_t* strides_a,
+                   const int64_t* strides_b, int dtype, mg_stream stream) {
+  return mg::map_strided_dispatch<mg::kMapAdd>("add_strided", a, b, dst, rank, shape, strides_a, strides_b, dtype, dtype,
+                                               mg::to_stream(stream));
+}
+
+int mg_relu_strided(const void* a, void* dst, int rank, const int64_t* shape, const int64_t* strides, int dtype,
+                    mg_stream stream) {
+  return mg::map_strided_dispatch<mg::kMapRelu>("relu_strided", a, nullptr, dst, rank, shape, strides, nullptr, dtype, dtype,
+                                                mg::to_stream(stream));
+}
+
+int mg_relu_grad_strided(const void* out, const void* upstream, void* dst, int rank, const int64_t* shape,
+                         const int64_t* strides_out, const int64_t* strides_upstream, int dtype, mg_stream stream) {
+  return mg::map_strided_dispatch<mg::kMapReluGrad>("relu_grad_strided", out, upstream, dst, rank, shape, strides_out,
+                                                    strides_upstream, dtype, dtype, mg::to_stream(stream));
+}
+
+int mg_cast_strided(const void* a, void* dst, int rank, const int64_t* shape, const int64_t* strides, int in_dtype,
+                    int out_dtype, mg_stream stream) {
+  return mg::map_strided_dispatch<mg::kMapCast>("cast_strided", a, nullptr, dst, rank, shape, strides, nullptr, in_dtype,
+                                                out_dtype, mg::to_stream(stream));
 }
 
 }  // extern "C"

@@ -10,18 +10,14 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 // y = exp(x - max) / sum exp(x - max).  Pass 1: running maximum and rescaled sum in one
 // sweep; pass 2 re-reads the row (it is still in cache) and writes the result.
+// One wave, one row.  `xs`: elements between neighbours of the input row (1 whenever VEC > 1).
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void softmax_rows_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows,
-                                                           int64_t cols) {
-  const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
-  if (row >= rows) return;  // wave-uniform
-  const int lane = threadIdx.x % kWave;
-  const T* xr = x + row * cols;
-  T* yr = y + row * cols;
+__device__ __forceinline__ void softmax_row(const T* __restrict__ xr, int64_t xs, T* __restrict__ yr, int64_t cols,
+                                            int lane) {
   float m = -INFINITY, l = 0.f;
   for (int64_t c = static_cast<int64_t>(lane) * VEC; c < cols; c += kWave * VEC) {
     float v[VEC];
-    VecIO<T, VEC>::load(xr + c, v);
+    VecIO<T, VEC>::load(xr + c * xs, v);
     float cm = v[0];
 #pragma unroll
     for (int e = 1; e < VEC; ++e) cm = fmaxf(cm, v[e]);
@@ -39,11 +35,35 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const T* __restrict__
   const float inv = 1.0f / wave_sum(l);
   for (int64_t c = static_cast<int64_t>(lane) * VEC; c < cols; c += kWave * VEC) {
     float v[VEC];
-    VecIO<T, VEC>::load(xr + c, v);
+    VecIO<T, VEC>::load(xr + c * xs, v);
 #pragma unroll
     for (int e = 0; e < VEC; ++e) v[e] = __builtin_amdgcn_exp2f((v[e] - gm) * kLog2e) * inv;
     VecIO<T, VEC>::store(yr + c, v);
   }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void softmax_rows_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows,
+                                                           int64_t cols) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+  if (row >= rows) return;  // wave-uniform
+  softmax_row<T, VEC>(x + row * cols, 1, y + row * cols, cols, threadIdx.x % kWave);
+}
+
+// The rows of a strided view: `v` holds the extents and strides of the dims in front of the
+// last one, `xs` the stride of the last.  The result is row-major.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void softmax_view_kernel(const T* __restrict__ x, T* __restrict__ y, StridedView v, int64_t xs,
+                                                           int64_t rows, int64_t cols) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+  if (row >= rows) return;  // wave-uniform
+  int64_t rem = row, off = 0;
+  for (int d = v.rank - 1; d >= 0; --d) {
+    const int64_t q = rem / v.shape[d];
+    off += (rem - q * v.shape[d]) * v.stride[d];
+    rem = q;
+  }
+  softmax_row<T, VEC>(x + off, xs, y + row * cols, cols, threadIdx.x % kWave);
 }
 
 // dst = y * (upstream - sum_c y * upstream)
@@ -139,6 +159,21 @@ static int softmax_typed(const void* x, void* y, int64_t rows, int64_t cols, hip
 }
 
 template <typename T>
+static int softmax_view_typed(const void* x, void* y, const StridedView& v, int64_t xs, int64_t rows, int64_t cols, bool wide,
+                              hipStream_t s) {
+  constexpr int WIDE = WideVec<T>::value;
+  const dim3 grid(static_cast<unsigned>(ceil_div(rows, 4)));
+  if (wide && cols % WIDE == 0)
+    hipLaunchKernelGGL((softmax_view_kernel<T, WIDE>), grid, dim3(256), 0, s, static_cast<const T*>(x), static_cast<T*>(y),
+                       v, xs, rows, cols);
+  else
+    hipLaunchKernelGGL((softmax_view_kernel<T, 1>), grid, dim3(256), 0, s, static_cast<const T*>(x), static_cast<T*>(y), v,
+                       xs, rows, cols);
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
+template <typename T>
 static int softmax_grad_typed(const void* y, const void* up, void* dst, int64_t rows, int64_t cols, hipStream_t s) {
   constexpr int WIDE = WideVec<T>::value;
   const dim3 grid(static_cast<unsigned>(ceil_div(rows, 4)));
@@ -184,6 +219,37 @@ int mg_softmax(const void* x, void* y, int64_t rows, int64_t cols, int dtype, mg
     case MG_F32: return mg::softmax_typed<float>(x, y, rows, cols, s);
     case MG_F16: return mg::softmax_typed<mg::f16_t>(x, y, rows, cols, s);
     default: return mg::softmax_typed<mg::bf16_t>(x, y, rows, cols, s);
+  }
+}
+
+int mg_softmax_strided(const void* x, void* y, int rank, const int64_t* shape, const int64_t* strides, int dtype,
+                       mg_stream stream) {
+  if (rank < 1 || rank > mg::kMaxRank) return mg::fail(MG_ERR_INVALID, "softmax_strided: rank %d outside 1..%d", rank, mg::kMaxRank);
+  if (!shape || !strides) return mg::fail(MG_ERR_INVALID, "softmax_strided: null shape or strides");
+  int64_t rows = 1;
+  mg::StridedView v;
+  v.rank = rank - 1;
+  for (int d = 0; d < rank; ++d) {
+    if (shape[d] < 0 || strides[d] < 0)
+      return mg::fail(MG_ERR_INVALID, "softmax_strided: negative extent or stride at dim %d", d);
+    if (d + 1 < rank) {
+      rows *= shape[d];
+      v.shape[d] = shape[d];
+      v.stride[d] = strides[d];
+    }
+  }
+  const int64_t cols = shape[rank - 1], xs = strides[rank - 1];
+  MG_TRY(mg::check_rows("softmax_strided", rows, cols, dtype));
+  if (rows == 0 || cols == 0) return MG_OK;
+  if (!x || !y) return mg::fail(MG_ERR_INVALID, "softmax_strided: null pointer argument");
+  // 16-byte loads where a row is contiguous and every row starts on a 16-byte boundary
+  bool wide = xs == 1 && mg::aligned16(x) && mg::aligned16(y);
+  for (int d = 0; d + 1 < rank && wide; ++d) wide = shape[d] == 1 || strides[d] * mg::dtype_size(dtype) % 16 == 0;
+  hipStream_t s = mg::to_stream(stream);
+  switch (dtype) {
+    case MG_F32: return mg::softmax_view_typed<float>(x, y, v, xs, rows, cols, wide, s);
+    case MG_F16: return mg::softmax_view_typed<mg::f16_t>(x, y, v, xs, rows, cols, wide, s);
+    default: return mg::softmax_view_typed<mg::bf16_t>(x, y, v, xs, rows, cols, wide, s);
   }
 }
 

@@ -294,8 +294,17 @@ inline void require_float(DType d, const char* who) {  // dispatch_dtype[float_o
 }
 
 // The first `count` operands as contiguous buffers.  The reference reads strided views
-// element by element inside each kernel (kernels/strided.mojo); here a strided operand is
-// first copied row-major with mg_contiguous and the contiguous kernel runs on the copy.
+// element by element inside each kernel (kernels/strided.mojo).  add, relu, relu_grad, cast and
+// softmax have strided entries of their own; for the kernels that use this helper a strided operand
+// is first copied row-major with mg_contiguous and the contiguous kernel runs on the copy.
+// Whether the first `count` operands can take a flat kernel: contiguous, and starting on the
+// 16-byte boundary those kernels read from (a view into the middle of a buffer may not).
+inline bool flat(const OpRef& node, const Buffers& inputs, int count) {
+  for (int i = 0; i < count; ++i)
+    if (!node.src(i).layout().is_contiguous() || reinterpret_cast<uintptr_t>(inputs[i].data_ptr()) % 16 != 0) return false;
+  return true;
+}
+
 inline Buffers materialise(const OpRef& node, const Buffers& inputs, Device& device, int count) {
   Buffers out = inputs;
   for (int i = 0; i < count; ++i) {
@@ -484,37 +493,54 @@ inline Buffers sum(const OpRef& node, const Buffers& inputs, Device& device) {
 }
 
 // RELU_GRAD[relu_out, upstream].  runtime/__init__.mojo:351-352.
-inline Buffers relu_grad(const OpRef& node, const Buffers& inputs, Device& device) {
-  const Buffers in = detail::materialise(node, inputs, device, 2);
+inline Buffers relu_grad(const OpRef& node, const Buffers& in, Device& device) {
+  const Layout &la = node.src(0).layout(), &lb = node.src(1).layout();
   AnyBuffer out = AnyBuffer::create(node.dtype(), device, node.numel());
-  MOGRAD_CALL(device, mg_relu_grad, in[0].data_ptr(), in[1].data_ptr(), out.data_ptr(), node.numel(), node.dtype(),
-              device.stream());
+  if (detail::flat(node, in, 2))
+    MOGRAD_CALL(device, mg_relu_grad, in[0].data_ptr(), in[1].data_ptr(), out.data_ptr(), node.numel(), node.dtype(),
+                device.stream());
+  else
+    MOGRAD_CALL(device, mg_relu_grad_strided, in[0].data_ptr(), in[1].data_ptr(), out.data_ptr(), la.rank(),
+                la.shape().data(), la.stride().data(), lb.stride().data(), node.dtype(), device.stream());
   return {out};
 }
 
-// ADD[a, b] (residual connections, gradient accumulation).  runtime/__init__.mojo:319-333.
-inline Buffers add(const OpRef& node, const Buffers& inputs, Device& device) {
-  const Buffers in = detail::materialise(node, inputs, device, 2);
+// ADD[a, b] (residual connections, gradient accumulation, a broadcast bias).
+// runtime/__init__.mojo:319-333: contiguous operands take the flat kernel, views the strided one.
+inline Buffers add(const OpRef& node, const Buffers& in, Device& device) {
+  const Layout &la = node.src(0).layout(), &lb = node.src(1).layout();
   AnyBuffer out = AnyBuffer::create(node.dtype(), device, node.numel());
-  MOGRAD_CALL(device, mg_add, in[0].data_ptr(), in[1].data_ptr(), out.data_ptr(), node.numel(), node.dtype(),
-              device.stream());
+  if (detail::flat(node, in, 2))
+    MOGRAD_CALL(device, mg_add, in[0].data_ptr(), in[1].data_ptr(), out.data_ptr(), node.numel(), node.dtype(),
+                device.stream());
+  else
+    MOGRAD_CALL(device, mg_add_strided, in[0].data_ptr(), in[1].data_ptr(), out.data_ptr(), la.rank(), la.shape().data(),
+                la.stride().data(), lb.stride().data(), node.dtype(), device.stream());
   return {out};
 }
 
 // RELU[a].  runtime/__init__.mojo:296-297.
-inline Buffers relu(const OpRef& node, const Buffers& inputs, Device& device) {
-  const Buffers in = detail::materialise(node, inputs, device, 1);
+inline Buffers relu(const OpRef& node, const Buffers& in, Device& device) {
+  const Layout& l = node.src(0).layout();
   AnyBuffer out = AnyBuffer::create(node.dtype(), device, node.numel());
-  MOGRAD_CALL(device, mg_relu, in[0].data_ptr(), out.data_ptr(), node.numel(), node.dtype(), device.stream());
+  if (detail::flat(node, in, 1))
+    MOGRAD_CALL(device, mg_relu, in[0].data_ptr(), out.data_ptr(), node.numel(), node.dtype(), device.stream());
+  else
+    MOGRAD_CALL(device, mg_relu_strided, in[0].data_ptr(), out.data_ptr(), l.rank(), l.shape().data(), l.stride().data(),
+                node.dtype(), device.stream());
   return {out};
 }
 
 // CAST[a] to node.dtype().  runtime/__init__.mojo:300-311.
-inline Buffers cast(const OpRef& node, const Buffers& inputs, Device& device) {
-  const Buffers in = detail::materialise(node, inputs, device, 1);
+inline Buffers cast(const OpRef& node, const Buffers& in, Device& device) {
+  const Layout& l = node.src(0).layout();
   AnyBuffer out = AnyBuffer::create(node.dtype(), device, node.numel());
-  MOGRAD_CALL(device, mg_cast, in[0].data_ptr(), out.data_ptr(), node.numel(), node.src(0).dtype(), node.dtype(),
-              device.stream());
+  if (detail::flat(node, in, 1))
+    MOGRAD_CALL(device, mg_cast, in[0].data_ptr(), out.data_ptr(), node.numel(), node.src(0).dtype(), node.dtype(),
+                device.stream());
+  else
+    MOGRAD_CALL(device, mg_cast_strided, in[0].data_ptr(), out.data_ptr(), l.rank(), l.shape().data(), l.stride().data(),
+                node.src(0).dtype(), node.dtype(), device.stream());
   return {out};
 }
 
@@ -567,11 +593,15 @@ inline Buffers scatter_add(const OpRef& node, const Buffers& inputs, Device& dev
 // SOFTMAX[a] over the last axis.  kernels/__init__.mojo:1015-1030.
 inline Buffers softmax(const OpRef& node, const Buffers& inputs, Device& device) {
   const Layout& l = node.src(0).layout();
-  const Buffers in = detail::materialise(node, inputs, device, 1);
   detail::require_float(node.dtype(), "softmax");
-  const int64_t cols = l.shape(l.rank() - 1), rows = l.numel() / cols;
   AnyBuffer out = AnyBuffer::create(node.dtype(), device, node.numel());
-  MOGRAD_CALL(device, mg_softmax, in[0].data_ptr(), out.data_ptr(), rows, cols, node.dtype(), device.stream());
+  if (l.is_contiguous()) {
+    const int64_t cols = l.shape(l.rank() - 1), rows = cols ? l.numel() / cols : 0;
+    MOGRAD_CALL(device, mg_softmax, inputs[0].data_ptr(), out.data_ptr(), rows, cols, node.dtype(), device.stream());
+  } else {  // kernels/__init__.mojo:1033-1060: views go to the strided kernel
+    MOGRAD_CALL(device, mg_softmax_strided, inputs[0].data_ptr(), out.data_ptr(), l.rank(), l.shape().data(),
+                l.stride().data(), node.dtype(), device.stream());
+  }
   return {out};
 }
 

@@ -520,18 +520,25 @@ def sum(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
 
 def relu_grad(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     """RELU_GRAD[relu_out, upstream].  runtime/__init__.mojo:351-352."""
-    inputs = _materialise(node, inputs, device, 2)
     out = AnyBuffer.create(node.dtype(), device, node.numel())
-    device.lib.mg_relu_grad(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), node.numel(), node.dtype(),
-                            device.stream)
+    if _flat(node, inputs, 2):
+        device.lib.mg_relu_grad(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), node.numel(), node.dtype(),
+                                device.stream)
+    else:
+        la, lb = node.src(0).layout(), node.src(1).layout()
+        device.lib.mg_relu_grad_strided(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), la.rank(),
+                                        _i64_array(la.shape()), _i64_array(la.stride()), _i64_array(lb.stride()),
+                                        node.dtype(), device.stream)
     return [out]
 
 
 def _materialise(node: Node, inputs: List[AnyBuffer], device: Device, count: int) -> List[AnyBuffer]:
     """The first `count` operands as contiguous buffers.  The reference reads strided views
-    element by element inside each kernel (`*_strided` exports, kernels/strided.mojo); here a
-    strided operand is first copied row-major with mg_contiguous and the contiguous kernel
-    runs on the copy: same values, one extra pass for the rare strided case."""
+    element by element inside each kernel (`*_strided` exports, kernels/strided.mojo).  Here add,
+    relu, relu_grad, cast and softmax have strided entries of their own; the kernels that use this
+    helper (softmax_grad, argmax, axis sums, scatter_add) copy a strided operand row-major with
+    mg_contiguous first and run the contiguous kernel on the copy: same values, one extra
+    pass for the rare strided case."""
     out = list(inputs)
     for i in range(count):
         layout = node.src(i).layout()
@@ -545,29 +552,50 @@ def _materialise(node: Node, inputs: List[AnyBuffer], device: Device, count: int
     return out
 
 
+def _flat(node: Node, inputs: List[AnyBuffer], count: int) -> bool:
+    """Whether the first `count` operands can take a flat kernel: contiguous, and starting on the
+    16-byte boundary those kernels read from (a view into the middle of a buffer may not)."""
+    return all(node.src(i).layout().is_contiguous() and (inputs[i].data_ptr().value or 0) % 16 == 0
+               for i in range(count))
+
+
 def add(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
-    """ADD[a, b] (residual connections, gradient accumulation).  runtime/__init__.mojo:319-333."""
-    inputs = _materialise(node, inputs, device, 2)
+    """ADD[a, b] (residual connections, gradient accumulation, a broadcast bias).
+    runtime/__init__.mojo:319-333: contiguous operands take the flat kernel, views the strided one."""
     out = AnyBuffer.create(node.dtype(), device, node.numel())
-    device.lib.mg_add(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), node.numel(), node.dtype(),
-                      device.stream)
+    if _flat(node, inputs, 2):
+        device.lib.mg_add(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), node.numel(), node.dtype(),
+                          device.stream)
+    else:
+        la, lb = node.src(0).layout(), node.src(1).layout()
+        device.lib.mg_add_strided(inputs[0].data_ptr(), inputs[1].data_ptr(), out.data_ptr(), la.rank(),
+                                  _i64_array(la.shape()), _i64_array(la.stride()), _i64_array(lb.stride()),
+                                  node.dtype(), device.stream)
     return [out]
 
 
 def relu(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     """RELU[a].  runtime/__init__.mojo:296-297."""
-    inputs = _materialise(node, inputs, device, 1)
     out = AnyBuffer.create(node.dtype(), device, node.numel())
-    device.lib.mg_relu(inputs[0].data_ptr(), out.data_ptr(), node.numel(), node.dtype(), device.stream)
+    layout = node.src(0).layout()
+    if _flat(node, inputs, 1):
+        device.lib.mg_relu(inputs[0].data_ptr(), out.data_ptr(), node.numel(), node.dtype(), device.stream)
+    else:
+        device.lib.mg_relu_strided(inputs[0].data_ptr(), out.data_ptr(), layout.rank(), _i64_array(layout.shape()),
+                                   _i64_array(layout.stride()), node.dtype(), device.stream)
     return [out]
 
 
 def cast(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     """CAST[a] to node.dtype().  runtime/__init__.mojo:300-311."""
-    inputs = _materialise(node, inputs, device, 1)
     out = AnyBuffer.create(node.dtype(), device, node.numel())
-    device.lib.mg_cast(inputs[0].data_ptr(), out.data_ptr(), node.numel(), node.src(0).dtype(), node.dtype(),
-                       device.stream)
+    layout = node.src(0).layout()
+    if _flat(node, inputs, 1):
+        device.lib.mg_cast(inputs[0].data_ptr(), out.data_ptr(), node.numel(), node.src(0).dtype(), node.dtype(),
+                           device.stream)
+    else:
+        device.lib.mg_cast_strided(inputs[0].data_ptr(), out.data_ptr(), layout.rank(), _i64_array(layout.shape()),
+                                   _i64_array(layout.stride()), node.src(0).dtype(), node.dtype(), device.stream)
     return [out]
 
 
@@ -621,12 +649,15 @@ def scatter_add(node: Node, inputs: List[AnyBuffer], device: Device) -> List[Any
 def softmax(node: Node, inputs: List[AnyBuffer], device: Device) -> List[AnyBuffer]:
     """SOFTMAX[a] over the last axis.  runtime/__init__.mojo (softmax), kernels/__init__.mojo:1015-1030."""
     layout = node.src(0).layout()
-    inputs = _materialise(node, inputs, device, 1)
     _require_float(node.dtype(), "softmax")
-    cols = layout.shape(layout.rank() - 1)
-    rows = layout.numel() // cols
     out = AnyBuffer.create(node.dtype(), device, node.numel())
-    device.lib.mg_softmax(inputs[0].data_ptr(), out.data_ptr(), rows, cols, node.dtype(), device.stream)
+    if layout.is_contiguous():
+        cols = layout.shape(layout.rank() - 1)
+        rows = layout.numel() // cols if cols else 0
+        device.lib.mg_softmax(inputs[0].data_ptr(), out.data_ptr(), rows, cols, node.dtype(), device.stream)
+    else:  # kernels/__init__.mojo:1033-1060: views go to the strided kernel
+        device.lib.mg_softmax_strided(inputs[0].data_ptr(), out.data_ptr(), layout.rank(), _i64_array(layout.shape()),
+                                      _i64_array(layout.stride()), node.dtype(), device.stream)
     return [out]
 
 

@@ -283,9 +283,112 @@ def test_embedding_grad_adjoint_full_size(device):
     np.testing.assert_array_equal(hist[:, 0], np.bincount(idx, minlength=V).astype(np.float32))
 
 
+MAP_VIEWS = [
+    # shape, strides of operand a, strides of operand b, elements behind a, behind b
+    ((64, 48), (1, 64), (48, 1), 64 * 48, 64 * 48),                 # a transposed, b row-major
+    ((40, 96), (96, 1), (0, 1), 40 * 96, 96),                        # b a bias row broadcast over the rows
+    ((40, 96), (96, 1), (1, 0), 40 * 96, 40),                        # b a column broadcast along the rows
+    ((2, 5, 3, 16), (240, 16, 80, 1), (240, 48, 16, 1), 480, 480),   # a (B,H,S,D) read as (B,S,H,D)
+    ((6, 24), (48, 2), (24, 1), 6 * 48, 6 * 24),                     # every other column of a
+    ((3, 4, 32), (0, 32, 1), (128, 32, 1), 128, 384),                # a broadcast over the leading dim
+    ((7, 9), (9, 1), (0, 0), 63, 1),                                 # b one value
+    ((5, 8), (12, 1), (8, 1), 60, 40),                               # rows of a 12 apart: 16-byte rows in fp32, not in 16 bits
+    ((1 << 12, 1 << 7), (1 << 7, 1), (0, 1), 1 << 19, 1 << 7),       # large, bias
+    ((1 << 10, 1 << 9), (1, 1 << 10), (1 << 9, 1), 1 << 19, 1 << 19),  # large, transposed
+    ((13,), (3,), (1,), 39, 13),
+    ((1, 1), (1, 1), (1, 1), 1, 1),
+]
+
+
+@pytest.mark.parametrize("shape,sa,sb,na,nb", MAP_VIEWS)
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("offset", [0, 1])
+def test_maps_over_strided_views(device, shape, sa, sb, na, nb, dtype, offset):
+    # add, relu, relu_grad and cast read strided views themselves (the reference's *_strided
+    # kernels, kernels/strided.mojo:54-114): transposed, sliced and broadcast operands, at 16-byte
+    # aligned and at odd base offsets.  One rounding at most, so the results are compared bit for
+    # bit with numpy on the same views.
+    a = round_to_dtype(normal(75, 0, (na + offset,)), dtype)
+    b = round_to_dtype(normal(75, 1, (nb + offset,)), dtype)
+    item = a.itemsize
+    va = np.lib.stride_tricks.as_strided(a[offset:], shape, tuple(t * item for t in sa))
+    vb = np.lib.stride_tricks.as_strided(b[offset:], shape, tuple(t * item for t in sb))
+    la = Layout(*shape, strides=sa, base_offset=offset)
+    lb = Layout(*shape, strides=sb, base_offset=offset)
+    out = Layout(*shape)
+    got = _run(device, "ADD", out, [(a, la, dtype), (b, lb, dtype)], dtype)
+    np.testing.assert_array_equal(got, round_to_dtype(va + vb, dtype))
+    got = _run(device, "RELU_GRAD", out, [(a, la, dtype), (b, lb, dtype)], dtype)
+    np.testing.assert_array_equal(got, np.where(va > 0, vb, 0).astype(np.float32))
+    got = _run(device, "RELU", out, [(a, la, dtype)], dtype)
+    np.testing.assert_array_equal(got, np.maximum(va, 0))
+    for to in FLOATS:
+        got = _run(device, "CAST", out, [(a, la, dtype)], to)
+        np.testing.assert_array_equal(got, round_to_dtype(va, to))
+
+
+SOFTMAX_VIEWS = [
+    # shape, strides, elements behind the view
+    ((48, 64), (1, 48), 48 * 64),                    # transposed: a row runs down a column
+    ((2, 5, 3, 16), (240, 16, 80, 1), 480),          # permuted heads, contiguous rows of 16
+    ((6, 24), (48, 2), 6 * 48),                      # every other column
+    ((3, 4, 32), (0, 32, 1), 128),                   # broadcast leading dim
+    ((5, 40), (56, 1), 5 * 56),                      # rows with a gap between them
+    ((7,), (3,), 21),
+    ((300, 1000), (1000, 1), 300000),                # contiguous, through the strided entry at an odd offset
+]
+
+
+@pytest.mark.parametrize("shape,strides,n", SOFTMAX_VIEWS)
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("offset", [0, 3])
+def test_softmax_over_strided_views(device, shape, strides, n, dtype, offset):
+    # SOFTMAX of a view runs mograd_softmax_strided in the reference (kernels/__init__.mojo:1033-1060)
+    # and mg_softmax_strided here: the same arithmetic as the contiguous kernel, so it must agree
+    # with the contiguous kernel on a row-major copy of the view, and with the oracle, within the
+    # storage type's rounding.
+    a = round_to_dtype(normal(76, 0, (n + offset,), std=2.0), dtype)
+    view = np.lib.stride_tricks.as_strided(a[offset:], shape, tuple(t * a.itemsize for t in strides))
+    layout = Layout(*shape, strides=strides, base_offset=offset)
+    lib, st = device.lib, device.stream
+    buf = AnyBuffer.from_numpy(device, a, dtype).view(layout)
+    got = AnyBuffer.create(dtype, device, view.size)
+    lib.mg_softmax_strided(buf.data_ptr(), got.data_ptr(), len(shape), R._i64_array(shape), R._i64_array(strides), dtype, st)
+    flat = AnyBuffer.from_numpy(device, np.ascontiguousarray(view), dtype)
+    ref = AnyBuffer.create(dtype, device, view.size)
+    cols = shape[-1]
+    lib.mg_softmax(flat.data_ptr(), ref.data_ptr(), view.size // cols, cols, dtype, st)
+    # (a view whose rows cannot be read 16 bytes at a time is summed in another order: a few ulps)
+    tol = {F32: 1e-6, F16: 1e-3, BF16: 8e-3}[dtype]
+    np.testing.assert_allclose(got.to_numpy(shape), ref.to_numpy(shape), rtol=tol, atol=0)
+    np.testing.assert_allclose(got.to_numpy(shape), O.softmax(view.astype(np.float64)), rtol=tol, atol=tol)
+    # and through the scheduler entry
+    out = _run(device, "SOFTMAX", Layout(*shape), [(a, layout, dtype)], dtype)
+    np.testing.assert_array_equal(out, got.to_numpy(shape))
+
+
+def test_strided_maps_check_their_arguments(device):
+    lib, st = device.lib, device.stream
+    buf = AnyBuffer.create(F32, device, 64, fill=1.0)
+    arr = lambda *v: R._i64_array(v)  # noqa: E731
+    with pytest.raises(MogradError, match="rank"):
+        lib.mg_relu_strided(buf.data_ptr(), buf.data_ptr(), 9, arr(*[1] * 9), arr(*[1] * 9), F32, st)
+    with pytest.raises(MogradError, match="negative"):
+        lib.mg_add_strided(buf.data_ptr(), buf.data_ptr(), buf.data_ptr(), 1, arr(8), arr(1), arr(-1), F32, st)
+    with pytest.raises(MogradError, match="dtype"):
+        lib.mg_cast_strided(buf.data_ptr(), buf.data_ptr(), 1, arr(8), arr(1), F32, I32, st)
+    with pytest.raises(MogradError, match="null"):
+        lib.mg_relu_grad_strided(buf.data_ptr(), None, buf.data_ptr(), 1, arr(8), arr(1), arr(1), F32, st)
+    with pytest.raises(MogradError, match="rank"):
+        lib.mg_softmax_strided(buf.data_ptr(), buf.data_ptr(), 0, arr(1), arr(1), F32, st)
+    # an empty view is no work, whatever the pointers
+    lib.mg_softmax_strided(None, None, 2, arr(0, 8), arr(8, 1), F32, st)
+    lib.mg_add_strided(None, None, None, 2, arr(0, 8), arr(8, 1), arr(8, 1), F32, st)
+
+
 def test_strided_operands_are_materialised(device):
-    # The reference's *_strided kernels read views element by element; here the scheduler entry
-    # copies a strided operand row-major first.  Same values either way.
+    # Row kernels (axis sums, softmax, argmax) and the index operand of gather take a strided
+    # operand through a row-major copy; the elementwise maps read it in place.  Same values either way.
     a = normal(69, 0, (6, 8))
     b = normal(69, 1, (8, 6))
     at = Layout(6, 8).transpose()            # (8, 6) view of a
