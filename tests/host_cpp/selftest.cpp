@@ -368,6 +368,34 @@ int main(int argc, char** argv) {
     return close_to(download(g[0]), want, 0.0, "dx");
   });
 
+  run_case("elementwise maps and softmax read views in place", [&]() -> std::string {
+    // (6, 8) values; a bias row broadcast over the rows; the transpose of the values
+    const int64_t R = 6, C = 8;
+    const auto a = ints(R * C, 8, -5, 5), bias = ints(C, 9, -3, 3);
+    const Layout la{R, C}, lbias({R, C}, {0, 1}), lt({C, R}, {1, C});
+    auto sum = run(node("ADD", la, {OpRef::leaf(la), OpRef::leaf(lbias)}), {upload(dev, a), upload(dev, bias).view(lbias)}, dev);
+    std::vector<double> want(R * C);
+    for (int64_t i = 0; i < R; ++i)
+      for (int64_t j = 0; j < C; ++j) want[i * C + j] = a[i * C + j] + bias[j];
+    std::string why = close_to(download(sum[0]), want, 0.0, "a + bias row");
+    if (!why.empty()) return why;
+    auto rt = run(node("RELU", Layout{C, R}, {OpRef::leaf(lt)}), {upload(dev, a).view(lt)}, dev);
+    for (int64_t j = 0; j < C; ++j)
+      for (int64_t i = 0; i < R; ++i) want[j * R + i] = std::max(a[i * C + j], 0.0f);
+    why = close_to(download(rt[0]), want, 0.0, "relu of the transpose");
+    if (!why.empty()) return why;
+    auto gt = run(node("RELU_GRAD", Layout{C, R}, {OpRef::leaf(lt), OpRef::leaf(Layout{C, R})}),
+                  {upload(dev, a).view(lt), upload(dev, ints(R * C, 10, -9, 9))}, dev);
+    const auto up = ints(R * C, 10, -9, 9);
+    for (int64_t j = 0; j < C; ++j)
+      for (int64_t i = 0; i < R; ++i) want[j * R + i] = a[i * C + j] > 0 ? up[j * R + i] : 0.0;
+    why = close_to(download(gt[0]), want, 0.0, "relu_grad with a transposed output");
+    if (!why.empty()) return why;
+    // softmax down the columns of zeros: every entry 1 / R
+    auto sm = run(node("SOFTMAX", Layout{C, R}, {OpRef::leaf(lt)}), {upload(dev, std::vector<float>(R * C, 0.f)).view(lt)}, dev);
+    return close_to(download(sm[0]), std::vector<double>(R * C, 1.0 / R), 1e-6, "softmax of a transposed view");
+  });
+
   // Error conditions of the reference, with its messages
   run_case("matmul rejects non-collapsible batch dims", [&]() -> std::string {
     // transpose(1, 2) of a rank-4 tensor: batch dims no longer fold into one stride (kernels/__init__.mojo:633-634)
