@@ -155,16 +155,21 @@ static int launch_16bit_mfma(const GemmArgs& g, hipStream_t stream) {
   // Tiles copied straight into LDS (gemm_16bit_pipe_kernel) where that measured faster: an
   // operand that is not k-contiguous is transposed by the LDS read instead of in registers
   // (dX 15-25 %, dW 5-20 % faster at Linear-layer shapes, 20-30 % at 4096^3 and up), and long
-  // K loops gain from the single barrier per step (forward 8-10 % from K = 1024).  Short-K
-  // products of two k-contiguous operands stay with the register-staged kernel (4-8 %
-  // faster there), as does every shape the copy cannot take.  The pair is k per step and
-  // copies of the tiles: (32, 2) runs four workgroups per CU, (64, 2) two.
+  // K loops gain from the single barrier per step.  Two k-contiguous operands: from 384 k per
+  // workgroup on (2-8 % faster at 16384 rows, 10-25 % at 256-2048 rows), and from 192 for
+  // outputs of at most two tiles per CU (8-15 %); shorter K loops, and 192-383 on larger outputs
+  // (3-8 % slower there), stay with the register-staged kernel, as does every shape the copy
+  // cannot take (MOGRAD_HIP_GEMM16_PIPE_MIN_K moves the 384).  The pair is k per step and copies
+  // of the tiles: (32, 2) runs four workgroups per CU, (64, 2) two.
   // MOGRAD_HIP_GEMM16_PIPE = 0 | 322 | 642 | 2322 | 2642 overrides the choice (2xxx: 256 x 128 tiles).
   int pipe = 0;
   if constexpr (!RAGGED) {
     if (g.K % kG16BK == 0 && mult8(g.M) && mult8(g.N)) {
       const int64_t k_wg = ceil_div(g.K, splits);  // the K range one workgroup walks
-      if (A_KC && B_KC) pipe = k_wg >= 1024 ? 642 : 0;
+      if (A_KC && B_KC) {
+        const int64_t min_k = env_int("MOGRAD_HIP_GEMM16_PIPE_MIN_K", 384);
+        pipe = k_wg >= min_k || (2 * k_wg >= min_k && blocks <= 2 * cus) ? 642 : 0;
+      }
       else pipe = k_wg >= 4096 ? 642 : 322;
       // Large products: 256 x 128 tiles (eight waves), a quarter fewer operand bytes per FLOP
       // through L2, once they still give every CU two workgroups (4096^3: 3-11 % faster).
