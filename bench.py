@@ -441,36 +441,38 @@ def bench_attention(args, dev) -> dict:
 
     lib, st = dev.lib, dev.stream
 
-    def make(B, H, S, D, cfg):
+    def make(B, H, S, D, cfg, dtype=BF16):
         n = B * S * H * D
-        q, k, v, do = (AnyBuffer.from_numpy(dev, _rng(4, cfg * 10 + i).standard_normal(n, dtype=np.float32), BF16)
+        q, k, v, do = (AnyBuffer.from_numpy(dev, _rng(4, cfg * 10 + i).standard_normal(n, dtype=np.float32), dtype)
                        for i in range(4))
-        o, dq, dk, dv = (AnyBuffer.create(BF16, dev, n) for _ in range(4))
+        o, dq, dk, dv = (AnyBuffer.create(dtype, dev, n) for _ in range(4))
         lse = AnyBuffer.create(F32, dev, B * H * S)
         return q, k, v, do, o, dq, dk, dv, lse
 
-    def runner(B, H, S, D, causal, bufs):
+    def runner(B, H, S, D, causal, bufs, dtype=BF16):
         q, k, v, do, o, dq, dk, dv, lse = bufs
         sc = 1.0 / float(np.sqrt(D))
         P = lambda b: b.data_ptr()  # noqa: E731
-        f = lambda i: lib.mg_flash_attn_fwd(P(q), P(k), P(v), None, P(o), P(lse), B, S, H, D, sc, causal, 0, BF16, st)  # noqa: E731
+        f = lambda i: lib.mg_flash_attn_fwd(P(q), P(k), P(v), None, P(o), P(lse), B, S, H, D, sc, causal, 0, dtype, st)  # noqa: E731
         b = lambda i: lib.mg_flash_attn_bwd(P(do), P(o), P(q), P(k), P(v), None, P(lse), P(dq), P(dk), P(dv), B, S, H, D,  # noqa: E731
-                                            sc, causal, 0, BF16, st)
+                                            sc, causal, 0, dtype, st)
         return f, b
 
     c1 = (8, 12, 1024, 64)
     c2 = (2, 12, 4096, 64)
-    bufs1, bufs2 = make(*c1, 1), make(*c2, 2)
+    bufs1, bufs2, bufs3 = make(*c1, 1), make(*c2, 2), make(*c2, 3, F32)
     f1, b1 = runner(*c1, 1, bufs1)
     f2, b2 = runner(*c2, 0, bufs2)
-    for (Bc, Hc, Sc, Dc), causal, bufs, f, b in ((c1, True, bufs1, f1, b1), (c2, False, bufs2, f2, b2)):
+    f3, b3 = runner(*c2, 0, bufs3, F32)  # the same tensors' shape in fp32: the fp32 matrix-core kernels
+    for (Bc, Hc, Sc, Dc), causal, bufs, f, b, rtol in ((c1, True, bufs1, f1, b1, 3e-2), (c2, False, bufs2, f2, b2, 3e-2),
+                                                       (c2, False, bufs3, f3, b3, 1e-4)):
         f(0)
         b(0)
         q_, k_, v_, do_, o_, dq_, dk_, dv_, lse_ = bufs
         bshd, bhsd = (Bc, Sc, Hc, Dc), (Bc, Hc, Sc, Dc)
         _verify_attention(q_.to_numpy(bshd), k_.to_numpy(bshd), v_.to_numpy(bshd), do_.to_numpy(bhsd), o_.to_numpy(bhsd),
                           lse_.to_numpy((Bc, Hc, Sc)), dq_.to_numpy(bshd), dk_.to_numpy(bshd), dv_.to_numpy(bshd),
-                          Bc, Hc, Sc, Dc, causal)
+                          Bc, Hc, Sc, Dc, causal, rtol)
 
     def step(i):
         f1(i)
@@ -486,6 +488,9 @@ def bench_attention(args, dev) -> dict:
         ("flash_attn_fwd bf16 causal B8 H12 S1024 D64 (2 B H S^2 D)", f1, 2.0 * fl1, "F", MFMA_BF16_PEAK_TFLOPS),
         ("flash_attn_bwd bf16 B2 H12 S4096 D64 (10 B H S^2 D)", b2, 10.0 * fl2, "F", MFMA_BF16_PEAK_TFLOPS),
         ("flash_attn_fwd bf16 B2 H12 S4096 D64 (4 B H S^2 D)", f2, 4.0 * fl2, "F", MFMA_BF16_PEAK_TFLOPS),
+        ("flash_attn_bwd fp32 B2 H12 S4096 D64 (10 B H S^2 D; not a BASELINE configuration: fp32 tensors on the fp32 "
+         "matrix pipe)", b3, 10.0 * fl2, "F", MFMA_F32_PEAK_TFLOPS),
+        ("flash_attn_fwd fp32 B2 H12 S4096 D64 (4 B H S^2 D; likewise)", f3, 4.0 * fl2, "F", MFMA_F32_PEAK_TFLOPS),
     ]
     kernels = _kernel_table(dev, entries, max(10, min(args.steps, 50)))
     dom = kernels[0]

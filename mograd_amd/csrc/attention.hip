@@ -1,5 +1,6 @@
 // C ABI for flash attention: argument checks, routing between the MFMA kernels (16-bit
 // storage, head dimension up to 128) and the general fp32-arithmetic kernels.
+#include "attention_f32_mfma.h"
 #include "attention_generic.h"
 #include "attention_tiled.h"
 #include "mg_internal.h"
@@ -30,6 +31,63 @@ static int check_attn(const char* who, int64_t B, int64_t S, int64_t H, int64_t 
 // workgroup; MOGRAD_HIP_ATTN_TILED=0 keeps the wave-per-row kernels.
 static bool attn_tiled_ok(const AttnDims& a) {
   return a.D <= 512 && a.S >= 64 && static_cast<int64_t>(a.B) * a.H <= 65535 && env_int("MOGRAD_HIP_ATTN_TILED", 1) != 0;
+}
+
+// fp32 arithmetic on the matrix cores (attention_f32_mfma.h): head dims up to 128 once a sequence
+// has rows for a workgroup; MOGRAD_HIP_ATTN_F32_MFMA=0 keeps the row-per-thread kernels.
+static bool attn_f32_mfma_ok(const AttnDims& a) {
+  return a.D <= kF32AttnMaxD && a.S >= 64 && ceil_div(a.S, kF32AttnBlock) <= 65535 &&
+         env_int("MOGRAD_HIP_ATTN_F32_MFMA", 1) != 0;
+}
+
+template <typename T>
+static void fwd_f32_mfma_launch(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse,
+                                const AttnDims& a, float scale, bool causal, bool has_bias, hipStream_t stream) {
+  const dim3 grid(static_cast<unsigned>(a.B * a.H), static_cast<unsigned>(ceil_div(a.S, kF32AttnBlock)));
+#define MG_FWD_DP(DP_, C_, B_)                                                                                      \
+  hipLaunchKernelGGL((attn_fwd_f32_mfma_kernel<T, DP_, C_, B_>), grid, dim3(256), 0, stream,                        \
+                     static_cast<const T*>(q), static_cast<const T*>(k), static_cast<const T*>(v),                  \
+                     static_cast<const T*>(mask), static_cast<T*>(o), lse, a, scale)
+#define MG_FWD(C_, B_)                                                                                              \
+  do {                                                                                                              \
+    if (a.D <= 32) MG_FWD_DP(32, C_, B_);                                                                           \
+    else if (a.D <= 64) MG_FWD_DP(64, C_, B_);                                                                      \
+    else MG_FWD_DP(128, C_, B_);                                                                                    \
+  } while (0)
+  if (causal) MG_FWD(true, false);
+  else if (has_bias) MG_FWD(false, true);
+  else MG_FWD(false, false);
+#undef MG_FWD
+#undef MG_FWD_DP
+}
+
+template <typename T>
+static void bwd_f32_mfma_launch(const void* d_o, const void* q, const void* k, const void* v, const void* mask,
+                                const float* lse, const float* delta, void* dq, void* dk, void* dv, const AttnDims& a,
+                                float scale, bool causal, bool has_bias, hipStream_t stream) {
+  const dim3 grid(static_cast<unsigned>(a.B * a.H), static_cast<unsigned>(ceil_div(a.S, kF32AttnBlock)));
+#define MG_BWD_DP(DP_, C_, B_)                                                                                     \
+  do {                                                                                                             \
+    hipLaunchKernelGGL((attn_dkdv_f32_mfma_kernel<T, DP_, C_, B_>), grid, dim3(256), 0, stream,                    \
+                       static_cast<const T*>(d_o), static_cast<const T*>(q), static_cast<const T*>(k),             \
+                       static_cast<const T*>(v), static_cast<const T*>(mask), lse, delta, static_cast<T*>(dk),     \
+                       static_cast<T*>(dv), a, scale);                                                             \
+    hipLaunchKernelGGL((attn_dq_f32_mfma_kernel<T, DP_, C_, B_>), grid, dim3(256), 0, stream,                      \
+                       static_cast<const T*>(d_o), static_cast<const T*>(q), static_cast<const T*>(k),             \
+                       static_cast<const T*>(v), static_cast<const T*>(mask), lse, delta, static_cast<T*>(dq), a,  \
+                       scale);                                                                                     \
+  } while (0)
+#define MG_BWD(C_, B_)                                                                                             \
+  do {                                                                                                             \
+    if (a.D <= 32) MG_BWD_DP(32, C_, B_);                                                                          \
+    else if (a.D <= 64) MG_BWD_DP(64, C_, B_);                                                                     \
+    else MG_BWD_DP(128, C_, B_);                                                                                   \
+  } while (0)
+  if (causal) MG_BWD(true, false);
+  else if (has_bias) MG_BWD(false, true);
+  else MG_BWD(false, false);
+#undef MG_BWD
+#undef MG_BWD_DP
 }
 
 template <typename T, int NT, int DL>
@@ -73,6 +131,11 @@ template <typename T>
 static int fwd_generic(const void* q, const void* k, const void* v, const void* mask, void* o, float* lse, AttnDims a,
                        float scale, bool causal, bool has_bias, hipStream_t stream) {
   const int64_t rows = static_cast<int64_t>(a.B) * a.H * a.S;
+  if (attn_f32_mfma_ok(a)) {
+    fwd_f32_mfma_launch<T>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
+    MG_LAUNCH_CHECK();
+    return MG_OK;
+  }
   if (attn_tiled_ok(a)) {
     if (a.D <= 32) fwd_tiled_launch<T, 1, 32>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
     else if (a.D <= 64) fwd_tiled_launch<T, 2, 32>(q, k, v, mask, o, lse, a, scale, causal, has_bias, stream);
@@ -106,6 +169,11 @@ static int bwd_generic(const void* d_o, const void* o, const void* q, const void
   hipLaunchKernelGGL((attn_delta_kernel<T>), grid, dim3(256), 0, stream, static_cast<const T*>(d_o),
                      static_cast<const T*>(o), delta.as<float>(), rows, a.D, a.S, a.H, a.o_bshd);
   MG_LAUNCH_CHECK();
+  if (attn_f32_mfma_ok(a)) {
+    bwd_f32_mfma_launch<T>(d_o, q, k, v, mask, lse, delta.as<float>(), dq, dk, dv, a, scale, causal, has_bias, stream);
+    MG_LAUNCH_CHECK();
+    return MG_OK;
+  }
   if (attn_tiled_ok(a)) {
     const float* dl = delta.as<float>();
     if (a.D <= 32) bwd_tiled_launch<T, 1, 32, 1, 32>(d_o, q, k, v, mask, lse, dl, dq, dk, dv, a, scale, causal, has_bias, stream);

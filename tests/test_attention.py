@@ -94,11 +94,39 @@ def test_f32_row_per_thread_and_wave_per_row_kernels(device, monkeypatch, name, 
     q, k, v, do, m = _inputs(58, B, S, H, D, F32, with_mask)
     ro, rl = O.sdpa_fwd(q, k, v, m, causal)
     want = (ro, rl) + tuple(O.sdpa_bwd(q, k, v, do, m, causal))
+    monkeypatch.setenv("MOGRAD_HIP_ATTN_F32_MFMA", "0")  # (the matrix-core form has its own test below)
     for mode in ("0", "1"):
         monkeypatch.setenv("MOGRAD_HIP_ATTN_TILED", mode)
         got = _fwd_bwd(device, q, k, v, do, m, causal)
         for g, w, what in zip(got, want, ("o", "lse", "dq", "dk", "dv")):
             assert _max_err(g, w) <= budget, f"{what} (tiled={mode}): {_max_err(g, w)}"
+
+
+@pytest.mark.parametrize("name,causal,with_mask", MODES)
+@pytest.mark.parametrize("B,H,S,D,budget", [(1, 2, 300, 64, 5e-6), (2, 2, 96, 64, 5e-6), (1, 3, 64, 24, 5e-6),
+                                            (2, 2, 130, 32, 5e-6), (1, 1, 257, 40, 5e-6), (1, 2, 129, 7, 5e-6),
+                                            (1, 1, 1000, 64, 1e-5), (1, 2, 128, 48, 5e-6), (2, 1, 100, 128, 1e-5),
+                                            (1, 1, 257, 72, 1e-5), (1, 2, 130, 100, 1e-5), (1, 2, 96, 16, 5e-6)])
+def test_f32_matrix_core_kernels(device, monkeypatch, name, causal, with_mask, B, H, S, D, budget):
+    # fp32 tensors with heads of up to 128 columns and at least 64 tokens take fp32 MFMA kernels
+    # (32 resident rows per wave, tiles of 32 streamed rows; kernels for 32, 64 and 128 columns); they must meet the reference's fp32
+    # budget against the f64 oracle like the FMA forms (tests/kernels/attention/generic.mojo:440-665),
+    # at lengths that leave ragged tiles and blocks, head dims that are not multiples of four
+    # (element-wise loads and stores) and both layouts of O.
+    q, k, v, do, m = _inputs(60, B, S, H, D, F32, with_mask)
+    ro, rl = O.sdpa_fwd(q, k, v, m, causal)
+    want = (ro, rl) + tuple(O.sdpa_bwd(q, k, v, do, m, causal))
+    results = {}
+    for mfma in ("1", "0"):
+        monkeypatch.setenv("MOGRAD_HIP_ATTN_F32_MFMA", mfma)
+        results[mfma] = _fwd_bwd(device, q, k, v, do, m, causal)
+        for g, w, what in zip(results[mfma], want, ("o", "lse", "dq", "dk", "dv")):
+            assert _max_err(g, w) <= budget, f"{what} (mfma={mfma}): {_max_err(g, w)}"
+    # and it is deterministic
+    monkeypatch.setenv("MOGRAD_HIP_ATTN_F32_MFMA", "1")
+    again = _fwd_bwd(device, q, k, v, do, m, causal)
+    for a_, b_ in zip(again, results["1"]):
+        np.testing.assert_array_equal(a_, b_)
 
 
 HALF_SHAPES = [(2, 2, 96, 64), (1, 3, 200, 64), (2, 1, 128, 128), (1, 2, 257, 32), (1, 1, 4, 8), (1, 2, 96, 256),
