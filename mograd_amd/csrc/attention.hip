@@ -1,5 +1,6 @@
-// C ABI for flash attention: argument checks, routing between the MFMA kernels (16-bit
-// storage, head dimension up to 128) and the general fp32-arithmetic kernels.
+// C ABI for flash attention: argument checks, routing between the 16-bit MFMA kernels (16-bit
+// storage, head dimension up to 256), the fp32 MFMA kernels (head dimension up to 128) and the
+// general fp32 FMA kernels.
 #include "attention_f32_mfma.h"
 #include "attention_generic.h"
 #include "attention_tiled.h"
