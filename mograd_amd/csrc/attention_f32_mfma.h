@@ -161,7 +161,9 @@ __device__ __forceinline__ void f32_attn_store(T* __restrict__ row, const f32x16
     }
 }
 
-// Bias of (row i, columns j0 + f32_acc_row(r, half)) for the sixteen registers, in log2 units.
+// Bias of (row i, columns j0 + f32_acc_row(r, half)) for the sixteen registers, as loaded: any
+// arithmetic on the values here would put the wait for them in front of the products that are
+// meant to hide it.
 template <typename T>
 __device__ __forceinline__ void f32_attn_bias_row(const T* __restrict__ mrow, int j0, int half, int S, bool vec_ok,
                                                   float (&b)[16]) {
@@ -171,15 +173,15 @@ __device__ __forceinline__ void f32_attn_bias_row(const T* __restrict__ mrow, in
     if constexpr (sizeof(T) == 4) {
       if (vec_ok && j + 4 <= S) {
         const float4 w = *reinterpret_cast<const float4*>(mrow + j);
-        b[g * 4] = w.x * kAttnLog2e;
-        b[g * 4 + 1] = w.y * kAttnLog2e;
-        b[g * 4 + 2] = w.z * kAttnLog2e;
-        b[g * 4 + 3] = w.w * kAttnLog2e;
+        b[g * 4] = w.x;
+        b[g * 4 + 1] = w.y;
+        b[g * 4 + 2] = w.z;
+        b[g * 4 + 3] = w.w;
         continue;
       }
     }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) b[g * 4 + e] = to_float(mrow[min(j + e, S - 1)]) * kAttnLog2e;
+    for (int e = 0; e < 4; ++e) b[g * 4 + e] = to_float(mrow[min(j + e, S - 1)]);
   }
 }
 
@@ -225,15 +227,18 @@ __global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_fwd_f32_mfma_kernel
     __syncthreads();
     if (j0 + kF32AttnRows < j_end) f32_attn_fetch<T, DP>(kbase, a.ld, vbase, a.ld, j0 + kF32AttnRows, a.S, a.D, vec_qkv, st);
     if (CAUSAL && j0 > wave_last) continue;  // wave-uniform: nothing of this tile is visible
+    float bias[16];  // requested before the products that hide the loads (and kept there)
+    if (HAS_BIAS) {
+      f32_attn_bias_row<T>(mrow, j0, half, a.S, vec_m, bias);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     f32x16 s = f32_attn_scores<DP>(k_s, qr, lane, f32x16_zero());
-    float bias[16];
-    if (HAS_BIAS) f32_attn_bias_row<T>(mrow, j0, half, a.S, vec_m, bias);
     float m_tile = -INFINITY;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int j = j0 + f32_acc_row(r, half);
       float sv = s[r];
-      if (HAS_BIAS) sv += bias[r];
+      if (HAS_BIAS) sv = fmaf(bias[r], kAttnLog2e, sv);
       const bool valid = j < a.S && (!CAUSAL || j <= i);
       s[r] = valid ? sv : -INFINITY;
       m_tile = fmaxf(m_tile, s[r]);
@@ -306,15 +311,18 @@ __global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_dq_f32_mfma_kernel(
     __syncthreads();
     if (j0 + kF32AttnRows < j_end) f32_attn_fetch<T, DP>(kbase, a.ld, vbase, a.ld, j0 + kF32AttnRows, a.S, a.D, vec_qkv, st);
     if (CAUSAL && j0 > wave_last) continue;
+    float bias[16];
+    if (HAS_BIAS) {
+      f32_attn_bias_row<T>(mrow, j0, half, a.S, vec_m, bias);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     f32x16 s = f32_attn_scores<DP>(k_s, qr, lane, f32x16_zero());
     const f32x16 dp = f32_attn_scores<DP>(v_s, dor, lane, f32x16_zero());
-    float bias[16];
-    if (HAS_BIAS) f32_attn_bias_row<T>(mrow, j0, half, a.S, vec_m, bias);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int j = j0 + f32_acc_row(r, half);
       float sv = s[r];
-      if (HAS_BIAS) sv += bias[r];
+      if (HAS_BIAS) sv = fmaf(bias[r], kAttnLog2e, sv);
       const bool valid = j < a.S && (!CAUSAL || j <= i);
       const float p = valid ? exp2f(sv - lse2) : 0.f;
       s[r] = p * (dp[r] - dl);  // dS without the scale: K was staged unscaled, the scale goes on at the end
@@ -381,6 +389,14 @@ __global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_dkdv_f32_mfma_kerne
     __syncthreads();
     if (i0 + kF32AttnRows < a.S) fetch(i0 + kF32AttnRows);
     if (CAUSAL && i0 + kF32AttnRows - 1 < wave_first) continue;  // wave-uniform: no query of the tile sees these keys
+    float bias[16];  // rows i0 + f32_acc_row(r, half) of the bias, this lane's key column
+    if (HAS_BIAS) {
+      const T* mcol = mask + static_cast<int64_t>(bh) * a.S * a.S + jc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        bias[r] = to_float(mcol[static_cast<int64_t>(min(i0 + f32_acc_row(r, half), a.S - 1)) * a.S]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     f32x16 s = f32_attn_scores<DP>(q_s, kr, lane, f32x16_zero());
     f32x16 dp = f32_attn_scores<DP>(do_s, vr, lane, f32x16_zero());
 #pragma unroll
@@ -393,8 +409,7 @@ __global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_dkdv_f32_mfma_kerne
       for (int e = 0; e < 4; ++e) {
         const int r = g * 4 + e, i = i0 + rr + e;
         float sv = s[r];
-        if (HAS_BIAS)
-          sv = fmaf(to_float(mask[(static_cast<int64_t>(bh) * a.S + min(i, a.S - 1)) * a.S + jc]), kAttnLog2e, sv);
+        if (HAS_BIAS) sv = fmaf(bias[r], kAttnLog2e, sv);
         const bool valid = i < a.S && (!CAUSAL || j <= i);
         const float p = valid ? exp2f(sv - lv[e]) : 0.f;
         s[r] = p;
