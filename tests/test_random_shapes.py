@@ -146,6 +146,43 @@ def test_random_attention_shapes(device):
             assert_close(got, want, tol, tol * max(np.abs(want).max(), 1e-3), what + " " + name)
 
 
+def test_random_f32_attention_shapes(device):
+    # fp32 tensors: head dims 1-160 (the matrix-core kernels for 32, 64 and 128 columns, element-wise
+    # loads when D is not a multiple of four, the row-per-thread kernels above 128), lengths on both
+    # sides of the 64-token threshold, every mask mode; the reference's widest fp32 budget for these
+    # head dims (tests/kernels/attention/generic.mojo:440-665) against the f64 oracle.
+    rng = np.random.Generator(np.random.PCG64(98_000))
+    lib, st = device.lib, device.stream
+    for case in range(24):
+        B, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
+        S = int(rng.integers(1, 400))
+        D = int(rng.integers(1, 161))
+        causal, with_mask = case % 3 == 0, case % 3 == 1
+        scale = 1.0 / math.sqrt(D)
+        q, k, v = (rng.standard_normal((B, S, H, D)).astype(np.float32) for _ in range(3))
+        do = rng.standard_normal((B, H, S, D)).astype(np.float32)
+        m = rng.standard_normal((B, H, S, S)).astype(np.float32) if with_mask else None
+        bq, bk, bv, bdo = (AnyBuffer.from_numpy(device, a, F32) for a in (q, k, v, do))
+        bm = AnyBuffer.from_numpy(device, m, F32) if with_mask else None
+        pm = bm.data_ptr() if with_mask else None
+        n = B * S * H * D
+        o, dq, dk, dv = (AnyBuffer.create(F32, device, n) for _ in range(4))
+        lse = AnyBuffer.create(F32, device, B * H * S)
+        lib.mg_flash_attn_fwd(bq.data_ptr(), bk.data_ptr(), bv.data_ptr(), pm, o.data_ptr(), lse.data_ptr(), B, S, H, D,
+                              scale, int(causal), int(with_mask), F32, st)
+        lib.mg_flash_attn_bwd(bdo.data_ptr(), o.data_ptr(), bq.data_ptr(), bk.data_ptr(), bv.data_ptr(), pm,
+                              lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, S, H, D, scale, int(causal),
+                              int(with_mask), F32, st)
+        wo, wl = O.sdpa_fwd(q, k, v, m, causal, scale)
+        wdq, wdk, wdv = O.sdpa_bwd(q, k, v, do, m, causal, scale)
+        what = f"case {case} B{B} S{S} H{H} D{D} causal={causal} bias={with_mask}"
+        for got, want, name in ((lse.to_numpy((B, H, S)), wl, "lse"), (o.to_numpy((B, H, S, D)), wo, "o"),
+                                (dq.to_numpy((B, S, H, D)), wdq, "dq"), (dk.to_numpy((B, S, H, D)), wdk, "dk"),
+                                (dv.to_numpy((B, S, H, D)), wdv, "dv")):
+            err = float(np.max(np.abs(got.astype(np.float64) - want)))
+            assert np.all(np.isfinite(got)) and err <= 2e-5, f"{what} {name}: {err}"
+
+
 def test_random_row_kernel_shapes(device):
     rng = np.random.Generator(np.random.PCG64(97_000))
     lib, st = device.lib, device.stream
