@@ -2120,11 +2120,12 @@ static int bwd_typed(const void* d_o, const void* o, const void* q, const void* 
   }
   MG_TRY(launch_delta(static_cast<const T*>(d_o), static_cast<const T*>(o), delta.as<float>(), rows, a, stream, ps));
   const int64_t blocks = static_cast<int64_t>(a.B) * a.H * ceil_div(a.S, 128);
-  // One launch for both walks up to this sequence length (measured: 3-5% faster up to 512,
-  // even at 1024, 2-3% slower from 2048 on, where the two walks compete for the same CU
-  // instead of filling each other's gaps).  MOGRAD_HIP_ATTN_FUSED_BWD_MAX_S overrides it; 0
-  // always launches dK/dV and dQ separately.
-  const int fused_max_s = env_int("MOGRAD_HIP_ATTN_FUSED_BWD_MAX_S", 1024);
+  // One launch for both walks up to this sequence length.  Measured at 8192 tokens per batch of
+  // twelve heads: causal, where the short walks of one kind fill the gaps the other leaves, 6-10 %
+  // faster up to 2048 tokens and even at 4096; non-causal 4-6 % faster at 512 and 3-6 % slower
+  // from 1024 on, where the two walks compete for the same CU.  MOGRAD_HIP_ATTN_FUSED_BWD_MAX_S
+  // overrides it; 0 always launches dK/dV and dQ separately.
+  const int fused_max_s = env_int("MOGRAD_HIP_ATTN_FUSED_BWD_MAX_S", causal ? 2048 : 512);
   const bool fused = DP <= 64 && a.S <= fused_max_s && 2 * (blocks + 7) < 0x7fffffffLL;
   const T* d_o_ = static_cast<const T*>(d_o);
   const T* q_ = static_cast<const T*>(q);
