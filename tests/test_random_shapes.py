@@ -11,7 +11,8 @@ from oracle import oracle_np as O
 
 pytestmark = pytest.mark.gpu
 
-from mograd_amd import BF16, F16, F32, I32, AnyBuffer  # noqa: E402
+from mograd_amd import BF16, F16, F32, I32, AnyBuffer, Layout, Node  # noqa: E402
+from mograd_amd import runtime as R  # noqa: E402
 from mograd_amd.runtime import round_to_dtype  # noqa: E402
 
 RT = {F32: 2e-4, F16: 2e-3, BF16: 1.6e-2}
@@ -181,6 +182,65 @@ def test_random_f32_attention_shapes(device):
                                 (dv.to_numpy((B, S, H, D)), wdv, "dv")):
             err = float(np.max(np.abs(got.astype(np.float64) - want)))
             assert np.all(np.isfinite(got)) and err <= 2e-5, f"{what} {name}: {err}"
+
+
+def _random_view(rng, shape):
+    """Strides (elements), base offset and backing size of a random view of `shape`: the dims laid
+    out in a random order, some broadcast (stride 0), some with a gap after them or every other
+    element taken."""
+    rank = len(shape)
+    order = list(rng.permutation(rank))
+    strides = [0] * rank
+    step = int(rng.integers(1, 3))  # innermost memory dim: every element or every other
+    for d in order:
+        if shape[d] > 1 and rng.random() < 0.2:
+            strides[d] = 0  # broadcast
+            continue
+        strides[d] = step
+        step = step * shape[d] + int(rng.integers(0, 3)) * (rng.random() < 0.3)
+    offset = int(rng.integers(0, 5))
+    size = offset + 1 + sum((n - 1) * t for n, t in zip(shape, strides))
+    return strides, offset, size
+
+
+def test_random_strided_views(device):
+    # add, relu, relu_grad, cast and softmax over random views of rank 1-5 (permuted, broadcast, gapped,
+    # strided, offset), bit for bit against numpy on the same views (softmax: the oracle at the storage
+    # type's rounding): the merging of dims and the choice of 16-byte accesses must never change a value.
+    rng = np.random.Generator(np.random.PCG64(99_000))
+    for case in range(60):
+        dtype = (F32, BF16, F16)[case % 3]
+        rank = int(rng.integers(1, 6))
+        shape = [int(rng.choice([1, 2, 3, 4, 8, 16, 24, 32])) for _ in range(rank)]
+        if case % 4 == 0:
+            shape[-1] = int(rng.choice([8, 16, 64]))  # rows that can be read 16 bytes at a time
+        (sa, oa, na), (sb, ob, nb) = _random_view(rng, shape), _random_view(rng, shape)
+        if case % 5 == 0:
+            sa, oa, na = list(Layout(*shape).stride()), 0, int(np.prod(shape))  # one operand plain
+        a = round_to_dtype(rng.standard_normal(na).astype(np.float32), dtype)
+        b = round_to_dtype(rng.standard_normal(nb).astype(np.float32), dtype)
+        item = a.itemsize
+        va = np.lib.stride_tricks.as_strided(a[oa:], shape, tuple(t * item for t in sa))
+        vb = np.lib.stride_tricks.as_strided(b[ob:], shape, tuple(t * item for t in sb))
+        la, lb = Layout(*shape, strides=sa, base_offset=oa), Layout(*shape, strides=sb, base_offset=ob)
+        out = Layout(*shape)
+        what = f"case {case} shape {shape} a {sa}+{oa} b {sb}+{ob} dtype {dtype}"
+
+        def run(op, operands, to=dtype):
+            srcs = [Node.leaf(l, d) for _, l, d in operands]
+            bufs = [AnyBuffer.from_numpy(device, h, d).view(l) for h, l, d in operands]
+            (res,) = R.run(Node(op, out, to, srcs, {}), bufs, device)
+            return res.to_numpy(tuple(shape))
+
+        np.testing.assert_array_equal(run("ADD", [(a, la, dtype), (b, lb, dtype)]), round_to_dtype(va + vb, dtype), what)
+        np.testing.assert_array_equal(run("RELU_GRAD", [(a, la, dtype), (b, lb, dtype)]),
+                                      np.where(va > 0, vb, 0).astype(np.float32), what)
+        np.testing.assert_array_equal(run("RELU", [(a, la, dtype)]), np.maximum(va, 0), what)
+        to = (BF16, F32, F16)[case % 3]
+        np.testing.assert_array_equal(run("CAST", [(a, la, dtype)], to), round_to_dtype(va, to), what)
+        tol = {F32: 2e-6, F16: 1e-3, BF16: 8e-3}[dtype]
+        np.testing.assert_allclose(run("SOFTMAX", [(a, la, dtype)]), O.softmax(va.astype(np.float64)), rtol=tol, atol=tol,
+                                   err_msg=what)
 
 
 def test_random_row_kernel_shapes(device):
