@@ -190,10 +190,12 @@ __device__ __forceinline__ bool f32_attn_vec_ok(const void* p, int64_t ld, int D
 }
 
 // Forward.  Grid (B * H, query blocks of 128): the heads of one block position run side by side, and a
-// causal launch starts with the last positions, whose walks are the longest.  Scores come out as keys x queries, so a query's
+// causal launch starts with the last positions, whose walks are the longest.  Scores come out as
+// keys x queries, so a query's
 // maximum and sum are over a lane's sixteen registers and its partner lane in the other half.
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
-__global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_fwd_f32_mfma_kernel(const T* __restrict__ q, const T* __restrict__ k,
+__global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_fwd_f32_mfma_kernel(
+    const T* __restrict__ q, const T* __restrict__ k,
                                                                    const T* __restrict__ v, const T* __restrict__ mask,
                                                                    T* __restrict__ o, float* __restrict__ lse, AttnDims a,
                                                                    float scale) {
@@ -273,7 +275,8 @@ __global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_fwd_f32_mfma_kernel
 
 // dQ.  Grid as the forward; P is recomputed from LSE, dP = V dO^T comes out in the same layout.
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
-__global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_dq_f32_mfma_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
+__global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_dq_f32_mfma_kernel(
+    const T* __restrict__ d_o, const T* __restrict__ q,
                                                                   const T* __restrict__ k, const T* __restrict__ v,
                                                                   const T* __restrict__ mask, const float* __restrict__ lse,
                                                                   const float* __restrict__ delta, T* __restrict__ dq,
@@ -336,7 +339,8 @@ __global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_dq_f32_mfma_kernel(
 // dK, dV.  Grid (B * H, key blocks of 128).  The wave's keys are along the lanes, the streamed
 // queries along the registers, so LSE and delta of a tile's rows are read per register.
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
-__global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_dkdv_f32_mfma_kernel(const T* __restrict__ d_o, const T* __restrict__ q,
+__global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_dkdv_f32_mfma_kernel(
+    const T* __restrict__ d_o, const T* __restrict__ q,
                                                                     const T* __restrict__ k, const T* __restrict__ v,
                                                                     const T* __restrict__ mask,
                                                                     const float* __restrict__ lse,

@@ -371,7 +371,8 @@ static int map_strided_dispatch(const char* who, const void* a, const void* b, v
                                 hipStream_t s) {
   constexpr bool kBinary = OP == kMapAdd || OP == kMapReluGrad;
   if (!is_float_dtype(in_dtype) || !is_float_dtype(out_dtype))
-    return fail(MG_ERR_INVALID, "%s: unsupported dtype %s", who, dtype_name(is_float_dtype(in_dtype) ? out_dtype : in_dtype));
+    return fail(MG_ERR_INVALID, "%s: unsupported dtype %s", who,
+                dtype_name(is_float_dtype(in_dtype) ? out_dtype : in_dtype));
   if (rank < 0 || rank > kMaxRank) return fail(MG_ERR_INVALID, "%s: rank %d outside 0..%d", who, rank, kMaxRank);
   if (rank > 0 && (!shape || !strides_a || (kBinary && !strides_b)))
     return fail(MG_ERR_INVALID, "%s: null shape or strides", who);

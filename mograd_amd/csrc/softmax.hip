@@ -53,8 +53,8 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const T* __restrict__
 // The rows of a strided view: `v` holds the extents and strides of the dims in front of the
 // last one, `xs` the stride of the last.  The result is row-major.
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void softmax_view_kernel(const T* __restrict__ x, T* __restrict__ y, StridedView v, int64_t xs,
-                                                           int64_t rows, int64_t cols) {
+__global__ __launch_bounds__(256) void softmax_view_kernel(const T* __restrict__ x, T* __restrict__ y, StridedView v,
+                                                           int64_t xs, int64_t rows, int64_t cols) {
   const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
   if (row >= rows) return;  // wave-uniform
   int64_t rem = row, off = 0;
@@ -159,8 +159,8 @@ static int softmax_typed(const void* x, void* y, int64_t rows, int64_t cols, hip
 }
 
 template <typename T>
-static int softmax_view_typed(const void* x, void* y, const StridedView& v, int64_t xs, int64_t rows, int64_t cols, bool wide,
-                              hipStream_t s) {
+static int softmax_view_typed(const void* x, void* y, const StridedView& v, int64_t xs, int64_t rows, int64_t cols,
+                              bool wide, hipStream_t s) {
   constexpr int WIDE = WideVec<T>::value;
   const dim3 grid(static_cast<unsigned>(ceil_div(rows, 4)));
   if (wide && cols % WIDE == 0)
@@ -224,7 +224,8 @@ int mg_softmax(const void* x, void* y, int64_t rows, int64_t cols, int dtype, mg
 
 int mg_softmax_strided(const void* x, void* y, int rank, const int64_t* shape, const int64_t* strides, int dtype,
                        mg_stream stream) {
-  if (rank < 1 || rank > mg::kMaxRank) return mg::fail(MG_ERR_INVALID, "softmax_strided: rank %d outside 1..%d", rank, mg::kMaxRank);
+  if (rank < 1 || rank > mg::kMaxRank)
+    return mg::fail(MG_ERR_INVALID, "softmax_strided: rank %d outside 1..%d", rank, mg::kMaxRank);
   if (!shape || !strides) return mg::fail(MG_ERR_INVALID, "softmax_strided: null shape or strides");
   int64_t rows = 1;
   mg::StridedView v;
