@@ -18,7 +18,9 @@
 //    per register (dK/dV).
 // A workgroup is four waves of 32 resident rows each; tiles of 32 streamed rows of two tensors go
 // through LDS as fp32 (rows padded by four floats: the 128-bit reads of sixteen rows then fall in
-// sixteen different bank groups), fetched into registers one tile ahead.  The 128-column kernels
+// sixteen different bank groups), fetched into registers one tile ahead (a second copy of the tiles
+// in LDS, which saves one of the two barriers per step, measured no faster: the steps are bound by the
+// matrix pipe, not by the barriers).  The 128-column kernels
 // run one workgroup per CU with the 512-register budget (two resident rows of 64 values and
 // eight accumulators per lane in dK/dV).  Same mathematics, masks,
 // layouts, LSE and error budget as the other fp32 forms; nothing of size S x S is stored.
@@ -195,10 +197,8 @@ __device__ __forceinline__ bool f32_attn_vec_ok(const void* p, int64_t ld, int D
 // maximum and sum are over a lane's sixteen registers and its partner lane in the other half.
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
 __global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_fwd_f32_mfma_kernel(
-    const T* __restrict__ q, const T* __restrict__ k,
-                                                                   const T* __restrict__ v, const T* __restrict__ mask,
-                                                                   T* __restrict__ o, float* __restrict__ lse, AttnDims a,
-                                                                   float scale) {
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const T* __restrict__ mask,
+    T* __restrict__ o, float* __restrict__ lse, AttnDims a, float scale) {
   __shared__ __attribute__((aligned(16))) float k_s[kF32AttnRows * (DP + 4)];
   __shared__ __attribute__((aligned(16))) float v_s[kF32AttnRows * (DP + 4)];
   const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H;
@@ -276,11 +276,9 @@ __global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_fwd_f32_mfma_kernel
 // dQ.  Grid as the forward; P is recomputed from LSE, dP = V dO^T comes out in the same layout.
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
 __global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_dq_f32_mfma_kernel(
-    const T* __restrict__ d_o, const T* __restrict__ q,
-                                                                  const T* __restrict__ k, const T* __restrict__ v,
-                                                                  const T* __restrict__ mask, const float* __restrict__ lse,
-                                                                  const float* __restrict__ delta, T* __restrict__ dq,
-                                                                  AttnDims a, float scale) {
+    const T* __restrict__ d_o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+    const T* __restrict__ mask, const float* __restrict__ lse, const float* __restrict__ delta, T* __restrict__ dq,
+    AttnDims a, float scale) {
   __shared__ __attribute__((aligned(16))) float k_s[kF32AttnRows * (DP + 4)];
   __shared__ __attribute__((aligned(16))) float v_s[kF32AttnRows * (DP + 4)];
   const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H;
@@ -340,12 +338,9 @@ __global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_dq_f32_mfma_kernel(
 // queries along the registers, so LSE and delta of a tile's rows are read per register.
 template <typename T, int DP, bool CAUSAL, bool HAS_BIAS>
 __global__ __launch_bounds__(256, DP > 64 ? 1 : 2) void attn_dkdv_f32_mfma_kernel(
-    const T* __restrict__ d_o, const T* __restrict__ q,
-                                                                    const T* __restrict__ k, const T* __restrict__ v,
-                                                                    const T* __restrict__ mask,
-                                                                    const float* __restrict__ lse,
-                                                                    const float* __restrict__ delta, T* __restrict__ dk,
-                                                                    T* __restrict__ dv, AttnDims a, float scale) {
+    const T* __restrict__ d_o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+    const T* __restrict__ mask, const float* __restrict__ lse, const float* __restrict__ delta, T* __restrict__ dk,
+    T* __restrict__ dv, AttnDims a, float scale) {
   __shared__ __attribute__((aligned(16))) float q_s[kF32AttnRows * (DP + 4)];
   __shared__ __attribute__((aligned(16))) float do_s[kF32AttnRows * (DP + 4)];
   __shared__ __attribute__((aligned(16))) float lse_s[kF32AttnRows];
