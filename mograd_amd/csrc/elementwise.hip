@@ -196,6 +196,55 @@ __global__ __launch_bounds__(256) void map_strided_kernel(const S* __restrict__ 
   }
 }
 
+// The same copy for a view whose innermost dim is strided while another dim is contiguous in the
+// source (a transpose, possibly with outer dims around and between): TILE x TILE elements go
+// through LDS, read along the source's contiguous dim and written along the result's, so both
+// sides move whole cache lines where the element-wise kernel reads one element per line.
+// `col` is the source-contiguous dim (stride 1), `row` the innermost dim of the result; the
+// other dims are batch dims, decomposed per workgroup.
+struct TransposeView {
+  int nbatch;                  // batch dims
+  int64_t bshape[kMaxRank];    // their extents, outermost first
+  int64_t bsrc[kMaxRank];      // their source strides (elements)
+  int64_t bdst[kMaxRank];      // their strides in the result
+  int64_t rows, cols;          // extents of the two transposed dims
+  int64_t row_src_stride;      // source stride of the row dim
+  int64_t col_dst_stride;      // stride of the col dim in the result
+};
+
+template <typename V, int TILE>
+__global__ __launch_bounds__(256) void contiguous_transpose_kernel(const V* __restrict__ src, V* __restrict__ dst,
+                                                                   TransposeView v, int64_t col_tiles,
+                                                                   int64_t row_tiles) {
+  constexpr int TY = 256 / TILE;
+  __shared__ V tile[TILE][TILE + 1];
+  int64_t w = blockIdx.x;
+  const int64_t ct = w % col_tiles;
+  w /= col_tiles;
+  const int64_t rt = w % row_tiles;
+  w /= row_tiles;
+  int64_t src_at = 0, dst_at = 0;
+  for (int d = v.nbatch - 1; d >= 0; --d) {
+    const int64_t q = w / v.bshape[d], i = w - q * v.bshape[d];
+    src_at += i * v.bsrc[d];
+    dst_at += i * v.bdst[d];
+    w = q;
+  }
+  const int tx = threadIdx.x % TILE, ty = threadIdx.x / TILE;
+  const int64_t c0 = ct * TILE, r0 = rt * TILE;
+#pragma unroll
+  for (int k = 0; k < TILE; k += TY) {
+    const int64_t r = r0 + ty + k, c = c0 + tx;
+    if (r < v.rows && c < v.cols) tile[ty + k][tx] = src[src_at + r * v.row_src_stride + c];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < TILE; k += TY) {
+    const int64_t c = c0 + ty + k, r = r0 + tx;
+    if (r < v.rows && c < v.cols) dst[dst_at + c * v.col_dst_stride + r] = tile[tx][ty + k];
+  }
+}
+
 static unsigned stream_blocks(int64_t n, int per_thread) {
   int64_t blocks = ceil_div(n, static_cast<int64_t>(256) * per_thread);
   const int64_t cap = static_cast<int64_t>(device_info().cu_count) * 16;
@@ -249,6 +298,45 @@ static int contiguous_launch(const void* src, void* dst, const CopyView& v, int6
   return MG_OK;
 }
 
+// The tiled transpose for normalised dims (sh, st): taken when the innermost dim is strided, one
+// other dim has stride 1, and both are long enough to fill tiles.  Returns false when the view is
+// not of that kind (kNotTransposed), else the launch's status.
+constexpr int kNotTransposed = -1;
+template <typename V, int TILE>
+static int contiguous_transpose_try(const void* src, void* dst, int r, const int64_t* sh, const int64_t* st,
+                                    hipStream_t s) {
+  if (r < 2 || st[r - 1] == 1 || st[r - 1] == 0) return kNotTransposed;
+  int p = -1;
+  for (int d = 0; d + 1 < r; ++d)
+    if (st[d] == 1) p = d;
+  if (p < 0 || sh[p] < TILE / 2 || sh[r - 1] < TILE / 2) return kNotTransposed;
+  int64_t dstride[kMaxRank];
+  dstride[r - 1] = 1;
+  for (int d = r - 2; d >= 0; --d) dstride[d] = dstride[d + 1] * sh[d + 1];
+  TransposeView v;
+  v.nbatch = 0;
+  int64_t batch = 1;
+  for (int d = 0; d + 1 < r; ++d) {
+    if (d == p) continue;
+    v.bshape[v.nbatch] = sh[d];
+    v.bsrc[v.nbatch] = st[d];
+    v.bdst[v.nbatch] = dstride[d];
+    ++v.nbatch;
+    batch *= sh[d];
+  }
+  v.rows = sh[r - 1];
+  v.cols = sh[p];
+  v.row_src_stride = st[r - 1];
+  v.col_dst_stride = dstride[p];
+  const int64_t col_tiles = ceil_div(v.cols, TILE), row_tiles = ceil_div(v.rows, TILE);
+  const int64_t blocks = col_tiles * row_tiles * batch;
+  if (blocks > 0x7fffffffLL) return kNotTransposed;
+  hipLaunchKernelGGL((contiguous_transpose_kernel<V, TILE>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s,
+                     static_cast<const V*>(src), static_cast<V*>(dst), v, col_tiles, row_tiles);
+  MG_LAUNCH_CHECK();
+  return MG_OK;
+}
+
 static int contiguous_dispatch(const void* src, void* dst, int rank, const int64_t* shape, const int64_t* strides,
                                int dtype, hipStream_t s) {
   const int esz = dtype_size(dtype);
@@ -281,6 +369,16 @@ static int contiguous_dispatch(const void* src, void* dst, int rank, const int64
     sh[0] = 1;
     st[0] = 1;
     r = 1;
+  }
+  if (env_int("MOGRAD_HIP_CONTIGUOUS_TRANSPOSE", 1) != 0) {  // transposes go through LDS tiles
+    int status = kNotTransposed;
+    switch (esz) {
+      case 8: status = contiguous_transpose_try<uint2, 32>(src, dst, r, sh, st, s); break;
+      case 4: status = contiguous_transpose_try<uint32_t, 32>(src, dst, r, sh, st, s); break;
+      case 2: status = contiguous_transpose_try<uint16_t, 64>(src, dst, r, sh, st, s); break;
+      default: break;
+    }
+    if (status != kNotTransposed) return status;
   }
   // Widest chunk (bytes) that divides the innermost run and every outer stride.
   int chunk = esz;
@@ -384,6 +482,39 @@ static int map_strided_dispatch(const char* who, const void* a, const void* b, v
   }
   if (n == 0) return MG_OK;
   if (!a || (kBinary && !b) || !dst) return fail(MG_ERR_INVALID, "%s: null pointer argument", who);
+  // A large operand that is a transpose (innermost dim strided, another dim contiguous in memory)
+  // would be read one element per cache line: it is first copied row-major through the tiled
+  // transpose (3-5 x the rate of the element-wise read) and the map then runs on the copy.
+  Scratch copy_a, copy_b;
+  int64_t row_major[kMaxRank];
+  {
+    int64_t run = 1;
+    for (int d = rank - 1; d >= 0; --d) {
+      row_major[d] = run;
+      run *= shape[d];
+    }
+  }
+  auto transposed = [&](const int64_t* st) {
+    if (n < (int64_t{1} << 16) || env_int("MOGRAD_HIP_CONTIGUOUS_TRANSPOSE", 1) == 0) return false;
+    int inner = rank - 1;
+    while (inner >= 0 && shape[inner] == 1) --inner;
+    if (inner < 0 || st[inner] <= 1 || shape[inner] < 32) return false;
+    for (int d = 0; d < inner; ++d)
+      if (st[d] == 1 && shape[d] >= 32) return true;
+    return false;
+  };
+  if (transposed(strides_a)) {
+    MG_TRY(copy_a.take(n * static_cast<int64_t>(dtype_size(in_dtype))));
+    MG_TRY(contiguous_dispatch(a, copy_a.as<char>(), rank, shape, strides_a, in_dtype, s));
+    a = copy_a.as<char>();
+    strides_a = row_major;
+  }
+  if (kBinary && transposed(strides_b)) {
+    MG_TRY(copy_b.take(n * static_cast<int64_t>(dtype_size(in_dtype))));
+    MG_TRY(contiguous_dispatch(b, copy_b.as<char>(), rank, shape, strides_b, in_dtype, s));
+    b = copy_b.as<char>();
+    strides_b = row_major;
+  }
   int64_t sh[kMaxRank], sa[kMaxRank], sb[kMaxRank];
   int r = 0;
   for (int d = 0; d < rank; ++d) {

@@ -236,6 +236,7 @@ def test_random_strided_views(device):
         np.testing.assert_array_equal(run("RELU_GRAD", [(a, la, dtype), (b, lb, dtype)]),
                                       np.where(va > 0, vb, 0).astype(np.float32), what)
         np.testing.assert_array_equal(run("RELU", [(a, la, dtype)]), np.maximum(va, 0), what)
+        np.testing.assert_array_equal(run("CONTIGUOUS", [(b, lb, dtype)]), vb, what)
         to = (BF16, F32, F16)[case % 3]
         np.testing.assert_array_equal(run("CAST", [(a, la, dtype)], to), round_to_dtype(va, to), what)
         tol = {F32: 2e-6, F16: 1e-3, BF16: 8e-3}[dtype]

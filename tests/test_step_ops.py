@@ -65,6 +65,14 @@ CONTIG_CASES = [
     ((2, 3, 4), (12, 4, 1), 24),                 # already contiguous
     ((6,), (3,), 18),
     ((1, 1), (1, 1), 1),
+    # transposes long enough for the tiled kernel (one dim contiguous in the source, the innermost strided)
+    ((100, 70), (1, 100), 7000),                 # plain 2-D transpose, ragged tiles
+    ((64, 128), (1, 64), 8192),                  # whole tiles
+    ((3, 50, 40), (2000, 1, 50), 6000),          # batched transpose
+    ((33, 5, 47), (1, 33, 165), 33 * 5 * 47),    # dims reversed: a batch dim between the two
+    ((2, 40, 3, 36), (40, 1, 2880, 80), 8640),   # batch dims outside and between, a permuted 4-D tensor
+    ((48, 20), (2, 100), 2000),                  # strided both ways: not a transpose, element by element
+    ((40, 33), (1, 80), 80 * 33),                # a transposed slice: rows of the source 80 apart
 ]
 
 
