@@ -243,6 +243,18 @@ int mg_softmax_strided(const void* x, void* y, int rank, const int64_t* shape, c
   MG_TRY(mg::check_rows("softmax_strided", rows, cols, dtype));
   if (rows == 0 || cols == 0) return MG_OK;
   if (!x || !y) return mg::fail(MG_ERR_INVALID, "softmax_strided: null pointer argument");
+  // Rows that run across memory lines (a transposed view) of a large tensor: copy the view
+  // row-major first (mg_contiguous moves transposes through LDS tiles) and take the flat kernel.
+  if (xs > 1 && cols >= 32 && rows * cols >= (int64_t{1} << 16)) {
+    bool has_unit = false;
+    for (int d = 0; d + 1 < rank; ++d) has_unit = has_unit || (strides[d] == 1 && shape[d] >= 32);
+    if (has_unit) {
+      mg::Scratch copy;
+      MG_TRY(copy.take(rows * cols * static_cast<int64_t>(mg::dtype_size(dtype))));
+      MG_TRY(mg_contiguous(x, copy.as<char>(), rank, shape, strides, dtype, stream));
+      return mg_softmax(copy.as<char>(), y, rows, cols, dtype, stream);
+    }
+  }
   // 16-byte loads where a row is contiguous and every row starts on a 16-byte boundary
   bool wide = xs == 1 && mg::aligned16(x) && mg::aligned16(y);
   for (int d = 0; d + 1 < rank && wide; ++d) wide = shape[d] == 1 || strides[d] * mg::dtype_size(dtype) % 16 == 0;

@@ -344,6 +344,7 @@ SOFTMAX_VIEWS = [
     ((5, 40), (56, 1), 5 * 56),                      # rows with a gap between them
     ((7,), (3,), 21),
     ((300, 1000), (1000, 1), 300000),                # contiguous, through the strided entry at an odd offset
+    ((512, 256), (1, 512), 512 * 256),               # a large transpose: copied through the tiled transpose first
 ]
 
 
